@@ -1,0 +1,201 @@
+"""ctypes front-end of the CPU oracle (oracle/liboracle.so) and of the compiled reference
+kernels (oracle/_ref/libhodu_cpu_ref.so, when built).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline
+leg of bench.py as the checker.  The product (hodu_amd and the C-ABI library) never imports it.
+
+Narrow types travel as raw bit patterns: bf16 / f16 in uint16 arrays, f8e4m3 / f8e5m2 / bool in
+uint8 arrays -- the little-endian element encodings of crates/hodu_core/src/tensor/bytes.rs:90-180.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+# dtype ids: crates/hodu_core/src/types/dtype.rs:6-28
+DTYPE_ID = {
+    "bool": 0, "f8e4m3": 1, "f8e5m2": 2, "bf16": 3, "f16": 4, "f32": 5, "f64": 6,
+    "u8": 7, "u16": 8, "u32": 9, "u64": 10, "i8": 11, "i16": 12, "i32": 13, "i64": 14,
+}
+# numpy container for each dtype's storage
+STORAGE = {
+    "bool": np.uint8, "f8e4m3": np.uint8, "f8e5m2": np.uint8, "bf16": np.uint16, "f16": np.uint16,
+    "f32": np.float32, "f64": np.float64, "u8": np.uint8, "u16": np.uint16, "u32": np.uint32,
+    "u64": np.uint64, "i8": np.int8, "i16": np.int16, "i32": np.int32, "i64": np.int64,
+}
+MATMUL_DTYPES = [d for d in DTYPE_ID if d != "bool"]
+F8_HODU, F8_OCP = 0, 1
+
+
+def build(force: bool = False) -> None:
+    """Compile liboracle.so (and _ref when the reference tree is present) with oracle/Makefile."""
+    if force or not os.path.exists(os.path.join(_HERE, "liboracle.so")):
+        subprocess.check_call(["make", "-C", _HERE, "all"], stdout=subprocess.DEVNULL)
+
+
+def _md(md) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(md, dtype=np.uint64))
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(os.path.join(_HERE, "liboracle.so"))
+        _lib.oracle_f8e4m3_to_f32.restype = ctypes.c_float
+        _lib.oracle_f8e4m3_to_f32.argtypes = [ctypes.c_uint8, ctypes.c_int]
+        _lib.oracle_f32_to_f8e4m3.restype = ctypes.c_uint8
+        _lib.oracle_f32_to_f8e4m3.argtypes = [ctypes.c_float]
+        _lib.oracle_f32_to_f16.restype = ctypes.c_uint16
+        _lib.oracle_f32_to_f16.argtypes = [ctypes.c_float]
+        _lib.oracle_f16_to_f32.restype = ctypes.c_float
+        _lib.oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+        _lib.oracle_reference_threads.restype = ctypes.c_size_t
+        _lib.oracle_reference_threads.argtypes = [ctypes.c_size_t] * 3
+    return _lib
+
+
+def set_threads(n: int) -> None:
+    lib().oracle_set_threads(int(n))
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"oracle: {what} failed (rc={rc})")
+
+
+def matmul_out_elems(md) -> int:
+    return int(md[0])
+
+
+def dot_out_elems(md) -> int:
+    return int(md[0]) * int(md[2])
+
+
+def matmul_asis(dt: str, lhs: np.ndarray, rhs: np.ndarray, md) -> np.ndarray:
+    """hodu_cpu_matmul_<dt>, bit-faithful."""
+    md = _md(md)
+    out = np.empty(matmul_out_elems(md), dtype=STORAGE[dt])
+    _check(lib().oracle_matmul_asis(DTYPE_ID[dt], _ptr(lhs), _ptr(rhs), _ptr(out), _ptr(md)), "matmul_asis")
+    return out
+
+
+def dot_asis(dt: str, lhs: np.ndarray, rhs: np.ndarray, md) -> np.ndarray:
+    """hodu_cpu_dot_<dt>, bit-faithful."""
+    md = _md(md)
+    out = np.empty(dot_out_elems(md), dtype=STORAGE[dt])
+    _check(lib().oracle_dot_asis(DTYPE_ID[dt], _ptr(lhs), _ptr(rhs), _ptr(out), _ptr(md)), "dot_asis")
+    return out
+
+
+def _spec(fn, n, l_dt, r_dt, lhs, rhs, md, decode, want64):
+    out32 = np.empty(n, dtype=np.float32)
+    out64 = np.empty(n, dtype=np.float64) if want64 else None
+    outabs = np.empty(n, dtype=np.float64) if want64 else None
+    rc = fn(DTYPE_ID[l_dt], DTYPE_ID[r_dt], decode, _ptr(lhs), _ptr(rhs), _ptr(out32),
+            _ptr(out64) if want64 else None, _ptr(outabs) if want64 else None, _ptr(md))
+    _check(rc, "spec")
+    return out32, out64, outabs
+
+
+def matmul_spec(l_dt, r_dt, lhs, rhs, md, decode=F8_OCP, want64=True):
+    """f32-accumulated comparator (matmul metadata).  Returns (f32 sums, f64 sums, f64 sum|a*b|)."""
+    md = _md(md)
+    return _spec(lib().oracle_matmul_spec, matmul_out_elems(md), l_dt, r_dt, lhs, rhs, md, decode, want64)
+
+
+def dot_spec(l_dt, r_dt, lhs, rhs, md, decode=F8_OCP, want64=True):
+    """f32-accumulated comparator (dot metadata)."""
+    md = _md(md)
+    return _spec(lib().oracle_dot_spec, dot_out_elems(md), l_dt, r_dt, lhs, rhs, md, decode, want64)
+
+
+def cast(src: str, dst: str, x: np.ndarray, md, decode=F8_HODU) -> np.ndarray:
+    """hodu_cpu_cast_<src>_to_<dst>; decode picks the f8e4m3 table (hodu CPU or OCP)."""
+    md = _md(md)
+    out = np.empty(int(md[0]), dtype=STORAGE[dst])
+    _check(lib().oracle_cast(DTYPE_ID[src], DTYPE_ID[dst], decode, _ptr(x), _ptr(out), _ptr(md)), "cast")
+    return out
+
+
+def contiguous(dt: str, x: np.ndarray, md) -> np.ndarray:
+    """hodu_cpu_contiguous_<dt>"""
+    md = _md(md)
+    out = np.empty(int(md[0]), dtype=STORAGE[dt])
+    _check(lib().oracle_contiguous(DTYPE_ID[dt], _ptr(x), _ptr(out), _ptr(md)), "contiguous")
+    return out
+
+
+def f8e4m3_table(decode: int) -> np.ndarray:
+    """All 256 decoded values as f32."""
+    return np.array([lib().oracle_f8e4m3_to_f32(b, decode) for b in range(256)], dtype=np.float32)
+
+
+def reference_threads(work: int, min_per_thread: int, online: int) -> int:
+    return int(lib().oracle_reference_threads(work, min_per_thread, online))
+
+
+# ---------------------------------------------------------------------------------------------
+# the compiled reference (only where oracle/_ref was built; never present in git history)
+# ---------------------------------------------------------------------------------------------
+class RefLib:
+    """hodu_cpu_* symbols of the reference's own C kernels compiled by oracle/Makefile."""
+
+    PATH = os.path.join(_HERE, "_ref", "libhodu_cpu_ref.so")
+
+    @classmethod
+    def available(cls) -> bool:
+        return os.path.exists(cls.PATH)
+
+    def __init__(self):
+        self.lib = ctypes.CDLL(self.PATH)
+
+    @staticmethod
+    def _sfx(dt: str) -> str:
+        # on Linux the plain f32/f64 product symbols exist only with the openblas feature
+        # (build.rs:137-159); the C file defines *_fallback
+        return dt + "_fallback" if dt in ("f32", "f64") else dt
+
+    def matmul(self, dt, lhs, rhs, md):
+        md = _md(md)
+        out = np.empty(matmul_out_elems(md), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_matmul_{self._sfx(dt)}")
+        fn.restype = None
+        fn(_ptr(lhs), _ptr(rhs), _ptr(out), _ptr(md))
+        return out
+
+    def dot(self, dt, lhs, rhs, md):
+        md = _md(md)
+        out = np.empty(dot_out_elems(md), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_dot_{self._sfx(dt)}")
+        fn.restype = None
+        fn(_ptr(lhs), _ptr(rhs), _ptr(out), _ptr(md))
+        return out
+
+    def cast(self, src, dst, x, md):
+        md = _md(md)
+        out = np.empty(int(md[0]), dtype=STORAGE[dst])
+        fn = getattr(self.lib, f"hodu_cpu_cast_{src}_to_{dst}")
+        fn.restype = None
+        fn(_ptr(x), _ptr(out), _ptr(md))
+        return out
+
+    def contiguous(self, dt, x, md):
+        md = _md(md)
+        out = np.empty(int(md[0]), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_contiguous_{dt}")
+        fn.restype = None
+        fn(_ptr(x), _ptr(out), _ptr(md))
+        return out

@@ -1,0 +1,69 @@
+"""Where oracle/_ref was built (the build container), the oracle is compared bit for bit with the
+reference's own compiled C kernels on fresh seeded cases beyond the committed fixtures."""
+import numpy as np
+import pytest
+
+import helpers as H
+import oracle
+
+pytestmark = pytest.mark.skipif(not oracle.RefLib.available(), reason="oracle/_ref not built on this machine")
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint8)
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return oracle.RefLib()
+
+
+CASES = [
+    ("dot", H.View([64, 130]), H.View([130, 70])),
+    ("dot", H.View([530, 33]), H.View([33, 9])),
+    ("dot", H.View([12, 300]), H.View([16, 300]).t()),
+    ("dot", H.View([50, 12], offset=9).t(), H.View([50, 12], offset=1)),
+    ("matmul", H.View([5, 8, 33]), H.View([5, 33, 6])),
+    ("matmul", H.View([300, 20]), H.View([20, 8])),
+    ("matmul", H.View([2, 3, 4, 20]), H.View([7, 20]).t().broadcast_to([2, 3, 20, 7])),
+    ("matmul", H.View([1, 6, 20]), H.View([4, 20, 5])),
+]
+
+
+@pytest.mark.parametrize("dt", oracle.MATMUL_DTYPES)
+def test_products_match_compiled_reference(ref, dt):
+    for n, (op, lv, rv) in enumerate(CASES):
+        a = H.random_storage(dt, lv.span(), 1000 + n, 2.0)
+        b = H.random_storage(dt, rv.span(), 2000 + n, 2.0)
+        md = H.dot_md(lv, rv) if op == "dot" else H.matmul_md(lv, rv)
+        want = ref.dot(dt, a, b, md) if op == "dot" else ref.matmul(dt, a, b, md)
+        got = oracle.dot_asis(dt, a, b, md) if op == "dot" else oracle.matmul_asis(dt, a, b, md)
+        assert np.array_equal(_bits(got), _bits(want)), (dt, n)
+
+
+def test_every_cast_pair_matches_compiled_reference(ref):
+    v = H.View([7, 9, 5], offset=3).t(0, 2)
+    md = H.cast_md(v)
+    for src in oracle.DTYPE_ID:
+        for dst in oracle.DTYPE_ID:
+            x = H.random_storage(src, v.span(), 77, 3.0)
+            if src in ("f32", "f64") and dst.startswith("u") or dst == "bool" and src in ("f32", "f64"):
+                x = np.abs(x)
+            if src in ("bf16", "f16") and dst.startswith("u"):
+                x = x & 0x7FFF
+            if src in ("f8e4m3", "f8e5m2") and dst.startswith("u"):
+                x = x & 0x7F
+            want, got = ref.cast(src, dst, x, md), oracle.cast(src, dst, x, md)
+            if dst in ("f32", "f64"):
+                gf, wf = got, want
+                assert np.array_equal(np.isnan(gf), np.isnan(wf)), (src, dst)
+                assert np.array_equal(gf[~np.isnan(gf)], wf[~np.isnan(wf)]), (src, dst)
+            else:
+                assert np.array_equal(_bits(got), _bits(want)), (src, dst)
+
+
+def test_contiguous_matches_compiled_reference(ref):
+    for v in (H.View([300]), H.View([13, 21]).t(), H.View([4, 5, 6], offset=2).slice(1, 1, 5, 2)):
+        for dt in oracle.DTYPE_ID:
+            x = H.random_storage(dt, v.span(), 5)
+            assert np.array_equal(_bits(ref.contiguous(dt, x, H.cast_md(v))), _bits(oracle.contiguous(dt, x, H.cast_md(v))))
