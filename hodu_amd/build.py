@@ -1,0 +1,70 @@
+"""Builds hodu_amd/lib/libhodu_rocm_kernels.so from hodu_amd/csrc with hipcc for gfx950.
+
+hipcc cross-compiles without a GPU, so this runs in the build container; the resulting library is
+kept in-tree (git-ignored) and loaded by hodu_amd.ffi.  `python -m hodu_amd.build` rebuilds it.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "_build")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIB_DIR, "libhodu_rocm_kernels.so")
+
+ARCH = "gfx950"
+# -packed-fp32-ops off: keep hipcc from forming v_pk_{add,mul,fma}_f32 out of scalar float code
+FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
+]
+
+
+def hipcc() -> str:
+    path = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(path):
+        raise RuntimeError("hipcc not found: the HIP extension cannot be built on this machine")
+    return path
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+    cmd = [hipcc(), *FLAGS, "-c", src, "-o", obj]
+    if src.endswith(".cpp"):
+        cmd[1:1] = ["-x", "hip"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr[-6000:]}")
+    return obj
+
+
+def sources():
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".cpp")))
+
+
+def build(verbose: bool = True, jobs: int = 8) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    srcs = sources()
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, srcs))
+    tmp = LIB + ".tmp"
+    r = subprocess.run([hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+    os.replace(tmp, LIB)
+    if verbose:
+        print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,167 @@
+// extern "C" compute entry points: metadata parsing, kernel-family selection, launch.
+#include "common.hpp"
+
+namespace hodu {
+namespace {
+
+int check_ptrs(const char *op, hodu_rocm_ctx *ctx, const void *a, const void *b, const void *out) {
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "%s: context is null", op);
+    if (!a || !b || !out) return fail(HODU_ROCM_INVALID_ARG, "%s: null operand pointer", op);
+    if (out == a || out == b) return fail(HODU_ROCM_INVALID_ARG, "%s: out aliases an input", op);
+    return HODU_ROCM_OK;
+}
+
+// Picks the kernel family for one launch-sized product.
+int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
+                 const DevProduct &g) {
+    int rc = launch_skinny(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    rc = launch_mfma(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    ctx->last_kernel = "generic";
+    return launch_generic(ctx, kind, dtype, a, b, c, g);
+}
+
+size_t out_elem_size(int kind, int dtype) {
+    if (kind == PK_BF16_F8W) return 2;
+    if (kind == PK_I32_I8I8) return 4;
+    return dtype_size(dtype);
+}
+
+// Splits a parsed product into launches: the innermost kKernelBatchDims merged batch dims go to
+// the kernel, any further outer dims are walked here.
+int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p) {
+    HODU_HIP(hipSetDevice(ctx->device));
+    if (p.M > 0x7FFFFFFFL || p.N > 0x7FFFFFFFL || p.K > 0x7FFFFFFFL)
+        return fail(HODU_ROCM_UNSUPPORTED, "matrix extent exceeds 2^31-1");
+    if (p.batches == 0 || p.M == 0 || p.N == 0) return HODU_ROCM_OK;  // empty output: nothing to write
+
+    DevProduct g{};
+    g.M = (int)p.M; g.N = (int)p.N; g.K = (int)p.K;
+    g.a_m = p.a_m; g.a_k = p.a_k; g.b_k = p.b_k; g.b_n = p.b_n;
+    const int inner = p.nb < kKernelBatchDims ? p.nb : kKernelBatchDims;
+    const int outer = p.nb - inner;
+    g.nb = inner;
+    g.batches = 1;
+    for (int d = 0; d < inner; d++) {
+        if (p.bshape[outer + d] > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "batch extent exceeds 2^31-1");
+        g.bshape[d] = (int)p.bshape[outer + d];
+        g.a_bs[d] = p.a_bs[outer + d];
+        g.b_bs[d] = p.b_bs[outer + d];
+        g.batches *= p.bshape[outer + d];
+    }
+    long outer_count = 1;
+    for (int d = 0; d < outer; d++) outer_count *= p.bshape[d];
+    const size_t out_step = (size_t)g.batches * (size_t)p.M * (size_t)p.N * out_elem_size(kind, dtype);
+    for (long o = 0; o < outer_count; o++) {
+        long rem = o, ao = p.a_off, bo = p.b_off;
+        for (int d = outer - 1; d >= 0; d--) {
+            const long i = rem % p.bshape[d];
+            rem /= p.bshape[d];
+            ao += i * p.a_bs[d];
+            bo += i * p.b_bs[d];
+        }
+        g.a_off = ao; g.b_off = bo;
+        int rc = dispatch_one(ctx, kind, dtype, a, b, (char *)c + (size_t)o * out_step, g);
+        if (rc != HODU_ROCM_OK) return rc;
+    }
+    return HODU_ROCM_OK;
+}
+
+int matmul_entry(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const size_t *md,
+                 size_t len) {
+    clear_error();
+    int rc = check_ptrs("matmul", ctx, a, b, c);
+    if (rc) return rc;
+    Product p;
+    rc = parse_matmul_metadata(md, len, &p);
+    if (rc) return rc;
+    return run_product(ctx, kind, dtype, a, b, c, p);
+}
+
+int dot_entry(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const size_t *md,
+              size_t len) {
+    clear_error();
+    int rc = check_ptrs("dot", ctx, a, b, c);
+    if (rc) return rc;
+    Product p;
+    rc = parse_dot_metadata(md, len, &p);
+    if (rc) return rc;
+    return run_product(ctx, kind, dtype, a, b, c, p);
+}
+
+}  // namespace
+}  // namespace hodu
+
+using namespace hodu;
+
+extern "C" {
+
+#define HODU_ROCM_DEF_PRODUCT(dt, ID)                                                                          \
+    int hodu_rocm_matmul_##dt(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,     \
+                              size_t n) {                                                                      \
+        return matmul_entry(ctx, PK_SAME, ID, l, r, o, md, n);                                                 \
+    }                                                                                                          \
+    int hodu_rocm_dot_##dt(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,        \
+                           size_t n) {                                                                         \
+        return dot_entry(ctx, PK_SAME, ID, l, r, o, md, n);                                                    \
+    }
+HODU_ROCM_DEF_PRODUCT(f8e4m3, HODU_F8E4M3)
+HODU_ROCM_DEF_PRODUCT(f8e5m2, HODU_F8E5M2)
+HODU_ROCM_DEF_PRODUCT(bf16, HODU_BF16)
+HODU_ROCM_DEF_PRODUCT(f16, HODU_F16)
+HODU_ROCM_DEF_PRODUCT(f32, HODU_F32)
+HODU_ROCM_DEF_PRODUCT(f64, HODU_F64)
+HODU_ROCM_DEF_PRODUCT(u8, HODU_U8)
+HODU_ROCM_DEF_PRODUCT(u16, HODU_U16)
+HODU_ROCM_DEF_PRODUCT(u32, HODU_U32)
+HODU_ROCM_DEF_PRODUCT(u64, HODU_U64)
+HODU_ROCM_DEF_PRODUCT(i8, HODU_I8)
+HODU_ROCM_DEF_PRODUCT(i16, HODU_I16)
+HODU_ROCM_DEF_PRODUCT(i32, HODU_I32)
+HODU_ROCM_DEF_PRODUCT(i64, HODU_I64)
+
+int hodu_rocm_matmul_bf16_f8e4m3w(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,
+                                  size_t n) {
+    return matmul_entry(ctx, PK_BF16_F8W, HODU_BF16, l, r, o, md, n);
+}
+int hodu_rocm_dot_bf16_f8e4m3w(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,
+                               size_t n) {
+    return dot_entry(ctx, PK_BF16_F8W, HODU_BF16, l, r, o, md, n);
+}
+int hodu_rocm_matmul_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,
+                              size_t n) {
+    return matmul_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
+}
+int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md, size_t n) {
+    return dot_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
+}
+
+int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const size_t *md, size_t len) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "cast: context is null");
+    if (!in || !out) return fail(HODU_ROCM_INVALID_ARG, "cast: null operand pointer");
+    if (in == out) return fail(HODU_ROCM_INVALID_ARG, "cast: out aliases the input");
+    if (dtype_size(src) == 0 || dtype_size(dst) == 0)
+        return fail(HODU_ROCM_UNSUPPORTED, "cast: unknown dtype id (%d -> %d)", src, dst);
+    Strided s;
+    int rc = parse_cast_metadata(md, len, &s);
+    if (rc) return rc;
+    HODU_HIP(hipSetDevice(ctx->device));
+    return launch_cast(ctx, src, dst, in, out, s);
+}
+
+int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "contiguous: context is null");
+    if (!in || !out) return fail(HODU_ROCM_INVALID_ARG, "contiguous: null operand pointer");
+    if (in == out) return fail(HODU_ROCM_INVALID_ARG, "contiguous: out aliases the input");
+    if (dtype_size(dtype) == 0) return fail(HODU_ROCM_UNSUPPORTED, "contiguous: unknown dtype id %d", dtype);
+    Strided s;
+    int rc = parse_cast_metadata(md, len, &s);
+    if (rc) return rc;
+    HODU_HIP(hipSetDevice(ctx->device));
+    return launch_gather(ctx, dtype, in, out, s);
+}
+
+}  // extern "C"

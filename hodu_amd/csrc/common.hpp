@@ -1,0 +1,126 @@
+// Internal declarations shared by the translation units of libhodu_rocm_kernels.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "hodu_rocm_kernels.h"
+
+namespace hodu {
+
+// ------------------------------------------------------------------------------------------------
+// context
+// ------------------------------------------------------------------------------------------------
+struct Workspace {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+
+}  // namespace hodu
+
+struct hodu_rocm_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t props{};
+    hodu::Workspace workspace;  // split-K partial sums; grown on demand, owned by the context
+    const char *last_kernel = "";
+};
+
+namespace hodu {
+
+// per-thread error text (any host thread may call into one context)
+void set_error(const char *fmt, ...);
+const char *get_error();
+void clear_error();
+
+int fail(int code, const char *fmt, ...);
+
+#define HODU_HIP(expr)                                                                         \
+    do {                                                                                       \
+        hipError_t _e = (expr);                                                                \
+        if (_e != hipSuccess)                                                                  \
+            return ::hodu::fail(_e == hipErrorOutOfMemory ? HODU_ROCM_OOM : HODU_ROCM_HIP_ERROR, \
+                                "%s: %s", #expr, hipGetErrorString(_e));                       \
+    } while (0)
+
+// grows ctx->workspace to at least `bytes`
+int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes);
+
+inline size_t dtype_size(int dt) {
+    static const size_t sz[15] = {1, 1, 1, 2, 2, 4, 8, 1, 2, 4, 8, 1, 2, 4, 8};
+    return (dt >= 0 && dt < 15) ? sz[dt] : 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// parsed product problem: `batches` independent (M x K)(K x N) products
+// ------------------------------------------------------------------------------------------------
+constexpr int kMaxBatchDims = 16;  // the reference kernels index batch_indices[16] (ops_matrix.c:152)
+constexpr int kKernelBatchDims = 4; // innermost merged batch dims a single launch decomposes
+
+struct Product {
+    long M = 0, N = 0, K = 0;
+    long a_m = 0, a_k = 0, b_k = 0, b_n = 0;  // element strides of the two matrix dims
+    long a_off = 0, b_off = 0;                // element offsets
+    // batch space after merging: up to kMaxBatchDims dims, innermost last; stride 0 = broadcast
+    int nb = 0;
+    long bshape[kMaxBatchDims] = {};
+    long a_bs[kMaxBatchDims] = {};
+    long b_bs[kMaxBatchDims] = {};
+    long batches = 1;
+};
+
+// Validates and converts the reference's metadata vectors.  Returns a status code.
+int parse_matmul_metadata(const size_t *md, size_t len, Product *p);
+int parse_dot_metadata(const size_t *md, size_t len, Product *p);
+
+struct Strided {
+    long n = 0;
+    int nd = 0;
+    long shape[16];
+    long strides[16];
+    long offset = 0;
+    bool contiguous = false;  // reference rule: extent-1 dims do not constrain (utils.h:16-27)
+};
+int parse_cast_metadata(const size_t *md, size_t len, Strided *s);
+
+// What one launch needs to know about a product; passed by value as a kernel argument.
+struct DevProduct {
+    int M, N, K;
+    long a_m, a_k, b_k, b_n;
+    long a_off, b_off;
+    int nb;                        // batch dims decomposed by the kernel (<= kKernelBatchDims)
+    int bshape[kKernelBatchDims];  // innermost last
+    long a_bs[kKernelBatchDims];
+    long b_bs[kKernelBatchDims];
+    long batches;                  // product of bshape
+};
+
+// ------------------------------------------------------------------------------------------------
+// kernel families (each in its own .hip file)
+// ------------------------------------------------------------------------------------------------
+// "kind" of a product = (lhs storage, rhs storage, out) triple
+enum ProductKind {
+    PK_SAME = 0,     // all three share `dtype`
+    PK_BF16_F8W = 1, // bf16 x f8e4m3 -> bf16
+    PK_I32_I8I8 = 2  // i8 x i8 -> i32
+};
+
+// Each launcher handles one DevProduct whose output starts at `c` (batches * M * N elements).
+// generic strided kernel: every dtype, any strides; slow, always correct
+int launch_generic(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
+                   const DevProduct &g);
+// MFMA tile kernel: returns HODU_ROCM_UNSUPPORTED (without setting an error) when it has no variant
+int launch_mfma(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
+                const DevProduct &g);
+// bandwidth-bound small-M path: returns HODU_ROCM_UNSUPPORTED when not applicable
+int launch_skinny(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
+                  const DevProduct &g);
+
+int launch_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const Strided &s);
+int launch_gather(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Strided &s);
+
+}  // namespace hodu

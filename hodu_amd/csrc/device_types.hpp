@@ -1,0 +1,67 @@
+// Device-side element types, vector types and scalar conversions for gfx950.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "common.hpp"
+
+namespace hodu {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x2_t __attribute__((ext_vector_type(2)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
+// batch index -> element offsets of the two operands
+__device__ __forceinline__ void batch_offsets(const DevProduct &g, long batch, long &ao, long &bo) {
+    ao = g.a_off;
+    bo = g.b_off;
+#pragma unroll
+    for (int d = kKernelBatchDims - 1; d >= 0; d--) {
+        if (d < g.nb) {
+            const long i = batch % g.bshape[d];
+            batch /= g.bshape[d];
+            ao += i * g.a_bs[d];
+            bo += i * g.b_bs[d];
+        }
+    }
+}
+
+// ---- scalar conversions ---------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// round-to-nearest-even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits_rne(float f) {
+    __bf16 h = (__bf16)f;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t f32_to_f16_bits_rne(float f) {
+    _Float16 h = (_Float16)f;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// OCP E4M3FN / E5M2 decode in hardware (v_cvt_f32_fp8 / v_cvt_f32_bf8)
+__device__ __forceinline__ float f8e4m3_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
+__device__ __forceinline__ float f8e5m2_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_bf8((int)b, 0); }
+
+// round-to-nearest-even, saturating to the largest finite value, NaN stays NaN
+__device__ __forceinline__ uint8_t f32_to_f8e4m3_sat(float f) {
+    f = (f != f) ? f : fminf(fmaxf(f, -448.0f), 448.0f);
+    return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false) & 0xFF);
+}
+__device__ __forceinline__ uint8_t f32_to_f8e5m2_sat(float f) {
+    f = (f != f) ? f : fminf(fmaxf(f, -57344.0f), 57344.0f);
+    return (uint8_t)(__builtin_amdgcn_cvt_pk_bf8_f32(f, f, 0, false) & 0xFF);
+}
+
+}  // namespace hodu

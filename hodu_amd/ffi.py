@@ -1,0 +1,209 @@
+"""ctypes binding of include/hodu_rocm_kernels.h -- the same C ABI a Rust `hodu_rocm_kernels`
+crate would bind.  Loading fails loudly when the HIP library has not been built: there is no CPU
+fallback anywhere in this package.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhodu_rocm_kernels.so")
+
+OK, INVALID_ARG, UNSUPPORTED, HIP_ERROR, OOM = 0, 1, 2, 3, 4
+_STATUS = {1: "INVALID_ARG", 2: "UNSUPPORTED", 3: "HIP_ERROR", 4: "OOM"}
+
+# dtype ids: crates/hodu_core/src/types/dtype.rs:6-28
+DTYPE_ID = {
+    "bool": 0, "f8e4m3": 1, "f8e5m2": 2, "bf16": 3, "f16": 4, "f32": 5, "f64": 6,
+    "u8": 7, "u16": 8, "u32": 9, "u64": 10, "i8": 11, "i16": 12, "i32": 13, "i64": 14,
+}
+DTYPE_SIZE = {"bool": 1, "f8e4m3": 1, "f8e5m2": 1, "bf16": 2, "f16": 2, "f32": 4, "f64": 8, "u8": 1, "u16": 2,
+              "u32": 4, "u64": 8, "i8": 1, "i16": 2, "i32": 4, "i64": 8}
+PRODUCT_DTYPES = [d for d in DTYPE_ID if d != "bool"]
+FUSED_PRODUCTS = ("bf16_f8e4m3w", "i32_i8i8")
+
+
+class HoduRocmError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"hodu_rocm {_STATUS.get(status, status)}: {message}")
+        self.status = status
+        self.message = message
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the built HIP library; raises if it is missing (build with `python -m hodu_amd.build`)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build the HIP extension first (python -m hodu_amd.build). "
+            "hodu_amd has no CPU fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    szp = ctypes.POINTER(ctypes.c_size_t)
+    lib.hodu_rocm_device_count.argtypes = [ctypes.POINTER(ci)]
+    lib.hodu_rocm_ctx_create.argtypes = [ci, ctypes.POINTER(vp)]
+    lib.hodu_rocm_ctx_destroy.argtypes = [vp]
+    lib.hodu_rocm_alloc.argtypes = [vp, sz, ctypes.POINTER(vp)]
+    lib.hodu_rocm_free.argtypes = [vp, vp]
+    lib.hodu_rocm_memcpy_h2d.argtypes = [vp, vp, vp, sz]
+    lib.hodu_rocm_memcpy_d2h.argtypes = [vp, vp, vp, sz]
+    lib.hodu_rocm_memcpy_d2d.argtypes = [vp, vp, vp, sz]
+    lib.hodu_rocm_memset.argtypes = [vp, vp, ci, sz]
+    lib.hodu_rocm_sync.argtypes = [vp]
+    lib.hodu_rocm_last_error.argtypes = [vp]
+    lib.hodu_rocm_last_error.restype = ctypes.c_char_p
+    lib.hodu_rocm_last_kernel.argtypes = [vp]
+    lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
+    lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
+                                          ctypes.POINTER(sz)]
+    lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
+    lib.hodu_rocm_timer_start.argtypes = [vp, vp]
+    lib.hodu_rocm_timer_stop.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
+    lib.hodu_rocm_timer_destroy.argtypes = [vp, vp]
+    for dt in PRODUCT_DTYPES + list(FUSED_PRODUCTS):
+        for op in ("matmul", "dot"):
+            getattr(lib, f"hodu_rocm_{op}_{dt}").argtypes = [vp, vp, vp, vp, szp, sz]
+    lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
+    lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
+    _lib = lib
+    return lib
+
+
+def device_count() -> int:
+    n = ctypes.c_int(0)
+    load().hodu_rocm_device_count(ctypes.byref(n))
+    return n.value
+
+
+def _md_array(md: Sequence[int]):
+    arr = (ctypes.c_size_t * len(md))(*[int(v) for v in md])
+    return arr, len(md)
+
+
+class DeviceBuffer:
+    """A device allocation owned by a Context (what CudaSlice is to the CUDA sibling)."""
+
+    def __init__(self, ctx: "Context", nbytes: int):
+        self.ctx = ctx
+        self.nbytes = int(nbytes)
+        p = ctypes.c_void_p()
+        ctx._check(ctx.lib.hodu_rocm_alloc(ctx.handle, self.nbytes, ctypes.byref(p)))
+        self.ptr = p.value
+
+    def free(self):
+        if self.ptr is not None and self.ctx.handle is not None:
+            self.ctx.lib.hodu_rocm_free(self.ctx.handle, self.ptr)
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context:
+    """One device context: stream, allocations, kernel launches (hodu_rocm_ctx)."""
+
+    def __init__(self, device: int = 0):
+        self.lib = load()
+        h = ctypes.c_void_p()
+        rc = self.lib.hodu_rocm_ctx_create(int(device), ctypes.byref(h))
+        self.handle = h.value if rc == 0 else None
+        if rc != 0:
+            raise HoduRocmError(rc, self.lib.hodu_rocm_last_error(None).decode())
+        self.device = device
+
+    def close(self):
+        if self.handle is not None:
+            self.lib.hodu_rocm_ctx_destroy(self.handle)
+            self.handle = None
+
+    def _check(self, rc: int):
+        if rc != 0:
+            raise HoduRocmError(rc, self.lib.hodu_rocm_last_error(self.handle).decode())
+
+    # memory ---------------------------------------------------------------------------------
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        return DeviceBuffer(self, nbytes)
+
+    def upload(self, host: np.ndarray) -> DeviceBuffer:
+        host = np.ascontiguousarray(host)
+        buf = DeviceBuffer(self, host.nbytes)
+        self._check(self.lib.hodu_rocm_memcpy_h2d(self.handle, buf.ptr, host.ctypes.data, host.nbytes))
+        return buf
+
+    def download(self, buf: DeviceBuffer, dtype, count: Optional[int] = None) -> np.ndarray:
+        dtype = np.dtype(dtype)
+        n = buf.nbytes // dtype.itemsize if count is None else int(count)
+        out = np.empty(n, dtype=dtype)
+        self._check(self.lib.hodu_rocm_memcpy_d2h(self.handle, out.ctypes.data, buf.ptr, out.nbytes))
+        return out
+
+    def fill(self, buf: DeviceBuffer, byte: int):
+        self._check(self.lib.hodu_rocm_memset(self.handle, buf.ptr, int(byte), buf.nbytes))
+
+    def sync(self):
+        self._check(self.lib.hodu_rocm_sync(self.handle))
+
+    # compute --------------------------------------------------------------------------------
+    def product(self, op: str, name: str, lhs: DeviceBuffer, rhs: DeviceBuffer, out: DeviceBuffer, md):
+        """op in {'matmul','dot'}; name a dtype ('bf16') or a fused kind ('bf16_f8e4m3w')."""
+        arr, n = _md_array(md)
+        fn = getattr(self.lib, f"hodu_rocm_{op}_{name}")
+        self._check(fn(self.handle, lhs.ptr, rhs.ptr, out.ptr, arr, n))
+
+    def cast(self, src: str, dst: str, x: DeviceBuffer, out: DeviceBuffer, md):
+        arr, n = _md_array(md)
+        self._check(self.lib.hodu_rocm_cast(self.handle, DTYPE_ID[src], DTYPE_ID[dst], x.ptr, out.ptr, arr, n))
+
+    def contiguous(self, dt: str, x: DeviceBuffer, out: DeviceBuffer, md):
+        arr, n = _md_array(md)
+        self._check(self.lib.hodu_rocm_contiguous(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
+
+    def last_kernel(self) -> str:
+        return self.lib.hodu_rocm_last_kernel(self.handle).decode()
+
+    def device_info(self) -> dict:
+        name = ctypes.create_string_buffer(256)
+        cus, khz, mem = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+        self._check(self.lib.hodu_rocm_device_info(self.handle, name, 256, ctypes.byref(cus), ctypes.byref(khz),
+                                                   ctypes.byref(mem)))
+        return {"name": name.value.decode(), "compute_units": cus.value, "clock_khz": khz.value,
+                "total_mem": mem.value}
+
+    # timing ---------------------------------------------------------------------------------
+    def timer(self) -> "Timer":
+        return Timer(self)
+
+
+class Timer:
+    """HIP-event stopwatch on the context's stream."""
+
+    def __init__(self, ctx: Context):
+        self.ctx = ctx
+        h = ctypes.c_void_p()
+        ctx._check(ctx.lib.hodu_rocm_timer_create(ctx.handle, ctypes.byref(h)))
+        self.handle = h.value
+
+    def start(self):
+        self.ctx._check(self.ctx.lib.hodu_rocm_timer_start(self.ctx.handle, self.handle))
+
+    def stop_ms(self) -> float:
+        ms = ctypes.c_float()
+        self.ctx._check(self.ctx.lib.hodu_rocm_timer_stop(self.ctx.handle, self.handle, ctypes.byref(ms)))
+        return float(ms.value)
+
+    def close(self):
+        if self.handle is not None:
+            self.ctx.lib.hodu_rocm_timer_destroy(self.ctx.handle, self.handle)
+            self.handle = None

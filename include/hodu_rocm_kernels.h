@@ -1,0 +1,136 @@
+/*
+ * hodu_rocm_kernels.h -- C ABI of the MI355X (gfx950) matmul / dot / to_dtype / contiguous backend.
+ *
+ * This is the seam a `crates/hodu_rocm_kernels` FFI crate binds, a sibling of
+ * crates/hodu_cpu_kernels (plain C ABI) and crates/hodu_cuda_kernels.  Every compute entry point
+ * mirrors one reference kernel symbol:
+ *
+ *   hodu_cpu_matmul_<dt>(lhs, rhs, out, metadata)      kernels/ops_matrix.h:56-69
+ *   hodu_cpu_dot_<dt>(lhs, rhs, out, metadata)         kernels/ops_matrix.h:97-110
+ *   hodu_cpu_cast_<a>_to_<b>(in, out, metadata)        kernels/ops_cast.h:41-88
+ *   hodu_cpu_contiguous_<dt>(in, out, metadata)        kernels/ops_memory.h:44
+ *
+ * with three differences forced by the device: (1) a context handle comes first; (2) operand
+ * pointers are DEVICE pointers while `metadata` stays a HOST array of size_t in exactly the
+ * reference's formats (crates/hodu_core/src/op_metadatas.rs:192-291, :464-506, :1615-1656) and
+ * is parsed on the host -- it is never copied to the device (the CUDA sibling re-uploads it on
+ * every call, crates/hodu_cuda_kernels/src/kernels/ops_matrix.rs:372-374); (3) every call
+ * returns a status instead of void (the CPU kernels have no error channel,
+ * crates/hodu_cpu_kernels/src/kernels/ops_matrix.rs:56-68).
+ *
+ * Contract shared by all compute calls
+ *   - strides and offsets are in ELEMENTS; stride 0 broadcasts; operands may be transposed,
+ *     sliced or batch-broadcast views and are consumed in place (no contiguous copy);
+ *   - `out` is caller-allocated, contiguous, uninitialised (crates/hodu_core/src/be_cpu/device.rs:19-24)
+ *     and every element of it is written; it must not alias an input; inputs may alias each other;
+ *   - launches are asynchronous on the context's stream; hodu_rocm_sync and hodu_rocm_memcpy_d2h
+ *     synchronise;
+ *   - the library keeps no caller pointer after the call returns and never calls back.
+ */
+#ifndef HODU_ROCM_KERNELS_H
+#define HODU_ROCM_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hodu_rocm_ctx hodu_rocm_ctx;
+
+/* status codes (0 = ok).  Maps onto CudaKernelError::{InvalidInput, InvalidKernel, LaunchError,
+ * MemoryError} of crates/hodu_cuda_kernels/src/error.rs:7-18. */
+enum {
+    HODU_ROCM_OK = 0,
+    HODU_ROCM_INVALID_ARG = 1, /* null pointer, malformed or inconsistent metadata */
+    HODU_ROCM_UNSUPPORTED = 2, /* dtype / rank outside what the device implements */
+    HODU_ROCM_HIP_ERROR = 3,   /* a HIP runtime call failed; see hodu_rocm_last_error */
+    HODU_ROCM_OOM = 4          /* device allocation failed */
+};
+
+/* dtype ids, equal to hodu's repr(u8) DType (crates/hodu_core/src/types/dtype.rs:6-28) */
+enum {
+    HODU_BOOL = 0, HODU_F8E4M3 = 1, HODU_F8E5M2 = 2, HODU_BF16 = 3, HODU_F16 = 4, HODU_F32 = 5,
+    HODU_F64 = 6, HODU_U8 = 7, HODU_U16 = 8, HODU_U32 = 9, HODU_U64 = 10, HODU_I8 = 11,
+    HODU_I16 = 12, HODU_I32 = 13, HODU_I64 = 14
+};
+
+/* ---- runtime (replaces what cudarc gives the CUDA sibling: context, stream, slices;
+ *      crates/hodu_core/src/be_cuda/device.rs:20-65, be_cuda/storage.rs:165-173) ---------------- */
+int hodu_rocm_device_count(int *count);
+int hodu_rocm_ctx_create(int device, hodu_rocm_ctx **ctx);
+int hodu_rocm_ctx_destroy(hodu_rocm_ctx *ctx);
+int hodu_rocm_alloc(hodu_rocm_ctx *ctx, size_t bytes, void **dptr);
+int hodu_rocm_free(hodu_rocm_ctx *ctx, void *dptr);
+int hodu_rocm_memcpy_h2d(hodu_rocm_ctx *ctx, void *dst_device, const void *src_host, size_t bytes);
+int hodu_rocm_memcpy_d2h(hodu_rocm_ctx *ctx, void *dst_host, const void *src_device, size_t bytes);
+int hodu_rocm_memcpy_d2d(hodu_rocm_ctx *ctx, void *dst_device, const void *src_device, size_t bytes);
+int hodu_rocm_memset(hodu_rocm_ctx *ctx, void *dptr, int byte, size_t bytes);
+int hodu_rocm_sync(hodu_rocm_ctx *ctx);
+/* message of the last failing call made on this context by the calling thread ("" if none) */
+const char *hodu_rocm_last_error(hodu_rocm_ctx *ctx);
+/* device facts for roofline reporting: name (<=255 chars), compute units, clock (kHz), memory bytes */
+int hodu_rocm_device_info(hodu_rocm_ctx *ctx, char *name, size_t name_len, int *compute_units,
+                          int *clock_khz, size_t *total_mem);
+/* HIP-event stopwatch on the context's stream (the stream the kernels run on) */
+int hodu_rocm_timer_create(hodu_rocm_ctx *ctx, void **timer);
+int hodu_rocm_timer_start(hodu_rocm_ctx *ctx, void *timer);
+int hodu_rocm_timer_stop(hodu_rocm_ctx *ctx, void *timer, float *elapsed_ms); /* synchronises */
+int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
+/* name of the kernel family the last matmul/dot call on this context dispatched to (diagnostics) */
+const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
+
+/* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
+ * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>
+ * (kernels/ops_matrix.c:423, :581).  Narrow floats accumulate in f32 and round once on store.   */
+#define HODU_ROCM_DECL_PRODUCT(dt)                                                               \
+    int hodu_rocm_matmul_##dt(hodu_rocm_ctx *ctx, const void *lhs, const void *rhs, void *out,   \
+                              const size_t *metadata, size_t metadata_len);                      \
+    int hodu_rocm_dot_##dt(hodu_rocm_ctx *ctx, const void *lhs, const void *rhs, void *out,      \
+                           const size_t *metadata, size_t metadata_len);
+HODU_ROCM_DECL_PRODUCT(f8e4m3)
+HODU_ROCM_DECL_PRODUCT(f8e5m2)
+HODU_ROCM_DECL_PRODUCT(bf16)
+HODU_ROCM_DECL_PRODUCT(f16)
+HODU_ROCM_DECL_PRODUCT(f32)
+HODU_ROCM_DECL_PRODUCT(f64)
+HODU_ROCM_DECL_PRODUCT(u8)
+HODU_ROCM_DECL_PRODUCT(u16)
+HODU_ROCM_DECL_PRODUCT(u32)
+HODU_ROCM_DECL_PRODUCT(u64)
+HODU_ROCM_DECL_PRODUCT(i8)
+HODU_ROCM_DECL_PRODUCT(i16)
+HODU_ROCM_DECL_PRODUCT(i32)
+HODU_ROCM_DECL_PRODUCT(i64)
+
+/* ---- fused to_dtype + matmul / dot ------------------------------------------------------------ *
+ * `x.matmul(w8.to_dtype(bf16))`: Tensor::to_dtype (tensor/ops/cast_memory.rs:11-38) followed by
+ * Tensor::matmul (tensor/ops/matrix.rs:13-92) without materialising the cast.  The logical dtype
+ * contract of the product is unchanged (bf16 x bf16 -> bf16, i32 x i32 -> i32); only the physical
+ * storage of the named operand differs, and its metadata strides/offsets count ITS elements.
+ *   _bf16_f8e4m3w : lhs bf16, rhs stored f8e4m3 (OCP E4M3FN), out bf16
+ *   _i32_i8i8     : lhs and rhs stored i8 (sign-extended), out i32, wrap-around i32 arithmetic   */
+int hodu_rocm_matmul_bf16_f8e4m3w(hodu_rocm_ctx *ctx, const void *lhs_bf16, const void *rhs_f8e4m3,
+                                  void *out_bf16, const size_t *metadata, size_t metadata_len);
+int hodu_rocm_dot_bf16_f8e4m3w(hodu_rocm_ctx *ctx, const void *lhs_bf16, const void *rhs_f8e4m3,
+                               void *out_bf16, const size_t *metadata, size_t metadata_len);
+int hodu_rocm_matmul_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void *rhs_i8,
+                              void *out_i32, const size_t *metadata, size_t metadata_len);
+int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void *rhs_i8,
+                           void *out_i32, const size_t *metadata, size_t metadata_len);
+
+/* ---- casts and strided gather ------------------------------------------------------------------ *
+ * replaces hodu_cpu_cast_<src>_to_<dst> (kernels/ops_cast.c:53, table :108-388) and
+ * hodu_cpu_contiguous_<dt> (kernels/ops_memory.c:36).  One entry point taking dtype ids stands
+ * for the 225 + 15 symbols; a Rust wrapper maps the kernel-name string to the two ids the way
+ * crates/hodu_cpu_kernels/src/kernels/ops_cast.rs:70-81 maps it to a function pointer.           */
+int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src_dtype, int dst_dtype, const void *in, void *out,
+                   const size_t *metadata, size_t metadata_len);
+int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out,
+                         const size_t *metadata, size_t metadata_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HODU_ROCM_KERNELS_H */

@@ -1,0 +1,52 @@
+"""No-GPU checks of the C-ABI library: it loads, exports every symbol the header declares, and its
+host-side entry points fail with a status code (never a crash) when there is no device."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from hodu_amd import ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hodu_rocm_kernels.h")
+
+
+def declared_symbols():
+    text = subprocess.check_output(["gcc", "-E", "-P", HEADER], text=True)
+    return sorted(set(re.findall(r"\b(hodu_rocm_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ffi.load()
+    names = declared_symbols()
+    assert len(names) >= 50
+    for op in ("matmul", "dot"):
+        for dt in ffi.PRODUCT_DTYPES + list(ffi.FUSED_PRODUCTS):
+            assert f"hodu_rocm_{op}_{dt}" in names
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_header_compiles_as_c_and_cxx(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "hodu_rocm_kernels.h"\nint main(void){return HODU_ROCM_OK;}\n')
+    subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Werror", "-fsyntax-only", f"-I{ROOT}/include", str(src)])
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", f"-I{ROOT}/include", str(src)])
+
+
+def test_null_arguments_are_rejected_without_a_device():
+    lib = ffi.load()
+    md = (ctypes.c_size_t * 9)(2, 3, 2, 3, 1, 2, 1, 0, 0)
+    assert lib.hodu_rocm_dot_f32(None, None, None, None, md, 9) == ffi.INVALID_ARG
+    assert b"context is null" in lib.hodu_rocm_last_error(None)
+    assert lib.hodu_rocm_cast(None, 5, 3, None, None, md, 9) == ffi.INVALID_ARG
+    assert lib.hodu_rocm_ctx_create(0, None) == ffi.INVALID_ARG
+    assert lib.hodu_rocm_ctx_destroy(None) == ffi.OK
+
+
+@pytest.mark.skipif(ffi.device_count() > 0, reason="a GPU is present")
+def test_context_creation_fails_cleanly_without_a_gpu():
+    with pytest.raises(ffi.HoduRocmError):
+        ffi.Context(0)
