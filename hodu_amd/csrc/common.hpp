@@ -28,6 +28,7 @@ struct hodu_rocm_ctx {
     hipDeviceProp_t props{};
     hodu::Workspace workspace;  // split-K partial sums; grown on demand, owned by the context
     const char *last_kernel = "";
+    int force_tile = -1;  // testing hook: pins the MFMA tile size
 };
 
 namespace hodu {

@@ -165,6 +165,13 @@ const char *hodu_rocm_last_error(hodu_rocm_ctx *) { return get_error(); }
 
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
 
+int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
+    if (tile < -1 || tile > 2) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..2", tile);
+    ctx->force_tile = tile;
+    return HODU_ROCM_OK;
+}
+
 int hodu_rocm_device_info(hodu_rocm_ctx *ctx, char *name, size_t name_len, int *cus, int *clock_khz,
                           size_t *total_mem) {
     REQUIRE_CTX(ctx);

@@ -1,6 +1,168 @@
+// Bandwidth-bound products with at most 16 rows on the left (decode-shape GEMV / skinny GEMM):
+// y[m, n] = sum_k x[m, k] * W[n, k]  with the weight's k dense in memory -- the layout a Linear
+// layer hands over (`input.matmul(weight.transpose(-2, -1))`, crates/hodu_nn/src/modules/linear.rs:38-47).
+// Replaces the M < 512 single-thread paths of hodu_cpu_dot_<dt> (kernels/ops_matrix.c:486-548).
+//
+// The weight is the only operand that matters: every byte of it is read from HBM exactly once with
+// 128-bit loads, 16 consecutive k of one row per lane, four neighbouring lanes covering 64
+// contiguous bytes of that row.  Those 16 bytes ARE a lane's MFMA operand (k-packed), so the loaded
+// registers feed the matrix core directly (f8e4m3 weights pass through v_cvt_scalef32_pk_bf16_fp8
+// first) -- no LDS staging, no shuffles.  The left operand's rows occupy the MFMA's 16 m slots;
+// slots beyond M are zero, which costs nothing on a memory-bound kernel and makes M = 1..16 one
+// code path.
+//
+// Work split: a workgroup owns 16 weight rows (one MFMA column block); its 8 wavefronts split K, so
+// a 4096-wide row keeps 8 KB per wavefront in flight; partial sums meet in LDS (a wavefront-level
+// reduction per output element), are rounded once and stored.
 #include "common.hpp"
+#include "device_types.hpp"
+#include "gemm_mfma.hpp"
+
 namespace hodu {
-int launch_skinny(hodu_rocm_ctx *, int, int, const void *, const void *, void *, const DevProduct &) {
-    return HODU_ROCM_UNSUPPORTED;
+namespace {
+
+using mfma::bitcast;
+using mfma::CK_BF16;
+using mfma::CK_F16;
+using mfma::CK_F32;
+using mfma::CK_I8;
+using mfma::Compute;
+using mfma::Out;
+using mfma::SK_F8;
+using mfma::SK_SAME;
+
+constexpr int WAVES = 8;
+constexpr int UNROLL = 4;  // weight vectors in flight per lane
+
+__device__ __forceinline__ u32x4_t ldg16(const char *p) { return *reinterpret_cast<const u32x4_t *>(p); }
+
+// 16 f8e4m3 -> two chunks of 8 bf16 (exact)
+__device__ __forceinline__ void widen_f8x16(const u32x4_t &w, u32x4_t &lo, u32x4_t &hi) {
+    lo.x = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, false));
+    lo.y = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, true));
+    lo.z = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, false));
+    lo.w = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, true));
+    hi.x = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, false));
+    hi.y = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, true));
+    hi.z = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, false));
+    hi.w = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, true));
 }
+
+// CK: type fed to the matrix core; SKB: weight storage (CK itself, or f8e4m3 widened to bf16)
+template <int CK, int SKB, int OUT>
+__global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *__restrict__ X,
+                                                                  const char *__restrict__ W,
+                                                                  typename Out<OUT>::T *__restrict__ Y, DevProduct g,
+                                                                  int tiles_n, int k_per_wave) {
+    typedef Compute<CK> Cmp;
+    typedef typename Cmp::acc_t acc_t;
+    typedef typename Out<OUT>::T out_t;
+    constexpr int ES = Cmp::ES;                         // bytes per element of x (and of W unless f8)
+    constexpr int SB = SKB == SK_F8 ? 1 : ES;           // bytes per stored weight element
+    constexpr int EPL = 16 / SB;                        // weight elements per lane per load
+    __shared__ acc_t red[WAVES][64];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const long batch = blockIdx.x / tiles_n;
+    const int n0 = (int)(blockIdx.x % tiles_n) * 16;
+    long ao, bo;
+    batch_offsets(g, batch, ao, bo);
+
+    int n = n0 + lr;
+    n = n < g.N ? n : g.N - 1;
+    const char *wrow = W + (bo + (long)n * g.b_n) * SB;
+    const bool has_x = lr < g.M;
+    const char *xrow = X + (ao + (long)(has_x ? lr : 0) * g.a_m) * ES;
+
+    const int kbeg = wave * k_per_wave;
+    int kend = kbeg + k_per_wave;
+    kend = kend < g.K ? kend : g.K;
+
+    acc_t acc = acc_t{0, 0, 0, 0};
+    for (int kb = kbeg; kb < kend; kb += UNROLL * 4 * EPL) {
+        u32x4_t wv[UNROLL], xa[UNROLL], xb[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int k = kb + (u * 4 + lg) * EPL;
+            const bool ok = k < kend;
+            wv[u] = ok ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+            xa[u] = (ok && has_x) ? ldg16(xrow + (long)k * ES) : mfma::zero4();
+            if (SKB == SK_F8) xb[u] = (ok && has_x) ? ldg16(xrow + (long)(k + 8) * ES) : mfma::zero4();
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            if (SKB == SK_F8) {
+                u32x4_t lo, hi;
+                widen_f8x16(wv[u], lo, hi);
+                Cmp::mma(xa[u], lo, acc);
+                Cmp::mma(xb[u], hi, acc);
+            } else {
+                Cmp::mma(xa[u], wv[u], acc);
+            }
+        }
+    }
+
+    // lane holds y[m = 4*lg + e][n = n0 + lr] for e = 0..3 over this wavefront's k range
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (tid < 64) {
+        acc_t s = red[0][tid];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) {
+            const acc_t t = red[w][tid];
+            s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+        }
+        out_t *Yb = Y + batch * (long)g.M * g.N;
+        const int col = n0 + lr;
+        if (col < g.N) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int m = 4 * lg + e;
+                if (m < g.M) Yb[(long)m * g.N + col] = Out<OUT>::cvt(s[e]);
+            }
+        }
+    }
+}
+
+template <int CK, int SKB, int OUT>
+int run_kdense(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g, const char *name) {
+    constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB;
+    // applicability: both operands k-dense and every vector load 16-byte aligned
+    auto al = [](long elems, int bytes) { return (elems * bytes) % 16 == 0; };
+    if (g.M > 16 || g.K % EPL != 0 || g.K < 4 * EPL) return HODU_ROCM_UNSUPPORTED;
+    if (!(g.a_k == 1) || !(g.b_k == 1)) return HODU_ROCM_UNSUPPORTED;
+    if (!(g.M == 1 || al(g.a_m, ES)) || !(g.N == 1 || al(g.b_n, SB))) return HODU_ROCM_UNSUPPORTED;
+    if (((uintptr_t)x + (uintptr_t)g.a_off * ES) % 16 || ((uintptr_t)w + (uintptr_t)g.b_off * SB) % 16)
+        return HODU_ROCM_UNSUPPORTED;
+    for (int d = 0; d < g.nb; d++)
+        if (!al(g.a_bs[d], ES) || !al(g.b_bs[d], SB)) return HODU_ROCM_UNSUPPORTED;
+
+    const int tiles_n = (g.N + 15) / 16;
+    const long blocks = g.batches * tiles_n;
+    if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
+    const int step = 4 * EPL;  // k covered by one wavefront-wide load
+    int k_per_wave = ((g.K + WAVES - 1) / WAVES + step - 1) / step * step;
+    ctx->last_kernel = name;
+    hipLaunchKernelGGL((skinny_kdense_kernel<CK, SKB, OUT>), dim3((unsigned)blocks), dim3(WAVES * 64), 0, ctx->stream,
+                       (const char *)x, (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
+}  // namespace
+
+int launch_skinny(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
+                  const DevProduct &g) {
+    if (g.M > 16 || g.K == 0) return HODU_ROCM_UNSUPPORTED;
+    if (kind == PK_BF16_F8W) return run_kdense<CK_BF16, SK_F8, mfma::OUT_BF16>(ctx, a, b, c, g, "skinny_bf16_f8w");
+    if (kind == PK_I32_I8I8) return run_kdense<CK_I8, SK_SAME, mfma::OUT_I32>(ctx, a, b, c, g, "skinny_i32_i8i8");
+    switch (dtype) {
+    case HODU_BF16: return run_kdense<CK_BF16, SK_SAME, mfma::OUT_BF16>(ctx, a, b, c, g, "skinny_bf16");
+    case HODU_F16: return run_kdense<CK_F16, SK_SAME, mfma::OUT_F16>(ctx, a, b, c, g, "skinny_f16");
+    case HODU_F32: return run_kdense<CK_F32, SK_SAME, mfma::OUT_F32>(ctx, a, b, c, g, "skinny_f32");
+    default: return HODU_ROCM_UNSUPPORTED;
+    }
+}
+
 }  // namespace hodu

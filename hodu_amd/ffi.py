@@ -63,6 +63,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_last_error.restype = ctypes.c_char_p
     lib.hodu_rocm_last_kernel.argtypes = [vp]
     lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
+    lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
     lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
                                           ctypes.POINTER(sz)]
     lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
@@ -169,6 +170,10 @@ class Context:
     def contiguous(self, dt: str, x: DeviceBuffer, out: DeviceBuffer, md):
         arr, n = _md_array(md)
         self._check(self.lib.hodu_rocm_contiguous(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
+
+    def force_tile(self, tile: int):
+        """testing hook: 0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic"""
+        self._check(self.lib.hodu_rocm_debug_force_tile(self.handle, int(tile)))
 
     def last_kernel(self) -> str:
         return self.lib.hodu_rocm_last_kernel(self.handle).decode()

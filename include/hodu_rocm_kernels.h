@@ -80,6 +80,9 @@ int hodu_rocm_timer_stop(hodu_rocm_ctx *ctx, void *timer, float *elapsed_ms); /*
 int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
 /* name of the kernel family the last matmul/dot call on this context dispatched to (diagnostics) */
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
+/* testing hook: pin the MFMA output tile (0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic) so
+ * that every compiled variant can be exercised at small sizes */
+int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
 
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>

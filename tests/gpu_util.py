@@ -58,6 +58,17 @@ def check_product(ctx, op, name, lv, rv, seed=0, scale=1.0, rscale=None, expect_
             want = (oracle.dot_asis if op == "dot" else oracle.matmul_asis)(name, a, b, md)
         assert np.array_equal(got, want), f"{op} {name}: integer result differs"
         return
+    if out_dt == "f64":
+        # f64 has no narrower comparator: sequential-k f64 (the reference's own arithmetic) and
+        # sum|a b| from numpy
+        want = (oracle.dot_asis if op == "dot" else oracle.matmul_asis)("f64", a, b, md)
+        bshape = list(np.broadcast_shapes(tuple(lv.shape[:-2]), tuple(rv.shape[:-2])))
+        A = np.abs(lv.broadcast_to(bshape + lv.shape[-2:]).take(a)); B = np.abs(rv.broadcast_to(bshape + rv.shape[-2:]).take(b))
+        oabs = (A @ B).ravel()
+        assert np.all(np.isfinite(got))
+        rel = H.rel_err(got, want, oabs, k)
+        assert rel.max() <= 1e-12, f"{op} f64: max rel err {rel.max():.3e}"
+        return
     fn = oracle.dot_spec if op == "dot" else oracle.matmul_spec
     o32, o64, oabs = fn(l_dt, r_dt, a, b, md)
     gotf = H.widen(out_dt, got)

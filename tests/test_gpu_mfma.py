@@ -1,0 +1,88 @@
+"""GPU parity of the MFMA tile kernels: every compiled variant (dtype kind x tile x load-mode pair)
+is driven through the C ABI at ragged sizes and compared with the oracle."""
+import numpy as np
+import pytest
+
+import helpers as H
+from gpu_util import check_product
+from hodu_amd import ffi
+
+pytestmark = pytest.mark.gpu
+V = H.View
+
+KINDS = {
+    # name: (kernel prefix, K multiple for the k-dense path, row multiple for the row-dense path)
+    "bf16": ("mfma_bf16", 8, 8),
+    "f16": ("mfma_f16", 8, 8),
+    "f32": ("mfma_f32", 4, 4),
+    "bf16_f8e4m3w": ("mfma_bf16_f8w", 8, 8),
+    "i32_i8i8": ("mfma_i32_i8i8", 16, 8),
+}
+TILES = {0: "256x256", 1: "128x128", 2: "64x64"}
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = ffi.Context(0)
+    yield c
+    c.force_tile(-1)
+    c.close()
+
+
+def views(combo, M, K, N):
+    lv = V([M, K]) if combo[0] == "K" else V([K, M]).t()
+    rv = V([N, K]).t() if combo[1] == "K" else V([K, N])
+    return lv, rv
+
+
+@pytest.mark.parametrize("kind", list(KINDS))
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_every_variant_ragged(ctx, kind, tile):
+    prefix, kmul, rmul = KINDS[kind]
+    ctx.force_tile(tile)
+    M, N, K = 296, 200, 9 * 16  # M, N not multiples of any tile; K = 144 leaves a ragged last K step
+    scale = 1.0
+    for combo in ("KK", "KM", "MK", "MM"):
+        lv, rv = views(combo, M, K, N)
+        check_product(ctx, "dot", kind, lv, rv, seed=tile, scale=scale, rscale=2.0 if "f8" in kind else None,
+                      expect_kernel=f"{prefix}_{TILES[tile]}_{combo}")
+    ctx.force_tile(-1)
+
+
+@pytest.mark.parametrize("kind", list(KINDS))
+def test_scalar_load_variant(ctx, kind):
+    prefix, _, _ = KINDS[kind]
+    # odd K, odd strides, odd offsets: nothing is vector-loadable
+    lv = V([45, 77], offset=1)
+    rv = V([77, 2 * 31]).slice(1, 1, 62, 2)
+    check_product(ctx, "dot", kind, lv, rv, seed=3, rscale=2.0 if "f8" in kind else None,
+                  expect_kernel=f"{prefix}_64x64_scalar")
+
+
+@pytest.mark.parametrize("kind", list(KINDS))
+def test_batched_and_broadcast(ctx, kind):
+    prefix, _, _ = KINDS[kind]
+    rs = 2.0 if "f8" in kind else None
+    # strided batch on both sides, rhs a transposed view (BASELINE config 2 in small)
+    check_product(ctx, "matmul", kind, V([3, 72, 64]), V([3, 80, 64]).t(), seed=11, rscale=rs, expect_kernel=prefix)
+    # weight shared across the batch (stride 0) and transposed: folds into one tall product
+    check_product(ctx, "matmul", kind, V([4, 40, 96]), V([56, 96]).t().broadcast_to([4, 96, 56]), seed=12, rscale=rs,
+                  expect_kernel=prefix)
+    # 2-D rhs, two batch dims on the lhs
+    check_product(ctx, "matmul", kind, V([2, 3, 24, 32]), V([32, 40]), seed=13, rscale=rs, expect_kernel=prefix)
+    # lhs broadcast over the batch, batched rhs (cannot fold: stays batched with a stride-0 operand)
+    check_product(ctx, "matmul", kind, V([24, 32]).broadcast_to([3, 24, 32]), V([3, 32, 40]), seed=14, rscale=rs,
+                  expect_kernel=prefix)
+    # aligned offsets into larger buffers
+    check_product(ctx, "dot", kind, V([40, 64], offset=64), V([64, 48], offset=128), seed=15, rscale=rs,
+                  expect_kernel=prefix)
+    # row slices: leading dimension larger than the extent
+    check_product(ctx, "dot", kind, V([40, 128]).slice(1, 32, 96), V([64, 96]).slice(1, 16, 64), seed=16, rscale=rs,
+                  expect_kernel=prefix)
+
+
+def test_deep_k_accumulation(ctx):
+    """K = 4096 products at ordinary magnitudes: f32 accumulation keeps bf16 results inside 2e-2"""
+    check_product(ctx, "dot", "bf16", V([64, 4096]), V([96, 4096]).t(), seed=21, scale=1.0)
+    check_product(ctx, "dot", "f32", V([64, 4096]), V([4096, 96]), seed=22, scale=1.0)
+    check_product(ctx, "dot", "bf16_f8e4m3w", V([64, 4096]), V([96, 4096]).t(), seed=23, scale=1.0, rscale=100.0)
