@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X matmul / dot / to_dtype backend on BASELINE.json's five configurations.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c1,c2,c3,c4,c5] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of synthetic input: one matmul/dot call through
+the C ABI with operands resident in HBM.  The headline (`value`, `roofline`, `cpu_baseline`) is
+BASELINE.json configs[1]: bf16 batched matmul [16,1024,1024] x [16,1024,1024] with the right
+operand a transposed view.  Every other configuration is measured in the same run and reported
+under "all_configs" with its own roofline fraction (TFLOP/s against the MFMA dense peak of the
+type the matrix cores consume, GB/s against HBM peak for the M <= 16 GEMV shapes).
+
+Timing: HIP events recorded on the stream the kernels are launched on (the context's stream),
+W untimed warm-up launches, then K launches back to back; `achieved` = algorithmic flops (or
+bytes) per launch / average launch duration.  The GEMV configurations rotate through enough
+distinct weight buffers to exceed the 256 MB Infinity Cache so that reads come from HBM.
+
+cpu_baseline: the oracle (a restatement of hodu's CPU kernels, kind "port") timed on this host on
+a bounded sample of the same workload, under the reference's own threading policy.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+# published MI355X peaks (dense)
+PEAK = {"bf16": 2500.0, "f16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}  # TFLOP/s or TOP/s
+HBM_PEAK_GBS = 8000.0
+INFINITY_CACHE_BYTES = 256 << 20
+
+# HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc runs summarised under
+# profiles/ (FETCH_SIZE + WRITE_SIZE scaled by the copy-kernel calibration); None = not measured
+MEASURED_TRAFFIC = {}
+
+
+def bf16(x):
+    import helpers as H
+    return H.f32_to_bf16_rne(np.asarray(x, dtype=np.float32))
+
+
+def normal(seed, n, scale=1.0):
+    g = np.random.default_rng(seed)
+    out = g.standard_normal(n, dtype=np.float32)
+    if scale != 1.0:
+        out *= np.float32(scale)
+    return out
+
+
+def fp8_weights(seed, n, top=448.0):
+    import helpers as H
+    w = normal(seed, n, 0.02)
+    s = top / float(np.abs(w).max())
+    return H.f32_to_ocp_e4m3_rne(np.clip(w * s, -448, 448))
+
+
+class Case:
+    """one timed launch shape"""
+
+    def __init__(self, key, label, op, name, lv, rv, make_a, make_b, flops, alg_bytes, bound, peak_key, rotate=False):
+        self.key, self.label, self.op, self.name = key, label, op, name
+        self.lv, self.rv, self.make_a, self.make_b = lv, rv, make_a, make_b
+        self.flops, self.alg_bytes, self.bound, self.peak_key, self.rotate = flops, alg_bytes, bound, peak_key, rotate
+
+
+def build_cases(which):
+    import helpers as H
+    V = H.View
+    cases = []
+    if "c1" in which:
+        n = 512
+        cases.append(Case("c1", "C1 f32 dot 512x512x512", "dot", "f32", V([n, n]), V([n, n]),
+                          lambda n=n: normal(101, n * n), lambda n=n: normal(102, n * n),
+                          2.0 * n ** 3, 3 * n * n * 4, "mfma", "f32"))
+    if "c2" in which:
+        B, n = 16, 1024
+        cases.append(Case("c2", "C2 bf16 matmul [16,1024,1024]x[16,1024,1024]^T-view", "matmul", "bf16",
+                          V([B, n, n]), V([B, n, n]).t(),
+                          lambda B=B, n=n: bf16(normal(201, B * n * n, 1 / 32)),
+                          lambda B=B, n=n: bf16(normal(202, B * n * n, 1 / 32)),
+                          2.0 * B * n ** 3, 3 * B * n * n * 2, "mfma", "bf16"))
+    if "c3" in which:
+        n = k = 4096
+        for m in (1, 16, 256, 4096):
+            cases.append(Case(f"c3_m{m}", f"C3 bf16[{m},4096] x f8e4m3[4096,4096]^T-view (fused to_dtype)", "dot",
+                              "bf16_f8e4m3w", V([m, k]), V([n, k]).t(),
+                              (lambda m=m, k=k: bf16(normal(302, m * k))), (lambda n=n, k=k: fp8_weights(301, n * k)),
+                              2.0 * m * n * k, n * k + m * k * 2 + m * n * 2,
+                              "hbm" if m <= 16 else "mfma", "bf16", rotate=(m <= 16)))
+    if "c4" in which:
+        n = 2048
+        ints = lambda seed, n=n: np.random.default_rng(seed).integers(-127, 128, n * n).astype(np.int8)  # noqa: E731
+        cases.append(Case("c4", "C4 i8-valued i32 dot 2048^3 (fused to_dtype)", "dot", "i32_i8i8", V([n, n]), V([n, n]),
+                          lambda: ints(401), lambda: ints(402), 2.0 * n ** 3, 2 * n * n + n * n * 4, "mfma", "int8"))
+    if "c5" in which:
+        b, s, d, f = 8, 512, 4096, 14336
+        for wk in ("bf16", "f8e4m3"):
+            name = "bf16" if wk == "bf16" else "bf16_f8e4m3w"
+            wbytes = d * f * (2 if wk == "bf16" else 1)
+            mk_w = (lambda seed, d=d, f=f: (lambda: bf16(normal(seed, d * f, 0.02)))) if wk == "bf16" else \
+                (lambda seed, d=d, f=f: (lambda: fp8_weights(seed, d * f)))
+            cases.append(Case(f"c5_up_{wk}", f"C5 up   bf16[8,512,4096] x {wk}[4096,14336] (batch-broadcast)", "matmul",
+                              name, V([b, s, d]), V([d, f]).broadcast_to([b, d, f]),
+                              lambda b=b, s=s, d=d: bf16(normal(501, b * s * d)), mk_w(502),
+                              2.0 * b * s * d * f, b * s * d * 2 + wbytes + b * s * f * 2, "mfma", "bf16"))
+            cases.append(Case(f"c5_down_{wk}", f"C5 down bf16[8,512,14336] x {wk}[4096,14336]^T-view (batch-broadcast)",
+                              "matmul", name, V([b, s, f]), V([d, f]).t().broadcast_to([b, f, d]),
+                              lambda b=b, s=s, f=f: bf16(normal(504, b * s * f, 0.3)), mk_w(503),
+                              2.0 * b * s * d * f, b * s * f * 2 + wbytes + b * s * d * 2, "mfma", "bf16"))
+    return cases
+
+
+def out_bytes(case):
+    import helpers as H
+    md = H.dot_md(case.lv, case.rv) if case.op == "dot" else H.matmul_md(case.lv, case.rv)
+    n = md[0] * md[2] if case.op == "dot" else md[0]
+    return md, n * {"f32": 4, "bf16": 2, "bf16_f8e4m3w": 2, "i32_i8i8": 4}[case.name]
+
+
+def time_case(ctx, case, steps, warmup):
+    """returns a result dict; operands are uploaded before the timed region starts"""
+    md, obytes = out_bytes(case)
+    a = ctx.upload(case.make_a())
+    w_host = case.make_b()
+    copies = 1
+    if case.rotate:
+        copies = max(2, int(3 * INFINITY_CACHE_BYTES // max(w_host.nbytes, 1)) + 1)
+    ws = [ctx.upload(w_host)]
+    for i in range(1, copies):
+        # distinct buffers with the same contents: what matters is that the addresses differ
+        extra = ctx.alloc(w_host.nbytes)
+        ctx.lib.hodu_rocm_memcpy_d2d(ctx.handle, extra.ptr, ws[0].ptr, w_host.nbytes)
+        ws.append(extra)
+    out = ctx.alloc(obytes)
+    ctx.sync()
+    for i in range(warmup):
+        ctx.product(case.op, case.name, a, ws[i % copies], out, md)
+    ctx.sync()
+    kernel = ctx.last_kernel()
+    # the K timed launches are issued back to back from C (hodu_rocm_debug_time_product) so that a
+    # 3 us GEMV is not hidden behind the interpreter's per-call cost; HIP events on the same stream
+    ms = ctx.time_product(case.op, case.name, a, ws, out, md, steps)
+    for buf in [a, out] + ws:
+        buf.free()
+    per_launch_s = ms / 1e3 / steps
+    tflops = case.flops / per_launch_s / 1e12
+    gbs = case.alg_bytes / per_launch_s / 1e9
+    if case.bound == "hbm":
+        roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}
+    else:
+        peak = PEAK[case.peak_key]
+        roof = {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak}
+    roof["traffic"] = MEASURED_TRAFFIC.get(f"{kernel}@{case.key}")
+    roof["kernel"] = kernel
+    return {"config": case.key, "label": case.label, "kernel": kernel, "us_per_launch": per_launch_s * 1e6,
+            "tflops": tflops, "algorithmic_gbs": gbs, "weight_buffers_rotated": copies, "roofline": roof}
+
+
+def cpu_baseline_c2(budget_s=12.0):
+    """hodu's CPU path for config 2, timed on a bounded sample.
+
+    hodu routes a >= 3-D matmul to hodu_cpu_matmul_bf16, whose batched path runs on ONE thread and
+    accumulates in bf16 (crates/hodu_cpu_kernels/kernels/ops_matrix.c:292-337); through the public
+    API the transposed operand is first copied (tensor/ops/shape.rs:232-237), which is not timed.
+    The sample is the first `rows` rows of batch 0 against the full [1024,1024] right operand;
+    the rate is per flop, so it scales linearly to the whole job.
+    """
+    import helpers as H
+    import oracle
+    n = 1024
+    a = bf16(normal(201, n * n, 1 / 32))
+    b = bf16(normal(202, n * n, 1 / 32))
+    oracle.set_threads(1)
+    rows, rate = 8, None
+    t_used = 0.0
+    while True:
+        lv, rv = H.View([1, rows, n]), H.View([1, n, n]).t()
+        t0 = time.perf_counter()
+        oracle.matmul_asis("bf16", a, b, H.matmul_md(lv, rv))
+        dt = time.perf_counter() - t0
+        t_used += dt
+        rate = 2.0 * rows * n * n / dt
+        nxt = min(n, int(rows * min(8.0, max(2.0, (budget_s - t_used) / max(dt, 1e-6) * 0.5))))
+        if t_used + dt * nxt / rows > budget_s or rows >= n or nxt <= rows:
+            break
+        rows = nxt
+    # the f32-accumulated comparator path (to_dtype(f32) + sgemm), all cores, for scale
+    af = H.bf16_to_f32(a).reshape(n, n)
+    bfm = H.bf16_to_f32(b).reshape(n, n)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 1.5:
+        af @ bfm.T
+        reps += 1
+    sgemm_rate = 2.0 * n ** 3 * reps / (time.perf_counter() - t0)
+    oracle.set_threads(os.cpu_count() or 1)
+    return {"value": rate / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"hodu_cpu_matmul_bf16 semantics (bf16-accumulate, batched path, 1 thread) on {rows} of 1024 rows "
+                      f"of batch 0 x full [1024,1024]^T-view; {t_used:.1f} s of CPU work",
+            "host_cores_online": os.cpu_count(),
+            "f32_comparator_sgemm_tflops": sgemm_rate / 1e12,
+            "f32_comparator_note": "to_dtype(f32) inputs through numpy's OpenBLAS sgemm on all host cores (1024^3)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; every GPU box here has one GPU and no collective or sharded "
+              "path exists in this round (the design for sharding is in DESIGN.md). Re-run with --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    from hodu_amd import ffi
+    ctx = ffi.Context(0)
+    info = ctx.device_info()
+    which = set(args.configs.split(",")) | {"c2"}
+    results = []
+    for case in build_cases(which):
+        steps = args.steps if case.flops < 4e11 else max(5, args.steps // 5)
+        results.append(time_case(ctx, case, steps, args.warmup))
+        print(f"# {results[-1]['label']}: {results[-1]['us_per_launch']:.1f} us  {results[-1]['tflops']:.1f} TFLOP/s  "
+              f"{results[-1]['algorithmic_gbs']:.0f} GB/s  [{results[-1]['kernel']}] "
+              f"{100 * results[-1]['roofline']['frac']:.1f}% of {results[-1]['roofline']['bound']} peak",
+              file=sys.stderr, flush=True)
+    head = next(r for r in results if r["config"] == "c2")
+    # the headline is re-timed with exactly the requested step count
+    case2 = [c for c in build_cases({"c2"})][0]
+    head = time_case(ctx, case2, args.steps, args.warmup)
+    line = {
+        "metric": "TFLOP/s & % MFMA peak per dtype; M=1 GEMV GB/s & % HBM peak",
+        "value": head["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["us_per_launch"] / 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: bf16 batched matmul A[16,1024,1024] x B[16,1024,1024], "
+                               "B a transposed (non-contiguous) view, f32 accumulate, bf16 out; one matmul call per step",
+                   "flop_per_step": case2.flops, "algorithmic_bytes_per_step": case2.alg_bytes},
+        "roofline": {k: head["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+        "dominant_kernel": head["kernel"],
+        "device": info,
+        "all_configs": results,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_c2()
+    ctx.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

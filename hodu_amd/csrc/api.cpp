@@ -137,6 +137,37 @@ int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, voi
     return dot_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
 }
 
+int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                 const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
+                                 int iters, float *elapsed_ms) {
+    clear_error();
+    if (!ctx || !rhs_list || n_rhs == 0 || !elapsed_ms || iters <= 0)
+        return fail(HODU_ROCM_INVALID_ARG, "time_product: bad argument");
+    if (kind < PK_SAME || kind > PK_I32_I8I8) return fail(HODU_ROCM_INVALID_ARG, "time_product: kind %d", kind);
+    for (size_t i = 0; i < n_rhs; i++) {
+        int rc = check_ptrs("time_product", ctx, lhs, rhs_list[i], out);
+        if (rc) return rc;
+    }
+    Product p;
+    int rc = is_matmul ? parse_matmul_metadata(md, len, &p) : parse_dot_metadata(md, len, &p);
+    if (rc) return rc;
+    HODU_HIP(hipSetDevice(ctx->device));
+    hipEvent_t t0, t1;
+    HODU_HIP(hipEventCreate(&t0));
+    HODU_HIP(hipEventCreate(&t1));
+    HODU_HIP(hipEventRecord(t0, ctx->stream));
+    for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
+        rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p);
+    hipError_t e = hipEventRecord(t1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_product: %s", hipGetErrorString(e));
+    return HODU_ROCM_OK;
+}
+
 int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "cast: context is null");

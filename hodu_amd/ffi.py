@@ -64,6 +64,8 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_last_kernel.argtypes = [vp]
     lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
     lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
+    lib.hodu_rocm_debug_time_product.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz, ci,
+                                                 ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
                                           ctypes.POINTER(sz)]
     lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
@@ -83,6 +85,37 @@ def device_count() -> int:
     n = ctypes.c_int(0)
     load().hodu_rocm_device_count(ctypes.byref(n))
     return n.value
+
+
+def _view_span(shape, strides, offset) -> int:
+    """elements a strided view can touch: highest index + 1 (0 for an empty view)"""
+    if any(int(d) == 0 for d in shape):
+        return 0
+    return int(offset) + sum((int(d) - 1) * int(s) for d, s in zip(shape, strides)) + 1
+
+
+def product_spans(op: str, md: Sequence[int]):
+    """(lhs elements, rhs elements, out elements) a matmul / dot metadata vector addresses.
+
+    The C ABI receives bare pointers, as the reference's kernels do, so the extents of the buffers
+    behind them can only be checked by the caller that owns them; this is that check."""
+    md = [int(v) for v in md]
+    if op == "dot":
+        if len(md) != 9:
+            return None
+        m, k, n, am, ak, bk, bn, ao, bo = md
+        return _view_span([m, k], [am, ak], ao), _view_span([k, n], [bk, bn], bo), m * n
+    if len(md) < 4:
+        return None
+    lnd, rnd, bnd = md[1], md[2], md[3]
+    if len(md) != 4 + 2 * lnd + 2 * rnd + bnd + 5:
+        return None
+    ls = md[4:4 + lnd]
+    rs = md[4 + lnd:4 + lnd + rnd]
+    p = 4 + lnd + rnd + bnd
+    lst, rst = md[p:p + lnd], md[p + lnd:p + lnd + rnd]
+    lo, ro = md[p + lnd + rnd], md[p + lnd + rnd + 1]
+    return _view_span(ls, lst, lo), _view_span(rs, rst, ro), md[0]
 
 
 def _md_array(md: Sequence[int]):
@@ -159,17 +192,57 @@ class Context:
     # compute --------------------------------------------------------------------------------
     def product(self, op: str, name: str, lhs: DeviceBuffer, rhs: DeviceBuffer, out: DeviceBuffer, md):
         """op in {'matmul','dot'}; name a dtype ('bf16') or a fused kind ('bf16_f8e4m3w')."""
+        self._check_extents(op, name, lhs, [rhs], out, md)
         arr, n = _md_array(md)
         fn = getattr(self.lib, f"hodu_rocm_{op}_{name}")
         self._check(fn(self.handle, lhs.ptr, rhs.ptr, out.ptr, arr, n))
 
+    @staticmethod
+    def _check_extents(op, name, lhs, rhs_list, out, md):
+        """refuse a launch whose metadata reaches past one of the device buffers"""
+        spans = product_spans(op, md)
+        if spans is None:
+            return  # malformed metadata: the library reports it
+        l_sz, r_sz, o_sz = {"bf16_f8e4m3w": (2, 1, 2), "i32_i8i8": (1, 1, 4)}.get(name) or (DTYPE_SIZE[name],) * 3
+        need = [("lhs", lhs, spans[0] * l_sz), ("out", out, spans[2] * o_sz)] + \
+               [("rhs", r, spans[1] * r_sz) for r in rhs_list]
+        for what, buf, nbytes in need:
+            if nbytes > buf.nbytes:
+                raise HoduRocmError(INVALID_ARG, f"{op}_{name}: metadata addresses {nbytes} bytes of {what} "
+                                                 f"but the buffer holds {buf.nbytes}")
+
+    @staticmethod
+    def _check_strided(what, src_size, dst_size, x, out, md):
+        md = [int(v) for v in md]
+        if len(md) < 2 or len(md) != 2 + 2 * md[1] + 1:
+            return
+        nd = md[1]
+        span = _view_span(md[2:2 + nd], md[2 + nd:2 + 2 * nd], md[2 + 2 * nd])
+        if span * src_size > x.nbytes or md[0] * dst_size > out.nbytes:
+            raise HoduRocmError(INVALID_ARG, f"{what}: metadata reaches past a device buffer")
+
     def cast(self, src: str, dst: str, x: DeviceBuffer, out: DeviceBuffer, md):
+        self._check_strided(f"cast_{src}_to_{dst}", DTYPE_SIZE[src], DTYPE_SIZE[dst], x, out, md)
         arr, n = _md_array(md)
         self._check(self.lib.hodu_rocm_cast(self.handle, DTYPE_ID[src], DTYPE_ID[dst], x.ptr, out.ptr, arr, n))
 
     def contiguous(self, dt: str, x: DeviceBuffer, out: DeviceBuffer, md):
+        self._check_strided(f"contiguous_{dt}", DTYPE_SIZE[dt], DTYPE_SIZE[dt], x, out, md)
         arr, n = _md_array(md)
         self._check(self.lib.hodu_rocm_contiguous(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
+
+    def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int) -> float:
+        """back-to-back launches issued from C, HIP-event timed on the context's stream; total ms"""
+        self._check_extents(op, name, lhs, rhs_list, out, md)
+        kind = {"bf16_f8e4m3w": 1, "i32_i8i8": 2}.get(name, 0)
+        dtype = DTYPE_ID["bf16"] if kind == 1 else DTYPE_ID["i32"] if kind == 2 else DTYPE_ID[name]
+        arr, n = _md_array(md)
+        ptrs = (ctypes.c_void_p * len(rhs_list))(*[b.ptr for b in rhs_list])
+        ms = ctypes.c_float()
+        self._check(self.lib.hodu_rocm_debug_time_product(self.handle, 1 if op == "matmul" else 0, kind, dtype,
+                                                          lhs.ptr, ptrs, len(rhs_list), out.ptr, arr, n, int(iters),
+                                                          ctypes.byref(ms)))
+        return float(ms.value)
 
     def force_tile(self, tile: int):
         """testing hook: 0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic"""

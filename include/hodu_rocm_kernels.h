@@ -83,6 +83,13 @@ const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
 /* testing hook: pin the MFMA output tile (0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic) so
  * that every compiled variant can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
+/* measurement hook: issues the same product `iters` times back to back from C (no per-launch
+ * interpreter overhead), cycling through `n_rhs` right-hand buffers so a small operand cannot sit
+ * in the Infinity Cache, bracketed by HIP events on the context's stream; *elapsed_ms is the total.
+ * is_matmul selects the metadata format; kind: 0 = plain `dtype`, 1 = bf16 x f8e4m3, 2 = i8 x i8 -> i32 */
+int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                 const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
+                                 size_t metadata_len, int iters, float *elapsed_ms);
 
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>

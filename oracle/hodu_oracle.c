@@ -447,15 +447,23 @@ static int spec_run(int l_dt, int r_dt, int f8_decode, const void *lhs, const vo
                 for (size_t j = 0; j < N; j++) o[j] += av * brow[j];
             }
             if (out64 || outabs) {
-                for (size_t j = 0; j < N; j++) {
-                    double s = 0.0, sa = 0.0;
-                    for (size_t k = 0; k < K; k++) {
-                        double p = (double)A[i * K + k] * (double)B[k * N + j];
-                        s += p; sa += fabs(p);
+                /* same i-k-j order in f64: row-wise passes over B keep the oracle fast */
+                double *s = (double *)calloc(2 * (N + 1), sizeof(double));
+                double *sa = s + N + 1;
+                for (size_t k = 0; k < K; k++) {
+                    const double av = (double)A[i * K + k];
+                    const float *brow = B + k * N;
+                    for (size_t j = 0; j < N; j++) {
+                        const double p = av * (double)brow[j];
+                        s[j] += p;
+                        sa[j] += fabs(p);
                     }
-                    if (out64) out64[bt * MN + i * N + j] = s;
-                    if (outabs) outabs[bt * MN + i * N + j] = sa;
                 }
+                for (size_t j = 0; j < N; j++) {
+                    if (out64) out64[bt * MN + i * N + j] = s[j];
+                    if (outabs) outabs[bt * MN + i * N + j] = sa[j];
+                }
+                free(s);
             }
         }
     }

@@ -50,3 +50,26 @@ def test_null_arguments_are_rejected_without_a_device():
 def test_context_creation_fails_cleanly_without_a_gpu():
     with pytest.raises(ffi.HoduRocmError):
         ffi.Context(0)
+
+
+def test_host_binding_refuses_metadata_that_reaches_past_a_buffer():
+    """The C ABI takes bare pointers like the reference's kernels; the binding that owns the buffers
+    checks that a metadata vector stays inside them before anything is launched."""
+    class Buf:
+        def __init__(self, n):
+            self.nbytes, self.ptr = n, 0
+
+    chk = ffi.Context._check_extents
+    md = [4, 8, 4, 8, 1, 1, 8, 0, 0]  # dot: [4,8] x [8,4] with the rhs a transposed view of [4,8]
+    chk("dot", "bf16", Buf(64), [Buf(64)], Buf(32), md)
+    with pytest.raises(ffi.HoduRocmError):
+        chk("dot", "bf16", Buf(64), [Buf(62)], Buf(32), md)
+    with pytest.raises(ffi.HoduRocmError):
+        chk("dot", "bf16", Buf(64), [Buf(64)], Buf(30), md)
+    with pytest.raises(ffi.HoduRocmError):
+        chk("dot", "bf16_f8e4m3w", Buf(64), [Buf(31)], Buf(32), md)
+    # matmul with a stride-0 batch-broadcast rhs only needs one copy of it
+    mm = [64, 3, 3, 1, 4, 4, 8, 4, 8, 4, 4, 32, 8, 1, 0, 1, 8, 0, 0, 4, 8, 4]
+    assert ffi.product_spans("matmul", mm) == (128, 32, 64)
+    with pytest.raises(ffi.HoduRocmError):
+        ffi.Context._check_strided("cast", 1, 2, Buf(15), Buf(32), [16, 2, 4, 4, 1, 4, 0])
