@@ -217,6 +217,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every GPU box here has one GPU and no collective or sharded "
@@ -227,6 +228,7 @@ def main():
     from hodu_amd import ffi
     ctx = ffi.Context(0)
     info = ctx.device_info()
+    ctx.force_tile(args.force_tile)
     which = set(args.configs.split(",")) | {"c2"}
     results = []
     for case in build_cases(which):

@@ -84,11 +84,17 @@ template <> struct Compute<CK_F32> {
 // ------------------------------------------------------------------------------------------------
 // LDS layouts.  Both give conflict-free ds_read_b128 for "16 lanes = 16 consecutive rows, one chunk".
 // ------------------------------------------------------------------------------------------------
-// row-major, padded: written by LM_K / LM_SCALAR (a lane owns one chunk)
-__device__ __forceinline__ int lds_rowmajor(int row, int chunk) { return row * ROW_PITCH + chunk * 16; }
+// Row-major with an XOR swizzle, in blocks of 8 rows (1 KB) separated by 128 bytes: chunk c of
+// row r sits at slot c ^ (r % 8).  A block is exactly what one wavefront-wide 16-byte-per-lane
+// LDS-DMA load writes (lane l -> byte 16*l), which is why there is no padding INSIDE a block; the
+// swizzle is applied on the global-address side of that load.  Used by LM_K and LM_SCALAR.
+constexpr int SWZ_BLOCK = 8 * ROW_BYTES + 128;
+__device__ __forceinline__ int lds_swizzled(int row, int chunk) {
+    return (row >> 3) * SWZ_BLOCK + (row & 7) * ROW_BYTES + ((chunk ^ (row & 7)) << 4);
+}
 
-// written by LM_MN, where a lane owns the same chunk of G consecutive rows: rows are split by
-// (row % G) into G sub-planes so that neighbouring lanes (row groups) write neighbouring 16 bytes
+// Written by LM_MN, where a lane owns the same chunk of G consecutive rows: rows are split by
+// (row % G) into G sub-planes so that neighbouring lanes (row groups) write neighbouring 16 bytes.
 template <int ROWS, int G> struct MnLayout {
     static constexpr int SUB = (ROWS / G) * 16 + (G == 8 ? 32 : 64);  // bytes per (row % G) sub-plane
     static constexpr int PLANE = G * SUB;                              // bytes per chunk index
@@ -96,11 +102,6 @@ template <int ROWS, int G> struct MnLayout {
         return chunk * PLANE + (row % G) * SUB + (row / G) * 16;
     }
 };
-
-template <int ROWS, int G> constexpr int operand_lds_bytes() {
-    return (ROWS * ROW_PITCH) > (CHUNKS * MnLayout<ROWS, G>::PLANE) ? (ROWS * ROW_PITCH)
-                                                                  : (CHUNKS * MnLayout<ROWS, G>::PLANE);
-}
 
 // ------------------------------------------------------------------------------------------------
 // operand description handed to the loaders
@@ -114,6 +115,17 @@ struct Operand {
 };
 
 __device__ __forceinline__ u32x4_t zero4() { return u32x4_t{0u, 0u, 0u, 0u}; }
+__device__ __forceinline__ u32x4_t ldg128(const char *p) { return *reinterpret_cast<const u32x4_t *>(p); }
+__device__ __forceinline__ u32x2_t ldg64(const char *p) { return *reinterpret_cast<const u32x2_t *>(p); }
+__device__ __forceinline__ void lds_put(char *lds, int off, const u32x4_t &v) { *reinterpret_cast<u32x4_t *>(lds + off) = v; }
+__device__ __forceinline__ u32x4_t lds_get(const char *lds, int off) { return *reinterpret_cast<const u32x4_t *>(lds + off); }
+
+// 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): the wavefront
+// writes 1 KB starting at `lds_block` (wave-uniform), lane l at byte 16*l
+__device__ __forceinline__ void dma16(const char *gptr, char *lds_block) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gptr,
+                                     (__attribute__((address_space(3))) void *)lds_block, 16, 0, 0);
+}
 
 // two f8e4m3 -> two bf16 packed (lo = first)
 __device__ __forceinline__ uint32_t f8pair_to_bf16pair(uint32_t word, bool hi) {
@@ -122,36 +134,44 @@ __device__ __forceinline__ uint32_t f8pair_to_bf16pair(uint32_t word, bool hi) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Loader<LM, SK, CK, ROWS, NT>: stages one operand tile (ROWS rows x 128 bytes of compute type)
-//   load()  global -> registers (issued early)       store() registers -> LDS (after the MFMAs)
-//   at()    LDS byte offset of (row, chunk) for the fragment reads
+// Loader<LM, SK, CK, ROWS, NT>: stages one operand tile (ROWS rows x 128 bytes of compute type).
+//   issue_full()   start moving a K step that lies fully inside K (no k checks, rows clamped): either
+//                  LDS-DMA straight into `dst`, or global loads into registers
+//   commit_full()  registers -> LDS for the register paths; nothing for the DMA path
+//   tail()         the ragged last K step: guarded loads, zero fill, written to `dst` at once
+//   at()           LDS byte offset of (row, chunk) for the fragment reads
 // ------------------------------------------------------------------------------------------------
 template <int LM, int SK, int CK, int ROWS, int NT> struct Loader;
 
-// ---- k-dense, storage type == compute type: one 16-byte load per chunk ---------------------------
+// ---- k-dense, storage type == compute type: LDS-DMA, no registers, no LDS store instructions ----
 template <int CK, int ROWS, int NT> struct Loader<LM_K, SK_SAME, CK, ROWS, NT> {
     static constexpr int ES = Compute<CK>::ES, EPC = 16 / ES;
-    static constexpr int UNITS = ROWS * CHUNKS / NT;
-    static_assert(ROWS * CHUNKS % NT == 0, "tile/threads");
-    static constexpr int LDS_BYTES = ROWS * ROW_PITCH;
-    u32x4_t r[UNITS];
-    static __device__ __forceinline__ int at(int row, int chunk) { return lds_rowmajor(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+    static constexpr int NW = NT / 64, BLOCKS = ROWS / 8;
+    static constexpr int PER_WAVE = (BLOCKS + NW - 1) / NW;
+    static constexpr int LDS_BYTES = BLOCKS * SWZ_BLOCK;
+    static __device__ __forceinline__ int at(int row, int chunk) { return lds_swizzled(row, chunk); }
+    __device__ __forceinline__ void issue_full(const Operand &op, int row0, int k0, int tid, char *dst) {
+        const int lane = tid & 63, wave = tid >> 6;
+        const int ri = lane >> 3, kc = (lane & 7) ^ ri;  // the swizzle, applied to the source address
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int c = tid + u * NT, row = c >> 3, kc = c & 7;
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int blk = i * NW + wave;
+            if (BLOCKS % NW != 0 && blk >= BLOCKS) break;
+            int grow = row0 + blk * 8 + ri;
+            grow = grow < op.rows ? grow : op.rows - 1;
+            dma16(op.base + ((long)grow * op.row_stride + k0 + kc * EPC) * ES, dst + blk * SWZ_BLOCK);
+        }
+    }
+    __device__ __forceinline__ void commit_full(char *, int) const {}
+    __device__ __forceinline__ void tail(const Operand &op, int row0, int k0, int tid, char *dst) {
+        for (int c = tid; c < ROWS * CHUNKS; c += NT) {
+            const int row = c >> 3, kc = c & 7;
             int grow = row0 + row;
             grow = grow < op.rows ? grow : op.rows - 1;
             const int k = k0 + kc * EPC;
-            r[u] = zero4();
-            if (k < op.K) r[u] = *reinterpret_cast<const u32x4_t *>(op.base + ((long)grow * op.row_stride + k) * ES);
-        }
-    }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int c = tid + u * NT;
-            *reinterpret_cast<u32x4_t *>(lds + lds_rowmajor(c >> 3, c & 7)) = r[u];
+            u32x4_t v = zero4();
+            if (k < op.K) v = ldg128(op.base + ((long)grow * op.row_stride + k) * ES);
+            lds_put(dst, lds_swizzled(row, kc), v);
         }
     }
 };
@@ -160,10 +180,30 @@ template <int CK, int ROWS, int NT> struct Loader<LM_K, SK_SAME, CK, ROWS, NT> {
 template <int ROWS, int NT> struct Loader<LM_K, SK_F8, CK_BF16, ROWS, NT> {
     static constexpr int UNITS = ROWS * CHUNKS / NT;
     static_assert(ROWS * CHUNKS % NT == 0, "tile/threads");
-    static constexpr int LDS_BYTES = ROWS * ROW_PITCH;
+    static constexpr int LDS_BYTES = (ROWS / 8) * SWZ_BLOCK;
     u32x2_t r[UNITS];
-    static __device__ __forceinline__ int at(int row, int chunk) { return lds_rowmajor(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+    static __device__ __forceinline__ int at(int row, int chunk) { return lds_swizzled(row, chunk); }
+    static __device__ __forceinline__ u32x4_t widen(const u32x2_t &v) {
+        return u32x4_t{f8pair_to_bf16pair(v.x, false), f8pair_to_bf16pair(v.x, true), f8pair_to_bf16pair(v.y, false),
+                       f8pair_to_bf16pair(v.y, true)};
+    }
+    __device__ __forceinline__ void issue_full(const Operand &op, int row0, int k0, int tid, char *) {
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const int c = tid + u * NT, row = c >> 3, kc = c & 7;
+            int grow = row0 + row;
+            grow = grow < op.rows ? grow : op.rows - 1;
+            r[u] = ldg64(op.base + (long)grow * op.row_stride + k0 + kc * 8);
+        }
+    }
+    __device__ __forceinline__ void commit_full(char *dst, int tid) const {
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const int c = tid + u * NT;
+            lds_put(dst, lds_swizzled(c >> 3, c & 7), widen(r[u]));
+        }
+    }
+    __device__ __forceinline__ void tail(const Operand &op, int row0, int k0, int tid, char *dst) {
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             const int c = tid + u * NT, row = c >> 3, kc = c & 7;
@@ -171,214 +211,154 @@ template <int ROWS, int NT> struct Loader<LM_K, SK_F8, CK_BF16, ROWS, NT> {
             grow = grow < op.rows ? grow : op.rows - 1;
             const int k = k0 + kc * 8;
             r[u] = u32x2_t{0u, 0u};
-            if (k < op.K) r[u] = *reinterpret_cast<const u32x2_t *>(op.base + (long)grow * op.row_stride + k);
+            if (k < op.K) r[u] = ldg64(op.base + (long)grow * op.row_stride + k);
         }
-    }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int c = tid + u * NT;
-            u32x4_t w;
-            w.x = f8pair_to_bf16pair(r[u].x, false);
-            w.y = f8pair_to_bf16pair(r[u].x, true);
-            w.z = f8pair_to_bf16pair(r[u].y, false);
-            w.w = f8pair_to_bf16pair(r[u].y, true);
-            *reinterpret_cast<u32x4_t *>(lds + lds_rowmajor(c >> 3, c & 7)) = w;
-        }
+        commit_full(dst, tid);
     }
 };
 
-// ---- row-dense 16-bit storage: 8 loads of 8 rows (16 B) for 8 consecutive k, 8x8 transpose ---------
-template <int CK, int ROWS, int NT> struct Loader<LM_MN, SK_SAME, CK, ROWS, NT> {
-    static_assert(Compute<CK>::ES == 2, "specialised below for 1- and 4-byte types");
-    typedef MnLayout<ROWS, 8> L;
-    static constexpr int TOTAL = ROWS;  // (ROWS/8 row groups) x 8 chunks
-    static constexpr int UNITS = (TOTAL + NT - 1) / NT;
-    static constexpr int LDS_BYTES = CHUNKS * L::PLANE;
-    u32x4_t r[UNITS][8];
-    static __device__ __forceinline__ int at(int row, int chunk) { return L::at(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+// ---- row-dense operands: loads run along the rows for VK consecutive k, then a register transpose.
+// RowDense<...> supplies the per-type pieces: VB bytes per load (RG rows), VK loads per unit, and
+// transpose() turning the VK loaded vectors into RG chunks of 16 bytes (one per row).
+template <int SK, int CK> struct RowDense;
+
+// 16-bit storage: 8 loads of 8 rows (16 B) for 8 consecutive k
+template <int CK> struct RowDenseHalf {
+    static constexpr int RG = 8, VK = 8, SES = 2;
+    typedef u32x4_t vec_t;
+    static __device__ __forceinline__ vec_t zero() { return zero4(); }
+    static __device__ __forceinline__ vec_t load(const char *p) { return ldg128(p); }
+    static __device__ __forceinline__ void transpose(const vec_t (&v)[8], u32x4_t (&w)[8]) {
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int id = tid + u * NT;
-            const int rg = id % (ROWS / 8), kc = id / (ROWS / 8);
-            const int row = row0 + rg * 8;
-            const bool row_ok = (TOTAL % NT == 0 || id < TOTAL) && row < op.rows;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int k = k0 + kc * 8 + j;
-                r[u][j] = zero4();
-                if (row_ok && k < op.K)
-                    r[u][j] = *reinterpret_cast<const u32x4_t *>(op.base + ((long)k * op.k_stride + row) * 2);
-            }
+        for (int rr = 0; rr < 8; rr++) {
+            // rows 2q, 2q+1 live in dword q of every k-vector
+            const uint32_t sel = (rr & 1) ? 0x07060302u : 0x05040100u;
+            w[rr].x = __builtin_amdgcn_perm(v[1][rr >> 1], v[0][rr >> 1], sel);
+            w[rr].y = __builtin_amdgcn_perm(v[3][rr >> 1], v[2][rr >> 1], sel);
+            w[rr].z = __builtin_amdgcn_perm(v[5][rr >> 1], v[4][rr >> 1], sel);
+            w[rr].w = __builtin_amdgcn_perm(v[7][rr >> 1], v[6][rr >> 1], sel);
         }
     }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
+};
+template <> struct RowDense<SK_SAME, CK_BF16> : RowDenseHalf<CK_BF16> {};
+template <> struct RowDense<SK_SAME, CK_F16> : RowDenseHalf<CK_F16> {};
+
+// f8e4m3 storage -> bf16: 8 loads of 8 rows (8 B) for 8 consecutive k; the widening conversion
+// yields f32 pairs whose high halves are packed across k, so the transpose costs nothing extra
+template <> struct RowDense<SK_F8, CK_BF16> {
+    static constexpr int RG = 8, VK = 8, SES = 1;
+    typedef u32x2_t vec_t;
+    static __device__ __forceinline__ vec_t zero() { return u32x2_t{0u, 0u}; }
+    static __device__ __forceinline__ vec_t load(const char *p) { return ldg64(p); }
+    static __device__ __forceinline__ void transpose(const vec_t (&v)[8], u32x4_t (&w)[8]) {
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int id = tid + u * NT;
-            if (TOTAL % NT != 0 && id >= TOTAL) continue;
-            const int rg = id % (ROWS / 8), kc = id / (ROWS / 8);
+        for (int p = 0; p < 4; p++) {      // k pair (2p, 2p+1)
 #pragma unroll
-            for (int rr = 0; rr < 8; rr++) {
-                // rows 2q, 2q+1 live in dword q of every k-vector
-                const uint32_t sel = (rr & 1) ? 0x07060302u : 0x05040100u;
-                u32x4_t w;
-                w.x = __builtin_amdgcn_perm(r[u][1][rr >> 1], r[u][0][rr >> 1], sel);
-                w.y = __builtin_amdgcn_perm(r[u][3][rr >> 1], r[u][2][rr >> 1], sel);
-                w.z = __builtin_amdgcn_perm(r[u][5][rr >> 1], r[u][4][rr >> 1], sel);
-                w.w = __builtin_amdgcn_perm(r[u][7][rr >> 1], r[u][6][rr >> 1], sel);
-                *reinterpret_cast<u32x4_t *>(lds + L::at(rg * 8 + rr, kc)) = w;
+            for (int q = 0; q < 4; q++) {  // row pair (2q, 2q+1): byte pair q of the 8-byte vector
+                const uint32_t wa = q < 2 ? v[2 * p].x : v[2 * p].y;
+                const uint32_t wb = q < 2 ? v[2 * p + 1].x : v[2 * p + 1].y;
+                const f32x2_t fa = (q & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)wa, true)
+                                           : __builtin_amdgcn_cvt_pk_f32_fp8((int)wa, false);
+                const f32x2_t fb = (q & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)wb, true)
+                                           : __builtin_amdgcn_cvt_pk_f32_fp8((int)wb, false);
+                w[2 * q][p] = __builtin_amdgcn_perm(__float_as_uint(fb.x), __float_as_uint(fa.x), 0x07060302u);
+                w[2 * q + 1][p] = __builtin_amdgcn_perm(__float_as_uint(fb.y), __float_as_uint(fa.y), 0x07060302u);
             }
         }
     }
 };
 
-// ---- row-dense f8e4m3 storage -> bf16: 8 loads of 8 rows (8 B), widen + transpose ------------------
-template <int ROWS, int NT> struct Loader<LM_MN, SK_F8, CK_BF16, ROWS, NT> {
-    typedef MnLayout<ROWS, 8> L;
-    static constexpr int TOTAL = ROWS;
-    static constexpr int UNITS = (TOTAL + NT - 1) / NT;
-    static constexpr int LDS_BYTES = CHUNKS * L::PLANE;
-    u32x2_t r[UNITS][8];
-    static __device__ __forceinline__ int at(int row, int chunk) { return L::at(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+// 8-bit storage: 16 loads of 8 rows (8 B) for 16 consecutive k, two-level byte transpose
+template <> struct RowDense<SK_SAME, CK_I8> {
+    static constexpr int RG = 8, VK = 16, SES = 1;
+    typedef u32x2_t vec_t;
+    static __device__ __forceinline__ vec_t zero() { return u32x2_t{0u, 0u}; }
+    static __device__ __forceinline__ vec_t load(const char *p) { return ldg64(p); }
+    static __device__ __forceinline__ void transpose(const vec_t (&v)[16], u32x4_t (&w)[8]) {
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int id = tid + u * NT;
-            const int rg = id % (ROWS / 8), kc = id / (ROWS / 8);
-            const int row = row0 + rg * 8;
-            const bool row_ok = (TOTAL % NT == 0 || id < TOTAL) && row < op.rows;
+        for (int q = 0; q < 4; q++) {  // k quad (4q .. 4q+3) -> dword q of the output chunk
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int k = k0 + kc * 8 + j;
-                r[u][j] = u32x2_t{0u, 0u};
-                if (row_ok && k < op.K)
-                    r[u][j] = *reinterpret_cast<const u32x2_t *>(op.base + (long)k * op.k_stride + row);
+            for (int h = 0; h < 2; h++) {  // rows 4h .. 4h+3 live in dword h of every k-vector
+                const uint32_t v0 = h ? v[4 * q].y : v[4 * q].x;
+                const uint32_t v1 = h ? v[4 * q + 1].y : v[4 * q + 1].x;
+                const uint32_t v2 = h ? v[4 * q + 2].y : v[4 * q + 2].x;
+                const uint32_t v3 = h ? v[4 * q + 3].y : v[4 * q + 3].x;
+                // level 1: interleave bytes of (k, k+1): [k.r0, k1.r0, k.r1, k1.r1] and rows 2, 3
+                const uint32_t a01 = __builtin_amdgcn_perm(v1, v0, 0x05010400u);
+                const uint32_t a23 = __builtin_amdgcn_perm(v1, v0, 0x07030602u);
+                const uint32_t b01 = __builtin_amdgcn_perm(v3, v2, 0x05010400u);
+                const uint32_t b23 = __builtin_amdgcn_perm(v3, v2, 0x07030602u);
+                // level 2: [k0, k1, k2, k3] of one row
+                w[4 * h + 0][q] = __builtin_amdgcn_perm(b01, a01, 0x05040100u);
+                w[4 * h + 1][q] = __builtin_amdgcn_perm(b01, a01, 0x07060302u);
+                w[4 * h + 2][q] = __builtin_amdgcn_perm(b23, a23, 0x05040100u);
+                w[4 * h + 3][q] = __builtin_amdgcn_perm(b23, a23, 0x07060302u);
             }
-        }
-    }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int id = tid + u * NT;
-            if (TOTAL % NT != 0 && id >= TOTAL) continue;
-            const int rg = id % (ROWS / 8), kc = id / (ROWS / 8);
-            uint32_t w[8][4];
-#pragma unroll
-            for (int p = 0; p < 4; p++) {      // k pair (2p, 2p+1)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {  // row pair (2q, 2q+1): byte pair q of the 8-byte vector
-                    const uint32_t wa = q < 2 ? r[u][2 * p].x : r[u][2 * p].y;
-                    const uint32_t wb = q < 2 ? r[u][2 * p + 1].x : r[u][2 * p + 1].y;
-                    const f32x2_t fa = (q & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)wa, true)
-                                               : __builtin_amdgcn_cvt_pk_f32_fp8((int)wa, false);
-                    const f32x2_t fb = (q & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)wb, true)
-                                               : __builtin_amdgcn_cvt_pk_f32_fp8((int)wb, false);
-                    w[2 * q][p] = __builtin_amdgcn_perm(__float_as_uint(fb.x), __float_as_uint(fa.x), 0x07060302u);
-                    w[2 * q + 1][p] = __builtin_amdgcn_perm(__float_as_uint(fb.y), __float_as_uint(fa.y), 0x07060302u);
-                }
-            }
-#pragma unroll
-            for (int rr = 0; rr < 8; rr++)
-                *reinterpret_cast<u32x4_t *>(lds + L::at(rg * 8 + rr, kc)) = u32x4_t{w[rr][0], w[rr][1], w[rr][2], w[rr][3]};
         }
     }
 };
 
-// ---- row-dense 8-bit storage: 16 loads of 8 rows (8 B) for 16 consecutive k, byte transpose --------
-template <int ROWS, int NT> struct Loader<LM_MN, SK_SAME, CK_I8, ROWS, NT> {
-    typedef MnLayout<ROWS, 8> L;
-    static constexpr int TOTAL = ROWS;
-    static constexpr int UNITS = (TOTAL + NT - 1) / NT;
-    static constexpr int LDS_BYTES = CHUNKS * L::PLANE;
-    u32x2_t r[UNITS][16];
-    static __device__ __forceinline__ int at(int row, int chunk) { return L::at(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+// f32 storage: 4 loads of 4 rows (16 B) for 4 consecutive k; the transpose is register renaming
+template <> struct RowDense<SK_SAME, CK_F32> {
+    static constexpr int RG = 4, VK = 4, SES = 4;
+    typedef u32x4_t vec_t;
+    static __device__ __forceinline__ vec_t zero() { return zero4(); }
+    static __device__ __forceinline__ vec_t load(const char *p) { return ldg128(p); }
+    static __device__ __forceinline__ void transpose(const vec_t (&v)[4], u32x4_t (&w)[4]) {
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int id = tid + u * NT;
-            const int rg = id % (ROWS / 8), kc = id / (ROWS / 8);
-            const int row = row0 + rg * 8;
-            const bool row_ok = (TOTAL % NT == 0 || id < TOTAL) && row < op.rows;
-#pragma unroll
-            for (int j = 0; j < 16; j++) {
-                const int k = k0 + kc * 16 + j;
-                r[u][j] = u32x2_t{0u, 0u};
-                if (row_ok && k < op.K)
-                    r[u][j] = *reinterpret_cast<const u32x2_t *>(op.base + (long)k * op.k_stride + row);
-            }
-        }
-    }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const int id = tid + u * NT;
-            if (TOTAL % NT != 0 && id >= TOTAL) continue;
-            const int rg = id % (ROWS / 8), kc = id / (ROWS / 8);
-            uint32_t w[8][4];
-#pragma unroll
-            for (int q = 0; q < 4; q++) {  // k quad (4q .. 4q+3) -> dword q of the output chunk
-#pragma unroll
-                for (int h = 0; h < 2; h++) {  // rows 4h .. 4h+3 live in dword h of every k-vector
-                    const uint32_t v0 = h ? r[u][4 * q].y : r[u][4 * q].x;
-                    const uint32_t v1 = h ? r[u][4 * q + 1].y : r[u][4 * q + 1].x;
-                    const uint32_t v2 = h ? r[u][4 * q + 2].y : r[u][4 * q + 2].x;
-                    const uint32_t v3 = h ? r[u][4 * q + 3].y : r[u][4 * q + 3].x;
-                    // level 1: interleave bytes of (k, k+1): [k.r0, k1.r0, k.r1, k1.r1] and rows 2,3
-                    const uint32_t a01 = __builtin_amdgcn_perm(v1, v0, 0x05010400u);
-                    const uint32_t a23 = __builtin_amdgcn_perm(v1, v0, 0x07030602u);
-                    const uint32_t b01 = __builtin_amdgcn_perm(v3, v2, 0x05010400u);
-                    const uint32_t b23 = __builtin_amdgcn_perm(v3, v2, 0x07030602u);
-                    // level 2: [k0,k1,k2,k3] of one row
-                    w[4 * h + 0][q] = __builtin_amdgcn_perm(b01, a01, 0x05040100u);
-                    w[4 * h + 1][q] = __builtin_amdgcn_perm(b01, a01, 0x07060302u);
-                    w[4 * h + 2][q] = __builtin_amdgcn_perm(b23, a23, 0x05040100u);
-                    w[4 * h + 3][q] = __builtin_amdgcn_perm(b23, a23, 0x07060302u);
-                }
-            }
-#pragma unroll
-            for (int rr = 0; rr < 8; rr++)
-                *reinterpret_cast<u32x4_t *>(lds + L::at(rg * 8 + rr, kc)) = u32x4_t{w[rr][0], w[rr][1], w[rr][2], w[rr][3]};
-        }
+        for (int rr = 0; rr < 4; rr++) w[rr] = u32x4_t{v[0][rr], v[1][rr], v[2][rr], v[3][rr]};
     }
 };
 
-// ---- row-dense f32 storage: 4 loads of 4 rows (16 B) for 4 consecutive k, transpose by renaming ---
-template <int ROWS, int NT> struct Loader<LM_MN, SK_SAME, CK_F32, ROWS, NT> {
-    typedef MnLayout<ROWS, 4> L;
-    static constexpr int TOTAL = (ROWS / 4) * CHUNKS;
+template <int SK, int CK, int ROWS, int NT> struct Loader<LM_MN, SK, CK, ROWS, NT> {
+    typedef RowDense<SK, CK> RD;
+    static constexpr int RG = RD::RG, VK = RD::VK, SES = RD::SES;
+    typedef MnLayout<ROWS, RG> L;
+    static constexpr int GROUPS = ROWS / RG;
+    static constexpr int TOTAL = GROUPS * CHUNKS;  // units: (row group, chunk)
     static constexpr int UNITS = (TOTAL + NT - 1) / NT;
     static constexpr int LDS_BYTES = CHUNKS * L::PLANE;
-    u32x4_t r[UNITS][4];
+    typename RD::vec_t r[UNITS][VK];
     static __device__ __forceinline__ int at(int row, int chunk) { return L::at(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+    __device__ __forceinline__ void issue_full(const Operand &op, int row0, int k0, int tid, char *) {
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             const int id = tid + u * NT;
-            const int rg = id % (ROWS / 4), kc = id / (ROWS / 4);
-            const int row = row0 + rg * 4;
-            const bool row_ok = (TOTAL % NT == 0 || id < TOTAL) && row < op.rows;
+            const int rg = id % GROUPS, kc = (id / GROUPS) % CHUNKS;  // ids past TOTAL wrap: harmless reloads
+            int row = row0 + rg * RG;
+            row = row < op.rows ? row : op.rows - RG;  // op.rows % RG == 0: the clamped vector is in range
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int k = k0 + kc * 4 + j;
-                r[u][j] = zero4();
-                if (row_ok && k < op.K)
-                    r[u][j] = *reinterpret_cast<const u32x4_t *>(op.base + ((long)k * op.k_stride + row) * 4);
-            }
+            for (int j = 0; j < VK; j++)
+                r[u][j] = RD::load(op.base + ((long)(k0 + kc * VK + j) * op.k_stride + row) * SES);
         }
     }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
+    __device__ __forceinline__ void commit_full(char *dst, int tid) const {
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             const int id = tid + u * NT;
             if (TOTAL % NT != 0 && id >= TOTAL) continue;
-            const int rg = id % (ROWS / 4), kc = id / (ROWS / 4);
+            const int rg = id % GROUPS, kc = id / GROUPS;
+            u32x4_t w[RG];
+            RD::transpose(r[u], w);
 #pragma unroll
-            for (int rr = 0; rr < 4; rr++)
-                *reinterpret_cast<u32x4_t *>(lds + L::at(rg * 4 + rr, kc)) =
-                    u32x4_t{r[u][0][rr], r[u][1][rr], r[u][2][rr], r[u][3][rr]};
+            for (int rr = 0; rr < RG; rr++) lds_put(dst, L::at(rg * RG + rr, kc), w[rr]);
         }
+    }
+    __device__ __forceinline__ void tail(const Operand &op, int row0, int k0, int tid, char *dst) {
+        // same registers as the full path, guarded loads with zero fill
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const int id = tid + u * NT;
+            const int rg = id % GROUPS, kc = (id / GROUPS) % CHUNKS;
+            const int row = row0 + rg * RG;
+#pragma unroll
+            for (int j = 0; j < VK; j++) {
+                const int k = k0 + kc * VK + j;
+                r[u][j] = RD::zero();
+                if (row < op.rows && k < op.K) r[u][j] = RD::load(op.base + ((long)k * op.k_stride + row) * SES);
+            }
+        }
+        commit_full(dst, tid);
     }
 };
 
@@ -405,10 +385,10 @@ template <> struct ScalarFetch<SK_F8, CK_BF16> {
 template <int SK, int CK, int ROWS, int NT> struct Loader<LM_SCALAR, SK, CK, ROWS, NT> {
     static constexpr int ES = Compute<CK>::ES, EPC = 16 / ES;
     static constexpr int UNITS = ROWS * CHUNKS / NT;
-    static constexpr int LDS_BYTES = ROWS * ROW_PITCH;
+    static constexpr int LDS_BYTES = (ROWS / 8) * SWZ_BLOCK;
     u32x4_t r[UNITS];
-    static __device__ __forceinline__ int at(int row, int chunk) { return lds_rowmajor(row, chunk); }
-    __device__ __forceinline__ void load(const Operand &op, int row0, int k0, int tid) {
+    static __device__ __forceinline__ int at(int row, int chunk) { return lds_swizzled(row, chunk); }
+    __device__ __forceinline__ void issue_full(const Operand &op, int row0, int k0, int tid, char *) {
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             const int c = tid + u * NT, row = c >> 3, kc = c & 7;
@@ -427,12 +407,16 @@ template <int SK, int CK, int ROWS, int NT> struct Loader<LM_SCALAR, SK, CK, ROW
             r[u] = u32x4_t{w[0], w[1], w[2], w[3]};
         }
     }
-    __device__ __forceinline__ void store(char *lds, int tid) const {
+    __device__ __forceinline__ void commit_full(char *dst, int tid) const {
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             const int c = tid + u * NT;
-            *reinterpret_cast<u32x4_t *>(lds + lds_rowmajor(c >> 3, c & 7)) = r[u];
+            lds_put(dst, lds_swizzled(c >> 3, c & 7), r[u]);
         }
+    }
+    __device__ __forceinline__ void tail(const Operand &op, int row0, int k0, int tid, char *dst) {
+        issue_full(op, row0, k0, tid, dst);  // the scalar path is guarded throughout
+        commit_full(dst, tid);
     }
 };
 
@@ -472,6 +456,9 @@ template <int CK_, int SKA_, int SKB_, int OUT_, int BM_, int BN_, int WM_, int 
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
     static constexpr int TM = BM / WM / 16, TN = BN / WN / 16;  // 16x16 MFMA tiles per wave
+    // with one wavefront per SIMD (256 threads) nothing else hides LDS latency, so the A fragments of
+    // the next k-slice are prefetched into a second register set while the current slice multiplies
+    static constexpr bool PIPE_A = NT <= 256 && TM * TN * 4 <= 128;  // not when the accumulators fill the AGPR file
     static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "wave tiling");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
@@ -492,13 +479,64 @@ __device__ __forceinline__ void tile_of(long pid, long total, int tiles_m, int t
     tn = (t % width) / gsize;
 }
 
+// One K step (two k-slices of 64 bytes) out of LDS.  Fragment reads run ahead of the MFMAs that
+// consume them: the next B fragment is fetched while the current one multiplies, and (PIPE_A) the
+// A fragments of slice 1 are fetched one per B fragment during slice 0.
+template <class Cfg, class acc_t>
+__device__ __forceinline__ void compute_stage(const char *As, const char *Bs, acc_t (&acc)[Cfg::TM][Cfg::TN], int a_row,
+                                              int b_row, int lg) {
+    typedef Compute<Cfg::CK> Cmp;
+    typedef typename Cfg::LoaderA LoaderA;
+    typedef typename Cfg::LoaderB LoaderB;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+    if constexpr (Cfg::PIPE_A) {
+        u32x4_t af[2][TM], bf[2];
+#pragma unroll
+        for (int i = 0; i < TM; i++) af[0][i] = lds_get(As, LoaderA::at(a_row + i * 16, lg));
+        bf[0] = lds_get(Bs, LoaderB::at(b_row, lg));
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int cur = (s * TN + j) & 1;
+                if (j + 1 < TN) bf[cur ^ 1] = lds_get(Bs, LoaderB::at(b_row + (j + 1) * 16, s * 4 + lg));
+                else if (s == 0) bf[cur ^ 1] = lds_get(Bs, LoaderB::at(b_row, 4 + lg));
+                if (s == 0) {
+#pragma unroll
+                    for (int i = j * TM / TN; i < (j + 1) * TM / TN; i++)
+                        af[1][i] = lds_get(As, LoaderA::at(a_row + i * 16, 4 + lg));
+                }
+                // operands swapped: the accumulator then holds, per lane, 4 consecutive n of one m
+#pragma unroll
+                for (int i = 0; i < TM; i++) Cmp::mma(bf[cur], af[s][i], acc[i][j]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            u32x4_t af[TM], bf[2];
+#pragma unroll
+            for (int i = 0; i < TM; i++) af[i] = lds_get(As, LoaderA::at(a_row + i * 16, s * 4 + lg));
+            bf[0] = lds_get(Bs, LoaderB::at(b_row, s * 4 + lg));
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                if (j + 1 < TN) bf[(j + 1) & 1] = lds_get(Bs, LoaderB::at(b_row + (j + 1) * 16, s * 4 + lg));
+#pragma unroll
+                for (int i = 0; i < TM; i++) Cmp::mma(bf[j & 1], af[i], acc[i][j]);
+            }
+        }
+    }
+}
+
+// LDS-DMA loads are tracked by vmcnt; wait for them before the barrier that publishes the stage
+__device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                typename Out<Cfg::OUT>::T *__restrict__ C,
                                                                DevProduct g, int tiles_m, int tiles_n) {
     extern __shared__ __align__(16) char smem[];
-    typedef Compute<Cfg::CK> Cmp;
-    typedef typename Cmp::acc_t acc_t;
+    typedef typename Compute<Cfg::CK>::acc_t acc_t;
     typedef typename Cfg::LoaderA LoaderA;
     typedef typename Cfg::LoaderB LoaderB;
     typedef typename Out<Cfg::OUT>::T out_t;
@@ -525,12 +563,17 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
 
     LoaderA la;
     LoaderB lb;
-    const int KT = (g.K + BK - 1) / BK;
-    if (KT > 0) {
-        la.load(opA, m0, 0, tid);
-        lb.load(opB, n0, 0, tid);
-        la.store(smem, tid);
-        lb.store(smem + Cfg::A_BYTES, tid);
+    const int KT_full = g.K / BK;             // K steps that lie fully inside K
+    const int KT = (g.K + BK - 1) / BK;       // plus the ragged one, if any
+    if (KT_full > 0) {
+        la.issue_full(opA, m0, 0, tid, smem);
+        lb.issue_full(opB, n0, 0, tid, smem + Cfg::A_BYTES);
+        la.commit_full(smem, tid);
+        lb.commit_full(smem + Cfg::A_BYTES, tid);
+        wait_vm();
+    } else {
+        la.tail(opA, m0, 0, tid, smem);
+        lb.tail(opB, n0, 0, tid, smem + Cfg::A_BYTES);
     }
     __syncthreads();
 
@@ -538,30 +581,20 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
     for (int kt = 0; kt < KT; kt++) {
         char *cur = smem + (kt & 1) * Cfg::STAGE_BYTES;
         char *nxt = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
-        const bool more = kt + 1 < KT;
-        if (more) {  // in flight while the matrix cores work on the current stage
-            la.load(opA, m0, (kt + 1) * BK, tid);
-            lb.load(opB, n0, (kt + 1) * BK, tid);
+        const bool more_full = kt + 1 < KT_full;
+        if (more_full) {  // in flight while the matrix cores work on the current stage
+            la.issue_full(opA, m0, (kt + 1) * BK, tid, nxt);
+            lb.issue_full(opB, n0, (kt + 1) * BK, tid, nxt + Cfg::A_BYTES);
         }
-        const char *As = cur, *Bs = cur + Cfg::A_BYTES;
-#pragma unroll
-        for (int s = 0; s < 2; s++) {
-            u32x4_t af[TM];
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                af[i] = *reinterpret_cast<const u32x4_t *>(As + LoaderA::at(a_row + i * 16, s * 4 + lg));
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const u32x4_t bf = *reinterpret_cast<const u32x4_t *>(Bs + LoaderB::at(b_row + j * 16, s * 4 + lg));
-                // operands swapped: the accumulator then holds, per lane, 4 consecutive n of one m
-#pragma unroll
-                for (int i = 0; i < TM; i++) Cmp::mma(bf, af[i], acc[i][j]);
-            }
+        compute_stage<Cfg>(cur, cur + Cfg::A_BYTES, acc, a_row, b_row, lg);
+        if (more_full) {
+            la.commit_full(nxt, tid);
+            lb.commit_full(nxt + Cfg::A_BYTES, tid);
+        } else if (kt + 1 < KT) {  // the ragged last step: guarded loads, zero fill
+            la.tail(opA, m0, (kt + 1) * BK, tid, nxt);
+            lb.tail(opB, n0, (kt + 1) * BK, tid, nxt + Cfg::A_BYTES);
         }
-        if (more) {
-            la.store(nxt, tid);
-            lb.store(nxt + Cfg::A_BYTES, tid);
-        }
+        wait_vm();
         __syncthreads();
     }
 
@@ -629,46 +662,52 @@ template <class Cfg> int launch_config(hodu_rocm_ctx *ctx, const void *a, const 
     return HODU_ROCM_OK;
 }
 
-// One compute kind = 13 kernels: {KK, KM, MK, MM} x {256x256, 128x128, 64x64} tiles plus a scalar-load
-// 64x64 kernel.  The tile is the largest that still yields at least one workgroup per compute unit.
+// One compute kind = 15 kernels: {KK, KM, MK, MM} x {256x256 with 4 wavefronts, 128x128, 64x64},
+// {KK, KM} x 256x256 with 8 wavefronts, plus a scalar-load 64x64 kernel.  The tile is the largest that still yields at least
+// one workgroup per compute unit.
+constexpr int kVariants = 17;
 template <int CK, int SKA, int SKB, int OUT>
-int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g, const char *const names[13]) {
+int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
+                const char *const names[kVariants]) {
     constexpr int ES = Compute<CK>::ES, EPC = 16 / ES;
     constexpr int SA = SKA == SK_F8 ? 1 : ES, SB = SKB == SK_F8 ? 1 : ES;
     constexpr int ROWVEC = ES == 4 ? 4 : 8;
     const int la = pick_mode(a, g.a_off, g.a_m, g.a_k, g.M, g.K, SA, EPC, ROWVEC, g, g.a_bs);
     const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, SB, EPC, ROWVEC, g, g.b_bs);
     if (la == LM_SCALAR || lb == LM_SCALAR) {
-        ctx->last_kernel = names[12];
+        ctx->last_kernel = names[16];
         return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_SCALAR>>(ctx, a, b, c, g);
     }
     const long cus = ctx->props.multiProcessorCount;
     auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
-    const int size = ctx->force_tile >= 0 ? ctx->force_tile : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 1 : 2;
+    // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64
+    int size = ctx->force_tile >= 0 ? ctx->force_tile : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 2 : 3;
     const int combo = (la == LM_MN ? 2 : 0) + (lb == LM_MN ? 1 : 0);
+    // a row-dense LEFT operand needs 32 staging registers more than the 8-wavefront variant has
+    // (two wavefronts share a SIMD's register file): those layouts use the 4-wavefront variant
+    if (size == 0 && la == LM_MN) size = 1;
     ctx->last_kernel = names[size * 4 + combo];
-#define HODU_MFMA_CASE(SZ, CB, BM, BN, LA, LB)                                                             \
-    if (size == SZ && combo == CB) return launch_config<Config<CK, SKA, SKB, OUT, BM, BN, 2, 2, LA, LB>>(ctx, a, b, c, g);
-    HODU_MFMA_CASE(0, 0, 256, 256, LM_K, LM_K)
-    HODU_MFMA_CASE(0, 1, 256, 256, LM_K, LM_MN)
-    HODU_MFMA_CASE(0, 2, 256, 256, LM_MN, LM_K)
-    HODU_MFMA_CASE(0, 3, 256, 256, LM_MN, LM_MN)
-    HODU_MFMA_CASE(1, 0, 128, 128, LM_K, LM_K)
-    HODU_MFMA_CASE(1, 1, 128, 128, LM_K, LM_MN)
-    HODU_MFMA_CASE(1, 2, 128, 128, LM_MN, LM_K)
-    HODU_MFMA_CASE(1, 3, 128, 128, LM_MN, LM_MN)
-    HODU_MFMA_CASE(2, 0, 64, 64, LM_K, LM_K)
-    HODU_MFMA_CASE(2, 1, 64, 64, LM_K, LM_MN)
-    HODU_MFMA_CASE(2, 2, 64, 64, LM_MN, LM_K)
-    HODU_MFMA_CASE(2, 3, 64, 64, LM_MN, LM_MN)
+#define HODU_MFMA_CASE(SZ, CB, BM, BN, WM, WN, LA, LB)                                                     \
+    if (size == SZ && combo == CB) return launch_config<Config<CK, SKA, SKB, OUT, BM, BN, WM, WN, LA, LB>>(ctx, a, b, c, g);
+#define HODU_MFMA_SIZE(SZ, BM, BN, WM, WN)               \
+    HODU_MFMA_CASE(SZ, 0, BM, BN, WM, WN, LM_K, LM_K)    \
+    HODU_MFMA_CASE(SZ, 1, BM, BN, WM, WN, LM_K, LM_MN)   \
+    HODU_MFMA_CASE(SZ, 2, BM, BN, WM, WN, LM_MN, LM_K)   \
+    HODU_MFMA_CASE(SZ, 3, BM, BN, WM, WN, LM_MN, LM_MN)
+    HODU_MFMA_CASE(0, 0, 256, 256, 2, 4, LM_K, LM_K)
+    HODU_MFMA_CASE(0, 1, 256, 256, 2, 4, LM_K, LM_MN)
+    HODU_MFMA_SIZE(1, 256, 256, 2, 2)
+    HODU_MFMA_SIZE(2, 128, 128, 2, 2)
+    HODU_MFMA_SIZE(3, 64, 64, 2, 2)
+#undef HODU_MFMA_SIZE
 #undef HODU_MFMA_CASE
     return fail(HODU_ROCM_UNSUPPORTED, "no MFMA variant");
 }
 
-#define HODU_MFMA_NAMES(P)                                                                                 \
-    {P "_256x256_KK", P "_256x256_KM", P "_256x256_MK", P "_256x256_MM", P "_128x128_KK", P "_128x128_KM", \
-     P "_128x128_MK", P "_128x128_MM", P "_64x64_KK",   P "_64x64_KM",   P "_64x64_MK",   P "_64x64_MM",   \
-     P "_64x64_scalar"}
+#define HODU_MFMA_NAMES(P)                                                                                       \
+    {P "_256x256w8_KK", P "_256x256w8_KM", P "_256x256w8_MK", P "_256x256w8_MM", P "_256x256_KK", P "_256x256_KM", \
+     P "_256x256_MK",   P "_256x256_MM",   P "_128x128_KK",   P "_128x128_KM",   P "_128x128_MK", P "_128x128_MM", \
+     P "_64x64_KK",     P "_64x64_KM",     P "_64x64_MK",     P "_64x64_MM",     P "_64x64_scalar"}
 
 }  // namespace mfma
 }  // namespace hodu

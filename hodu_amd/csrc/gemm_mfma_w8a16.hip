@@ -3,7 +3,7 @@
 #include "gemm_mfma.hpp"
 namespace hodu {
 int launch_mfma_w8a16(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
-    static const char *const names[13] = HODU_MFMA_NAMES("mfma_bf16_f8w");
+    static const char *const names[mfma::kVariants] = HODU_MFMA_NAMES("mfma_bf16_f8w");
     return mfma::launch_kind<mfma::CK_BF16, mfma::SK_SAME, mfma::SK_F8, mfma::OUT_BF16>(ctx, a, b, c, g, names);
 }
 }  // namespace hodu

@@ -245,7 +245,7 @@ class Context:
         return float(ms.value)
 
     def force_tile(self, tile: int):
-        """testing hook: 0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic"""
+        """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, -1 = automatic"""
         self._check(self.lib.hodu_rocm_debug_force_tile(self.handle, int(tile)))
 
     def last_kernel(self) -> str:

@@ -18,7 +18,7 @@ KINDS = {
     "bf16_f8e4m3w": ("mfma_bf16_f8w", 8, 8),
     "i32_i8i8": ("mfma_i32_i8i8", 16, 8),
 }
-TILES = {0: "256x256", 1: "128x128", 2: "64x64"}
+TILES = {0: "256x256w8", 1: "256x256", 2: "128x128", 3: "64x64"}
 
 
 @pytest.fixture(scope="module")
@@ -36,16 +36,20 @@ def views(combo, M, K, N):
 
 
 @pytest.mark.parametrize("kind", list(KINDS))
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
 def test_every_variant_ragged(ctx, kind, tile):
     prefix, kmul, rmul = KINDS[kind]
     ctx.force_tile(tile)
-    M, N, K = 296, 200, 9 * 16  # M, N not multiples of any tile; K = 144 leaves a ragged last K step
+    M, N = 296, 200  # not multiples of any tile
+    # K = 400: full K steps (through the LDS-DMA path where the layout allows) and a ragged last one
+    K = 400
     scale = 1.0
     for combo in ("KK", "KM", "MK", "MM"):
         lv, rv = views(combo, M, K, N)
+        # the 8-wavefront variant exists for k-dense left operands only; others use the 4-wavefront one
+        name = TILES[1] if (tile == 0 and combo[0] == "M") else TILES[tile]
         check_product(ctx, "dot", kind, lv, rv, seed=tile, scale=scale, rscale=2.0 if "f8" in kind else None,
-                      expect_kernel=f"{prefix}_{TILES[tile]}_{combo}")
+                      expect_kernel=f"{prefix}_{name}_{combo}")
     ctx.force_tile(-1)
 
 
