@@ -217,6 +217,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -229,6 +230,11 @@ def main():
     ctx = ffi.Context(0)
     info = ctx.device_info()
     ctx.force_tile(args.force_tile)
+    if args.only:
+        case = next(c for c in build_cases({args.only.split("_")[0]}) if c.key == args.only)
+        print(json.dumps(time_case(ctx, case, args.steps, args.warmup)))
+        ctx.close()
+        return
     which = set(args.configs.split(",")) | {"c2"}
     results = []
     for case in build_cases(which):

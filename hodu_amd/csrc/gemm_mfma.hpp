@@ -81,6 +81,45 @@ template <> struct Compute<CK_F32> {
     }
 };
 
+// 32x32 MFMA tiles for the tile kernels.  One 4-pass 16x16x32 MFMA can be issued by a wavefront only
+// about every 28 cycles (measured: a single wavefront per SIMD sustains 56 % of the matrix-core peak
+// with it), whereas the 8-pass 32x32x16 form keeps the pipe full from one wavefront and leaves issue
+// slots for LDS and address instructions in between.
+// Fragment: lane l supplies row (or column) l % 32 and the 16 bytes of k-half l / 32; a 64-byte
+// slice of K therefore takes two MFMAs per tile, fed by chunks 2*s + (l / 32).
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef int i32x16_t __attribute__((ext_vector_type(16)));
+template <int CK> struct Compute32;
+template <> struct Compute32<CK_BF16> {
+    typedef f32x16_t acc_t;
+    static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bitcast<bf16x8_t>(a), bitcast<bf16x8_t>(b), c, 0, 0, 0);
+    }
+};
+template <> struct Compute32<CK_F16> {
+    typedef f32x16_t acc_t;
+    static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(bitcast<f16x8_t>(a), bitcast<f16x8_t>(b), c, 0, 0, 0);
+    }
+};
+template <> struct Compute32<CK_I8> {
+    typedef i32x16_t acc_t;
+    static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(bitcast<i32x4_t>(a), bitcast<i32x4_t>(b), c, 0, 0, 0);
+    }
+};
+template <> struct Compute32<CK_F32> {
+    typedef f32x16_t acc_t;
+    // a lane's chunk holds 4 consecutive k; MFMA t consumes element t of both lane halves (k = t, 4 + t)
+    static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
+        const f32x4_t af = bitcast<f32x4_t>(a), bf = bitcast<f32x4_t>(b);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.x, bf.x, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.y, bf.y, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.z, bf.z, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.w, bf.w, c, 0, 0, 0);
+    }
+};
+
 // ------------------------------------------------------------------------------------------------
 // LDS layouts.  Both give conflict-free ds_read_b128 for "16 lanes = 16 consecutive rows, one chunk".
 // ------------------------------------------------------------------------------------------------
@@ -441,6 +480,32 @@ template <> struct Out<OUT_I32> {
     static __device__ __forceinline__ T cvt(int v) { return v; }
 };
 
+// Stores the 32x32 accumulator tile of one wavefront.  With the operands swapped in the MFMA (the
+// right operand's fragment in the A slot) a lane holds, for ONE output row m = m_base + l % 32, four
+// runs of four consecutive columns n = n_base + 8*q + 4*(l / 32) + e.
+template <int OUT, class acc_t>
+__device__ __forceinline__ void store_tile32(typename Out<OUT>::T *Cb, const acc_t &acc, int m, int n_base, int lh,
+                                             int M, int N, bool vec_ok) {
+    typedef typename Out<OUT>::T out_t;
+    if (m >= M) return;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int n = n_base + 8 * q + 4 * lh;
+        out_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = Out<OUT>::cvt(acc[4 * q + e]);
+        out_t *dst = Cb + (long)m * N + n;
+        if (vec_ok && n + 3 < N) {
+            struct alignas(sizeof(out_t) * 4) Quad { out_t q[4]; };
+            *reinterpret_cast<Quad *>(dst) = Quad{{v[0], v[1], v[2], v[3]}};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (n + e < N) dst[e] = v[e];
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // the kernel
 // ------------------------------------------------------------------------------------------------
@@ -455,11 +520,8 @@ template <int CK_, int SKA_, int SKB_, int OUT_, int BM_, int BN_, int WM_, int 
     static constexpr int A_BYTES = LoaderA::LDS_BYTES, B_BYTES = LoaderB::LDS_BYTES;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-    static constexpr int TM = BM / WM / 16, TN = BN / WN / 16;  // 16x16 MFMA tiles per wave
-    // with one wavefront per SIMD (256 threads) nothing else hides LDS latency, so the A fragments of
-    // the next k-slice are prefetched into a second register set while the current slice multiplies
-    static constexpr bool PIPE_A = NT <= 256 && TM * TN * 4 <= 128;  // not when the accumulators fill the AGPR file
-    static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "wave tiling");
+    static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
 
@@ -479,52 +541,33 @@ __device__ __forceinline__ void tile_of(long pid, long total, int tiles_m, int t
     tn = (t % width) / gsize;
 }
 
-// One K step (two k-slices of 64 bytes) out of LDS.  Fragment reads run ahead of the MFMAs that
-// consume them: the next B fragment is fetched while the current one multiplies, and (PIPE_A) the
-// A fragments of slice 1 are fetched one per B fragment during slice 0.
+// One K step (128 bytes of K = four 32-byte slices) out of LDS.  The fragments of slice s+1 are read
+// into a second register set while slice s multiplies.
 template <class Cfg, class acc_t>
 __device__ __forceinline__ void compute_stage(const char *As, const char *Bs, acc_t (&acc)[Cfg::TM][Cfg::TN], int a_row,
-                                              int b_row, int lg) {
-    typedef Compute<Cfg::CK> Cmp;
+                                              int b_row, int lh) {
+    typedef Compute32<Cfg::CK> Cmp;
     typedef typename Cfg::LoaderA LoaderA;
     typedef typename Cfg::LoaderB LoaderB;
     constexpr int TM = Cfg::TM, TN = Cfg::TN;
-    if constexpr (Cfg::PIPE_A) {
-        u32x4_t af[2][TM], bf[2];
+    u32x4_t af[2][TM], bf[2][TN];
 #pragma unroll
-        for (int i = 0; i < TM; i++) af[0][i] = lds_get(As, LoaderA::at(a_row + i * 16, lg));
-        bf[0] = lds_get(Bs, LoaderB::at(b_row, lg));
+    for (int i = 0; i < TM; i++) af[0][i] = lds_get(As, LoaderA::at(a_row + i * 32, lh));
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
+    for (int j = 0; j < TN; j++) bf[0][j] = lds_get(Bs, LoaderB::at(b_row + j * 32, lh));
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int cur = (s * TN + j) & 1;
-                if (j + 1 < TN) bf[cur ^ 1] = lds_get(Bs, LoaderB::at(b_row + (j + 1) * 16, s * 4 + lg));
-                else if (s == 0) bf[cur ^ 1] = lds_get(Bs, LoaderB::at(b_row, 4 + lg));
-                if (s == 0) {
+    for (int s = 0; s < 4; s++) {
+        if (s + 1 < 4) {
 #pragma unroll
-                    for (int i = j * TM / TN; i < (j + 1) * TM / TN; i++)
-                        af[1][i] = lds_get(As, LoaderA::at(a_row + i * 16, 4 + lg));
-                }
-                // operands swapped: the accumulator then holds, per lane, 4 consecutive n of one m
+            for (int i = 0; i < TM; i++) af[(s + 1) & 1][i] = lds_get(As, LoaderA::at(a_row + i * 32, 2 * (s + 1) + lh));
 #pragma unroll
-                for (int i = 0; i < TM; i++) Cmp::mma(bf[cur], af[s][i], acc[i][j]);
-            }
+            for (int j = 0; j < TN; j++) bf[(s + 1) & 1][j] = lds_get(Bs, LoaderB::at(b_row + j * 32, 2 * (s + 1) + lh));
         }
-    } else {
+        // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            u32x4_t af[TM], bf[2];
+        for (int j = 0; j < TN; j++)
 #pragma unroll
-            for (int i = 0; i < TM; i++) af[i] = lds_get(As, LoaderA::at(a_row + i * 16, s * 4 + lg));
-            bf[0] = lds_get(Bs, LoaderB::at(b_row, s * 4 + lg));
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if (j + 1 < TN) bf[(j + 1) & 1] = lds_get(Bs, LoaderB::at(b_row + (j + 1) * 16, s * 4 + lg));
-#pragma unroll
-                for (int i = 0; i < TM; i++) Cmp::mma(bf[j & 1], af[i], acc[i][j]);
-            }
-        }
+            for (int i = 0; i < TM; i++) Cmp::mma(bf[s & 1][j], af[s & 1][i], acc[i][j]);
     }
 }
 
@@ -536,7 +579,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
                                                                typename Out<Cfg::OUT>::T *__restrict__ C,
                                                                DevProduct g, int tiles_m, int tiles_n) {
     extern __shared__ __align__(16) char smem[];
-    typedef typename Compute<Cfg::CK>::acc_t acc_t;
+    typedef typename Compute32<Cfg::CK>::acc_t acc_t;
     typedef typename Cfg::LoaderA LoaderA;
     typedef typename Cfg::LoaderB LoaderB;
     typedef typename Out<Cfg::OUT>::T out_t;
@@ -544,7 +587,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
-    const int lr = lane & 15, lg = lane >> 4;
+    const int lr = lane & 31, lh = lane >> 5;
 
     long batch;
     int tm, tn;
@@ -559,7 +602,9 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = acc_t{0, 0, 0, 0};
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
 
     LoaderA la;
     LoaderB lb;
@@ -577,7 +622,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
     }
     __syncthreads();
 
-    const int a_row = wave_m * TM * 16 + lr, b_row = wave_n * TN * 16 + lr;
+    const int a_row = wave_m * TM * 32 + lr, b_row = wave_n * TN * 32 + lr;
     for (int kt = 0; kt < KT; kt++) {
         char *cur = smem + (kt & 1) * Cfg::STAGE_BYTES;
         char *nxt = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
@@ -586,7 +631,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
             la.issue_full(opA, m0, (kt + 1) * BK, tid, nxt);
             lb.issue_full(opB, n0, (kt + 1) * BK, tid, nxt + Cfg::A_BYTES);
         }
-        compute_stage<Cfg>(cur, cur + Cfg::A_BYTES, acc, a_row, b_row, lg);
+        compute_stage<Cfg>(cur, cur + Cfg::A_BYTES, acc, a_row, b_row, lh);
         if (more_full) {
             la.commit_full(nxt, tid);
             lb.commit_full(nxt + Cfg::A_BYTES, tid);
@@ -601,26 +646,11 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
     out_t *Cb = C + batch * (long)g.M * g.N;
     const bool vec_ok = (g.N & 3) == 0;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int m = m0 + wave_m * TM * 16 + i * 16 + lr;
-        if (m >= g.M) continue;
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + wave_n * TN * 16 + j * 16 + lg * 4;
-            out_t v[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = Out<Cfg::OUT>::cvt(acc[i][j][e]);
-            out_t *dst = Cb + (long)m * g.N + n;
-            if (vec_ok && n + 3 < g.N) {
-                struct alignas(sizeof(out_t) * 4) Quad { out_t q[4]; };
-                *reinterpret_cast<Quad *>(dst) = Quad{{v[0], v[1], v[2], v[3]}};
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (n + e < g.N) dst[e] = v[e];
-            }
-        }
-    }
+        for (int j = 0; j < TN; j++)
+            store_tile32<Cfg::OUT>(Cb, acc[i][j], m0 + wave_m * TM * 32 + i * 32 + lr, n0 + wave_n * TN * 32 + j * 32, lh,
+                                   g.M, g.N, vec_ok);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -661,53 +691,6 @@ template <class Cfg> int launch_config(hodu_rocm_ctx *ctx, const void *a, const 
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }
-
-// One compute kind = 15 kernels: {KK, KM, MK, MM} x {256x256 with 4 wavefronts, 128x128, 64x64},
-// {KK, KM} x 256x256 with 8 wavefronts, plus a scalar-load 64x64 kernel.  The tile is the largest that still yields at least
-// one workgroup per compute unit.
-constexpr int kVariants = 17;
-template <int CK, int SKA, int SKB, int OUT>
-int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
-                const char *const names[kVariants]) {
-    constexpr int ES = Compute<CK>::ES, EPC = 16 / ES;
-    constexpr int SA = SKA == SK_F8 ? 1 : ES, SB = SKB == SK_F8 ? 1 : ES;
-    constexpr int ROWVEC = ES == 4 ? 4 : 8;
-    const int la = pick_mode(a, g.a_off, g.a_m, g.a_k, g.M, g.K, SA, EPC, ROWVEC, g, g.a_bs);
-    const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, SB, EPC, ROWVEC, g, g.b_bs);
-    if (la == LM_SCALAR || lb == LM_SCALAR) {
-        ctx->last_kernel = names[16];
-        return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_SCALAR>>(ctx, a, b, c, g);
-    }
-    const long cus = ctx->props.multiProcessorCount;
-    auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
-    // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64
-    int size = ctx->force_tile >= 0 ? ctx->force_tile : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 2 : 3;
-    const int combo = (la == LM_MN ? 2 : 0) + (lb == LM_MN ? 1 : 0);
-    // a row-dense LEFT operand needs 32 staging registers more than the 8-wavefront variant has
-    // (two wavefronts share a SIMD's register file): those layouts use the 4-wavefront variant
-    if (size == 0 && la == LM_MN) size = 1;
-    ctx->last_kernel = names[size * 4 + combo];
-#define HODU_MFMA_CASE(SZ, CB, BM, BN, WM, WN, LA, LB)                                                     \
-    if (size == SZ && combo == CB) return launch_config<Config<CK, SKA, SKB, OUT, BM, BN, WM, WN, LA, LB>>(ctx, a, b, c, g);
-#define HODU_MFMA_SIZE(SZ, BM, BN, WM, WN)               \
-    HODU_MFMA_CASE(SZ, 0, BM, BN, WM, WN, LM_K, LM_K)    \
-    HODU_MFMA_CASE(SZ, 1, BM, BN, WM, WN, LM_K, LM_MN)   \
-    HODU_MFMA_CASE(SZ, 2, BM, BN, WM, WN, LM_MN, LM_K)   \
-    HODU_MFMA_CASE(SZ, 3, BM, BN, WM, WN, LM_MN, LM_MN)
-    HODU_MFMA_CASE(0, 0, 256, 256, 2, 4, LM_K, LM_K)
-    HODU_MFMA_CASE(0, 1, 256, 256, 2, 4, LM_K, LM_MN)
-    HODU_MFMA_SIZE(1, 256, 256, 2, 2)
-    HODU_MFMA_SIZE(2, 128, 128, 2, 2)
-    HODU_MFMA_SIZE(3, 64, 64, 2, 2)
-#undef HODU_MFMA_SIZE
-#undef HODU_MFMA_CASE
-    return fail(HODU_ROCM_UNSUPPORTED, "no MFMA variant");
-}
-
-#define HODU_MFMA_NAMES(P)                                                                                       \
-    {P "_256x256w8_KK", P "_256x256w8_KM", P "_256x256w8_MK", P "_256x256w8_MM", P "_256x256_KK", P "_256x256_KM", \
-     P "_256x256_MK",   P "_256x256_MM",   P "_128x128_KK",   P "_128x128_KM",   P "_128x128_MK", P "_128x128_MM", \
-     P "_64x64_KK",     P "_64x64_KM",     P "_64x64_MK",     P "_64x64_MM",     P "_64x64_scalar"}
 
 }  // namespace mfma
 }  // namespace hodu

@@ -1,4 +1,4 @@
-#include "gemm_mfma.hpp"
+#include "gemm_mfma_launch.hpp"
 namespace hodu {
 int launch_mfma_bf16(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
     static const char *const names[mfma::kVariants] = HODU_MFMA_NAMES("mfma_bf16");

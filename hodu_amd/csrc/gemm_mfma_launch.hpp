@@ -1,0 +1,71 @@
+// Variant selection and launch for one compute kind of the MFMA tile kernels.
+#pragma once
+
+#include "gemm_mfma.hpp"
+#include "gemm_mfma_pipe.hpp"
+
+namespace hodu {
+namespace mfma {
+
+// One compute kind: {KK, KM, MK, MM} x {256x256 with 4 wavefronts, 128x128, 64x64}, {KK, KM} x 256x256
+// with 8 wavefronts, a scalar-load 64x64 kernel, and -- when both operands are stored in the compute
+// type -- the four software-pipelined KK kernels of gemm_mfma_pipe.hpp.  The tile is the largest that
+// still yields at least one workgroup per compute unit.
+constexpr int kVariants = 21;
+template <int CK, int SKA, int SKB, int OUT>
+int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
+                const char *const names[kVariants]) {
+    constexpr int ES = Compute<CK>::ES, EPC = 16 / ES;
+    constexpr int SA = SKA == SK_F8 ? 1 : ES, SB = SKB == SK_F8 ? 1 : ES;
+    constexpr int ROWVEC = ES == 4 ? 4 : 8;
+    const int la = pick_mode(a, g.a_off, g.a_m, g.a_k, g.M, g.K, SA, EPC, ROWVEC, g, g.a_bs);
+    const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, SB, EPC, ROWVEC, g, g.b_bs);
+    if (la == LM_SCALAR || lb == LM_SCALAR) {
+        ctx->last_kernel = names[16];
+        return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_SCALAR>>(ctx, a, b, c, g);
+    }
+    const long cus = ctx->props.multiProcessorCount;
+    auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
+    // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64
+    const int forced = ctx->force_tile;
+    int size = forced >= 0 ? forced % 10 : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 2 : 3;
+    const int combo = (la == LM_MN ? 2 : 0) + (lb == LM_MN ? 1 : 0);
+    if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
+        // testing hook values 10..13 pin the pipelined kernel's tile, 0..3 the general kernel's
+        if (pipe_eligible<CK>(la, lb, g) && (forced < 0 || forced >= 10)) {
+            ctx->last_kernel = names[17 + size];
+            if (size == 0) return launch_pipe<PipeConfig<CK, OUT, 256, 256, 2, 4>>(ctx, a, b, c, g);
+            if (size == 1) return launch_pipe<PipeConfig<CK, OUT, 256, 256, 2, 2>>(ctx, a, b, c, g);
+            if (size == 2) return launch_pipe<PipeConfig<CK, OUT, 128, 128, 2, 2>>(ctx, a, b, c, g);
+            return launch_pipe<PipeConfig<CK, OUT, 64, 64, 2, 2>>(ctx, a, b, c, g);
+        }
+    }
+    // a row-dense LEFT operand needs 32 staging registers more than the 8-wavefront variant has
+    // (two wavefronts share a SIMD's register file): those layouts use the 4-wavefront variant
+    if (size == 0 && la == LM_MN) size = 1;
+    ctx->last_kernel = names[size * 4 + combo];
+#define HODU_MFMA_CASE(SZ, CB, BM, BN, WM, WN, LA, LB)                                                     \
+    if (size == SZ && combo == CB) return launch_config<Config<CK, SKA, SKB, OUT, BM, BN, WM, WN, LA, LB>>(ctx, a, b, c, g);
+#define HODU_MFMA_SIZE(SZ, BM, BN, WM, WN)               \
+    HODU_MFMA_CASE(SZ, 0, BM, BN, WM, WN, LM_K, LM_K)    \
+    HODU_MFMA_CASE(SZ, 1, BM, BN, WM, WN, LM_K, LM_MN)   \
+    HODU_MFMA_CASE(SZ, 2, BM, BN, WM, WN, LM_MN, LM_K)   \
+    HODU_MFMA_CASE(SZ, 3, BM, BN, WM, WN, LM_MN, LM_MN)
+    HODU_MFMA_CASE(0, 0, 256, 256, 2, 4, LM_K, LM_K)
+    HODU_MFMA_CASE(0, 1, 256, 256, 2, 4, LM_K, LM_MN)
+    HODU_MFMA_SIZE(1, 256, 256, 2, 2)
+    HODU_MFMA_SIZE(2, 128, 128, 2, 2)
+    HODU_MFMA_SIZE(3, 64, 64, 2, 2)
+#undef HODU_MFMA_SIZE
+#undef HODU_MFMA_CASE
+    return fail(HODU_ROCM_UNSUPPORTED, "no MFMA variant");
+}
+
+#define HODU_MFMA_NAMES(P)                                                                                       \
+    {P "_256x256w8_KK", P "_256x256w8_KM", P "_256x256w8_MK", P "_256x256w8_MM", P "_256x256_KK", P "_256x256_KM", \
+     P "_256x256_MK",   P "_256x256_MM",   P "_128x128_KK",   P "_128x128_KM",   P "_128x128_MK", P "_128x128_MM", \
+     P "_64x64_KK",     P "_64x64_KM",     P "_64x64_MK",     P "_64x64_MM",     P "_64x64_scalar",                \
+     P "_pipe256x256w8_KK", P "_pipe256x256_KK", P "_pipe128x128_KK", P "_pipe64x64_KK"}
+
+}  // namespace mfma
+}  // namespace hodu

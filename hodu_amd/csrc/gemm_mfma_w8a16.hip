@@ -1,6 +1,6 @@
 // bf16 activations x f8e4m3 weights -> bf16: the weight's to_dtype(bf16) happens between the global
 // load and the LDS store.
-#include "gemm_mfma.hpp"
+#include "gemm_mfma_launch.hpp"
 namespace hodu {
 int launch_mfma_w8a16(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
     static const char *const names[mfma::kVariants] = HODU_MFMA_NAMES("mfma_bf16_f8w");

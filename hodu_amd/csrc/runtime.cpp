@@ -167,7 +167,8 @@ const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_k
 
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
-    if (tile < -1 || tile > 3) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3", tile);
+    if (tile < -1 || (tile > 3 && tile < 10) || tile > 13)
+        return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3 or 10..13", tile);
     ctx->force_tile = tile;
     return HODU_ROCM_OK;
 }

@@ -32,7 +32,8 @@ using mfma::SK_F8;
 using mfma::SK_SAME;
 
 constexpr int WAVES = 8;
-constexpr int UNROLL = 4;  // weight vectors in flight per lane
+constexpr int CHUNK = 8;                 // weight vectors in flight per lane (8 KB per wavefront)
+constexpr int X_LDS_LIMIT = 144 * 1024;  // bytes of LDS the staged left operand may take
 
 __device__ __forceinline__ u32x4_t ldg16(const char *p) { return *reinterpret_cast<const u32x4_t *>(p); }
 
@@ -48,18 +49,22 @@ __device__ __forceinline__ void widen_f8x16(const u32x4_t &w, u32x4_t &lo, u32x4
     hi.w = bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, true));
 }
 
-// CK: type fed to the matrix core; SKB: weight storage (CK itself, or f8e4m3 widened to bf16)
+// CK: type fed to the matrix core; SKB: weight storage (CK itself, or f8e4m3 widened to bf16).
+// x_pitch > 0: the left operand (M x K, a few KB) is first copied to LDS, rows x_pitch bytes apart,
+// so that the MFMA's left fragments come from LDS instead of nearly-empty global loads (for M = 1
+// only 4 of 64 lanes carry a left-operand row).  x_pitch == 0: it does not fit; read it from global.
 template <int CK, int SKB, int OUT>
 __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *__restrict__ X,
                                                                   const char *__restrict__ W,
                                                                   typename Out<OUT>::T *__restrict__ Y, DevProduct g,
-                                                                  int tiles_n, int k_per_wave) {
+                                                                  int tiles_n, int k_per_wave, int x_pitch) {
     typedef Compute<CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<OUT>::T out_t;
     constexpr int ES = Cmp::ES;                         // bytes per element of x (and of W unless f8)
     constexpr int SB = SKB == SK_F8 ? 1 : ES;           // bytes per stored weight element
     constexpr int EPL = 16 / SB;                        // weight elements per lane per load
+    extern __shared__ __align__(16) char xs[];
     __shared__ acc_t red[WAVES][64];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -79,26 +84,53 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *_
     int kend = kbeg + k_per_wave;
     kend = kend < g.K ? kend : g.K;
 
-    acc_t acc = acc_t{0, 0, 0, 0};
-    for (int kb = kbeg; kb < kend; kb += UNROLL * 4 * EPL) {
-        u32x4_t wv[UNROLL], xa[UNROLL], xb[UNROLL];
+    // the first chunk of weight loads goes out before anything else
+    u32x4_t wv[CHUNK];
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const int k = kb + (u * 4 + lg) * EPL;
-            const bool ok = k < kend;
-            wv[u] = ok ? ldg16(wrow + (long)k * SB) : mfma::zero4();
-            xa[u] = (ok && has_x) ? ldg16(xrow + (long)k * ES) : mfma::zero4();
-            if (SKB == SK_F8) xb[u] = (ok && has_x) ? ldg16(xrow + (long)(k + 8) * ES) : mfma::zero4();
+    for (int u = 0; u < CHUNK; u++) {
+        const int k = kbeg + (u * 4 + lg) * EPL;
+        wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+    }
+    if (x_pitch > 0) {
+        const int vec_per_row = g.K * ES / 16;
+        for (int v = tid; v < g.M * vec_per_row; v += WAVES * 64) {
+            const int row = v / vec_per_row, col = v - row * vec_per_row;
+            *reinterpret_cast<u32x4_t *>(xs + row * x_pitch + col * 16) = ldg16(X + (ao + (long)row * g.a_m) * ES + col * 16);
+        }
+        __syncthreads();
+    }
+    const char *xl = xs + lr * x_pitch;
+
+    acc_t acc = acc_t{0, 0, 0, 0};
+    for (int kb = kbeg; kb < kend; kb += CHUNK * 4 * EPL) {
+        if (kb != kbeg) {
+#pragma unroll
+            for (int u = 0; u < CHUNK; u++) {
+                const int k = kb + (u * 4 + lg) * EPL;
+                wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+            }
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
+        for (int u = 0; u < CHUNK; u++) {
+            const int k = kb + (u * 4 + lg) * EPL;
+            const bool ok = k < kend && has_x;
+            u32x4_t xa = mfma::zero4(), xb = mfma::zero4();
+            if (x_pitch > 0) {
+                if (ok) {
+                    xa = *reinterpret_cast<const u32x4_t *>(xl + k * ES);
+                    if (SKB == SK_F8) xb = *reinterpret_cast<const u32x4_t *>(xl + (k + 8) * ES);
+                }
+            } else if (ok) {
+                xa = ldg16(xrow + (long)k * ES);
+                if (SKB == SK_F8) xb = ldg16(xrow + (long)(k + 8) * ES);
+            }
             if (SKB == SK_F8) {
                 u32x4_t lo, hi;
                 widen_f8x16(wv[u], lo, hi);
-                Cmp::mma(xa[u], lo, acc);
-                Cmp::mma(xb[u], hi, acc);
+                Cmp::mma(xa, lo, acc);
+                Cmp::mma(xb, hi, acc);
             } else {
-                Cmp::mma(xa[u], wv[u], acc);
+                Cmp::mma(xa, wv[u], acc);
             }
         }
     }
@@ -143,9 +175,21 @@ int run_kdense(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const 
     if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
     const int step = 4 * EPL;  // k covered by one wavefront-wide load
     int k_per_wave = ((g.K + WAVES - 1) / WAVES + step - 1) / step * step;
+    // rows of the staged left operand are padded by 16 bytes so that the 16 row slots of a fragment
+    // read hit different LDS banks
+    const long pitch = (long)g.K * ES + 16;
+    const int x_pitch = (g.M * pitch <= X_LDS_LIMIT) ? (int)pitch : 0;
+    const size_t lds = x_pitch > 0 ? (size_t)g.M * x_pitch : 0;
+    auto kernel = skinny_kdense_kernel<CK, SKB, OUT>;
+    static bool configured = false;  // benign race: the attribute call is idempotent
+    if (!configured) {
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     X_LDS_LIMIT));
+        configured = true;
+    }
     ctx->last_kernel = name;
-    hipLaunchKernelGGL((skinny_kdense_kernel<CK, SKB, OUT>), dim3((unsigned)blocks), dim3(WAVES * 64), 0, ctx->stream,
-                       (const char *)x, (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WAVES * 64), lds, ctx->stream, (const char *)x,
+                       (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave, x_pitch);
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }

@@ -81,7 +81,8 @@ int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
 /* name of the kernel family the last matmul/dot call on this context dispatched to (diagnostics) */
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
 /* testing hook: pin the MFMA tile variant (0 = 256x256 with 8 wavefronts, 1 = 256x256 with 4,
- * 2 = 128x128, 3 = 64x64, -1 = automatic) so that every compiled variant can be exercised at small sizes */
+ * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; -1 = automatic) so that
+ * every compiled variant can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
 /* measurement hook: issues the same product `iters` times back to back from C (no per-launch
  * interpreter overhead), cycling through `n_rhs` right-hand buffers so a small operand cannot sit

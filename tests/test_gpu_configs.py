@@ -59,7 +59,7 @@ def test_config2_bf16_batched_transposed(ctx):
     b = H.f32_to_bf16_rne((H.rng(202).standard_normal(B * n * n) / 32).astype(np.float32))
     lv, rv = V([B, n, n]), V([B, n, n]).t()  # rhs: transposed view of contiguous [B, N, K]
     got = run_product(ctx, "matmul", "bf16", a, b, H.matmul_md(lv, rv)).reshape(B, n, n)
-    assert ctx.last_kernel().startswith("mfma_bf16_256x256") and ctx.last_kernel().endswith("_KK")
+    assert ctx.last_kernel().startswith("mfma_bf16_") and "256x256" in ctx.last_kernel() and ctx.last_kernel().endswith("_KK")
     for bi in (0, 7, 15):
         rows = V([n, n], offset=bi * n * n).slice(0, 3, n, 97)
         md = H.dot_md(rows, V([n, n], offset=bi * n * n).t())
@@ -133,13 +133,13 @@ def test_config5_mlp_broadcast(ctx, wkind):
     xv = V([b, s, d])
     up_v = V([d, f]).broadcast_to([b, d, f])
     y = run_product(ctx, "matmul", name, x, w_up, H.matmul_md(xv, up_v))
-    assert ctx.last_kernel().startswith(prefix + "256x256") and ctx.last_kernel().endswith("_KM"), ctx.last_kernel()
+    assert ctx.last_kernel().startswith(prefix) and "256x256" in ctx.last_kernel() and ctx.last_kernel().endswith("_KM"), ctx.last_kernel()
     rows = V([b * s, d]).slice(0, 7, b * s, 311)
     check_rows(y.reshape(b * s, f)[7::311].ravel(), "bf16", r_dt, x, w_up, H.dot_md(rows, V([d, f])), d, 2e-2)
     # down: Y [8,512,14336] x W_down, stored [4096,14336] and passed as a transposed, broadcast view
     yv = V([b, s, f])
     down_v = V([d, f]).t().broadcast_to([b, f, d])
     z = run_product(ctx, "matmul", name, y, w_down, H.matmul_md(yv, down_v))
-    assert ctx.last_kernel().startswith(prefix + "256x256") and ctx.last_kernel().endswith("_KK"), ctx.last_kernel()
+    assert ctx.last_kernel().startswith(prefix) and "256x256" in ctx.last_kernel() and ctx.last_kernel().endswith("_KK"), ctx.last_kernel()
     rows = V([b * s, f]).slice(0, 11, b * s, 409)
     check_rows(z.reshape(b * s, d)[11::409].ravel(), "bf16", r_dt, y, w_down, H.dot_md(rows, V([d, f]).t()), f, 2e-2)

@@ -53,6 +53,23 @@ def test_every_variant_ragged(ctx, kind, tile):
     ctx.force_tile(-1)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "f16", "f32", "i32_i8i8"])
+@pytest.mark.parametrize("tile,name", [(10, "pipe256x256w8"), (11, "pipe256x256"), (12, "pipe128x128"), (13, "pipe64x64")])
+def test_pipelined_kk_variants(ctx, kind, tile, name):
+    """the software-pipelined kernel (both operands k-dense): 1 to 11 stages of 64 bytes, ragged M and N"""
+    prefix = KINDS[kind][0]
+    ctx.force_tile(tile)
+    es = {"bf16": 2, "f16": 2, "f32": 4, "i32_i8i8": 1}[kind]
+    for stages in (1, 2, 3, 4, 5, 11):
+        K = stages * 64 // es
+        check_product(ctx, "dot", kind, V([296, K]), V([200, K]).t(), seed=stages, expect_kernel=f"{prefix}_{name}_KK")
+    # batched, with a row-sliced operand (leading dimension > K) and an offset
+    K = 6 * 64 // es
+    check_product(ctx, "matmul", kind, V([3, 72, 2 * K]).slice(2, K, 2 * K), V([3, 80, K], offset=64).t(), seed=7,
+                  expect_kernel=f"{prefix}_{name}_KK")
+    ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("kind", list(KINDS))
 def test_scalar_load_variant(ctx, kind):
     prefix, _, _ = KINDS[kind]
