@@ -39,7 +39,11 @@ INFINITY_CACHE_BYTES = 256 << 20
 
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc runs summarised under
 # profiles/ (FETCH_SIZE + WRITE_SIZE scaled by the copy-kernel calibration); None = not measured
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    "mfma_bf16_pipe256x256w8_KK@c2": 100.57e6,
+    "skinny_bf16_f8w@c3_m1": 16.90e6,
+    "mfma_bf16_pipe256x256w8_KK@c5_down_bf16": 735.9e6,
+}
 
 
 def bf16(x):
@@ -164,14 +168,15 @@ def time_case(ctx, case, steps, warmup):
             "tflops": tflops, "algorithmic_gbs": gbs, "weight_buffers_rotated": copies, "roofline": roof}
 
 
-def cpu_baseline_c2(budget_s=12.0):
+def cpu_baseline_c2(budget_s=15.0):
     """hodu's CPU path for config 2, timed on a bounded sample.
 
     hodu routes a >= 3-D matmul to hodu_cpu_matmul_bf16, whose batched path runs on ONE thread and
     accumulates in bf16 (crates/hodu_cpu_kernels/kernels/ops_matrix.c:292-337); through the public
     API the transposed operand is first copied (tensor/ops/shape.rs:232-237), which is not timed.
-    The sample is the first `rows` rows of batch 0 against the full [1024,1024] right operand;
-    the rate is per flop, so it scales linearly to the whole job.
+    The sample is the first few of the 16 batches (all 1024 rows of each, or fewer rows of one batch
+    on a slow host), sized by a short probe to about `budget_s` seconds; the rate is per flop, so it
+    scales linearly to the whole job.
     """
     import helpers as H
     import oracle
@@ -179,19 +184,20 @@ def cpu_baseline_c2(budget_s=12.0):
     a = bf16(normal(201, n * n, 1 / 32))
     b = bf16(normal(202, n * n, 1 / 32))
     oracle.set_threads(1)
-    rows, rate = 8, None
-    t_used = 0.0
-    while True:
-        lv, rv = H.View([1, rows, n]), H.View([1, n, n]).t()
-        t0 = time.perf_counter()
-        oracle.matmul_asis("bf16", a, b, H.matmul_md(lv, rv))
-        dt = time.perf_counter() - t0
-        t_used += dt
-        rate = 2.0 * rows * n * n / dt
-        nxt = min(n, int(rows * min(8.0, max(2.0, (budget_s - t_used) / max(dt, 1e-6) * 0.5))))
-        if t_used + dt * nxt / rows > budget_s or rows >= n or nxt <= rows:
-            break
-        rows = nxt
+    # a short probe fixes the rate, then one run sized to the budget: `rows` rows of each of `nb` batches
+    lv, rv = H.View([1, 32, n]), H.View([1, n, n]).t()
+    t0 = time.perf_counter()
+    oracle.matmul_asis("bf16", a[:32 * n], b, H.matmul_md(lv, rv))
+    probe = time.perf_counter() - t0
+    rows_total = max(32, int(budget_s / (probe / 32)))
+    nb = max(1, min(16, rows_total // n))
+    rows = n if rows_total >= n else rows_total
+    lv, rv = H.View([nb, rows, n]), H.View([nb, n, n]).t()
+    a_s, b_s = np.tile(a[:rows * n], nb), np.tile(b, nb)
+    t0 = time.perf_counter()
+    oracle.matmul_asis("bf16", a_s, b_s, H.matmul_md(lv, rv))
+    t_used = time.perf_counter() - t0
+    rate = 2.0 * nb * rows * n * n / t_used
     # the f32-accumulated comparator path (to_dtype(f32) + sgemm), all cores, for scale
     af = H.bf16_to_f32(a).reshape(n, n)
     bfm = H.bf16_to_f32(b).reshape(n, n)
@@ -203,8 +209,8 @@ def cpu_baseline_c2(budget_s=12.0):
     sgemm_rate = 2.0 * n ** 3 * reps / (time.perf_counter() - t0)
     oracle.set_threads(os.cpu_count() or 1)
     return {"value": rate / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"hodu_cpu_matmul_bf16 semantics (bf16-accumulate, batched path, 1 thread) on {rows} of 1024 rows "
-                      f"of batch 0 x full [1024,1024]^T-view; {t_used:.1f} s of CPU work",
+            "sample": f"hodu_cpu_matmul_bf16 semantics (bf16-accumulate, batched path, 1 thread) on {nb} of the 16 "
+                      f"batches, {rows} of 1024 rows each, x full [1024,1024]^T-view; {t_used:.1f} s of CPU work",
             "host_cores_online": os.cpu_count(),
             "f32_comparator_sgemm_tflops": sgemm_rate / 1e12,
             "f32_comparator_note": "to_dtype(f32) inputs through numpy's OpenBLAS sgemm on all host cores (1024^3)"}
@@ -230,6 +236,21 @@ def main():
     ctx = ffi.Context(0)
     info = ctx.device_info()
     ctx.force_tile(args.force_tile)
+    if args.only == "copy":
+        # calibration for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain dense copy of known size
+        # (hodu_rocm_contiguous on a contiguous f32 buffer reads n bytes and writes n bytes)
+        import helpers as H
+        n = 64 << 20
+        src, dst = ctx.alloc(4 * n), ctx.alloc(4 * n)
+        ctx.fill(src, 0)
+        md = H.cast_md(H.View([n]))
+        for _ in range(args.steps):
+            ctx.contiguous("f32", src, dst, md)
+        ctx.sync()
+        print(json.dumps({"config": "copy", "kernel": ctx.last_kernel(), "bytes_read": 4 * n, "bytes_written": 4 * n,
+                          "launches": args.steps}))
+        ctx.close()
+        return
     if args.only:
         case = next(c for c in build_cases({args.only.split("_")[0]}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup)))
