@@ -17,6 +17,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "_build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libhodu_rocm_kernels.so")
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(LIB_DIR, "libhodu_rocm_host.so")
 
 ARCH = "gfx950"
 # -packed-fp32-ops off: keep hipcc from forming v_pk_{add,mul,fma}_f32 out of scalar float code
@@ -63,7 +65,23 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     os.replace(tmp, LIB)
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
+    build_host(verbose)
     return LIB
+
+
+def build_host(verbose: bool = True) -> str:
+    """The host-side Tensor/Layout/storage mirror: plain C++ over the C ABI, linked against the kernel library."""
+    tmp = HOST_LIB + ".tmp"
+    cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra", f"-I{os.path.join(ROOT, 'include')}",
+           f"-I{HOST_DIR}", os.path.join(HOST_DIR, "capi.cpp"), "-o", tmp, f"-L{LIB_DIR}", "-lhodu_rocm_kernels",
+           "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host library build failed:\n{r.stderr[-4000:]}")
+    os.replace(tmp, HOST_LIB)
+    if verbose:
+        print(f"built {HOST_LIB}", file=sys.stderr)
+    return HOST_LIB
 
 
 if __name__ == "__main__":

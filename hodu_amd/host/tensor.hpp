@@ -1,0 +1,153 @@
+// Host-side mirror of the hodu Tensor methods on the matmul / dot / to_dtype path
+// (crates/hodu_core/src/tensor/ops/matrix.rs, cast_memory.rs, shape.rs).  A Tensor is an immutable
+// (storage, layout) pair; views share the storage (tensor/internal.rs:50-79).
+#pragma once
+
+#include "storage.hpp"
+
+namespace hodu_host {
+
+// How matmul_batched treats a non-contiguous operand:
+//   Reference  exactly hodu today: Tensor::broadcast / transpose / reshape / squeeze first force
+//              contiguity (shape.rs:232-237, :296-299), so a transposed weight is copied per call
+//   NoCopy     the patched path: the broadcast layout is built straight on the existing layout
+//              (Layout::broadcast_to) and the strided view goes to the kernel as is
+enum class MatmulMode { Reference = 0, NoCopy = 1 };
+
+inline MatmulMode &matmul_mode() {
+    static MatmulMode mode = MatmulMode::NoCopy;
+    return mode;
+}
+
+class Tensor {
+public:
+    Tensor(std::shared_ptr<const RocmStorage> storage, Layout layout)
+        : storage_(std::move(storage)), layout_(std::move(layout)) {}
+
+    // Tensor::from_bytes-like constructor: row-major elements of `dtype`, given as raw bits
+    static Tensor from_bytes(int device, DType dtype, const Dims &shape, const void *bytes, size_t nbytes) {
+        const size_t n = product(shape);
+        if (nbytes != n * dtype_size(dtype))
+            throw Error(ErrorKind::InvalidArgument, "from_bytes: byte count does not match the shape");
+        auto dev = RocmDevice::get(device);
+        return Tensor(std::make_shared<RocmStorage>(RocmStorage::from_host(dev, dtype, bytes, n)), Layout::from_shape(shape));
+    }
+
+    const Layout &layout() const { return layout_; }
+    const Dims &shape() const { return layout_.shape(); }
+    DType dtype() const { return storage_->dtype(); }
+    DType physical_dtype() const { return storage_->physical_dtype(); }
+    bool is_contiguous() const { return layout_.is_contiguous(); }  // tensor/core.rs:222-224
+    size_t size() const { return layout_.size(); }
+    bool shares_storage_with(const Tensor &o) const { return storage_->ptr() == o.storage_->ptr(); }
+
+    void to_bytes(void *out) const { storage_->to_host(layout_, out); }
+
+    // cast_memory.rs:11-38: result is contiguous in the tensor's shape
+    Tensor to_dtype(DType target) const {
+        return Tensor(std::make_shared<RocmStorage>(storage_->to_dtype(layout_, target)), Layout::from_shape(shape()));
+    }
+
+    // cast_memory.rs:56-83: an already contiguous tensor is returned as is (offset included)
+    Tensor contiguous() const {
+        if (is_contiguous()) return *this;
+        return Tensor(std::make_shared<RocmStorage>(storage_->contiguous(layout_)), Layout::from_shape(shape()));
+    }
+
+    // shape.rs:13-60, :125-170, :232-279, :295-346: each forces contiguity first, then is a pure view
+    Tensor reshape(const Dims &s) const { return is_contiguous() ? view(layout_.reshape(s)) : contiguous().reshape(s); }
+    Tensor squeeze(const std::vector<int> &d) const { return is_contiguous() ? view(layout_.squeeze(d)) : contiguous().squeeze(d); }
+    Tensor unsqueeze(int d) const { return is_contiguous() ? view(layout_.unsqueeze(d)) : contiguous().unsqueeze(d); }
+    Tensor broadcast(const Dims &s) const { return is_contiguous() ? view(layout_.broadcast_to(s)) : contiguous().broadcast(s); }
+    Tensor transpose(int a, int b) const { return is_contiguous() ? view(layout_.transpose(a, b)) : contiguous().transpose(a, b); }
+    Tensor t() const { return transpose(-2, -1); }
+    Tensor slice(int dim, int start, bool has_end, int end, int step) const {
+        return view(layout_.slice(dim, start, has_end, end, step));
+    }
+    // a view with an arbitrary layout over the same storage (bounds are checked when it is used)
+    Tensor view(const Layout &l) const { return Tensor(storage_, l); }
+
+    // matrix.rs:13-92
+    Tensor matmul(const Tensor &other) const {
+        const size_t ln = layout_.ndim(), rn = other.layout_.ndim();
+        if (ln < 1 || rn < 1) throw incompatible(other, "matmul");
+        if (ln == 1 && rn == 1) return inner(other, "matmul");
+        if (ln == 2 && rn == 1) {
+            if (shape()[1] != other.shape()[0]) throw incompatible(other, "matmul");
+            return dot_2d(other.reshape({other.shape()[0], 1})).squeeze({-1});
+        }
+        if (ln == 1 && rn == 2) {
+            if (shape()[0] != other.shape()[0]) throw incompatible(other, "matmul");
+            return reshape({1, shape()[0]}).dot_2d(other).squeeze({0});
+        }
+        if (ln == 2 && rn == 2) return dot_2d(other);
+        return matmul_batched(other);
+    }
+
+    // matrix.rs:226-299: 1-D and 2-D only
+    Tensor dot(const Tensor &other) const {
+        const size_t ln = layout_.ndim(), rn = other.layout_.ndim();
+        if (ln == 1 && rn == 1) return inner(other, "dot");
+        if (ln == 2 && rn == 1) {
+            if (shape()[1] != other.shape()[0]) throw incompatible(other, "dot");
+            return dot_2d(other.reshape({other.shape()[0], 1})).squeeze({-1});
+        }
+        if (ln == 1 && rn == 2) {
+            if (shape()[0] != other.shape()[0]) throw incompatible(other, "dot");
+            return reshape({1, shape()[0]}).dot_2d(other).squeeze({0});
+        }
+        if (ln == 2 && rn == 2) return dot_2d(other);
+        throw Error(ErrorKind::InternalError, "dot - only supports 1D and 2D tensors. Use matmul() for batched operations");
+    }
+
+private:
+    Error incompatible(const Tensor &o, const char *op) const {
+        return Error(ErrorKind::IncompatibleShapes, std::string(op) + ": " + dims_str(shape()) + " vs " + dims_str(o.shape()));
+    }
+
+    // matrix.rs:38-47 computes mul + sum_all for two vectors.  Element-wise ops are not part of this
+    // backend; the same number is produced as the [1,K] x [K,1] product (for floating point the
+    // summation order may differ from the reference's reduce kernel).  Result shape: scalar [].
+    Tensor inner(const Tensor &other, const char *op) const {
+        if (shape()[0] != other.shape()[0]) throw incompatible(other, op);
+        const size_t k = shape()[0];
+        return reshape({1, k}).dot_2d(other.reshape({k, 1})).reshape({});
+    }
+
+    // matrix.rs:302-371: both layouts go to the kernel unchanged
+    Tensor dot_2d(const Tensor &other) const {
+        if (shape()[1] != other.shape()[0]) throw incompatible(other, "dot");
+        auto out = std::make_shared<RocmStorage>(storage_->call_ops_dot(*other.storage_, layout_, other.layout_));
+        return Tensor(out, Layout::from_shape({shape()[0], other.shape()[1]}));
+    }
+
+    // matrix.rs:95-224
+    Tensor matmul_batched(const Tensor &other) const {
+        const Dims &ld = shape(), &rd = other.shape();
+        const size_t ln = ld.size(), rn = rd.size();
+        if (ln < 2 || rn < 2 || ld[ln - 1] != rd[rn - 2]) throw incompatible(other, "matmul");
+        const size_t lb = ln - 2, rb = rn - 2, bn = std::max(lb, rb);
+        Dims batch(bn);
+        for (size_t i = 0; i < bn; i++) {  // i counts from the innermost batch dim
+            const size_t a = i < lb ? ld[lb - 1 - i] : 1, b = i < rb ? rd[rb - 1 - i] : 1;
+            if (a != 1 && b != 1 && a != b) throw incompatible(other, "matmul");
+            batch[bn - 1 - i] = std::max(a, b);
+        }
+        Dims ls = batch, rs = batch;
+        ls.push_back(ld[ln - 2]); ls.push_back(ld[ln - 1]);
+        rs.push_back(rd[rn - 2]); rs.push_back(rd[rn - 1]);
+        const bool copy = matmul_mode() == MatmulMode::Reference;
+        const Tensor l = copy ? broadcast(ls) : view(layout_.broadcast_to(ls));
+        const Tensor r = copy ? other.broadcast(rs) : other.view(other.layout_.broadcast_to(rs));
+        Dims out_shape = batch;
+        out_shape.push_back(ld[ln - 2]);
+        out_shape.push_back(rd[rn - 1]);
+        auto out = std::make_shared<RocmStorage>(l.storage_->call_ops_matmul(*r.storage_, l.layout_, r.layout_));
+        return Tensor(out, Layout::from_shape(out_shape));
+    }
+
+    std::shared_ptr<const RocmStorage> storage_;
+    Layout layout_;
+};
+
+}  // namespace hodu_host
