@@ -1,25 +1,27 @@
 // Software-pipelined MFMA tile kernel for products whose operands are BOTH k-dense in their
 // compute type (bf16 x bf16, f16 x f16, i8 x i8, f32 x f32 with `stride_k == 1`, 16-byte aligned
-// rows, K a multiple of 64 bytes).  Same tiles, same MFMA instructions and same results as the
+// rows, K a multiple of 128 bytes).  Same tiles, same MFMA instructions and same results as the
 // general kernel in gemm_mfma.hpp; what differs is how the K loop is fed:
 //
-//   * K advances 64 bytes per stage (32 bf16 / 64 i8 / 16 f32: one MFMA k-slice), four stages of
-//     LDS; each stage is written by LDS-DMA only (global_load_lds_dwordx4: no staging registers,
-//     no ds_write), three stages ahead of the stage being multiplied;
-//   * a stage is an array of 1 KB blocks, one block = 16 rows x 64 B = exactly what one wavefront-wide
-//     DMA instruction writes.  The four 16-byte chunks of a row are XOR-swizzled by (row / 4) % 4 --
-//     applied to the SOURCE address of the DMA -- so that the MFMA fragment read (16 lanes = 16
-//     rows, one chunk) touches all 64 banks once;
-//   * the MFMA fragments live in one register set that is refilled half a step ahead of its use, each
-//     ds_read_b128 interleaved with the MFMAs of the other k-slice, so that LDS (128 B/clk, about as
-//     busy as the matrix cores at this tile shape) and the matrix cores run side by side instead of
-//     in alternating bursts;
-//   * the barrier is a bare s_barrier preceded by an s_waitcnt vmcnt(n) that leaves the DMA of the
-//     two newest stages in flight (a __syncthreads() would drain them).
+//   * K advances 128 bytes per stage (64 bf16 / 128 i8 / 32 f32 = four MFMA k-slices).  Every DMA
+//     request is one whole 128-byte cache line of one row: fetching rows in 64-byte halves feeds a
+//     compute unit at 29 B/clk, whole lines at 47 B/clk (measured on the 4096 x 4096 x 14336 sweep);
+//   * two stages of LDS, written by LDS-DMA only (global_load_lds_dwordx4: no staging registers, no
+//     ds_write).  The DMA of stage t+2 is issued, into the buffer stage t just vacated, while the
+//     last k-slice of stage t multiplies, so it has the whole of stage t+1 to land;
+//   * a stage is an array of 1 KB blocks, one block = 8 rows x 128 B = exactly what one wavefront-wide
+//     DMA instruction writes, 128 bytes apart; the eight 16-byte chunks of a row are XOR-swizzled by
+//     row % 8 -- applied to the SOURCE address of the DMA -- so that an MFMA fragment read (16 lanes =
+//     16 rows, one chunk) touches all 64 banks once (lds_swizzled in gemm_mfma.hpp);
+//   * the MFMA fragments live in one register set that is refilled one k-slice ahead of its use, each
+//     ds_read_b128 interleaved with the MFMAs of the previous slice, so that LDS and the matrix cores
+//     run side by side instead of in alternating bursts;
+//   * one bare s_barrier per stage, preceded by s_waitcnt vmcnt(0) lgkmcnt(0): at that point the only
+//     DMA in flight is the next stage's, and every fragment read of the current stage has returned.
 //
-// Hazards.  DMA of stage t+3 is issued right after the barrier of step t into the buffer that held
-// stage t-1.  Every wavefront reaches that barrier only after issuing the slice-0 MFMAs of stage t,
-// which follow its last reads of stage t-1 and the MFMAs that consumed them.
+// Hazards.  The barrier in stage t is reached by a wavefront only after all its reads of stage t
+// have RETURNED (lgkmcnt(0)) and its own share of stage t+1 has landed (vmcnt(0)); past it, stage t's
+// buffer is dead for everybody and stage t+1 is complete for everybody.
 #pragma once
 
 #include <type_traits>
@@ -29,31 +31,33 @@
 namespace hodu {
 namespace mfma {
 
-constexpr int P_ROW_BYTES = 64;
-constexpr int P_STAGES = 4;
-constexpr int P_AHEAD = 3;
+constexpr int P_ROW_BYTES = 128;   // == ROW_BYTES of the swizzled layout
+constexpr int P_SLICES = 4;        // 32-byte k-slices per stage
 
 // s_waitcnt immediate for gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
 constexpr int waitcnt_vm(int n) { return (n & 15) | 0x70 | 0xF00 | ((n >> 4) << 14); }
+constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | 0x70 | ((n >> 4) << 14); }
 
 template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_> struct PipeConfig {
     static constexpr int CK = CK_, OUT = OUT_, BM = BM_, BN = BN_, WM = WM_, WN = WN_;
     static constexpr int NT = WM * WN * 64, NW = WM * WN;
     static constexpr int ES = Compute<CK>::ES;
     static constexpr int BK = P_ROW_BYTES / ES;
-    static constexpr int A_BYTES = BM * P_ROW_BYTES, B_BYTES = BN * P_ROW_BYTES;
+    static constexpr int A_BYTES = (BM / 8) * SWZ_BLOCK, B_BYTES = (BN / 8) * SWZ_BLOCK;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int LDS_BYTES = P_STAGES * STAGE_BYTES;
-    static constexpr int BLOCKS = (BM + BN) / 16;    // DMA instructions per stage
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int BLOCKS = (BM + BN) / 8;     // DMA instructions per stage
     static constexpr int DMA_PER_WAVE = BLOCKS / NW;
     static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
+    static_assert(P_ROW_BYTES == ROW_BYTES, "the pipelined kernel uses the swizzled 128-byte-row layout");
     static_assert(BLOCKS % NW == 0, "DMA split");
+    static_assert(DMA_PER_WAVE * 2 < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
 
 // issued through inline assembly so that the compiler's own wait-count bookkeeping (which would put
 // an s_waitcnt vmcnt(0) in front of the next LDS read) stays out of the way; completion is awaited
-// explicitly with waitcnt_vm() before the barrier that publishes the stage
+// explicitly before the barrier that publishes the stage
 __device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
 }
@@ -79,56 +83,47 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     batch_offsets(g, batch, ao, bo);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
 
-    // ---- DMA plan of this wavefront: P instructions per stage, each one 1 KB block (16 rows) ----
-    // lane -> (row in block, slot); the slot holds global chunk slot ^ ((row / 4) % 4)
-    const int drow = lane >> 2, dchunk = (lane & 3) ^ ((lane >> 4) & 3);
+    // ---- DMA plan of this wavefront: P instructions per stage, each one 1 KB block (8 rows) ----
+    // lane -> (row in block, slot); the slot holds global chunk slot ^ row
+    const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
     const char *gp[P];       // source address of this lane for stage 0
     unsigned lds_off[P];     // block offset inside a stage (wave-uniform)
 #pragma unroll
     for (int p = 0; p < P; p++) {
-        const int q = wave * P + p;
-        if (q < Cfg::BM / 16) {
-            int row = m0 + q * 16 + drow;
+        const int q = p * Cfg::NW + wave;
+        if (q < Cfg::BM / 8) {
+            int row = m0 + q * 8 + drow;
             row = row < g.M ? row : g.M - 1;
             gp[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
-            lds_off[p] = q * 1024;
+            lds_off[p] = q * SWZ_BLOCK;
         } else {
-            const int qb = q - Cfg::BM / 16;
-            int row = n0 + qb * 16 + drow;
+            const int qb = q - Cfg::BM / 8;
+            int row = n0 + qb * 8 + drow;
             row = row < g.N ? row : g.N - 1;
             gp[p] = B + (bo + (long)row * g.b_n) * ES + dchunk * 16;
-            lds_off[p] = Cfg::A_BYTES + qb * 1024;
+            lds_off[p] = Cfg::A_BYTES + qb * SWZ_BLOCK;
         }
     }
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
     auto issue = [&](int t) {
-        const unsigned stage = lds0 + (unsigned)(t % P_STAGES) * Cfg::STAGE_BYTES;
+        const unsigned stage = lds0 + (unsigned)(t & 1) * Cfg::STAGE_BYTES;
         const long koff = (long)t * P_ROW_BYTES;
 #pragma unroll
         for (int p = 0; p < P; p++)
             dma16_raw(gp[p] + koff, __builtin_amdgcn_readfirstlane(stage + lds_off[p]));
     };
 
-    // ---- fragment addresses: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile, which is
-    // two consecutive 16-row blocks; the chunk sits at slot chunk ^ ((row / 4) % 4) of its row ----
-    const int row16 = lr & 15, swz = (row16 >> 2) & 3;
-    const int frag_row = (lr >> 4) * 1024 + row16 * P_ROW_BYTES;
-    int a_frag[2], b_frag[2];
+    // ---- fragment addresses: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile (four
+    // consecutive 8-row blocks); the chunk sits at slot chunk ^ (row % 8) of its row ----
+    const int frag_row = (lr >> 3) * SWZ_BLOCK + (lr & 7) * P_ROW_BYTES;
+    int a_frag[P_SLICES], b_frag[P_SLICES];
 #pragma unroll
-    for (int sl = 0; sl < 2; sl++) {
-        const int slot = ((2 * sl + lh) ^ swz) << 4;
-        a_frag[sl] = (wave_m * TM) * 2048 + frag_row + slot;
-        b_frag[sl] = Cfg::A_BYTES + (wave_n * TN) * 2048 + frag_row + slot;
+    for (int sl = 0; sl < P_SLICES; sl++) {
+        const int slot = ((2 * sl + lh) ^ (lr & 7)) << 4;
+        a_frag[sl] = (wave_m * TM) * 4 * SWZ_BLOCK + frag_row + slot;
+        b_frag[sl] = Cfg::A_BYTES + (wave_n * TN) * 4 * SWZ_BLOCK + frag_row + slot;
     }
-    u32x4_t fa[2][TM], fb[2][TN];  // [k slice][tile]: ONE register set, refilled slice by slice
-    auto read_slice = [&](int t, auto slice) {
-        constexpr int SL = decltype(slice)::value;
-        const char *stage = smem + (t % P_STAGES) * Cfg::STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < TM; i++) fa[SL][i] = lds_get(stage, a_frag[SL] + i * 2048);
-#pragma unroll
-        for (int j = 0; j < TN; j++) fb[SL][j] = lds_get(stage, b_frag[SL] + j * 2048);
-    };
+    u32x4_t fa[2][TM], fb[2][TN];  // [register set][tile]: slice s lives in set s % 2
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -139,55 +134,74 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
 
     const int T = g.K * ES / P_ROW_BYTES;
-    // publish a stage: wait until at most `newer` younger stages' DMA are still in flight, then meet
-    auto publish = [&](int newer) {
-        if (newer >= 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * P));
-        else if (newer == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(P));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+
+    // One k-slice of work, in an explicitly pinned order: the MFMAs of slice CUR (register set CUR % 2),
+    // with the fragment reads of slice RD of stage t_rd (RD < 0: none) and DMA instructions
+    // [D0, D0 + DN) of stage t_dma spread evenly between them.  Neither the reads nor the DMA then
+    // arrive in bursts: a burst of DMA instructions fills the memory pipeline's issue queue and
+    // stalls the wavefront in front of its next MFMA.
+    auto slice_step = [&](auto cur_, auto rd_, auto d0_, auto dn_, int t_rd, int t_dma, bool do_dma) {
+        constexpr int SET = decltype(cur_)::value & 1, RD = decltype(rd_)::value;
+        constexpr int D0 = decltype(d0_)::value, DN = decltype(dn_)::value;
+        constexpr int MF = TM * TN, RN = RD >= 0 ? TM + TN : 0;
+        const char *stage_rd = smem + (t_rd & 1) * Cfg::STAGE_BYTES;
+        const unsigned stage_dma = lds0 + (unsigned)(t_dma & 1) * Cfg::STAGE_BYTES;
+        const long koff = (long)t_dma * P_ROW_BYTES;
+#pragma unroll
+        for (int idx = 0; idx < MF; idx++) {
+#pragma unroll
+            for (int r = 0; r < RN; r++) {
+                if (r * MF / (RN > 0 ? RN : 1) != idx) continue;
+                constexpr int RS = RD >= 0 ? RD : 0;
+                if (r < TM) fa[RS & 1][r] = lds_get(stage_rd, a_frag[RS] + r * 4 * SWZ_BLOCK);
+                else fb[RS & 1][r - TM] = lds_get(stage_rd, b_frag[RS] + (r - TM) * 4 * SWZ_BLOCK);
+            }
+            // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
+            Cmp::mma(fb[SET][idx / TM], fa[SET][idx % TM], acc[idx % TM][idx / TM]);
+#pragma unroll
+            for (int d = 0; d < DN; d++) {
+                if (d * MF / (DN > 0 ? DN : 1) != idx) continue;
+                if (do_dma) dma16_raw(gp[D0 + d] + koff, __builtin_amdgcn_readfirstlane(stage_dma + lds_off[D0 + d]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    typedef std::integral_constant<int, 2> I2;
+    typedef std::integral_constant<int, 3> I3;
+    constexpr int PH = P / 2;  // DMA instructions of a stage issued during slice 3; the rest during the next slice 0
+    typedef std::integral_constant<int, PH> DH;
+    typedef std::integral_constant<int, P - PH> DR;
+
+    issue(0);
+    if (T > 1) {
+        issue(1);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(P));
+    } else {
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[0][i] = lds_get(smem, a_frag[0] + i * 4 * SWZ_BLOCK);
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb[0][j] = lds_get(smem, b_frag[0] + j * 4 * SWZ_BLOCK);
+
+    // The loop body is branch-free apart from the DMA predicates: past the last stage the reads fetch
+    // LDS bytes nobody uses and the barrier is one too many, both harmless and cheaper than a second
+    // copy of the MFMA code.
+    for (int t = 0; t < T; t++) {
+        // slice 0: multiply it, read slice 1, issue the second half of stage t+1's DMA (stage 1 came whole)
+        slice_step(I0{}, I1{}, DH{}, DR{}, t, t + 1, t >= 1 && t + 1 < T);
+        slice_step(I1{}, I2{}, I0{}, I0{}, t, 0, false);
+        slice_step(I2{}, I3{}, I0{}, I0{}, t, 0, false);
+        // stage t+1 (the only DMA in flight) has landed and every read of stage t has returned
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-    };
-    auto multiply = [&](auto slice) {
-        constexpr int SL = decltype(slice)::value;
-        // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int i = 0; i < TM; i++) Cmp::mma(fb[SL][j], fa[SL][i], acc[i][j]);
-    };
-    // asks the scheduler to put one fragment read behind every PER-th MFMA of the block just written
-    auto interleave = [&]() {
-        constexpr int READS = TM + TN, MFMAS = TM * TN, PER = MFMAS / READS > 0 ? MFMAS / READS : 1;
-#pragma unroll
-        for (int r = 0; r < READS; r++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // DS read
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS > PER * READS ? MFMAS - PER * READS : 0, 0);
-    };
-    typedef std::integral_constant<int, 0> S0;
-    typedef std::integral_constant<int, 1> S1;
-
-    for (int t = 0; t < P_AHEAD && t < T; t++) issue(t);
-    publish((T - 1 < P_AHEAD - 1 ? T - 1 : P_AHEAD - 1));
-    read_slice(0, S0{});
-
-    // One register set of fragments, refilled half a step ahead of its use: while slice 0 of stage t
-    // multiplies, slice 1 of stage t is read; then the barrier that publishes stage t+1; while slice 1
-    // multiplies, slice 0 of stage t+1 is read.  Each read goes into registers whose last consumer
-    // has already been issued, and LDS (128 B/clk -- a step's fragment reads take about as long as
-    // its MFMAs at this tile shape) runs beside the matrix cores instead of in bursts.
-    for (int t = 0; t < T; t++) {
-        read_slice(t, S1{});
-        multiply(S0{});
-        interleave();
-        if (t + 1 < T) {
-            publish(t + 2 < T ? 1 : 0);
-            if (t + P_AHEAD < T) issue(t + P_AHEAD);
-            read_slice(t + 1, S0{});
-        }
-        multiply(S1{});
-        interleave();
+        // slice 3: multiply it, read slice 0 of stage t+1, issue the first half of stage t+2's DMA
+        slice_step(I3{}, I0{}, I0{}, DH{}, t + 1, t + 2, t + 2 < T);
     }
 
     out_t *Cb = C + batch * (long)g.M * g.N;
@@ -217,7 +231,7 @@ template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const vo
     return HODU_ROCM_OK;
 }
 
-// both operands k-dense, 16-byte aligned, K a whole number of 64-byte stages
+// both operands k-dense, 16-byte aligned, K a whole number of 128-byte stages
 template <int CK> bool pipe_eligible(int la, int lb, const DevProduct &g) {
     return la == LM_K && lb == LM_K && g.K > 0 && ((long)g.K * Compute<CK>::ES) % P_ROW_BYTES == 0;
 }

@@ -61,10 +61,10 @@ def test_pipelined_kk_variants(ctx, kind, tile, name):
     ctx.force_tile(tile)
     es = {"bf16": 2, "f16": 2, "f32": 4, "i32_i8i8": 1}[kind]
     for stages in (1, 2, 3, 4, 5, 11):
-        K = stages * 64 // es
+        K = stages * 128 // es
         check_product(ctx, "dot", kind, V([296, K]), V([200, K]).t(), seed=stages, expect_kernel=f"{prefix}_{name}_KK")
     # batched, with a row-sliced operand (leading dimension > K) and an offset
-    K = 6 * 64 // es
+    K = 6 * 128 // es
     check_product(ctx, "matmul", kind, V([3, 72, 2 * K]).slice(2, K, 2 * K), V([3, 80, K], offset=64).t(), seed=7,
                   expect_kernel=f"{prefix}_{name}_KK")
     ctx.force_tile(-1)
