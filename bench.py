@@ -129,7 +129,7 @@ def out_bytes(case):
     return md, n * {"f32": 4, "bf16": 2, "bf16_f8e4m3w": 2, "i32_i8i8": 4}[case.name]
 
 
-def time_case(ctx, case, steps, warmup):
+def time_case(ctx, case, steps, warmup, graph=False):
     """returns a result dict; operands are uploaded before the timed region starts"""
     md, obytes = out_bytes(case)
     a = ctx.upload(case.make_a())
@@ -151,7 +151,7 @@ def time_case(ctx, case, steps, warmup):
     kernel = ctx.last_kernel()
     # the K timed launches are issued back to back from C (hodu_rocm_debug_time_product) so that a
     # 3 us GEMV is not hidden behind the interpreter's per-call cost; HIP events on the same stream
-    ms = ctx.time_product(case.op, case.name, a, ws, out, md, steps)
+    ms = ctx.time_product(case.op, case.name, a, ws, out, md, steps, graph=graph)
     for buf in [a, out] + ws:
         buf.free()
     per_launch_s = ms / 1e3 / steps
@@ -225,6 +225,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
+    ap.add_argument("--graph", action="store_true", help="with --only: replay the K launches as one HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every GPU box here has one GPU and no collective or sharded "
@@ -253,7 +254,7 @@ def main():
         return
     if args.only:
         case = next(c for c in build_cases({args.only.split("_")[0]}) if c.key == args.only)
-        print(json.dumps(time_case(ctx, case, args.steps, args.warmup)))
+        print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
         ctx.close()
         return
     which = set(args.configs.split(",")) | {"c2"}

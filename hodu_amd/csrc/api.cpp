@@ -14,7 +14,9 @@ int check_ptrs(const char *op, hodu_rocm_ctx *ctx, const void *a, const void *b,
 // Picks the kernel family for one launch-sized product.
 int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                  const DevProduct &g) {
-    int rc = launch_skinny(ctx, kind, dtype, a, b, c, g);
+    int rc = ctx->force_tile == 30 ? HODU_ROCM_UNSUPPORTED : launch_gemv(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    rc = launch_skinny(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     rc = launch_mfma(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
@@ -137,7 +139,7 @@ int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, voi
     return dot_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
 }
 
-int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
                                  const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
                                  int iters, float *elapsed_ms) {
     clear_error();
@@ -155,17 +157,53 @@ int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, in
     hipEvent_t t0, t1;
     HODU_HIP(hipEventCreate(&t0));
     HODU_HIP(hipEventCreate(&t1));
+    hipGraph_t g = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (graph) {
+        // the launches are recorded once (kernel nodes only) and replayed as one graph: what a decode loop
+        // that cannot afford a host round trip per product would do
+        HODU_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+        for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
+            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p);
+        hipError_t ce = hipStreamEndCapture(ctx->stream, &g);
+        if (rc == HODU_ROCM_OK && ce != hipSuccess) rc = fail(HODU_ROCM_HIP_ERROR, "graph capture: %s", hipGetErrorString(ce));
+        if (rc == HODU_ROCM_OK && hipGraphInstantiate(&exec, g, nullptr, nullptr, 0) != hipSuccess)
+            rc = fail(HODU_ROCM_HIP_ERROR, "graph instantiate failed");
+        if (rc == HODU_ROCM_OK) {  // one untimed replay uploads the graph
+            (void)hipGraphLaunch(exec, ctx->stream);
+            (void)hipStreamSynchronize(ctx->stream);
+        }
+    }
     HODU_HIP(hipEventRecord(t0, ctx->stream));
-    for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
-        rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p);
+    if (graph) {
+        if (rc == HODU_ROCM_OK && hipGraphLaunch(exec, ctx->stream) != hipSuccess)
+            rc = fail(HODU_ROCM_HIP_ERROR, "graph launch failed");
+    } else {
+        for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
+            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p);
+    }
     hipError_t e = hipEventRecord(t1, ctx->stream);
     if (e == hipSuccess) e = hipEventSynchronize(t1);
     if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
     (void)hipEventDestroy(t0);
     (void)hipEventDestroy(t1);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (g) (void)hipGraphDestroy(g);
     if (rc) return rc;
     if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_product: %s", hipGetErrorString(e));
     return HODU_ROCM_OK;
+}
+
+int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                 const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
+                                 int iters, float *elapsed_ms) {
+    return time_product_impl(false, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms);
+}
+
+int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                       const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md,
+                                       size_t len, int iters, float *elapsed_ms) {
+    return time_product_impl(true, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms);
 }
 
 int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const size_t *md, size_t len) {

@@ -118,6 +118,7 @@ int launch_generic(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const
 int launch_mfma(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                 const DevProduct &g);
 // bandwidth-bound small-M path: returns HODU_ROCM_UNSUPPORTED when not applicable
+int launch_gemv(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g);
 int launch_skinny(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                   const DevProduct &g);
 

@@ -1,0 +1,202 @@
+// Decode-shape products with 1..4 rows on the left: y[m, n] = sum_k x[m, k] * W[n, k], W k-dense
+// (`input.matmul(weight.transpose(-2, -1))`, crates/hodu_nn/src/modules/linear.rs:38-47), bf16
+// activations against bf16 or f8e4m3 weights.  Replaces the single-thread M < 512 path of
+// hodu_cpu_dot_bf16 (kernels/ops_matrix.c:486-548) for the shape where only the weight bytes matter.
+//
+// Pure streaming: a wavefront owns R whole weight rows and reads each one as consecutive 1 KB
+// pieces (64 lanes x 16 bytes: every request is whole cache lines of one row).  All loads of a
+// wavefront -- R rows x up to 4 KB -- are issued before the first is consumed, so with a few
+// wavefronts per SIMD a compute unit keeps tens of KB in flight and the kernel is one memory
+// latency plus the transfer.  The arithmetic rides on the vector ALU: f8e4m3 pairs widen to bf16
+// pairs (v_cvt_scalef32_pk_bf16_fp8, exact) and v_dot2_f32_bf16 accumulates in f32; the 64 partial
+// sums of an output meet through DPP row operations, and the sum is rounded once to bf16.
+//
+// Measured alternatives that did not pay on 4096 x 4096 f8e4m3 weights (5.1 us as built): staging the
+// activations in LDS (+0.7 us: a barrier in front of the first multiply), renumbering workgroups so
+// that one XCD writes whole output lines (+0.1 us), four rows per wavefront (+0.3 us).  Of the 5.1 us,
+// 2.5 us is the launch cadence of an empty kernel and about 0.3 us the acknowledged output store.
+#include "common.hpp"
+#include "device_types.hpp"
+#include "gemm_mfma.hpp"
+
+namespace hodu {
+namespace {
+
+using mfma::bitcast;
+using mfma::SK_F8;
+using mfma::SK_SAME;
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int GEMV_NCH = 4;    // 1 KB pieces of a row in flight per row
+
+template <int SKB> struct WeightVec {
+    static constexpr int EPL = SKB == SK_F8 ? 16 : 8;  // elements in one 16-byte lane load
+    static constexpr int XV = EPL / 8;                  // 16-byte vectors of bf16 activations matching it
+};
+
+// acc += dot(w (EPL elements), x (EPL bf16))
+template <int SKB>
+__device__ __forceinline__ float dot16(const u32x4_t &w, const u32x4_t *x, float acc) {
+    if constexpr (SKB == SK_F8) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const bf16x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], 1.0f, false);
+            const bf16x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], 1.0f, true);
+            // 16 bytes of f8 = elements 4q..4q+3 in word q; x[0] holds bf16 0..7, x[1] holds 8..15
+            acc = __builtin_amdgcn_fdot2_f32_bf16(lo, bitcast<bf16x2_t>(x[q >> 1][(2 * q) & 3]), acc, false);
+            acc = __builtin_amdgcn_fdot2_f32_bf16(hi, bitcast<bf16x2_t>(x[q >> 1][(2 * q + 1) & 3]), acc, false);
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            acc = __builtin_amdgcn_fdot2_f32_bf16(bitcast<bf16x2_t>(w[q]), bitcast<bf16x2_t>(x[0][q]), acc, false);
+    }
+    return acc;
+}
+
+// sum over the 64 lanes of a wavefront, result in every lane: four DPP steps inside each row of 16
+// lanes (a few cycles each, no LDS round trips), then the four row sums through scalar registers
+__device__ __forceinline__ float wave_sum(float v) {
+    int x = bitcast<int>(v);
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    x = bitcast<int>(v);
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    x = bitcast<int>(v);
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true));  // row_half_mirror
+    x = bitcast<int>(v);
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, true));  // row_mirror
+    x = bitcast<int>(v);
+    return bitcast<float>(__builtin_amdgcn_readlane(x, 0)) + bitcast<float>(__builtin_amdgcn_readlane(x, 16)) +
+           bitcast<float>(__builtin_amdgcn_readlane(x, 32)) + bitcast<float>(__builtin_amdgcn_readlane(x, 48));
+}
+
+// second launch bound: wavefronts per SIMD to leave room for (caps the register budget at 128 for M <= 2)
+template <int SKB, int M, int R, int NW>
+__global__ __launch_bounds__(NW * 64, (M <= 2 ? 4 : 2)) void gemv_rowstream_kernel(const char *__restrict__ X,
+                                                                                  const char *__restrict__ W,
+                                                                                  uint16_t *__restrict__ Y, int N, int K,
+                                                                                  long x_row_bytes, long w_row_bytes) {
+    constexpr int EPL = WeightVec<SKB>::EPL, XV = WeightVec<SKB>::XV, SB = SKB == SK_F8 ? 1 : 2;
+    constexpr int STEP = GEMV_NCH * 64 * EPL;  // k covered by one pass of a wavefront
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int n0 = (blockIdx.x * NW + (tid >> 6)) * R;
+
+    float acc[M][R];
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[m][r] = 0.f;
+
+    const char *wrow[R];  // rows past N repeat the last one; their results are not stored
+#pragma unroll
+    for (int r = 0; r < R; r++) wrow[r] = W + (long)(n0 + r < N ? n0 + r : N - 1) * w_row_bytes;
+
+    auto load_weights = [&](int kc, u32x4_t (&wv)[R][GEMV_NCH]) {
+#pragma unroll
+        for (int c = 0; c < GEMV_NCH; c++) {
+            const int k = kc + (c * 64 + lane) * EPL;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                wv[r][c] = u32x4_t{0u, 0u, 0u, 0u};
+                if (k < K) wv[r][c] = *reinterpret_cast<const u32x4_t *>(wrow[r] + (long)k * SB);
+            }
+        }
+    };
+    auto multiply = [&](const u32x4_t (&wv)[R][GEMV_NCH], const u32x4_t (&xv)[M][GEMV_NCH][XV]) {
+#pragma unroll
+        for (int c = 0; c < GEMV_NCH; c++)
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int m = 0; m < M; m++) acc[m][r] = dot16<SKB>(wv[r][c], xv[m][c], acc[m][r]);
+    };
+
+    for (int kc = 0; kc < K; kc += STEP) {
+        u32x4_t wv[R][GEMV_NCH], xv[M][GEMV_NCH][XV];
+        // activations first (issue order is return order), then the weights
+#pragma unroll
+        for (int c = 0; c < GEMV_NCH; c++) {
+            const int k = kc + (c * 64 + lane) * EPL;
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int v = 0; v < XV; v++) {
+                    xv[m][c][v] = u32x4_t{0u, 0u, 0u, 0u};
+                    if (k < K) xv[m][c][v] = *reinterpret_cast<const u32x4_t *>(X + m * x_row_bytes + (long)k * 2 + v * 16);
+                }
+        }
+        load_weights(kc, wv);
+        multiply(wv, xv);
+    }
+
+    // the R results of a row of x leave in one store instruction: lane r writes column n0 + r
+#pragma unroll
+    for (int m = 0; m < M; m++) {
+        float mine = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float v = wave_sum(acc[m][r]);
+            mine = lane == r ? v : mine;
+        }
+        if (lane < R && n0 + lane < N) Y[(long)m * N + n0 + lane] = mfma::Out<mfma::OUT_BF16>::cvt(mine);
+    }
+}
+
+template <int SKB, int M, int R, int NW>
+int launch_one(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g) {
+    constexpr int ES = 2, SB = SKB == SK_F8 ? 1 : 2;
+    const char *X = (const char *)x + g.a_off * ES;
+    const char *Wp = (const char *)w + g.b_off * SB;
+    const long waves = (g.N + R - 1) / R;
+    const unsigned blocks = (unsigned)((waves + NW - 1) / NW);
+    hipLaunchKernelGGL((gemv_rowstream_kernel<SKB, M, R, NW>), dim3(blocks), dim3(NW * 64), 0, ctx->stream, X, Wp,
+                       (uint16_t *)y, g.N, g.K, g.a_m * (long)ES, g.b_n * (long)SB);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
+// shape: 0 = 4 wavefronts x 1 row each, 1 = 4 x 2, 2 = 8 x 2
+template <int SKB, int M>
+int launch_rows(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g, int shape) {
+    if (shape == 0) return launch_one<SKB, M, 1, 4>(ctx, x, w, y, g);
+    if (shape == 1) return launch_one<SKB, M, 2, 4>(ctx, x, w, y, g);
+    return launch_one<SKB, M, 2, 8>(ctx, x, w, y, g);
+}
+
+template <int SKB>
+int run_gemv(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g, const char *name) {
+    constexpr int ES = 2, SB = SKB == SK_F8 ? 1 : 2, EPL = WeightVec<SKB>::EPL;
+    // applicability: one product, both operands k-dense, every 16-byte vector load aligned and inside its row
+    auto al = [](long elems, int bytes) { return (elems * bytes) % 16 == 0; };
+    if (g.M < 1 || g.M > 4 || g.batches != 1 || g.K % EPL != 0) return HODU_ROCM_UNSUPPORTED;
+    if (g.a_k != 1 || g.b_k != 1) return HODU_ROCM_UNSUPPORTED;
+    if (!(g.M == 1 || al(g.a_m, ES)) || !(g.N == 1 || al(g.b_n, SB))) return HODU_ROCM_UNSUPPORTED;
+    if (((uintptr_t)x + (uintptr_t)g.a_off * ES) % 16 || ((uintptr_t)w + (uintptr_t)g.b_off * SB) % 16)
+        return HODU_ROCM_UNSUPPORTED;
+    // two rows per wavefront (activation registers shared by both) once that still leaves every compute
+    // unit two workgroups; measured on 4096 x 4096 f8 weights, 4 x 1, 4 x 2 and 8 x 2 are within 3 %
+    const long cus = ctx->props.multiProcessorCount;
+    int shape = g.N >= 16 * cus ? 1 : 0;
+    if (ctx->force_tile == 31) shape = 0;
+    if (ctx->force_tile == 32) shape = 1;
+    if (ctx->force_tile == 34) shape = 2;
+    ctx->last_kernel = name;
+    switch (g.M) {
+    case 1: return launch_rows<SKB, 1>(ctx, x, w, y, g, shape);
+    case 2: return launch_rows<SKB, 2>(ctx, x, w, y, g, shape);
+    case 3: return launch_rows<SKB, 3>(ctx, x, w, y, g, shape);
+    default: return launch_rows<SKB, 4>(ctx, x, w, y, g, shape);
+    }
+}
+
+}  // namespace
+
+int launch_gemv(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
+    if (g.M > 4 || g.K == 0) return HODU_ROCM_UNSUPPORTED;
+    if (kind == PK_BF16_F8W) return run_gemv<SK_F8>(ctx, a, b, c, g, "gemv_bf16_f8w");
+    if (kind == PK_SAME && dtype == HODU_BF16) return run_gemv<SK_SAME>(ctx, a, b, c, g, "gemv_bf16");
+    return HODU_ROCM_UNSUPPORTED;
+}
+
+}  // namespace hodu

@@ -66,6 +66,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
     lib.hodu_rocm_debug_time_product.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz, ci,
                                                  ctypes.POINTER(ctypes.c_float)]
+    lib.hodu_rocm_debug_time_product_graph.argtypes = lib.hodu_rocm_debug_time_product.argtypes
     lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
                                           ctypes.POINTER(sz)]
     lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
@@ -231,17 +232,19 @@ class Context:
         arr, n = _md_array(md)
         self._check(self.lib.hodu_rocm_contiguous(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
 
-    def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int) -> float:
-        """back-to-back launches issued from C, HIP-event timed on the context's stream; total ms"""
+    def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int,
+                     graph: bool = False) -> float:
+        """back-to-back launches issued from C (graph=True: recorded once into a HIP graph and replayed as
+        one graph launch), HIP-event timed on the context's stream; total ms"""
         self._check_extents(op, name, lhs, rhs_list, out, md)
         kind = {"bf16_f8e4m3w": 1, "i32_i8i8": 2}.get(name, 0)
         dtype = DTYPE_ID["bf16"] if kind == 1 else DTYPE_ID["i32"] if kind == 2 else DTYPE_ID[name]
         arr, n = _md_array(md)
         ptrs = (ctypes.c_void_p * len(rhs_list))(*[b.ptr for b in rhs_list])
         ms = ctypes.c_float()
-        self._check(self.lib.hodu_rocm_debug_time_product(self.handle, 1 if op == "matmul" else 0, kind, dtype,
-                                                          lhs.ptr, ptrs, len(rhs_list), out.ptr, arr, n, int(iters),
-                                                          ctypes.byref(ms)))
+        fn = self.lib.hodu_rocm_debug_time_product_graph if graph else self.lib.hodu_rocm_debug_time_product
+        self._check(fn(self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr,
+                       n, int(iters), ctypes.byref(ms)))
         return float(ms.value)
 
     def force_tile(self, tile: int):

@@ -81,7 +81,8 @@ int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
 /* name of the kernel family the last matmul/dot call on this context dispatched to (diagnostics) */
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
 /* testing hook: pin the MFMA tile variant (0 = 256x256 with 8 wavefronts, 1 = 256x256 with 4,
- * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; -1 = automatic) so that
+ * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
+ * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; -1 = automatic) so that
  * every compiled variant can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
 /* measurement hook: issues the same product `iters` times back to back from C (no per-launch
@@ -91,6 +92,12 @@ int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
 int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
                                  const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
                                  size_t metadata_len, int iters, float *elapsed_ms);
+/* the same, with the `iters` launches captured once into a HIP graph (kernel nodes only) and replayed as
+ * one graph launch inside the timed region: the per-launch time a caller sees who replays a recorded
+ * decode step instead of paying a host round trip per product */
+int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                       const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
+                                       size_t metadata_len, int iters, float *elapsed_ms);
 
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>

@@ -11,6 +11,9 @@ KINDS = {"bf16_f8e4m3w": "skinny_bf16_f8w", "bf16": "skinny_bf16", "f16": "skinn
          "i32_i8i8": "skinny_i32_i8i8"}
 
 
+GEMV_KINDS = {"bf16_f8e4m3w": "gemv_bf16_f8w", "bf16": "gemv_bf16"}
+
+
 @pytest.fixture(scope="module")
 def ctx():
     c = ffi.Context(0)
@@ -18,9 +21,18 @@ def ctx():
     c.close()
 
 
+@pytest.fixture()
+def no_gemv(ctx):
+    """route M <= 4 products past the row-streaming GEMV kernel so that the MFMA skinny kernel is exercised"""
+    ctx.force_tile(30)
+    yield ctx
+    ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("kind", list(KINDS))
 @pytest.mark.parametrize("m", [1, 3, 16])
-def test_linear_idiom_weight_k_dense(ctx, kind, m):
+def test_linear_idiom_weight_k_dense(no_gemv, kind, m):
+    ctx = no_gemv
     rs = 2.0 if "f8" in kind else None
     # ragged N (not a multiple of 16), K leaves an uneven split over the 8 wavefronts
     check_product(ctx, "dot", kind, V([m, 1040]), V([203, 1040]).t(), seed=m, rscale=rs, expect_kernel=KINDS[kind])
@@ -29,7 +41,8 @@ def test_linear_idiom_weight_k_dense(ctx, kind, m):
 
 
 @pytest.mark.parametrize("kind", list(KINDS))
-def test_batched_rows_fold_or_stay_batched(ctx, kind):
+def test_batched_rows_fold_or_stay_batched(no_gemv, kind):
+    ctx = no_gemv
     rs = 2.0 if "f8" in kind else None
     # [4, 1, K] x shared weight: the batch folds into 4 rows
     check_product(ctx, "matmul", kind, V([4, 1, 256]), V([40, 256]).t().broadcast_to([4, 256, 40]), seed=1, rscale=rs,
@@ -46,3 +59,38 @@ def test_not_applicable_layouts_fall_through(ctx):
     check_product(ctx, "dot", "bf16_f8e4m3w", V([1, 256]), V([256, 64]), seed=4, rscale=2.0, expect_kernel="mfma_")
     # misaligned activation rows
     check_product(ctx, "dot", "bf16", V([2, 100], offset=1), V([32, 100]).t(), seed=5, expect_kernel="mfma_")
+
+
+# ---- row-streaming GEMV kernel (M <= 4, bf16 activations, bf16 or f8e4m3 weights) ---------------------
+@pytest.mark.parametrize("kind", list(GEMV_KINDS))
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("rows", [-1, 31, 32, 34])
+def test_gemv_rowstream(ctx, kind, m, rows):
+    rs = 2.0 if "f8" in kind else None
+    name = GEMV_KINDS[kind]
+    ctx.force_tile(rows)
+    try:
+        # ragged N (not a multiple of the rows per wavefront or per workgroup), ragged last 1 KB piece
+        check_product(ctx, "dot", kind, V([m, 1040]), V([203, 1040]).t(), seed=m, rscale=rs, expect_kernel=name)
+        # K shorter than one piece; tiny N
+        check_product(ctx, "dot", kind, V([m, 64]), V([5, 64]).t(), seed=10 + m, rscale=rs, expect_kernel=name)
+        # K longer than what a wavefront keeps in flight (several passes, ragged tail)
+        check_product(ctx, "dot", kind, V([m, 4112]), V([37, 4112]).t(), seed=20 + m, rscale=rs, expect_kernel=name)
+        # row-sliced weight and activations (leading dimension > K) at aligned offsets
+        check_product(ctx, "dot", kind, V([m, 512]).slice(1, 128, 384), V([24, 512], offset=64).slice(1, 64, 320).t(),
+                      seed=30 + m, rscale=rs, expect_kernel=name)
+    finally:
+        ctx.force_tile(-1)
+
+
+@pytest.mark.parametrize("kind", list(GEMV_KINDS))
+def test_gemv_batch_folding_and_fallbacks(ctx, kind):
+    rs = 2.0 if "f8" in kind else None
+    # [4, 1, K] x shared weight: the batch folds into 4 rows of one GEMV
+    check_product(ctx, "matmul", kind, V([4, 1, 256]), V([40, 256]).t().broadcast_to([4, 256, 40]), seed=1, rscale=rs,
+                  expect_kernel=GEMV_KINDS[kind])
+    # per-batch weights: not one product; the MFMA skinny kernel takes it
+    check_product(ctx, "matmul", kind, V([3, 2, 256]), V([3, 40, 256]).t(), seed=2, rscale=rs, expect_kernel=KINDS[kind])
+    # K not a multiple of the 16-byte vector: falls through
+    k = 72 if "f8" in kind else 68
+    check_product(ctx, "dot", kind, V([1, k]), V([16, k]).t(), seed=3, rscale=rs, expect_kernel="")
