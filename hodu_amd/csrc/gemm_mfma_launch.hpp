@@ -9,9 +9,10 @@ namespace mfma {
 
 // One compute kind: {KK, KM, MK, MM} x {256x256 with 4 wavefronts, 128x128, 64x64}, {KK, KM} x 256x256
 // with 8 wavefronts, a scalar-load 64x64 kernel, and -- when both operands are stored in the compute
-// type -- the four software-pipelined KK kernels of gemm_mfma_pipe.hpp.  The tile is the largest that
-// still yields at least one workgroup per compute unit.
-constexpr int kVariants = 21;
+// type -- the software-pipelined kernels of gemm_mfma_pipe.hpp: KK at four tile shapes and, for the
+// 16-bit types, KM / MK / MM at the three larger ones.  The tile is the largest that still yields at
+// least one workgroup per compute unit.
+constexpr int kVariants = 30;
 template <int CK, int SKA, int SKB, int OUT>
 int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
                 const char *const names[kVariants]) {
@@ -32,12 +33,25 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     const int combo = (la == LM_MN ? 2 : 0) + (lb == LM_MN ? 1 : 0);
     if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
         // testing hook values 10..13 pin the pipelined kernel's tile, 0..3 the general kernel's
-        if (pipe_eligible<CK>(la, lb, g) && (forced < 0 || forced >= 10)) {
-            ctx->last_kernel = names[17 + size];
-            if (size == 0) return launch_pipe<PipeConfig<CK, OUT, 256, 256, 2, 4>>(ctx, a, b, c, g);
-            if (size == 1) return launch_pipe<PipeConfig<CK, OUT, 256, 256, 2, 2>>(ctx, a, b, c, g);
-            if (size == 2) return launch_pipe<PipeConfig<CK, OUT, 128, 128, 2, 2>>(ctx, a, b, c, g);
-            return launch_pipe<PipeConfig<CK, OUT, 64, 64, 2, 2>>(ctx, a, b, c, g);
+        if (pipe_eligible<CK>(la, lb, g) && (forced < 0 || forced >= 10) && (combo == 0 || size < 3)) {
+            ctx->last_kernel = combo == 0 ? names[17 + size] : names[21 + (combo - 1) * 3 + size];
+#define HODU_PIPE_CASE(SZ, BM, BN, WM, WN, LA, LB) \
+    if (size == SZ) return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LA, LB>>(ctx, a, b, c, g);
+#define HODU_PIPE_COMBO(CB, LA, LB)                       \
+    if (combo == CB) {                                    \
+        HODU_PIPE_CASE(0, 256, 256, 2, 4, LA, LB)         \
+        HODU_PIPE_CASE(1, 256, 256, 2, 2, LA, LB)         \
+        HODU_PIPE_CASE(2, 128, 128, 2, 2, LA, LB)         \
+    }
+            HODU_PIPE_COMBO(0, LM_K, LM_K)
+            if constexpr (ES == 2) {
+                HODU_PIPE_COMBO(1, LM_K, LM_MN)
+                HODU_PIPE_COMBO(2, LM_MN, LM_K)
+                HODU_PIPE_COMBO(3, LM_MN, LM_MN)
+            }
+            if (combo == 0) return launch_pipe<PipeConfig<CK, OUT, 64, 64, 2, 2>>(ctx, a, b, c, g);
+#undef HODU_PIPE_COMBO
+#undef HODU_PIPE_CASE
         }
     }
     // a row-dense LEFT operand needs 32 staging registers more than the 8-wavefront variant has
@@ -65,7 +79,10 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     {P "_256x256w8_KK", P "_256x256w8_KM", P "_256x256w8_MK", P "_256x256w8_MM", P "_256x256_KK", P "_256x256_KM", \
      P "_256x256_MK",   P "_256x256_MM",   P "_128x128_KK",   P "_128x128_KM",   P "_128x128_MK", P "_128x128_MM", \
      P "_64x64_KK",     P "_64x64_KM",     P "_64x64_MK",     P "_64x64_MM",     P "_64x64_scalar",                \
-     P "_pipe256x256w8_KK", P "_pipe256x256_KK", P "_pipe128x128_KK", P "_pipe64x64_KK"}
+     P "_pipe256x256w8_KK", P "_pipe256x256_KK", P "_pipe128x128_KK", P "_pipe64x64_KK",                           \
+     P "_pipe256x256w8_KM", P "_pipe256x256_KM", P "_pipe128x128_KM",                                              \
+     P "_pipe256x256w8_MK", P "_pipe256x256_MK", P "_pipe128x128_MK",                                              \
+     P "_pipe256x256w8_MM", P "_pipe256x256_MM", P "_pipe128x128_MM"}
 
 }  // namespace mfma
 }  // namespace hodu

@@ -19,6 +19,15 @@
 //   * one bare s_barrier per stage, preceded by s_waitcnt vmcnt(0) lgkmcnt(0): at that point the only
 //     DMA in flight is the next stage's, and every fragment read of the current stage has returned.
 //
+// Row-dense operands (stride 1 along m or n: a [K, N] row-major right operand, a transposed left
+// operand) of the 16-bit types take the same path.  A stage of such an operand is 64 k-rows of the
+// tile's ROWS contiguous elements, DMA'd as whole rows (1 KB = 1024 / (2 * ROWS) k-rows per
+// instruction) into a plain [k][ROWS] array whose 16-byte chunks are XOR-swizzled by (k % 4) << 2.
+// The MFMA fragment -- 8 consecutive k of ONE row per lane -- comes out of that k-major array
+// through two ds_read_b64_tr_b16 (LDS transpose reads: each hands a lane 4 consecutive k of its own
+// column from four rows that 16 lanes read together), so no register-level transpose and no second
+// LDS layout is needed.
+//
 // Hazards.  The barrier in stage t is reached by a wavefront only after all its reads of stage t
 // have RETURNED (lgkmcnt(0)) and its own share of stage t+1 has landed (vmcnt(0)); past it, stage t's
 // buffer is dead for everybody and stage t+1 is complete for everybody.
@@ -38,19 +47,23 @@ constexpr int P_SLICES = 4;        // 32-byte k-slices per stage
 constexpr int waitcnt_vm(int n) { return (n & 15) | 0x70 | 0xF00 | ((n >> 4) << 14); }
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | 0x70 | ((n >> 4) << 14); }
 
-template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_> struct PipeConfig {
-    static constexpr int CK = CK_, OUT = OUT_, BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_, int LA_ = LM_K, int LB_ = LM_K> struct PipeConfig {
+    static constexpr int CK = CK_, OUT = OUT_, BM = BM_, BN = BN_, WM = WM_, WN = WN_, LA = LA_, LB = LB_;
     static constexpr int NT = WM * WN * 64, NW = WM * WN;
     static constexpr int ES = Compute<CK>::ES;
     static constexpr int BK = P_ROW_BYTES / ES;
-    static constexpr int A_BYTES = (BM / 8) * SWZ_BLOCK, B_BYTES = (BN / 8) * SWZ_BLOCK;
+    // k-dense: 8-row blocks of 1 KB, 128 bytes apart; row-dense: [64 k][ROWS] with no gaps
+    static constexpr int A_BYTES = (BM / 8) * (LA == LM_K ? SWZ_BLOCK : 1024);
+    static constexpr int B_BYTES = (BN / 8) * (LB == LM_K ? SWZ_BLOCK : 1024);
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
     static constexpr int BLOCKS = (BM + BN) / 8;     // DMA instructions per stage
     static constexpr int DMA_PER_WAVE = BLOCKS / NW;
     static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
     static_assert(P_ROW_BYTES == ROW_BYTES, "the pipelined kernel uses the swizzled 128-byte-row layout");
-    static_assert(BLOCKS % NW == 0, "DMA split");
+    static_assert(BLOCKS % NW == 0 && (BM / 8) % NW == 0, "DMA split");
+    static_assert((LA == LM_K || (ES == 2 && BM >= 128)) && (LB == LM_K || (ES == 2 && BN >= 128)),
+                  "row-dense operands: 16-bit types, tiles of at least 128 rows");
     static_assert(DMA_PER_WAVE * 2 < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
@@ -60,6 +73,15 @@ template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_> struct PipeConf
 // explicitly before the barrier that publishes the stage
 __device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
+}
+
+// 4 x 16-bit per lane with the LDS transpose: of the 16 lanes that execute together, lane s supplies the
+// address of 4 consecutive elements; lane i receives element (i % 4) of lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2_t lds_get_tr16(const char *lds, int off) {
+    typedef s16x4_t __attribute__((address_space(3))) * lds_ptr_t;
+    const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)(lds + off));
+    return bitcast<u32x2_t>(v);
 }
 
 template <class Cfg>
@@ -83,46 +105,108 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     batch_offsets(g, batch, ao, bo);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
 
-    // ---- DMA plan of this wavefront: P instructions per stage, each one 1 KB block (8 rows) ----
-    // lane -> (row in block, slot); the slot holds global chunk slot ^ row
-    const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+    // ---- DMA plan of this wavefront: P instructions per stage, each one 1 KB of LDS ----
+    // k-dense operand: a block of 8 rows x 128 B; lane -> (row in block, slot), the slot holds chunk slot ^ row.
+    // row-dense operand: KPI consecutive k-rows of ROWS elements; lane -> (k-row, slot), slot holds chunk
+    // slot ^ ((k % 4) << 2); a chunk that starts past the operand's last row is fetched from the last
+    // whole chunk instead (its columns are never stored).
+    constexpr int PA = (Cfg::BM / 8) / Cfg::NW;  // the first PA instructions of a wavefront belong to A
     const char *gp[P];       // source address of this lane for stage 0
     unsigned lds_off[P];     // block offset inside a stage (wave-uniform)
 #pragma unroll
     for (int p = 0; p < P; p++) {
-        const int q = p * Cfg::NW + wave;
-        if (q < Cfg::BM / 8) {
-            int row = m0 + q * 8 + drow;
-            row = row < g.M ? row : g.M - 1;
-            gp[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
-            lds_off[p] = q * SWZ_BLOCK;
+        if (p < PA) {
+            const int q = p * Cfg::NW + wave;
+            if constexpr (Cfg::LA == LM_K) {
+                const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+                int row = m0 + q * 8 + drow;
+                row = row < g.M ? row : g.M - 1;
+                gp[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
+                lds_off[p] = q * SWZ_BLOCK;
+            } else {
+                constexpr int CPR = Cfg::BM / 8, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
+                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ ((k & 3) << 2);
+                int col = m0 + c * 8;
+                col = col <= g.M - 8 ? col : g.M - 8;
+                gp[p] = A + (ao + (long)k * g.a_k + col) * ES;
+                lds_off[p] = q * 1024;
+            }
         } else {
-            const int qb = q - Cfg::BM / 8;
-            int row = n0 + qb * 8 + drow;
-            row = row < g.N ? row : g.N - 1;
-            gp[p] = B + (bo + (long)row * g.b_n) * ES + dchunk * 16;
-            lds_off[p] = Cfg::A_BYTES + qb * SWZ_BLOCK;
+            const int q = (p - PA) * Cfg::NW + wave;
+            if constexpr (Cfg::LB == LM_K) {
+                const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+                int row = n0 + q * 8 + drow;
+                row = row < g.N ? row : g.N - 1;
+                gp[p] = B + (bo + (long)row * g.b_n) * ES + dchunk * 16;
+                lds_off[p] = Cfg::A_BYTES + q * SWZ_BLOCK;
+            } else {
+                constexpr int CPR = Cfg::BN / 8, KPI = 64 / CPR;
+                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ ((k & 3) << 2);
+                int col = n0 + c * 8;
+                col = col <= g.N - 8 ? col : g.N - 8;
+                gp[p] = B + (bo + (long)k * g.b_k + col) * ES;
+                lds_off[p] = Cfg::A_BYTES + q * 1024;
+            }
         }
     }
+    // bytes a stage advances each operand's source by: 128 bytes of k, or 64 k-rows
+    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : 64 * g.a_k * ES;
+    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : 64 * g.b_k * ES;
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
     auto issue = [&](int t) {
         const unsigned stage = lds0 + (unsigned)(t & 1) * Cfg::STAGE_BYTES;
-        const long koff = (long)t * P_ROW_BYTES;
 #pragma unroll
         for (int p = 0; p < P; p++)
-            dma16_raw(gp[p] + koff, __builtin_amdgcn_readfirstlane(stage + lds_off[p]));
+            dma16_raw(gp[p] + t * (p < PA ? a_adv : b_adv), __builtin_amdgcn_readfirstlane(stage + lds_off[p]));
     };
 
-    // ---- fragment addresses: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile (four
-    // consecutive 8-row blocks); the chunk sits at slot chunk ^ (row % 8) of its row ----
+    // ---- fragment addresses ----
+    // k-dense: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile (four consecutive 8-row
+    // blocks); the chunk sits at slot chunk ^ (row % 8) of its row.
+    // row-dense: lane (lr, lh) needs k = 16*s + 8*lh + 0..7 of row lr.  With s16 = lane % 16 it supplies,
+    // for each half e of those 8 k, the address of columns 4*(s16 % 4)..+3 (of its 16-column half of
+    // the tile) in k-row 16*s + 8*lh + 4*e + s16/4.  (k % 4) == s16/4 whatever s and e are, so the
+    // swizzle is a per-lane constant and the slice/half offsets are immediates.
     const int frag_row = (lr >> 3) * SWZ_BLOCK + (lr & 7) * P_ROW_BYTES;
-    int a_frag[P_SLICES], b_frag[P_SLICES];
+    const int s16 = lane & 15, kq = s16 >> 2;
+    int a_frag[P_SLICES], b_frag[P_SLICES];  // k-dense: one address per slice, tiles are immediates
+    int a_mn[TM], b_mn[TN];                  // row-dense: one address per tile, slices are immediates
 #pragma unroll
     for (int sl = 0; sl < P_SLICES; sl++) {
         const int slot = ((2 * sl + lh) ^ (lr & 7)) << 4;
         a_frag[sl] = (wave_m * TM) * 4 * SWZ_BLOCK + frag_row + slot;
         b_frag[sl] = Cfg::A_BYTES + (wave_n * TN) * 4 * SWZ_BLOCK + frag_row + slot;
     }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int c = (wave_m * TM + i) * 4 + ((lane >> 4) & 1) * 2 + ((s16 & 3) >> 1);
+        a_mn[i] = (lh * 8 + kq) * Cfg::BM * ES + ((c ^ (kq << 2)) << 4) + (s16 & 1) * 8;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int c = (wave_n * TN + j) * 4 + ((lane >> 4) & 1) * 2 + ((s16 & 3) >> 1);
+        b_mn[j] = Cfg::A_BYTES + (lh * 8 + kq) * Cfg::BN * ES + ((c ^ (kq << 2)) << 4) + (s16 & 1) * 8;
+    }
+    auto read_a = [&](const char *stage, auto sl_, int i) -> u32x4_t {
+        constexpr int SL = decltype(sl_)::value;
+        if constexpr (Cfg::LA == LM_K) {
+            return lds_get(stage, a_frag[SL] + i * 4 * SWZ_BLOCK);
+        } else {
+            const u32x2_t lo = lds_get_tr16(stage, a_mn[i] + (SL * 16) * Cfg::BM * ES);
+            const u32x2_t hi = lds_get_tr16(stage, a_mn[i] + (SL * 16 + 4) * Cfg::BM * ES);
+            return u32x4_t{lo.x, lo.y, hi.x, hi.y};
+        }
+    };
+    auto read_b = [&](const char *stage, auto sl_, int j) -> u32x4_t {
+        constexpr int SL = decltype(sl_)::value;
+        if constexpr (Cfg::LB == LM_K) {
+            return lds_get(stage, b_frag[SL] + j * 4 * SWZ_BLOCK);
+        } else {
+            const u32x2_t lo = lds_get_tr16(stage, b_mn[j] + (SL * 16) * Cfg::BN * ES);
+            const u32x2_t hi = lds_get_tr16(stage, b_mn[j] + (SL * 16 + 4) * Cfg::BN * ES);
+            return u32x4_t{lo.x, lo.y, hi.x, hi.y};
+        }
+    };
     u32x4_t fa[2][TM], fb[2][TN];  // [register set][tile]: slice s lives in set s % 2
 
     acc_t acc[TM][TN];
@@ -146,22 +230,23 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         constexpr int MF = TM * TN, RN = RD >= 0 ? TM + TN : 0;
         const char *stage_rd = smem + (t_rd & 1) * Cfg::STAGE_BYTES;
         const unsigned stage_dma = lds0 + (unsigned)(t_dma & 1) * Cfg::STAGE_BYTES;
-        const long koff = (long)t_dma * P_ROW_BYTES;
 #pragma unroll
         for (int idx = 0; idx < MF; idx++) {
 #pragma unroll
             for (int r = 0; r < RN; r++) {
                 if (r * MF / (RN > 0 ? RN : 1) != idx) continue;
-                constexpr int RS = RD >= 0 ? RD : 0;
-                if (r < TM) fa[RS & 1][r] = lds_get(stage_rd, a_frag[RS] + r * 4 * SWZ_BLOCK);
-                else fb[RS & 1][r - TM] = lds_get(stage_rd, b_frag[RS] + (r - TM) * 4 * SWZ_BLOCK);
+                typedef std::integral_constant<int, (RD >= 0 ? RD : 0)> RS;
+                if (r < TM) fa[RS::value & 1][r] = read_a(stage_rd, RS{}, r);
+                else fb[RS::value & 1][r - TM] = read_b(stage_rd, RS{}, r - TM);
             }
             // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
             Cmp::mma(fb[SET][idx / TM], fa[SET][idx % TM], acc[idx % TM][idx / TM]);
 #pragma unroll
             for (int d = 0; d < DN; d++) {
                 if (d * MF / (DN > 0 ? DN : 1) != idx) continue;
-                if (do_dma) dma16_raw(gp[D0 + d] + koff, __builtin_amdgcn_readfirstlane(stage_dma + lds_off[D0 + d]));
+                if (do_dma)
+                    dma16_raw(gp[D0 + d] + t_dma * (D0 + d < PA ? a_adv : b_adv),
+                              __builtin_amdgcn_readfirstlane(stage_dma + lds_off[D0 + d]));
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -184,9 +269,9 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[0][i] = lds_get(smem, a_frag[0] + i * 4 * SWZ_BLOCK);
+    for (int i = 0; i < TM; i++) fa[0][i] = read_a(smem, I0{}, i);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[0][j] = lds_get(smem, b_frag[0] + j * 4 * SWZ_BLOCK);
+    for (int j = 0; j < TN; j++) fb[0][j] = read_b(smem, I0{}, j);
 
     // The loop body is branch-free apart from the DMA predicates: past the last stage the reads fetch
     // LDS bytes nobody uses and the barrier is one too many, both harmless and cheaper than a second
@@ -231,9 +316,14 @@ template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const vo
     return HODU_ROCM_OK;
 }
 
-// both operands k-dense, 16-byte aligned, K a whole number of 128-byte stages
+// K a whole number of 128-byte stages (64 k for the row-dense layouts, which exist for 16-bit types
+// and need at least one whole 8-column chunk); alignment is what pick_mode already established
 template <int CK> bool pipe_eligible(int la, int lb, const DevProduct &g) {
-    return la == LM_K && lb == LM_K && g.K > 0 && ((long)g.K * Compute<CK>::ES) % P_ROW_BYTES == 0;
+    constexpr int ES = Compute<CK>::ES;
+    if (g.K <= 0 || ((long)g.K * ES) % P_ROW_BYTES != 0) return false;
+    if (la == LM_K && lb == LM_K) return true;
+    if (ES != 2 || la == LM_SCALAR || lb == LM_SCALAR) return false;
+    return (la == LM_K || g.M >= 8) && (lb == LM_K || g.N >= 8);
 }
 
 }  // namespace mfma

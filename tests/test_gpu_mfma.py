@@ -70,6 +70,33 @@ def test_pipelined_kk_variants(ctx, kind, tile, name):
     ctx.force_tile(-1)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("tile,name", [(10, "pipe256x256w8"), (11, "pipe256x256"), (12, "pipe128x128")])
+@pytest.mark.parametrize("combo", ["KM", "MK", "MM"])
+def test_pipelined_row_dense_variants(ctx, kind, tile, name, combo):
+    """the pipelined kernel with row-dense operands (LDS transpose reads): 1 to 5 stages of 64 k; M and N ragged
+    against every tile but multiples of 8, as the 16-byte row chunks require"""
+    prefix = KINDS[kind][0]
+    ctx.force_tile(tile)
+    try:
+        for stages in (1, 2, 3, 5):
+            K = stages * 64
+            lv, rv = views(combo, 296, K, 200)
+            check_product(ctx, "dot", kind, lv, rv, seed=stages, expect_kernel=f"{prefix}_{name}_{combo}")
+        # fewer rows than one tile, and a tile edge that cuts through a 16-column group
+        lv, rv = views(combo, 24, 128, 40)
+        check_product(ctx, "dot", kind, lv, rv, seed=9, expect_kernel=f"{prefix}_{name}_{combo}")
+        # batched with a shared row-dense weight (stride-0 batch) and offsets into larger buffers
+        if combo == "KM":
+            check_product(ctx, "matmul", kind, V([3, 72, 128], offset=64), V([128, 80], offset=128).broadcast_to([3, 128, 80]),
+                          seed=10, expect_kernel=f"{prefix}_{name}_{combo}")
+            # column-sliced weight: leading dimension larger than N
+            check_product(ctx, "dot", kind, V([72, 128]), V([128, 160]).slice(1, 16, 120), seed=11,
+                          expect_kernel=f"{prefix}_{name}_{combo}")
+    finally:
+        ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("kind", list(KINDS))
 def test_scalar_load_variant(ctx, kind):
     prefix, _, _ = KINDS[kind]
