@@ -44,7 +44,7 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
         HODU_PIPE_CASE(2, 128, 128, 2, 2, LA, LB)         \
     }
             HODU_PIPE_COMBO(0, LM_K, LM_K)
-            if constexpr (ES == 2) {
+            if constexpr (ES <= 2) {
                 HODU_PIPE_COMBO(1, LM_K, LM_MN)
                 HODU_PIPE_COMBO(2, LM_MN, LM_K)
                 HODU_PIPE_COMBO(3, LM_MN, LM_MN)

@@ -62,8 +62,8 @@ template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_, int LA_ = LM_K,
     static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
     static_assert(P_ROW_BYTES == ROW_BYTES, "the pipelined kernel uses the swizzled 128-byte-row layout");
     static_assert(BLOCKS % NW == 0 && (BM / 8) % NW == 0, "DMA split");
-    static_assert((LA == LM_K || (ES == 2 && BM >= 128)) && (LB == LM_K || (ES == 2 && BN >= 128)),
-                  "row-dense operands: 16-bit types, tiles of at least 128 rows");
+    static_assert((LA == LM_K || (ES <= 2 && BM >= 128)) && (LB == LM_K || (ES <= 2 && BN >= 128)),
+                  "row-dense operands: 8- and 16-bit types, tiles of at least 128 rows");
     static_assert(DMA_PER_WAVE * 2 < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
@@ -75,14 +75,35 @@ __device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
 }
 
-// 4 x 16-bit per lane with the LDS transpose: of the 16 lanes that execute together, lane s supplies the
-// address of 4 consecutive elements; lane i receives element (i % 4) of lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ u32x2_t lds_get_tr16(const char *lds, int off) {
-    typedef s16x4_t __attribute__((address_space(3))) * lds_ptr_t;
-    const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)(lds + off));
-    return bitcast<u32x2_t>(v);
+// 64 bits per lane through the LDS transpose.  Of the 16 lanes that execute together, lane s supplies the
+// address of 8 consecutive bytes.
+//   16-bit elements: lane i receives element (i % 4) of lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4 -- with lanes
+//     4e..4e+3 pointing at 16 consecutive columns of k-row e, lane i gets column i of k-rows 0..3;
+//   8-bit elements: lane i receives element (i % 8) of lanes i/8, 2 + i/8, .., 14 + i/8 -- with lanes 2e, 2e+1
+//     pointing at 16 consecutive columns of k-row e, lane i gets column i of k-rows 0..7.
+template <int ES> __device__ __forceinline__ u32x2_t lds_get_tr(const char *lds, int off) {
+    if constexpr (ES == 2) {
+        typedef short s16x4_t __attribute__((ext_vector_type(4)));
+        typedef s16x4_t __attribute__((address_space(3))) * lds_ptr_t;
+        return bitcast<u32x2_t>(__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)(lds + off)));
+    } else {
+        typedef int i32x2_t __attribute__((ext_vector_type(2)));
+        typedef i32x2_t __attribute__((address_space(3))) * lds_ptr_t;
+        return bitcast<u32x2_t>(__builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr_t)(uintptr_t)(lds + off)));
+    }
 }
+
+// Row-dense operand geometry for element size ES (1 or 2 bytes); a "chunk" is 16 bytes of one k-row.
+//   swizzle   chunk c of k-row k sits at slot c ^ swz(k); one transpose read takes its 16 lanes through
+//             RPT consecutive k-rows, 32 (ES = 2) or 16 (ES = 1) bytes of each, and the swizzle puts those rows
+//             into different banks
+template <int ES> struct RowDenseGeom {
+    static constexpr int RPT = ES == 2 ? 4 : 8;          // k-rows one transpose read covers
+    static constexpr int EPC = 16 / ES;                   // elements per chunk
+    static constexpr int STAGE_K = 128 / ES;              // k-rows per stage
+    static constexpr int SLICE_K = 32 / ES;               // k per MFMA slice
+    static __device__ __forceinline__ int swz(int k) { return ES == 2 ? (k & 3) << 2 : (k & 7); }
+};
 
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restrict__ A, const char *__restrict__ B,
@@ -124,10 +145,11 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
                 gp[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
                 lds_off[p] = q * SWZ_BLOCK;
             } else {
-                constexpr int CPR = Cfg::BM / 8, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
-                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ ((k & 3) << 2);
-                int col = m0 + c * 8;
-                col = col <= g.M - 8 ? col : g.M - 8;
+                typedef RowDenseGeom<ES> RD;
+                constexpr int CPR = Cfg::BM / RD::EPC, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
+                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ RD::swz(k);
+                int col = m0 + c * RD::EPC;
+                col = col <= g.M - RD::EPC ? col : g.M - RD::EPC;
                 gp[p] = A + (ao + (long)k * g.a_k + col) * ES;
                 lds_off[p] = q * 1024;
             }
@@ -140,18 +162,19 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
                 gp[p] = B + (bo + (long)row * g.b_n) * ES + dchunk * 16;
                 lds_off[p] = Cfg::A_BYTES + q * SWZ_BLOCK;
             } else {
-                constexpr int CPR = Cfg::BN / 8, KPI = 64 / CPR;
-                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ ((k & 3) << 2);
-                int col = n0 + c * 8;
-                col = col <= g.N - 8 ? col : g.N - 8;
+                typedef RowDenseGeom<ES> RD;
+                constexpr int CPR = Cfg::BN / RD::EPC, KPI = 64 / CPR;
+                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ RD::swz(k);
+                int col = n0 + c * RD::EPC;
+                col = col <= g.N - RD::EPC ? col : g.N - RD::EPC;
                 gp[p] = B + (bo + (long)k * g.b_k + col) * ES;
                 lds_off[p] = Cfg::A_BYTES + q * 1024;
             }
         }
     }
     // bytes a stage advances each operand's source by: 128 bytes of k, or 64 k-rows
-    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : 64 * g.a_k * ES;
-    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : 64 * g.b_k * ES;
+    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : P_ROW_BYTES * g.a_k;
+    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : P_ROW_BYTES * g.b_k;
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
     auto issue = [&](int t) {
         const unsigned stage = lds0 + (unsigned)(t & 1) * Cfg::STAGE_BYTES;
@@ -163,12 +186,17 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     // ---- fragment addresses ----
     // k-dense: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile (four consecutive 8-row
     // blocks); the chunk sits at slot chunk ^ (row % 8) of its row.
-    // row-dense: lane (lr, lh) needs k = 16*s + 8*lh + 0..7 of row lr.  With s16 = lane % 16 it supplies,
-    // for each half e of those 8 k, the address of columns 4*(s16 % 4)..+3 (of its 16-column half of
-    // the tile) in k-row 16*s + 8*lh + 4*e + s16/4.  (k % 4) == s16/4 whatever s and e are, so the
-    // swizzle is a per-lane constant and the slice/half offsets are immediates.
+    // row-dense: lane (lr, lh) needs the 16 bytes of k that start at k = SLICE_K * s + (SLICE_K / 2) * lh, of
+    // row lr.  Two transpose reads of RPT k-rows each deliver them; for both the lane supplies the
+    // address of its share of k-row (that start) + RPT * e + kq, columns of its 16-column half of the tile.
+    // (k % RPT) == kq whatever s and e are, so the swizzle is a per-lane constant and the slice / half offsets
+    // are immediates.
     const int frag_row = (lr >> 3) * SWZ_BLOCK + (lr & 7) * P_ROW_BYTES;
-    const int s16 = lane & 15, kq = s16 >> 2;
+    typedef RowDenseGeom<ES> RD;
+    const int s16 = lane & 15;
+    const int kq = ES == 2 ? s16 >> 2 : s16 >> 1;                         // k-row within a transpose read
+    const int sub = ES == 2 ? (s16 & 3) : (s16 & 1);                      // 8-byte piece within the 16 columns
+    const int col_bytes = ((lane >> 4) & 1) * 16 * ES + sub * 8;          // of this lane's address, inside the tile
     int a_frag[P_SLICES], b_frag[P_SLICES];  // k-dense: one address per slice, tiles are immediates
     int a_mn[TM], b_mn[TN];                  // row-dense: one address per tile, slices are immediates
 #pragma unroll
@@ -179,21 +207,21 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-        const int c = (wave_m * TM + i) * 4 + ((lane >> 4) & 1) * 2 + ((s16 & 3) >> 1);
-        a_mn[i] = (lh * 8 + kq) * Cfg::BM * ES + ((c ^ (kq << 2)) << 4) + (s16 & 1) * 8;
+        const int bytes = (wave_m * TM + i) * 32 * ES + col_bytes, c = bytes >> 4;
+        a_mn[i] = (lh * (RD::SLICE_K / 2) + kq) * Cfg::BM * ES + ((c ^ RD::swz(kq)) << 4) + (bytes & 8);
     }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-        const int c = (wave_n * TN + j) * 4 + ((lane >> 4) & 1) * 2 + ((s16 & 3) >> 1);
-        b_mn[j] = Cfg::A_BYTES + (lh * 8 + kq) * Cfg::BN * ES + ((c ^ (kq << 2)) << 4) + (s16 & 1) * 8;
+        const int bytes = (wave_n * TN + j) * 32 * ES + col_bytes, c = bytes >> 4;
+        b_mn[j] = Cfg::A_BYTES + (lh * (RD::SLICE_K / 2) + kq) * Cfg::BN * ES + ((c ^ RD::swz(kq)) << 4) + (bytes & 8);
     }
     auto read_a = [&](const char *stage, auto sl_, int i) -> u32x4_t {
         constexpr int SL = decltype(sl_)::value;
         if constexpr (Cfg::LA == LM_K) {
             return lds_get(stage, a_frag[SL] + i * 4 * SWZ_BLOCK);
         } else {
-            const u32x2_t lo = lds_get_tr16(stage, a_mn[i] + (SL * 16) * Cfg::BM * ES);
-            const u32x2_t hi = lds_get_tr16(stage, a_mn[i] + (SL * 16 + 4) * Cfg::BM * ES);
+            const u32x2_t lo = lds_get_tr<ES>(stage, a_mn[i] + (SL * RD::SLICE_K) * Cfg::BM * ES);
+            const u32x2_t hi = lds_get_tr<ES>(stage, a_mn[i] + (SL * RD::SLICE_K + RD::RPT) * Cfg::BM * ES);
             return u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
     };
@@ -202,8 +230,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         if constexpr (Cfg::LB == LM_K) {
             return lds_get(stage, b_frag[SL] + j * 4 * SWZ_BLOCK);
         } else {
-            const u32x2_t lo = lds_get_tr16(stage, b_mn[j] + (SL * 16) * Cfg::BN * ES);
-            const u32x2_t hi = lds_get_tr16(stage, b_mn[j] + (SL * 16 + 4) * Cfg::BN * ES);
+            const u32x2_t lo = lds_get_tr<ES>(stage, b_mn[j] + (SL * RD::SLICE_K) * Cfg::BN * ES);
+            const u32x2_t hi = lds_get_tr<ES>(stage, b_mn[j] + (SL * RD::SLICE_K + RD::RPT) * Cfg::BN * ES);
             return u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
     };
@@ -316,14 +344,15 @@ template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const vo
     return HODU_ROCM_OK;
 }
 
-// K a whole number of 128-byte stages (64 k for the row-dense layouts, which exist for 16-bit types
-// and need at least one whole 8-column chunk); alignment is what pick_mode already established
+// K a whole number of 128-byte stages; the row-dense layouts exist for 8- and 16-bit types and fetch whole
+// 16-byte chunks of a k-row; alignment is what pick_mode already established
 template <int CK> bool pipe_eligible(int la, int lb, const DevProduct &g) {
     constexpr int ES = Compute<CK>::ES;
     if (g.K <= 0 || ((long)g.K * ES) % P_ROW_BYTES != 0) return false;
     if (la == LM_K && lb == LM_K) return true;
-    if (ES != 2 || la == LM_SCALAR || lb == LM_SCALAR) return false;
-    return (la == LM_K || g.M >= 8) && (lb == LM_K || g.N >= 8);
+    if (ES > 2 || la == LM_SCALAR || lb == LM_SCALAR) return false;
+    constexpr int EPC = 16 / ES;  // a row-dense operand is fetched in whole 16-byte chunks of a k-row
+    return (la == LM_K || (g.M >= EPC && g.M % EPC == 0)) && (lb == LM_K || (g.N >= EPC && g.N % EPC == 0));
 }
 
 }  // namespace mfma

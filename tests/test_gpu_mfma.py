@@ -70,28 +70,31 @@ def test_pipelined_kk_variants(ctx, kind, tile, name):
     ctx.force_tile(-1)
 
 
-@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("kind", ["bf16", "f16", "i32_i8i8"])
 @pytest.mark.parametrize("tile,name", [(10, "pipe256x256w8"), (11, "pipe256x256"), (12, "pipe128x128")])
 @pytest.mark.parametrize("combo", ["KM", "MK", "MM"])
 def test_pipelined_row_dense_variants(ctx, kind, tile, name, combo):
-    """the pipelined kernel with row-dense operands (LDS transpose reads): 1 to 5 stages of 64 k; M and N ragged
-    against every tile but multiples of 8, as the 16-byte row chunks require"""
+    """the pipelined kernel with row-dense operands (LDS transpose reads): 1 to 5 stages of 128 bytes of k; M
+    and N ragged against every tile but multiples of the 16-byte row chunk, as the layout requires"""
     prefix = KINDS[kind][0]
+    es = 1 if kind == "i32_i8i8" else 2
+    epc = 16 // es
     ctx.force_tile(tile)
     try:
         for stages in (1, 2, 3, 5):
-            K = stages * 64
-            lv, rv = views(combo, 296, K, 200)
+            K = stages * 128 // es
+            lv, rv = views(combo, 19 * 16 - (0 if es == 1 else 8), K, 13 * 16 - (0 if es == 1 else 8))
             check_product(ctx, "dot", kind, lv, rv, seed=stages, expect_kernel=f"{prefix}_{name}_{combo}")
         # fewer rows than one tile, and a tile edge that cuts through a 16-column group
-        lv, rv = views(combo, 24, 128, 40)
+        lv, rv = views(combo, 3 * epc, 256 // es, 5 * epc)
         check_product(ctx, "dot", kind, lv, rv, seed=9, expect_kernel=f"{prefix}_{name}_{combo}")
-        # batched with a shared row-dense weight (stride-0 batch) and offsets into larger buffers
         if combo == "KM":
-            check_product(ctx, "matmul", kind, V([3, 72, 128], offset=64), V([128, 80], offset=128).broadcast_to([3, 128, 80]),
+            K = 256 // es
+            # batched with a shared row-dense weight (stride-0 batch) and offsets into larger buffers
+            check_product(ctx, "matmul", kind, V([3, 72, K], offset=64), V([K, 80], offset=128).broadcast_to([3, K, 80]),
                           seed=10, expect_kernel=f"{prefix}_{name}_{combo}")
             # column-sliced weight: leading dimension larger than N
-            check_product(ctx, "dot", kind, V([72, 128]), V([128, 160]).slice(1, 16, 120), seed=11,
+            check_product(ctx, "dot", kind, V([72, K]), V([K, 160]).slice(1, 16, 16 + 6 * 16), seed=11,
                           expect_kernel=f"{prefix}_{name}_{combo}")
     finally:
         ctx.force_tile(-1)
