@@ -54,6 +54,20 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
 #undef HODU_PIPE_CASE
         }
     }
+    if constexpr (SKA == SK_SAME && SKB == SK_F8) {
+        if (pipe_f8_eligible(la, lb, b, g) && (forced < 0 || forced >= 10) && size < 3) {
+            ctx->last_kernel = combo == 0 ? names[17 + size] : names[21 + size];
+#define HODU_PIPE_F8(SZ, BM, BN, WM, WN)                                                                          \
+    if (size == SZ && combo == 0)                                                                                 \
+        return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LM_K, LM_K, SK_F8>>(ctx, a, b, c, g);               \
+    if (size == SZ && combo == 1)                                                                                 \
+        return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LM_K, LM_MN, SK_F8>>(ctx, a, b, c, g);
+            HODU_PIPE_F8(0, 256, 256, 2, 4)
+            HODU_PIPE_F8(1, 256, 256, 2, 2)
+            HODU_PIPE_F8(2, 128, 128, 2, 2)
+#undef HODU_PIPE_F8
+        }
+    }
     // a row-dense LEFT operand needs 32 staging registers more than the 8-wavefront variant has
     // (two wavefronts share a SIMD's register file): those layouts use the 4-wavefront variant
     if (size == 0 && la == LM_MN) size = 1;

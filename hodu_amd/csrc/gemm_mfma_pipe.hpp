@@ -28,6 +28,12 @@
 // column from four rows that 16 lanes read together), so no register-level transpose and no second
 // LDS layout is needed.
 //
+// f8e4m3 right operands (the fused to_dtype of a weight) are DMA'd as the bytes they are and widened
+// to bf16 between the fragment read and the MFMA (v_cvt_scalef32_pk_bf16_fp8, exact): no widened
+// copy ever exists in LDS or HBM.  k-dense f8 rows still move as whole 128-byte lines, which is 128 k
+// = two stages of the bf16 left operand, so the right operand's two buffers each hold a PAIR of
+// stages and are refilled one half per stage; row-dense f8 ([K, N] bytes) moves 64 k-rows per stage.
+//
 // Hazards.  The barrier in stage t is reached by a wavefront only after all its reads of stage t
 // have RETURNED (lgkmcnt(0)) and its own share of stage t+1 has landed (vmcnt(0)); past it, stage t's
 // buffer is dead for everybody and stage t+1 is complete for everybody.
@@ -41,31 +47,51 @@ namespace hodu {
 namespace mfma {
 
 constexpr int P_ROW_BYTES = 128;   // == ROW_BYTES of the swizzled layout
-constexpr int P_SLICES = 4;        // 32-byte k-slices per stage
+constexpr int P_SLICES = 4;        // 32-byte k-slices (of the compute type) per stage
 
 // s_waitcnt immediate for gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
 constexpr int waitcnt_vm(int n) { return (n & 15) | 0x70 | 0xF00 | ((n >> 4) << 14); }
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | 0x70 | ((n >> 4) << 14); }
 
-template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_, int LA_ = LM_K, int LB_ = LM_K> struct PipeConfig {
-    static constexpr int CK = CK_, OUT = OUT_, BM = BM_, BN = BN_, WM = WM_, WN = WN_, LA = LA_, LB = LB_;
+// Row-dense operand geometry for elements of SB bytes in memory feeding a compute type of ES bytes
+// (SB == ES, or SB == 1 under ES == 2 for f8e4m3 storage); a "chunk" is 16 bytes of one k-row.
+//   swizzle   chunk c of k-row k sits at slot c ^ swz(k); one transpose read takes its 16 lanes through
+//             RPT consecutive k-rows, 32 (SB = 2) or 16 (SB = 1) bytes of each, and the swizzle puts those
+//             rows into different banks
+template <int SB, int ES> struct RowDenseGeom {
+    static constexpr int RPT = SB == 2 ? 4 : 8;           // k-rows one transpose read covers
+    static constexpr int EPC = 16 / SB;                    // elements per chunk
+    static constexpr int STAGE_K = 128 / ES;               // k-rows per stage
+    static constexpr int SLICE_K = 32 / ES;                // k per MFMA slice
+    static constexpr int READS = (SLICE_K / 2) / RPT;      // transpose reads per fragment (8 or 16 k per lane)
+    static __device__ __forceinline__ int swz(int k) { return SB == 2 ? (k & 3) << 2 : (k & 7); }
+};
+
+template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_, int LA_ = LM_K, int LB_ = LM_K, int SKB_ = SK_SAME>
+struct PipeConfig {
+    static constexpr int CK = CK_, OUT = OUT_, BM = BM_, BN = BN_, WM = WM_, WN = WN_, LA = LA_, LB = LB_, SKB = SKB_;
     static constexpr int NT = WM * WN * 64, NW = WM * WN;
     static constexpr int ES = Compute<CK>::ES;
+    static constexpr bool B_F8 = SKB == SK_F8;
+    static constexpr int SB = B_F8 ? 1 : ES;               // bytes of a right-operand element in memory
+    static constexpr bool B_PAIR = B_F8 && LB == LM_K;     // right-operand buffers hold two stages each
     static constexpr int BK = P_ROW_BYTES / ES;
-    // k-dense: 8-row blocks of 1 KB, 128 bytes apart; row-dense: [64 k][ROWS] with no gaps
+    // k-dense: 8-row blocks of 1 KB, 128 bytes apart; row-dense: [k-rows of a stage][ROWS] with no gaps
     static constexpr int A_BYTES = (BM / 8) * (LA == LM_K ? SWZ_BLOCK : 1024);
-    static constexpr int B_BYTES = (BN / 8) * (LB == LM_K ? SWZ_BLOCK : 1024);
-    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-    static constexpr int BLOCKS = (BM + BN) / 8;     // DMA instructions per stage
-    static constexpr int DMA_PER_WAVE = BLOCKS / NW;
+    static constexpr int B_BYTES = LB == LM_K ? (BN / 8) * SWZ_BLOCK : (BK * BN * SB);
+    static constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES);
+    static constexpr int PA = (BM / 8) / NW;                                    // DMA instructions per wavefront: a stage of A,
+    static constexpr int PB = (LB == LM_K ? BN / 8 : BK * BN * SB / 1024) / NW;  // a buffer of B,
+    static constexpr int PBS = B_PAIR ? PB / 2 : PB;                            // what of B goes out per stage
+    static constexpr int P = PA + PBS;
     static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
+    static_assert(!B_F8 || CK == CK_BF16, "f8e4m3 storage widens to bf16");
     static_assert(P_ROW_BYTES == ROW_BYTES, "the pipelined kernel uses the swizzled 128-byte-row layout");
-    static_assert(BLOCKS % NW == 0 && (BM / 8) % NW == 0, "DMA split");
+    static_assert((BM / 8) % NW == 0 && PB >= 1 && (!B_PAIR || PB % 2 == 0), "DMA split");
+    static_assert((PA + PB) * 2 < 64, "vmcnt is a 6-bit counter");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
     static_assert((LA == LM_K || (ES <= 2 && BM >= 128)) && (LB == LM_K || (ES <= 2 && BN >= 128)),
                   "row-dense operands: 8- and 16-bit types, tiles of at least 128 rows");
-    static_assert(DMA_PER_WAVE * 2 < 64, "vmcnt is a 6-bit counter");
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
 
 // issued through inline assembly so that the compiler's own wait-count bookkeeping (which would put
@@ -81,8 +107,8 @@ __device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
 //     4e..4e+3 pointing at 16 consecutive columns of k-row e, lane i gets column i of k-rows 0..3;
 //   8-bit elements: lane i receives element (i % 8) of lanes i/8, 2 + i/8, .., 14 + i/8 -- with lanes 2e, 2e+1
 //     pointing at 16 consecutive columns of k-row e, lane i gets column i of k-rows 0..7.
-template <int ES> __device__ __forceinline__ u32x2_t lds_get_tr(const char *lds, int off) {
-    if constexpr (ES == 2) {
+template <int SB> __device__ __forceinline__ u32x2_t lds_get_tr(const char *lds, int off) {
+    if constexpr (SB == 2) {
         typedef short s16x4_t __attribute__((ext_vector_type(4)));
         typedef s16x4_t __attribute__((address_space(3))) * lds_ptr_t;
         return bitcast<u32x2_t>(__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)(lds + off)));
@@ -92,18 +118,13 @@ template <int ES> __device__ __forceinline__ u32x2_t lds_get_tr(const char *lds,
         return bitcast<u32x2_t>(__builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr_t)(uintptr_t)(lds + off)));
     }
 }
+__device__ __forceinline__ u32x2_t lds_get64(const char *lds, int off) { return *reinterpret_cast<const u32x2_t *>(lds + off); }
 
-// Row-dense operand geometry for element size ES (1 or 2 bytes); a "chunk" is 16 bytes of one k-row.
-//   swizzle   chunk c of k-row k sits at slot c ^ swz(k); one transpose read takes its 16 lanes through
-//             RPT consecutive k-rows, 32 (ES = 2) or 16 (ES = 1) bytes of each, and the swizzle puts those rows
-//             into different banks
-template <int ES> struct RowDenseGeom {
-    static constexpr int RPT = ES == 2 ? 4 : 8;          // k-rows one transpose read covers
-    static constexpr int EPC = 16 / ES;                   // elements per chunk
-    static constexpr int STAGE_K = 128 / ES;              // k-rows per stage
-    static constexpr int SLICE_K = 32 / ES;               // k per MFMA slice
-    static __device__ __forceinline__ int swz(int k) { return ES == 2 ? (k & 3) << 2 : (k & 7); }
-};
+// 8 f8e4m3 -> 8 bf16 (exact)
+__device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
+    return u32x4_t{f8pair_to_bf16pair(v.x, false), f8pair_to_bf16pair(v.x, true), f8pair_to_bf16pair(v.y, false),
+                   f8pair_to_bf16pair(v.y, true)};
+}
 
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restrict__ A, const char *__restrict__ B,
@@ -113,7 +134,11 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     typedef Compute32<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;
-    constexpr int TM = Cfg::TM, TN = Cfg::TN, ES = Cfg::ES, P = Cfg::DMA_PER_WAVE;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, ES = Cfg::ES, SB = Cfg::SB, PA = Cfg::PA, PB = Cfg::PB, PBS = Cfg::PBS,
+                  P = Cfg::P;
+    constexpr bool B_F8 = Cfg::B_F8, B_PAIR = Cfg::B_PAIR;
+    typedef RowDenseGeom<ES, ES> GA;
+    typedef RowDenseGeom<SB, ES> GB;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
@@ -126,112 +151,148 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     batch_offsets(g, batch, ao, bo);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
 
-    // ---- DMA plan of this wavefront: P instructions per stage, each one 1 KB of LDS ----
+    // LDS: [A stage 0][A stage 1][B buffer 0][B buffer 1]
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
+    constexpr int B_BASE = 2 * Cfg::A_BYTES;
+
+    // ---- DMA plan of this wavefront: PA + PB instructions, each one 1 KB of LDS ----
     // k-dense operand: a block of 8 rows x 128 B; lane -> (row in block, slot), the slot holds chunk slot ^ row.
-    // row-dense operand: KPI consecutive k-rows of ROWS elements; lane -> (k-row, slot), slot holds chunk
-    // slot ^ ((k % 4) << 2); a chunk that starts past the operand's last row is fetched from the last
-    // whole chunk instead (its columns are never stored).
-    constexpr int PA = (Cfg::BM / 8) / Cfg::NW;  // the first PA instructions of a wavefront belong to A
-    const char *gp[P];       // source address of this lane for stage 0
-    unsigned lds_off[P];     // block offset inside a stage (wave-uniform)
+    // row-dense operand: KPI consecutive k-rows of ROWS elements; lane -> (k-row, slot), the slot holds chunk
+    // slot ^ swz(k); a chunk that starts past the operand's last row is fetched from the last whole chunk
+    // instead (its columns are never stored).
+    const char *gpa[PA], *gpb[PB];    // source address of this lane for stage (buffer) 0
+    unsigned lda[PA], ldb[PB];        // block offset inside a buffer (wave-uniform)
 #pragma unroll
-    for (int p = 0; p < P; p++) {
-        if (p < PA) {
-            const int q = p * Cfg::NW + wave;
-            if constexpr (Cfg::LA == LM_K) {
-                const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
-                int row = m0 + q * 8 + drow;
-                row = row < g.M ? row : g.M - 1;
-                gp[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
-                lds_off[p] = q * SWZ_BLOCK;
-            } else {
-                typedef RowDenseGeom<ES> RD;
-                constexpr int CPR = Cfg::BM / RD::EPC, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
-                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ RD::swz(k);
-                int col = m0 + c * RD::EPC;
-                col = col <= g.M - RD::EPC ? col : g.M - RD::EPC;
-                gp[p] = A + (ao + (long)k * g.a_k + col) * ES;
-                lds_off[p] = q * 1024;
-            }
+    for (int p = 0; p < PA; p++) {
+        const int q = p * Cfg::NW + wave;
+        if constexpr (Cfg::LA == LM_K) {
+            const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+            int row = m0 + q * 8 + drow;
+            row = row < g.M ? row : g.M - 1;
+            gpa[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
+            lda[p] = q * SWZ_BLOCK;
         } else {
-            const int q = (p - PA) * Cfg::NW + wave;
-            if constexpr (Cfg::LB == LM_K) {
-                const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
-                int row = n0 + q * 8 + drow;
-                row = row < g.N ? row : g.N - 1;
-                gp[p] = B + (bo + (long)row * g.b_n) * ES + dchunk * 16;
-                lds_off[p] = Cfg::A_BYTES + q * SWZ_BLOCK;
-            } else {
-                typedef RowDenseGeom<ES> RD;
-                constexpr int CPR = Cfg::BN / RD::EPC, KPI = 64 / CPR;
-                const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ RD::swz(k);
-                int col = n0 + c * RD::EPC;
-                col = col <= g.N - RD::EPC ? col : g.N - RD::EPC;
-                gp[p] = B + (bo + (long)k * g.b_k + col) * ES;
-                lds_off[p] = Cfg::A_BYTES + q * 1024;
-            }
+            constexpr int CPR = Cfg::BM / GA::EPC, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ GA::swz(k);
+            int col = m0 + c * GA::EPC;
+            col = col <= g.M - GA::EPC ? col : g.M - GA::EPC;
+            gpa[p] = A + (ao + (long)k * g.a_k + col) * ES;
+            lda[p] = q * 1024;
         }
     }
-    // bytes a stage advances each operand's source by: 128 bytes of k, or 64 k-rows
-    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : P_ROW_BYTES * g.a_k;
-    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : P_ROW_BYTES * g.b_k;
-    const unsigned lds0 = (unsigned)(uintptr_t)smem;
-    auto issue = [&](int t) {
-        const unsigned stage = lds0 + (unsigned)(t & 1) * Cfg::STAGE_BYTES;
 #pragma unroll
-        for (int p = 0; p < P; p++)
-            dma16_raw(gp[p] + t * (p < PA ? a_adv : b_adv), __builtin_amdgcn_readfirstlane(stage + lds_off[p]));
+    for (int p = 0; p < PB; p++) {
+        const int q = p * Cfg::NW + wave;
+        if constexpr (Cfg::LB == LM_K) {
+            const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+            int row = n0 + q * 8 + drow;
+            row = row < g.N ? row : g.N - 1;
+            gpb[p] = B + (bo + (long)row * g.b_n) * SB + dchunk * 16;
+            ldb[p] = B_BASE + q * SWZ_BLOCK;
+        } else {
+            constexpr int CPR = Cfg::BN / GB::EPC, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ GB::swz(k);
+            int col = n0 + c * GB::EPC;
+            col = col <= g.N - GB::EPC ? col : g.N - GB::EPC;
+            gpb[p] = B + (bo + (long)k * g.b_k + col) * SB;
+            ldb[p] = B_BASE + q * 1024;
+        }
+    }
+    // bytes a stage advances an operand's source by: 128 bytes of k, or a stage's k-rows; a k-dense f8 buffer
+    // is 128 bytes of k as well, but that is two stages
+    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : (long)GA::STAGE_K * g.a_k * ES;
+    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : (long)GB::STAGE_K * g.b_k * SB;
+
+    const int T = g.K * ES / P_ROW_BYTES;           // stages
+    const int TB = B_PAIR ? (T + 1) / 2 : T;        // right-operand buffers' worth of k
+
+    // element e of a stage's issue list: its PA instructions of A (stage t_a), then PBS of B (buffer tb; a paired
+    // buffer goes out in two halves, and which half is a run-time fact: the issuing stage's parity).  After
+    // unrolling, e is a constant and the chains below fold to one instruction.
+    auto dma_element = [&](int e, int t_a, bool do_a, int tb, int half, bool do_b) {
+#pragma unroll
+        for (int p = 0; p < PA; p++)
+            if (e == p && do_a)
+                dma16_raw(gpa[p] + t_a * a_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(t_a & 1) * Cfg::A_BYTES + lda[p]));
+#pragma unroll
+        for (int p = 0; p < PBS; p++)
+            if (e == PA + p && do_b) {
+                const char *src = gpb[p];
+                unsigned off = ldb[p];
+                if constexpr (B_PAIR) {
+                    src = half ? gpb[p + PBS] : gpb[p];
+                    off = half ? ldb[p + PBS] : ldb[p];
+                }
+                dma16_raw(src + tb * b_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(tb & 1) * Cfg::B_BYTES + off));
+            }
     };
 
     // ---- fragment addresses ----
     // k-dense: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile (four consecutive 8-row
-    // blocks); the chunk sits at slot chunk ^ (row % 8) of its row.
-    // row-dense: lane (lr, lh) needs the 16 bytes of k that start at k = SLICE_K * s + (SLICE_K / 2) * lh, of
-    // row lr.  Two transpose reads of RPT k-rows each deliver them; for both the lane supplies the
+    // blocks); the chunk sits at slot chunk ^ (row % 8) of its row.  f8 storage: the lane's 8 k are 8 bytes,
+    // half lh of chunk s (second stage of the pair: s + 4) of the 128-byte row.
+    // row-dense: lane (lr, lh) needs the (SLICE_K / 2) k that start at k = SLICE_K * s + (SLICE_K / 2) * lh, of
+    // row lr.  One or two transpose reads of RPT k-rows each deliver them; for each the lane supplies the
     // address of its share of k-row (that start) + RPT * e + kq, columns of its 16-column half of the tile.
     // (k % RPT) == kq whatever s and e are, so the swizzle is a per-lane constant and the slice / half offsets
     // are immediates.
     const int frag_row = (lr >> 3) * SWZ_BLOCK + (lr & 7) * P_ROW_BYTES;
-    typedef RowDenseGeom<ES> RD;
     const int s16 = lane & 15;
-    const int kq = ES == 2 ? s16 >> 2 : s16 >> 1;                         // k-row within a transpose read
-    const int sub = ES == 2 ? (s16 & 3) : (s16 & 1);                      // 8-byte piece within the 16 columns
-    const int col_bytes = ((lane >> 4) & 1) * 16 * ES + sub * 8;          // of this lane's address, inside the tile
     int a_frag[P_SLICES], b_frag[P_SLICES];  // k-dense: one address per slice, tiles are immediates
     int a_mn[TM], b_mn[TN];                  // row-dense: one address per tile, slices are immediates
 #pragma unroll
     for (int sl = 0; sl < P_SLICES; sl++) {
-        const int slot = ((2 * sl + lh) ^ (lr & 7)) << 4;
-        a_frag[sl] = (wave_m * TM) * 4 * SWZ_BLOCK + frag_row + slot;
-        b_frag[sl] = Cfg::A_BYTES + (wave_n * TN) * 4 * SWZ_BLOCK + frag_row + slot;
+        a_frag[sl] = (wave_m * TM) * 4 * SWZ_BLOCK + frag_row + (((2 * sl + lh) ^ (lr & 7)) << 4);
+        b_frag[sl] = B_BASE + (wave_n * TN) * 4 * SWZ_BLOCK + frag_row +
+                     (B_F8 ? ((sl ^ (lr & 7)) << 4) + lh * 8 : (((2 * sl + lh) ^ (lr & 7)) << 4));
     }
+    {
+        const int kq = ES == 2 ? s16 >> 2 : s16 >> 1, sub = ES == 2 ? (s16 & 3) : (s16 & 1);
+        const int col_bytes = ((lane >> 4) & 1) * 16 * ES + sub * 8;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int bytes = (wave_m * TM + i) * 32 * ES + col_bytes, c = bytes >> 4;
-        a_mn[i] = (lh * (RD::SLICE_K / 2) + kq) * Cfg::BM * ES + ((c ^ RD::swz(kq)) << 4) + (bytes & 8);
+        for (int i = 0; i < TM; i++) {
+            const int bytes = (wave_m * TM + i) * 32 * ES + col_bytes, c = bytes >> 4;
+            a_mn[i] = (lh * (GA::SLICE_K / 2) + kq) * Cfg::BM * ES + ((c ^ GA::swz(kq)) << 4) + (bytes & 8);
+        }
     }
+    {
+        const int kq = SB == 2 ? s16 >> 2 : s16 >> 1, sub = SB == 2 ? (s16 & 3) : (s16 & 1);
+        const int col_bytes = ((lane >> 4) & 1) * 16 * SB + sub * 8;
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int bytes = (wave_n * TN + j) * 32 * ES + col_bytes, c = bytes >> 4;
-        b_mn[j] = Cfg::A_BYTES + (lh * (RD::SLICE_K / 2) + kq) * Cfg::BN * ES + ((c ^ RD::swz(kq)) << 4) + (bytes & 8);
+        for (int j = 0; j < TN; j++) {
+            const int bytes = (wave_n * TN + j) * 32 * SB + col_bytes, c = bytes >> 4;
+            b_mn[j] = B_BASE + (lh * (GB::SLICE_K / 2) + kq) * Cfg::BN * SB + ((c ^ GB::swz(kq)) << 4) + (bytes & 8);
+        }
     }
-    auto read_a = [&](const char *stage, auto sl_, int i) -> u32x4_t {
+    // fragment of the left operand: tile i, slice SL of stage t
+    auto read_a = [&](int t, auto sl_, int i) -> u32x4_t {
         constexpr int SL = decltype(sl_)::value;
+        const char *buf = smem + (t & 1) * Cfg::A_BYTES;
         if constexpr (Cfg::LA == LM_K) {
-            return lds_get(stage, a_frag[SL] + i * 4 * SWZ_BLOCK);
+            return lds_get(buf, a_frag[SL] + i * 4 * SWZ_BLOCK);
         } else {
-            const u32x2_t lo = lds_get_tr<ES>(stage, a_mn[i] + (SL * RD::SLICE_K) * Cfg::BM * ES);
-            const u32x2_t hi = lds_get_tr<ES>(stage, a_mn[i] + (SL * RD::SLICE_K + RD::RPT) * Cfg::BM * ES);
+            const u32x2_t lo = lds_get_tr<ES>(buf, a_mn[i] + (SL * GA::SLICE_K) * Cfg::BM * ES);
+            const u32x2_t hi = lds_get_tr<ES>(buf, a_mn[i] + (SL * GA::SLICE_K + GA::RPT) * Cfg::BM * ES);
             return u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
     };
-    auto read_b = [&](const char *stage, auto sl_, int j) -> u32x4_t {
+    // fragment of the right operand; f8 storage comes back as 8 raw bytes in .x/.y and is widened at its use
+    auto read_b = [&](int t, auto sl_, int j) -> u32x4_t {
         constexpr int SL = decltype(sl_)::value;
-        if constexpr (Cfg::LB == LM_K) {
-            return lds_get(stage, b_frag[SL] + j * 4 * SWZ_BLOCK);
+        const int tb = B_PAIR ? t >> 1 : t;
+        const char *buf = smem + (tb & 1) * Cfg::B_BYTES;
+        if constexpr (Cfg::LB == LM_K && !B_F8) {
+            return lds_get(buf, b_frag[SL] + j * 4 * SWZ_BLOCK);
+        } else if constexpr (Cfg::LB == LM_K) {
+            // second stage of the pair: chunk s + 4, i.e. bit 6 of the byte offset flipped (the swizzle is an XOR)
+            const u32x2_t v = lds_get64(buf, (b_frag[SL] ^ ((t & 1) << 6)) + j * 4 * SWZ_BLOCK);
+            return u32x4_t{v.x, v.y, 0u, 0u};
+        } else if constexpr (B_F8) {
+            const u32x2_t v = lds_get_tr<1>(buf, b_mn[j] + (SL * GB::SLICE_K) * Cfg::BN * SB);
+            return u32x4_t{v.x, v.y, 0u, 0u};
         } else {
-            const u32x2_t lo = lds_get_tr<ES>(stage, b_mn[j] + (SL * RD::SLICE_K) * Cfg::BN * ES);
-            const u32x2_t hi = lds_get_tr<ES>(stage, b_mn[j] + (SL * RD::SLICE_K + RD::RPT) * Cfg::BN * ES);
+            const u32x2_t lo = lds_get_tr<SB>(buf, b_mn[j] + (SL * GB::SLICE_K) * Cfg::BN * SB);
+            const u32x2_t hi = lds_get_tr<SB>(buf, b_mn[j] + (SL * GB::SLICE_K + GB::RPT) * Cfg::BN * SB);
             return u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
     };
@@ -245,36 +306,35 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
 
-    const int T = g.K * ES / P_ROW_BYTES;
-
     // One k-slice of work, in an explicitly pinned order: the MFMAs of slice CUR (register set CUR % 2),
-    // with the fragment reads of slice RD of stage t_rd (RD < 0: none) and DMA instructions
-    // [D0, D0 + DN) of stage t_dma spread evenly between them.  Neither the reads nor the DMA then
-    // arrive in bursts: a burst of DMA instructions fills the memory pipeline's issue queue and
-    // stalls the wavefront in front of its next MFMA.
-    auto slice_step = [&](auto cur_, auto rd_, auto d0_, auto dn_, int t_rd, int t_dma, bool do_dma) {
+    // with the fragment reads of slice RD of stage t_rd and DMA instructions [D0, D0 + DN) of the issue list
+    // spread evenly between them.  The issue list of a stage is its PA instructions of A followed by PBS of B.
+    // Neither the reads nor the DMA then arrive in bursts: a burst of DMA instructions fills the memory
+    // pipeline's issue queue and stalls the wavefront in front of its next MFMA.
+    //   t_a / do_a   stage of A to fetch, and whether it exists
+    //   tb / half / do_b   buffer of B to fetch (a half of it when the buffers hold pairs), and whether it exists
+    auto slice_step = [&](auto cur_, auto rd_, auto d0_, auto dn_, int t_rd, int t_a, bool do_a, int tb, int half,
+                          bool do_b) {
         constexpr int SET = decltype(cur_)::value & 1, RD = decltype(rd_)::value;
         constexpr int D0 = decltype(d0_)::value, DN = decltype(dn_)::value;
-        constexpr int MF = TM * TN, RN = RD >= 0 ? TM + TN : 0;
-        const char *stage_rd = smem + (t_rd & 1) * Cfg::STAGE_BYTES;
-        const unsigned stage_dma = lds0 + (unsigned)(t_dma & 1) * Cfg::STAGE_BYTES;
+        constexpr int MF = TM * TN, RN = TM + TN;
+        u32x4_t bcur = fb[SET][0];
 #pragma unroll
         for (int idx = 0; idx < MF; idx++) {
 #pragma unroll
             for (int r = 0; r < RN; r++) {
-                if (r * MF / (RN > 0 ? RN : 1) != idx) continue;
-                typedef std::integral_constant<int, (RD >= 0 ? RD : 0)> RS;
-                if (r < TM) fa[RS::value & 1][r] = read_a(stage_rd, RS{}, r);
-                else fb[RS::value & 1][r - TM] = read_b(stage_rd, RS{}, r - TM);
+                if (r * MF / RN != idx) continue;
+                typedef std::integral_constant<int, RD> RS;
+                if (r < TM) fa[RD & 1][r] = read_a(t_rd, RS{}, r);
+                else fb[RD & 1][r - TM] = read_b(t_rd, RS{}, r - TM);
             }
+            if (idx % TM == 0) bcur = B_F8 ? widen_f8x8(u32x2_t{fb[SET][idx / TM].x, fb[SET][idx / TM].y}) : fb[SET][idx / TM];
             // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
-            Cmp::mma(fb[SET][idx / TM], fa[SET][idx % TM], acc[idx % TM][idx / TM]);
+            Cmp::mma(bcur, fa[SET][idx % TM], acc[idx % TM][idx / TM]);
 #pragma unroll
             for (int d = 0; d < DN; d++) {
                 if (d * MF / (DN > 0 ? DN : 1) != idx) continue;
-                if (do_dma)
-                    dma16_raw(gp[D0 + d] + t_dma * (D0 + d < PA ? a_adv : b_adv),
-                              __builtin_amdgcn_readfirstlane(stage_dma + lds_off[D0 + d]));
+                dma_element(D0 + d, t_a, do_a, tb, half, do_b);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -287,34 +347,68 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     typedef std::integral_constant<int, PH> DH;
     typedef std::integral_constant<int, P - PH> DR;
 
-    issue(0);
+    // prologue: stages 0 and 1 of A, buffers 0 and 1 of B (with paired buffers that is stages 0..3 of B)
+    auto issue_all = [&](int t, bool do_a, bool do_b) {
+#pragma unroll
+        for (int p = 0; p < PA; p++)
+            if (do_a) dma16_raw(gpa[p] + t * a_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(t & 1) * Cfg::A_BYTES + lda[p]));
+#pragma unroll
+        for (int p = 0; p < PB; p++)
+            if (do_b) dma16_raw(gpb[p] + t * b_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(t & 1) * Cfg::B_BYTES + ldb[p]));
+    };
+    issue_all(0, true, true);
     if (T > 1) {
-        issue(1);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(P));
+        issue_all(1, true, TB > 1);
+        // everything of stage 0 has landed once at most stage 1's instructions are outstanding
+        if (TB > 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA + PB));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA));
     } else {
         __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[0][i] = read_a(smem, I0{}, i);
+    for (int i = 0; i < TM; i++) fa[0][i] = read_a(0, I0{}, i);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[0][j] = read_b(smem, I0{}, j);
+    for (int j = 0; j < TN; j++) fb[0][j] = read_b(0, I0{}, j);
+
+    // What stage t issues behind its barrier (second half of the list: during slice 0 of stage t+1):
+    //   A: stage t+2.
+    //   B, one buffer per stage: buffer t+2.
+    //   B, paired buffers: buffer b holds stages 2b, 2b+1 and is free once stage 2b+1 is done.  Odd t frees
+    //      buffer (t-1)/2 and issues the first half of buffer (t+3)/2 into it; the following even stage issues
+    //      the second half.  Both have two or more stages to land.
+    auto b_target = [&](int t, int &tb, int &half, bool &ok) {
+        if constexpr (B_PAIR) {
+            tb = (t + 2 + (t & 1)) >> 1;
+            half = (t & 1) ? 0 : 1;
+            ok = t >= 1 && tb < TB;
+        } else {
+            tb = t + 2;
+            half = 0;
+            ok = tb < TB;
+        }
+    };
 
     // The loop body is branch-free apart from the DMA predicates: past the last stage the reads fetch
     // LDS bytes nobody uses and the barrier is one too many, both harmless and cheaper than a second
     // copy of the MFMA code.
     for (int t = 0; t < T; t++) {
-        // slice 0: multiply it, read slice 1, issue the second half of stage t+1's DMA (stage 1 came whole)
-        slice_step(I0{}, I1{}, DH{}, DR{}, t, t + 1, t >= 1 && t + 1 < T);
-        slice_step(I1{}, I2{}, I0{}, I0{}, t, 0, false);
-        slice_step(I2{}, I3{}, I0{}, I0{}, t, 0, false);
-        // stage t+1 (the only DMA in flight) has landed and every read of stage t has returned
+        int tb, half;
+        bool ok_b;
+        // slice 0: multiply it, read slice 1, issue the second half of what stage t-1 started (stage 1 came whole)
+        b_target(t - 1, tb, half, ok_b);
+        slice_step(I0{}, I1{}, DH{}, DR{}, t, t + 1, t >= 1 && t + 1 < T, tb, half, t >= 1 && ok_b);
+        slice_step(I1{}, I2{}, I0{}, I0{}, t, 0, false, 0, 0, false);
+        slice_step(I2{}, I3{}, I0{}, I0{}, t, 0, false, 0, 0, false);
+        // everything issued so far has landed (the youngest of it a whole stage ago) and every read of stage t
+        // has returned
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        // slice 3: multiply it, read slice 0 of stage t+1, issue the first half of stage t+2's DMA
-        slice_step(I3{}, I0{}, I0{}, DH{}, t + 1, t + 2, t + 2 < T);
+        // slice 3: multiply it, read slice 0 of stage t+1, issue the first half of this stage's list
+        b_target(t, tb, half, ok_b);
+        slice_step(I3{}, I0{}, I0{}, DH{}, t + 1, t + 2, t + 2 < T, tb, half, ok_b);
     }
 
     out_t *Cb = C + batch * (long)g.M * g.N;
@@ -353,6 +447,18 @@ template <int CK> bool pipe_eligible(int la, int lb, const DevProduct &g) {
     if (ES > 2 || la == LM_SCALAR || lb == LM_SCALAR) return false;
     constexpr int EPC = 16 / ES;  // a row-dense operand is fetched in whole 16-byte chunks of a k-row
     return (la == LM_K || (g.M >= EPC && g.M % EPC == 0)) && (lb == LM_K || (g.N >= EPC && g.N % EPC == 0));
+}
+
+// bf16 left operand k-dense, f8e4m3 right operand k-dense or row-dense.  DMA moves 16-byte chunks, so the
+// byte-sized operand needs 16-byte alignment of everything pick_mode only checked to 8; its k-dense form
+// moves whole 128-byte lines of k, i.e. K is a multiple of 128.
+inline bool pipe_f8_eligible(int la, int lb, const void *b, const DevProduct &g) {
+    if (la != LM_K || lb == LM_SCALAR || g.K <= 0 || g.K % 64 != 0) return false;
+    if (((uintptr_t)b + (uintptr_t)g.b_off) % 16 != 0) return false;
+    for (int d = 0; d < g.nb; d++)
+        if (g.b_bs[d] % 16 != 0) return false;
+    if (lb == LM_K) return g.K % 128 == 0 && (g.N == 1 || g.b_n % 16 == 0);
+    return g.N >= 16 && g.N % 16 == 0 && g.b_k % 16 == 0;
 }
 
 }  // namespace mfma

@@ -100,6 +100,31 @@ def test_pipelined_row_dense_variants(ctx, kind, tile, name, combo):
         ctx.force_tile(-1)
 
 
+@pytest.mark.parametrize("tile,name", [(10, "pipe256x256w8"), (11, "pipe256x256"), (12, "pipe128x128")])
+@pytest.mark.parametrize("combo", ["KK", "KM"])
+def test_pipelined_f8_weight_variants(ctx, tile, name, combo):
+    """fused f8e4m3 weights in the pipelined kernel: raw bytes through LDS-DMA, widened between fragment read and
+    MFMA.  k-dense weights move 128 k per buffer (pairs of stages: 1, 2, 3 and 5 pairs), row-dense ones 64 k-rows
+    per stage (odd and even stage counts)."""
+    kind, prefix = "bf16_f8e4m3w", KINDS["bf16_f8e4m3w"][0]
+    ctx.force_tile(tile)
+    try:
+        for K in ((128, 256, 384, 640) if combo == "KK" else (64, 128, 192, 320)):
+            lv, rv = views(combo, 296, K, 208)
+            check_product(ctx, "dot", kind, lv, rv, seed=K, rscale=2.0, expect_kernel=f"{prefix}_{name}_{combo}")
+        lv, rv = views(combo, 24, 256, 48)
+        check_product(ctx, "dot", kind, lv, rv, seed=9, rscale=2.0, expect_kernel=f"{prefix}_{name}_{combo}")
+        # weight shared across a batch (stride 0), at a 16-byte-aligned offset, with a leading dimension larger
+        # than its extent
+        if combo == "KK":
+            w = V([80, 512], offset=64).slice(1, 128, 384).t().broadcast_to([3, 256, 80])
+        else:
+            w = V([256, 160], offset=32).slice(1, 16, 112).broadcast_to([3, 256, 96])
+        check_product(ctx, "matmul", kind, V([3, 72, 256]), w, seed=10, rscale=2.0, expect_kernel=f"{prefix}_{name}_{combo}")
+    finally:
+        ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("kind", list(KINDS))
 def test_scalar_load_variant(ctx, kind):
     prefix, _, _ = KINDS[kind]
