@@ -226,6 +226,7 @@ def main():
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
     ap.add_argument("--graph", action="store_true", help="with --only: replay the K launches as one HIP graph")
+    ap.add_argument("--force-splitk", type=int, default=-1, help="testing hook: pin the number of K ranges")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every GPU box here has one GPU and no collective or sharded "
@@ -237,6 +238,7 @@ def main():
     ctx = ffi.Context(0)
     info = ctx.device_info()
     ctx.force_tile(args.force_tile)
+    ctx.force_splitk(args.force_splitk)
     if args.only == "copy":
         # calibration for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain dense copy of known size
         # (hodu_rocm_contiguous on a contiguous f32 buffer reads n bytes and writes n bytes)

@@ -28,7 +28,9 @@ struct hodu_rocm_ctx {
     hipDeviceProp_t props{};
     hodu::Workspace workspace;  // split-K partial sums; grown on demand, owned by the context
     const char *last_kernel = "";
-    int force_tile = -1;  // testing hook: pins the MFMA tile size
+    int force_tile = -1;    // testing hook: pins the MFMA tile size
+    int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
+    char kernel_name[96] = {0};  // storage for a composed last_kernel name
 };
 
 namespace hodu {

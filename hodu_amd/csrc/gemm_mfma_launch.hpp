@@ -12,7 +12,7 @@ namespace mfma {
 // type -- the software-pipelined kernels of gemm_mfma_pipe.hpp: KK at four tile shapes and, for the
 // 16-bit types, KM / MK / MM at the three larger ones.  The tile is the largest that still yields at
 // least one workgroup per compute unit.
-constexpr int kVariants = 30;
+constexpr int kVariants = 32;
 template <int CK, int SKA, int SKB, int OUT>
 int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
                 const char *const names[kVariants]) {
@@ -30,18 +30,47 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64
     const int forced = ctx->force_tile;
     int size = forced >= 0 ? forced % 10 : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 2 : 3;
+    // A product too small to fill the machine with 128x128 tiles is cut along K instead of shrinking the tile
+    // further (pipelined kernels only): same HBM traffic, four times fewer bytes through LDS per flop.
+    const int stages = (int)((long)g.K * ES / 128);
+    const long elems = g.batches * (long)g.M * g.N;
+    bool pipe_ok = false;  // one of the pipelined kernels will take this product
+    if constexpr (SKA == SK_SAME && SKB == SK_SAME) pipe_ok = pipe_eligible<CK>(la, lb, g) && (forced < 0 || forced >= 10);
+    if constexpr (SKA == SK_SAME && SKB == SK_F8) pipe_ok = pipe_f8_eligible(la, lb, b, g) && (forced < 0 || forced >= 10);
+    int splits = 1;
+    if (!pipe_ok) {
+    } else if (forced < 0 && size == 3) {
+        splits = pick_splits(tiles(128, 128), cus, stages, elems, ctx->force_splits);
+        if (splits > 1) size = 2;
+    } else if (ctx->force_splits >= 1 && (size < 3 || size == 4)) {
+        splits = pick_splits(1, cus, stages, elems, ctx->force_splits);
+    }
+    if (size == 4 && !pipe_ok) size = 2;  // 256x128 exists as a pipelined kernel only
+    auto named = [&](const char *base, int sp) -> const char * {
+        if (sp <= 1) return base;
+        snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_splitk%d", base, sp);
+        return ctx->kernel_name;
+    };
     const int combo = (la == LM_MN ? 2 : 0) + (lb == LM_MN ? 1 : 0);
     if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
         // testing hook values 10..13 pin the pipelined kernel's tile, 0..3 the general kernel's
-        if (pipe_eligible<CK>(la, lb, g) && (forced < 0 || forced >= 10) && (combo == 0 || size < 3)) {
-            ctx->last_kernel = combo == 0 ? names[17 + size] : names[21 + (combo - 1) * 3 + size];
+        if (pipe_ok && size == 4 && combo <= 1) {
+            ctx->last_kernel = named(names[30 + combo], splits);
+            if (combo == 0) return launch_pipe<PipeConfig<CK, OUT, 256, 128, 2, 2, LM_K, LM_K, SK_SAME, 3>>(ctx, a, b, c, g, splits);
+            if constexpr (ES <= 2)
+                return launch_pipe<PipeConfig<CK, OUT, 256, 128, 2, 2, LM_K, LM_MN, SK_SAME, 3>>(ctx, a, b, c, g, splits);
+        }
+        if (pipe_ok && size < 4 && (combo == 0 || size < 3)) {
+            ctx->last_kernel = named(combo == 0 ? names[17 + size] : names[21 + (combo - 1) * 3 + size], splits);
 #define HODU_PIPE_CASE(SZ, BM, BN, WM, WN, LA, LB) \
-    if (size == SZ) return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LA, LB>>(ctx, a, b, c, g);
+    if (size == SZ) return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LA, LB>>(ctx, a, b, c, g, splits);
+#define HODU_PIPE_CASE4(SZ, BM, BN, WM, WN, LA, LB) \
+    if (size == SZ) return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LA, LB, SK_SAME, 4>>(ctx, a, b, c, g, splits);
 #define HODU_PIPE_COMBO(CB, LA, LB)                       \
     if (combo == CB) {                                    \
         HODU_PIPE_CASE(0, 256, 256, 2, 4, LA, LB)         \
         HODU_PIPE_CASE(1, 256, 256, 2, 2, LA, LB)         \
-        HODU_PIPE_CASE(2, 128, 128, 2, 2, LA, LB)         \
+        HODU_PIPE_CASE4(2, 128, 128, 2, 2, LA, LB)        \
     }
             HODU_PIPE_COMBO(0, LM_K, LM_K)
             if constexpr (ES <= 2) {
@@ -49,22 +78,28 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
                 HODU_PIPE_COMBO(2, LM_MN, LM_K)
                 HODU_PIPE_COMBO(3, LM_MN, LM_MN)
             }
-            if (combo == 0) return launch_pipe<PipeConfig<CK, OUT, 64, 64, 2, 2>>(ctx, a, b, c, g);
+            if (combo == 0) return launch_pipe<PipeConfig<CK, OUT, 64, 64, 2, 2, LM_K, LM_K, SK_SAME, 4>>(ctx, a, b, c, g, 1);
 #undef HODU_PIPE_COMBO
+#undef HODU_PIPE_CASE4
 #undef HODU_PIPE_CASE
         }
     }
     if constexpr (SKA == SK_SAME && SKB == SK_F8) {
-        if (pipe_f8_eligible(la, lb, b, g) && (forced < 0 || forced >= 10) && size < 3) {
-            ctx->last_kernel = combo == 0 ? names[17 + size] : names[21 + size];
-#define HODU_PIPE_F8(SZ, BM, BN, WM, WN)                                                                          \
+        if (pipe_ok && size == 4 && combo <= 1) {
+            ctx->last_kernel = named(names[30 + combo], splits);
+            if (combo == 0) return launch_pipe<PipeConfig<CK, OUT, 256, 128, 2, 2, LM_K, LM_K, SK_F8, 3>>(ctx, a, b, c, g, splits);
+            return launch_pipe<PipeConfig<CK, OUT, 256, 128, 2, 2, LM_K, LM_MN, SK_F8, 3>>(ctx, a, b, c, g, splits);
+        }
+        if (pipe_ok && size < 3) {
+            ctx->last_kernel = named(combo == 0 ? names[17 + size] : names[21 + size], splits);
+#define HODU_PIPE_F8(SZ, BM, BN, WM, WN, NST)                                                                     \
     if (size == SZ && combo == 0)                                                                                 \
-        return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LM_K, LM_K, SK_F8>>(ctx, a, b, c, g);               \
+        return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LM_K, LM_K, SK_F8, NST>>(ctx, a, b, c, g, splits);  \
     if (size == SZ && combo == 1)                                                                                 \
-        return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LM_K, LM_MN, SK_F8>>(ctx, a, b, c, g);
-            HODU_PIPE_F8(0, 256, 256, 2, 4)
-            HODU_PIPE_F8(1, 256, 256, 2, 2)
-            HODU_PIPE_F8(2, 128, 128, 2, 2)
+        return launch_pipe<PipeConfig<CK, OUT, BM, BN, WM, WN, LM_K, LM_MN, SK_F8, NST>>(ctx, a, b, c, g, splits);
+            HODU_PIPE_F8(0, 256, 256, 2, 4, 2)
+            HODU_PIPE_F8(1, 256, 256, 2, 2, 2)
+            HODU_PIPE_F8(2, 128, 128, 2, 2, 4)
 #undef HODU_PIPE_F8
         }
     }
@@ -96,7 +131,8 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
      P "_pipe256x256w8_KK", P "_pipe256x256_KK", P "_pipe128x128_KK", P "_pipe64x64_KK",                           \
      P "_pipe256x256w8_KM", P "_pipe256x256_KM", P "_pipe128x128_KM",                                              \
      P "_pipe256x256w8_MK", P "_pipe256x256_MK", P "_pipe128x128_MK",                                              \
-     P "_pipe256x256w8_MM", P "_pipe256x256_MM", P "_pipe128x128_MM"}
+     P "_pipe256x256w8_MM", P "_pipe256x256_MM", P "_pipe128x128_MM",                                              \
+     P "_pipe256x128_KK", P "_pipe256x128_KM"}
 
 }  // namespace mfma
 }  // namespace hodu

@@ -67,29 +67,37 @@ template <int SB, int ES> struct RowDenseGeom {
     static __device__ __forceinline__ int swz(int k) { return SB == 2 ? (k & 3) << 2 : (k & 7); }
 };
 
-template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_, int LA_ = LM_K, int LB_ = LM_K, int SKB_ = SK_SAME>
+// k-dense LDS layout of the pipelined kernels: rows of 128 bytes back to back (no padding: it buys a deeper
+// stage ring), 16-byte chunk c of row r at slot c ^ ((r >> 1) & 7).  The 16 rows one ds_read_b128 phase touches
+// then spread over all 64 banks: bank group (of 16) = (r & 1) * 8 + (c ^ ((r >> 1) & 7)).
+__device__ __forceinline__ int kd_slot(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+template <int CK_, int OUT_, int BM_, int BN_, int WM_, int WN_, int LA_ = LM_K, int LB_ = LM_K, int SKB_ = SK_SAME,
+          int NST_ = 2>
 struct PipeConfig {
     static constexpr int CK = CK_, OUT = OUT_, BM = BM_, BN = BN_, WM = WM_, WN = WN_, LA = LA_, LB = LB_, SKB = SKB_;
+    static constexpr int NST = NST_;                       // stages of the LDS ring
     static constexpr int NT = WM * WN * 64, NW = WM * WN;
     static constexpr int ES = Compute<CK>::ES;
     static constexpr bool B_F8 = SKB == SK_F8;
     static constexpr int SB = B_F8 ? 1 : ES;               // bytes of a right-operand element in memory
     static constexpr bool B_PAIR = B_F8 && LB == LM_K;     // right-operand buffers hold two stages each
     static constexpr int BK = P_ROW_BYTES / ES;
-    // k-dense: 8-row blocks of 1 KB, 128 bytes apart; row-dense: [k-rows of a stage][ROWS] with no gaps
-    static constexpr int A_BYTES = (BM / 8) * (LA == LM_K ? SWZ_BLOCK : 1024);
-    static constexpr int B_BYTES = LB == LM_K ? (BN / 8) * SWZ_BLOCK : (BK * BN * SB);
-    static constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES);
+    // k-dense: rows of 128 bytes; row-dense: [k-rows of a stage][ROWS]; both without gaps
+    static constexpr int A_BYTES = BM * P_ROW_BYTES;
+    static constexpr int B_BYTES = LB == LM_K ? BN * P_ROW_BYTES : (BK * BN * SB);
+    static constexpr int LDS_BYTES = NST * (A_BYTES + B_BYTES);
     static constexpr int PA = (BM / 8) / NW;                                    // DMA instructions per wavefront: a stage of A,
     static constexpr int PB = (LB == LM_K ? BN / 8 : BK * BN * SB / 1024) / NW;  // a buffer of B,
     static constexpr int PBS = B_PAIR ? PB / 2 : PB;                            // what of B goes out per stage
     static constexpr int P = PA + PBS;
     static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 MFMA tiles per wave
+    static_assert(NST >= 2 && NST <= 4, "ring depth");
     static_assert(!B_F8 || CK == CK_BF16, "f8e4m3 storage widens to bf16");
-    static_assert(P_ROW_BYTES == ROW_BYTES, "the pipelined kernel uses the swizzled 128-byte-row layout");
     static_assert((BM / 8) % NW == 0 && PB >= 1 && (!B_PAIR || PB % 2 == 0), "DMA split");
-    static_assert((PA + PB) * 2 < 64, "vmcnt is a 6-bit counter");
+    static_assert((NST - 1) * (PA + PB) < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
+    static_assert(NW * 32 * (TN * 128 + 16) <= LDS_BYTES, "the epilogue stages a 32-row band per wavefront in LDS");
     static_assert((LA == LM_K || (ES <= 2 && BM >= 128)) && (LB == LM_K || (ES <= 2 && BN >= 128)),
                   "row-dense operands: 8- and 16-bit types, tiles of at least 128 rows");
 };
@@ -126,10 +134,57 @@ __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
                    f8pair_to_bf16pair(v.y, true)};
 }
 
+// Epilogue for one 32-row band of a wavefront's tile (TN accumulator tiles side by side): the values go through a
+// wavefront-private patch of LDS so that they leave as whole rows -- 16 contiguous bytes per lane, a row of the
+// band per 2..16 lanes -- instead of the accumulator layout's 8-byte pieces of 32 different rows per instruction
+// (measured: 13 us of a 37 us launch spent storing a 256 x 256 bf16 tile that way).
+//   acc layout (operands swapped): lane (lr, lh) holds row lr, columns 32*j + 8*q + 4*lh + e of the band.
+template <int OUT, int TN, class acc_t>
+__device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,
+                                                   int n_base, int lane, int M, int N) {
+    typedef typename Out<OUT>::T out_t;
+    constexpr int OS = sizeof(out_t), ROWB = TN * 32 * OS, PITCH = ROWB + 16, EPV = 16 / OS;
+    constexpr int CPR = ROWB / 16, RPP = 64 / CPR;  // 16-byte chunks per row, rows per pass of the wavefront
+    static_assert(CPR <= 64 && 32 % RPP == 0, "band geometry");
+    const int lr = lane & 31, lh = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            struct alignas(OS * 4) Quad { out_t v[4]; };
+            Quad w;
+#pragma unroll
+            for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][4 * q + e]);
+            *reinterpret_cast<Quad *>(patch + lr * PITCH + (j * 32 + 8 * q + 4 * lh) * OS) = w;
+        }
+    // the same wavefront reads what it wrote: the LDS operations of one wavefront complete in order, and the
+    // compiler is told not to move the differently-typed accesses across each other
+    asm volatile("" ::: "memory");
+    const bool vec_ok = ((long)N * OS) % 16 == 0;
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, chunk = lane % CPR;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(patch + row * PITCH + chunk * 16);
+        const int m = m_base + row, n = n_base + chunk * EPV;
+        if (m >= M || n >= N) continue;
+        out_t *dst = Cb + (long)m * N + n;
+        if (vec_ok && n + EPV <= N) {
+            *reinterpret_cast<u32x4_t *>(dst) = v;
+        } else {
+            const out_t *e = reinterpret_cast<const out_t *>(&v);
+#pragma unroll
+            for (int k = 0; k < EPV; k++)
+                if (n + k < N) dst[k] = e[k];
+        }
+    }
+    asm volatile("" ::: "memory");  // the next band overwrites the patch
+}
+
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                             typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
-                                                            int tiles_m, int tiles_n) {
+                                                            int tiles_m, int tiles_n, int stages_per_split,
+                                                            void *__restrict__ partials) {
     extern __shared__ __align__(16) char smem[];
     typedef Compute32<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
@@ -151,12 +206,13 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     batch_offsets(g, batch, ao, bo);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
 
-    // LDS: [A stage 0][A stage 1][B buffer 0][B buffer 1]
+    // LDS: NST stages of A, then NST buffers of B
+    constexpr int NST = Cfg::NST;
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
-    constexpr int B_BASE = 2 * Cfg::A_BYTES;
+    constexpr int B_BASE = NST * Cfg::A_BYTES;
 
     // ---- DMA plan of this wavefront: PA + PB instructions, each one 1 KB of LDS ----
-    // k-dense operand: a block of 8 rows x 128 B; lane -> (row in block, slot), the slot holds chunk slot ^ row.
+    // k-dense operand: 8 rows x 128 B; lane -> (row, slot), the slot holds chunk slot ^ ((row >> 1) & 7).
     // row-dense operand: KPI consecutive k-rows of ROWS elements; lane -> (k-row, slot), the slot holds chunk
     // slot ^ swz(k); a chunk that starts past the operand's last row is fetched from the last whole chunk
     // instead (its columns are never stored).
@@ -166,85 +222,102 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     for (int p = 0; p < PA; p++) {
         const int q = p * Cfg::NW + wave;
         if constexpr (Cfg::LA == LM_K) {
-            const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
-            int row = m0 + q * 8 + drow;
+            const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
+            int row = m0 + trow;
             row = row < g.M ? row : g.M - 1;
             gpa[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
-            lda[p] = q * SWZ_BLOCK;
         } else {
             constexpr int CPR = Cfg::BM / GA::EPC, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
             const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ GA::swz(k);
             int col = m0 + c * GA::EPC;
             col = col <= g.M - GA::EPC ? col : g.M - GA::EPC;
             gpa[p] = A + (ao + (long)k * g.a_k + col) * ES;
-            lda[p] = q * 1024;
         }
+        lda[p] = q * 1024;
     }
 #pragma unroll
     for (int p = 0; p < PB; p++) {
         const int q = p * Cfg::NW + wave;
         if constexpr (Cfg::LB == LM_K) {
-            const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
-            int row = n0 + q * 8 + drow;
+            const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
+            int row = n0 + trow;
             row = row < g.N ? row : g.N - 1;
             gpb[p] = B + (bo + (long)row * g.b_n) * SB + dchunk * 16;
-            ldb[p] = B_BASE + q * SWZ_BLOCK;
         } else {
             constexpr int CPR = Cfg::BN / GB::EPC, KPI = 64 / CPR;
             const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ GB::swz(k);
             int col = n0 + c * GB::EPC;
             col = col <= g.N - GB::EPC ? col : g.N - GB::EPC;
             gpb[p] = B + (bo + (long)k * g.b_k + col) * SB;
-            ldb[p] = B_BASE + q * 1024;
         }
+        ldb[p] = B_BASE + q * 1024;
     }
     // bytes a stage advances an operand's source by: 128 bytes of k, or a stage's k-rows; a k-dense f8 buffer
     // is 128 bytes of k as well, but that is two stages
     const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : (long)GA::STAGE_K * g.a_k * ES;
     const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : (long)GB::STAGE_K * g.b_k * SB;
 
-    const int T = g.K * ES / P_ROW_BYTES;           // stages
+    // Split K: blockIdx.y owns stages [t0, t0 + T) and writes its accumulators, unrounded, to its own slab of
+    // `partials`; a second kernel adds the slabs in a fixed order and rounds once.  (stages_per_split is even
+    // when the right operand's buffers hold pairs of stages.)
+    const int T_all = g.K * ES / P_ROW_BYTES;
+    const int t0 = blockIdx.y * stages_per_split;
+    const int T = T_all - t0 < stages_per_split ? T_all - t0 : stages_per_split;  // stages of this workgroup
     const int TB = B_PAIR ? (T + 1) / 2 : T;        // right-operand buffers' worth of k
+#pragma unroll
+    for (int p = 0; p < PA; p++) gpa[p] += t0 * a_adv;
+#pragma unroll
+    for (int p = 0; p < PB; p++) gpb[p] += (B_PAIR ? t0 >> 1 : t0) * b_adv;
 
-    // element e of a stage's issue list: its PA instructions of A (stage t_a), then PBS of B (buffer tb; a paired
-    // buffer goes out in two halves, and which half is a run-time fact: the issuing stage's parity).  After
-    // unrolling, e is a constant and the chains below fold to one instruction.
-    auto dma_element = [&](int e, int t_a, bool do_a, int tb, int half, bool do_b) {
+    // What to fetch next, decided at a stage's barrier and carried to the slices that issue it.  Every stage
+    // issues a full list -- PA instructions of A, PBS of B -- so that the number of instructions in flight at any
+    // barrier is a compile-time constant (s_waitcnt takes an immediate): past the end of K the list re-fetches the
+    // last stage into a buffer nobody reads any more.
+    struct Fetch {
+        int a_src;       // stage of A (already clamped to T - 1)
+        unsigned a_dst;  // byte offset of its LDS buffer
+        int b_src;       // buffer's worth of B (clamped to TB - 1)
+        unsigned b_dst;
+        int b_half;      // paired buffers go out in two halves
+        bool b_on;       // paired buffers: the very first stage has no free buffer to refill
+    };
+    // element e of a stage's issue list; after unrolling, e is a constant and the chains fold to one instruction
+    auto dma_element = [&](int e, const Fetch &f) {
 #pragma unroll
         for (int p = 0; p < PA; p++)
-            if (e == p && do_a)
-                dma16_raw(gpa[p] + t_a * a_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(t_a & 1) * Cfg::A_BYTES + lda[p]));
+            if (e == p) dma16_raw(gpa[p] + f.a_src * a_adv, __builtin_amdgcn_readfirstlane(lds0 + f.a_dst + lda[p]));
 #pragma unroll
         for (int p = 0; p < PBS; p++)
-            if (e == PA + p && do_b) {
+            if (e == PA + p && f.b_on) {
                 const char *src = gpb[p];
                 unsigned off = ldb[p];
                 if constexpr (B_PAIR) {
-                    src = half ? gpb[p + PBS] : gpb[p];
-                    off = half ? ldb[p + PBS] : ldb[p];
+                    src = f.b_half ? gpb[p + PBS] : gpb[p];
+                    off = f.b_half ? ldb[p + PBS] : ldb[p];
                 }
-                dma16_raw(src + tb * b_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(tb & 1) * Cfg::B_BYTES + off));
+                dma16_raw(src + f.b_src * b_adv, __builtin_amdgcn_readfirstlane(lds0 + f.b_dst + off));
             }
     };
 
     // ---- fragment addresses ----
-    // k-dense: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile (four consecutive 8-row
-    // blocks); the chunk sits at slot chunk ^ (row % 8) of its row.  f8 storage: the lane's 8 k are 8 bytes,
-    // half lh of chunk s (second stage of the pair: s + 4) of the 128-byte row.
+    // k-dense: lane (lr, lh) reads chunk 2*s + lh of row lr of a 32-row tile; the chunk sits at slot
+    // chunk ^ ((row >> 1) & 7) of its row.  f8 storage: the lane's 8 k are 8 bytes, half lh of chunk s (second
+    // stage of the pair: s + 4) of the 128-byte row.
     // row-dense: lane (lr, lh) needs the (SLICE_K / 2) k that start at k = SLICE_K * s + (SLICE_K / 2) * lh, of
     // row lr.  One or two transpose reads of RPT k-rows each deliver them; for each the lane supplies the
     // address of its share of k-row (that start) + RPT * e + kq, columns of its 16-column half of the tile.
     // (k % RPT) == kq whatever s and e are, so the swizzle is a per-lane constant and the slice / half offsets
     // are immediates.
-    const int frag_row = (lr >> 3) * SWZ_BLOCK + (lr & 7) * P_ROW_BYTES;
+    constexpr int TILE_BYTES = 32 * P_ROW_BYTES;  // k-dense: 32 rows
+    const int frag_row = lr * P_ROW_BYTES;
     const int s16 = lane & 15;
     int a_frag[P_SLICES], b_frag[P_SLICES];  // k-dense: one address per slice, tiles are immediates
     int a_mn[TM], b_mn[TN];                  // row-dense: one address per tile, slices are immediates
 #pragma unroll
     for (int sl = 0; sl < P_SLICES; sl++) {
-        a_frag[sl] = (wave_m * TM) * 4 * SWZ_BLOCK + frag_row + (((2 * sl + lh) ^ (lr & 7)) << 4);
-        b_frag[sl] = B_BASE + (wave_n * TN) * 4 * SWZ_BLOCK + frag_row +
-                     (B_F8 ? ((sl ^ (lr & 7)) << 4) + lh * 8 : (((2 * sl + lh) ^ (lr & 7)) << 4));
+        a_frag[sl] = (wave_m * TM) * TILE_BYTES + frag_row + (kd_slot(lr, 2 * sl + lh) << 4);
+        b_frag[sl] = B_BASE + (wave_n * TN) * TILE_BYTES + frag_row +
+                     (B_F8 ? (kd_slot(lr, sl) << 4) + lh * 8 : (kd_slot(lr, 2 * sl + lh) << 4));
     }
     {
         const int kq = ES == 2 ? s16 >> 2 : s16 >> 1, sub = ES == 2 ? (s16 & 3) : (s16 & 1);
@@ -264,35 +337,33 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             b_mn[j] = B_BASE + (lh * (GB::SLICE_K / 2) + kq) * Cfg::BN * SB + ((c ^ GB::swz(kq)) << 4) + (bytes & 8);
         }
     }
-    // fragment of the left operand: tile i, slice SL of stage t
-    auto read_a = [&](int t, auto sl_, int i) -> u32x4_t {
+    // fragment of the left operand: tile i, slice SL, from the stage buffer at byte offset `buf`
+    auto read_a = [&](unsigned buf, auto sl_, int i) -> u32x4_t {
         constexpr int SL = decltype(sl_)::value;
-        const char *buf = smem + (t & 1) * Cfg::A_BYTES;
         if constexpr (Cfg::LA == LM_K) {
-            return lds_get(buf, a_frag[SL] + i * 4 * SWZ_BLOCK);
+            return lds_get(smem + buf, a_frag[SL] + i * TILE_BYTES);
         } else {
-            const u32x2_t lo = lds_get_tr<ES>(buf, a_mn[i] + (SL * GA::SLICE_K) * Cfg::BM * ES);
-            const u32x2_t hi = lds_get_tr<ES>(buf, a_mn[i] + (SL * GA::SLICE_K + GA::RPT) * Cfg::BM * ES);
+            const u32x2_t lo = lds_get_tr<ES>(smem + buf, a_mn[i] + (SL * GA::SLICE_K) * Cfg::BM * ES);
+            const u32x2_t hi = lds_get_tr<ES>(smem + buf, a_mn[i] + (SL * GA::SLICE_K + GA::RPT) * Cfg::BM * ES);
             return u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
     };
-    // fragment of the right operand; f8 storage comes back as 8 raw bytes in .x/.y and is widened at its use
-    auto read_b = [&](int t, auto sl_, int j) -> u32x4_t {
+    // fragment of the right operand; f8 storage comes back as 8 raw bytes in .x/.y and is widened at its use.
+    // `second`: the stage is the second of its pair (paired buffers only)
+    auto read_b = [&](unsigned buf, int second, auto sl_, int j) -> u32x4_t {
         constexpr int SL = decltype(sl_)::value;
-        const int tb = B_PAIR ? t >> 1 : t;
-        const char *buf = smem + (tb & 1) * Cfg::B_BYTES;
         if constexpr (Cfg::LB == LM_K && !B_F8) {
-            return lds_get(buf, b_frag[SL] + j * 4 * SWZ_BLOCK);
+            return lds_get(smem + buf, b_frag[SL] + j * TILE_BYTES);
         } else if constexpr (Cfg::LB == LM_K) {
-            // second stage of the pair: chunk s + 4, i.e. bit 6 of the byte offset flipped (the swizzle is an XOR)
-            const u32x2_t v = lds_get64(buf, (b_frag[SL] ^ ((t & 1) << 6)) + j * 4 * SWZ_BLOCK);
+            // chunk s + 4 instead of s: bit 6 of the byte offset flipped (the swizzle is an XOR)
+            const u32x2_t v = lds_get64(smem + buf, (b_frag[SL] ^ (second << 6)) + j * TILE_BYTES);
             return u32x4_t{v.x, v.y, 0u, 0u};
         } else if constexpr (B_F8) {
-            const u32x2_t v = lds_get_tr<1>(buf, b_mn[j] + (SL * GB::SLICE_K) * Cfg::BN * SB);
+            const u32x2_t v = lds_get_tr<1>(smem + buf, b_mn[j] + (SL * GB::SLICE_K) * Cfg::BN * SB);
             return u32x4_t{v.x, v.y, 0u, 0u};
         } else {
-            const u32x2_t lo = lds_get_tr<SB>(buf, b_mn[j] + (SL * GB::SLICE_K) * Cfg::BN * SB);
-            const u32x2_t hi = lds_get_tr<SB>(buf, b_mn[j] + (SL * GB::SLICE_K + GB::RPT) * Cfg::BN * SB);
+            const u32x2_t lo = lds_get_tr<SB>(smem + buf, b_mn[j] + (SL * GB::SLICE_K) * Cfg::BN * SB);
+            const u32x2_t hi = lds_get_tr<SB>(smem + buf, b_mn[j] + (SL * GB::SLICE_K + GB::RPT) * Cfg::BN * SB);
             return u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
     };
@@ -307,14 +378,11 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
 
     // One k-slice of work, in an explicitly pinned order: the MFMAs of slice CUR (register set CUR % 2),
-    // with the fragment reads of slice RD of stage t_rd and DMA instructions [D0, D0 + DN) of the issue list
-    // spread evenly between them.  The issue list of a stage is its PA instructions of A followed by PBS of B.
-    // Neither the reads nor the DMA then arrive in bursts: a burst of DMA instructions fills the memory
-    // pipeline's issue queue and stalls the wavefront in front of its next MFMA.
-    //   t_a / do_a   stage of A to fetch, and whether it exists
-    //   tb / half / do_b   buffer of B to fetch (a half of it when the buffers hold pairs), and whether it exists
-    auto slice_step = [&](auto cur_, auto rd_, auto d0_, auto dn_, int t_rd, int t_a, bool do_a, int tb, int half,
-                          bool do_b) {
+    // with the fragment reads of slice RD (from the buffers at rd_a / rd_b) and elements [D0, D0 + DN) of the
+    // issue list `f` spread evenly between them.  Neither the reads nor the DMA then arrive in bursts: a burst of
+    // DMA instructions fills the memory pipeline's issue queue and stalls the wavefront in front of its next MFMA.
+    auto slice_step = [&](auto cur_, auto rd_, auto d0_, auto dn_, unsigned rd_a, unsigned rd_b, int rd_second,
+                          const Fetch &f, bool do_dma) {
         constexpr int SET = decltype(cur_)::value & 1, RD = decltype(rd_)::value;
         constexpr int D0 = decltype(d0_)::value, DN = decltype(dn_)::value;
         constexpr int MF = TM * TN, RN = TM + TN;
@@ -325,8 +393,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             for (int r = 0; r < RN; r++) {
                 if (r * MF / RN != idx) continue;
                 typedef std::integral_constant<int, RD> RS;
-                if (r < TM) fa[RD & 1][r] = read_a(t_rd, RS{}, r);
-                else fb[RD & 1][r - TM] = read_b(t_rd, RS{}, r - TM);
+                if (r < TM) fa[RD & 1][r] = read_a(rd_a, RS{}, r);
+                else fb[RD & 1][r - TM] = read_b(rd_b, rd_second, RS{}, r - TM);
             }
             if (idx % TM == 0) bcur = B_F8 ? widen_f8x8(u32x2_t{fb[SET][idx / TM].x, fb[SET][idx / TM].y}) : fb[SET][idx / TM];
             // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
@@ -334,7 +402,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
 #pragma unroll
             for (int d = 0; d < DN; d++) {
                 if (d * MF / (DN > 0 ? DN : 1) != idx) continue;
-                dma_element(D0 + d, t_a, do_a, tb, half, do_b);
+                if (do_dma) dma_element(D0 + d, f);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -343,85 +411,165 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     typedef std::integral_constant<int, 1> I1;
     typedef std::integral_constant<int, 2> I2;
     typedef std::integral_constant<int, 3> I3;
-    constexpr int PH = P / 2;  // DMA instructions of a stage issued during slice 3; the rest during the next slice 0
+    constexpr int PH = P / 2;  // elements of a stage's list issued during its slice 3; the rest during the next slice 0
     typedef std::integral_constant<int, PH> DH;
     typedef std::integral_constant<int, P - PH> DR;
 
-    // prologue: stages 0 and 1 of A, buffers 0 and 1 of B (with paired buffers that is stages 0..3 of B)
-    auto issue_all = [&](int t, bool do_a, bool do_b) {
+    // ---- prologue: ring slot j gets stage j of A and buffer j of B (with paired buffers: stages 2j, 2j+1), clamped
+    // to the last one so that every group has PA + PB instructions ----
+#pragma unroll
+    for (int j = 0; j < NST; j++) {
+        const int ta = j < T ? j : T - 1, tb = j < TB ? j : TB - 1;
 #pragma unroll
         for (int p = 0; p < PA; p++)
-            if (do_a) dma16_raw(gpa[p] + t * a_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(t & 1) * Cfg::A_BYTES + lda[p]));
+            dma16_raw(gpa[p] + ta * a_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)j * Cfg::A_BYTES + lda[p]));
 #pragma unroll
         for (int p = 0; p < PB; p++)
-            if (do_b) dma16_raw(gpb[p] + t * b_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(t & 1) * Cfg::B_BYTES + ldb[p]));
-    };
-    issue_all(0, true, true);
-    if (T > 1) {
-        issue_all(1, true, TB > 1);
-        // everything of stage 0 has landed once at most stage 1's instructions are outstanding
-        if (TB > 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA + PB));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA));
-    } else {
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            dma16_raw(gpb[p] + tb * b_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)j * Cfg::B_BYTES + ldb[p]));
     }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 1) * (PA + PB)));  // group 0 has landed
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[0][i] = read_a(0, I0{}, i);
+    for (int i = 0; i < TM; i++) fa[0][i] = read_a(0u, I0{}, i);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[0][j] = read_b(0, I0{}, j);
+    for (int j = 0; j < TN; j++) fb[0][j] = read_b(0u, 0, I0{}, j);
 
-    // What stage t issues behind its barrier (second half of the list: during slice 0 of stage t+1):
-    //   A: stage t+2.
-    //   B, one buffer per stage: buffer t+2.
-    //   B, paired buffers: buffer b holds stages 2b, 2b+1 and is free once stage 2b+1 is done.  Odd t frees
-    //      buffer (t-1)/2 and issues the first half of buffer (t+3)/2 into it; the following even stage issues
-    //      the second half.  Both have two or more stages to land.
-    auto b_target = [&](int t, int &tb, int &half, bool &ok) {
-        if constexpr (B_PAIR) {
-            tb = (t + 2 + (t & 1)) >> 1;
-            half = (t & 1) ? 0 : 1;
-            ok = t >= 1 && tb < TB;
-        } else {
-            tb = t + 2;
-            half = 0;
-            ok = tb < TB;
-        }
+    // Instructions that may still be in flight at the barrier of stage t without touching what stage t+1 reads:
+    // the NST - 2 youngest issue groups.  Groups, oldest first: the NST groups of the prologue (PA + PB each), then
+    // one list per stage (P each; with paired buffers stage 0's list has no B part).  Loads return in issue order.
+    auto list_size = [](int j) { return j < NST ? PA + PB : (j == NST && B_PAIR ? PA : P); };
+    auto allowed_at = [&](int t) {
+        int n = 0;
+        for (int j = t + 2; j <= NST + t - 1; j++) n += list_size(j);
+        return n;
     };
+    auto wait_stage = [&](int t) {
+        // t < NST: the window still overlaps the prologue; one immediate per case
+        if constexpr (NST == 2) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        } else if constexpr (NST == 3) {
+            constexpr int W0 = PA + PB, W1 = B_PAIR ? PA : P;
+            if (t == 0) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(W0));
+            else if (t == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(W1));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(P));
+        } else {
+            constexpr int L0 = B_PAIR ? PA : P;
+            constexpr int W0 = 2 * (PA + PB), W1 = PA + PB + L0, W2 = L0 + P;
+            if (t == 0) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(W0));
+            else if (t == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(W1));
+            else if (t == 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(W2));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * P));
+        }
+        (void)allowed_at;
+    };
+
+    // Ring bookkeeping (byte offsets): where stage t and stage t+1 live, and which pair buffer was vacated last.
+    unsigned a_cur = 0, b_cur = 0;          // buffers of stage t
+    unsigned b_prev_pair = 0;               // paired buffers: the buffer of the pair before the current one
+    int a_slot = 0, b_slot = 0;             // ring slots of stage t
+    Fetch f{};                              // list decided at the previous stage's barrier (second half pending)
+    bool f_on = false;
 
     // The loop body is branch-free apart from the DMA predicates: past the last stage the reads fetch
     // LDS bytes nobody uses and the barrier is one too many, both harmless and cheaper than a second
     // copy of the MFMA code.
     for (int t = 0; t < T; t++) {
-        int tb, half;
-        bool ok_b;
-        // slice 0: multiply it, read slice 1, issue the second half of what stage t-1 started (stage 1 came whole)
-        b_target(t - 1, tb, half, ok_b);
-        slice_step(I0{}, I1{}, DH{}, DR{}, t, t + 1, t >= 1 && t + 1 < T, tb, half, t >= 1 && ok_b);
-        slice_step(I1{}, I2{}, I0{}, I0{}, t, 0, false, 0, 0, false);
-        slice_step(I2{}, I3{}, I0{}, I0{}, t, 0, false, 0, 0, false);
-        // everything issued so far has landed (the youngest of it a whole stage ago) and every read of stage t
-        // has returned
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        const int a_next_slot = a_slot + 1 == NST ? 0 : a_slot + 1;
+        // B moves to its next buffer every stage, or every second stage when the buffers hold pairs
+        const bool b_moves = !B_PAIR || (t & 1);
+        const int b_next_slot = b_moves ? (b_slot + 1 == NST ? 0 : b_slot + 1) : b_slot;
+        const unsigned a_next = (unsigned)a_next_slot * Cfg::A_BYTES, b_next = (unsigned)b_next_slot * Cfg::B_BYTES;
+
+        // slice 0: multiply it, read slice 1, issue the second half of the list the previous stage started
+        slice_step(I0{}, I1{}, DH{}, DR{}, a_cur, b_cur, t & 1, f, f_on);
+        slice_step(I1{}, I2{}, I0{}, I0{}, a_cur, b_cur, t & 1, f, false);
+        slice_step(I2{}, I3{}, I0{}, I0{}, a_cur, b_cur, t & 1, f, false);
+        // stage t+1 has landed and every read of stage t has returned
+        wait_stage(t);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        // slice 3: multiply it, read slice 0 of stage t+1, issue the first half of this stage's list
-        b_target(t, tb, half, ok_b);
-        slice_step(I3{}, I0{}, I0{}, DH{}, t + 1, t + 2, t + 2 < T, tb, half, ok_b);
+        // the list of this stage: A's stage t + NST into the buffer stage t just vacated; B likewise, or -- paired
+        // buffers -- a half of the pair that goes where the last finished pair was: odd t finishes pair t/2 and
+        // sends the first half of pair t/2 + NST there, the next even stage sends the second half
+        f.a_src = t + NST < T ? t + NST : T - 1;
+        f.a_dst = a_cur;
+        if constexpr (B_PAIR) {
+            const int pair = (t & 1) ? (t >> 1) + NST : ((t - 2) >> 1) + NST;
+            f.b_src = pair < TB ? pair : TB - 1;
+            f.b_dst = (t & 1) ? b_cur : b_prev_pair;
+            f.b_half = (t & 1) ? 0 : 1;
+            f.b_on = t >= 1;
+            if (t & 1) b_prev_pair = b_cur;
+        } else {
+            f.b_src = t + NST < TB ? t + NST : TB - 1;
+            f.b_dst = b_cur;
+            f.b_half = 0;
+            f.b_on = true;
+        }
+        f_on = true;
+        // slice 3: multiply it, read slice 0 of stage t+1, issue the first half of the list
+        slice_step(I3{}, I0{}, I0{}, DH{}, a_next, b_next, (t + 1) & 1, f, true);
+        a_cur = a_next;
+        b_cur = b_next;
+        a_slot = a_next_slot;
+        b_slot = b_next_slot;
     }
 
-    out_t *Cb = C + batch * (long)g.M * g.N;
-    const bool vec_ok = (g.N & 3) == 0;
+    // the clamped re-fetches of the last stages are still writing LDS: the workgroup must not end (and hand its
+    // LDS to another) before they are done
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+
+    out_t *Cb;
+    // every wavefront's DMA has landed before any wavefront reuses LDS for its epilogue
+    __syncthreads();
+    char *patch = smem + wave * (32 * (TN * 32 * 4 + 16));  // sized for 4-byte outputs, the largest
+    if (gridDim.y > 1) {
+        constexpr int ACC = Cfg::CK == CK_I8 ? OUT_I32 : OUT_F32;
+        typedef typename Out<ACC>::T part_t;
+        part_t *Pb = (part_t *)partials + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            store_band_via_lds<ACC, TN>(patch, Pb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N);
+        return;
+    }
+    Cb = C + batch * (long)g.M * g.N;
 #pragma unroll
     for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-            store_tile32<Cfg::OUT>(Cb, acc[i][j], m0 + wave_m * TM * 32 + i * 32 + lr, n0 + wave_n * TN * 32 + j * 32, lh,
-                                   g.M, g.N, vec_ok);
+        store_band_via_lds<Cfg::OUT, TN>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N);
 }
 
-template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
+// out[i] = round(partials[0][i] + partials[1][i] + ...), the slabs added in index order: bit-reproducible
+template <int OUT, class part_t>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const part_t *__restrict__ partials,
+                                                           typename Out<OUT>::T *__restrict__ out, long elems, int splits) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= elems) return;
+    if (i + 3 < elems) {
+        struct alignas(16) Quad { part_t q[4]; };
+        Quad s = *reinterpret_cast<const Quad *>(partials + i);
+        for (int k = 1; k < splits; k++) {
+            const Quad t = *reinterpret_cast<const Quad *>(partials + (long)k * elems + i);
+#pragma unroll
+            for (int e = 0; e < 4; e++) s.q[e] += t.q[e];
+        }
+        struct alignas(sizeof(typename Out<OUT>::T) * 4) OutQuad { typename Out<OUT>::T q[4]; };
+        *reinterpret_cast<OutQuad *>(out + i) = OutQuad{{Out<OUT>::cvt(s.q[0]), Out<OUT>::cvt(s.q[1]), Out<OUT>::cvt(s.q[2]),
+                                                       Out<OUT>::cvt(s.q[3])}};
+    } else {
+        for (long j = i; j < elems; j++) {
+            part_t s = partials[j];
+            for (int k = 1; k < splits; k++) s += partials[(long)k * elems + j];
+            out[j] = Out<OUT>::cvt(s);
+        }
+    }
+}
+
+// splits > 1: K is cut into that many ranges of whole stages, each range a workgroup of its own (grid.y);
+// the partial sums go through the context's workspace (splits x batches x M x N accumulators, which requires
+// batches * M * N to be a multiple of 4 for the vectorised second pass -- the caller checks)
+template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
+                                     int splits = 1) {
     static bool configured = false;  // benign race: the attribute call is idempotent
     auto kernel = mfma_pipe_kernel<Cfg>;
     if (!configured) {
@@ -432,10 +580,47 @@ template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const vo
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     const long total = g.batches * tiles_m * tiles_n;
     if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a,
-                       (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n);
+    const int T = (int)((long)g.K * Cfg::ES / P_ROW_BYTES);
+    int per = T;
+    void *partials = nullptr;
+    if (splits > 1) {
+        per = (T + splits - 1) / splits;
+        if (Cfg::B_PAIR && (per & 1)) per++;
+        splits = (T + per - 1) / per;
+    }
+    const long elems = g.batches * (long)g.M * g.N;
+    if (splits > 1) {
+        int rc = ensure_workspace(ctx, (size_t)splits * elems * 4);
+        if (rc != HODU_ROCM_OK) return rc;
+        partials = ctx->workspace.ptr;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)total, (unsigned)(splits > 1 ? splits : 1)), dim3(Cfg::NT), Cfg::LDS_BYTES,
+                       ctx->stream, (const char *)a, (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n,
+                       per, partials);
     HODU_HIP(hipGetLastError());
+    if (splits > 1) {
+        const unsigned blocks = (unsigned)((elems + 1023) / 1024);
+        if (Cfg::CK == CK_I8)
+            hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, int32_t>), dim3(blocks), dim3(256), 0, ctx->stream,
+                               (const int32_t *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits);
+        else
+            hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, float>), dim3(blocks), dim3(256), 0, ctx->stream,
+                               (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits);
+        HODU_HIP(hipGetLastError());
+    }
     return HODU_ROCM_OK;
+}
+
+// How many ways to cut K for a product that fills `tiles` workgroups of the chosen shape on `cus` compute
+// units: enough to occupy the machine, at most 8, and never fewer than 4 stages per range.  1 = do not split.
+inline int pick_splits(long tiles, long cus, int stages, long elems, int forced) {
+    if (elems % 4 != 0 || stages < 2) return 1;
+    if (forced >= 1) return forced < stages ? forced : stages;
+    if (tiles * 2 > cus) return 1;
+    long s = cus / tiles;
+    if (s > 8) s = 8;
+    if (s > stages / 4) s = stages / 4;
+    return s >= 2 ? (int)s : 1;
 }
 
 // K a whole number of 128-byte stages; the row-dense layouts exist for 8- and 16-bit types and fetch whole

@@ -167,10 +167,17 @@ const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_k
 
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
-    const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 13) || tile == 30 || tile == 31 ||
+    const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 14) || tile == 30 || tile == 31 ||
                     tile == 32 || tile == 34;
-    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..13, 30, 31, 32, 34", tile);
+    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..14, 30, 31, 32, 34", tile);
     ctx->force_tile = tile;
+    return HODU_ROCM_OK;
+}
+
+int hodu_rocm_debug_force_splitk(hodu_rocm_ctx *ctx, int splits) {
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
+    if (splits < -1 || splits == 0 || splits > 64) return fail(HODU_ROCM_INVALID_ARG, "splits %d not in -1, 1..64", splits);
+    ctx->force_splits = splits;
     return HODU_ROCM_OK;
 }
 

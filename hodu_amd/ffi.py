@@ -64,6 +64,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_last_kernel.argtypes = [vp]
     lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
     lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
+    lib.hodu_rocm_debug_force_splitk.argtypes = [vp, ci]
     lib.hodu_rocm_debug_time_product.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz, ci,
                                                  ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_debug_time_product_graph.argtypes = lib.hodu_rocm_debug_time_product.argtypes
@@ -250,6 +251,10 @@ class Context:
     def force_tile(self, tile: int):
         """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, -1 = automatic"""
         self._check(self.lib.hodu_rocm_debug_force_tile(self.handle, int(tile)))
+
+    def force_splitk(self, splits: int):
+        """testing hook: K ranges of the pipelined kernels (-1 automatic, 1 never, n forced)"""
+        self._check(self.lib.hodu_rocm_debug_force_splitk(self.handle, int(splits)))
 
     def last_kernel(self) -> str:
         return self.lib.hodu_rocm_last_kernel(self.handle).decode()

@@ -85,6 +85,10 @@ const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
  * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; -1 = automatic) so that
  * every compiled variant can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
+/* testing hook: number of K ranges the pipelined tile kernels cut a product into (each range a workgroup of its
+ * own, partial sums added in a fixed order by a second kernel): -1 = automatic (only products too small to
+ * fill the machine are cut), 1 = never, n = n ranges wherever the kernel can */
+int hodu_rocm_debug_force_splitk(hodu_rocm_ctx *ctx, int splits);
 /* measurement hook: issues the same product `iters` times back to back from C (no per-launch
  * interpreter overhead), cycling through `n_rhs` right-hand buffers so a small operand cannot sit
  * in the Infinity Cache, bracketed by HIP events on the context's stream; *elapsed_ms is the total.

@@ -162,3 +162,31 @@ def test_deep_k_accumulation(ctx):
     check_product(ctx, "dot", "bf16", V([64, 4096]), V([96, 4096]).t(), seed=21, scale=1.0)
     check_product(ctx, "dot", "f32", V([64, 4096]), V([4096, 96]), seed=22, scale=1.0)
     check_product(ctx, "dot", "bf16_f8e4m3w", V([64, 4096]), V([96, 4096]).t(), seed=23, scale=1.0, rscale=100.0)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16", "f32", "i32_i8i8", "bf16_f8e4m3w"])
+@pytest.mark.parametrize("splits", [2, 3, 8])
+def test_split_k(ctx, kind, splits):
+    """K cut into ranges, one workgroup each, partial sums added by a second kernel: same numbers as one pass"""
+    prefix = KINDS[kind][0]
+    es = {"bf16": 2, "f16": 2, "f32": 4, "i32_i8i8": 1, "bf16_f8e4m3w": 2}[kind]
+    rs = 2.0 if "f8" in kind else None
+    ctx.force_splitk(splits)
+    try:
+        for tile, name in ((10, "pipe256x256w8"), (12, "pipe128x128")):
+            ctx.force_tile(tile)
+            K = 10 * 128 // es  # ten stages: uneven ranges for 3 and 8 ways
+            check_product(ctx, "dot", kind, V([296, K]), V([200, K]).t(), seed=splits, rscale=rs,
+                          expect_kernel=f"{prefix}_{name}_KK_splitk")
+            if kind in ("bf16", "bf16_f8e4m3w"):
+                check_product(ctx, "matmul", kind, V([2, 72, K]), V([K, 80]).broadcast_to([2, K, 80]), seed=splits + 10,
+                              rscale=rs, expect_kernel=f"{prefix}_{name}_KM_splitk")
+        # automatic: a product too small for 128x128 tiles to fill the machine is cut along K
+        ctx.force_tile(-1)
+        ctx.force_splitk(-1)
+        K = 32 * 128 // es
+        check_product(ctx, "dot", kind, V([256, K]), V([384, K]).t(), seed=5, rscale=rs,
+                      expect_kernel=f"{prefix}_pipe128x128_KK_splitk")
+    finally:
+        ctx.force_tile(-1)
+        ctx.force_splitk(-1)
