@@ -1,42 +1,46 @@
-// Software-pipelined MFMA tile kernel for products whose operands are BOTH k-dense in their
-// compute type (bf16 x bf16, f16 x f16, i8 x i8, f32 x f32 with `stride_k == 1`, 16-byte aligned
-// rows, K a multiple of 128 bytes).  Same tiles, same MFMA instructions and same results as the
-// general kernel in gemm_mfma.hpp; what differs is how the K loop is fed:
+// Software-pipelined MFMA tile kernel for products whose operands are vector-loadable (k-dense, or
+// row-dense for the 8- and 16-bit types) and whose K is a multiple of 128 bytes.  Same MFMA
+// instructions and the same results as the general kernel in gemm_mfma.hpp; what differs is how
+// the K loop is fed and how the tile leaves:
 //
 //   * K advances 128 bytes per stage (64 bf16 / 128 i8 / 32 f32 = four MFMA k-slices).  Every DMA
 //     request is one whole 128-byte cache line of one row: fetching rows in 64-byte halves feeds a
 //     compute unit at 29 B/clk, whole lines at 47 B/clk (measured on the 4096 x 4096 x 14336 sweep);
-//   * two stages of LDS, written by LDS-DMA only (global_load_lds_dwordx4: no staging registers, no
-//     ds_write).  The DMA of stage t+2 is issued, into the buffer stage t just vacated, while the
-//     last k-slice of stage t multiplies, so it has the whole of stage t+1 to land;
-//   * a stage is an array of 1 KB blocks, one block = 8 rows x 128 B = exactly what one wavefront-wide
-//     DMA instruction writes, 128 bytes apart; the eight 16-byte chunks of a row are XOR-swizzled by
-//     row % 8 -- applied to the SOURCE address of the DMA -- so that an MFMA fragment read (16 lanes =
-//     16 rows, one chunk) touches all 64 banks once (lds_swizzled in gemm_mfma.hpp);
+//   * a ring of NST (2..4) stages of LDS, written by LDS-DMA only (global_load_lds_dwordx4: no staging
+//     registers, no ds_write).  Behind the barrier of stage t the DMA of stage t + NST is issued into
+//     the buffer stage t just vacated, spread between the MFMAs of the following two k-slices;
+//   * a k-dense stage is rows of 128 bytes back to back; one wavefront-wide DMA instruction writes
+//     8 rows.  The eight 16-byte chunks of a row are XOR-swizzled by (row >> 1) & 7 -- applied to the
+//     SOURCE address of the DMA -- so that an MFMA fragment read (16 lanes = 16 rows, one chunk)
+//     touches all 64 banks once without any padding;
 //   * the MFMA fragments live in one register set that is refilled one k-slice ahead of its use, each
-//     ds_read_b128 interleaved with the MFMAs of the previous slice, so that LDS and the matrix cores
-//     run side by side instead of in alternating bursts;
-//   * one bare s_barrier per stage, preceded by s_waitcnt vmcnt(0) lgkmcnt(0): at that point the only
-//     DMA in flight is the next stage's, and every fragment read of the current stage has returned.
+//     LDS read placed between the MFMAs of the previous slice in a pinned order, so that LDS and the
+//     matrix cores run side by side instead of in alternating bursts;
+//   * one bare s_barrier per stage, preceded by s_waitcnt vmcnt(n) lgkmcnt(0) with n = what the NST - 2
+//     youngest stages' DMA amounts to (loads return in issue order): stage t+1 has landed, every
+//     fragment read of stage t has returned, younger stages stay in flight;
+//   * the epilogue stages each 32-row band of a wavefront's accumulators in LDS and stores whole rows.
 //
 // Row-dense operands (stride 1 along m or n: a [K, N] row-major right operand, a transposed left
-// operand) of the 16-bit types take the same path.  A stage of such an operand is 64 k-rows of the
-// tile's ROWS contiguous elements, DMA'd as whole rows (1 KB = 1024 / (2 * ROWS) k-rows per
-// instruction) into a plain [k][ROWS] array whose 16-byte chunks are XOR-swizzled by (k % 4) << 2.
-// The MFMA fragment -- 8 consecutive k of ONE row per lane -- comes out of that k-major array
-// through two ds_read_b64_tr_b16 (LDS transpose reads: each hands a lane 4 consecutive k of its own
-// column from four rows that 16 lanes read together), so no register-level transpose and no second
-// LDS layout is needed.
+// operand) take the same path.  A stage of such an operand is the stage's k-rows of the tile's ROWS
+// contiguous elements, DMA'd as whole rows into a plain [k][ROWS] array whose 16-byte chunks are
+// XOR-swizzled by (k % 4) << 2 (16-bit) or k % 8 (8-bit).  The MFMA fragment -- 16 bytes of
+// consecutive k of ONE row per lane -- comes out of that k-major array through two LDS transpose
+// reads (ds_read_b64_tr_b16 / _tr_b8: each hands a lane 4 or 8 consecutive k of its own column from
+// the k-rows that 16 lanes read together), so no register-level transpose and no second LDS layout
+// is needed.
 //
 // f8e4m3 right operands (the fused to_dtype of a weight) are DMA'd as the bytes they are and widened
 // to bf16 between the fragment read and the MFMA (v_cvt_scalef32_pk_bf16_fp8, exact): no widened
 // copy ever exists in LDS or HBM.  k-dense f8 rows still move as whole 128-byte lines, which is 128 k
-// = two stages of the bf16 left operand, so the right operand's two buffers each hold a PAIR of
-// stages and are refilled one half per stage; row-dense f8 ([K, N] bytes) moves 64 k-rows per stage.
+// = two stages of the bf16 left operand, so the right operand's buffers each hold a PAIR of stages
+// and are refilled one half per stage; row-dense f8 ([K, N] bytes) moves 64 k-rows per stage.
 //
 // Hazards.  The barrier in stage t is reached by a wavefront only after all its reads of stage t
-// have RETURNED (lgkmcnt(0)) and its own share of stage t+1 has landed (vmcnt(0)); past it, stage t's
-// buffer is dead for everybody and stage t+1 is complete for everybody.
+// have RETURNED (lgkmcnt(0)) and its own share of stage t+1 has landed (vmcnt); past it, stage t's
+// buffer is dead for everybody and stage t+1 is complete for everybody.  Past the end of K every
+// stage still issues a full (re-fetching) list so that the in-flight count stays a constant; those
+// land in buffers nobody reads, and the workgroup waits for them before it touches LDS again or ends.
 #pragma once
 
 #include <type_traits>
