@@ -99,6 +99,13 @@ def build_cases(which):
                               (lambda m=m, k=k: bf16(normal(302, m * k))), (lambda n=n, k=k: fp8_weights(301, n * k)),
                               2.0 * m * n * k, n * k + m * k * 2 + m * n * 2,
                               "hbm" if m <= 16 else "mfma", "bf16", rotate=(m <= 16)))
+    if "f8" in which:
+        # not a BASELINE configuration: hodu's own f8e4m3 x f8e4m3 -> f8e4m3 product at 4096^3 on the native 8-bit
+        # matrix instruction, reported against the fp8 dense peak
+        n = 4096
+        cases.append(Case("f8_4096", "f8e4m3 dot 4096^3 (native fp8 MFMA), rhs a transposed view", "dot", "f8e4m3",
+                          V([n, n]), V([n, n]).t(), lambda n=n: fp8_weights(601, n * n, top=8.0),
+                          lambda n=n: fp8_weights(602, n * n, top=8.0), 2.0 * n ** 3, 3 * n * n, "mfma", "fp8"))
     if "c4" in which:
         n = 2048
         ints = lambda seed, n=n: np.random.default_rng(seed).integers(-127, 128, n * n).astype(np.int8)  # noqa: E731
@@ -126,7 +133,7 @@ def out_bytes(case):
     import helpers as H
     md = H.dot_md(case.lv, case.rv) if case.op == "dot" else H.matmul_md(case.lv, case.rv)
     n = md[0] * md[2] if case.op == "dot" else md[0]
-    return md, n * {"f32": 4, "bf16": 2, "bf16_f8e4m3w": 2, "i32_i8i8": 4}[case.name]
+    return md, n * {"f32": 4, "bf16": 2, "bf16_f8e4m3w": 2, "i32_i8i8": 4, "f8e4m3": 1}[case.name]
 
 
 def time_case(ctx, case, steps, warmup, graph=False):
@@ -221,7 +228,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="c1,c2,c3,c4,c5")
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")

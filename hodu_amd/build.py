@@ -25,6 +25,9 @@ ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the K loops are written as fully unrolled compile-time schedules; the default pragma-unroll size limit
+    # would quietly leave the largest tile rolled (accumulators indexed at run time, i.e. in scratch memory)
+    "-mllvm", "-pragma-unroll-threshold=200000",
     f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
 ]
 

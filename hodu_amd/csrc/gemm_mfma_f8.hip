@@ -1,0 +1,30 @@
+// f8e4m3 x f8e4m3 -> f8e4m3 on the 8-bit matrix instruction (gemm_mfma_pipe_f8.hpp): applicability and launch.
+#include "gemm_mfma_pipe_f8.hpp"
+namespace hodu {
+int launch_mfma_f8(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
+    using namespace mfma;
+    // both operands k-dense with every 16-byte chunk aligned, K a whole number of 128-byte stages;
+    // anything else stays with the generic kernel
+    const int la = pick_mode(a, g.a_off, g.a_m, g.a_k, g.M, g.K, 1, 16, 16, g, g.a_bs);
+    const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, 1, 16, 16, g, g.b_bs);
+    const int forced = ctx->force_tile;
+    if (la != LM_K || lb != LM_K || g.K % P_ROW_BYTES != 0 || (forced >= 0 && forced < 10)) return HODU_ROCM_UNSUPPORTED;
+    const long cus = ctx->props.multiProcessorCount;
+    auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
+    const bool big = forced >= 10 ? forced != 12 : tiles(256, 256) >= cus;
+    const int stages = (int)(g.K / P_ROW_BYTES);
+    const long elems = g.batches * (long)g.M * g.N;
+    int splits = 1;
+    if (ctx->force_splits >= 1) splits = pick_splits(1, cus, stages, elems, ctx->force_splits);
+    else if (!big) splits = pick_splits(tiles(128, 128), cus, stages, elems, -1);
+    const char *base = big ? "mfma_f8e4m3_pipe256x256_KK" : "mfma_f8e4m3_pipe128x128_KK";
+    if (splits > 1) {
+        snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_splitk%d", base, splits);
+        ctx->last_kernel = ctx->kernel_name;
+    } else {
+        ctx->last_kernel = base;
+    }
+    if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 256, 256>>(ctx, a, b, c, g, splits);
+    return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 128, 128>>(ctx, a, b, c, g, splits);
+}
+}  // namespace hodu

@@ -31,7 +31,6 @@ using mfma::Out;
 using mfma::SK_F8;
 using mfma::SK_SAME;
 
-constexpr int WAVES = 8;
 constexpr int CHUNK = 8;                 // weight vectors in flight per lane (8 KB per wavefront)
 constexpr int X_LDS_LIMIT = 144 * 1024;  // bytes of LDS the staged left operand may take
 
@@ -53,8 +52,10 @@ __device__ __forceinline__ void widen_f8x16(const u32x4_t &w, u32x4_t &lo, u32x4
 // x_pitch > 0: the left operand (M x K, a few KB) is first copied to LDS, rows x_pitch bytes apart,
 // so that the MFMA's left fragments come from LDS instead of nearly-empty global loads (for M = 1
 // only 4 of 64 lanes carry a left-operand row).  x_pitch == 0: it does not fit; read it from global.
-template <int CK, int SKB, int OUT>
-__global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *__restrict__ X,
+// NBLK blocks of 16 weight rows per workgroup, KW wavefronts splitting K for each: the staged copy of x is shared
+// by all of them, so a larger NBLK means proportionally fewer copies of x through the memory pipeline
+template <int CK, int SKB, int OUT, int NBLK, int KW>
+__global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const char *__restrict__ X,
                                                                   const char *__restrict__ W,
                                                                   typename Out<OUT>::T *__restrict__ Y, DevProduct g,
                                                                   int tiles_n, int k_per_wave, int x_pitch) {
@@ -65,12 +66,14 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *_
     constexpr int SB = SKB == SK_F8 ? 1 : ES;           // bytes per stored weight element
     constexpr int EPL = 16 / SB;                        // weight elements per lane per load
     extern __shared__ __align__(16) char xs[];
-    __shared__ acc_t red[WAVES][64];
+    constexpr int NT = NBLK * KW * 64;
+    __shared__ acc_t red[NBLK * KW][64];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
     const long batch = blockIdx.x / tiles_n;
-    const int n0 = (int)(blockIdx.x % tiles_n) * 16;
+    const int blk = wave / KW, kw = wave % KW;
+    const int n0 = ((int)(blockIdx.x % tiles_n) * NBLK + blk) * 16;
     long ao, bo;
     batch_offsets(g, batch, ao, bo);
 
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *_
     const bool has_x = lr < g.M;
     const char *xrow = X + (ao + (long)(has_x ? lr : 0) * g.a_m) * ES;
 
-    const int kbeg = wave * k_per_wave;
+    const int kbeg = kw * k_per_wave;
     int kend = kbeg + k_per_wave;
     kend = kend < g.K ? kend : g.K;
 
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *_
     }
     if (x_pitch > 0) {
         const int vec_per_row = g.K * ES / 16;
-        for (int v = tid; v < g.M * vec_per_row; v += WAVES * 64) {
+        for (int v = tid; v < g.M * vec_per_row; v += NT) {
             const int row = v / vec_per_row, col = v - row * vec_per_row;
             *reinterpret_cast<u32x4_t *>(xs + row * x_pitch + col * 16) = ldg16(X + (ao + (long)row * g.a_m) * ES + col * 16);
         }
@@ -138,15 +141,15 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *_
     // lane holds y[m = 4*lg + e][n = n0 + lr] for e = 0..3 over this wavefront's k range
     red[wave][lane] = acc;
     __syncthreads();
-    if (tid < 64) {
-        acc_t s = red[0][tid];
+    if (tid < 64 * NBLK) {  // wavefront b adds up row block b; (lr, lg) are the same in every wavefront
+        acc_t s = red[wave * KW][lane];
 #pragma unroll
-        for (int w = 1; w < WAVES; w++) {
-            const acc_t t = red[w][tid];
+        for (int w = 1; w < KW; w++) {
+            const acc_t t = red[wave * KW + w][lane];
             s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
         }
         out_t *Yb = Y + batch * (long)g.M * g.N;
-        const int col = n0 + lr;
+        const int col = ((int)(blockIdx.x % tiles_n) * NBLK + wave) * 16 + lr;
         if (col < g.N) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -155,6 +158,32 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kdense_kernel(const char *_
             }
         }
     }
+}
+
+template <int CK, int SKB, int OUT, int NBLK, int KW>
+int launch_shape(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g) {
+    constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB;
+    const int tiles_n = (g.N + 16 * NBLK - 1) / (16 * NBLK);
+    const long blocks = g.batches * tiles_n;
+    if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
+    const int step = 4 * EPL;  // k covered by one wavefront-wide load
+    const int k_per_wave = ((g.K + KW - 1) / KW + step - 1) / step * step;
+    // rows of the staged left operand are padded by 16 bytes so that the 16 row slots of a fragment
+    // read hit different LDS banks
+    const long pitch = (long)g.K * ES + 16;
+    const int x_pitch = (g.M * pitch <= X_LDS_LIMIT) ? (int)pitch : 0;
+    const size_t lds = x_pitch > 0 ? (size_t)g.M * x_pitch : 0;
+    auto kernel = skinny_kdense_kernel<CK, SKB, OUT, NBLK, KW>;
+    static bool configured = false;  // benign race: the attribute call is idempotent
+    if (!configured) {
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     X_LDS_LIMIT));
+        configured = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NBLK * KW * 64), lds, ctx->stream, (const char *)x,
+                       (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave, x_pitch);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
 }
 
 template <int CK, int SKB, int OUT>
@@ -170,28 +199,16 @@ int run_kdense(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const 
     for (int d = 0; d < g.nb; d++)
         if (!al(g.a_bs[d], ES) || !al(g.b_bs[d], SB)) return HODU_ROCM_UNSUPPORTED;
 
-    const int tiles_n = (g.N + 15) / 16;
-    const long blocks = g.batches * tiles_n;
-    if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
-    const int step = 4 * EPL;  // k covered by one wavefront-wide load
-    int k_per_wave = ((g.K + WAVES - 1) / WAVES + step - 1) / step * step;
-    // rows of the staged left operand are padded by 16 bytes so that the 16 row slots of a fragment
-    // read hit different LDS banks
-    const long pitch = (long)g.K * ES + 16;
-    const int x_pitch = (g.M * pitch <= X_LDS_LIMIT) ? (int)pitch : 0;
-    const size_t lds = x_pitch > 0 ? (size_t)g.M * x_pitch : 0;
-    auto kernel = skinny_kdense_kernel<CK, SKB, OUT>;
-    static bool configured = false;  // benign race: the attribute call is idempotent
-    if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     X_LDS_LIMIT));
-        configured = true;
-    }
+    // workgroup shape: (row blocks, wavefronts per block).  Every workgroup stages its own copy of x, so when x is
+    // as large as the weights a workgroup streams (M near 16), fewer and fatter workgroups move fewer bytes.
+    int shape = g.M > 8 && g.N >= 32 * 128 ? 1 : 0;  // measured at M = 16, N = K = 4096 (f8 weights): 11.6, 11.1, 14.5 us
+    if (ctx->force_tile == 35) shape = 0;
+    if (ctx->force_tile == 36) shape = 1;
+    if (ctx->force_tile == 37) shape = 2;
     ctx->last_kernel = name;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WAVES * 64), lds, ctx->stream, (const char *)x,
-                       (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave, x_pitch);
-    HODU_HIP(hipGetLastError());
-    return HODU_ROCM_OK;
+    if (shape == 1) return launch_shape<CK, SKB, OUT, 2, 8>(ctx, x, w, y, g);
+    if (shape == 2) return launch_shape<CK, SKB, OUT, 4, 4>(ctx, x, w, y, g);
+    return launch_shape<CK, SKB, OUT, 1, 8>(ctx, x, w, y, g);
 }
 
 }  // namespace

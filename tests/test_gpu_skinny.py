@@ -54,6 +54,20 @@ def test_batched_rows_fold_or_stay_batched(no_gemv, kind):
                   rscale=rs, expect_kernel=KINDS[kind])
 
 
+@pytest.mark.parametrize("kind", list(KINDS))
+@pytest.mark.parametrize("shape", [35, 36, 37])
+def test_workgroup_shapes(ctx, kind, shape):
+    """1, 2 or 4 blocks of 16 weight rows per workgroup: N ragged against all of them, M from 5 to 16"""
+    rs = 2.0 if "f8" in kind else None
+    ctx.force_tile(shape)
+    try:
+        for m in (5, 16):
+            check_product(ctx, "dot", kind, V([m, 1040]), V([203, 1040]).t(), seed=m, rscale=rs, expect_kernel=KINDS[kind])
+        check_product(ctx, "matmul", kind, V([3, 9, 256]), V([3, 40, 256]).t(), seed=2, rscale=rs, expect_kernel=KINDS[kind])
+    finally:
+        ctx.force_tile(-1)
+
+
 def test_not_applicable_layouts_fall_through(ctx):
     # weight with n dense ([K, N] row-major): not this kernel's layout; still correct via the tile kernel
     check_product(ctx, "dot", "bf16_f8e4m3w", V([1, 256]), V([256, 64]), seed=4, rscale=2.0, expect_kernel="mfma_")
