@@ -27,6 +27,7 @@ struct hodu_rocm_ctx {
     hipStream_t stream = nullptr;
     hipDeviceProp_t props{};
     hodu::Workspace workspace;  // split-K partial sums; grown on demand, owned by the context
+    int *arrival = nullptr;     // kArrivalSlots zeroed counters for kernels whose last workgroup finishes a reduction
     const char *last_kernel = "";
     int force_tile = -1;    // testing hook: pins the MFMA tile size
     int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
@@ -52,6 +53,9 @@ int fail(int code, const char *fmt, ...);
 
 // grows ctx->workspace to at least `bytes`
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes);
+// allocates (once) and zeroes ctx->arrival; kernels that use a counter leave it at zero again
+constexpr int kArrivalSlots = 4096;
+int ensure_arrival(hodu_rocm_ctx *ctx);
 
 inline size_t dtype_size(int dt) {
     static const size_t sz[15] = {1, 1, 1, 2, 2, 4, 8, 1, 2, 4, 8, 1, 2, 4, 8};

@@ -40,6 +40,13 @@ int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
     return HODU_ROCM_OK;
 }
 
+int ensure_arrival(hodu_rocm_ctx *ctx) {
+    if (ctx->arrival) return HODU_ROCM_OK;
+    HODU_HIP(hipMalloc((void **)&ctx->arrival, kArrivalSlots * sizeof(int)));
+    HODU_HIP(hipMemsetAsync(ctx->arrival, 0, kArrivalSlots * sizeof(int), ctx->stream));
+    return HODU_ROCM_OK;
+}
+
 }  // namespace hodu
 
 using namespace hodu;
@@ -95,6 +102,7 @@ int hodu_rocm_ctx_destroy(hodu_rocm_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->workspace.ptr) (void)hipFree(ctx->workspace.ptr);
+    if (ctx->arrival) (void)hipFree(ctx->arrival);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return HODU_ROCM_OK;
@@ -168,8 +176,8 @@ const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_k
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
     const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 14) || tile == 30 || tile == 31 ||
-                    tile == 32 || tile == 34 || (tile >= 35 && tile <= 37);
-    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..14, 30, 31, 32, 34", tile);
+                    tile == 32 || tile == 34 || (tile >= 35 && tile <= 38);
+    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..14, 30, 31, 32, 34..38", tile);
     ctx->force_tile = tile;
     return HODU_ROCM_OK;
 }

@@ -87,7 +87,22 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
     int kend = kbeg + k_per_wave;
     kend = kend < g.K ? kend : g.K;
 
-    // the first chunk of weight loads goes out before anything else
+    // Loads return in issue order.  The copy of x into LDS therefore starts FIRST: its loads (cache hits) are all
+    // in flight together, the first chunk of weight loads (HBM) goes out right behind them, and the copy
+    // finishes while the weights are still on their way.  (Issued after the weights, every load of the copy
+    // loop waited for all of them, and the loop made one cache round trip per iteration.)
+    constexpr int XB = 16;  // vectors of x a thread keeps in flight
+    const int vec_per_row = g.K * ES / 16, x_vecs = x_pitch > 0 ? g.M * vec_per_row : 0;
+    u32x4_t xr[XB];
+#pragma unroll
+    for (int i = 0; i < XB; i++) {
+        const int v = tid + i * NT;
+        xr[i] = mfma::zero4();
+        if (v < x_vecs) {
+            const int row = v / vec_per_row, col = v - row * vec_per_row;
+            xr[i] = ldg16(X + (ao + (long)row * g.a_m) * ES + col * 16);
+        }
+    }
     u32x4_t wv[CHUNK];
 #pragma unroll
     for (int u = 0; u < CHUNK; u++) {
@@ -95,8 +110,15 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
         wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
     }
     if (x_pitch > 0) {
-        const int vec_per_row = g.K * ES / 16;
-        for (int v = tid; v < g.M * vec_per_row; v += NT) {
+#pragma unroll
+        for (int i = 0; i < XB; i++) {
+            const int v = tid + i * NT;
+            if (v < x_vecs) {
+                const int row = v / vec_per_row, col = v - row * vec_per_row;
+                *reinterpret_cast<u32x4_t *>(xs + row * x_pitch + col * 16) = xr[i];
+            }
+        }
+        for (int v = tid + XB * NT; v < x_vecs; v += NT) {  // a left operand larger than XB vectors per thread
             const int row = v / vec_per_row, col = v - row * vec_per_row;
             *reinterpret_cast<u32x4_t *>(xs + row * x_pitch + col * 16) = ldg16(X + (ao + (long)row * g.a_m) * ES + col * 16);
         }
@@ -160,6 +182,208 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
     }
 }
 
+// ---- the same product cut along K across workgroups -------------------------------------------------
+// For M near 16 the left operand (M x K) is twice the bytes of the weight rows one workgroup streams, and in the
+// kernel above every workgroup stages all of it: measured on M = 16, N = K = 4096 (f8 weights), 4.1 of 11.4 us.
+// Here a workgroup takes 128 weight rows (8 wavefronts x 16) and ONE slice of K, stages only that slice of x (a
+// few KB; x crosses the memory pipeline N/128 times in total instead of N/16 times), and there are still as many
+// workgroups as compute units.  Each writes its 16 x 128 partial sums (laid out [slice][n][16]: a lane's four
+// values are one 16-byte store) and bumps its column block's arrival counter; the workgroup that arrives last
+// adds the slices in slice order -- so the result does not depend on who was last --, rounds once, stores, and
+// zeroes the counter for the next launch.
+// 16-byte accesses at device scope (sc1): the store goes through to memory, the load does not take a line that this
+// compute unit's cache complex may hold from an earlier launch
+template <typename V>
+__device__ __forceinline__ void st16_device(V *p, const V &v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+template <typename V>
+__device__ __forceinline__ V ld16_device(const V *p) {
+    V v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(p) : "memory");
+    return v;
+}
+
+constexpr int SK_ROWS = 128;  // weight rows per workgroup
+constexpr int SK_XVEC = 8;    // 16-byte vectors of x per thread: 512 threads x 8 x 16 B = 64 KB covers M = 16 x 2048 k of bf16
+constexpr int SK_XBYTES = SK_XVEC * 512 * 16;
+
+template <int CK, int SKB, int OUT>
+__global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restrict__ X, const char *__restrict__ W,
+                                                           typename Out<OUT>::T *__restrict__ Y,
+                                                           typename Compute<CK>::acc_t *__restrict__ partials,
+                                                           int *__restrict__ arrival, DevProduct g, int n_blocks,
+                                                           int slices, int k_per_slice, int x_pitch) {
+    typedef Compute<CK> Cmp;
+    typedef typename Cmp::acc_t acc_t;
+    typedef decltype(acc_t{}.x) part_t;
+    constexpr int ES = Cmp::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB;
+    extern __shared__ __align__(16) char xs[];
+    __shared__ int last_flag;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int nb = blockIdx.x % n_blocks, ks = blockIdx.x / n_blocks;
+    const int kbeg = ks * k_per_slice;
+    int kend = kbeg + k_per_slice;
+    kend = kend < g.K ? kend : g.K;
+
+    int n = nb * SK_ROWS + wave * 16 + lr;
+    const bool n_ok = n < g.N;
+    n = n_ok ? n : g.N - 1;
+    const char *wrow = W + (g.b_off + (long)n * g.b_n) * SB;
+
+    // loads return in issue order: the slice of x (cache hits) first, the weights (HBM) right behind
+    constexpr int XB = SK_XVEC;
+    const int vec_per_row = (kend - kbeg) * ES / 16, x_vecs = g.M * vec_per_row;
+    u32x4_t xr[XB];
+#pragma unroll
+    for (int i = 0; i < XB; i++) {
+        const int v = tid + i * 512;
+        xr[i] = mfma::zero4();
+        if (v < x_vecs) {
+            const int row = v / vec_per_row, col = v - row * vec_per_row;
+            xr[i] = ldg16(X + (g.a_off + (long)row * g.a_m + kbeg) * ES + col * 16);
+        }
+    }
+    u32x4_t wv[CHUNK];
+#pragma unroll
+    for (int u = 0; u < CHUNK; u++) {
+        const int k = kbeg + (u * 4 + lg) * EPL;
+        wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+    }
+#pragma unroll
+    for (int i = 0; i < XB; i++) {
+        const int v = tid + i * 512;
+        if (v < x_vecs) {
+            const int row = v / vec_per_row, col = v - row * vec_per_row;
+            *reinterpret_cast<u32x4_t *>(xs + row * x_pitch + col * 16) = xr[i];
+        }
+    }
+    __syncthreads();
+    const char *xl = xs + lr * x_pitch;
+    const bool has_x = lr < g.M;
+
+    acc_t acc = acc_t{0, 0, 0, 0};
+    for (int kb = kbeg; kb < kend; kb += CHUNK * 4 * EPL) {
+        if (kb != kbeg) {
+#pragma unroll
+            for (int u = 0; u < CHUNK; u++) {
+                const int k = kb + (u * 4 + lg) * EPL;
+                wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < CHUNK; u++) {
+            const int k = kb + (u * 4 + lg) * EPL;
+            const bool ok = k < kend && has_x;
+            u32x4_t xa = mfma::zero4(), xb = mfma::zero4();
+            if (ok) {
+                xa = *reinterpret_cast<const u32x4_t *>(xl + (k - kbeg) * ES);
+                if (SKB == SK_F8) xb = *reinterpret_cast<const u32x4_t *>(xl + (k - kbeg + 8) * ES);
+            }
+            if (SKB == SK_F8) {
+                u32x4_t lo, hi;
+                widen_f8x16(wv[u], lo, hi);
+                Cmp::mma(xa, lo, acc);
+                Cmp::mma(xb, hi, acc);
+            } else {
+                Cmp::mma(xa, wv[u], acc);
+            }
+        }
+    }
+    // lane holds y[m = 4*lg + e][n] for e = 0..3: one 16-byte store into [slice][n][16]
+    // written THROUGH the cache at device scope, and waited for: the sums are then visible to every compute unit
+    // without a cache write-back (which costs 7 us per launch here when the counter update carries one)
+    if (n_ok) st16_device(&partials[((long)ks * g.N + n) * 4 + lg], acc);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // every thread's sums have landed before the barrier; thread 0 then counts this workgroup in.  Whoever sees
+    // slices - 1 in the counter is last.
+    __syncthreads();
+    if (tid == 0) {
+        const int before = __hip_atomic_fetch_add(&arrival[nb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = before == slices - 1;
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    // 128 columns x 4 quads of m: thread -> (column, quad); the other workgroups' sums are read at device scope
+    // (a plain load could be served from a line this compute unit cached during an earlier launch)
+    const int col = nb * SK_ROWS + (tid >> 2), quad = tid & 3;
+    if (col < g.N) {
+        acc_t s = acc_t{0, 0, 0, 0};
+        for (int k0 = 0; k0 < slices; k0 += 8) {  // eight loads in flight
+            acc_t v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                v[j] = acc_t{0, 0, 0, 0};
+                if (k0 + j < slices) v[j] = ld16_device(&partials[((long)(k0 + j) * g.N + col) * 4 + quad]);
+            }
+            // the loaded registers are operands of the wait, so that no use of them can be scheduled ahead of it
+            asm volatile("s_waitcnt vmcnt(0)"
+                         : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+                         :
+                         : "memory");
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (k0 + j < slices) s += v[j];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int m = quad * 4 + e;
+            if (m < g.M) Y[(long)m * g.N + col] = Out<OUT>::cvt(s[e]);
+        }
+    }
+    if (tid == 0) __hip_atomic_store(&arrival[nb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// applicable when one product (no batch) is wide and deep enough to be cut; returns UNSUPPORTED otherwise
+template <int CK, int SKB, int OUT>
+int launch_splitk(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g) {
+    typedef typename Compute<CK>::acc_t acc_t;
+    constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB, STEP = CHUNK * 4 * EPL;
+    if (g.batches != 1 || g.M <= 4 || g.N < 8 * SK_ROWS || g.K < 4 * STEP) return HODU_ROCM_UNSUPPORTED;
+    const int n_blocks = (g.N + SK_ROWS - 1) / SK_ROWS;
+    if (n_blocks > kArrivalSlots) return HODU_ROCM_UNSUPPORTED;
+    // Measured against the one-pass kernel (f8 and bf16 weights, M = 5..16): the arrival counter and the last
+    // workgroup's second look at the sums cost about 2 us, which pays off once the weights take 16 MB and x is
+    // half as large as a workgroup's share of them, or 32 MB whatever M is, or when N is too small to give the
+    // one-pass kernel a workgroup per compute unit.
+    const long cus = ctx->props.multiProcessorCount;
+    const long w_bytes = (long)g.N * g.K * SB;
+    const bool pays = w_bytes >= (32L << 20) || (w_bytes >= (16L << 20) && g.M >= 8) ||
+                      (g.N / 16 < cus / 2 && g.K >= 4096 && g.M >= 12);
+    if (!pays && ctx->force_tile != 38) return HODU_ROCM_UNSUPPORTED;
+    // as many slices as fill the machine, each a whole number of passes (STEP k) of a wavefront and small enough
+    // that the slice of x fits the staging registers of one workgroup
+    const int passes = (g.K + STEP - 1) / STEP;
+    int slices = (int)((cus + n_blocks - 1) / n_blocks);
+    slices = slices < passes ? slices : passes;
+    int pass_per_slice = (passes + slices - 1) / slices;
+    const int fit = SK_XBYTES / (g.M * ES) / STEP;
+    if (fit < 1) return HODU_ROCM_UNSUPPORTED;
+    pass_per_slice = pass_per_slice < fit ? pass_per_slice : fit;
+    const int k_per_slice = pass_per_slice * STEP;
+    slices = (g.K + k_per_slice - 1) / k_per_slice;
+    if (slices < 2 || slices > 64) return HODU_ROCM_UNSUPPORTED;
+    const int x_pitch = k_per_slice * ES + 16;
+    const size_t lds = (size_t)g.M * x_pitch;
+    int rc = ensure_workspace(ctx, (size_t)slices * g.N * 16 * sizeof(float));
+    if (rc == HODU_ROCM_OK) rc = ensure_arrival(ctx);
+    if (rc != HODU_ROCM_OK) return rc;
+    auto kernel = skinny_splitk_kernel<CK, SKB, OUT>;
+    static bool configured = false;  // benign race: the attribute call is idempotent
+    if (!configured) {
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SK_XBYTES + 16 * 16));
+        configured = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(n_blocks * slices)), dim3(512), lds, ctx->stream, (const char *)x, (const char *)w,
+                       (typename Out<OUT>::T *)y, (acc_t *)ctx->workspace.ptr, ctx->arrival, g, n_blocks, slices, k_per_slice,
+                       x_pitch);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
 template <int CK, int SKB, int OUT, int NBLK, int KW>
 int launch_shape(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g) {
     constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB;
@@ -206,6 +430,14 @@ int run_kdense(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const 
     if (ctx->force_tile == 36) shape = 1;
     if (ctx->force_tile == 37) shape = 2;
     ctx->last_kernel = name;
+    if (ctx->force_tile < 35 || ctx->force_tile > 37) {  // the hook values 35..37 pin the one-pass kernel's shape, 38 this one
+        const int rc = launch_splitk<CK, SKB, OUT>(ctx, x, w, y, g);
+        if (rc != HODU_ROCM_UNSUPPORTED) {
+            snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_splitk", name);
+            ctx->last_kernel = ctx->kernel_name;
+            return rc;
+        }
+    }
     if (shape == 1) return launch_shape<CK, SKB, OUT, 2, 8>(ctx, x, w, y, g);
     if (shape == 2) return launch_shape<CK, SKB, OUT, 4, 4>(ctx, x, w, y, g);
     return launch_shape<CK, SKB, OUT, 1, 8>(ctx, x, w, y, g);

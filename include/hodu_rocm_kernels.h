@@ -82,8 +82,10 @@ int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
 /* testing hook: pin the MFMA tile variant (0 = 256x256 with 8 wavefronts, 1 = 256x256 with 4,
  * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
- * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; -1 = automatic) so that
- * every compiled variant can be exercised at small sizes */
+ * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; 14 = the pipelined 256x128 tile;
+ * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
+ * variant that cuts K across workgroups wherever it applies; -1 = automatic) so that every compiled variant
+ * can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
 /* testing hook: number of K ranges the pipelined tile kernels cut a product into (each range a workgroup of its
  * own, partial sums added in a fixed order by a second kernel): -1 = automatic (only products too small to

@@ -74,7 +74,7 @@ def test_config3_fp8_weight_linear(ctx, m, top):
     x = H.f32_to_bf16_rne(H.rng(302).standard_normal(m * k).astype(np.float32))
     lv, wt = V([m, k]), V([n, k]).t()  # linear idiom: W stored [N, K], passed transposed
     got = run_product(ctx, "dot", "bf16_f8e4m3w", x, w, H.dot_md(lv, wt)).reshape(m, n)
-    want = "gemv_bf16_f8w" if m <= 4 else "skinny_bf16_f8w" if m <= 16 else "mfma_bf16_f8w"
+    want = "gemv_bf16_f8w" if m <= 4 else "skinny_bf16_f8w_splitk" if m <= 16 else "mfma_bf16_f8w"
     assert ctx.last_kernel().startswith(want), ctx.last_kernel()
     step = max(1, m // 24)
     rows = lv.slice(0, 0, m, step)

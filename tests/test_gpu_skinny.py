@@ -68,6 +68,29 @@ def test_workgroup_shapes(ctx, kind, shape):
         ctx.force_tile(-1)
 
 
+@pytest.mark.parametrize("kind", list(KINDS))
+@pytest.mark.parametrize("m", [5, 16])
+def test_split_k_across_workgroups(ctx, kind, m):
+    """wide and deep products with 5..16 rows: 128 weight rows and one slice of K per workgroup, the last workgroup
+    of a column block to arrive adds the slices; N ragged against 128, K ragged against the slice; run twice in a
+    row (the arrival counters must be back at zero) and compared bit for bit"""
+    rs = 2.0 if "f8" in kind else None
+    ctx.force_tile(38)  # the automatic choice keeps products this small on the one-pass kernel
+    try:
+        for _ in range(2):
+            check_product(ctx, "dot", kind, V([m, 2064]), V([1100, 2064]).t(), seed=m, rscale=rs,
+                          expect_kernel=KINDS[kind] + "_splitk")
+        # row-sliced operands at aligned offsets
+        check_product(ctx, "dot", kind, V([m, 4096]).slice(1, 1024, 3072),
+                      V([1030, 4096], offset=64).slice(1, 512, 2560).t(), seed=20 + m, rscale=rs,
+                      expect_kernel=KINDS[kind] + "_splitk")
+        # deep K: more slices than the last workgroup adds in one round of loads
+        check_product(ctx, "dot", kind, V([m, 4224]), V([1030, 4224]).t(), seed=40 + m, rscale=rs,
+                      expect_kernel=KINDS[kind] + "_splitk")
+    finally:
+        ctx.force_tile(-1)
+
+
 def test_not_applicable_layouts_fall_through(ctx):
     # weight with n dense ([K, N] row-major): not this kernel's layout; still correct via the tile kernel
     check_product(ctx, "dot", "bf16_f8e4m3w", V([1, 256]), V([256, 64]), seed=4, rscale=2.0, expect_kernel="mfma_")
