@@ -100,6 +100,14 @@ def build_cases(which):
                               (lambda m=m, k=k: bf16(normal(302, m * k))), (lambda n=n, k=k: fp8_weights(301, n * k)),
                               2.0 * m * n * k, n * k + m * k * 2 + m * n * 2,
                               "hbm" if m <= 16 else "mfma", "bf16", rotate=(m <= 16)))
+    if "c3" in which:
+        # not a BASELINE configuration: the same M = 1 product against the 14336 x 4096 weight of config 5, where the
+        # launch and ramp-up that dominate a 2 us transfer are a smaller share
+        n, k = 14336, 4096
+        cases.append(Case("gemv_14336x4096", "bf16[1,4096] x f8e4m3[14336,4096]^T-view (fused to_dtype; not a BASELINE config)",
+                          "dot", "bf16_f8e4m3w", V([1, k]), V([n, k]).t(),
+                          (lambda k=k: bf16(normal(302, k))), (lambda n=n, k=k: fp8_weights(303, n * k)),
+                          2.0 * n * k, n * k + k * 2 + n * 2, "hbm", "bf16", rotate=True))
     if "f8" in which:
         # not a BASELINE configuration: hodu's own f8e4m3 x f8e4m3 -> f8e4m3 product at 4096^3 on the native 8-bit
         # matrix instruction, reported against the fp8 dense peak
@@ -263,7 +271,7 @@ def main():
         ctx.close()
         return
     if args.only:
-        case = next(c for c in build_cases({args.only.split("_")[0]}) if c.key == args.only)
+        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8"}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
         ctx.close()
         return
