@@ -70,10 +70,17 @@ def fp8_weights(seed, n, top=448.0):
 class Case:
     """one timed launch shape"""
 
-    def __init__(self, key, label, op, name, lv, rv, make_a, make_b, flops, alg_bytes, bound, peak_key, rotate=False):
+    def __init__(self, key, label, op, name, lv, rv, make_a, make_b, flops, alg_bytes, bound, peak_key, rotate=False,
+                 fused=()):
         self.key, self.label, self.op, self.name = key, label, op, name
         self.lv, self.rv, self.make_a, self.make_b = lv, rv, make_a, make_b
         self.flops, self.alg_bytes, self.bound, self.peak_key, self.rotate = flops, alg_bytes, bound, peak_key, rotate
+        self.fused = tuple(fused)  # element-wise steps fused into the store: "bias", "scale", "relu"
+
+    def with_steps(self, key, label, fused):
+        """the same launch with the caller's next element-wise kernels fused in (not a BASELINE configuration)"""
+        return Case(key, label, self.op, self.name, self.lv, self.rv, self.make_a, self.make_b, self.flops,
+                    self.alg_bytes, self.bound, self.peak_key, self.rotate, fused)
 
 
 def build_cases(which):
@@ -135,6 +142,13 @@ def build_cases(which):
                               "matmul", name, V([b, s, f]), V([d, f]).t().broadcast_to([b, f, d]),
                               lambda b=b, s=s, f=f: bf16(normal(504, b * s * f, 0.3)), mk_w(503),
                               2.0 * b * s * d * f, b * s * f * 2 + wbytes + b * s * d * 2, "mfma", "bf16"))
+    if "fused" in which:
+        base = {c.key: c for c in build_cases({"c2", "c3", "c5"})}
+        cases.append(base["c3_m1"].with_steps("c3_m1_linear", "C3 M=1 as a Linear layer: + bias fused", ("bias",)))
+        cases.append(base["c3_m16"].with_steps("c3_m16_linear", "C3 M=16 as a Linear layer: + bias fused", ("bias",)))
+        cases.append(base["c2"].with_steps("c2_scaled", "C2 as attention scores: * scalar fused", ("scale",)))
+        cases.append(base["c5_up_bf16"].with_steps("c5_up_bf16_bias_relu", "C5 up as Linear + ReLU: + bias, relu fused",
+                                                   ("bias", "relu")))
     return cases
 
 
@@ -160,15 +174,28 @@ def time_case(ctx, case, steps, warmup, graph=False):
         ctx.lib.hodu_rocm_memcpy_d2d(ctx.handle, extra.ptr, ws[0].ptr, w_host.nbytes)
         ws.append(extra)
     out = ctx.alloc(obytes)
+    from hodu_amd import ffi
+    fused_steps, bias = [], None
+    for what in case.fused:
+        if what == "bias":
+            bias = ctx.upload(bf16(normal(700, case.rv.shape[-1], 0.1)))
+            fused_steps.append(ffi.add_row(bias))
+        elif what == "scale":
+            fused_steps.append(ffi.mul_scalar(bf16(np.array([0.125], dtype=np.float32))))
+        else:
+            fused_steps.append(ffi.relu())
     ctx.sync()
     for i in range(warmup):
-        ctx.product(case.op, case.name, a, ws[i % copies], out, md)
+        if fused_steps:
+            ctx.product_ex(case.op, case.name, a, ws[i % copies], out, md, fused_steps)
+        else:
+            ctx.product(case.op, case.name, a, ws[i % copies], out, md)
     ctx.sync()
     kernel = ctx.last_kernel()
     # the K timed launches are issued back to back from C (hodu_rocm_debug_time_product) so that a
     # 3 us GEMV is not hidden behind the interpreter's per-call cost; HIP events on the same stream
-    ms = ctx.time_product(case.op, case.name, a, ws, out, md, steps, graph=graph)
-    for buf in [a, out] + ws:
+    ms = ctx.time_product(case.op, case.name, a, ws, out, md, steps, graph=graph, steps=fused_steps)
+    for buf in [a, out] + ws + ([bias] if bias else []):
         buf.free()
     per_launch_s = ms / 1e3 / steps
     tflops = case.flops / per_launch_s / 1e12
@@ -237,7 +264,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8")
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,fused")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
@@ -271,7 +298,7 @@ def main():
         ctx.close()
         return
     if args.only:
-        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8"}) if c.key == args.only)
+        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "fused"}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
         ctx.close()
         return

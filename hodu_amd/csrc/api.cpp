@@ -1,6 +1,8 @@
 // extern "C" compute entry points: metadata parsing, kernel-family selection, launch.
 #include "common.hpp"
 
+#include <cstring>
+
 namespace hodu {
 namespace {
 
@@ -32,13 +34,15 @@ size_t out_elem_size(int kind, int dtype) {
 
 // Splits a parsed product into launches: the innermost kKernelBatchDims merged batch dims go to
 // the kernel, any further outer dims are walked here.
-int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p) {
+int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p,
+                const DevEpilogue &epi) {
     HODU_HIP(hipSetDevice(ctx->device));
     if (p.M > 0x7FFFFFFFL || p.N > 0x7FFFFFFFL || p.K > 0x7FFFFFFFL)
         return fail(HODU_ROCM_UNSUPPORTED, "matrix extent exceeds 2^31-1");
     if (p.batches == 0 || p.M == 0 || p.N == 0) return HODU_ROCM_OK;  // empty output: nothing to write
 
     DevProduct g{};
+    g.epi = epi;
     g.M = (int)p.M; g.N = (int)p.N; g.K = (int)p.K;
     g.a_m = p.a_m; g.a_k = p.a_k; g.b_k = p.b_k; g.b_n = p.b_n;
     const int inner = p.nb < kKernelBatchDims ? p.nb : kKernelBatchDims;
@@ -70,26 +74,71 @@ int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const vo
     return HODU_ROCM_OK;
 }
 
+// Validates the caller's fused steps for an output of `dtype` and turns them into what the kernels read.
+int build_epilogue(const char *op, int kind, int dtype, const void *out, const hodu_rocm_epilogue_step *steps, size_t n,
+                   DevEpilogue *epi) {
+    *epi = DevEpilogue{};
+    if (n == 0) return HODU_ROCM_OK;
+    if (!steps) return fail(HODU_ROCM_INVALID_ARG, "%s: %zu fused steps but the step array is null", op, n);
+    if (n > (size_t)kMaxEpilogueSteps)
+        return fail(HODU_ROCM_INVALID_ARG, "%s: %zu fused steps, at most %d", op, n, kMaxEpilogueSteps);
+    const int out_dtype = kind == PK_BF16_F8W ? HODU_BF16 : kind == PK_I32_I8I8 ? HODU_I32 : dtype;
+    if (out_dtype == HODU_F8E4M3 || out_dtype == HODU_F8E5M2 || out_dtype == HODU_BOOL)
+        return fail(HODU_ROCM_UNSUPPORTED, "%s: fused steps are not defined for dtype id %d", op, out_dtype);
+    const bool floating = out_dtype == HODU_BF16 || out_dtype == HODU_F16 || out_dtype == HODU_F32 || out_dtype == HODU_F64;
+    const size_t es = dtype_size(out_dtype);
+    for (size_t i = 0; i < n; i++) {
+        DevEpilogueStep &d = epi->step[i];
+        d = DevEpilogueStep{};
+        d.op = steps[i].op;
+        switch (steps[i].op) {
+        case HODU_ROCM_EPI_ADD_ROW:
+            if (!steps[i].vector) return fail(HODU_ROCM_INVALID_ARG, "%s: step %zu adds a null vector", op, i);
+            if (steps[i].vector == out) return fail(HODU_ROCM_INVALID_ARG, "%s: step %zu reads the output buffer", op, i);
+            if (steps[i].stride > 0x7FFFFFFFFFFFL || steps[i].offset > 0x7FFFFFFFFFFFL)
+                return fail(HODU_ROCM_INVALID_ARG, "%s: step %zu stride/offset out of range", op, i);
+            d.vec = (const char *)steps[i].vector + steps[i].offset * es;
+            d.stride = (long)steps[i].stride;
+            break;
+        case HODU_ROCM_EPI_MUL_SCALAR:
+            memcpy(&d.scalar, steps[i].scalar, es);  // low bytes; the rest stays zero
+            break;
+        case HODU_ROCM_EPI_RELU:
+            if (!floating) return fail(HODU_ROCM_INVALID_ARG, "%s: relu is defined for floating dtypes only", op);
+            break;
+        default: return fail(HODU_ROCM_INVALID_ARG, "%s: step %zu has unknown op %d", op, i, steps[i].op);
+        }
+    }
+    epi->n = (int)n;
+    return HODU_ROCM_OK;
+}
+
 int matmul_entry(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const size_t *md,
-                 size_t len) {
+                 size_t len, const hodu_rocm_epilogue_step *steps = nullptr, size_t n_steps = 0) {
     clear_error();
     int rc = check_ptrs("matmul", ctx, a, b, c);
     if (rc) return rc;
     Product p;
     rc = parse_matmul_metadata(md, len, &p);
     if (rc) return rc;
-    return run_product(ctx, kind, dtype, a, b, c, p);
+    DevEpilogue epi;
+    rc = build_epilogue("matmul", kind, dtype, c, steps, n_steps, &epi);
+    if (rc) return rc;
+    return run_product(ctx, kind, dtype, a, b, c, p, epi);
 }
 
 int dot_entry(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const size_t *md,
-              size_t len) {
+              size_t len, const hodu_rocm_epilogue_step *steps = nullptr, size_t n_steps = 0) {
     clear_error();
     int rc = check_ptrs("dot", ctx, a, b, c);
     if (rc) return rc;
     Product p;
     rc = parse_dot_metadata(md, len, &p);
     if (rc) return rc;
-    return run_product(ctx, kind, dtype, a, b, c, p);
+    DevEpilogue epi;
+    rc = build_epilogue("dot", kind, dtype, c, steps, n_steps, &epi);
+    if (rc) return rc;
+    return run_product(ctx, kind, dtype, a, b, c, p, epi);
 }
 
 }  // namespace
@@ -139,9 +188,34 @@ int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, voi
     return dot_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
 }
 
+#define HODU_ROCM_DEF_PRODUCT_EX(dt, KIND, ID)                                                                  \
+    int hodu_rocm_matmul_##dt##_ex(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md, \
+                                   size_t n, const hodu_rocm_epilogue_step *steps, size_t n_steps) {           \
+        return matmul_entry(ctx, KIND, ID, l, r, o, md, n, steps, n_steps);                                    \
+    }                                                                                                          \
+    int hodu_rocm_dot_##dt##_ex(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,    \
+                                size_t n, const hodu_rocm_epilogue_step *steps, size_t n_steps) {              \
+        return dot_entry(ctx, KIND, ID, l, r, o, md, n, steps, n_steps);                                       \
+    }
+HODU_ROCM_DEF_PRODUCT_EX(bf16, PK_SAME, HODU_BF16)
+HODU_ROCM_DEF_PRODUCT_EX(f16, PK_SAME, HODU_F16)
+HODU_ROCM_DEF_PRODUCT_EX(f32, PK_SAME, HODU_F32)
+HODU_ROCM_DEF_PRODUCT_EX(f64, PK_SAME, HODU_F64)
+HODU_ROCM_DEF_PRODUCT_EX(u8, PK_SAME, HODU_U8)
+HODU_ROCM_DEF_PRODUCT_EX(u16, PK_SAME, HODU_U16)
+HODU_ROCM_DEF_PRODUCT_EX(u32, PK_SAME, HODU_U32)
+HODU_ROCM_DEF_PRODUCT_EX(u64, PK_SAME, HODU_U64)
+HODU_ROCM_DEF_PRODUCT_EX(i8, PK_SAME, HODU_I8)
+HODU_ROCM_DEF_PRODUCT_EX(i16, PK_SAME, HODU_I16)
+HODU_ROCM_DEF_PRODUCT_EX(i32, PK_SAME, HODU_I32)
+HODU_ROCM_DEF_PRODUCT_EX(i64, PK_SAME, HODU_I64)
+HODU_ROCM_DEF_PRODUCT_EX(bf16_f8e4m3w, PK_BF16_F8W, HODU_BF16)
+HODU_ROCM_DEF_PRODUCT_EX(i32_i8i8, PK_I32_I8I8, HODU_I32)
+
 static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
                                  const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
-                                 int iters, float *elapsed_ms) {
+                                 int iters, float *elapsed_ms, const hodu_rocm_epilogue_step *steps = nullptr,
+                                 size_t n_steps = 0) {
     clear_error();
     if (!ctx || !rhs_list || n_rhs == 0 || !elapsed_ms || iters <= 0)
         return fail(HODU_ROCM_INVALID_ARG, "time_product: bad argument");
@@ -152,6 +226,9 @@ static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int 
     }
     Product p;
     int rc = is_matmul ? parse_matmul_metadata(md, len, &p) : parse_dot_metadata(md, len, &p);
+    if (rc) return rc;
+    DevEpilogue epi;
+    rc = build_epilogue("time_product", kind, dtype, out, steps, n_steps, &epi);
     if (rc) return rc;
     HODU_HIP(hipSetDevice(ctx->device));
     hipEvent_t t0, t1;
@@ -164,7 +241,7 @@ static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int 
         // that cannot afford a host round trip per product would do
         HODU_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
         for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
-            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p);
+            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p, epi);
         hipError_t ce = hipStreamEndCapture(ctx->stream, &g);
         if (rc == HODU_ROCM_OK && ce != hipSuccess) rc = fail(HODU_ROCM_HIP_ERROR, "graph capture: %s", hipGetErrorString(ce));
         if (rc == HODU_ROCM_OK && hipGraphInstantiate(&exec, g, nullptr, nullptr, 0) != hipSuccess)
@@ -180,7 +257,7 @@ static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int 
             rc = fail(HODU_ROCM_HIP_ERROR, "graph launch failed");
     } else {
         for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
-            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p);
+            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p, epi);
     }
     hipError_t e = hipEventRecord(t1, ctx->stream);
     if (e == hipSuccess) e = hipEventSynchronize(t1);
@@ -204,6 +281,13 @@ int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int ki
                                        const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md,
                                        size_t len, int iters, float *elapsed_ms) {
     return time_product_impl(true, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms);
+}
+
+int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                    const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
+                                    const hodu_rocm_epilogue_step *steps, size_t n_steps, int iters, float *elapsed_ms) {
+    return time_product_impl(false, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms,
+                             steps, n_steps);
 }
 
 int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const size_t *md, size_t len) {

@@ -15,6 +15,7 @@
 // decoder (t_f8e4m3.h:34-38) reads those 14 codes as inf/NaN.
 #include "common.hpp"
 #include "device_types.hpp"
+#include "epilogue.hpp"  // ref_f32_to_f16
 
 namespace hodu {
 namespace {
@@ -22,23 +23,6 @@ namespace {
 #pragma clang fp contract(off)
 
 // ---- the reference's narrowing routines, restated for the device -------------------------------
-__device__ __forceinline__ uint16_t ref_f32_to_f16(float val) {
-    if (val == 0.0f) return 0;
-    if (val != val) return 0x7E00;
-    const uint32_t sign = val < 0 ? 1u : 0u;
-    val = fabsf(val);
-    if (isinf(val) || val > 65504.0f) return (uint16_t)((sign << 15) | 0x7C00u);
-    if (val < 0.00006103515625f) return (uint16_t)(sign << 15);
-    int e;
-    float m = frexpf(val, &e);
-    e += 14;
-    if (e <= 0) { m = ldexpf(m, e); e = 0; }
-    else if (e >= 31) return (uint16_t)((sign << 15) | 0x7C00u);
-    int mb = (int)((m * 2.0f - 1.0f) * 1024.0f + 0.5f);
-    if (mb > 1023) mb = 1023;
-    return (uint16_t)((sign << 15) | ((uint32_t)e << 10) | (uint32_t)mb);
-}
-
 __device__ __forceinline__ uint8_t ref_f32_to_f8e4m3(float val) {
     if (val == 0.0f) return 0;
     if (val != val) return 0x7F;

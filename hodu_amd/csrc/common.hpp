@@ -94,6 +94,28 @@ struct Strided {
 };
 int parse_cast_metadata(const size_t *md, size_t len, Strided *s);
 
+// Element-wise steps applied to every output of a product before it is stored: what the callers of the product
+// run next in the reference as kernels of their own (hodu_nn/src/modules/linear.rs:40-46: matmul, then add(bias);
+// attention.rs:37: matmul, then mul_scalar).  A step works on the value the product alone would have stored, with
+// the arithmetic of the reference's element-wise kernel for the output dtype, so the fused result equals the two
+// launches' bit for bit.
+enum EpilogueOp {
+    EPI_ADD_ROW = 1,     // + vec[n * stride]: a vector along the output's last axis (ops_binary.c, add)
+    EPI_MUL_SCALAR = 2,  // * scalar (ops_unary.c, mul_scalar; the scalar in the output dtype)
+    EPI_RELU = 3         // x > 0 ? x : 0 (ops_unary.c, relu; floating dtypes only)
+};
+constexpr int kMaxEpilogueSteps = 3;
+struct DevEpilogueStep {
+    int op;
+    const void *vec;            // device pointer, already offset to element 0 of the vector
+    long stride;                // elements between consecutive entries of the vector
+    unsigned long long scalar;  // bit pattern of the scalar, in the output dtype, in the low bytes
+};
+struct DevEpilogue {
+    int n;  // 0: store the product as it is
+    DevEpilogueStep step[kMaxEpilogueSteps];
+};
+
 // What one launch needs to know about a product; passed by value as a kernel argument.
 struct DevProduct {
     int M, N, K;
@@ -104,6 +126,7 @@ struct DevProduct {
     long a_bs[kKernelBatchDims];
     long b_bs[kKernelBatchDims];
     long batches;                  // product of bshape
+    DevEpilogue epi;
 };
 
 // ------------------------------------------------------------------------------------------------

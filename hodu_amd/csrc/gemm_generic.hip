@@ -10,6 +10,7 @@
 // (RNE; f8 saturates); f64 in f64; integers wrap in their own width, as the reference's do.
 #include "common.hpp"
 #include "device_types.hpp"
+#include "epilogue.hpp"
 
 namespace hodu {
 namespace {
@@ -20,6 +21,7 @@ template <int DT> struct Elem;
     template <> struct Elem<ID> {                                                              \
         typedef S storage;                                                                     \
         typedef A acc;                                                                         \
+        static constexpr int id = ID;                                                          \
         static __device__ __forceinline__ A load(S v) { return (A)v; }                         \
         static __device__ __forceinline__ S store(A v) { return (S)v; }                        \
     };
@@ -37,6 +39,7 @@ NATIVE_ELEM(HODU_I64, int64_t, uint64_t)
     template <> struct Elem<ID> {                                                              \
         typedef S storage;                                                                     \
         typedef uint32_t acc;                                                                  \
+        static constexpr int id = ID;                                                          \
         static __device__ __forceinline__ uint32_t load(S v) { return (uint32_t)(int32_t)v; }  \
         static __device__ __forceinline__ S store(uint32_t v) { return (S)v; }                 \
     };
@@ -46,24 +49,28 @@ SIGNED_ELEM(HODU_I32, int32_t)
 #undef SIGNED_ELEM
 
 template <> struct Elem<HODU_BF16> {
+    static constexpr int id = HODU_BF16;
     typedef uint16_t storage;
     typedef float acc;
     static __device__ __forceinline__ float load(uint16_t v) { return bf16_bits_to_f32(v); }
     static __device__ __forceinline__ uint16_t store(float v) { return f32_to_bf16_bits_rne(v); }
 };
 template <> struct Elem<HODU_F16> {
+    static constexpr int id = HODU_F16;
     typedef uint16_t storage;
     typedef float acc;
     static __device__ __forceinline__ float load(uint16_t v) { return f16_bits_to_f32(v); }
     static __device__ __forceinline__ uint16_t store(float v) { return f32_to_f16_bits_rne(v); }
 };
 template <> struct Elem<HODU_F8E4M3> {
+    static constexpr int id = HODU_F8E4M3;
     typedef uint8_t storage;
     typedef float acc;
     static __device__ __forceinline__ float load(uint8_t v) { return f8e4m3_to_f32(v); }
     static __device__ __forceinline__ uint8_t store(float v) { return f32_to_f8e4m3_sat(v); }
 };
 template <> struct Elem<HODU_F8E5M2> {
+    static constexpr int id = HODU_F8E5M2;
     typedef uint8_t storage;
     typedef float acc;
     static __device__ __forceinline__ float load(uint8_t v) { return f8e5m2_to_f32(v); }
@@ -74,7 +81,9 @@ constexpr int TILE = 64;  // output tile edge
 constexpr int TK = 16;    // k-slice staged per step
 
 // EA / EB: element traits of the operands as stored; EC: of the output.  EA::acc == EB::acc == EC::acc.
-template <class EA, class EB, class EC>
+// EPI: the instantiation that applies fused element-wise steps (behind a call: the plain product should not pay for
+// the stack that costs)
+template <class EA, class EB, class EC, bool EPI>
 __global__ __launch_bounds__(256) void generic_product_kernel(const typename EA::storage *__restrict__ A,
                                                              const typename EB::storage *__restrict__ B,
                                                              typename EC::storage *__restrict__ C, DevProduct g,
@@ -143,7 +152,11 @@ __global__ __launch_bounds__(256) void generic_product_kernel(const typename EA:
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int n = n0 + tx + 16 * j;
-            if (n < g.N) Cb[(long)m * g.N + n] = EC::store(acc[i][j]);
+            if (n < g.N) {
+                typename EC::storage v = EC::store(acc[i][j]);
+                if constexpr (EPI) v = epilogue_apply_call<EC::id>(g.epi, v, n);
+                Cb[(long)m * g.N + n] = v;
+            }
         }
     }
 }
@@ -154,9 +167,9 @@ int run(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProd
     const long blocks = g.batches * tiles_m * tiles_n;
     if (blocks <= 0) return HODU_ROCM_OK;
     if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", blocks);
-    hipLaunchKernelGGL((generic_product_kernel<EA, EB, EC>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
-                       (const typename EA::storage *)a, (const typename EB::storage *)b,
-                       (typename EC::storage *)c, g, tiles_m, tiles_n);
+    auto kernel = g.epi.n != 0 ? generic_product_kernel<EA, EB, EC, true> : generic_product_kernel<EA, EB, EC, false>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const typename EA::storage *)a,
+                       (const typename EB::storage *)b, (typename EC::storage *)c, g, tiles_m, tiles_n);
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }

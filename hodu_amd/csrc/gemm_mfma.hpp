@@ -27,6 +27,7 @@
 
 #include "common.hpp"
 #include "device_types.hpp"
+#include "epilogue.hpp"
 
 namespace hodu {
 namespace mfma {
@@ -464,28 +465,46 @@ template <int SK, int CK, int ROWS, int NT> struct Loader<LM_SCALAR, SK, CK, ROW
 // ------------------------------------------------------------------------------------------------
 template <int OUT> struct Out;
 template <> struct Out<OUT_BF16> {
+    static constexpr int DT = HODU_BF16;
     typedef uint16_t T;
     static __device__ __forceinline__ T cvt(float v) { return f32_to_bf16_bits_rne(v); }
 };
 template <> struct Out<OUT_F16> {
+    static constexpr int DT = HODU_F16;
     typedef uint16_t T;
     static __device__ __forceinline__ T cvt(float v) { return f32_to_f16_bits_rne(v); }
 };
 template <> struct Out<OUT_F32> {
+    static constexpr int DT = HODU_F32;
     typedef float T;
     static __device__ __forceinline__ T cvt(float v) { return v; }
 };
 template <> struct Out<OUT_I32> {
+    static constexpr int DT = HODU_I32;
     typedef int32_t T;
     static __device__ __forceinline__ T cvt(int v) { return v; }
 };
 
+// accumulator -> stored element: the product's own rounding, then the fused element-wise steps for column n
+template <int OUT, class A>
+__device__ __forceinline__ typename Out<OUT>::T finish(const DevEpilogue &epi, A acc, long n) {
+    return epilogue_apply<Out<OUT>::DT>(epi, Out<OUT>::cvt(acc), n);
+}
+
+// the same for the kernel below, which has TM x TN x 16 store sites per lane: the steps sit behind a call, in an
+// instantiation of the kernel of its own (a call costs the kernel a stack, which the plain product should not pay)
+template <int OUT, class A>
+__device__ __forceinline__ typename Out<OUT>::T finish_call(const DevEpilogue &epi, A acc, long n) {
+    const typename Out<OUT>::T v = Out<OUT>::cvt(acc);
+    return epi.n == 0 ? v : epilogue_apply_call<Out<OUT>::DT>(epi, v, n);
+}
+
 // Stores the 32x32 accumulator tile of one wavefront.  With the operands swapped in the MFMA (the
 // right operand's fragment in the A slot) a lane holds, for ONE output row m = m_base + l % 32, four
 // runs of four consecutive columns n = n_base + 8*q + 4*(l / 32) + e.
-template <int OUT, class acc_t>
+template <int OUT, bool EPI, class acc_t>
 __device__ __forceinline__ void store_tile32(typename Out<OUT>::T *Cb, const acc_t &acc, int m, int n_base, int lh,
-                                             int M, int N, bool vec_ok) {
+                                             int M, int N, bool vec_ok, const DevEpilogue &epi) {
     typedef typename Out<OUT>::T out_t;
     if (m >= M) return;
 #pragma unroll
@@ -493,7 +512,10 @@ __device__ __forceinline__ void store_tile32(typename Out<OUT>::T *Cb, const acc
         const int n = n_base + 8 * q + 4 * lh;
         out_t v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = Out<OUT>::cvt(acc[4 * q + e]);
+        for (int e = 0; e < 4; e++) {
+            if constexpr (EPI) v[e] = finish_call<OUT>(epi, acc[4 * q + e], n + e < N ? n + e : N - 1);  // ragged: stay inside the vector
+            else v[e] = Out<OUT>::cvt(acc[4 * q + e]);
+        }
         out_t *dst = Cb + (long)m * N + n;
         if (vec_ok && n + 3 < N) {
             struct alignas(sizeof(out_t) * 4) Quad { out_t q[4]; };
@@ -574,7 +596,7 @@ __device__ __forceinline__ void compute_stage(const char *As, const char *Bs, ac
 // LDS-DMA loads are tracked by vmcnt; wait for them before the barrier that publishes the stage
 __device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-template <class Cfg>
+template <class Cfg, bool EPI>
 __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                typename Out<Cfg::OUT>::T *__restrict__ C,
                                                                DevProduct g, int tiles_m, int tiles_n) {
@@ -649,8 +671,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++)
-            store_tile32<Cfg::OUT>(Cb, acc[i][j], m0 + wave_m * TM * 32 + i * 32 + lr, n0 + wave_n * TN * 32 + j * 32, lh,
-                                   g.M, g.N, vec_ok);
+            store_tile32<Cfg::OUT, EPI>(Cb, acc[i][j], m0 + wave_m * TM * 32 + i * 32 + lr, n0 + wave_n * TN * 32 + j * 32, lh,
+                                   g.M, g.N, vec_ok, g.epi);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -677,10 +699,12 @@ inline int pick_mode(const void *base, long off, long row_stride, long k_stride,
 
 template <class Cfg> int launch_config(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
     static bool configured = false;  // benign race: the attribute call is idempotent
-    auto kernel = mfma_product_kernel<Cfg>;
+    auto kernel = g.epi.n != 0 ? mfma_product_kernel<Cfg, true> : mfma_product_kernel<Cfg, false>;
     if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     Cfg::LDS_BYTES));
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_product_kernel<Cfg, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_product_kernel<Cfg, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
         configured = true;
     }
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;

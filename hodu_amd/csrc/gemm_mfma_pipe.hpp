@@ -143,9 +143,10 @@ __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
 // band per 2..16 lanes -- instead of the accumulator layout's 8-byte pieces of 32 different rows per instruction
 // (measured: 13 us of a 37 us launch spent storing a 256 x 256 bf16 tile that way).
 //   acc layout (operands swapped): lane (lr, lh) holds row lr, columns 32*j + 8*q + 4*lh + e of the band.
-template <int OUT, int TN, class acc_t>
+// EPI: the values are final outputs and take the fused element-wise steps (partial sums of a K range do not).
+template <int OUT, int TN, bool EPI, class acc_t>
 __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,
-                                                   int n_base, int lane, int M, int N) {
+                                                   int n_base, int lane, int M, int N, const DevEpilogue &epi) {
     typedef typename Out<OUT>::T out_t;
     constexpr int OS = sizeof(out_t), ROWB = TN * 32 * OS, PITCH = ROWB + 16, EPV = 16 / OS;
     constexpr int CPR = ROWB / 16, RPP = 64 / CPR;  // 16-byte chunks per row, rows per pass of the wavefront
@@ -165,12 +166,19 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
     // compiler is told not to move the differently-typed accesses across each other
     asm volatile("" ::: "memory");
     const bool vec_ok = ((long)N * OS) % 16 == 0;
-#pragma unroll
-    for (int pass = 0; pass < 32 / RPP; pass++) {
+    // the fused element-wise steps work on the rounded values, here where a lane holds EPV neighbouring columns
+    // of one row -- the same columns in every pass, so what the steps need for them is fetched once
+    EpiPrepared<Out<OUT>::DT, EPV> prepared;
+    if (EPI && epi.n != 0) {
+        const int n = n_base + (lane % CPR) * EPV;
+        prepared = epilogue_prepare<Out<OUT>::DT, EPV>(epi, n < N ? n : N - 1, N);
+    }
+    auto row_chunk = [&](int pass, auto fused) {
         const int row = pass * RPP + lane / CPR, chunk = lane % CPR;
-        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(patch + row * PITCH + chunk * 16);
+        u32x4_t v = *reinterpret_cast<const u32x4_t *>(patch + row * PITCH + chunk * 16);
         const int m = m_base + row, n = n_base + chunk * EPV;
-        if (m >= M || n >= N) continue;
+        if (m >= M || n >= N) return;
+        if constexpr (decltype(fused)::value) epilogue_apply_prepared<Out<OUT>::DT, EPV>(prepared, reinterpret_cast<out_t *>(&v));
         out_t *dst = Cb + (long)m * N + n;
         if (vec_ok && n + EPV <= N) {
             *reinterpret_cast<u32x4_t *>(dst) = v;
@@ -180,6 +188,20 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
             for (int k = 0; k < EPV; k++)
                 if (n + k < N) dst[k] = e[k];
         }
+    };
+    if (EPI && epi.n != 0) {
+        // f16 stays rolled (nothing here indexes registers by `pass`): its narrowing routine is some fifty
+        // instructions per element, inlined once per band this way instead of once per pass
+        if constexpr (Out<OUT>::DT == HODU_F16) {
+#pragma unroll 1
+            for (int pass = 0; pass < 32 / RPP; pass++) row_chunk(pass, std::true_type{});
+        } else {
+#pragma unroll
+            for (int pass = 0; pass < 32 / RPP; pass++) row_chunk(pass, std::true_type{});
+        }
+    } else {
+#pragma unroll
+        for (int pass = 0; pass < 32 / RPP; pass++) row_chunk(pass, std::false_type{});
     }
     asm volatile("" ::: "memory");  // the next band overwrites the patch
 }
@@ -534,21 +556,29 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         part_t *Pb = (part_t *)partials + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
 #pragma unroll
         for (int i = 0; i < TM; i++)
-            store_band_via_lds<ACC, TN>(patch, Pb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N);
+            store_band_via_lds<ACC, TN, false>(patch, Pb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
         return;
     }
     Cb = C + batch * (long)g.M * g.N;
 #pragma unroll
     for (int i = 0; i < TM; i++)
-        store_band_via_lds<Cfg::OUT, TN>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N);
+        store_band_via_lds<Cfg::OUT, TN, true>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
 }
 
 // out[i] = round(partials[0][i] + partials[1][i] + ...), the slabs added in index order: bit-reproducible
 template <int OUT, class part_t>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const part_t *__restrict__ partials,
-                                                           typename Out<OUT>::T *__restrict__ out, long elems, int splits) {
+                                                           typename Out<OUT>::T *__restrict__ out, long elems, int splits,
+                                                           int N, DevEpilogue epi) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= elems) return;
+    // column of element i + e, for the fused element-wise steps (rows are N long, outputs contiguous)
+    long col[4] = {0, 0, 0, 0};
+    if (epi.n != 0) {
+        col[0] = i % N;
+#pragma unroll
+        for (int e = 1; e < 4; e++) col[e] = col[e - 1] + 1 == N ? 0 : col[e - 1] + 1;
+    }
     if (i + 3 < elems) {
         struct alignas(16) Quad { part_t q[4]; };
         Quad s = *reinterpret_cast<const Quad *>(partials + i);
@@ -558,13 +588,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const part_t *__rest
             for (int e = 0; e < 4; e++) s.q[e] += t.q[e];
         }
         struct alignas(sizeof(typename Out<OUT>::T) * 4) OutQuad { typename Out<OUT>::T q[4]; };
-        *reinterpret_cast<OutQuad *>(out + i) = OutQuad{{Out<OUT>::cvt(s.q[0]), Out<OUT>::cvt(s.q[1]), Out<OUT>::cvt(s.q[2]),
-                                                       Out<OUT>::cvt(s.q[3])}};
+        *reinterpret_cast<OutQuad *>(out + i) = OutQuad{{finish<OUT>(epi, s.q[0], col[0]), finish<OUT>(epi, s.q[1], col[1]),
+                                                       finish<OUT>(epi, s.q[2], col[2]), finish<OUT>(epi, s.q[3], col[3])}};
     } else {
         for (long j = i; j < elems; j++) {
             part_t s = partials[j];
             for (int k = 1; k < splits; k++) s += partials[(long)k * elems + j];
-            out[j] = Out<OUT>::cvt(s);
+            out[j] = finish<OUT>(epi, s, col[j - i]);
         }
     }
 }
@@ -606,10 +636,10 @@ template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const vo
         const unsigned blocks = (unsigned)((elems + 1023) / 1024);
         if (Cfg::CK == CK_I8)
             hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, int32_t>), dim3(blocks), dim3(256), 0, ctx->stream,
-                               (const int32_t *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits);
+                               (const int32_t *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits, g.N, g.epi);
         else
             hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, float>), dim3(blocks), dim3(256), 0, ctx->stream,
-                               (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits);
+                               (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits, g.N, g.epi);
         HODU_HIP(hipGetLastError());
     }
     return HODU_ROCM_OK;

@@ -24,6 +24,7 @@ namespace mfma {
 enum { OUT_F8E4M3 = 4 };
 
 template <> struct Out<OUT_F8E4M3> {
+    static constexpr int DT = HODU_F8E4M3;
     typedef uint8_t T;
     // same narrowing as the generic kernel's f8e4m3 products: round to nearest even, saturating at +-448
     static __device__ __forceinline__ T cvt(float v) { return f32_to_f8e4m3_sat(v); }
@@ -234,13 +235,13 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
         float *Pb = (float *)partials + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
 #pragma unroll
         for (int i = 0; i < TM; i++)
-            store_band_via_lds<OUT_F32, TN>(patch, Pb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N);
+            store_band_via_lds<OUT_F32, TN, false>(patch, Pb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
         return;
     }
     out_t *Cb = C + batch * (long)g.M * g.N;
 #pragma unroll
     for (int i = 0; i < TM; i++)
-        store_band_via_lds<Cfg::OUT, TN>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N);
+        store_band_via_lds<Cfg::OUT, TN, false>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
 }
 
 template <class Cfg>
@@ -275,7 +276,7 @@ int launch_pipe_f8(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, co
     if (splits > 1) {
         const unsigned blocks = (unsigned)((elems + 1023) / 1024);
         hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, float>), dim3(blocks), dim3(256), 0, ctx->stream,
-                           (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits);
+                           (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits, g.N, g.epi);
         HODU_HIP(hipGetLastError());
     }
     return HODU_ROCM_OK;

@@ -76,7 +76,8 @@ template <int SKB, int M, int R, int NW>
 __global__ __launch_bounds__(NW * 64, (M <= 2 ? 4 : 2)) void gemv_rowstream_kernel(const char *__restrict__ X,
                                                                                   const char *__restrict__ W,
                                                                                   uint16_t *__restrict__ Y, int N, int K,
-                                                                                  long x_row_bytes, long w_row_bytes) {
+                                                                                  long x_row_bytes, long w_row_bytes,
+                                                                                  DevEpilogue epi) {
     constexpr int EPL = WeightVec<SKB>::EPL, XV = WeightVec<SKB>::XV, SB = SKB == SK_F8 ? 1 : 2;
     constexpr int STEP = GEMV_NCH * 64 * EPL;  // k covered by one pass of a wavefront
     const int tid = threadIdx.x, lane = tid & 63;
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(NW * 64, (M <= 2 ? 4 : 2)) void gemv_rowstream_kern
             const float v = wave_sum(acc[m][r]);
             mine = lane == r ? v : mine;
         }
-        if (lane < R && n0 + lane < N) Y[(long)m * N + n0 + lane] = mfma::Out<mfma::OUT_BF16>::cvt(mine);
+        if (lane < R && n0 + lane < N) Y[(long)m * N + n0 + lane] = mfma::finish<mfma::OUT_BF16>(epi, mine, n0 + lane);
     }
 }
 
@@ -151,7 +152,7 @@ int launch_one(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const 
     const long waves = (g.N + R - 1) / R;
     const unsigned blocks = (unsigned)((waves + NW - 1) / NW);
     hipLaunchKernelGGL((gemv_rowstream_kernel<SKB, M, R, NW>), dim3(blocks), dim3(NW * 64), 0, ctx->stream, X, Wp,
-                       (uint16_t *)y, g.N, g.K, g.a_m * (long)ES, g.b_n * (long)SB);
+                       (uint16_t *)y, g.N, g.K, g.a_m * (long)ES, g.b_n * (long)SB, g.epi);
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }

@@ -173,10 +173,15 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
         out_t *Yb = Y + batch * (long)g.M * g.N;
         const int col = ((int)(blockIdx.x % tiles_n) * NBLK + wave) * 16 + lr;
         if (col < g.N) {
+            // the lane's four outputs share a column: what the fused steps need for it is fetched once
+            EpiPrepared<Out<OUT>::DT, 1> prepared;
+            if (g.epi.n != 0) prepared = epilogue_prepare<Out<OUT>::DT, 1>(g.epi, col, g.N);
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int m = 4 * lg + e;
-                if (m < g.M) Yb[(long)m * g.N + col] = Out<OUT>::cvt(s[e]);
+                out_t v = Out<OUT>::cvt(s[e]);
+                if (g.epi.n != 0) epilogue_apply_prepared<Out<OUT>::DT, 1>(prepared, &v);
+                if (m < g.M) Yb[(long)m * g.N + col] = v;
             }
         }
     }
@@ -328,10 +333,14 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
             for (int j = 0; j < 8; j++)
                 if (k0 + j < slices) s += v[j];
         }
+        EpiPrepared<Out<OUT>::DT, 1> prepared;  // the lane's four outputs share a column
+        if (g.epi.n != 0) prepared = epilogue_prepare<Out<OUT>::DT, 1>(g.epi, col, g.N);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const int m = quad * 4 + e;
-            if (m < g.M) Y[(long)m * g.N + col] = Out<OUT>::cvt(s[e]);
+            typename Out<OUT>::T v = Out<OUT>::cvt(s[e]);
+            if (g.epi.n != 0) epilogue_apply_prepared<Out<OUT>::DT, 1>(prepared, &v);
+            if (m < g.M) Y[(long)m * g.N + col] = v;
         }
     }
     if (tid == 0) __hip_atomic_store(&arrival[nb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

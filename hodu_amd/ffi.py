@@ -37,6 +37,38 @@ class HoduRocmError(RuntimeError):
 _lib: Optional[ctypes.CDLL] = None
 
 
+class EpilogueStep(ctypes.Structure):
+    """hodu_rocm_epilogue_step of include/hodu_rocm_kernels.h"""
+    _fields_ = [("op", ctypes.c_int), ("vector", ctypes.c_void_p), ("stride", ctypes.c_size_t),
+                ("offset", ctypes.c_size_t), ("scalar", ctypes.c_ubyte * 8)]
+
+
+EPI_ADD_ROW, EPI_MUL_SCALAR, EPI_RELU = 1, 2, 3
+# dtypes whose products take fused element-wise steps (the 8-bit floats do not)
+EPILOGUE_DTYPES = ["bf16", "f16", "f32", "f64", "u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
+
+
+def add_row(vector: "DeviceBuffer", stride: int = 1, offset: int = 0) -> EpilogueStep:
+    """out[.., m, n] += vector[offset + n * stride] (a bias along the last axis)"""
+    return EpilogueStep(EPI_ADD_ROW, vector.ptr, int(stride), int(offset), (ctypes.c_ubyte * 8)())
+
+
+def mul_scalar(scalar) -> EpilogueStep:
+    """out *= scalar; scalar: a numpy scalar / 1-element array in the output dtype's storage"""
+    raw = np.ascontiguousarray(scalar).reshape(1).tobytes()
+    buf = (ctypes.c_ubyte * 8)(*raw, *([0] * (8 - len(raw))))
+    return EpilogueStep(EPI_MUL_SCALAR, None, 0, 0, buf)
+
+
+def relu() -> EpilogueStep:
+    return EpilogueStep(EPI_RELU, None, 0, 0, (ctypes.c_ubyte * 8)())
+
+
+def _steps_array(steps):
+    steps = list(steps)
+    return (EpilogueStep * max(1, len(steps)))(*steps), len(steps)
+
+
 def load() -> ctypes.CDLL:
     """Load the built HIP library; raises if it is missing (build with `python -m hodu_amd.build`)."""
     global _lib
@@ -77,6 +109,11 @@ def load() -> ctypes.CDLL:
     for dt in PRODUCT_DTYPES + list(FUSED_PRODUCTS):
         for op in ("matmul", "dot"):
             getattr(lib, f"hodu_rocm_{op}_{dt}").argtypes = [vp, vp, vp, vp, szp, sz]
+    for dt in EPILOGUE_DTYPES + list(FUSED_PRODUCTS):
+        for op in ("matmul", "dot"):
+            getattr(lib, f"hodu_rocm_{op}_{dt}_ex").argtypes = [vp, vp, vp, vp, szp, sz, ctypes.POINTER(EpilogueStep), sz]
+    lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz,
+                                                    ctypes.POINTER(EpilogueStep), sz, ci, ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     _lib = lib
@@ -199,6 +236,15 @@ class Context:
         fn = getattr(self.lib, f"hodu_rocm_{op}_{name}")
         self._check(fn(self.handle, lhs.ptr, rhs.ptr, out.ptr, arr, n))
 
+    def product_ex(self, op: str, name: str, lhs: DeviceBuffer, rhs: DeviceBuffer, out: DeviceBuffer, md, steps):
+        """hodu_rocm_<op>_<name>_ex: the product with element-wise steps (add_row / mul_scalar / relu) fused into
+        its store"""
+        self._check_extents(op, name, lhs, [rhs], out, md)
+        arr, n = _md_array(md)
+        sarr, ns = _steps_array(steps)
+        fn = getattr(self.lib, f"hodu_rocm_{op}_{name}_ex")
+        self._check(fn(self.handle, lhs.ptr, rhs.ptr, out.ptr, arr, n, sarr, ns))
+
     @staticmethod
     def _check_extents(op, name, lhs, rhs_list, out, md):
         """refuse a launch whose metadata reaches past one of the device buffers"""
@@ -234,7 +280,7 @@ class Context:
         self._check(self.lib.hodu_rocm_contiguous(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
 
     def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int,
-                     graph: bool = False) -> float:
+                     graph: bool = False, steps=None) -> float:
         """back-to-back launches issued from C (graph=True: recorded once into a HIP graph and replayed as
         one graph launch), HIP-event timed on the context's stream; total ms"""
         self._check_extents(op, name, lhs, rhs_list, out, md)
@@ -243,6 +289,12 @@ class Context:
         arr, n = _md_array(md)
         ptrs = (ctypes.c_void_p * len(rhs_list))(*[b.ptr for b in rhs_list])
         ms = ctypes.c_float()
+        if steps:
+            sarr, ns = _steps_array(steps)
+            self._check(self.lib.hodu_rocm_debug_time_product_ex(
+                self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr, n,
+                sarr, ns, int(iters), ctypes.byref(ms)))
+            return float(ms.value)
         fn = self.lib.hodu_rocm_debug_time_product_graph if graph else self.lib.hodu_rocm_debug_time_product
         self._check(fn(self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr,
                        n, int(iters), ctypes.byref(ms)))

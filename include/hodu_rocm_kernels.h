@@ -144,6 +144,67 @@ int hodu_rocm_matmul_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void
 int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void *rhs_i8,
                            void *out_i32, const size_t *metadata, size_t metadata_len);
 
+/* ---- matmul / dot with the caller's next element-wise kernels fused into the store -------------- *
+ * The reference's callers of the product launch an element-wise kernel on its output straight away:
+ *   Linear::forward (crates/hodu_nn/src/modules/linear.rs:40-46): matmul, then add(bias)
+ *       -> hodu_cpu_add_<dt> (kernels/ops_binary.c:208-262 and the native-type macro above it)
+ *   scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:37): matmul, then mul_scalar
+ *       -> hodu_cpu_mul_scalar_<dt> (kernels/ops_unary.c:138-200, :352-386)
+ *   ReLU after a Linear (crates/hodu_nn/src/modules/activation.rs:8-17): relu
+ *       -> hodu_cpu_relu_<dt> (kernels/ops_unary.c:648-697, :1404, :1484)
+ * The _ex entry points apply up to HODU_ROCM_MAX_EPILOGUE_STEPS such steps, in order, to every output element
+ * before it is stored.  Each step takes the value the plain product would have stored (already rounded to the
+ * output dtype) and uses the reference kernel's arithmetic for that dtype -- bf16 adds in f32 and truncates,
+ * f16 narrows through the reference's own routine, integers wrap --, so the result equals running the plain
+ * entry point followed by the reference's kernels bit for bit, with one pass over the output instead of
+ * 1 + 2 per step.  n_steps == 0 is the plain product.  The f8 dtypes have no _ex form.
+ *   ADD_ROW:    out[.., m, n] += vector[offset + n * stride]; `vector` is device storage of the output dtype.
+ *               This is what Tensor::add makes of a bias: broadcast_tensors2 (tensor/ops/binary.rs:21) gives the
+ *               operand the output's shape with stride 0 on every axis but the last; pass that last stride
+ *               (0 allowed: one value for all columns) and the layout's offset.
+ *   MUL_SCALAR: out *= scalar; `scalar` holds the value in the output dtype, as the reference kernel's
+ *               `const void *scalar` argument points to it (low bytes first).
+ *   RELU:       out = out > 0 ? out : 0 (floating dtypes only; NaN and -0 become +0 as in the reference).      */
+enum {
+    HODU_ROCM_EPI_ADD_ROW = 1,
+    HODU_ROCM_EPI_MUL_SCALAR = 2,
+    HODU_ROCM_EPI_RELU = 3
+};
+#define HODU_ROCM_MAX_EPILOGUE_STEPS 3
+typedef struct hodu_rocm_epilogue_step {
+    int op;
+    const void *vector;
+    size_t stride;
+    size_t offset;
+    unsigned char scalar[8];
+} hodu_rocm_epilogue_step;
+#define HODU_ROCM_DECL_PRODUCT_EX(dt)                                                                        \
+    int hodu_rocm_matmul_##dt##_ex(hodu_rocm_ctx *ctx, const void *lhs, const void *rhs, void *out,          \
+                                   const size_t *metadata, size_t metadata_len,                              \
+                                   const hodu_rocm_epilogue_step *steps, size_t n_steps);                    \
+    int hodu_rocm_dot_##dt##_ex(hodu_rocm_ctx *ctx, const void *lhs, const void *rhs, void *out,             \
+                                const size_t *metadata, size_t metadata_len,                                 \
+                                const hodu_rocm_epilogue_step *steps, size_t n_steps);
+HODU_ROCM_DECL_PRODUCT_EX(bf16)
+HODU_ROCM_DECL_PRODUCT_EX(f16)
+HODU_ROCM_DECL_PRODUCT_EX(f32)
+HODU_ROCM_DECL_PRODUCT_EX(f64)
+HODU_ROCM_DECL_PRODUCT_EX(u8)
+HODU_ROCM_DECL_PRODUCT_EX(u16)
+HODU_ROCM_DECL_PRODUCT_EX(u32)
+HODU_ROCM_DECL_PRODUCT_EX(u64)
+HODU_ROCM_DECL_PRODUCT_EX(i8)
+HODU_ROCM_DECL_PRODUCT_EX(i16)
+HODU_ROCM_DECL_PRODUCT_EX(i32)
+HODU_ROCM_DECL_PRODUCT_EX(i64)
+HODU_ROCM_DECL_PRODUCT_EX(bf16_f8e4m3w) /* vector / scalar in bf16 */
+HODU_ROCM_DECL_PRODUCT_EX(i32_i8i8)     /* vector / scalar in i32 */
+/* measurement hook: hodu_rocm_debug_time_product with fused steps */
+int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
+                                    const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
+                                    size_t metadata_len, const hodu_rocm_epilogue_step *steps, size_t n_steps,
+                                    int iters, float *elapsed_ms);
+
 /* ---- casts and strided gather ------------------------------------------------------------------ *
  * replaces hodu_cpu_cast_<src>_to_<dst> (kernels/ops_cast.c:53, table :108-388) and
  * hodu_cpu_contiguous_<dt> (kernels/ops_memory.c:36).  One entry point taking dtype ids stands

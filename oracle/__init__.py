@@ -138,6 +138,31 @@ def contiguous(dt: str, x: np.ndarray, md) -> np.ndarray:
     return out
 
 
+def add(dt: str, lhs: np.ndarray, rhs: np.ndarray, md) -> np.ndarray:
+    """hodu_cpu_add_<dt>; md in the binary-op format [n, nd, lhs_shape, rhs_shape, lhs_strides, rhs_strides, lo, ro]"""
+    md = _md(md)
+    out = np.empty(int(md[0]), dtype=STORAGE[dt])
+    _check(lib().oracle_add(DTYPE_ID[dt], _ptr(lhs), _ptr(rhs), _ptr(out), _ptr(md)), "add")
+    return out
+
+
+def mul_scalar(dt: str, x: np.ndarray, md, scalar: np.ndarray) -> np.ndarray:
+    """hodu_cpu_mul_scalar_<dt>; scalar: one element in dt's storage; md in the unary format"""
+    md = _md(md)
+    scalar = np.ascontiguousarray(scalar, dtype=STORAGE[dt]).reshape(1)
+    out = np.empty(int(md[0]), dtype=STORAGE[dt])
+    _check(lib().oracle_mul_scalar(DTYPE_ID[dt], _ptr(x), _ptr(out), _ptr(md), _ptr(scalar)), "mul_scalar")
+    return out
+
+
+def relu(dt: str, x: np.ndarray, md) -> np.ndarray:
+    """hodu_cpu_relu_<dt>"""
+    md = _md(md)
+    out = np.empty(int(md[0]), dtype=STORAGE[dt])
+    _check(lib().oracle_relu(DTYPE_ID[dt], _ptr(x), _ptr(out), _ptr(md)), "relu")
+    return out
+
+
 def f8e4m3_table(decode: int) -> np.ndarray:
     """All 256 decoded values as f32."""
     return np.array([lib().oracle_f8e4m3_to_f32(b, decode) for b in range(256)], dtype=np.float32)
@@ -196,6 +221,31 @@ class RefLib:
         md = _md(md)
         out = np.empty(int(md[0]), dtype=STORAGE[dt])
         fn = getattr(self.lib, f"hodu_cpu_contiguous_{dt}")
+        fn.restype = None
+        fn(_ptr(x), _ptr(out), _ptr(md))
+        return out
+
+    def add(self, dt, lhs, rhs, md):
+        md = _md(md)
+        out = np.empty(int(md[0]), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_add_{dt}")
+        fn.restype = None
+        fn(_ptr(lhs), _ptr(rhs), _ptr(out), _ptr(md))
+        return out
+
+    def mul_scalar(self, dt, x, md, scalar):
+        md = _md(md)
+        scalar = np.ascontiguousarray(scalar, dtype=STORAGE[dt]).reshape(1)
+        out = np.empty(int(md[0]), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_mul_scalar_{dt}")
+        fn.restype = None
+        fn(_ptr(x), _ptr(out), _ptr(md), _ptr(scalar))
+        return out
+
+    def relu(self, dt, x, md):
+        md = _md(md)
+        out = np.empty(int(md[0]), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_relu_{dt}")
         fn.restype = None
         fn(_ptr(x), _ptr(out), _ptr(md))
         return out

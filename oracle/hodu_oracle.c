@@ -14,6 +14,11 @@
  *   dot      crates/hodu_cpu_kernels/kernels/ops_matrix.c:399-549, :556-701, metadata :371-380
  *   cast     crates/hodu_cpu_kernels/kernels/ops_cast.c:34-103 and the table :108-388
  *   gather   crates/hodu_cpu_kernels/kernels/ops_memory.c:19-84
+ *   add      crates/hodu_cpu_kernels/kernels/ops_binary.c:208-262 (bf16/f16/f8: widen, add in f32, narrow with the
+ *            type's own routine) and the native-type macro :60-118; metadata :214-222
+ *   mul_scalar, relu
+ *            crates/hodu_cpu_kernels/kernels/ops_unary.c:138-200, :352-386 (scalar arrives in the storage type),
+ *            :648-697, :1233, :1319, :1404, :1484 ((x > 0) ? x : 0 in f32)
  *   scalars  kernels/t_bf16.h:27-55, t_f16.h:27-84, t_f8e4m3.h:27-85, t_f8e5m2.h:27-84
  *   helpers  kernels/utils.h:16-38 (is_contiguous, get_strided_index)
  *
@@ -33,6 +38,10 @@
  * reference C compiled from /root/reference) and with the committed fixtures tests/golden/ that
  * were produced from it; with the literal vectors of the reference's own kernel tests; integer
  * results with numpy int64 matmul; SPEC with float64 matmul and torch's float8/bfloat16 tables.
+ *
+ * The element-wise functions (add, mul_scalar, relu) are compared bit for bit with oracle/_ref on random bit
+ * patterns of every dtype, with the literal vectors of the reference's tests (tests/ops_binary.rs:68-73,
+ * tests/ops_unary.rs:143-147, :503-507) and, for bf16, with an independent numpy f32 sum whose low 16 bits are cut.
  *
  * Parity unpinned: float->integer casts of out-of-range or NaN inputs are undefined behaviour
  * in the reference C ((T)x) and are not checked.
@@ -615,6 +624,104 @@ int oracle_contiguous(int dt, const void *in, void *out, const size_t *md) {
     }
     return 0;
 }
+
+/* ------------------------------------------------------------------------------------------ */
+/* element-wise kernels that the callers of the product run on its output                       */
+/* ------------------------------------------------------------------------------------------ */
+enum { EW_ADD = 1, EW_MUL = 2, EW_RELU = 3 };
+
+/* one element of `op` in the arithmetic of dtype dt; a, b, out point at single elements.
+ * Narrow floats: ops_binary.c:228-232 / ops_unary.c:359-371 (float x = TO_FLOAT(..); out = FROM_FLOAT(FUNC)).
+ * Native types: the expression is evaluated in TYPE (`TYPE x = ...; out[i] = x + y`), which for the integer types
+ * means C's promotion to int followed by conversion back -- modular arithmetic on two's-complement machines. */
+static int ew_one(int dt, int op, const void *a, const void *b, void *out) {
+#define EW_NARROW(T, WIDEN, NARROW)                                                    \
+    {                                                                                  \
+        const float x = WIDEN(*(const T *)a);                                          \
+        float r;                                                                       \
+        if (op == EW_RELU) r = (x > 0.0f) ? x : 0.0f;                                  \
+        else {                                                                         \
+            const float y = WIDEN(*(const T *)b);                                      \
+            r = op == EW_ADD ? x + y : x * y;                                          \
+        }                                                                              \
+        *(T *)out = NARROW(r);                                                         \
+        return 0;                                                                      \
+    }
+#define EW_FLOAT(T)                                                                    \
+    {                                                                                  \
+        const T x = *(const T *)a;                                                     \
+        if (op == EW_RELU) *(T *)out = (x > (T)0) ? x : (T)0;                          \
+        else *(T *)out = op == EW_ADD ? x + *(const T *)b : x * *(const T *)b;         \
+        return 0;                                                                      \
+    }
+#define EW_INT(T, U)                                                                   \
+    {                                                                                  \
+        if (op == EW_RELU) return -1; /* the reference has no relu for integer types */\
+        const U x = (U) * (const T *)a, y = (U) * (const T *)b;                        \
+        *(T *)out = (T)(U)(op == EW_ADD ? x + y : x * y);                              \
+        return 0;                                                                      \
+    }
+    switch (dt) {
+    case DT_BF16: EW_NARROW(uint16_t, bf16_widen, bf16_truncate)
+    case DT_F16: EW_NARROW(uint16_t, f16_widen, f16_narrow)
+    case DT_F8E4M3: EW_NARROW(uint8_t, f8e4m3_widen_hodu, f8e4m3_narrow)
+    case DT_F8E5M2: EW_NARROW(uint8_t, f8e5m2_widen, f8e5m2_narrow)
+    case DT_F32: EW_FLOAT(float)
+    case DT_F64: EW_FLOAT(double)
+    case DT_U8: EW_INT(uint8_t, uint8_t)
+    case DT_U16: EW_INT(uint16_t, uint16_t)
+    case DT_U32: EW_INT(uint32_t, uint32_t)
+    case DT_U64: EW_INT(uint64_t, uint64_t)
+    case DT_I8: EW_INT(int8_t, uint8_t)
+    case DT_I16: EW_INT(int16_t, uint16_t)
+    case DT_I32: EW_INT(int32_t, uint32_t)
+    case DT_I64: EW_INT(int64_t, uint64_t)
+    default: return -1;
+    }
+#undef EW_NARROW
+#undef EW_FLOAT
+#undef EW_INT
+}
+
+/* hodu_cpu_add_<dt>(lhs, rhs, out, metadata); metadata = [num_els, nd, lhs_shape.., rhs_shape.., lhs_strides..,
+ * rhs_strides.., lhs_offset, rhs_offset] (ops_binary.c:214-222, op_metadatas.rs:36-73).  All four
+ * contiguous / strided branches of the reference compute the same element positions. */
+int oracle_add(int dt, const void *lhs, const void *rhs, void *out, const size_t *md) {
+    if (dt < 0 || dt >= DT_COUNT) return -1;
+    const size_t n = md[0], nd = md[1], es = k_dtype_size[dt];
+    const size_t *ls = md + 2, *rs = md + 2 + nd, *lst = md + 2 + 2 * nd, *rst = md + 2 + 3 * nd;
+    const size_t lo = md[2 + 4 * nd], ro = md[2 + 4 * nd + 1];
+    const int ld = oracle_is_contiguous(nd, ls, lst), rd = oracle_is_contiguous(nd, rs, rst);
+    int bad = 0;
+    _Pragma("omp parallel for schedule(static) reduction(|:bad)")
+    for (size_t i = 0; i < n; i++) {
+        const size_t li = lo + (ld ? i : strided_pos(i, nd, ls, lst));
+        const size_t ri = ro + (rd ? i : strided_pos(i, nd, rs, rst));
+        bad |= ew_one(dt, EW_ADD, (const char *)lhs + li * es, (const char *)rhs + ri * es, (char *)out + i * es) != 0;
+    }
+    return bad ? -1 : 0;
+}
+
+/* hodu_cpu_mul_scalar_<dt>(in, out, metadata, scalar) and hodu_cpu_relu_<dt>(in, out, metadata); metadata =
+ * [num_els, nd, shape.., strides.., offset] (ops_unary.c:64-76).  `scalar` points at one element of dtype dt. */
+static int ew_unary(int dt, int op, const void *in, void *out, const size_t *md, const void *scalar) {
+    if (dt < 0 || dt >= DT_COUNT) return -1;
+    const size_t n = md[0], nd = md[1], es = k_dtype_size[dt];
+    const size_t *dims = md + 2, *strides = md + 2 + nd;
+    const size_t off = nd > 0 ? md[2 + 2 * nd] : 0;
+    const int dense = oracle_is_contiguous(nd, dims, strides);
+    int bad = 0;
+    _Pragma("omp parallel for schedule(static) reduction(|:bad)")
+    for (size_t i = 0; i < n; i++) {
+        const size_t pos = off + (dense ? i : strided_pos(i, nd, dims, strides));
+        bad |= ew_one(dt, op, (const char *)in + pos * es, scalar, (char *)out + i * es) != 0;
+    }
+    return bad ? -1 : 0;
+}
+int oracle_mul_scalar(int dt, const void *in, void *out, const size_t *md, const void *scalar) {
+    return ew_unary(dt, EW_MUL, in, out, md, scalar);
+}
+int oracle_relu(int dt, const void *in, void *out, const size_t *md) { return ew_unary(dt, EW_RELU, in, out, md, NULL); }
 
 /* ------------------------------------------------------------------------------------------ */
 /* single-thread timing entry points for the cpu_baseline (the reference runs batched / strided */

@@ -1,7 +1,7 @@
 """Writes the golden fixtures of this directory from the reference's own C kernels.
 
 Run in the build container only (needs oracle/_ref/libhodu_cpu_ref.so, i.e. `make -C oracle ref`,
-which compiles crates/hodu_cpu_kernels/kernels/{ops_matrix,ops_cast,ops_memory}.c where they lie
+which compiles crates/hodu_cpu_kernels/kernels/{ops_matrix,ops_cast,ops_memory,ops_binary,ops_unary}.c where they lie
 under /root/reference):
 
     python tests/golden/make_fixtures.py
@@ -188,6 +188,63 @@ def write_casts(ref):
     return len(names)
 
 
+ELEMENTWISE_FLOATS = ["f8e4m3", "f8e5m2", "bf16", "f16", "f32", "f64"]
+ELEMENTWISE_INTS = ["u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64"]
+
+
+def elementwise_input(dt, n, seed):
+    """values spread over the dtype's range, so that narrowing overflows, underflows and ties all occur"""
+    g = H.rng(seed)
+    if dt in ELEMENTWISE_INTS:
+        info = np.iinfo(oracle.STORAGE[dt])
+        return g.integers(info.min, info.max, n, dtype=info.dtype, endpoint=True)
+    mag = {"f8e4m3": 6.0, "f8e5m2": 12.0, "bf16": 30.0, "f16": 14.0, "f32": 30.0, "f64": 30.0}[dt]
+    x = g.standard_normal(n) * np.exp2(g.uniform(-mag, mag, n))
+    x[:: 37] = 0.0
+    if dt == "f64":
+        return x
+    if dt == "f32":
+        return x.astype(np.float32)
+    return cast_input_from_f32(dt, x.astype(np.float32))
+
+
+def cast_input_from_f32(dt, x):
+    md = H.cast_md(H.View([x.size]))
+    return oracle.RefLib().cast("f32", dt, np.clip(x, -3e38, 3e38), md)
+
+
+def write_elementwise(ref):
+    """add (a contiguous [.., M, N] plus a vector broadcast along the last axis -- what Linear::forward adds --,
+    and two contiguous operands), mul_scalar and relu of every dtype the reference defines them for"""
+    V = H.View
+    out, names = {}, []
+    for dt in ELEMENTWISE_FLOATS + ELEMENTWISE_INTS:
+        lv = V([3, 7, 19])
+        for tag, rv in (("bias", V([19], offset=2).broadcast_to([3, 7, 19])), ("bias_strided", V([19], [3], 1).broadcast_to([3, 7, 19])),
+                        ("full", V([3, 7, 19], offset=4))):
+            a, b = elementwise_input(dt, lv.span(), 11), elementwise_input(dt, rv.span(), 12)
+            md = np.array(H.binary_md(lv, rv), dtype=np.uint64)
+            key = f"add_{tag}__{dt}"
+            out[key + "__lhs"], out[key + "__rhs"], out[key + "__md"] = a, b, md
+            out[key + "__out"] = ref.add(dt, a, b, md)
+            names.append(f"{key}|add|{dt}")
+        x = elementwise_input(dt, 1024, 13)
+        md = np.array(H.cast_md(V([1024])), dtype=np.uint64)
+        for j, c in enumerate(elementwise_input(dt, 64, 14)[[3, 5, 8]]):
+            key = f"mul_scalar{j}__{dt}"
+            out[key + "__in"], out[key + "__md"], out[key + "__scalar"] = x, md, np.array([c], dtype=x.dtype)
+            out[key + "__out"] = ref.mul_scalar(dt, x, md, np.array([c], dtype=x.dtype))
+            names.append(f"{key}|mul_scalar|{dt}")
+        if dt in ELEMENTWISE_FLOATS:
+            key = f"relu__{dt}"
+            out[key + "__in"], out[key + "__md"] = x, md
+            out[key + "__out"] = ref.relu(dt, x, md)
+            names.append(f"{key}|relu|{dt}")
+    out["index"] = np.array(names)
+    np.savez_compressed(os.path.join(HERE, "elementwise.npz"), **out)
+    return len(names)
+
+
 def main():
     if not oracle.RefLib.available():
         raise SystemExit("oracle/_ref/libhodu_cpu_ref.so missing: run `make -C oracle ref` first")
@@ -195,7 +252,8 @@ def main():
     n = write_products(ref)
     write_tables(ref)
     m = write_casts(ref)
-    print(f"wrote {n} product cases, {m} cast/contiguous cases, tables")
+    e = write_elementwise(ref)
+    print(f"wrote {n} product cases, {m} cast/contiguous cases, {e} element-wise cases, tables")
 
 
 if __name__ == "__main__":

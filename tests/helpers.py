@@ -117,6 +117,12 @@ def cast_md(v: View):
     return [v.size, v.ndim] + v.shape + v.strides + [v.offset]
 
 
+def binary_md(lv: View, rv: View):
+    """binary_metadata of crates/hodu_core/src/op_metadatas.rs:36-73 (both operands already broadcast to one shape)"""
+    assert lv.shape == rv.shape
+    return [lv.size, lv.ndim] + lv.shape + rv.shape + lv.strides + rv.strides + [lv.offset, rv.offset]
+
+
 # ---------------------------------------------------------------------------------------------
 # narrow-float encoders used to GENERATE inputs (independent of the oracle's C code)
 # ---------------------------------------------------------------------------------------------

@@ -254,3 +254,67 @@ def test_reference_thread_policy():
     assert oracle.reference_threads(512, 256, 64) == 2
     assert oracle.reference_threads(2048, 256, 64) == 8
     assert oracle.reference_threads(4096, 128, 8) == 8
+
+
+# ---------------------------------------------------------------------------------------------
+# element-wise kernels the callers of the product run on its output (add, mul_scalar, relu)
+# ---------------------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def elementwise():
+    return np.load(os.path.join(GOLD, "elementwise.npz"))
+
+
+def _elementwise_got(ew, key, op, dt):
+    if op == "add":
+        return oracle.add(dt, ew[key + "__lhs"], ew[key + "__rhs"], ew[key + "__md"])
+    if op == "mul_scalar":
+        return oracle.mul_scalar(dt, ew[key + "__in"], ew[key + "__md"], ew[key + "__scalar"])
+    return oracle.relu(dt, ew[key + "__in"], ew[key + "__md"])
+
+
+def test_elementwise_bit_exact_vs_reference_fixtures(elementwise):
+    index = [s.split("|") for s in elementwise["index"]]
+    assert len(index) == 90
+    for key, op, dt in index:
+        got, want = _elementwise_got(elementwise, key, op, dt), elementwise[key + "__out"]
+        if dt in ("f32", "f64"):  # NaN payloads are not part of the contract
+            assert np.array_equal(np.isnan(got), np.isnan(want)), key
+            got, want = np.nan_to_num(got, nan=0.0), np.nan_to_num(want, nan=0.0)
+        assert np.array_equal(_bits(got), _bits(want)), key
+
+
+def test_elementwise_known_answers_of_the_reference_tests():
+    """crates/hodu_cpu_kernels/tests/ops_binary.rs:68-73, tests/ops_unary.rs:143-147, :503-507"""
+    one = lambda n: H.cast_md(H.View([n]))  # noqa: E731
+    f = lambda *v: np.array(v, dtype=np.float32)  # noqa: E731
+    md = H.binary_md(H.View([4]), H.View([4]))
+    assert np.array_equal(oracle.add("f32", f(1, 2, 3, 4), f(5, 6, 7, 8), md), f(6, 8, 10, 12))
+    assert np.array_equal(oracle.relu("f32", f(-2, -1, 0, 1, 2), one(5)), f(0, 0, 0, 1, 2))
+    assert np.array_equal(oracle.mul_scalar("f32", f(1, 2, 3, 4), one(4), f(3)), f(3, 6, 9, 12))
+
+
+def test_elementwise_against_independent_arithmetic():
+    """bf16: the exact f32 sum / product with its low 16 bits cut (kernels/t_bf16.h:35-39); integers: numpy's
+    modular arithmetic; relu: NaN and -0 become +0"""
+    g = H.rng(5)
+    a = g.integers(0, 1 << 16, 4096).astype(np.uint16)
+    b = g.integers(0, 1 << 16, 4096).astype(np.uint16)
+    a[(a & 0x7F80) == 0x7F80] = 0x3F80  # keep inf / NaN out of the random operands
+    b[(b & 0x7F80) == 0x7F80] = 0xBF80
+    af, bf = H.bf16_to_f32(a), H.bf16_to_f32(b)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = ((af + bf).view(np.uint32) >> 16).astype(np.uint16)
+    md = H.binary_md(H.View([4096]), H.View([4096]))
+    assert np.array_equal(oracle.add("bf16", a, b, md), want)
+    c = np.array([0x4049], dtype=np.uint16)  # 3.140625
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = ((af * H.bf16_to_f32(c)[0]).view(np.uint32) >> 16).astype(np.uint16)
+    assert np.array_equal(oracle.mul_scalar("bf16", a, H.cast_md(H.View([4096])), c), want)
+    x = g.integers(-2 ** 31, 2 ** 31, 4096).astype(np.int32)
+    y = g.integers(-2 ** 31, 2 ** 31, 4096).astype(np.int32)
+    assert np.array_equal(oracle.add("i32", x, y, md), (x.astype(np.int64) + y.astype(np.int64)).astype(np.int32))
+    s = np.array([-77777], dtype=np.int32)
+    assert np.array_equal(oracle.mul_scalar("i32", x, H.cast_md(H.View([4096])), s),
+                          (x.astype(np.int64) * int(s[0])).astype(np.int32))
+    r = oracle.relu("bf16", np.array([0x7FC0, 0x8000, 0xBF80, 0x3F80, 0xFF80, 0x7F80], dtype=np.uint16), H.cast_md(H.View([6])))
+    assert list(r) == [0, 0, 0, 0x3F80, 0, 0x7F80]

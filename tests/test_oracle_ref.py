@@ -67,3 +67,31 @@ def test_contiguous_matches_compiled_reference(ref):
         for dt in oracle.DTYPE_ID:
             x = H.random_storage(dt, v.span(), 5)
             assert np.array_equal(_bits(ref.contiguous(dt, x, H.cast_md(v))), _bits(oracle.contiguous(dt, x, H.cast_md(v))))
+
+
+ELEMENTWISE_DTYPES = [d for d in oracle.DTYPE_ID if d != "bool"]
+
+
+@pytest.mark.parametrize("dt", ELEMENTWISE_DTYPES)
+def test_elementwise_match_compiled_reference(ref, dt):
+    """add over every layout branch of the reference (both contiguous, one strided, both strided), mul_scalar and
+    relu, on fresh seeded values"""
+    V = H.View
+    full = V([5, 6, 33])
+    layouts = [(full, V([33], offset=1).broadcast_to([5, 6, 33])), (V([33]).broadcast_to([5, 6, 33]), full),
+               (full, V([5, 6, 33], offset=7)), (V([33, 6, 5]).t(0, 2), V([5, 1, 33], offset=2).broadcast_to([5, 6, 33]))]
+    floating = dt in ("f8e4m3", "f8e5m2", "bf16", "f16", "f32", "f64")
+    for n, (lv, rv) in enumerate(layouts):
+        a = H.random_storage(dt, lv.span(), 300 + n, 3.0)
+        b = H.random_storage(dt, rv.span(), 400 + n, 3.0)
+        md = H.binary_md(lv, rv)
+        assert np.array_equal(_bits(oracle.add(dt, a, b, md)), _bits(ref.add(dt, a, b, md))), (dt, n)
+    x = H.random_storage(dt, 200_000, 9, 3.0)  # above the reference's threading threshold (ops_unary.c:164)
+    md = H.cast_md(V([200_000]))
+    c = H.random_storage(dt, 8, 10, 3.0)[3:4]
+    assert np.array_equal(_bits(oracle.mul_scalar(dt, x, md, c)), _bits(ref.mul_scalar(dt, x, md, c))), dt
+    v = V([40, 50], offset=3).t()
+    assert np.array_equal(_bits(oracle.mul_scalar(dt, x, H.cast_md(v), c)), _bits(ref.mul_scalar(dt, x, H.cast_md(v), c))), dt
+    if floating:
+        assert np.array_equal(_bits(oracle.relu(dt, x, md)), _bits(ref.relu(dt, x, md))), dt
+        assert np.array_equal(_bits(oracle.relu(dt, x, H.cast_md(v))), _bits(ref.relu(dt, x, H.cast_md(v)))), dt
