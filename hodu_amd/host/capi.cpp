@@ -69,6 +69,29 @@ int hodu_host_tensor_to_bytes(const hodu_host_tensor *t, void *out, size_t nbyte
 int hodu_host_matmul(const hodu_host_tensor *a, const hodu_host_tensor *b, hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(T(a)->matmul(*T(b)))); });
 }
+// steps: n_steps entries of {op, operand tensor (add) or null, scalar bits (mul_scalar)}
+typedef struct hodu_host_then {
+    int op;
+    const hodu_host_tensor *operand;
+    unsigned char scalar[8];
+} hodu_host_then;
+int hodu_host_matmul_then(const hodu_host_tensor *a, const hodu_host_tensor *b, const hodu_host_then *steps, size_t n_steps,
+                          hodu_host_tensor **out) {
+    return guarded([&] {
+        std::vector<Tensor::Then> then(n_steps);
+        for (size_t i = 0; i < n_steps; i++) {
+            then[i].op = steps[i].op;
+            then[i].operand = T(steps[i].operand);
+            std::memcpy(then[i].scalar, steps[i].scalar, 8);
+        }
+        *out = H(box(T(a)->matmul_then(*T(b), then)));
+    });
+}
+int hodu_host_linear(const hodu_host_tensor *input, const hodu_host_tensor *weight, const hodu_host_tensor *bias, int relu,
+                     hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(Tensor::linear(*T(input), *T(weight), bias ? T(bias) : nullptr, relu != 0))); });
+}
+long hodu_host_stats_fused_steps(void) { return stats().fused_steps; }
 int hodu_host_dot(const hodu_host_tensor *a, const hodu_host_tensor *b, hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(T(a)->dot(*T(b)))); });
 }

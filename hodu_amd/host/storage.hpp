@@ -36,8 +36,9 @@ inline const char *dtype_name(DType d) {
 // Counters that let a caller (and the tests) see which device passes a Tensor-level call cost.
 struct Stats {
     std::atomic<long> cast_kernels{0}, contiguous_kernels{0}, product_kernels{0}, fused_products{0};
+    std::atomic<long> fused_steps{0};        // element-wise kernels that ran inside a product's store instead
     std::atomic<long long> bytes_copied{0};  // written by cast/contiguous passes
-    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = 0; bytes_copied = 0; }
+    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = 0; bytes_copied = 0; }
 };
 inline Stats &stats() {
     static Stats s;
@@ -97,6 +98,18 @@ private:
 // physical != dtype marks a deferred to_dtype: the cast has not run, and a following matmul/dot
 // reads the narrow elements directly (fused entry points of the C ABI).  Every other consumer
 // materialises first.  Deferred pairs: f8e4m3 -> bf16 and i8 -> i32.
+class RocmStorage;
+
+// An element-wise kernel the caller would launch on the product's output next, handed to the product instead
+// (hodu_nn/src/modules/linear.rs:40-46: add(bias); attention.rs:37: mul_scalar; activation.rs:8-17: relu).
+struct FusedStep {
+    int op = 0;                         // HODU_ROCM_EPI_*
+    const RocmStorage *vector = nullptr;  // ADD_ROW: storage of the operand, output dtype
+    size_t stride = 0, offset = 0;      // ADD_ROW: the operand's layout along the output's last axis
+    unsigned char scalar[8] = {0};      // MUL_SCALAR: the scalar in the output dtype
+};
+using FusedSteps = std::vector<FusedStep>;
+
 class RocmStorage {
 public:
     RocmStorage(std::shared_ptr<RocmDevice> dev, std::shared_ptr<DeviceBuf> buf, DType dtype, DType physical)
@@ -144,23 +157,24 @@ public:
     }
 
     // be_cpu/storage/ops_matrix.rs:24-185.  Output: fresh contiguous [batch.., M, N] in the logical dtype.
-    RocmStorage call_ops_matmul(const RocmStorage &rhs, const Layout &ll, const Layout &rl) const {
+    RocmStorage call_ops_matmul(const RocmStorage &rhs, const Layout &ll, const Layout &rl,
+                                const FusedSteps &fused = {}) const {
         check_pair(rhs, "matmul");
         check_span(ll, "matmul lhs");
         rhs.check_span(rl, "matmul rhs");
         Dims out_shape = matmul_out_shape(ll, rl);
         const Layout out_layout = Layout::from_shape(out_shape);
         const Metadata md = matmul_metadata(ll, rl, out_layout);
-        return product(rhs, ll, rl, md, out_layout.size(), true);
+        return product(rhs, ll, rl, md, out_layout.size(), true, fused);
     }
 
     // be_cpu/storage/ops_matrix.rs:201-321.  Output: fresh contiguous [M, N].
-    RocmStorage call_ops_dot(const RocmStorage &rhs, const Layout &ll, const Layout &rl) const {
+    RocmStorage call_ops_dot(const RocmStorage &rhs, const Layout &ll, const Layout &rl, const FusedSteps &fused = {}) const {
         check_pair(rhs, "dot");
         check_span(ll, "dot lhs");
         rhs.check_span(rl, "dot rhs");
         const Metadata md = dot_metadata(ll, rl);
-        return product(rhs, ll, rl, md, md[0] * md[2], false);
+        return product(rhs, ll, rl, md, md[0] * md[2], false, fused);
     }
 
     // be_cpu/storage/ops_matrix.rs:63-100: right-aligned broadcast of the batch dims, then [M, N]
@@ -240,10 +254,26 @@ private:
 #undef HODU_HOST_ENTRY
     }
 
+    using ProductFnEx = int (*)(hodu_rocm_ctx *, const void *, const void *, void *, const size_t *, size_t,
+                                const hodu_rocm_epilogue_step *, size_t);
+
+    static ProductFnEx fused_entry(DType dt, bool matmul) {
+#define HODU_HOST_ENTRY(DT, name) \
+    case DType::DT: return matmul ? hodu_rocm_matmul_##name##_ex : hodu_rocm_dot_##name##_ex;
+        switch (dt) {
+            HODU_HOST_ENTRY(BF16, bf16) HODU_HOST_ENTRY(F16, f16) HODU_HOST_ENTRY(F32, f32) HODU_HOST_ENTRY(F64, f64)
+            HODU_HOST_ENTRY(U8, u8) HODU_HOST_ENTRY(U16, u16) HODU_HOST_ENTRY(U32, u32) HODU_HOST_ENTRY(U64, u64)
+            HODU_HOST_ENTRY(I8, i8) HODU_HOST_ENTRY(I16, i16) HODU_HOST_ENTRY(I32, i32) HODU_HOST_ENTRY(I64, i64)
+            default: throw Error(ErrorKind::UnsupportedDTypeForOp, "products of this dtype take no fused steps");
+        }
+#undef HODU_HOST_ENTRY
+    }
+
     RocmStorage product(const RocmStorage &rhs, const Layout &ll, const Layout &rl, const Metadata &md, size_t out_elems,
-                        bool matmul) const {
+                        bool matmul, const FusedSteps &fused) const {
         RocmStorage out = fresh(dtype_, out_elems);
         if (out_elems == 0) return out;
+        if (!fused.empty()) return product_fused(rhs, md, matmul, fused, out);
         ProductFn fn = nullptr;
         const RocmStorage *l = this, *r = &rhs;
         RocmStorage lm = *this, rm = rhs;  // materialised copies, used only when a deferred operand cannot be fused
@@ -267,6 +297,53 @@ private:
         if (fn == hodu_rocm_matmul_bf16_f8e4m3w || fn == hodu_rocm_dot_bf16_f8e4m3w || fn == hodu_rocm_matmul_i32_i8i8 ||
             fn == hodu_rocm_dot_i32_i8i8)
             stats().fused_products++;
+        return out;
+    }
+
+    // the product with the caller's next element-wise kernels applied in its store; deferred casts fuse as well
+    RocmStorage product_fused(const RocmStorage &rhs, const Metadata &md, bool matmul, const FusedSteps &fused,
+                              RocmStorage out) const {
+        std::vector<hodu_rocm_epilogue_step> steps(fused.size());
+        std::vector<RocmStorage> keep;  // operands whose pending cast had to be run first
+        keep.reserve(fused.size());
+        for (size_t i = 0; i < fused.size(); i++) {
+            steps[i] = hodu_rocm_epilogue_step{};
+            steps[i].op = fused[i].op;
+            if (fused[i].op == HODU_ROCM_EPI_ADD_ROW) {
+                const RocmStorage *v = fused[i].vector;
+                if (!v) throw Error(ErrorKind::InvalidArgument, "fused add: no operand");
+                if (v->dev_->id() != dev_->id()) throw Error(ErrorKind::DeviceMismatch, "fused add: operand on another device");
+                if (v->dtype_ != dtype_)
+                    throw Error(ErrorKind::DTypeMismatch, std::string("fused add: ") + dtype_name(dtype_) + " vs " + dtype_name(v->dtype_));
+                if (v->deferred()) {
+                    keep.push_back(RocmStorage(v->dev_, v->buf_, v->physical_, v->physical_).cast_kernel(Layout::from_shape({v->elems()}), v->dtype_));
+                    v = &keep.back();
+                }
+                steps[i].vector = v->ptr();
+                steps[i].stride = fused[i].stride;
+                steps[i].offset = fused[i].offset;
+            }
+            std::memcpy(steps[i].scalar, fused[i].scalar, 8);
+        }
+        ProductFnEx fn = nullptr;
+        const RocmStorage *l = this, *r = &rhs;
+        RocmStorage lm = *this, rm = rhs;
+        bool fused_cast = true;
+        if (!deferred() && dtype_ == DType::BF16 && rhs.deferred() && rhs.physical_ == DType::F8E4M3) {
+            fn = matmul ? hodu_rocm_matmul_bf16_f8e4m3w_ex : hodu_rocm_dot_bf16_f8e4m3w_ex;
+        } else if (deferred() && rhs.deferred() && physical_ == DType::I8 && rhs.physical_ == DType::I8) {
+            fn = matmul ? hodu_rocm_matmul_i32_i8i8_ex : hodu_rocm_dot_i32_i8i8_ex;
+        } else {
+            fused_cast = false;
+            if (deferred()) { lm = RocmStorage(dev_, buf_, physical_, physical_).cast_kernel(Layout::from_shape({elems()}), dtype_); l = &lm; }
+            if (rhs.deferred()) { rm = RocmStorage(rhs.dev_, rhs.buf_, rhs.physical_, rhs.physical_).cast_kernel(Layout::from_shape({rhs.elems()}), rhs.dtype_); r = &rm; }
+            fn = fused_entry(dtype_, matmul);
+        }
+        dev_->check(fn(dev_->ctx(), l->ptr(), r->ptr(), (void *)out.ptr(), md.data(), md.size(), steps.data(), steps.size()),
+                    matmul ? "matmul" : "dot");
+        stats().product_kernels++;
+        stats().fused_steps += (long)fused.size();
+        if (fused_cast) stats().fused_products++;
         return out;
     }
 

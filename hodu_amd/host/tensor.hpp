@@ -100,7 +100,77 @@ public:
         throw Error(ErrorKind::InternalError, "dot - only supports 1D and 2D tensors. Use matmul() for batched operations");
     }
 
+    // ---- the product with its caller's next element-wise kernels fused in --------------------------------
+    // What follows the product in hodu_nn: Linear::forward adds the bias (linear.rs:40-46), attention scales
+    // the scores (attention.rs:37), ReLU follows a Linear (activation.rs:8-17).  Each Then is one such kernel,
+    // applied in order inside the product's store; the result equals matmul(..) followed by Tensor::add /
+    // mul_scalar / relu bit for bit.  Both operands must have at least two dimensions.
+    struct Then {
+        int op = 0;                    // HODU_ROCM_EPI_*
+        const Tensor *operand = nullptr;  // add: a tensor that broadcasts to the output along its last axis only
+        unsigned char scalar[8] = {0};    // mul_scalar: the scalar's bits in the output dtype (Scalar::to_dtype)
+        static Then add(const Tensor &bias) { Then t; t.op = HODU_ROCM_EPI_ADD_ROW; t.operand = &bias; return t; }
+        static Then mul_scalar(const void *bits, size_t n) {
+            Then t; t.op = HODU_ROCM_EPI_MUL_SCALAR;
+            std::memcpy(t.scalar, bits, n < 8 ? n : 8);
+            return t;
+        }
+        static Then relu() { Then t; t.op = HODU_ROCM_EPI_RELU; return t; }
+    };
+
+    Tensor matmul_then(const Tensor &other, const std::vector<Then> &then) const {
+        const size_t ln = layout_.ndim(), rn = other.layout_.ndim();
+        if (ln < 2 || rn < 2)
+            throw Error(ErrorKind::InvalidArgument, "matmul with fused steps needs operands of at least two dimensions");
+        if (ln == 2 && rn == 2) return dot_2d(other, &then);
+        return matmul_batched(other, &then);
+    }
+
+    // Linear::forward (hodu_nn/src/modules/linear.rs:40-46): input @ weight.T (+ bias); weight is [out, in]
+    static Tensor linear(const Tensor &input, const Tensor &weight, const Tensor *bias, bool relu = false) {
+        std::vector<Then> then;
+        if (bias) then.push_back(Then::add(*bias));
+        if (relu) then.push_back(Then::relu());
+        const Tensor wt = weight.transpose(-2, -1);
+        if (then.empty() || input.layout().ndim() < 2) {
+            if (!then.empty()) throw Error(ErrorKind::InvalidArgument, "linear: a 1-D input takes no fused steps");
+            return input.matmul(wt);
+        }
+        return input.matmul_then(wt, then);
+    }
+
 private:
+    // tensor/utils.rs broadcast_tensors2 as Tensor::add applies it to (output, operand): the operand's shape is
+    // right-aligned against the output's; a fused add needs every axis but the last to be broadcast (extent 1
+    // or missing), so that the operand is a vector along the output's last axis
+    FusedSteps lower(const std::vector<Then> &then, const Dims &out_shape) const {
+        FusedSteps steps;
+        for (const Then &t : then) {
+            FusedStep f;
+            f.op = t.op;
+            std::memcpy(f.scalar, t.scalar, 8);
+            if (t.op == HODU_ROCM_EPI_ADD_ROW) {
+                if (!t.operand) throw Error(ErrorKind::InvalidArgument, "fused add: no operand");
+                const Layout &bl = t.operand->layout();
+                const size_t bn = bl.ndim(), on = out_shape.size();
+                if (bn > on) throw Error(ErrorKind::IncompatibleShapes, "fused add: " + dims_str(out_shape) + " vs " + dims_str(bl.shape()));
+                for (size_t i = 0; i < bn; i++) {
+                    const size_t ext = bl.shape()[bn - 1 - i], want = out_shape[on - 1 - i];
+                    if (i == 0 ? (ext != want && ext != 1) : ext != 1)
+                        throw Error(ErrorKind::IncompatibleShapes,
+                                    "fused add: the operand must be a vector along the last axis: " + dims_str(out_shape) + " vs " + dims_str(bl.shape()));
+                }
+                if (bl.span() > t.operand->storage_->elems())
+                    throw Error(ErrorKind::InvalidLayout, "fused add: operand layout reaches past its storage");
+                f.vector = t.operand->storage_.get();
+                f.stride = bn == 0 || bl.shape()[bn - 1] == 1 ? 0 : bl.strides()[bn - 1];
+                f.offset = bl.offset();
+            }
+            steps.push_back(f);
+        }
+        return steps;
+    }
+
     Error incompatible(const Tensor &o, const char *op) const {
         return Error(ErrorKind::IncompatibleShapes, std::string(op) + ": " + dims_str(shape()) + " vs " + dims_str(o.shape()));
     }
@@ -115,14 +185,15 @@ private:
     }
 
     // matrix.rs:302-371: both layouts go to the kernel unchanged
-    Tensor dot_2d(const Tensor &other) const {
+    Tensor dot_2d(const Tensor &other, const std::vector<Then> *then = nullptr) const {
         if (shape()[1] != other.shape()[0]) throw incompatible(other, "dot");
-        auto out = std::make_shared<RocmStorage>(storage_->call_ops_dot(*other.storage_, layout_, other.layout_));
+        const FusedSteps fused = then ? lower(*then, {shape()[0], other.shape()[1]}) : FusedSteps{};
+        auto out = std::make_shared<RocmStorage>(storage_->call_ops_dot(*other.storage_, layout_, other.layout_, fused));
         return Tensor(out, Layout::from_shape({shape()[0], other.shape()[1]}));
     }
 
     // matrix.rs:95-224
-    Tensor matmul_batched(const Tensor &other) const {
+    Tensor matmul_batched(const Tensor &other, const std::vector<Then> *then = nullptr) const {
         const Dims &ld = shape(), &rd = other.shape();
         const size_t ln = ld.size(), rn = rd.size();
         if (ln < 2 || rn < 2 || ld[ln - 1] != rd[rn - 2]) throw incompatible(other, "matmul");
@@ -142,7 +213,8 @@ private:
         Dims out_shape = batch;
         out_shape.push_back(ld[ln - 2]);
         out_shape.push_back(rd[rn - 1]);
-        auto out = std::make_shared<RocmStorage>(l.storage_->call_ops_matmul(*r.storage_, l.layout_, r.layout_));
+        const FusedSteps fused = then ? lower(*then, out_shape) : FusedSteps{};
+        auto out = std::make_shared<RocmStorage>(l.storage_->call_ops_matmul(*r.storage_, l.layout_, r.layout_, fused));
         return Tensor(out, Layout::from_shape(out_shape));
     }
 

@@ -31,6 +31,10 @@ class HoduError(RuntimeError):
         super().__init__(f"{self.kind}: {message}")
 
 
+class _Then(ctypes.Structure):
+    _fields_ = [("op", ctypes.c_int), ("operand", ctypes.c_void_p), ("scalar", ctypes.c_ubyte * 8)]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -56,6 +60,9 @@ def load() -> ctypes.CDLL:
     lib.hodu_host_tensor_to_bytes.argtypes = [vp, vp, sz]
     lib.hodu_host_matmul.argtypes = [vp, vp, vpp]
     lib.hodu_host_dot.argtypes = [vp, vp, vpp]
+    lib.hodu_host_matmul_then.argtypes = [vp, vp, ctypes.POINTER(_Then), sz, vpp]
+    lib.hodu_host_linear.argtypes = [vp, vp, vp, ci, vpp]
+    lib.hodu_host_stats_fused_steps.restype = ctypes.c_long
     lib.hodu_host_to_dtype.argtypes = [vp, ci, vpp]
     lib.hodu_host_contiguous.argtypes = [vp, vpp]
     lib.hodu_host_transpose.argtypes = [vp, ci, ci, vpp]
@@ -88,10 +95,11 @@ def stats(reset: bool = False) -> dict:
     lib = load()
     a, b, c, d, e = (ctypes.c_long(), ctypes.c_long(), ctypes.c_long(), ctypes.c_long(), ctypes.c_longlong())
     lib.hodu_host_stats(a, b, c, d, e)
+    fused_steps = int(lib.hodu_host_stats_fused_steps())
     if reset:
         lib.hodu_host_stats_reset()
     return {"cast_kernels": a.value, "contiguous_kernels": b.value, "product_kernels": c.value,
-            "fused_products": d.value, "bytes_copied": e.value}
+            "fused_products": d.value, "bytes_copied": e.value, "fused_steps": fused_steps}
 
 
 class Tensor:
@@ -160,6 +168,25 @@ class Tensor:
     def matmul(self, other: "Tensor") -> "Tensor":
         return self._unary(load().hodu_host_matmul, other._h)
 
+    def matmul_then(self, other: "Tensor", steps) -> "Tensor":
+        """matmul with the caller's next element-wise kernels applied inside its store.  steps: a list of
+        ("add", tensor) -- a bias along the last axis, as Linear::forward adds it --, ("mul_scalar", bits) -- the
+        scalar as a 1-element array in the tensor dtype's storage -- and ("relu",)."""
+        arr = (_Then * max(1, len(steps)))()
+        for i, step in enumerate(steps):
+            if step[0] == "add":
+                arr[i].op, arr[i].operand = 1, step[1]._h
+            elif step[0] == "mul_scalar":
+                raw = np.ascontiguousarray(step[1]).reshape(1).tobytes()
+                arr[i].op = 2
+                arr[i].scalar = (ctypes.c_ubyte * 8)(*raw, *([0] * (8 - len(raw))))
+            elif step[0] == "relu":
+                arr[i].op = 3
+            else:
+                raise ValueError(f"unknown fused step {step[0]!r}")
+        out = ctypes.c_void_p()
+        return self._wrap(load().hodu_host_matmul_then(self._h, other._h, arr, len(steps), ctypes.byref(out)), out)
+
     def dot(self, other: "Tensor") -> "Tensor":
         return self._unary(load().hodu_host_dot, other._h)
 
@@ -194,3 +221,21 @@ class Tensor:
     def view(self, shape: Sequence[int], strides: Sequence[int], offset: int = 0) -> "Tensor":
         """an arbitrary strided view over the same storage (what chained view ops produce)"""
         return self._unary(load().hodu_host_view, _sizes(shape), _sizes(strides), len(shape), offset)
+
+
+class Linear:
+    """hodu_nn's Linear (crates/hodu_nn/src/modules/linear.rs:4-57): weight [out_features, in_features], optional
+    bias [out_features]; forward(input) = input @ weight.T + bias, as ONE launch (the bias add -- and a ReLU that
+    follows, if asked for -- run inside the product's store)."""
+
+    def __init__(self, weight: Tensor, bias: Optional[Tensor] = None):
+        self.weight, self.bias = weight, bias
+
+    def forward(self, x: Tensor, relu: bool = False) -> Tensor:
+        out = ctypes.c_void_p()
+        rc = load().hodu_host_linear(x._h, self.weight._h, self.bias._h if self.bias is not None else None, int(relu),
+                                     ctypes.byref(out))
+        return Tensor._wrap(rc, out)
+
+    def parameters(self):
+        return [self.weight] + ([self.bias] if self.bias is not None else [])

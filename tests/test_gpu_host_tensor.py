@@ -197,3 +197,107 @@ def test_to_dtype_of_a_view_matches_the_cast_oracle():
     assert got.layout() == ([m, n], [n, 1], 0) and np.array_equal(got.to_bits(), want)  # truncating f32 -> bf16
     same = t.to_dtype("f32")  # same dtype: contiguous()
     assert np.array_equal(same.to_bits().view(np.float32), xs.reshape(n, m).T.ravel())
+
+
+# ---- the product with its caller's next element-wise kernels fused in ------------------------------------
+def _oracle_after(dt, plain_bits, out_shape, steps):
+    """hodu_cpu_add / mul_scalar / relu (the oracle's restatement) applied to the plain product's output"""
+    V = H.View
+    x = plain_bits.view(oracle.STORAGE[dt])
+    for step in steps:
+        if step[0] == "add":
+            bias_bits, bias_view = step[1], step[2]
+            x = oracle.add(dt, x, bias_bits.view(oracle.STORAGE[dt]), H.binary_md(V(out_shape), bias_view.broadcast_to(out_shape)))
+        elif step[0] == "mul_scalar":
+            x = oracle.mul_scalar(dt, x, H.cast_md(V(out_shape)), step[1].view(oracle.STORAGE[dt]))
+        else:
+            x = oracle.relu(dt, x, H.cast_md(V(out_shape)))
+    return x.view(plain_bits.dtype)
+
+
+def test_linear_layer_equals_matmul_then_add():
+    """Linear::forward (hodu_nn/src/modules/linear.rs:40-46): 3-D input, [out, in] weight, bias -- one launch, and the
+    bits of matmul followed by add"""
+    V = H.View
+    g = H.rng(11)
+    x = H.f32_to_bf16_rne(g.standard_normal(2 * 5 * 64).astype(np.float32))
+    w = H.f32_to_bf16_rne((g.standard_normal(24 * 64) / 8).astype(np.float32))
+    b = H.f32_to_bf16_rne(g.standard_normal(24).astype(np.float32))
+    tx, tw, tb = (T.Tensor.from_bits(x, "bf16", [2, 5, 64]), T.Tensor.from_bits(w, "bf16", [24, 64]),
+                  T.Tensor.from_bits(b, "bf16", [24]))
+    plain = tx.matmul(tw.t()).to_bits()
+    T.stats(reset=True)
+    layer = T.Linear(tw, tb)
+    got = layer.forward(tx)
+    s = T.stats()
+    assert got.shape == [2, 5, 24] and s["product_kernels"] == 1 and s["fused_steps"] == 1
+    assert np.array_equal(got.to_bits(), _oracle_after("bf16", plain, [2, 5, 24], [("add", b, V([24]))]))
+    got = layer.forward(tx, relu=True).to_bits()
+    assert np.array_equal(got, _oracle_after("bf16", plain, [2, 5, 24], [("add", b, V([24])), ("relu",)]))
+    assert np.array_equal(T.Linear(tw).forward(tx).to_bits(), plain)  # no bias: the plain product
+    assert [p.shape for p in layer.parameters()] == [[24, 64], [24]]
+
+
+def test_linear_layer_with_deferred_f8_weight():
+    """x.matmul(w8.to_dtype(bf16).t()) + bias: cast, product and add in one launch (config 3 as a layer)"""
+    V = H.View
+    g = H.rng(12)
+    x = H.f32_to_bf16_rne(g.standard_normal(16 * 512).astype(np.float32))
+    w8 = H.f32_to_ocp_e4m3_rne(g.standard_normal(300 * 512) * 4)
+    b = H.f32_to_bf16_rne(g.standard_normal(300).astype(np.float32))
+    tx, tb = T.Tensor.from_bits(x, "bf16", [16, 512]), T.Tensor.from_bits(b, "bf16", [300])
+    tw = T.Tensor.from_bits(w8, "f8e4m3", [300, 512]).to_dtype("bf16")
+    assert tw.physical_dtype == "f8e4m3"
+    plain = tx.matmul(tw.t()).to_bits()
+    T.stats(reset=True)
+    got = T.Linear(tw, tb).forward(tx)
+    s = T.stats()
+    assert s == {"cast_kernels": 0, "contiguous_kernels": 0, "product_kernels": 1, "fused_products": 1, "bytes_copied": 0,
+                 "fused_steps": 1}
+    assert np.array_equal(got.to_bits(), _oracle_after("bf16", plain, [16, 300], [("add", b, V([300]))]))
+
+
+def test_matmul_then_scale_and_strided_bias():
+    """attention.rs:37 scales the scores; a bias that is a strided slice of a larger tensor, or a [1, N] row, or one
+    value, broadcasts the way Tensor::add broadcasts it"""
+    V = H.View
+    g = H.rng(13)
+    q = g.standard_normal(3 * 10 * 32).astype(np.float32)
+    k = g.standard_normal(3 * 12 * 32).astype(np.float32)
+    tq, tk = from_f32(q, [3, 10, 32]), from_f32(k, [3, 12, 32])
+    plain = tq.matmul(tk.t()).to_bits()
+    scale = np.array([1.0 / np.sqrt(32.0)], dtype=np.float32)
+    got = tq.matmul_then(tk.t(), [("mul_scalar", scale)]).to_bits()
+    assert np.array_equal(got, _oracle_after("f32", plain, [3, 10, 12], [("mul_scalar", scale.view(np.uint32))]))
+    big = g.standard_normal(40).astype(np.float32)
+    tbig = from_f32(big, [40])
+    sl = tbig.slice(0, 3, 39, 3)  # 12 entries, stride 3, offset 3
+    want = _oracle_after("f32", plain, [3, 10, 12], [("add", big.view(np.uint32), V([12], [3], 3))])
+    assert np.array_equal(tq.matmul_then(tk.t(), [("add", sl)]).to_bits(), want)
+    row = from_f32(big[:12], [1, 12])
+    want = _oracle_after("f32", plain, [3, 10, 12], [("add", big[:12].view(np.uint32), V([1, 12]))])
+    assert np.array_equal(tq.matmul_then(tk.t(), [("add", row)]).to_bits(), want)
+    one = from_f32(big[5:6], [1])
+    want = _oracle_after("f32", plain, [3, 10, 12], [("add", big[5:6].view(np.uint32), V([1]))])
+    assert np.array_equal(tq.matmul_then(tk.t(), [("add", one)]).to_bits(), want)
+
+
+def test_matmul_then_rejects_what_add_would_not_broadcast_along_the_last_axis():
+    a, b = from_f32(np.ones(6), [2, 3]), from_f32(np.ones(12), [3, 4])
+    with pytest.raises(T.HoduError) as e:
+        a.matmul_then(b, [("add", from_f32(np.ones(2), [2, 1]))])  # a column: a real add kernel's job
+    assert e.value.kind == "IncompatibleShapes"
+    with pytest.raises(T.HoduError) as e:
+        a.matmul_then(b, [("add", from_f32(np.ones(5), [5]))])
+    assert e.value.kind == "IncompatibleShapes"
+    with pytest.raises(T.HoduError) as e:
+        a.matmul_then(b, [("add", T.Tensor.from_bits(np.ones(4, np.uint16), "bf16", [4]))])
+    assert e.value.kind == "DTypeMismatch"
+    with pytest.raises(T.HoduError) as e:
+        from_f32(np.ones(3), [3]).matmul_then(b, [("relu",)])
+    assert e.value.kind == "InvalidArgument"
+    i = T.Tensor.from_bits(np.ones(6, np.uint32), "i32", [2, 3])
+    j = T.Tensor.from_bits(np.ones(12, np.uint32), "i32", [3, 4])
+    with pytest.raises(T.HoduError) as e:
+        i.matmul_then(j, [("relu",)])
+    assert e.value.kind == "RocmKernelError"
