@@ -211,6 +211,26 @@ def time_case(ctx, case, steps, warmup, graph=False):
             "tflops": tflops, "algorithmic_gbs": gbs, "weight_buffers_rotated": copies, "roofline": roof}
 
 
+def mfma_clock_probe(ctx):
+    """what the matrix cores sustain from registers (no LDS, no memory traffic), and at which shader clock, on
+    constant and on N(0,1) operands: the clock under full MFMA load depends on the data"""
+    import helpers as H
+    out = []
+    for kind, name, peak in ((0, "bf16 32x32x16", PEAK["bf16"]), (1, "f8e4m3 32x32x64 (unit scales)", PEAK["fp8"])):
+        for data in ("constant", "normal"):
+            if kind == 0:
+                bits = bf16(np.full(8192, 0.0111, dtype=np.float32) if data == "constant" else normal(900, 8192))
+            else:
+                vals = np.full(16384, 0.5, dtype=np.float32) if data == "constant" else normal(901, 16384)
+                bits = H.f32_to_ocp_e4m3_rne(np.clip(vals, -448, 448))
+            buf = ctx.upload(bits)
+            r = ctx.mfma_clock(kind, buf, 20000)
+            buf.free()
+            out.append({"instruction": name, "operands": data, "tflops": r["tflops"], "shader_mhz": r["shader_mhz"],
+                        "frac_of_datasheet_peak": r["tflops"] / peak})
+    return out
+
+
 def cpu_baseline_c2(budget_s=15.0):
     """hodu's CPU path for config 2, timed on a bounded sample.
 
@@ -297,6 +317,10 @@ def main():
                           "launches": args.steps}))
         ctx.close()
         return
+    if args.only == "clock":
+        print(json.dumps({"config": "clock", "register_only_mfma": mfma_clock_probe(ctx)}))
+        ctx.close()
+        return
     if args.only:
         case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "fused"}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
@@ -333,6 +357,9 @@ def main():
                    "flop_per_step": case2.flops, "algorithmic_bytes_per_step": case2.alg_bytes},
         "roofline": {k: head["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
         "dominant_kernel": head["kernel"],
+        # not part of the roofline (whose peak is the datasheet's): the rate a register-only MFMA loop sustains on
+        # this box, by operand data
+        "register_only_mfma": mfma_clock_probe(ctx),
         "device": info,
         "all_configs": results,
     }

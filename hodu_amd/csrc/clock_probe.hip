@@ -1,0 +1,106 @@
+// Measurement hook: what the matrix cores sustain when nothing else is in the way, and at which shader clock.
+//
+// A register-only loop of MFMAs (no LDS, no memory traffic inside the loop) on operand bits the caller supplies,
+// two workgroups of four wavefronts on every compute unit.  One wavefront reads the shader-clock counter
+// (s_memtime) and the constant 100 MHz counter (s_memrealtime) before and after its loop; their ratio is the clock
+// the wavefront ran at.  On this part the clock under full MFMA load depends on the operand data (how many
+// multiplier inputs toggle): the rate this probe reports for N(0,1) operands, not the datasheet peak, is what a
+// GEMM kernel can approach.
+#include "common.hpp"
+#include "device_types.hpp"
+
+namespace hodu {
+namespace {
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// KIND 0: v_mfma_f32_32x32x16_bf16; KIND 1: v_mfma_scale_f32_32x32x64_f8f6f4 on f8e4m3 with unit scales
+template <int KIND>
+__global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restrict__ operands, float *__restrict__ sink,
+                                                        unsigned long long *__restrict__ clocks, int iters) {
+    constexpr int NACC = 4;
+    const int t = threadIdx.x;
+    const u32x4_t a0 = operands[t], b0 = operands[256 + t], a1 = operands[512 + t], b1 = operands[768 + t];
+    f32x16_t acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; i++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[i][e] = 0.f;
+    const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < NACC; i++) {
+            if constexpr (KIND == 0) {
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, b0),
+                                                                 acc[i], 0, 0, 0);
+            } else {
+                const i32x8_t a = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                const i32x8_t b = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i], 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+            }
+        }
+    }
+    const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    f32x16_t s = acc[0];
+#pragma unroll
+    for (int i = 1; i < NACC; i++) s += acc[i];
+    float v = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) v += s[e];
+    sink[blockIdx.x * 256 + t] = v;
+    if (blockIdx.x == 0 && t == 0) {
+        clocks[0] = c1 - c0;
+        clocks[1] = r1 - r0;
+    }
+}
+
+}  // namespace
+}  // namespace hodu
+
+using namespace hodu;
+
+extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
+                                          double *tflops, double *shader_mhz) {
+    clear_error();
+    if (!ctx || !operands || iters <= 0 || !elapsed_ms || !tflops || !shader_mhz || kind < 0 || kind > 1)
+        return fail(HODU_ROCM_INVALID_ARG, "mfma_clock: bad argument");
+    HODU_HIP(hipSetDevice(ctx->device));
+    const unsigned blocks = 2u * (unsigned)ctx->props.multiProcessorCount;
+    float *sink = nullptr;
+    unsigned long long *clocks = nullptr;
+    HODU_HIP(hipMalloc((void **)&sink, (size_t)blocks * 256 * sizeof(float)));
+    if (hipMalloc((void **)&clocks, 16) != hipSuccess) {
+        (void)hipFree(sink);
+        return fail(HODU_ROCM_OOM, "mfma_clock: out of memory");
+    }
+    auto launch = [&](int n) {
+        if (kind == 0)
+            hipLaunchKernelGGL(mfma_clock_kernel<0>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
+        else
+            hipLaunchKernelGGL(mfma_clock_kernel<1>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
+    };
+    hipEvent_t t0, t1;
+    hipError_t e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    if (e == hipSuccess) {
+        launch(iters / 10 + 1);  // warm-up: the clock settles
+        launch(iters / 10 + 1);
+        e = hipEventRecord(t0, ctx->stream);
+        launch(iters);
+        if (e == hipSuccess) e = hipEventRecord(t1, ctx->stream);
+        if (e == hipSuccess) e = hipEventSynchronize(t1);
+        if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+    }
+    unsigned long long h[2] = {0, 0};
+    if (e == hipSuccess) e = hipMemcpy(h, clocks, 16, hipMemcpyDeviceToHost);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipFree(sink);
+    (void)hipFree(clocks);
+    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "mfma_clock: %s", hipGetErrorString(e));
+    // flop per MFMA: 32 x 32 x k x 2 with k = 16 (bf16) or 64 (f8)
+    const double per_mfma = kind == 0 ? 32768.0 : 131072.0;
+    *tflops = (double)blocks * 4 /* wavefronts */ * 4 /* accumulators */ * (double)iters * per_mfma / (*elapsed_ms * 1e-3) / 1e12;
+    *shader_mhz = h[1] ? (double)h[0] / (double)h[1] * 100.0 : 0.0;
+    return HODU_ROCM_OK;
+}

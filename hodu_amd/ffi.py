@@ -114,6 +114,8 @@ def load() -> ctypes.CDLL:
             getattr(lib, f"hodu_rocm_{op}_{dt}_ex").argtypes = [vp, vp, vp, vp, szp, sz, ctypes.POINTER(EpilogueStep), sz]
     lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz,
                                                     ctypes.POINTER(EpilogueStep), sz, ci, ctypes.POINTER(ctypes.c_float)]
+    lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, ctypes.POINTER(ctypes.c_float),
+                                               ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     _lib = lib
@@ -299,6 +301,15 @@ class Context:
         self._check(fn(self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr,
                        n, int(iters), ctypes.byref(ms)))
         return float(ms.value)
+
+    def mfma_clock(self, kind: int, operands: DeviceBuffer, iters: int = 20000) -> dict:
+        """register-only MFMA loop on the given operand bits (16 KB): sustained TFLOP/s and shader clock"""
+        if operands.nbytes < 16384:
+            raise HoduRocmError(INVALID_ARG, "mfma_clock: operands must hold 16 KB")
+        ms, tf, mhz = ctypes.c_float(), ctypes.c_double(), ctypes.c_double()
+        self._check(self.lib.hodu_rocm_debug_mfma_clock(self.handle, int(kind), operands.ptr, int(iters), ctypes.byref(ms),
+                                                        ctypes.byref(tf), ctypes.byref(mhz)))
+        return {"ms": ms.value, "tflops": tf.value, "shader_mhz": mhz.value}
 
     def force_tile(self, tile: int):
         """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, 10..14 the pipelined

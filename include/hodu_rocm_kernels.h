@@ -105,6 +105,15 @@ int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int ki
                                        const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
                                        size_t metadata_len, int iters, float *elapsed_ms);
 
+/* measurement hook: the rate and shader clock of a register-only MFMA loop (no LDS, no memory traffic) on
+ * caller-supplied operand bits, two workgroups per compute unit.  kind 0: bf16 32x32x16; kind 1: f8e4m3 32x32x64
+ * with unit scales.  `operands`: 16 KB of device memory (1024 x 16 bytes: per lane the a and b fragments, twice).
+ * *tflops is what the loop sustained, *shader_mhz the clock one wavefront saw (shader-clock counter over the
+ * 100 MHz counter).  Under full MFMA load the clock depends on the data, so this is the ceiling a GEMM kernel can
+ * approach on that data. */
+int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
+                               double *tflops, double *shader_mhz);
+
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>
  * (kernels/ops_matrix.c:423, :581).  Narrow floats accumulate in f32 and round once on store.   */
