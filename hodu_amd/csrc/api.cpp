@@ -304,6 +304,19 @@ int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *o
     return launch_cast(ctx, src, dst, in, out, s);
 }
 
+int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "sum: context is null");
+    if (!in || !out) return fail(HODU_ROCM_INVALID_ARG, "sum: null operand pointer");
+    if (in == out) return fail(HODU_ROCM_INVALID_ARG, "sum: out aliases the input");
+    if (dtype_size(dtype) == 0 || dtype == HODU_BOOL) return fail(HODU_ROCM_UNSUPPORTED, "sum: dtype id %d has no sum kernel", dtype);
+    Reduction r;
+    int rc = parse_reduce_metadata(md, len, &r);
+    if (rc) return rc;
+    HODU_HIP(hipSetDevice(ctx->device));
+    return launch_sum(ctx, dtype, in, out, r);
+}
+
 int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "contiguous: context is null");

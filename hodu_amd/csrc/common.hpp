@@ -151,6 +151,20 @@ int launch_gemv(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const vo
 int launch_skinny(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                   const DevProduct &g);
 
+// A sum over some dims of a strided tensor, as the reference's reduce metadata describes it: the dims that stay
+// (in input order: that is the row-major order of the output, kept extent-1 dims included or not) and the dims
+// that are summed, each list with extents and element strides, adjacent dims merged where the strides allow.
+struct Reduction {
+    long n_out = 1;       // output elements
+    long reduce_size = 1; // inputs per output
+    int kept_n = 0, red_n = 0;
+    long kept_shape[16], kept_stride[16];
+    long red_shape[16], red_stride[16];
+    long offset = 0;
+};
+int parse_reduce_metadata(const size_t *md, size_t len, Reduction *r);
+int launch_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r);
+
 int launch_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const Strided &s);
 int launch_gather(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Strided &s);
 

@@ -146,4 +146,60 @@ int parse_cast_metadata(const size_t *md, size_t len, Strided *s) {
     return HODU_ROCM_OK;
 }
 
+// reduce metadata (crates/hodu_core/src/op_metadatas.rs:525-586, read by kernels/ops_reduce.c:51-66):
+// [nd, shape.., strides.., offset, out_nd, out_shape.., n_reduce, reduce_dims.., keep_dim, reduce_size]
+int parse_reduce_metadata(const size_t *md, size_t len, Reduction *r) {
+    if (!md) return fail(HODU_ROCM_INVALID_ARG, "sum: metadata is null");
+    if (len < 1) return fail(HODU_ROCM_INVALID_ARG, "sum: metadata is empty");
+    for (size_t i = 0; i < len; i++)
+        if (!sane(md[i])) return fail(HODU_ROCM_INVALID_ARG, "sum: metadata[%zu] out of range", i);
+    const size_t nd = md[0];
+    if (nd > 16) return fail(HODU_ROCM_UNSUPPORTED, "sum: %zu dims (> 16)", nd);
+    if (len < 3 + 2 * nd) return fail(HODU_ROCM_INVALID_ARG, "sum: metadata has %zu words, too few for %zu dims", len, nd);
+    const size_t *shape = md + 1, *strides = md + 1 + nd;
+    const size_t offset = md[1 + 2 * nd], out_nd = md[2 + 2 * nd];
+    if (out_nd > 16 || len < 4 + 2 * nd + out_nd) return fail(HODU_ROCM_INVALID_ARG, "sum: output shape does not fit the metadata");
+    const size_t *out_shape = md + 3 + 2 * nd;
+    const size_t n_red = md[3 + 2 * nd + out_nd];
+    if (n_red > nd) return fail(HODU_ROCM_INVALID_ARG, "sum: %zu reduce dims of %zu", n_red, nd);
+    if (len != 6 + 2 * nd + out_nd + n_red)
+        return fail(HODU_ROCM_INVALID_ARG, "sum: metadata has %zu words, layout implies %zu", len, 6 + 2 * nd + out_nd + n_red);
+    const size_t *red = md + 4 + 2 * nd + out_nd;
+    const bool keep = md[4 + 2 * nd + out_nd + n_red] != 0;
+    const size_t reduce_size = md[5 + 2 * nd + out_nd + n_red];
+    bool is_red[16] = {false};
+    size_t rs = 1;
+    for (size_t i = 0; i < n_red; i++) {
+        if (red[i] >= nd || is_red[red[i]]) return fail(HODU_ROCM_INVALID_ARG, "sum: bad reduce dim %zu", red[i]);
+        is_red[red[i]] = true;
+        rs *= shape[red[i]];
+    }
+    if (rs != reduce_size) return fail(HODU_ROCM_INVALID_ARG, "sum: reduce_size %zu != product of the reduced extents %zu", reduce_size, rs);
+    // the output shape the encoder derives: kept dims in order, reduced dims as 1 when keep_dim, [1] if nothing is left
+    size_t want[16], wn = 0, n_out = 1;
+    for (size_t d = 0; d < nd; d++) {
+        if (!is_red[d]) { want[wn++] = shape[d]; n_out *= shape[d]; }
+        else if (keep) want[wn++] = 1;
+    }
+    if (wn == 0) want[wn++] = 1;
+    if (wn != out_nd) return fail(HODU_ROCM_INVALID_ARG, "sum: output has %zu dims, the reduction leaves %zu", out_nd, wn);
+    for (size_t d = 0; d < wn; d++)
+        if (want[d] != out_shape[d]) return fail(HODU_ROCM_INVALID_ARG, "sum: output extent %zu of dim %zu, expected %zu", out_shape[d], d, want[d]);
+    *r = Reduction{};
+    r->n_out = (long)n_out;
+    r->reduce_size = (long)reduce_size;
+    r->offset = (long)offset;
+    // split and merge: a dim joins its predecessor in the same list when stride_prev == extent * stride
+    auto push = [](long *sh, long *st, int &n, long extent, long stride) {
+        if (extent == 1) return;
+        if (n > 0 && st[n - 1] == extent * stride) { sh[n - 1] *= extent; st[n - 1] = stride; return; }
+        sh[n] = extent; st[n] = stride; n++;
+    };
+    for (size_t d = 0; d < nd; d++) {
+        if (is_red[d]) push(r->red_shape, r->red_stride, r->red_n, (long)shape[d], (long)strides[d]);
+        else push(r->kept_shape, r->kept_stride, r->kept_n, (long)shape[d], (long)strides[d]);
+    }
+    return HODU_ROCM_OK;
+}
+
 }  // namespace hodu

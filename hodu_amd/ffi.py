@@ -118,6 +118,7 @@ def load() -> ctypes.CDLL:
                                                ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
+    lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
     _lib = lib
     return lib
 
@@ -280,6 +281,20 @@ class Context:
         self._check_strided(f"contiguous_{dt}", DTYPE_SIZE[dt], DTYPE_SIZE[dt], x, out, md)
         arr, n = _md_array(md)
         self._check(self.lib.hodu_rocm_contiguous(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
+
+    def sum(self, dt: str, x: DeviceBuffer, out: DeviceBuffer, md):
+        """hodu_rocm_sum: md is reduce_metadata [nd, shape.., strides.., offset, out_nd, out_shape.., n_reduce,
+        reduce_dims.., keep_dim, reduce_size]"""
+        m = [int(v) for v in md]
+        if m and len(m) >= 3 + 2 * m[0]:
+            nd = m[0]
+            span = _view_span(m[1:1 + nd], m[1 + nd:1 + 2 * nd], m[1 + 2 * nd])
+            out_nd = m[2 + 2 * nd]
+            n_out = int(np.prod(m[3 + 2 * nd:3 + 2 * nd + out_nd], dtype=np.int64)) if len(m) >= 3 + 2 * nd + out_nd else 0
+            if span * DTYPE_SIZE[dt] > x.nbytes or n_out * DTYPE_SIZE[dt] > out.nbytes:
+                raise HoduRocmError(INVALID_ARG, f"sum_{dt}: metadata reaches past a device buffer")
+        arr, n = _md_array(md)
+        self._check(self.lib.hodu_rocm_sum(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
 
     def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int,
                      graph: bool = False, steps=None) -> float:

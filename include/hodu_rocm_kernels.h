@@ -224,6 +224,16 @@ int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src_dtype, int dst_dtype, const void 
 int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out,
                          const size_t *metadata, size_t metadata_len);
 
+/* ---- sum over dims (the reduce that the matmul gradient needs) ----------------------------------- *
+ * replaces hodu_cpu_sum_<dt> (kernels/ops_reduce.c:47-118 macro, instantiations :127-130, :133-237, :345-352) for
+ * the use Tensor::sum_to_shape makes of it on a matmul's gradients when an operand was broadcast
+ * (tensor/gradient/vjp_matrix.rs:41-43, tensor/ops/reduce.rs:19-50).  metadata is reduce_metadata
+ * (op_metadatas.rs:525-586): [nd, shape.., strides.., offset, out_nd, out_shape.., n_reduce, reduce_dims..,
+ * keep_dim, reduce_size]; any strided input, output contiguous in out_shape.  Narrow floats and f32 accumulate in
+ * f32 and round once on store, f64 in f64, integers wrap.  One entry point taking the dtype id, as for the casts. */
+int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *metadata,
+                  size_t metadata_len);
+
 #ifdef __cplusplus
 }
 #endif

@@ -163,6 +163,29 @@ def relu(dt: str, x: np.ndarray, md) -> np.ndarray:
     return out
 
 
+def reduce_out_elems(md) -> int:
+    nd = int(md[0])
+    out_nd = int(md[2 + 2 * nd])
+    return int(np.prod([int(v) for v in md[3 + 2 * nd:3 + 2 * nd + out_nd]], dtype=np.int64))
+
+
+def sum_asis(dt: str, x: np.ndarray, md) -> np.ndarray:
+    """hodu_cpu_sum_<dt>: accumulator in the storage type; md is reduce_metadata"""
+    md = _md(md)
+    out = np.empty(reduce_out_elems(md), dtype=STORAGE[dt])
+    _check(lib().oracle_sum_asis(DTYPE_ID[dt], _ptr(x), _ptr(out), _ptr(md)), "sum")
+    return out
+
+
+def sum_spec(dt: str, x: np.ndarray, md, decode=F8_OCP):
+    """(f32-accumulated sums, f64 sums, sums of magnitudes)"""
+    md = _md(md)
+    n = reduce_out_elems(md)
+    o32, o64, oabs = np.empty(n, np.float32), np.empty(n, np.float64), np.empty(n, np.float64)
+    _check(lib().oracle_sum_spec(DTYPE_ID[dt], decode, _ptr(x), _ptr(md), _ptr(o32), _ptr(o64), _ptr(oabs)), "sum_spec")
+    return o32, o64, oabs
+
+
 def f8e4m3_table(decode: int) -> np.ndarray:
     """All 256 decoded values as f32."""
     return np.array([lib().oracle_f8e4m3_to_f32(b, decode) for b in range(256)], dtype=np.float32)
@@ -246,6 +269,14 @@ class RefLib:
         md = _md(md)
         out = np.empty(int(md[0]), dtype=STORAGE[dt])
         fn = getattr(self.lib, f"hodu_cpu_relu_{dt}")
+        fn.restype = None
+        fn(_ptr(x), _ptr(out), _ptr(md))
+        return out
+
+    def sum(self, dt, x, md):
+        md = _md(md)
+        out = np.empty(reduce_out_elems(md), dtype=STORAGE[dt])
+        fn = getattr(self.lib, f"hodu_cpu_sum_{dt}")
         fn.restype = None
         fn(_ptr(x), _ptr(out), _ptr(md))
         return out

@@ -16,6 +16,9 @@
  *   gather   crates/hodu_cpu_kernels/kernels/ops_memory.c:19-84
  *   add      crates/hodu_cpu_kernels/kernels/ops_binary.c:208-262 (bf16/f16/f8: widen, add in f32, narrow with the
  *            type's own routine) and the native-type macro :60-118; metadata :214-222
+ *   sum      crates/hodu_cpu_kernels/kernels/ops_reduce.c:47-118 (generic macro: one output at a time, the reduced
+ *            dims walked innermost first, accumulator in the storage type -- bf16 / f16 / f8 re-round after every
+ *            add, :127-130), :133-237 (f32; a lane-wise SIMD order only when the last, dense dim alone is reduced)
  *   mul_scalar, relu
  *            crates/hodu_cpu_kernels/kernels/ops_unary.c:138-200, :352-386 (scalar arrives in the storage type),
  *            :648-697, :1233, :1319, :1404, :1484 ((x > 0) ? x : 0 in f32)
@@ -42,6 +45,10 @@
  * The element-wise functions (add, mul_scalar, relu) are compared bit for bit with oracle/_ref on random bit
  * patterns of every dtype, with the literal vectors of the reference's tests (tests/ops_binary.rs:68-73,
  * tests/ops_unary.rs:143-147, :503-507) and, for bf16, with an independent numpy f32 sum whose low 16 bits are cut.
+ *
+ * sum: ASIS is compared bit for bit with oracle/_ref on every dtype and layout, except f32 / f64 sums over the last
+ * dense dim alone, where the reference adds lane-wise (SIMD width of the build) and only a tolerance applies: the
+ * bits of that one case are parity unpinned.  Integer sums against numpy; SPEC against float64.
  *
  * Parity unpinned: float->integer casts of out-of-range or NaN inputs are undefined behaviour
  * in the reference C ((T)x) and are not checked.
@@ -722,6 +729,95 @@ int oracle_mul_scalar(int dt, const void *in, void *out, const size_t *md, const
     return ew_unary(dt, EW_MUL, in, out, md, scalar);
 }
 int oracle_relu(int dt, const void *in, void *out, const size_t *md) { return ew_unary(dt, EW_RELU, in, out, md, NULL); }
+
+/* ------------------------------------------------------------------------------------------ */
+/* sum over dims (ops_reduce.c)                                                                  */
+/* ------------------------------------------------------------------------------------------ */
+typedef struct {
+    size_t nd, out_nd, n_red, reduce_size, n_out, offset;
+    const size_t *dims, *strides, *out_shape, *red;
+    int keep;
+} reduce_space;
+
+static void reduce_space_from(const size_t *md, reduce_space *r) {
+    r->nd = md[0];
+    r->dims = md + 1;
+    r->strides = md + 1 + r->nd;
+    r->offset = md[1 + 2 * r->nd];
+    r->out_nd = md[2 + 2 * r->nd];
+    r->out_shape = md + 3 + 2 * r->nd;
+    r->n_red = md[3 + 2 * r->nd + r->out_nd];
+    r->red = md + 4 + 2 * r->nd + r->out_nd;
+    r->keep = md[4 + 2 * r->nd + r->out_nd + r->n_red] != 0;
+    r->reduce_size = md[5 + 2 * r->nd + r->out_nd + r->n_red];
+    r->n_out = 1;
+    for (size_t i = 0; i < r->out_nd; i++) r->n_out *= r->out_shape[i];
+}
+
+/* input position of reduced index `ri` for output `oi` (ops_reduce.c:68-110) */
+static size_t reduce_pos(const reduce_space *r, size_t oi, size_t ri) {
+    size_t oidx[16], iidx[16];
+    for (size_t d = r->out_nd; d-- > 0;) { oidx[d] = oi % r->out_shape[d]; oi /= r->out_shape[d]; }
+    if (r->keep) {
+        for (size_t i = 0; i < r->nd; i++) iidx[i] = oidx[i];
+    } else {
+        size_t o = 0;
+        for (size_t d = 0; d < r->nd; d++) {
+            int is_red = 0;
+            for (size_t k = 0; k < r->n_red; k++) is_red |= r->red[k] == d;
+            if (is_red) iidx[d] = 0;
+            else { iidx[d] = o < r->out_nd ? oidx[o] : 0; o++; }
+        }
+    }
+    for (size_t k = r->n_red; k-- > 0;) { iidx[r->red[k]] = ri % r->dims[r->red[k]]; ri /= r->dims[r->red[k]]; }
+    size_t pos = r->offset;
+    for (size_t d = 0; d < r->nd; d++) pos += iidx[d] * r->strides[d];
+    return pos;
+}
+
+/* hodu_cpu_sum_<dt>: accumulator in the storage type, reduced elements added in reduced-index order */
+int oracle_sum_asis(int dt, const void *in, void *out, const size_t *md) {
+    if (dt <= DT_BOOL || dt >= DT_COUNT) return -1;
+    reduce_space r;
+    reduce_space_from(md, &r);
+    const size_t es = k_dtype_size[dt];
+    _Pragma("omp parallel for schedule(static)")
+    for (size_t o = 0; o < r.n_out; o++) {
+        unsigned char acc[8] = {0};
+        for (size_t i = 0; i < r.reduce_size; i++) {
+            unsigned char next[8];
+            ew_one(dt, EW_ADD, acc, (const char *)in + reduce_pos(&r, o, i) * es, next);
+            memcpy(acc, next, es);
+        }
+        memcpy((char *)out + o * es, acc, es);
+    }
+    return 0;
+}
+
+/* comparator for the floating dtypes: elements widened exactly (f8e4m3 by `f8_decode`), summed in f32 in the same
+ * order; also the f64 sum and the sum of magnitudes (floor of the relative-error denominator) */
+int oracle_sum_spec(int dt, int f8_decode, const void *in, const size_t *md, float *out32, double *out64, double *out_abs) {
+    if (dt <= DT_BOOL || dt >= DT_COUNT) return -1;
+    reduce_space r;
+    reduce_space_from(md, &r);
+    _Pragma("omp parallel for schedule(static)")
+    for (size_t o = 0; o < r.n_out; o++) {
+        float s32 = 0.0f;
+        double s64 = 0.0, sabs = 0.0;
+        for (size_t i = 0; i < r.reduce_size; i++) {
+            const size_t pos = reduce_pos(&r, o, i);
+            const float v = dt == DT_F64 ? (float)((const double *)in)[pos] : widen_any(dt, in, pos, f8_decode);
+            const double d = dt == DT_F64 ? ((const double *)in)[pos] : (double)v;
+            s32 += v;
+            s64 += d;
+            sabs += fabs(d);
+        }
+        if (out32) out32[o] = s32;
+        if (out64) out64[o] = s64;
+        if (out_abs) out_abs[o] = sabs;
+    }
+    return 0;
+}
 
 /* ------------------------------------------------------------------------------------------ */
 /* single-thread timing entry points for the cpu_baseline (the reference runs batched / strided */

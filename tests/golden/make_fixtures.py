@@ -1,7 +1,7 @@
 """Writes the golden fixtures of this directory from the reference's own C kernels.
 
 Run in the build container only (needs oracle/_ref/libhodu_cpu_ref.so, i.e. `make -C oracle ref`,
-which compiles crates/hodu_cpu_kernels/kernels/{ops_matrix,ops_cast,ops_memory,ops_binary,ops_unary}.c where they lie
+which compiles crates/hodu_cpu_kernels/kernels/{ops_matrix,ops_cast,ops_memory,ops_binary,ops_unary,ops_reduce}.c where they lie
 under /root/reference):
 
     python tests/golden/make_fixtures.py
@@ -245,6 +245,37 @@ def write_elementwise(ref):
     return len(names)
 
 
+def sum_cases():
+    """(name, view, dims, keep_dim): what sum_to_shape runs on a matmul's gradients (leading dims, one at a time, and
+    kept extent-1 dims) plus the other shapes of the reference's walker"""
+    V = H.View
+    return [
+        ("lead", V([5, 7, 12]), [0], False),           # [B, K, N] -> [K, N]
+        ("lead_keep", V([5, 7, 12]), [0], True),       # -> [1, K, N]
+        ("middle_keep", V([3, 4, 6, 5]), [1], True),   # a broadcast batch dim of extent 1 in the target
+        ("two", V([3, 4, 6, 5]), [0, 1], False),
+        ("last", V([9, 33]), [1], False),              # strided rows: the reference's sequential order
+        ("last_keep_strided", V([9, 40]).slice(1, 1, 40, 3), [1], True),
+        ("transposed", V([6, 8, 10], offset=3).t(0, 2), [0], False),
+        ("all", V([4, 5, 6]), [0, 1, 2], False),
+    ]
+
+
+def write_sums(ref):
+    out, names = {}, []
+    for dt in ELEMENTWISE_FLOATS + ELEMENTWISE_INTS:
+        for name, v, dims, keep in sum_cases():
+            x = H.random_storage(dt, v.span(), 21, 2.0)
+            md = np.array(H.reduce_md(v, dims, keep), dtype=np.uint64)
+            key = f"sum_{name}__{dt}"
+            out[key + "__in"], out[key + "__md"] = x, md
+            out[key + "__out"] = ref.sum(dt, x, md)
+            names.append(f"{key}|{dt}")
+    out["index"] = np.array(names)
+    np.savez_compressed(os.path.join(HERE, "sums.npz"), **out)
+    return len(names)
+
+
 def main():
     if not oracle.RefLib.available():
         raise SystemExit("oracle/_ref/libhodu_cpu_ref.so missing: run `make -C oracle ref` first")
@@ -253,7 +284,8 @@ def main():
     write_tables(ref)
     m = write_casts(ref)
     e = write_elementwise(ref)
-    print(f"wrote {n} product cases, {m} cast/contiguous cases, {e} element-wise cases, tables")
+    k = write_sums(ref)
+    print(f"wrote {n} product cases, {m} cast/contiguous cases, {e} element-wise cases, {k} sum cases, tables")
 
 
 if __name__ == "__main__":

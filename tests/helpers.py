@@ -117,6 +117,24 @@ def cast_md(v: View):
     return [v.size, v.ndim] + v.shape + v.strides + [v.offset]
 
 
+def reduce_md(v: View, dims, keep_dim: bool):
+    """reduce_metadata of crates/hodu_core/src/op_metadatas.rs:525-586"""
+    dims = [d % v.ndim for d in dims]
+    out_shape = []
+    for i, s in enumerate(v.shape):
+        if i in dims:
+            if keep_dim:
+                out_shape.append(1)
+        else:
+            out_shape.append(s)
+    if not out_shape:
+        out_shape = [1]
+    rs = 1
+    for d in dims:
+        rs *= v.shape[d]
+    return [v.ndim] + v.shape + v.strides + [v.offset, len(out_shape)] + out_shape + [len(dims)] + dims + [int(keep_dim), rs]
+
+
 def binary_md(lv: View, rv: View):
     """binary_metadata of crates/hodu_core/src/op_metadatas.rs:36-73 (both operands already broadcast to one shape)"""
     assert lv.shape == rv.shape

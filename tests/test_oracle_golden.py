@@ -318,3 +318,40 @@ def test_elementwise_against_independent_arithmetic():
                           (x.astype(np.int64) * int(s[0])).astype(np.int32))
     r = oracle.relu("bf16", np.array([0x7FC0, 0x8000, 0xBF80, 0x3F80, 0xFF80, 0x7F80], dtype=np.uint16), H.cast_md(H.View([6])))
     assert list(r) == [0, 0, 0, 0x3F80, 0, 0x7F80]
+
+
+# ---------------------------------------------------------------------------------------------
+# sum over dims (what sum_to_shape runs on a matmul's gradients)
+# ---------------------------------------------------------------------------------------------
+def test_sums_bit_exact_vs_reference_fixtures():
+    sums = np.load(os.path.join(GOLD, "sums.npz"))
+    index = [s.split("|") for s in sums["index"]]
+    assert len(index) == 14 * 8
+    for key, dt in index:
+        got, want = oracle.sum_asis(dt, sums[key + "__in"], sums[key + "__md"]), sums[key + "__out"]
+        if dt in ("f32", "f64") and key.startswith("sum_last__"):
+            # the reference adds lane-wise (SIMD) when only the last, dense dim is reduced: same numbers, other order
+            assert np.allclose(got, want, rtol=1e-5 if dt == "f32" else 1e-13, atol=1e-5 if dt == "f32" else 1e-13), key
+            continue
+        assert np.array_equal(_bits(got), _bits(want)), key
+
+
+def test_sums_against_numpy():
+    """integers: numpy's modular sum; floats: the f32-accumulated comparator against a float64 sum; keep_dim only
+    changes the shape; bf16 accumulates in bf16 (kernels/ops_reduce.c:129): summing 1.0 513 times stalls at 256"""
+    V = H.View
+    g = H.rng(31)
+    v = V([6, 5, 7])
+    x = g.integers(-2 ** 31, 2 ** 31, v.size).astype(np.int32)
+    want = x.reshape(6, 5, 7).astype(np.int64).sum(axis=0).astype(np.int32).ravel()
+    assert np.array_equal(oracle.sum_asis("i32", x, H.reduce_md(v, [0], False)), want)
+    assert np.array_equal(oracle.sum_asis("i32", x, H.reduce_md(v, [0], True)), want)
+    want = x.reshape(6, 5, 7).astype(np.int64).sum(axis=(0, 2)).astype(np.int32).ravel()
+    assert np.array_equal(oracle.sum_asis("i32", x, H.reduce_md(v, [0, 2], False)), want)
+    f = g.standard_normal(v.size).astype(np.float32)
+    o32, o64, oabs = oracle.sum_spec("f32", f, H.reduce_md(v, [1], False))
+    assert np.allclose(o64, f.reshape(6, 5, 7).astype(np.float64).sum(axis=1).ravel(), rtol=1e-14)
+    assert np.allclose(o32, o64, rtol=1e-5, atol=1e-6) and np.allclose(oabs, np.abs(f.reshape(6, 5, 7)).sum(axis=1).ravel())
+    ones = np.full(513, 0x3F80, dtype=np.uint16)
+    assert oracle.sum_asis("bf16", ones, H.reduce_md(V([513]), [0], False))[0] == 0x4380  # 256.0
+    assert oracle.sum_spec("bf16", ones, H.reduce_md(V([513]), [0], False))[0][0] == 513.0

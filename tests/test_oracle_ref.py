@@ -95,3 +95,14 @@ def test_elementwise_match_compiled_reference(ref, dt):
     if floating:
         assert np.array_equal(_bits(oracle.relu(dt, x, md)), _bits(ref.relu(dt, x, md))), dt
         assert np.array_equal(_bits(oracle.relu(dt, x, H.cast_md(v))), _bits(ref.relu(dt, x, H.cast_md(v)))), dt
+
+
+@pytest.mark.parametrize("dt", ELEMENTWISE_DTYPES)
+def test_sums_match_compiled_reference(ref, dt):
+    V = H.View
+    cases = [(V([4, 9, 20]), [0], False), (V([4, 9, 20]), [0], True), (V([2, 3, 5, 8]), [1], True),
+             (V([2, 3, 5, 8]), [0, 2], False), (V([7, 30], offset=2).t(), [1], False), (V([5, 6]), [0, 1], False)]
+    for n, (v, dims, keep) in enumerate(cases):
+        x = H.random_storage(dt, v.span(), 500 + n, 2.0)
+        md = H.reduce_md(v, dims, keep)
+        assert np.array_equal(_bits(oracle.sum_asis(dt, x, md)), _bits(ref.sum(dt, x, md))), (dt, n)
