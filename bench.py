@@ -142,6 +142,14 @@ def build_cases(which):
                               "matmul", name, V([b, s, f]), V([d, f]).t().broadcast_to([b, f, d]),
                               lambda b=b, s=s, f=f: bf16(normal(504, b * s * f, 0.3)), mk_w(503),
                               2.0 * b * s * d * f, b * s * f * 2 + wbytes + b * s * d * 2, "mfma", "bf16"))
+    if "bwd" in which:
+        # not a BASELINE configuration: the weight gradient of config 5's up projection, dW = X^T . dY with the batch
+        # folded into the contraction (K = 8 * 512): both operands row-dense, the layout pair the forward never uses
+        b, s_, d, f = 8, 512, 4096, 14336
+        cases.append(Case("c5_up_dw_bf16", "C5 up weight gradient: bf16[4096,4096]^T-view x bf16[4096,14336] (not a BASELINE config)",
+                          "dot", "bf16", V([b * s_, d]).t(), V([b * s_, f]),
+                          lambda: bf16(normal(801, b * s_ * d)), lambda: bf16(normal(802, b * s_ * f, 0.05)),
+                          2.0 * d * b * s_ * f, (b * s_ * d + b * s_ * f + d * f) * 2, "mfma", "bf16"))
     if "fused" in which:
         base = {c.key: c for c in build_cases({"c2", "c3", "c5"})}
         cases.append(base["c3_m1"].with_steps("c3_m1_linear", "C3 M=1 as a Linear layer: + bias fused", ("bias",)))
@@ -284,7 +292,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,fused")
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,fused,bwd")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
@@ -322,7 +330,7 @@ def main():
         ctx.close()
         return
     if args.only:
-        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "fused"}) if c.key == args.only)
+        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "fused", "bwd"}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
         ctx.close()
         return

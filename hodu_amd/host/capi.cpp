@@ -92,6 +92,30 @@ int hodu_host_linear(const hodu_host_tensor *input, const hodu_host_tensor *weig
     return guarded([&] { *out = H(box(Tensor::linear(*T(input), *T(weight), bias ? T(bias) : nullptr, relu != 0))); });
 }
 long hodu_host_stats_fused_steps(void) { return stats().fused_steps; }
+long hodu_host_stats_sum_kernels(void) { return stats().sum_kernels; }
+int hodu_host_sum(const hodu_host_tensor *t, const int *dims, size_t n_dims, int keep_dim, hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(T(t)->sum(std::vector<int>(dims, dims + n_dims), keep_dim != 0))); });
+}
+int hodu_host_sum_to_shape(const hodu_host_tensor *t, const size_t *shape, size_t nd, hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(T(t)->sum_to_shape(dims_of(shape, nd)))); });
+}
+// gradients of matmul / dot with respect to both operands (vjp_matrix.rs:17-67)
+int hodu_host_matmul_vjp(const hodu_host_tensor *a, const hodu_host_tensor *b, const hodu_host_tensor *grad,
+                         hodu_host_tensor **da, hodu_host_tensor **db) {
+    return guarded([&] {
+        Tensor::Grads g = Tensor::matmul_vjp(*T(a), *T(b), *T(grad));
+        *da = H(box(g.first));
+        *db = H(box(g.second));
+    });
+}
+int hodu_host_dot_vjp(const hodu_host_tensor *a, const hodu_host_tensor *b, const hodu_host_tensor *grad,
+                      hodu_host_tensor **da, hodu_host_tensor **db) {
+    return guarded([&] {
+        Tensor::Grads g = Tensor::dot_vjp(*T(a), *T(b), *T(grad));
+        *da = H(box(g.first));
+        *db = H(box(g.second));
+    });
+}
 int hodu_host_dot(const hodu_host_tensor *a, const hodu_host_tensor *b, hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(T(a)->dot(*T(b)))); });
 }

@@ -209,13 +209,15 @@ public:
         return shape_ == o.shape_ && strides_ == o.strides_ && offset_ == o.offset_;
     }
 
-private:
+    // negative axes count from the end
     size_t axis(int d) const {
         const int n = (int)ndim();
         const int a = d < 0 ? n + d : d;
         if (a < 0 || a >= n) throw Error(ErrorKind::InternalError, "invalid axis: " + std::to_string(d));
         return (size_t)a;
     }
+
+private:
 
     Dims shape_, strides_;
     size_t offset_ = 0;

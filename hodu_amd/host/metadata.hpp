@@ -2,6 +2,8 @@
 // (crates/hodu_core/src/op_metadatas.rs).  Header-only, no GPU dependency.
 #pragma once
 
+#include <algorithm>
+
 #include "layout.hpp"
 
 namespace hodu_host {
@@ -64,5 +66,37 @@ inline Metadata cast_metadata(const Layout &l) {
 
 // op_metadatas.rs:1654-1656
 inline Metadata contiguous_metadata(const Layout &l) { return cast_metadata(l); }
+
+// op_metadatas.rs:525-586: [nd, shape.., strides.., offset, out_nd, out_shape.., n_reduce, reduce_dims.., keep_dim,
+// reduce_size]; reducing everything without keep_dim still encodes the output shape [1]
+inline Metadata reduce_metadata(const Layout &l, const std::vector<size_t> &dims, bool keep_dim) {
+    const size_t nd = l.ndim();
+    Dims out;
+    size_t reduce_size = 1;
+    for (size_t i = 0; i < nd; i++) {
+        const bool reduced = std::find(dims.begin(), dims.end(), i) != dims.end();
+        if (reduced) {
+            if (keep_dim) out.push_back(1);
+        } else {
+            out.push_back(l.shape()[i]);
+        }
+    }
+    if (out.empty()) out.push_back(1);
+    for (size_t d : dims) {
+        if (d >= nd) throw Error(ErrorKind::InvalidAxis, "sum: dim " + std::to_string(d) + " of " + std::to_string(nd));
+        reduce_size *= l.shape()[d];
+    }
+    Metadata md{nd};
+    md.insert(md.end(), l.shape().begin(), l.shape().end());
+    md.insert(md.end(), l.strides().begin(), l.strides().end());
+    md.push_back(l.offset());
+    md.push_back(out.size());
+    md.insert(md.end(), out.begin(), out.end());
+    md.push_back(dims.size());
+    md.insert(md.end(), dims.begin(), dims.end());
+    md.push_back(keep_dim ? 1 : 0);
+    md.push_back(reduce_size);
+    return md;
+}
 
 }  // namespace hodu_host

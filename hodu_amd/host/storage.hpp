@@ -37,8 +37,9 @@ inline const char *dtype_name(DType d) {
 struct Stats {
     std::atomic<long> cast_kernels{0}, contiguous_kernels{0}, product_kernels{0}, fused_products{0};
     std::atomic<long> fused_steps{0};        // element-wise kernels that ran inside a product's store instead
+    std::atomic<long> sum_kernels{0};
     std::atomic<long long> bytes_copied{0};  // written by cast/contiguous passes
-    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = 0; bytes_copied = 0; }
+    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = sum_kernels = 0; bytes_copied = 0; }
 };
 inline Stats &stats() {
     static Stats s;
@@ -175,6 +176,22 @@ public:
         rhs.check_span(rl, "dot rhs");
         const Metadata md = dot_metadata(ll, rl);
         return product(rhs, ll, rl, md, md[0] * md[2], false, fused);
+    }
+
+    // be_cpu/storage/ops_reduce.rs (call_ops_reduce, ReduceOp::Sum): output fresh and contiguous in the reduced shape
+    RocmStorage call_ops_reduce_sum(const Layout &layout, const std::vector<size_t> &dims, bool keep_dim) const {
+        check_span(layout, "sum");
+        if (dtype_ == DType::BOOL) throw Error(ErrorKind::UnsupportedDTypeForOp, "sum: bool is not supported");
+        if (deferred()) return gather(layout).call_ops_reduce_sum(Layout::from_shape(layout.shape()), dims, keep_dim);
+        const Metadata md = reduce_metadata(layout, dims, keep_dim);
+        size_t n_out = 1;
+        const size_t nd = md[0], out_nd = md[2 + 2 * nd];
+        for (size_t i = 0; i < out_nd; i++) n_out *= md[3 + 2 * nd + i];
+        RocmStorage out = fresh(dtype_, n_out);
+        if (n_out == 0) return out;
+        dev_->check(hodu_rocm_sum(dev_->ctx(), (int)dtype_, ptr(), (void *)out.ptr(), md.data(), md.size()), "sum");
+        stats().sum_kernels++;
+        return out;
     }
 
     // be_cpu/storage/ops_matrix.rs:63-100: right-aligned broadcast of the batch dims, then [M, N]

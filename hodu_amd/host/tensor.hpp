@@ -139,6 +139,61 @@ public:
         return input.matmul_then(wt, then);
     }
 
+    // ---- backward through the path ------------------------------------------------------------------------
+    // tensor/ops/reduce.rs:11-13, :135-175: negative dims count from the end; no dims = all of them
+    Tensor sum(const std::vector<int> &dims, bool keep_dim) const {
+        const size_t nd = layout_.ndim();
+        std::vector<size_t> red;
+        if (dims.empty()) for (size_t i = 0; i < nd; i++) red.push_back(i);
+        for (int d : dims) red.push_back(layout_.axis(d));
+        Dims out_shape;
+        for (size_t i = 0; i < nd; i++) {
+            const bool reduced = std::find(red.begin(), red.end(), i) != red.end();
+            if (!reduced) out_shape.push_back(shape()[i]);
+            else if (keep_dim) out_shape.push_back(1);
+        }
+        auto out = std::make_shared<RocmStorage>(storage_->call_ops_reduce_sum(layout_, red, keep_dim));
+        return Tensor(out, Layout::from_shape(out_shape));
+    }
+
+    // tensor/ops/reduce.rs:19-50: leading extra dims first (innermost of them first), then every dim the target
+    // holds at extent 1, one launch each
+    Tensor sum_to_shape(const Dims &target) const {
+        if (shape() == target) return *this;
+        Tensor result = *this;
+        if (shape().size() > target.size())
+            for (size_t d = shape().size() - target.size(); d-- > 0;) result = result.sum({(int)d}, false);
+        for (size_t i = 0; i < target.size() && i < result.shape().size(); i++)
+            if (target[i] == 1 && result.shape()[i] > 1) result = result.sum({(int)i}, true);
+        return result;
+    }
+
+    using Grads = std::pair<Tensor, Tensor>;  // (dA, dB)
+
+    // tensor/gradient/vjp_matrix.rs:17-45: dA = grad @ B^T, dB = A^T @ grad, each summed down to its operand's
+    // shape where matmul had broadcast it.  With a weight that has no batch dims (the Linear case) and dense a and
+    // grad, NoCopy mode folds the batch into the contraction instead: dB = [B*M, K]^T @ [B*M, N] is one product
+    // whose f32 accumulator runs over the batch as well -- no [B, K, N] intermediate, no sum launches, and one
+    // rounding instead of B + 1.
+    static Grads matmul_vjp(const Tensor &a, const Tensor &b, const Tensor &grad) {
+        const Tensor da = grad.matmul(b.transpose(-2, -1)).sum_to_shape(a.shape());
+        const size_t an = a.layout().ndim();
+        if (matmul_mode() == MatmulMode::NoCopy && b.layout().ndim() == 2 && an > 2 && a.is_contiguous() && grad.is_contiguous()) {
+            size_t rows = 1;
+            for (size_t i = 0; i + 1 < an; i++) rows *= a.shape()[i];
+            const Tensor a2 = a.view(Layout({rows, a.shape()[an - 1]}, {a.shape()[an - 1], 1}, a.layout().offset()));
+            const Tensor g2 = grad.view(Layout({rows, grad.shape().back()}, {grad.shape().back(), 1}, grad.layout().offset()));
+            return {da, a2.view(a2.layout().transpose(0, 1)).dot(g2)};
+        }
+        const Tensor db = a.transpose(-2, -1).matmul(grad).sum_to_shape(b.shape());
+        return {da, db};
+    }
+
+    // tensor/gradient/vjp_matrix.rs:46-67
+    static Grads dot_vjp(const Tensor &a, const Tensor &b, const Tensor &grad) {
+        return {grad.dot(b.transpose(-2, -1)), a.transpose(-2, -1).dot(grad)};
+    }
+
 private:
     // tensor/utils.rs broadcast_tensors2 as Tensor::add applies it to (output, operand): the operand's shape is
     // right-aligned against the output's; a fused add needs every axis but the last to be broadcast (extent 1

@@ -63,6 +63,11 @@ def load() -> ctypes.CDLL:
     lib.hodu_host_matmul_then.argtypes = [vp, vp, ctypes.POINTER(_Then), sz, vpp]
     lib.hodu_host_linear.argtypes = [vp, vp, vp, ci, vpp]
     lib.hodu_host_stats_fused_steps.restype = ctypes.c_long
+    lib.hodu_host_stats_sum_kernels.restype = ctypes.c_long
+    lib.hodu_host_sum.argtypes = [vp, ctypes.POINTER(ci), sz, ci, vpp]
+    lib.hodu_host_sum_to_shape.argtypes = [vp, szp, sz, vpp]
+    lib.hodu_host_matmul_vjp.argtypes = [vp, vp, vp, vpp, vpp]
+    lib.hodu_host_dot_vjp.argtypes = [vp, vp, vp, vpp, vpp]
     lib.hodu_host_to_dtype.argtypes = [vp, ci, vpp]
     lib.hodu_host_contiguous.argtypes = [vp, vpp]
     lib.hodu_host_transpose.argtypes = [vp, ci, ci, vpp]
@@ -95,11 +100,11 @@ def stats(reset: bool = False) -> dict:
     lib = load()
     a, b, c, d, e = (ctypes.c_long(), ctypes.c_long(), ctypes.c_long(), ctypes.c_long(), ctypes.c_longlong())
     lib.hodu_host_stats(a, b, c, d, e)
-    fused_steps = int(lib.hodu_host_stats_fused_steps())
+    fused_steps, sum_kernels = int(lib.hodu_host_stats_fused_steps()), int(lib.hodu_host_stats_sum_kernels())
     if reset:
         lib.hodu_host_stats_reset()
     return {"cast_kernels": a.value, "contiguous_kernels": b.value, "product_kernels": c.value,
-            "fused_products": d.value, "bytes_copied": e.value, "fused_steps": fused_steps}
+            "fused_products": d.value, "bytes_copied": e.value, "fused_steps": fused_steps, "sum_kernels": sum_kernels}
 
 
 class Tensor:
@@ -187,6 +192,14 @@ class Tensor:
         out = ctypes.c_void_p()
         return self._wrap(load().hodu_host_matmul_then(self._h, other._h, arr, len(steps), ctypes.byref(out)), out)
 
+    def sum(self, dims: Sequence[int] = (), keep_dim: bool = False) -> "Tensor":
+        """Tensor::sum (tensor/ops/reduce.rs:11-13): no dims = all of them"""
+        arr = (ctypes.c_int * max(1, len(dims)))(*dims)
+        return self._unary(load().hodu_host_sum, arr, len(dims), int(keep_dim))
+
+    def sum_to_shape(self, shape: Sequence[int]) -> "Tensor":
+        return self._unary(load().hodu_host_sum_to_shape, _sizes(shape), len(shape))
+
     def dot(self, other: "Tensor") -> "Tensor":
         return self._unary(load().hodu_host_dot, other._h)
 
@@ -221,6 +234,24 @@ class Tensor:
     def view(self, shape: Sequence[int], strides: Sequence[int], offset: int = 0) -> "Tensor":
         """an arbitrary strided view over the same storage (what chained view ops produce)"""
         return self._unary(load().hodu_host_view, _sizes(shape), _sizes(strides), len(shape), offset)
+
+
+def _vjp(fn, a: Tensor, b: Tensor, grad: Tensor):
+    da, db = ctypes.c_void_p(), ctypes.c_void_p()
+    rc = fn(a._h, b._h, grad._h, ctypes.byref(da), ctypes.byref(db))
+    if rc != 0:
+        raise HoduError(rc, load().hodu_host_last_error().decode())
+    return Tensor(da.value), Tensor(db.value)
+
+
+def matmul_vjp(a: Tensor, b: Tensor, grad: Tensor):
+    """(dA, dB) of matmul(a, b) for the output gradient `grad` (tensor/gradient/vjp_matrix.rs:17-45)"""
+    return _vjp(load().hodu_host_matmul_vjp, a, b, grad)
+
+
+def dot_vjp(a: Tensor, b: Tensor, grad: Tensor):
+    """(dA, dB) of dot(a, b) (tensor/gradient/vjp_matrix.rs:46-67)"""
+    return _vjp(load().hodu_host_dot_vjp, a, b, grad)
 
 
 class Linear:

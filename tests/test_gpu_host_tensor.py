@@ -253,7 +253,7 @@ def test_linear_layer_with_deferred_f8_weight():
     got = T.Linear(tw, tb).forward(tx)
     s = T.stats()
     assert s == {"cast_kernels": 0, "contiguous_kernels": 0, "product_kernels": 1, "fused_products": 1, "bytes_copied": 0,
-                 "fused_steps": 1}
+                 "fused_steps": 1, "sum_kernels": 0}
     assert np.array_equal(got.to_bits(), _oracle_after("bf16", plain, [16, 300], [("add", b, V([300]))]))
 
 
@@ -301,3 +301,90 @@ def test_matmul_then_rejects_what_add_would_not_broadcast_along_the_last_axis():
     with pytest.raises(T.HoduError) as e:
         i.matmul_then(j, [("relu",)])
     assert e.value.kind == "RocmKernelError"
+
+
+# ---- backward through the path (tensor/gradient/vjp_matrix.rs) ------------------------------------------
+def _i32(values, shape):
+    return T.Tensor.from_bits(np.asarray(values, np.int32).view(np.uint32), "i32", shape)
+
+
+def _i32_of(t):
+    return t.to_bits().view(np.int32)
+
+
+def test_sum_and_sum_to_shape_follow_the_reference_shapes():
+    x = np.arange(2 * 3 * 4, dtype=np.int32)
+    t = _i32(x, [2, 3, 4])
+    a = x.reshape(2, 3, 4)
+    assert t.sum([0]).shape == [3, 4] and np.array_equal(_i32_of(t.sum([0])), a.sum(0).ravel())
+    assert t.sum([-1], keep_dim=True).shape == [2, 3, 1] and np.array_equal(_i32_of(t.sum([-1], True)), a.sum(2).ravel())
+    assert t.sum().shape == [] and _i32_of(t.sum())[0] == a.sum()  # tensor/ops/reduce.rs:154-156: no dims = all
+    assert t.sum([0, 2]).shape == [3] and np.array_equal(_i32_of(t.sum([0, 2])), a.sum((0, 2)))
+    # sum_to_shape (tensor/ops/reduce.rs:19-50): leading dims go, extent-1 dims of the target are kept
+    assert t.sum_to_shape([3, 4]).shape == [3, 4] and np.array_equal(_i32_of(t.sum_to_shape([3, 4])), a.sum(0).ravel())
+    assert t.sum_to_shape([1, 4]).shape == [1, 4] and np.array_equal(_i32_of(t.sum_to_shape([1, 4])), a.sum((0, 1)))
+    assert t.sum_to_shape([2, 1, 4]).shape == [2, 1, 4]
+    assert np.array_equal(_i32_of(t.sum_to_shape([2, 1, 4])), a.sum(1).ravel())
+    assert t.sum_to_shape([2, 3, 4]).shares_storage_with(t)
+    # a transposed view sums like its contiguous copy
+    assert np.array_equal(_i32_of(t.t().sum([1])), a.transpose(0, 2, 1).sum(1).ravel())
+
+
+def test_matmul_vjp_integers_exact_in_both_modes():
+    """dA = grad @ B^T, dB = A^T @ grad summed over the batch the weight was broadcast along: exact in i32, so the
+    literal path (batched product, then sum launches) and the folded one (batch inside the contraction) must agree
+    with numpy and with each other"""
+    g = H.rng(21)
+    a = g.integers(-9, 10, (4, 5, 6)).astype(np.int32)
+    w = g.integers(-9, 10, (6, 7)).astype(np.int32)
+    go = g.integers(-9, 10, (4, 5, 7)).astype(np.int32)
+    want_da = (go.astype(np.int64) @ w.T.astype(np.int64)).astype(np.int32)
+    want_dw = np.einsum("bmk,bmn->kn", a.astype(np.int64), go.astype(np.int64)).astype(np.int32)
+    ta, tw, tg = _i32(a, [4, 5, 6]), _i32(w, [6, 7]), _i32(go, [4, 5, 7])
+    for mode, sums in (("reference", 1), ("nocopy", 0)):
+        T.set_matmul_mode(mode)
+        T.stats(reset=True)
+        try:
+            da, dw = T.matmul_vjp(ta, tw, tg)
+            s = T.stats()
+        finally:
+            T.set_matmul_mode("nocopy")
+        assert da.shape == [4, 5, 6] and dw.shape == [6, 7]
+        assert np.array_equal(_i32_of(da), want_da.ravel()) and np.array_equal(_i32_of(dw), want_dw.ravel()), mode
+        assert s["sum_kernels"] == sums and s["product_kernels"] == 2, (mode, s)
+    # both operands batched, the lhs broadcast along a batch dim of extent 1: dA is summed with keep_dim
+    a1 = g.integers(-9, 10, (1, 5, 6)).astype(np.int32)
+    wb = g.integers(-9, 10, (4, 6, 7)).astype(np.int32)
+    da, dw = T.matmul_vjp(_i32(a1, [1, 5, 6]), _i32(wb, [4, 6, 7]), tg)
+    assert da.shape == [1, 5, 6] and dw.shape == [4, 6, 7]
+    assert np.array_equal(_i32_of(da), np.einsum("bmn,bkn->mk", go.astype(np.int64), wb.astype(np.int64)).astype(np.int32).ravel())
+    assert np.array_equal(_i32_of(dw), np.einsum("mk,bmn->bkn", a1[0].astype(np.int64), go.astype(np.int64)).astype(np.int32).ravel())
+    # dot: no broadcasting, no sums (vjp_matrix.rs:46-67)
+    da, dw = T.dot_vjp(_i32(a[0], [5, 6]), tw, _i32(go[0], [5, 7]))
+    assert np.array_equal(_i32_of(da), (go[0].astype(np.int64) @ w.T).astype(np.int32).ravel())
+    assert np.array_equal(_i32_of(dw), (a[0].T.astype(np.int64) @ go[0]).astype(np.int32).ravel())
+
+
+def test_linear_backward_bf16_against_f32_accumulated_comparator():
+    """x[8, 64, 256] @ w[256, 192] in bf16: dW through the folded product (K = 8 * 64 rows, operands row-dense) and
+    through the literal batched path both sit within the bf16 bar of the f32-accumulated result"""
+    g = H.rng(22)
+    x = H.f32_to_bf16_rne(g.standard_normal(8 * 64 * 256).astype(np.float32))
+    w = H.f32_to_bf16_rne((g.standard_normal(256 * 192) / 16).astype(np.float32))
+    go = H.f32_to_bf16_rne(g.standard_normal(8 * 64 * 192).astype(np.float32))
+    tx, tw, tg = (T.Tensor.from_bits(x, "bf16", [8, 64, 256]), T.Tensor.from_bits(w, "bf16", [256, 192]),
+                  T.Tensor.from_bits(go, "bf16", [8, 64, 192]))
+    xf, wf, gf = (H.bf16_to_f32(x).astype(np.float64).reshape(512, 256), H.bf16_to_f32(w).astype(np.float64).reshape(256, 192),
+                  H.bf16_to_f32(go).astype(np.float64).reshape(512, 192))
+    want_dw, abs_dw = xf.T @ gf, np.abs(xf).T @ np.abs(gf)
+    want_dx, abs_dx = gf @ wf.T, np.abs(gf) @ np.abs(wf).T
+    for mode in ("nocopy", "reference"):
+        T.set_matmul_mode(mode)
+        try:
+            dx, dw = T.matmul_vjp(tx, tw, tg)
+        finally:
+            T.set_matmul_mode("nocopy")
+        rel = H.rel_err(H.bf16_to_f32(dw.to_bits()).astype(np.float64), want_dw.ravel(), abs_dw.ravel(), 512)
+        assert rel.max() <= 2e-2, (mode, rel.max())
+        rel = H.rel_err(H.bf16_to_f32(dx.to_bits()).astype(np.float64), want_dx.ravel(), abs_dx.ravel(), 192)
+        assert rel.max() <= 2e-2, (mode, rel.max())
