@@ -40,9 +40,11 @@ INFINITY_CACHE_BYTES = 256 << 20
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc runs summarised under
 # profiles/ (FETCH_SIZE + WRITE_SIZE scaled by the copy-kernel calibration); None = not measured
 MEASURED_TRAFFIC = {
-    "mfma_bf16_pipe256x256w8_KK@c2": 100.0e6,
-    "gemv_bf16_f8w@c3_m1": 16.82e6,
-    "mfma_bf16_pipe256x256w8_KK@c5_down_bf16": 734.2e6,
+    "mfma_bf16_pipe256x256w8_KK@c2": 100.2e6,
+    "gemv_bf16_f8w@c3_m1": 16.83e6,
+    "gemv_bf16_f8w@gemv_14336x4096": 58.6e6,
+    "skinny_bf16_f8w_splitk@c3_m16": 22.2e6,
+    "mfma_bf16_pipe256x256w8_KK@c5_down_bf16": 734.5e6,
     "mfma_f8e4m3_pipe256x256_KK@f8_4096": 124.1e6,
 }
 
