@@ -317,6 +317,23 @@ int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, cons
     return launch_sum(ctx, dtype, in, out, r);
 }
 
+int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len, int causal) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "softmax: context is null");
+    if (!in || !out) return fail(HODU_ROCM_INVALID_ARG, "softmax: null operand pointer");
+    if (in == out) return fail(HODU_ROCM_INVALID_ARG, "softmax: out aliases the input");
+    Reduction r;
+    int rc = parse_reduce_metadata(md, len, &r);
+    if (rc) return rc;
+    const size_t nd = md[0], out_nd = md[2 + 2 * nd], n_red = md[3 + 2 * nd + out_nd];
+    if (n_red != 1) return fail(HODU_ROCM_INVALID_ARG, "softmax: exactly one dim, got %zu", n_red);
+    const size_t dim = md[4 + 2 * nd + out_nd];
+    const bool last = dim + 1 == nd;
+    if (causal && (!last || nd < 2)) return fail(HODU_ROCM_INVALID_ARG, "softmax: the causal mask needs the last dim of a matrix");
+    HODU_HIP(hipSetDevice(ctx->device));
+    return launch_softmax(ctx, dtype, in, out, r, last, causal ? 1 : 0, nd >= 2 ? (long)md[1 + nd - 2] : 1);
+}
+
 int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "contiguous: context is null");

@@ -164,6 +164,10 @@ struct Reduction {
 };
 int parse_reduce_metadata(const size_t *md, size_t len, Reduction *r);
 int launch_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r);
+// softmax over the one reduced dim of `r`; dim_is_last: it is the tensor's last dim; causal: entries j > i of every
+// [sq, len] matrix count as -inf
+int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, bool dim_is_last,
+                   int causal, long sq);
 
 int launch_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const Strided &s);
 int launch_gather(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Strided &s);

@@ -1,0 +1,166 @@
+// Softmax along one dim, as one kernel.  Tensor::softmax (crates/hodu_core/src/tensor/ops/normalization.rs:4-21) is
+// five launches in the reference -- max(keep_dim), sub, exp, sum(keep_dim), div -- each a full pass over the tensor
+// with a rounding to the storage type in between; scaled_dot_product_attention (crates/hodu_nn/src/modules/
+// attention.rs:25-70) runs it on the [.., Sq, Sk] scores between its two batched products, after an optional causal
+// masked_fill(-inf) (:40-48, mask[i][j] = j > i, :73-86).
+//
+// Here a row is read once: a wavefront owns a row whose dim is dense and at most 4096 long and keeps it in
+// registers (max, exp, sum, scale without touching memory again); longer or strided rows take three passes from
+// memory with a thread per row.  Arithmetic: elements widened exactly to f32 (f64 stays f64), exp and the sum in that
+// type, one rounding (RNE) on store.  With `causal` the entries j > i of each [Sq, Sk] matrix count as -inf: they
+// come out as exact zeros, and the mask tensor is never built.
+#include "common.hpp"
+#include "device_types.hpp"
+#include "elem.hpp"
+
+namespace hodu {
+namespace {
+
+struct DevSoftmax {
+    long rows;         // kept positions
+    long len;          // extent of the softmax dim
+    long stride;       // its element stride in the input
+    long offset;
+    int kept_n;
+    long kept_shape[16], kept_stride[16];
+    int causal;        // 1: mask j > i, i = the row's index along the innermost kept dim (extent sq)
+    long sq;
+};
+
+__device__ __forceinline__ long row_offset(const DevSoftmax &s, long row) {
+    long off = 0;
+    for (int d = s.kept_n - 1; d >= 0; d--) {
+        off += (row % s.kept_shape[d]) * s.kept_stride[d];
+        row /= s.kept_shape[d];
+    }
+    return off;
+}
+
+template <class W> __device__ __forceinline__ W wexp(W x);
+template <> __device__ __forceinline__ float wexp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double wexp<double>(double x) { return exp(x); }
+
+template <class W> __device__ __forceinline__ W lanes_max(W v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const W o = __shfl_xor(v, m, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+template <class W> __device__ __forceinline__ W lanes_add(W v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+// one wavefront per row, the row (dense, len <= 64 * NPL) held in registers
+template <class E, int NPL>
+__global__ __launch_bounds__(256) void softmax_row_kernel(const typename E::storage *__restrict__ in,
+                                                         typename E::storage *__restrict__ out, DevSoftmax s) {
+    typedef typename E::acc W;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= s.rows) return;
+    const typename E::storage *x = in + s.offset + row_offset(s, row);
+    const long limit = s.causal ? (row % s.sq) + 1 : s.len;  // entries at or beyond `limit` are masked
+    const W ninf = -(W)INFINITY;
+    W v[NPL];
+    W m = ninf;
+#pragma unroll
+    for (int i = 0; i < NPL; i++) {
+        const long j = lane + 64L * i;
+        v[i] = (j < s.len && j < limit) ? (W)E::load(x[j]) : ninf;
+        m = v[i] > m ? v[i] : m;
+    }
+    m = lanes_max(m);
+    W sum = (W)0;
+#pragma unroll
+    for (int i = 0; i < NPL; i++) {
+        v[i] = v[i] == ninf ? (W)0 : wexp<W>(v[i] - m);
+        sum += v[i];
+    }
+    sum = lanes_add(sum);
+    typename E::storage *y = out + row * s.len;
+#pragma unroll
+    for (int i = 0; i < NPL; i++) {
+        const long j = lane + 64L * i;
+        if (j < s.len) y[j] = E::store(v[i] / sum);
+    }
+}
+
+// any stride, any length: a thread per row, three passes from memory
+template <class E>
+__global__ __launch_bounds__(256) void softmax_strided_kernel(const typename E::storage *__restrict__ in,
+                                                             typename E::storage *__restrict__ out, DevSoftmax s) {
+    typedef typename E::acc W;
+    const long row = (long)blockIdx.x * 256 + threadIdx.x;
+    if (row >= s.rows) return;
+    const typename E::storage *x = in + s.offset + row_offset(s, row);
+    const long limit = s.causal ? ((row % s.sq) + 1 < s.len ? (row % s.sq) + 1 : s.len) : s.len;
+    W m = -(W)INFINITY;
+    for (long j = 0; j < limit; j++) {
+        const W v = (W)E::load(x[j * s.stride]);
+        m = v > m ? v : m;
+    }
+    W sum = (W)0;
+    for (long j = 0; j < limit; j++) sum += wexp<W>((W)E::load(x[j * s.stride]) - m);
+    typename E::storage *y = out + row * s.len;
+    for (long j = 0; j < s.len; j++) y[j] = E::store(j < limit ? wexp<W>((W)E::load(x[j * s.stride]) - m) / sum : (W)0);
+}
+
+template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const DevSoftmax &s, bool dim_is_last) {
+    typedef typename E::storage S;
+    if (s.rows == 0 || s.len == 0) return HODU_ROCM_OK;
+    // the row kernel writes row `r` at out + r * len: the softmax dim must be the output's last dim
+    if (dim_is_last && s.stride == 1 && s.len <= 4096) {
+        const long blocks = (s.rows + 3) / 4;
+        if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "softmax needs %ld workgroups", blocks);
+        ctx->last_kernel = "softmax_row";
+#define LAUNCH(NPL) hipLaunchKernelGGL((softmax_row_kernel<E, NPL>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s)
+        if (s.len <= 64 * 2) LAUNCH(2);
+        else if (s.len <= 64 * 8) LAUNCH(8);
+        else if (s.len <= 64 * 16) LAUNCH(16);
+        else if (s.len <= 64 * 32) LAUNCH(32);
+        else LAUNCH(64);
+#undef LAUNCH
+        HODU_HIP(hipGetLastError());
+        return HODU_ROCM_OK;
+    }
+    if (!dim_is_last) return fail(HODU_ROCM_UNSUPPORTED, "softmax: only the last dim is supported");
+    const long blocks = (s.rows + 255) / 256;
+    if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "softmax needs %ld workgroups", blocks);
+    ctx->last_kernel = "softmax_strided";
+    hipLaunchKernelGGL(softmax_strided_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
+}  // namespace
+
+// r: the reduction over the softmax dim as parsed from reduce_metadata (one reduced dim); last_dim: that dim is
+// the tensor's last; sq: extent of the dim before it (for the causal mask)
+int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, bool dim_is_last,
+                   int causal, long sq) {
+    DevSoftmax s{};
+    s.rows = r.n_out;
+    s.len = r.reduce_size;
+    s.stride = r.red_n > 0 ? r.red_stride[0] : 1;
+    s.offset = r.offset;
+    s.kept_n = r.kept_n;
+    for (int d = 0; d < 16; d++) {
+        s.kept_shape[d] = d < r.kept_n ? r.kept_shape[d] : 1;
+        s.kept_stride[d] = d < r.kept_n ? r.kept_stride[d] : 0;
+    }
+    s.causal = causal;
+    s.sq = sq > 0 ? sq : 1;
+    switch (dtype) {
+    case HODU_BF16: return run<Elem<HODU_BF16>>(ctx, in, out, s, dim_is_last);
+    case HODU_F16: return run<Elem<HODU_F16>>(ctx, in, out, s, dim_is_last);
+    case HODU_F32: return run<Elem<HODU_F32>>(ctx, in, out, s, dim_is_last);
+    case HODU_F64: return run<Elem<HODU_F64>>(ctx, in, out, s, dim_is_last);
+    default: return fail(HODU_ROCM_UNSUPPORTED, "softmax: dtype id %d is not bf16 / f16 / f32 / f64", dtype);
+    }
+}
+
+}  // namespace hodu

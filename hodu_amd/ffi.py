@@ -119,6 +119,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
+    lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
     _lib = lib
     return lib
 
@@ -295,6 +296,19 @@ class Context:
                 raise HoduRocmError(INVALID_ARG, f"sum_{dt}: metadata reaches past a device buffer")
         arr, n = _md_array(md)
         self._check(self.lib.hodu_rocm_sum(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n))
+
+    def softmax(self, dt: str, x: DeviceBuffer, out: DeviceBuffer, md, causal: bool = False):
+        """hodu_rocm_softmax: md is reduce_metadata of the input layout with the softmax dim reduced; the output is
+        contiguous in the input's shape"""
+        m = [int(v) for v in md]
+        if m and len(m) >= 2 + 2 * m[0]:
+            nd = m[0]
+            span = _view_span(m[1:1 + nd], m[1 + nd:1 + 2 * nd], m[1 + 2 * nd])
+            n = int(np.prod(m[1:1 + nd], dtype=np.int64)) if nd else 1
+            if span * DTYPE_SIZE[dt] > x.nbytes or n * DTYPE_SIZE[dt] > out.nbytes:
+                raise HoduRocmError(INVALID_ARG, f"softmax_{dt}: metadata reaches past a device buffer")
+        arr, n_md = _md_array(md)
+        self._check(self.lib.hodu_rocm_softmax(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n_md, int(bool(causal))))
 
     def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int,
                      graph: bool = False, steps=None) -> float:

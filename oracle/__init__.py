@@ -186,6 +186,16 @@ def sum_spec(dt: str, x: np.ndarray, md, decode=F8_OCP):
     return o32, o64, oabs
 
 
+def softmax_spec(dt: str, x: np.ndarray, md, causal: bool = False):
+    """(f32, f64) softmax along the single reduced dim of md, contiguous in the input's shape"""
+    md = _md(md)
+    nd = int(md[0])
+    n = int(np.prod([int(v) for v in md[1:1 + nd]], dtype=np.int64)) if nd else 1
+    o32, o64 = np.empty(n, np.float32), np.empty(n, np.float64)
+    _check(lib().oracle_softmax_spec(DTYPE_ID[dt], _ptr(x), _ptr(md), int(causal), _ptr(o32), _ptr(o64)), "softmax_spec")
+    return o32, o64
+
+
 def f8e4m3_table(decode: int) -> np.ndarray:
     """All 256 decoded values as f32."""
     return np.array([lib().oracle_f8e4m3_to_f32(b, decode) for b in range(256)], dtype=np.float32)
@@ -279,4 +289,32 @@ class RefLib:
         fn = getattr(self.lib, f"hodu_cpu_sum_{dt}")
         fn.restype = None
         fn(_ptr(x), _ptr(out), _ptr(md))
+        return out
+
+    def softmax_chain_f32(self, x, shape):
+        """Tensor::softmax(-1) on a contiguous f32 tensor as the reference runs it: hodu_cpu_max_f32 (keep_dim),
+        sub_f32, exp_f32, sum_f32 (keep_dim), div_f32 (normalization.rs:14-20)"""
+        shape = [int(v) for v in shape]
+        nd, n = len(shape), int(np.prod(shape))
+        strides = [int(np.prod(shape[i + 1:])) for i in range(nd)]
+        red = _md([nd] + shape + strides + [0, nd] + shape[:-1] + [1] + [1, nd - 1, 1, shape[-1]])
+        kept = shape[:-1] + [1]
+        kstr = [int(np.prod(kept[i + 1:])) for i in range(nd)]
+        bstr = kstr[:-1] + [0]
+        binary = _md([n, nd] + shape + shape + strides + bstr + [0, 0])
+        unary = _md([n, nd] + shape + strides + [0])
+
+        def call(name, *args):
+            fn = getattr(self.lib, name)
+            fn.restype = None
+            fn(*[_ptr(a) for a in args])
+
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        mx = np.empty(n // shape[-1], np.float32)
+        call("hodu_cpu_max_f32", x, mx, red)
+        shifted, e, sm, out = np.empty(n, np.float32), np.empty(n, np.float32), np.empty(n // shape[-1], np.float32), np.empty(n, np.float32)
+        call("hodu_cpu_sub_f32", x, mx, shifted, binary)
+        call("hodu_cpu_exp_f32", shifted, e, unary)
+        call("hodu_cpu_sum_f32", e, sm, red)
+        call("hodu_cpu_div_f32", e, sm, out, binary)
         return out

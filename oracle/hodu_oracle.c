@@ -19,6 +19,8 @@
  *   sum      crates/hodu_cpu_kernels/kernels/ops_reduce.c:47-118 (generic macro: one output at a time, the reduced
  *            dims walked innermost first, accumulator in the storage type -- bf16 / f16 / f8 re-round after every
  *            add, :127-130), :133-237 (f32; a lane-wise SIMD order only when the last, dense dim alone is reduced)
+ *   softmax  crates/hodu_core/src/tensor/ops/normalization.rs:4-21 (max(keep_dim), sub, exp, sum(keep_dim), div) with
+ *            the causal masked_fill(-inf) of crates/hodu_nn/src/modules/attention.rs:40-48, :73-86 (mask j > i)
  *   mul_scalar, relu
  *            crates/hodu_cpu_kernels/kernels/ops_unary.c:138-200, :352-386 (scalar arrives in the storage type),
  *            :648-697, :1233, :1319, :1404, :1484 ((x > 0) ? x : 0 in f32)
@@ -49,6 +51,12 @@
  * sum: ASIS is compared bit for bit with oracle/_ref on every dtype and layout, except f32 / f64 sums over the last
  * dense dim alone, where the reference adds lane-wise (SIMD width of the build) and only a tolerance applies: the
  * bits of that one case are parity unpinned.  Integer sums against numpy; SPEC against float64.
+ *
+ * softmax: the comparator computes the function itself in f32 and f64 on exactly widened inputs (one rounding, none in
+ * between); it is held against a float64 numpy softmax, against sum-to-one and shift invariance, and -- for f32 --
+ * against the five-kernel chain run through oracle/_ref (hodu_cpu_max / sub / exp / sum / div), which it matches to
+ * rounding.  The reference's bf16 / f16 chain rounds after every kernel and accumulates the sum in the narrow type;
+ * as for the products, the GPU is gated against the f32 comparator, not against that chain.
  *
  * Parity unpinned: float->integer casts of out-of-range or NaN inputs are undefined behaviour
  * in the reference C ((T)x) and are not checked.
@@ -815,6 +823,54 @@ int oracle_sum_spec(int dt, int f8_decode, const void *in, const size_t *md, flo
         if (out32) out32[o] = s32;
         if (out64) out64[o] = s64;
         if (out_abs) out_abs[o] = sabs;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* softmax along one dim (normalization.rs:4-21), comparator form                                */
+/* ------------------------------------------------------------------------------------------ */
+/* md: reduce_metadata of the input with the softmax dim as the single reduced dim.  out32 / out64: the function in
+ * f32 (expf, f32 sum in index order) and in f64, contiguous in the input's shape.  causal: entries j > i of every
+ * [.., Sq, Sk] matrix (softmax dim last) are -inf before the softmax (attention.rs:40-48). */
+int oracle_softmax_spec(int dt, const void *in, const size_t *md, int causal, float *out32, double *out64) {
+    if (dt != DT_BF16 && dt != DT_F16 && dt != DT_F32 && dt != DT_F64) return -1;
+    reduce_space r;
+    reduce_space_from(md, &r);
+    if (r.n_red != 1) return -1;
+    const size_t dim = r.red[0], len = r.dims[dim];
+    if (causal && (dim + 1 != r.nd || r.nd < 2)) return -1;
+    const size_t sq = r.nd >= 2 ? r.dims[r.nd - 2] : 1;
+    size_t inner = 1;  /* contiguous output: elements between consecutive entries of the softmax dim */
+    for (size_t d = dim + 1; d < r.nd; d++) inner *= r.dims[d];
+    _Pragma("omp parallel for schedule(static)")
+    for (size_t o = 0; o < r.n_out; o++) {
+        /* n_out counts the kept positions (keep_dim or not): o = outer * inner + in_pos */
+        const size_t outer = o / inner, in_pos = o % inner;
+        const size_t limit = causal ? ((o % sq) + 1 < len ? (o % sq) + 1 : len) : len;
+        double m64 = -INFINITY;
+        float m32 = -INFINITY;
+        for (size_t j = 0; j < limit; j++) {
+            const size_t pos = reduce_pos(&r, o, j);
+            const double v = dt == DT_F64 ? ((const double *)in)[pos] : (double)widen_any(dt, in, pos, F8_DECODE_OCP);
+            if (v > m64) m64 = v;
+            if ((float)v > m32) m32 = (float)v;
+        }
+        double s64 = 0.0;
+        float s32 = 0.0f;
+        for (size_t j = 0; j < limit; j++) {
+            const size_t pos = reduce_pos(&r, o, j);
+            const double v = dt == DT_F64 ? ((const double *)in)[pos] : (double)widen_any(dt, in, pos, F8_DECODE_OCP);
+            s64 += exp(v - m64);
+            s32 += expf((float)v - m32);
+        }
+        for (size_t j = 0; j < len; j++) {
+            const size_t pos = reduce_pos(&r, o, j);
+            const double v = dt == DT_F64 ? ((const double *)in)[pos] : (double)widen_any(dt, in, pos, F8_DECODE_OCP);
+            const size_t q = (outer * len + j) * inner + in_pos;
+            if (out64) out64[q] = j < limit ? exp(v - m64) / s64 : 0.0;
+            if (out32) out32[q] = j < limit ? expf((float)v - m32) / s32 : 0.0f;
+        }
     }
     return 0;
 }

@@ -355,3 +355,36 @@ def test_sums_against_numpy():
     ones = np.full(513, 0x3F80, dtype=np.uint16)
     assert oracle.sum_asis("bf16", ones, H.reduce_md(V([513]), [0], False))[0] == 0x4380  # 256.0
     assert oracle.sum_spec("bf16", ones, H.reduce_md(V([513]), [0], False))[0][0] == 513.0
+
+
+# ---------------------------------------------------------------------------------------------
+# softmax (the step between attention's two products)
+# ---------------------------------------------------------------------------------------------
+def test_softmax_comparator_against_numpy_and_invariants():
+    V = H.View
+    g = H.rng(41)
+    x = (g.standard_normal(3 * 5 * 17) * 3).astype(np.float32)
+    md = H.reduce_md(V([3, 5, 17]), [2], True)
+    o32, o64 = oracle.softmax_spec("f32", x, md)
+    a = x.astype(np.float64).reshape(3, 5, 17)
+    e = np.exp(a - a.max(-1, keepdims=True))
+    want = (e / e.sum(-1, keepdims=True)).ravel()
+    assert np.allclose(o64, want, rtol=1e-14, atol=0) and np.allclose(o32, want, rtol=2e-6, atol=1e-12)
+    assert np.allclose(o64.reshape(15, 17).sum(1), 1.0, rtol=1e-14)
+    # shift invariance: softmax(x + c) == softmax(x)
+    assert np.allclose(oracle.softmax_spec("f32", x + np.float32(7.0), md)[1], o64, rtol=1e-5)
+    # a dim that is not the last one, through a transposed view
+    vt = V([3, 5, 17]).t(1, 2)  # [3, 17, 5] strided, softmax over what used to be the last dim
+    o64t = oracle.softmax_spec("f32", x, H.reduce_md(vt, [1], True))[1]
+    assert np.allclose(o64t.reshape(3, 17, 5), want.reshape(3, 5, 17).transpose(0, 2, 1), rtol=1e-14)
+    # causal (crates/hodu_nn/src/modules/attention.rs:73-86: masked where j > i): row i is a softmax of its first i + 1 entries
+    s = (g.standard_normal(2 * 6 * 6)).astype(np.float32)
+    c64 = oracle.softmax_spec("f32", s, H.reduce_md(V([2, 6, 6]), [2], True), causal=True)[1].reshape(2, 6, 6)
+    b = s.astype(np.float64).reshape(2, 6, 6)
+    for i in range(6):
+        row = np.exp(b[:, i, :i + 1] - b[:, i, :i + 1].max(-1, keepdims=True))
+        assert np.allclose(c64[:, i, :i + 1], row / row.sum(-1, keepdims=True), rtol=1e-14)
+        assert np.all(c64[:, i, i + 1:] == 0.0)
+    # bf16 inputs are widened exactly
+    xb = H.f32_to_bf16_rne(x)
+    assert np.allclose(oracle.softmax_spec("bf16", xb, md)[1], oracle.softmax_spec("f32", H.bf16_to_f32(xb), md)[1], rtol=0, atol=0)

@@ -106,3 +106,13 @@ def test_sums_match_compiled_reference(ref, dt):
         x = H.random_storage(dt, v.span(), 500 + n, 2.0)
         md = H.reduce_md(v, dims, keep)
         assert np.array_equal(_bits(oracle.sum_asis(dt, x, md)), _bits(ref.sum(dt, x, md))), (dt, n)
+
+
+def test_softmax_comparator_matches_the_reference_five_kernel_chain(ref):
+    """Tensor::softmax(-1) as hodu runs it on f32 (max, sub, exp, sum, div through the compiled reference kernels)
+    against the one-pass comparator: the same function to rounding"""
+    V = H.View
+    x = (H.rng(42).standard_normal(4 * 9 * 33) * 4).astype(np.float32)
+    chain = ref.softmax_chain_f32(x, [4, 9, 33])
+    o32, o64 = oracle.softmax_spec("f32", x, H.reduce_md(V([4, 9, 33]), [2], True))
+    assert np.allclose(chain, o64, rtol=3e-6, atol=1e-12) and np.allclose(chain, o32, rtol=3e-6, atol=1e-12)
