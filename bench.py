@@ -221,6 +221,48 @@ def time_case(ctx, case, steps, warmup, graph=False):
             "tflops": tflops, "algorithmic_gbs": gbs, "weight_buffers_rotated": copies, "roofline": roof}
 
 
+def attention_probe(ctx, steps):
+    """not a BASELINE configuration: hodu_nn's scaled_dot_product_attention (causal, bf16, 32 heads x 2048 x 128) as
+    the three launches the host mirror issues -- Q K^T with the scale in its store, masked softmax, P V -- each timed
+    with HIP events around `steps` back-to-back launches"""
+    import helpers as H
+    from hodu_amd import ffi
+    V = H.View
+    heads, s_len, d = 32, 2048, 128
+    q, k, v = (ctx.upload(bf16(normal(950 + i, heads * s_len * d))) for i in range(3))
+    scores, probs = ctx.alloc(heads * s_len * s_len * 2), ctx.alloc(heads * s_len * s_len * 2)
+    out = ctx.alloc(heads * s_len * d * 2)
+    md_qk = H.matmul_md(V([heads, s_len, d]), V([heads, s_len, d]).t())
+    md_pv = H.matmul_md(V([heads, s_len, s_len]), V([heads, s_len, d]))
+    md_sm = H.reduce_md(V([heads, s_len, s_len]), [2], True)
+    scale = [ffi.mul_scalar(bf16(np.array([1.0 / np.sqrt(d)], dtype=np.float32)))]
+    legs = {
+        "qk_scaled": lambda: ctx.product_ex("matmul", "bf16", q, k, scores, md_qk, scale),
+        "softmax_causal": lambda: ctx.softmax("bf16", scores, probs, md_sm, True),
+        "pv": lambda: ctx.product("matmul", "bf16", probs, v, out, md_pv),
+    }
+    res, total = {}, 0.0
+    for name, fn in legs.items():
+        for _ in range(3):
+            fn()
+        ctx.sync()
+        t = ctx.timer()
+        t.start()
+        for _ in range(steps):
+            fn()
+        us = t.stop_ms() * 1e3 / steps
+        res[name] = {"us": us, "kernel": ctx.last_kernel()}
+        total += us
+    flops = 2 * 2.0 * heads * s_len * s_len * d
+    res["qk_scaled"]["tflops"] = flops / 2 / res["qk_scaled"]["us"] / 1e6
+    res["pv"]["tflops"] = flops / 2 / res["pv"]["us"] / 1e6
+    res["softmax_causal"]["gbs"] = 2.0 * heads * s_len * s_len * 2 / res["softmax_causal"]["us"] / 1e3
+    for b in (q, k, v, scores, probs, out):
+        b.free()
+    return {"config": "attention", "shape": f"bf16 q,k,v [{heads},{s_len},{d}], causal", "us_total": total,
+            "tflops_total": flops / total / 1e6, "legs": res}
+
+
 def mfma_clock_probe(ctx):
     """what the matrix cores sustain from registers (no LDS, no memory traffic), and at which shader clock, on
     constant and on N(0,1) operands: the clock under full MFMA load depends on the data"""
@@ -325,6 +367,10 @@ def main():
         ctx.sync()
         print(json.dumps({"config": "copy", "kernel": ctx.last_kernel(), "bytes_read": 4 * n, "bytes_written": 4 * n,
                           "launches": args.steps}))
+        ctx.close()
+        return
+    if args.only == "attention":
+        print(json.dumps(attention_probe(ctx, args.steps)))
         ctx.close()
         return
     if args.only == "clock":

@@ -89,6 +89,55 @@ __global__ __launch_bounds__(256) void softmax_row_kernel(const typename E::stor
     }
 }
 
+// the same with 16-byte accesses: a lane holds NV vectors of V neighbouring entries (len a multiple of V, rows and
+// bases 16-byte aligned)
+template <class E, int NV, int V>
+__global__ __launch_bounds__(256) void softmax_row_vec_kernel(const typename E::storage *__restrict__ in,
+                                                             typename E::storage *__restrict__ out, DevSoftmax s) {
+    typedef typename E::acc W;
+    typedef typename E::storage S;
+    struct alignas(16) Vec { S e[V]; };
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= s.rows) return;
+    const S *x = in + s.offset + row_offset(s, row);
+    const long limit = s.causal ? (row % s.sq) + 1 : s.len;
+    const W ninf = -(W)INFINITY;
+    W v[NV][V];
+    W m = ninf;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const long j0 = (lane + 64L * i) * V;
+        Vec raw;
+        if (j0 < s.len && j0 < limit) raw = *reinterpret_cast<const Vec *>(x + j0);
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+            v[i][e] = (j0 + e < s.len && j0 + e < limit) ? (W)E::load(raw.e[e]) : ninf;
+            m = v[i][e] > m ? v[i][e] : m;
+        }
+    }
+    m = lanes_max(m);
+    W sum = (W)0;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+            v[i][e] = v[i][e] == ninf ? (W)0 : wexp<W>(v[i][e] - m);
+            sum += v[i][e];
+        }
+    sum = lanes_add(sum);
+    S *y = out + row * s.len;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const long j0 = (lane + 64L * i) * V;
+        if (j0 >= s.len) continue;
+        Vec o;
+#pragma unroll
+        for (int e = 0; e < V; e++) o.e[e] = E::store(v[i][e] / sum);
+        *reinterpret_cast<Vec *>(y + j0) = o;
+    }
+}
+
 // any stride, any length: a thread per row, three passes from memory
 template <class E>
 __global__ __launch_bounds__(256) void softmax_strided_kernel(const typename E::storage *__restrict__ in,
@@ -116,6 +165,22 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
     if (dim_is_last && s.stride == 1 && s.len <= 4096) {
         const long blocks = (s.rows + 3) / 4;
         if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "softmax needs %ld workgroups", blocks);
+        constexpr int V = 16 / (int)sizeof(S);
+        bool vec = s.len % V == 0 && s.offset % V == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0;
+        for (int d = 0; d < s.kept_n; d++) vec = vec && s.kept_stride[d] % V == 0;
+        if (vec) {
+            ctx->last_kernel = "softmax_row_vec";
+            const long vecs = s.len / V;
+#define LAUNCHV(NV) hipLaunchKernelGGL((softmax_row_vec_kernel<E, NV, V>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s)
+            if (vecs <= 64) LAUNCHV(1);
+            else if (vecs <= 128) LAUNCHV(2);
+            else if (vecs <= 256) LAUNCHV(4);
+            else if (vecs <= 512) LAUNCHV(8);
+            else LAUNCHV(64 / V);  // up to 4096 entries
+#undef LAUNCHV
+            HODU_HIP(hipGetLastError());
+            return HODU_ROCM_OK;
+        }
         ctx->last_kernel = "softmax_row";
 #define LAUNCH(NPL) hipLaunchKernelGGL((softmax_row_kernel<E, NPL>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s)
         if (s.len <= 64 * 2) LAUNCH(2);

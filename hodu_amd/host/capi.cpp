@@ -93,6 +93,18 @@ int hodu_host_linear(const hodu_host_tensor *input, const hodu_host_tensor *weig
 }
 long hodu_host_stats_fused_steps(void) { return stats().fused_steps; }
 long hodu_host_stats_sum_kernels(void) { return stats().sum_kernels; }
+long hodu_host_stats_softmax_kernels(void) { return stats().softmax_kernels; }
+int hodu_host_softmax(const hodu_host_tensor *t, int dim, int causal, hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(T(t)->softmax(dim, causal != 0))); });
+}
+int hodu_host_attention(const hodu_host_tensor *q, const hodu_host_tensor *k, const hodu_host_tensor *v, int is_causal,
+                        hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(Tensor::scaled_dot_product_attention(*T(q), *T(k), *T(v), is_causal != 0))); });
+}
+// the scalar `value` in dtype's storage (round-to-nearest-even), for mul_scalar steps; returns the byte count
+int hodu_host_scalar_bits(int dtype, double value, unsigned char out[8], size_t *n) {
+    return guarded([&] { *n = Tensor::scalar_bits(dtype_of(dtype), value, out); });
+}
 int hodu_host_sum(const hodu_host_tensor *t, const int *dims, size_t n_dims, int keep_dim, hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(T(t)->sum(std::vector<int>(dims, dims + n_dims), keep_dim != 0))); });
 }

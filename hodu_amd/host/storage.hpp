@@ -37,9 +37,9 @@ inline const char *dtype_name(DType d) {
 struct Stats {
     std::atomic<long> cast_kernels{0}, contiguous_kernels{0}, product_kernels{0}, fused_products{0};
     std::atomic<long> fused_steps{0};        // element-wise kernels that ran inside a product's store instead
-    std::atomic<long> sum_kernels{0};
+    std::atomic<long> sum_kernels{0}, softmax_kernels{0};
     std::atomic<long long> bytes_copied{0};  // written by cast/contiguous passes
-    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = sum_kernels = 0; bytes_copied = 0; }
+    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = sum_kernels = softmax_kernels = 0; bytes_copied = 0; }
 };
 inline Stats &stats() {
     static Stats s;
@@ -191,6 +191,19 @@ public:
         if (n_out == 0) return out;
         dev_->check(hodu_rocm_sum(dev_->ctx(), (int)dtype_, ptr(), (void *)out.ptr(), md.data(), md.size()), "sum");
         stats().sum_kernels++;
+        return out;
+    }
+
+    // Tensor::softmax (tensor/ops/normalization.rs:4-21) as one launch; output fresh and contiguous in the input's shape
+    RocmStorage call_ops_softmax(const Layout &layout, size_t dim, bool causal) const {
+        check_span(layout, "softmax");
+        if (deferred()) return gather(layout).call_ops_softmax(Layout::from_shape(layout.shape()), dim, causal);
+        const Metadata md = reduce_metadata(layout, {dim}, true);
+        RocmStorage out = fresh(dtype_, layout.size());
+        if (layout.size() == 0) return out;
+        dev_->check(hodu_rocm_softmax(dev_->ctx(), (int)dtype_, ptr(), (void *)out.ptr(), md.data(), md.size(), causal ? 1 : 0),
+                    "softmax");
+        stats().softmax_kernels++;
         return out;
     }
 

@@ -3,6 +3,8 @@
 // (storage, layout) pair; views share the storage (tensor/internal.rs:50-79).
 #pragma once
 
+#include <cmath>
+
 #include "storage.hpp"
 
 namespace hodu_host {
@@ -192,6 +194,65 @@ public:
     // tensor/gradient/vjp_matrix.rs:46-67
     static Grads dot_vjp(const Tensor &a, const Tensor &b, const Tensor &grad) {
         return {grad.dot(b.transpose(-2, -1)), a.transpose(-2, -1).dot(grad)};
+    }
+
+    // ---- attention's middle step and the function around it ---------------------------------------------------
+    // tensor/ops/normalization.rs:4-21, one launch instead of five; only the last dim (what attention uses).
+    // causal: the masked_fill(-inf) of attention.rs:40-48 folded in.
+    Tensor softmax(int dim, bool causal = false) const {
+        const size_t d = layout_.axis(dim);
+        if (d + 1 != layout_.ndim())
+            throw Error(ErrorKind::InvalidArgument, "softmax: only the last dim is supported on this device");
+        auto out = std::make_shared<RocmStorage>(storage_->call_ops_softmax(layout_, d, causal));
+        return Tensor(out, Layout::from_shape(shape()));
+    }
+
+    // `value` as a scalar of dtype `dt`, round-to-nearest-even (what Scalar::to_dtype does through the `half` crate's
+    // from_f32 for bf16 / f16: scalar.rs:391-404); only the floating dtypes
+    static size_t scalar_bits(DType dt, double value, unsigned char out[8]) {
+        std::memset(out, 0, 8);
+        const float f = (float)value;
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        switch (dt) {
+        case DType::F64: std::memcpy(out, &value, 8); return 8;
+        case DType::F32: std::memcpy(out, &f, 4); return 4;
+        case DType::BF16: {
+            const uint16_t h = (u & 0x7F800000u) == 0x7F800000u ? (uint16_t)(u >> 16) : (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+            std::memcpy(out, &h, 2);
+            return 2;
+        }
+        case DType::F16: {
+            const uint32_t sign = (u >> 16) & 0x8000u, absu = u & 0x7FFFFFFFu;
+            uint16_t h;
+            if (absu >= 0x7F800000u) h = (uint16_t)(sign | 0x7C00u | (absu > 0x7F800000u ? 0x200u : 0u));
+            else if (absu >= 0x477FF000u) h = (uint16_t)(sign | 0x7C00u);  // rounds to infinity
+            else if (absu < 0x33000001u) h = (uint16_t)sign;                // below half the smallest subnormal
+            else {
+                int e = (int)(absu >> 23) - 127;
+                uint32_t m = (absu & 0x7FFFFFu) | 0x800000u;
+                int shift = e < -14 ? 13 + (-14 - e) : 13;                   // subnormal results lose more bits
+                uint32_t r = m >> shift, rem = m & ((1u << shift) - 1), half = 1u << (shift - 1);
+                if (rem > half || (rem == half && (r & 1u))) r++;
+                h = e < -14 ? (uint16_t)(sign | r) : (uint16_t)(sign | (((uint32_t)(e + 15) << 10) + (r - 0x400u)));
+            }
+            std::memcpy(out, &h, 2);
+            return 2;
+        }
+        default: throw Error(ErrorKind::UnsupportedDTypeForOp, "attention: floating dtypes only");
+        }
+    }
+
+    // scaled_dot_product_attention (hodu_nn/src/modules/attention.rs:25-70) without attn_mask and dropout:
+    // softmax(Q K^T / sqrt(d_k) [+ causal mask]) V as three launches -- the scale rides in the first product's
+    // store, the mask and the five softmax kernels are one kernel, the second product is plain.
+    static Tensor scaled_dot_product_attention(const Tensor &q, const Tensor &k, const Tensor &v, bool is_causal) {
+        if (q.layout().ndim() < 2) throw Error(ErrorKind::InvalidArgument, "attention: query needs at least two dimensions");
+        const double scale = 1.0 / std::sqrt((double)q.shape().back());
+        unsigned char bits[8];
+        const size_t n = scalar_bits(q.dtype(), scale, bits);
+        const Tensor scores = q.matmul_then(k.transpose(-2, -1), {Then::mul_scalar(bits, n)});
+        return scores.softmax(-1, is_causal).matmul(v);
     }
 
 private:

@@ -64,6 +64,10 @@ def load() -> ctypes.CDLL:
     lib.hodu_host_linear.argtypes = [vp, vp, vp, ci, vpp]
     lib.hodu_host_stats_fused_steps.restype = ctypes.c_long
     lib.hodu_host_stats_sum_kernels.restype = ctypes.c_long
+    lib.hodu_host_stats_softmax_kernels.restype = ctypes.c_long
+    lib.hodu_host_softmax.argtypes = [vp, ci, ci, vpp]
+    lib.hodu_host_attention.argtypes = [vp, vp, vp, ci, vpp]
+    lib.hodu_host_scalar_bits.argtypes = [ci, ctypes.c_double, ctypes.POINTER(ctypes.c_ubyte), szp]
     lib.hodu_host_sum.argtypes = [vp, ctypes.POINTER(ci), sz, ci, vpp]
     lib.hodu_host_sum_to_shape.argtypes = [vp, szp, sz, vpp]
     lib.hodu_host_matmul_vjp.argtypes = [vp, vp, vp, vpp, vpp]
@@ -104,7 +108,8 @@ def stats(reset: bool = False) -> dict:
     if reset:
         lib.hodu_host_stats_reset()
     return {"cast_kernels": a.value, "contiguous_kernels": b.value, "product_kernels": c.value,
-            "fused_products": d.value, "bytes_copied": e.value, "fused_steps": fused_steps, "sum_kernels": sum_kernels}
+            "fused_products": d.value, "bytes_copied": e.value, "fused_steps": fused_steps, "sum_kernels": sum_kernels,
+            "softmax_kernels": int(lib.hodu_host_stats_softmax_kernels())}
 
 
 class Tensor:
@@ -192,6 +197,11 @@ class Tensor:
         out = ctypes.c_void_p()
         return self._wrap(load().hodu_host_matmul_then(self._h, other._h, arr, len(steps), ctypes.byref(out)), out)
 
+    def softmax(self, dim: int = -1, causal: bool = False) -> "Tensor":
+        """Tensor::softmax (tensor/ops/normalization.rs:4-21) as one launch; last dim only.  causal: entries j > i of
+        every [.., Sq, Sk] matrix are masked first (attention.rs:40-48)"""
+        return self._unary(load().hodu_host_softmax, int(dim), int(causal))
+
     def sum(self, dims: Sequence[int] = (), keep_dim: bool = False) -> "Tensor":
         """Tensor::sum (tensor/ops/reduce.rs:11-13): no dims = all of them"""
         arr = (ctypes.c_int * max(1, len(dims)))(*dims)
@@ -252,6 +262,23 @@ def matmul_vjp(a: Tensor, b: Tensor, grad: Tensor):
 def dot_vjp(a: Tensor, b: Tensor, grad: Tensor):
     """(dA, dB) of dot(a, b) (tensor/gradient/vjp_matrix.rs:46-67)"""
     return _vjp(load().hodu_host_dot_vjp, a, b, grad)
+
+
+def scalar_bits(dtype: str, value: float) -> np.ndarray:
+    """`value` as a 1-element array in dtype's storage, rounded to nearest even (Scalar::to_dtype)"""
+    buf, n = (ctypes.c_ubyte * 8)(), ctypes.c_size_t()
+    rc = load().hodu_host_scalar_bits(DTYPE_ID[dtype], float(value), buf, ctypes.byref(n))
+    if rc != 0:
+        raise HoduError(rc, load().hodu_host_last_error().decode())
+    return np.frombuffer(bytes(buf[:n.value]), dtype=_BITS[n.value]).copy()
+
+
+def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False) -> Tensor:
+    """hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) without attn_mask and
+    dropout: three launches (product with the scale in its store, masked softmax, product)"""
+    out = ctypes.c_void_p()
+    rc = load().hodu_host_attention(q._h, k._h, v._h, int(is_causal), ctypes.byref(out))
+    return Tensor._wrap(rc, out)
 
 
 class Linear:

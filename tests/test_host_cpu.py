@@ -24,7 +24,8 @@ def test_host_library_loads_and_exports_the_tensor_interface():
     lib = tensor.load()
     for name in ("tensor_from_bytes", "tensor_free", "tensor_to_bytes", "tensor_layout", "matmul", "dot", "to_dtype",
                  "contiguous", "transpose", "broadcast", "reshape", "squeeze", "unsqueeze", "slice", "view",
-                 "set_matmul_mode", "stats", "last_error"):
+                 "set_matmul_mode", "stats", "last_error", "matmul_then", "linear", "sum", "sum_to_shape", "matmul_vjp",
+                 "dot_vjp", "softmax", "attention", "scalar_bits"):
         assert hasattr(lib, f"hodu_host_{name}"), name
 
 
@@ -40,3 +41,24 @@ def test_from_bits_checks_the_element_width():
     import numpy as np
     with pytest.raises(ValueError):
         tensor.Tensor.from_bits(np.zeros(4, np.uint8), "f32", [2, 2])
+
+
+def test_scalar_bits_round_to_nearest_even():
+    """the scalar a mul_scalar step carries: f64 -> tensor dtype as Scalar::to_dtype does (crates/hodu_core/src/
+    scalar.rs:391-404); f16 / bf16 against numpy's and the test helpers' independent RNE conversions, ties, subnormals
+    and overflow included"""
+    import numpy as np
+    import helpers as H
+    from hodu_amd import tensor as T
+    g = np.random.default_rng(3)
+    vals = np.concatenate([g.standard_normal(300) * np.exp2(g.uniform(-30, 17, 300)),
+                           [0.0, -0.0, 1.0, 65504.0, 65519.9, 65520.0, 1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001,
+                            2.0 ** -14, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 1.0 / np.sqrt(128.0), np.inf, -np.inf]])
+    for v in vals:
+        f = np.float32(v)
+        with np.errstate(over="ignore"):
+            want16 = np.array([f], np.float32).astype(np.float16).view(np.uint16)[0]
+        assert T.scalar_bits("f16", float(v))[0] == want16, (v, hex(want16))
+        assert T.scalar_bits("bf16", float(v))[0] == H.f32_to_bf16_rne(np.array([f]))[0], v
+        assert T.scalar_bits("f32", float(v)).view(np.float32)[0] == f or np.isnan(f)
+        assert T.scalar_bits("f64", float(v)).view(np.float64)[0] == v
