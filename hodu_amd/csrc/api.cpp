@@ -36,6 +36,7 @@ size_t out_elem_size(int kind, int dtype) {
 // the kernel, any further outer dims are walked here.
 int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p,
                 const DevEpilogue &epi) {
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     if (p.M > 0x7FFFFFFFL || p.N > 0x7FFFFFFFL || p.K > 0x7FFFFFFFL)
         return fail(HODU_ROCM_UNSUPPORTED, "matrix extent exceeds 2^31-1");
@@ -230,6 +231,7 @@ static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int 
     DevEpilogue epi;
     rc = build_epilogue("time_product", kind, dtype, out, steps, n_steps, &epi);
     if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     hipEvent_t t0, t1;
     HODU_HIP(hipEventCreate(&t0));
@@ -300,6 +302,7 @@ int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *o
     Strided s;
     int rc = parse_cast_metadata(md, len, &s);
     if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     return launch_cast(ctx, src, dst, in, out, s);
 }
@@ -313,6 +316,7 @@ int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, cons
     Reduction r;
     int rc = parse_reduce_metadata(md, len, &r);
     if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     return launch_sum(ctx, dtype, in, out, r);
 }
@@ -330,6 +334,7 @@ int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, 
     const size_t dim = md[4 + 2 * nd + out_nd];
     const bool last = dim + 1 == nd;
     if (causal && (!last || nd < 2)) return fail(HODU_ROCM_INVALID_ARG, "softmax: the causal mask needs the last dim of a matrix");
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     return launch_softmax(ctx, dtype, in, out, r, last, causal ? 1 : 0, nd >= 2 ? (long)md[1 + nd - 2] : 1);
 }
@@ -343,6 +348,7 @@ int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *ou
     Strided s;
     int rc = parse_cast_metadata(md, len, &s);
     if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     return launch_gather(ctx, dtype, in, out, s);
 }

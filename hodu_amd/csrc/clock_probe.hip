@@ -64,6 +64,7 @@ extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const vo
     clear_error();
     if (!ctx || !operands || iters <= 0 || !elapsed_ms || !tflops || !shader_mhz || kind < 0 || kind > 1)
         return fail(HODU_ROCM_INVALID_ARG, "mfma_clock: bad argument");
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     const unsigned blocks = 2u * (unsigned)ctx->props.multiProcessorCount;
     float *sink = nullptr;

@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
@@ -32,6 +34,9 @@ struct hodu_rocm_ctx {
     int force_tile = -1;    // testing hook: pins the MFMA tile size
     int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
     char kernel_name[96] = {0};  // storage for a composed last_kernel name
+    // every entry point that launches kernels holds this for the call: the workspace, the arrival counters, the
+    // testing hooks and last_kernel belong to the context, and launches of one context go to one stream anyway
+    std::recursive_mutex mu;
 };
 
 namespace hodu {

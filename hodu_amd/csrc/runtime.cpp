@@ -178,6 +178,7 @@ int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
     const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 14) || tile == 30 || tile == 31 ||
                     tile == 32 || tile == 34 || (tile >= 35 && tile <= 38);
     if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..14, 30, 31, 32, 34..38", tile);
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     ctx->force_tile = tile;
     return HODU_ROCM_OK;
 }
@@ -185,6 +186,7 @@ int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
 int hodu_rocm_debug_force_splitk(hodu_rocm_ctx *ctx, int splits) {
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
     if (splits < -1 || splits == 0 || splits > 64) return fail(HODU_ROCM_INVALID_ARG, "splits %d not in -1, 1..64", splits);
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     ctx->force_splits = splits;
     return HODU_ROCM_OK;
 }
