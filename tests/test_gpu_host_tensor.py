@@ -444,3 +444,25 @@ def test_softmax_of_a_view_and_its_limits():
     with pytest.raises(T.HoduError) as err:
         t.softmax(0)
     assert err.value.kind == "InvalidArgument"
+
+
+# ---- .hdt files straight onto the device (crates/hodu_core/src/format/hdt.rs:25-52) ------------------------
+def test_hdt_round_trip_through_the_device(tmp_path):
+    from hodu_amd import hdt
+    g = H.rng(61)
+    w8 = H.f32_to_ocp_e4m3_rne(g.standard_normal(12 * 64) * 4)
+    x = H.f32_to_bf16_rne(g.standard_normal(5 * 64).astype(np.float32))
+    tw, tx = T.Tensor.from_bits(w8, "f8e4m3", [12, 64]), T.Tensor.from_bits(x, "bf16", [5, 64])
+    hdt.save_many({"linear.weight": tw, "x": tx}, tmp_path / "m.hdt")
+    back = hdt.load_many(tmp_path / "m.hdt")
+    assert set(back) == {"linear.weight", "x"}
+    assert back["linear.weight"].dtype == "f8e4m3" and back["linear.weight"].shape == [12, 64]
+    assert np.array_equal(back["linear.weight"].to_bits(), w8) and np.array_equal(back["x"].to_bits(), x)
+    # the loaded weight goes down the path like any other: deferred cast, one launch
+    y0 = tx.matmul(tw.to_dtype("bf16").t()).to_bits()
+    y1 = back["x"].matmul(back["linear.weight"].to_dtype("bf16").t()).to_bits()
+    assert np.array_equal(y0, y1)
+    # a view is saved as its contiguous elements (Tensor::to_bytes)
+    hdt.save(tx.t(), tmp_path / "t.hdt")
+    t2 = hdt.load(tmp_path / "t.hdt")
+    assert t2.shape == [64, 5] and np.array_equal(t2.to_bits(), x.reshape(5, 64).T.ravel())
