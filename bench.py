@@ -263,6 +263,25 @@ def attention_probe(ctx, steps):
             "tflops_total": flops / total / 1e6, "legs": res}
 
 
+def read_floor_probe(ctx):
+    """what a kernel that does nothing but read can reach at the sizes of the M = 1 configurations (weight buffers
+    rotated past the Infinity Cache like the GEMV's), and the launch cadence of an empty kernel"""
+    out = []
+    for label, nbytes in (("16.8 MB (config 3 weight)", 4096 * 4096), ("58.7 MB (config 5 weight)", 14336 * 4096)):
+        copies = max(2, int(3 * INFINITY_CACHE_BYTES // nbytes) + 1)
+        bufs = [ctx.alloc(nbytes) for _ in range(copies)]
+        for b in bufs:
+            ctx.fill(b, 0x5A)
+        ctx.sync()
+        r = ctx.read_floor(bufs, nbytes, 200)
+        for b in bufs:
+            b.free()
+        out.append({"bytes": nbytes, "label": label, "buffers_rotated": copies, "read_us": r["read_us"],
+                    "read_gbs": nbytes / r["read_us"] / 1e3, "frac_of_hbm_peak": nbytes / r["read_us"] / 1e3 / HBM_PEAK_GBS,
+                    "empty_kernel_us": r["empty_us"]})
+    return out
+
+
 def mfma_clock_probe(ctx):
     """what the matrix cores sustain from registers (no LDS, no memory traffic), and at which shader clock, on
     constant and on N(0,1) operands: the clock under full MFMA load depends on the data"""
@@ -374,7 +393,7 @@ def main():
         ctx.close()
         return
     if args.only == "clock":
-        print(json.dumps({"config": "clock", "register_only_mfma": mfma_clock_probe(ctx)}))
+        print(json.dumps({"config": "clock", "register_only_mfma": mfma_clock_probe(ctx), "streaming_read": read_floor_probe(ctx)}))
         ctx.close()
         return
     if args.only:
@@ -416,6 +435,8 @@ def main():
         # not part of the roofline (whose peak is the datasheet's): the rate a register-only MFMA loop sustains on
         # this box, by operand data
         "register_only_mfma": mfma_clock_probe(ctx),
+        # likewise for the HBM-bound rows: a kernel that only reads, at the M = 1 configurations' sizes
+        "streaming_read": read_floor_probe(ctx),
         "device": info,
         "all_configs": results,
     }

@@ -54,10 +54,72 @@ __global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restri
     }
 }
 
+// the simplest possible reader: every lane loads PER 16-byte vectors, all in flight at once, and folds them into a
+// value that is (almost) never stored
+template <int PER>
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t *__restrict__ src, unsigned *__restrict__ sink, long n_vec) {
+    const long base = (long)blockIdx.x * PER * 256 + threadIdx.x;
+    u32x4_t v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const long j = base + (long)i * 256;
+        v[i] = j < n_vec ? src[j] : u32x4_t{0u, 0u, 0u, 0u};
+    }
+    unsigned x = 0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) x += v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (x == 0x9E3779B9u) sink[threadIdx.x] = x;
+}
+
+__global__ void empty_kernel() {}
+
 }  // namespace
 }  // namespace hodu
 
 using namespace hodu;
+
+// iters launches of a flat streaming read of `bytes` from each of `n_src` buffers in turn (more buffers than the
+// Infinity Cache holds: the reads come from HBM), and iters launches of an empty kernel: what the memory system and
+// the launch path allow a kernel of this size, before any arithmetic
+extern "C" int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const *src_list, size_t n_src, size_t bytes, int iters,
+                                          float *read_us, float *empty_us) {
+    clear_error();
+    if (!ctx || !src_list || n_src == 0 || bytes == 0 || bytes % 16 != 0 || iters <= 0 || !read_us || !empty_us)
+        return fail(HODU_ROCM_INVALID_ARG, "read_floor: bad argument");
+    for (size_t i = 0; i < n_src; i++)
+        if (!src_list[i] || (uintptr_t)src_list[i] % 16 != 0) return fail(HODU_ROCM_INVALID_ARG, "read_floor: bad buffer %zu", i);
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    HODU_HIP(hipSetDevice(ctx->device));
+    constexpr int PER = 8;
+    const long n_vec = (long)(bytes / 16);
+    const long blocks = (n_vec + PER * 256 - 1) / (PER * 256);
+    if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "read_floor: buffer too large");
+    unsigned *sink = nullptr;
+    HODU_HIP(hipMalloc((void **)&sink, 256 * sizeof(unsigned)));
+    hipEvent_t t0, t1;
+    hipError_t e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    auto timed = [&](auto launch, float *us) {
+        for (int i = 0; i < 3; i++) launch(i);
+        if (e == hipSuccess) e = hipEventRecord(t0, ctx->stream);
+        for (int i = 0; i < iters; i++) launch(i);
+        if (e == hipSuccess) e = hipEventRecord(t1, ctx->stream);
+        if (e == hipSuccess) e = hipEventSynchronize(t1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+        *us = ms * 1e3f / (float)iters;
+    };
+    timed([&](int i) {
+        hipLaunchKernelGGL(stream_read_kernel<PER>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                           (const u32x4_t *)src_list[(size_t)i % n_src], sink, n_vec);
+    }, read_us);
+    timed([&](int) { hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, ctx->stream); }, empty_us);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipFree(sink);
+    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "read_floor: %s", hipGetErrorString(e));
+    return HODU_ROCM_OK;
+}
 
 extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
                                           double *tflops, double *shader_mhz) {

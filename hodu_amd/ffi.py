@@ -116,6 +116,8 @@ def load() -> ctypes.CDLL:
                                                     ctypes.POINTER(EpilogueStep), sz, ci, ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, ctypes.POINTER(ctypes.c_float),
                                                ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    lib.hodu_rocm_debug_read_floor.argtypes = [vp, ctypes.POINTER(vp), sz, sz, ci, ctypes.POINTER(ctypes.c_float),
+                                               ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
@@ -339,6 +341,16 @@ class Context:
         self._check(self.lib.hodu_rocm_debug_mfma_clock(self.handle, int(kind), operands.ptr, int(iters), ctypes.byref(ms),
                                                         ctypes.byref(tf), ctypes.byref(mhz)))
         return {"ms": ms.value, "tflops": tf.value, "shader_mhz": mhz.value}
+
+    def read_floor(self, buffers, nbytes: int, iters: int = 200) -> dict:
+        """flat streaming read of nbytes from each buffer in turn, and an empty kernel: microseconds per launch"""
+        if any(b.nbytes < nbytes for b in buffers):
+            raise HoduRocmError(INVALID_ARG, "read_floor: a buffer is smaller than nbytes")
+        ptrs = (ctypes.c_void_p * len(buffers))(*[b.ptr for b in buffers])
+        r, e = ctypes.c_float(), ctypes.c_float()
+        self._check(self.lib.hodu_rocm_debug_read_floor(self.handle, ptrs, len(buffers), int(nbytes), int(iters),
+                                                        ctypes.byref(r), ctypes.byref(e)))
+        return {"read_us": r.value, "empty_us": e.value}
 
     def force_tile(self, tile: int):
         """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, 10..14 the pipelined

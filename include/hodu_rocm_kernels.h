@@ -114,6 +114,13 @@ int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int ki
 int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
                                double *tflops, double *shader_mhz);
 
+/* measurement hook: `iters` launches of a flat streaming read (16 bytes per lane, eight loads in flight, nothing
+ * else) of `bytes` from each of the `n_src` device buffers in turn, and `iters` launches of an empty kernel, each
+ * bracketed by HIP events on the context's stream.  *read_us: time per read launch; *empty_us: time per empty launch
+ * (the launch cadence).  What the memory system and the launch path allow a kernel that moves `bytes`. */
+int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const *src_list, size_t n_src, size_t bytes, int iters,
+                               float *read_us, float *empty_us);
+
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>
  * (kernels/ops_matrix.c:423, :581).  Narrow floats accumulate in f32 and round once on store.   */
