@@ -339,6 +339,38 @@ int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, 
     return launch_softmax(ctx, dtype, in, out, r, last, causal ? 1 : 0, nd >= 2 ? (long)md[1 + nd - 2] : 1);
 }
 
+int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                        const size_t *md, size_t len, const void *scale, int causal) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "attention: context is null");
+    if (!q || !k || !v || !out || !scale) return fail(HODU_ROCM_INVALID_ARG, "attention: null pointer");
+    if (out == q || out == k || out == v) return fail(HODU_ROCM_INVALID_ARG, "attention: out aliases an input");
+    AttentionArgs a;
+    int rc = parse_attention_metadata(md, len, &a);
+    if (rc) return rc;
+    if (dtype == HODU_BF16) {
+        uint16_t h;
+        memcpy(&h, scale, 2);
+        uint32_t u = (uint32_t)h << 16;
+        memcpy(&a.scale, &u, 4);
+    } else if (dtype == HODU_F16) {
+        _Float16 h;
+        memcpy(&h, scale, 2);
+        a.scale = (float)h;
+    } else {
+        return fail(HODU_ROCM_UNSUPPORTED, "attention: the fused kernel takes bf16 and f16 (dtype id %d)", dtype);
+    }
+    a.causal = causal != 0;
+    if (a.batches == 0 || a.sq == 0) return HODU_ROCM_OK;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    HODU_HIP(hipSetDevice(ctx->device));
+    rc = launch_attention(ctx, dtype, q, k, v, out, a);
+    if (rc == HODU_ROCM_UNSUPPORTED)
+        return fail(HODU_ROCM_UNSUPPORTED, "attention: the fused kernel needs head dim 128, at most %d batch dims and 16-byte aligned rows",
+                    kKernelBatchDims);
+    return rc;
+}
+
 int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "contiguous: context is null");

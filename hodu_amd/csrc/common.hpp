@@ -174,6 +174,24 @@ int launch_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const R
 int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, bool dim_is_last,
                    int causal, long sq);
 
+// One fused attention call: q [batch.., sq, d], k and v [batch.., sk, d] (batch dims already broadcast, last dim
+// dense), out contiguous [batch.., sq, d]
+struct AttentionArgs {
+    long sq = 0, sk = 0, d = 0;
+    long q_row = 0, k_row = 0, v_row = 0;  // element strides between rows
+    int nb = 0;
+    long bshape[16];
+    long q_bs[16], k_bs[16], v_bs[16];
+    long q_off = 0, k_off = 0, v_off = 0;
+    long batches = 1;
+    float scale = 1.f;
+    bool causal = false;
+};
+int parse_attention_metadata(const size_t *md, size_t len, AttentionArgs *a);
+// HODU_ROCM_UNSUPPORTED without an error text when the fused kernel does not take the call
+int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                     const AttentionArgs &a);
+
 int launch_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const Strided &s);
 int launch_gather(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Strided &s);
 

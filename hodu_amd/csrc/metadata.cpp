@@ -202,4 +202,36 @@ int parse_reduce_metadata(const size_t *md, size_t len, Reduction *r) {
     return HODU_ROCM_OK;
 }
 
+// attention metadata (this library's own: the reference has no single kernel for the function):
+// [nb, batch_shape (nb).., Sq, Sk, D, q_strides (nb + 2).., k_strides (nb + 2).., v_strides (nb + 2).., q_off, k_off, v_off]
+// strides and offsets in elements; the batch dims of q, k and v are already broadcast to batch_shape (stride 0 where
+// an operand does not have the dim)
+int parse_attention_metadata(const size_t *md, size_t len, AttentionArgs *a) {
+    if (!md) return fail(HODU_ROCM_INVALID_ARG, "attention: metadata is null");
+    if (len < 1) return fail(HODU_ROCM_INVALID_ARG, "attention: metadata is empty");
+    for (size_t i = 0; i < len; i++)
+        if (!sane(md[i])) return fail(HODU_ROCM_INVALID_ARG, "attention: metadata[%zu] out of range", i);
+    const size_t nb = md[0];
+    if (nb > 14) return fail(HODU_ROCM_UNSUPPORTED, "attention: %zu batch dims (> 14)", nb);
+    const size_t want = 1 + nb + 3 + 3 * (nb + 2) + 3;
+    if (len != want) return fail(HODU_ROCM_INVALID_ARG, "attention: metadata has %zu words, layout implies %zu", len, want);
+    *a = AttentionArgs{};
+    a->nb = (int)nb;
+    a->batches = 1;
+    for (size_t d = 0; d < nb; d++) {
+        a->bshape[d] = (long)md[1 + d];
+        a->batches *= a->bshape[d];
+    }
+    a->sq = (long)md[1 + nb]; a->sk = (long)md[2 + nb]; a->d = (long)md[3 + nb];
+    const size_t *qs = md + 4 + nb, *ks = qs + nb + 2, *vs = ks + nb + 2;
+    if (a->d > 1 && (qs[nb + 1] != 1 || ks[nb + 1] != 1 || vs[nb + 1] != 1))
+        return fail(HODU_ROCM_UNSUPPORTED, "attention: the head dim must be dense in q, k and v");
+    for (size_t d = 0; d < nb; d++) {
+        a->q_bs[d] = (long)qs[d]; a->k_bs[d] = (long)ks[d]; a->v_bs[d] = (long)vs[d];
+    }
+    a->q_row = (long)qs[nb]; a->k_row = (long)ks[nb]; a->v_row = (long)vs[nb];
+    a->q_off = (long)md[want - 3]; a->k_off = (long)md[want - 2]; a->v_off = (long)md[want - 1];
+    return HODU_ROCM_OK;
+}
+
 }  // namespace hodu

@@ -122,6 +122,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
+    lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
     _lib = lib
     return lib
 
@@ -311,6 +312,27 @@ class Context:
                 raise HoduRocmError(INVALID_ARG, f"softmax_{dt}: metadata reaches past a device buffer")
         arr, n_md = _md_array(md)
         self._check(self.lib.hodu_rocm_softmax(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n_md, int(bool(causal))))
+
+    def attention(self, dt: str, q: DeviceBuffer, k: DeviceBuffer, v: DeviceBuffer, out: DeviceBuffer, md, scale, causal=False):
+        """hodu_rocm_attention; md = [nb, batch_shape.., Sq, Sk, D, q_strides.., k_strides.., v_strides.., q_off, k_off,
+        v_off]; scale: 1-element array in dt's storage"""
+        m = [int(x) for x in md]
+        nb = m[0] if m else 0
+        if len(m) == 1 + nb + 3 + 3 * (nb + 2) + 3:
+            bshape, (sq, sk, d) = m[1:1 + nb], m[1 + nb:4 + nb]
+            base = 4 + nb
+            for name, buf, rows, st, off in (("q", q, sq, m[base:base + nb + 2], m[-3]),
+                                             ("k", k, sk, m[base + nb + 2:base + 2 * (nb + 2)], m[-2]),
+                                             ("v", v, sk, m[base + 2 * (nb + 2):base + 3 * (nb + 2)], m[-1])):
+                if _view_span(bshape + [rows, d], st, off) * DTYPE_SIZE[dt] > buf.nbytes:
+                    raise HoduRocmError(INVALID_ARG, f"attention: metadata reaches past the {name} buffer")
+            n_out = int(np.prod(bshape + [sq, d], dtype=np.int64))
+            if n_out * DTYPE_SIZE[dt] > out.nbytes:
+                raise HoduRocmError(INVALID_ARG, "attention: the output buffer is too small")
+        arr, n = _md_array(md)
+        sc = np.ascontiguousarray(scale).reshape(1)
+        self._check(self.lib.hodu_rocm_attention(self.handle, DTYPE_ID[dt], q.ptr, k.ptr, v.ptr, out.ptr, arr, n,
+                                                 sc.ctypes.data, int(bool(causal))))
 
     def time_product(self, op: str, name: str, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int,
                      graph: bool = False, steps=None) -> float:

@@ -94,6 +94,7 @@ int hodu_host_linear(const hodu_host_tensor *input, const hodu_host_tensor *weig
 long hodu_host_stats_fused_steps(void) { return stats().fused_steps; }
 long hodu_host_stats_sum_kernels(void) { return stats().sum_kernels; }
 long hodu_host_stats_softmax_kernels(void) { return stats().softmax_kernels; }
+long hodu_host_stats_attention_kernels(void) { return stats().attention_kernels; }
 int hodu_host_softmax(const hodu_host_tensor *t, int dim, int causal, hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(T(t)->softmax(dim, causal != 0))); });
 }

@@ -37,9 +37,9 @@ inline const char *dtype_name(DType d) {
 struct Stats {
     std::atomic<long> cast_kernels{0}, contiguous_kernels{0}, product_kernels{0}, fused_products{0};
     std::atomic<long> fused_steps{0};        // element-wise kernels that ran inside a product's store instead
-    std::atomic<long> sum_kernels{0}, softmax_kernels{0};
+    std::atomic<long> sum_kernels{0}, softmax_kernels{0}, attention_kernels{0};
     std::atomic<long long> bytes_copied{0};  // written by cast/contiguous passes
-    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = sum_kernels = softmax_kernels = 0; bytes_copied = 0; }
+    void reset() { cast_kernels = contiguous_kernels = product_kernels = fused_products = fused_steps = sum_kernels = softmax_kernels = attention_kernels = 0; bytes_copied = 0; }
 };
 inline Stats &stats() {
     static Stats s;
@@ -204,6 +204,28 @@ public:
         dev_->check(hodu_rocm_softmax(dev_->ctx(), (int)dtype_, ptr(), (void *)out.ptr(), md.data(), md.size(), causal ? 1 : 0),
                     "softmax");
         stats().softmax_kernels++;
+        return out;
+    }
+
+    // the whole of scaled_dot_product_attention as one launch, where the fused kernel takes the call (bf16 / f16,
+    // head dim 128, dense aligned rows): *taken says whether it did.  md: hodu_rocm_attention's metadata.
+    RocmStorage call_ops_attention(const RocmStorage &k, const RocmStorage &v, const Layout &ql, const Layout &kl, const Layout &vl,
+                                   const Metadata &md, size_t out_elems, const unsigned char scale[8], bool causal,
+                                   bool *taken) const {
+        check_span(ql, "attention q");
+        k.check_span(kl, "attention k");
+        v.check_span(vl, "attention v");
+        *taken = false;
+        RocmStorage out = fresh(dtype_, out_elems);
+        if (deferred() || k.deferred() || v.deferred() || k.dtype_ != dtype_ || v.dtype_ != dtype_ ||
+            k.dev_->id() != dev_->id() || v.dev_->id() != dev_->id() || out_elems == 0)
+            return out;
+        const int rc = hodu_rocm_attention(dev_->ctx(), (int)dtype_, ptr(), k.ptr(), v.ptr(), (void *)out.ptr(), md.data(),
+                                           md.size(), scale, causal ? 1 : 0);
+        if (rc == HODU_ROCM_UNSUPPORTED) return out;
+        dev_->check(rc, "attention");
+        stats().attention_kernels++;
+        *taken = true;
         return out;
     }
 

@@ -244,13 +244,57 @@ public:
     }
 
     // scaled_dot_product_attention (hodu_nn/src/modules/attention.rs:25-70) without attn_mask and dropout:
-    // softmax(Q K^T / sqrt(d_k) [+ causal mask]) V as three launches -- the scale rides in the first product's
-    // store, the mask and the five softmax kernels are one kernel, the second product is plain.
+    // softmax(Q K^T / sqrt(d_k) [+ causal mask]) V.  One launch where the fused kernel applies (bf16 / f16, head dim
+    // 128, dense aligned rows); otherwise three -- the scale rides in the first product's store, the mask and the
+    // five softmax kernels are one kernel, the second product is plain.
     static Tensor scaled_dot_product_attention(const Tensor &q, const Tensor &k, const Tensor &v, bool is_causal) {
         if (q.layout().ndim() < 2) throw Error(ErrorKind::InvalidArgument, "attention: query needs at least two dimensions");
         const double scale = 1.0 / std::sqrt((double)q.shape().back());
         unsigned char bits[8];
         const size_t n = scalar_bits(q.dtype(), scale, bits);
+        // one kernel where it applies: q [.., Sq, D], k and v [.., Sk, D] with the batch dims broadcast the way the
+        // two matmuls would broadcast them
+        const size_t qn = q.layout().ndim(), kn = k.layout().ndim(), vn = v.layout().ndim();
+        if (kn >= 2 && vn >= 2 && q.shape()[qn - 1] == k.shape()[kn - 1] && k.shape()[kn - 2] == v.shape()[vn - 2] &&
+            v.shape()[vn - 1] == q.shape()[qn - 1]) {
+            const size_t bn = std::max({qn, kn, vn}) - 2;
+            Dims batch(bn, 1);
+            bool ok = true;
+            for (const Tensor *t : {&q, &k, &v}) {
+                const size_t tb = t->layout().ndim() - 2;
+                for (size_t i = 0; i < tb; i++) {
+                    const size_t ext = t->shape()[tb - 1 - i];
+                    size_t &slot = batch[bn - 1 - i];
+                    if (slot == 1) slot = ext;
+                    else if (ext != 1 && ext != slot) ok = false;
+                }
+            }
+            if (ok) {
+                auto spread = [&](const Tensor &t, size_t rows) {
+                    Dims s = batch;
+                    s.push_back(rows);
+                    s.push_back(q.shape()[qn - 1]);
+                    return t.layout().broadcast_to(s);
+                };
+                const Layout ql = spread(q, q.shape()[qn - 2]), kl = spread(k, k.shape()[kn - 2]), vl = spread(v, v.shape()[vn - 2]);
+                Metadata md{bn};
+                md.insert(md.end(), batch.begin(), batch.end());
+                md.push_back(q.shape()[qn - 2]);
+                md.push_back(k.shape()[kn - 2]);
+                md.push_back(q.shape()[qn - 1]);
+                for (const Layout *l : {&ql, &kl, &vl}) md.insert(md.end(), l->strides().begin(), l->strides().end());
+                md.push_back(ql.offset());
+                md.push_back(kl.offset());
+                md.push_back(vl.offset());
+                Dims out_shape = batch;
+                out_shape.push_back(q.shape()[qn - 2]);
+                out_shape.push_back(q.shape()[qn - 1]);
+                bool taken = false;
+                auto out = std::make_shared<RocmStorage>(q.storage_->call_ops_attention(*k.storage_, *v.storage_, ql, kl, vl, md,
+                                                                                        product(out_shape), bits, is_causal, &taken));
+                if (taken) return Tensor(out, Layout::from_shape(out_shape));
+            }
+        }
         const Tensor scores = q.matmul_then(k.transpose(-2, -1), {Then::mul_scalar(bits, n)});
         return scores.softmax(-1, is_causal).matmul(v);
     }

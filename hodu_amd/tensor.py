@@ -65,6 +65,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_host_stats_fused_steps.restype = ctypes.c_long
     lib.hodu_host_stats_sum_kernels.restype = ctypes.c_long
     lib.hodu_host_stats_softmax_kernels.restype = ctypes.c_long
+    lib.hodu_host_stats_attention_kernels.restype = ctypes.c_long
     lib.hodu_host_softmax.argtypes = [vp, ci, ci, vpp]
     lib.hodu_host_attention.argtypes = [vp, vp, vp, ci, vpp]
     lib.hodu_host_scalar_bits.argtypes = [ci, ctypes.c_double, ctypes.POINTER(ctypes.c_ubyte), szp]
@@ -109,7 +110,8 @@ def stats(reset: bool = False) -> dict:
         lib.hodu_host_stats_reset()
     return {"cast_kernels": a.value, "contiguous_kernels": b.value, "product_kernels": c.value,
             "fused_products": d.value, "bytes_copied": e.value, "fused_steps": fused_steps, "sum_kernels": sum_kernels,
-            "softmax_kernels": int(lib.hodu_host_stats_softmax_kernels())}
+            "softmax_kernels": int(lib.hodu_host_stats_softmax_kernels()),
+            "attention_kernels": int(lib.hodu_host_stats_attention_kernels())}
 
 
 class Tensor:
@@ -275,7 +277,8 @@ def scalar_bits(dtype: str, value: float) -> np.ndarray:
 
 def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False) -> Tensor:
     """hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) without attn_mask and
-    dropout: three launches (product with the scale in its store, masked softmax, product)"""
+    dropout: one launch where the fused kernel applies (bf16 / f16, head dim 128), otherwise three (product with the
+    scale in its store, masked softmax, product)"""
     out = ctypes.c_void_p()
     rc = load().hodu_host_attention(q._h, k._h, v._h, int(is_causal), ctypes.byref(out))
     return Tensor._wrap(rc, out)

@@ -254,6 +254,21 @@ int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, cons
 int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *metadata,
                       size_t metadata_len, int causal);
 
+/* ---- attention as one kernel --------------------------------------------------------------------------- *
+ * out = softmax(q k^T * scale [causal]) v for q [batch.., Sq, D], k and v [batch.., Sk, D]: what
+ * scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) computes with a batched matmul,
+ * mul_scalar, masked_fill, the five softmax kernels and a second batched matmul, without attn_mask and dropout.  The
+ * scores never leave the chip: scores and probabilities stay in f32 (the reference rounds them to the storage type
+ * after every kernel), the output is rounded once.  Takes bf16 / f16, D = 128, dense head dims, rows / offsets /
+ * batch strides that are multiples of 8 elements; returns HODU_ROCM_UNSUPPORTED otherwise, and the caller runs the
+ * three launches (hodu_rocm_matmul_<dt>_ex with MUL_SCALAR, hodu_rocm_softmax, hodu_rocm_matmul_<dt>).
+ * metadata (this library's own): [nb, batch_shape (nb).., Sq, Sk, D, q_strides (nb + 2).., k_strides (nb + 2)..,
+ * v_strides (nb + 2).., q_off, k_off, v_off], strides and offsets in elements, batch dims already broadcast (stride
+ * 0 where an operand lacks the dim).  scale: the scalar in `dtype` (what mul_scalar receives); causal != 0 masks
+ * key j > query i.  out: contiguous [batch.., Sq, D]. */
+int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                        const size_t *metadata, size_t metadata_len, const void *scale, int causal);
+
 #ifdef __cplusplus
 }
 #endif

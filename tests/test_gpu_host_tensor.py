@@ -466,3 +466,41 @@ def test_hdt_round_trip_through_the_device(tmp_path):
     hdt.save(tx.t(), tmp_path / "t.hdt")
     t2 = hdt.load(tmp_path / "t.hdt")
     assert t2.shape == [64, 5] and np.array_equal(t2.to_bits(), x.reshape(5, 64).T.ravel())
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_takes_the_fused_kernel_at_head_dim_128(causal):
+    """bf16, D = 128: one launch; k and v shared across the heads through broadcasting, as the two matmuls would"""
+    g = H.rng(54)
+    q = H.f32_to_bf16_rne(g.standard_normal(2 * 3 * 72 * 128).astype(np.float32))
+    k = H.f32_to_bf16_rne(g.standard_normal(2 * 1 * 90 * 128).astype(np.float32))
+    v = H.f32_to_bf16_rne(g.standard_normal(90 * 128).astype(np.float32))
+    tq, tk, tv = (T.Tensor.from_bits(q, "bf16", [2, 3, 72, 128]), T.Tensor.from_bits(k, "bf16", [2, 1, 90, 128]),
+                  T.Tensor.from_bits(v, "bf16", [90, 128]))
+    T.stats(reset=True)
+    out = T.scaled_dot_product_attention(tq, tk, tv, causal)
+    s = T.stats()
+    assert out.shape == [2, 3, 72, 128]
+    assert s["attention_kernels"] == 1 and s["product_kernels"] == 0 and s["softmax_kernels"] == 0 and s["contiguous_kernels"] == 0
+    qf = H.bf16_to_f32(q).astype(np.float64).reshape(2, 3, 72, 128)
+    kf = np.broadcast_to(H.bf16_to_f32(k).astype(np.float64).reshape(2, 1, 90, 128), (2, 3, 90, 128))
+    vf = np.broadcast_to(H.bf16_to_f32(v).astype(np.float64).reshape(90, 128), (2, 3, 90, 128))
+    scale = float(H.bf16_to_f32(T.scalar_bits("bf16", 1.0 / np.sqrt(128.0)))[0])
+    sc = qf @ np.swapaxes(kf, -1, -2) * scale
+    if causal:
+        i, j = np.arange(72)[:, None], np.arange(90)[None, :]
+        sc = np.where(j > i, -np.inf, sc)
+    e = np.exp(sc - sc.max(-1, keepdims=True))
+    p = e / e.sum(-1, keepdims=True)
+    want = p @ vf
+    got = H.bf16_to_f32(out.to_bits()).astype(np.float64).reshape(want.shape)
+    # floor of the denominator: the magnitude of an average of n unit-variance rows that may cancel
+    floor = np.abs(vf).mean() / np.sqrt((p > 0).sum(-1))[..., None]
+    assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), floor))
+    # a head dim the kernel does not take goes down the three-launch path, same function
+    T.stats(reset=True)
+    q64 = T.Tensor.from_bits(q[:2 * 3 * 72 * 64], "bf16", [2, 3, 72, 64])
+    k64 = T.Tensor.from_bits(k[:90 * 64], "bf16", [90, 64])
+    T.scaled_dot_product_attention(q64, k64, k64, causal)
+    s = T.stats()
+    assert s["attention_kernels"] == 0 and s["product_kernels"] == 2 and s["softmax_kernels"] == 1
