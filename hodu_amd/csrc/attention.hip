@@ -42,7 +42,8 @@ constexpr int AT_BK = 64;        // keys per step
 constexpr int AT_KSTEPS = AT_D / 16;
 constexpr int AT_K_BYTES = AT_BK * AT_D * 2;  // 16 KB: K block, two halves of [64 rows][128 bytes]
 constexpr int AT_V_BYTES = AT_BK * AT_D * 2;  // 16 KB: V block, [64 keys][256 bytes]
-constexpr int AT_LDS = AT_K_BYTES + AT_V_BYTES;
+constexpr int AT_BUF = AT_K_BYTES + AT_V_BYTES;  // one K block and one V block
+constexpr int AT_LDS = 2 * AT_BUF;              // two of them: the next block is written while this one is read
 
 struct DevAttention {
     int sq, sk;
@@ -52,23 +53,25 @@ struct DevAttention {
     long q_bs[kKernelBatchDims], k_bs[kKernelBatchDims], v_bs[kKernelBatchDims];
     long q_off, k_off, v_off;
     long batches;
-    float scale;
+    float scale_log2e;  // scale * log2(e): the softmax runs on base-2 exponentials
     int causal;
     int q_blocks;
 };
 
 template <int CK> struct Narrow;
 template <> struct Narrow<mfma::CK_BF16> {
-    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-        return (uint32_t)f32_to_bf16_bits_rne(lo) | ((uint32_t)f32_to_bf16_bits_rne(hi) << 16);
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {  // one v_cvt_pk_bf16_f32
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
     }
-    static __device__ __forceinline__ uint16_t one(float v) { return f32_to_bf16_bits_rne(v); }
 };
 template <> struct Narrow<mfma::CK_F16> {
     static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-        return (uint32_t)f32_to_f16_bits_rne(lo) | ((uint32_t)f32_to_f16_bits_rne(hi) << 16);
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
     }
-    static __device__ __forceinline__ uint16_t one(float v) { return f32_to_f16_bits_rne(v); }
 };
 
 // the value the other lane of the row (lane ^ 32) holds
@@ -86,11 +89,12 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
     typedef Compute32<CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     extern __shared__ __align__(16) char smem[];
-    char *k_lds = smem, *v_lds = smem + AT_K_BYTES;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, lh = lane >> 5;
-    const long batch = blockIdx.x / a.q_blocks;
-    const int q0 = (int)(blockIdx.x % a.q_blocks) * AT_BQ;
+    // the last query block of every head first: with the causal mask it walks the most keys, and the workgroups that
+    // finish the launch should be the short ones
+    const long batch = blockIdx.x % a.batches;
+    const int q0 = (a.q_blocks - 1 - (int)(blockIdx.x / a.batches)) * AT_BQ;
     long qo = a.q_off, ko = a.k_off, vo = a.v_off;
     {
         long b = batch;
@@ -139,17 +143,6 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
             vst[i] = *reinterpret_cast<const u32x4_t *>(V + vo + (long)key * a.v_row + (c & 15) * 8);
         }
     };
-    auto commit = [&]() {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + 256 * i, row = c >> 4, g = c & 15;
-            // K: half g / 8 of the row, chunk g % 8 at its swizzled slot
-            *reinterpret_cast<u32x4_t *>(k_lds + (g >> 3) * (AT_BK * 128) + row * 128 + (kd_slot(row, g & 7) << 4)) = kst[i];
-            // V: [key][256 bytes], chunk g at slot g ^ ((key & 3) << 2)
-            *reinterpret_cast<u32x4_t *>(v_lds + row * (AT_D * 2) + ((g ^ ((row & 3) << 2)) << 4)) = vst[i];
-        }
-    };
-
     // fragment addresses
     int k_frag[AT_KSTEPS];  // K block, tile 0; tile t adds t * 32 * 128
 #pragma unroll
@@ -166,23 +159,49 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
         }
     }
 
-    if (n_blocks > 0) fetch(0);
-    for (int kb = 0; kb < n_blocks; kb++) {
-        __syncthreads();  // every wavefront is done reading the previous block
-        commit();
-        __syncthreads();
-        if (kb + 1 < n_blocks) fetch(kb + 1);  // lands while this block is multiplied
+    auto commit_to = [&](char *buf) {
+        char *k_lds = buf, *v_lds = buf + AT_K_BYTES;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int c = tid + 256 * i, row = c >> 4, g = c & 15;
+            // K: half g / 8 of the row, chunk g % 8 at its swizzled slot
+            *reinterpret_cast<u32x4_t *>(k_lds + (g >> 3) * (AT_BK * 128) + row * 128 + (kd_slot(row, g & 7) << 4)) = kst[i];
+            // V: [key][256 bytes], chunk g at slot g ^ ((key & 3) << 2)
+            *reinterpret_cast<u32x4_t *>(v_lds + row * (AT_D * 2) + ((g ^ ((row & 3) << 2)) << 4)) = vst[i];
+        }
+    };
 
-        // ---- S = Q K^T: two 32-key tiles ----
+    if (n_blocks > 0) {
+        fetch(0);
+        commit_to(smem);
+        if (n_blocks > 1) fetch(1);
+    }
+    __syncthreads();
+    const int wave_row0 = q0 + wave * 32;  // the wavefront's first query row
+    for (int kb = 0; kb < n_blocks; kb++) {
+        const char *k_lds = smem + (kb & 1) * AT_BUF, *v_lds = k_lds + AT_K_BYTES;
+
+        // ---- S = Q K^T: two 32-key tiles, their accumulation chains interleaved ----
         acc_t s_acc[AT_BK / 32];
 #pragma unroll
-        for (int t = 0; t < AT_BK / 32; t++) {
+        for (int t = 0; t < AT_BK / 32; t++)
 #pragma unroll
             for (int e = 0; e < 16; e++) s_acc[t][e] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < AT_KSTEPS; ks++) Cmp::mma(lds_get(k_lds, k_frag[ks] + t * 32 * 128), qf[ks], s_acc[t]);
+        for (int ks = 0; ks < AT_KSTEPS; ks++)
+#pragma unroll
+            for (int t = 0; t < AT_BK / 32; t++) Cmp::mma(lds_get(k_lds, k_frag[ks] + t * 32 * 128), qf[ks], s_acc[t]);
+
+        // the next block's K and V have had the S phase to arrive: into the other buffer (nobody reads it: the
+        // barrier at the end of the previous iteration came after its last read), then fetch the one after
+        if (kb + 1 < n_blocks) {
+            commit_to(smem + ((kb + 1) & 1) * AT_BUF);
+            if (kb + 2 < n_blocks) fetch(kb + 2);
         }
-        // ---- scale, mask, running maximum ----
+
+        // ---- scale (base-2 logits), mask, running maximum ----
+        // a block needs the per-element mask only at the ragged end of the keys or where it meets the diagonal
+        const bool edge = (kb + 1) * AT_BK > a.sk || (a.causal && (kb + 1) * AT_BK - 1 > wave_row0);
         float m_blk = -INFINITY;
 #pragma unroll
         for (int t = 0; t < AT_BK / 32; t++)
@@ -190,17 +209,19 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
             for (int q = 0; q < 4; q++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const int key = kb * AT_BK + t * 32 + 8 * q + 4 * lh + e;
-                    float s = s_acc[t][4 * q + e] * a.scale;
-                    if (key >= a.sk || (a.causal && key > my_row)) s = -INFINITY;
-                    s_acc[t][4 * q + e] = s;
-                    m_blk = s > m_blk ? s : m_blk;
+                    float sv = s_acc[t][4 * q + e] * a.scale_log2e;
+                    if (edge) {
+                        const int key = kb * AT_BK + t * 32 + 8 * q + 4 * lh + e;
+                        if (key >= a.sk || (a.causal && key > my_row)) sv = -INFINITY;
+                    }
+                    s_acc[t][4 * q + e] = sv;
+                    m_blk = sv > m_blk ? sv : m_blk;
                 }
         const float m_other = partner(m_blk);
         m_blk = m_other > m_blk ? m_other : m_blk;
         const float m_new = m_blk > m_run ? m_blk : m_run;
         // every row has at least key 0 unmasked in its first block, so m_new is finite from the first block on
-        const float rescale = __expf(m_run - m_new);  // 0 on the first block (m_run = -inf)
+        const float rescale = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first block (m_run = -inf)
         m_run = m_new;
         float l_blk = 0.f;
         uint32_t p_pack[AT_BK / 32][8];  // [tile][2 * q + pair]: keys 8 * q + 4 * lh + {0, 1} and {2, 3}
@@ -211,7 +232,7 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
                 float p[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    p[e] = __expf(s_acc[t][4 * q + e] - m_new);  // exp(-inf) = 0 for masked keys
+                    p[e] = __builtin_amdgcn_exp2f(s_acc[t][4 * q + e] - m_new);  // exp2(-inf) = 0 for masked keys
                     l_blk += p[e];
                 }
                 p_pack[t][2 * q] = Narrow<CK>::pack(p[0], p[1]);
@@ -219,10 +240,13 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
             }
         l_blk += partner(l_blk);
         l_run = l_run * rescale + l_blk;
+        // the running maximum settles after a few blocks: the accumulators are rescaled only while some row's moves
+        if (__builtin_amdgcn_ballot_w64(rescale != 1.0f) != 0) {
 #pragma unroll
-        for (int j = 0; j < AT_D / 32; j++)
+            for (int j = 0; j < AT_D / 32; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) o_acc[j][e] *= rescale;
+                for (int e = 0; e < 16; e++) o_acc[j][e] *= rescale;
+        }
 
         // ---- O += P V: four 16-key slices ----
 #pragma unroll
@@ -240,6 +264,7 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
                 Cmp::mma(u32x4_t{lo.x, lo.y, hi.x, hi.y}, pf, o_acc[j]);
             }
         }
+        __syncthreads();  // this block's buffer may be overwritten, the next one's is complete
     }
 
     // ---- O / l, one rounding, 8-byte stores: lane (lr, lh) holds row lr, head-dim columns 32 j + 8 q + 4 lh + e ----
@@ -283,11 +308,19 @@ int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k
     }
     a.q_off = g.q_off; a.k_off = g.k_off; a.v_off = g.v_off;
     a.batches = g.batches;
-    a.scale = g.scale;
+    a.scale_log2e = g.scale * 1.44269504088896340736f;
     a.causal = g.causal ? 1 : 0;
     a.q_blocks = (int)((g.sq + AT_BQ - 1) / AT_BQ);
     const long blocks = g.batches * a.q_blocks;
     if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
+    static bool configured = false;  // benign race: the attribute calls are idempotent
+    if (!configured) {
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_BF16>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, AT_LDS));
+        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_F16>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, AT_LDS));
+        configured = true;
+    }
     if (dtype == HODU_BF16) {
         ctx->last_kernel = "attention_fwd_bf16";
         hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_BF16>, dim3((unsigned)blocks), dim3(256), AT_LDS, ctx->stream,
