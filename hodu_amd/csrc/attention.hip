@@ -3,11 +3,21 @@
 // hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) is, in the reference, a
 // batched matmul, mul_scalar, (mask construction + masked_fill,) the five kernels of Tensor::softmax
 // (crates/hodu_core/src/tensor/ops/normalization.rs:4-21) and a second batched matmul; the [.., Sq, Sk] scores cross
-// memory eight times.  Here a workgroup owns 128 query rows of one head (a wavefront 32 of them) and walks the keys
-// in blocks of 64: S = Q K^T on the matrix cores, the running row maximum and row sum of the online softmax in
-// registers, P = exp(S - max) converted in registers to the operand layout of the second product, O += P V on the
-// matrix cores, one division and one rounding at the end.  Head dim 128, bf16 or f16, K-dense rows; everything else
-// takes the three-launch path (product with fused scale, hodu_rocm_softmax, product).
+// memory eight times.  Here a workgroup owns 128 query rows of one head and walks the keys in blocks of 64.  Its
+// eight wavefronts are 4 groups of 32 query rows x 2 halves of every key block: a wavefront computes S = Q K^T for
+// its 32 rows and 32 keys on the matrix cores, keeps a reference maximum and the row sum of the online softmax of
+// ITS keys in registers, converts P = exp(S - m) in registers to the operand layout of the second product and
+// adds P V to its own accumulators on the matrix cores.  The two wavefronts of a row group meet once, at the end,
+// through LDS: O = (O1 w1 + O2 w2) / (l1 w1 + l2 w2) with w = exp(m - max(m1, m2)), one division and one rounding.
+// Spreading a query block over eight wavefronts instead of four halves the time a workgroup needs per key block,
+// which is what a causal launch with few heads waits for.  Head dim 128, bf16 or f16, K-dense rows, a positive
+// scale; everything else takes the three-launch path (product with fused scale, hodu_rocm_softmax, product).
+//
+// Pipeline: K and V blocks go from memory straight into LDS (global_load_lds, no registers in between), K one block
+// ahead of V, each into a ring of two; a wavefront computes the scores of block i + 1 on the matrix cores while its
+// vector ALU runs the softmax of block i (the two are independent, so the compiler interleaves them), then P V of
+// block i; one barrier per block.  The exponent reference of a row follows its running maximum lazily (see
+// row_max), so the accumulators are rescaled on the first block and then almost never.
 //
 // Layouts (the MFMAs run with swapped operands, as in the GEMM kernels, so that a lane owns ONE query row):
 //   * 32x32x16 MFMA, mma(first, second, acc): both operands hold, in lane (lr, lh) = (lane % 32, lane / 32), the 8
@@ -21,8 +31,9 @@
 //     trade one packed register pair (v_permlane32_swap).
 //
 // Arithmetic: scores and probabilities in f32 (no rounding of the scores to the storage type, unlike the
-// three-launch path and the reference), P rounded to the storage type only as the second product's operand, O
-// accumulated in f32 and rounded once.  The scale is the scalar in the storage type, widened.
+// three-launch path and the reference), exp(scale * (s - m)) as one fused multiply-add into a base-2 exponential, P
+// (at most 2^8) rounded to the storage type only as the second product's operand, O accumulated in f32 and rounded
+// once.  The scale is the scalar in the storage type, widened.
 #include "common.hpp"
 #include "device_types.hpp"
 #include "gemm_mfma_pipe.hpp"
@@ -37,13 +48,17 @@ using mfma::lds_get;
 using mfma::lds_get_tr;
 
 constexpr int AT_D = 128;        // head dim
-constexpr int AT_BQ = 128;       // query rows per workgroup (32 per wavefront)
-constexpr int AT_BK = 64;        // keys per step
+constexpr int AT_BQ = 128;       // query rows per workgroup (4 groups of 32)
+constexpr int AT_BK = 64;        // keys per step (2 halves of 32, one per wavefront of a row group)
+constexpr int AT_NT = 512;       // 8 wavefronts: wave & 3 = row group, wave >> 2 = key half
 constexpr int AT_KSTEPS = AT_D / 16;
 constexpr int AT_K_BYTES = AT_BK * AT_D * 2;  // 16 KB: K block, two halves of [64 rows][128 bytes]
 constexpr int AT_V_BYTES = AT_BK * AT_D * 2;  // 16 KB: V block, [64 keys][256 bytes]
 constexpr int AT_BUF = AT_K_BYTES + AT_V_BYTES;  // one K block and one V block
-constexpr int AT_LDS = 2 * AT_BUF;              // two of them: the next block is written while this one is read
+// two of them: the next block is written while this one is read.  The same memory carries, at the end, the second
+// key half's (m, l, O) of every row: 4 row groups x 66 floats x 64 lanes
+constexpr int AT_MERGE = 4 * (2 + AT_D / 2) * 64 * 4;
+constexpr int AT_LDS = AT_MERGE > 2 * AT_BUF ? AT_MERGE : 2 * AT_BUF;
 
 struct DevAttention {
     int sq, sk;
@@ -83,14 +98,16 @@ __device__ __forceinline__ float partner(float v) {
 }
 
 template <int CK>
-__global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
-                                                              const uint16_t *__restrict__ V, uint16_t *__restrict__ O,
-                                                              DevAttention a) {
+__global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
+                                                               const uint16_t *__restrict__ V, uint16_t *__restrict__ O,
+                                                               DevAttention a) {
     typedef Compute32<CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     extern __shared__ __align__(16) char smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, lh = lane >> 5;
+    const int qg = wave & 3, kh = wave >> 2;
     // the last query block of every head first: with the causal mask it walks the most keys, and the workgroups that
     // finish the launch should be the short ones
     const long batch = blockIdx.x % a.batches;
@@ -107,9 +124,73 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
             }
     }
 
+    // keys this workgroup needs: with the causal mask nothing beyond its last query row
+    int k_end = a.sk;
+    if (a.causal) {
+        const int last = q0 + AT_BQ < a.sq ? q0 + AT_BQ : a.sq;
+        k_end = last < a.sk ? last : a.sk;
+    }
+    const int n_blocks = (k_end + AT_BK - 1) / AT_BK;  // >= 1: Sk >= 1
+
+    // ---- global -> LDS without registers in between (global_load_lds_dwordx4: a wavefront's 64 lanes fill 1 KB of
+    // consecutive LDS, so the lane that owns an LDS slot fetches the chunk the swizzle puts there).  16 such
+    // instructions per K block and per V block, two of each per wavefront ----
+    const uint16_t *k_src[2], *v_src[2];   // the lane's source in block 0
+    int k_srow[2], v_srow[2];              // its key row within the block
+    unsigned k_dst[2], v_dst[2];           // LDS byte offset of the instruction within the block's buffer
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int i = wave + 8 * p;
+        // K: two halves of [64 rows][128 bytes]; instruction i fills rows (i % 8) * 8 .. + 7 of half i / 8
+        k_srow[p] = (i & 7) * 8 + (lane >> 3);
+        k_src[p] = K + ko + (long)k_srow[p] * a.k_row + (i >> 3) * 64 + ((lane & 7) ^ ((k_srow[p] >> 1) & 7)) * 8;
+        k_dst[p] = i * 1024;
+        // V: [64 keys][256 bytes]; instruction i fills keys 4 i .. 4 i + 3
+        v_srow[p] = i * 4 + (lane >> 4);
+        v_src[p] = V + vo + (long)v_srow[p] * a.v_row + ((lane & 15) ^ ((v_srow[p] & 3) << 2)) * 8;
+        v_dst[p] = i * 1024;
+    }
+    auto dma_k = [&](int kb, int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            int key = kb * AT_BK + k_srow[p];
+            key = key < a.sk ? key : a.sk - 1;  // ragged tail: clamped, masked below
+            mfma::dma16_raw(reinterpret_cast<const char *>(k_src[p] + (long)(key - k_srow[p]) * a.k_row),
+                            __builtin_amdgcn_readfirstlane(lds0 + buf * AT_K_BYTES + k_dst[p]));
+        }
+    };
+    auto dma_v = [&](int kb, int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            int key = kb * AT_BK + v_srow[p];
+            key = key < a.sk ? key : a.sk - 1;
+            mfma::dma16_raw(reinterpret_cast<const char *>(v_src[p] + (long)(key - v_srow[p]) * a.v_row),
+                            __builtin_amdgcn_readfirstlane(lds0 + 2 * AT_K_BYTES + buf * AT_V_BYTES + v_dst[p]));
+        }
+    };
+    // the same for a block that lies wholly inside the keys: one wavefront-uniform offset
+    auto dma_k_full = [&](int kb, int buf) {
+        const long step = (long)kb * AT_BK * a.k_row;
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+            mfma::dma16_raw(reinterpret_cast<const char *>(k_src[p] + step),
+                            __builtin_amdgcn_readfirstlane(lds0 + buf * AT_K_BYTES + k_dst[p]));
+    };
+    auto dma_v_full = [&](int kb, int buf) {
+        const long step = (long)kb * AT_BK * a.v_row;
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+            mfma::dma16_raw(reinterpret_cast<const char *>(v_src[p] + step),
+                            __builtin_amdgcn_readfirstlane(lds0 + 2 * AT_K_BYTES + buf * AT_V_BYTES + v_dst[p]));
+    };
+    // K runs one block ahead of V: the scores of block kb + 1 are computed while block kb goes through the softmax
+    dma_k(0, 0);
+    dma_v(0, 0);
+    if (n_blocks > 1) dma_k(1, 1);
+
     // Q fragments of the wavefront's 32 rows stay in registers: lane (lr, lh) holds, per 16-wide slice of the head
     // dim, the 8 elements at 16 * ks + 8 * lh of row lr (rows past Sq are clamped; their results are not stored)
-    const int my_row = q0 + wave * 32 + lr;
+    const int my_row = q0 + qg * 32 + lr;
     const int q_row = my_row < a.sq ? my_row : a.sq - 1;
     u32x4_t qf[AT_KSTEPS];
 #pragma unroll
@@ -121,150 +202,244 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const uint16_t *_
     for (int j = 0; j < AT_D / 32; j++)
 #pragma unroll
         for (int e = 0; e < 16; e++) o_acc[j][e] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;  // the maximum is kept on the raw scores (the scale is positive)
 
-    // keys this workgroup needs: with the causal mask nothing beyond its last query row
-    int k_end = a.sk;
-    if (a.causal) {
-        const int last = q0 + AT_BQ < a.sq ? q0 + AT_BQ : a.sq;
-        k_end = last < a.sk ? last : a.sk;
-    }
-    const int n_blocks = (k_end + AT_BK - 1) / AT_BK;
-
-    // global -> register staging of one K block and one V block: 1024 16-byte chunks each, 4 per thread
-    u32x4_t kst[4], vst[4];
-    auto fetch = [&](int kb) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + 256 * i;           // chunk id: key row = c / 16, chunk of the 256-byte row = c % 16
-            int key = kb * AT_BK + (c >> 4);
-            key = key < a.sk ? key : a.sk - 1;     // ragged tail: clamped, masked below
-            kst[i] = *reinterpret_cast<const u32x4_t *>(K + ko + (long)key * a.k_row + (c & 15) * 8);
-            vst[i] = *reinterpret_cast<const u32x4_t *>(V + vo + (long)key * a.v_row + (c & 15) * 8);
-        }
-    };
-    // fragment addresses
-    int k_frag[AT_KSTEPS];  // K block, tile 0; tile t adds t * 32 * 128
+    // fragment addresses within a buffer
+    int k_frag[AT_KSTEPS];  // K block, the wavefront's 32 keys
 #pragma unroll
     for (int ks = 0; ks < AT_KSTEPS; ks++)
-        k_frag[ks] = (ks >> 2) * (AT_BK * 128) + lr * 128 + (kd_slot(lr, 2 * (ks & 3) + lh) << 4);
-    int v_mn[AT_D / 32];    // V block through transpose reads: head-dim tile j, 16-key slice 0
+        k_frag[ks] = (ks >> 2) * (AT_BK * 128) + (kh * 32 + lr) * 128 + (kd_slot(lr, 2 * (ks & 3) + lh) << 4);
+    int v_mn[AT_D / 32];    // V block through transpose reads: head-dim tile j, first 16-key slice of the wavefront
     {
         const int s16 = lane & 15, kq = s16 >> 2, sub = s16 & 3;
         const int col_bytes = ((lane >> 4) & 1) * 32 + sub * 8;
 #pragma unroll
         for (int j = 0; j < AT_D / 32; j++) {
             const int bytes = j * 64 + col_bytes, c = bytes >> 4;
-            v_mn[j] = (lh * 8 + kq) * (AT_D * 2) + ((c ^ (kq << 2)) << 4) + (bytes & 8);
+            v_mn[j] = (kh * 32 + lh * 8 + kq) * (AT_D * 2) + ((c ^ (kq << 2)) << 4) + (bytes & 8);
         }
     }
-
-    auto commit_to = [&](char *buf) {
-        char *k_lds = buf, *v_lds = buf + AT_K_BYTES;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + 256 * i, row = c >> 4, g = c & 15;
-            // K: half g / 8 of the row, chunk g % 8 at its swizzled slot
-            *reinterpret_cast<u32x4_t *>(k_lds + (g >> 3) * (AT_BK * 128) + row * 128 + (kd_slot(row, g & 7) << 4)) = kst[i];
-            // V: [key][256 bytes], chunk g at slot g ^ ((key & 3) << 2)
-            *reinterpret_cast<u32x4_t *>(v_lds + row * (AT_D * 2) + ((g ^ ((row & 3) << 2)) << 4)) = vst[i];
-        }
+    const int wave_row0 = q0 + qg * 32;  // the wavefront's first query row
+    // the wavefront has nothing to do in a block whose 32 keys of its half lie past the end, or past the mask of all
+    // its 32 rows; the tile needs the per-element mask at the ragged end of the keys and where it meets the diagonal
+    auto idle_in = [&](int kb) {
+        const int key0 = kb * AT_BK + kh * 32;
+        return kb >= n_blocks || key0 >= a.sk || (a.causal && key0 > wave_row0 + 31);
+    };
+    auto edge_in = [&](int kb) {
+        const int key0 = kb * AT_BK + kh * 32;
+        return key0 + 32 > a.sk || (a.causal && key0 + 31 > wave_row0);
     };
 
-    if (n_blocks > 0) {
-        fetch(0);
-        commit_to(smem);
-        if (n_blocks > 1) fetch(1);
+    // ---- the phases ----
+    auto read_k = [&](u32x4_t (&kf)[AT_KSTEPS], int buf) {
+        const char *k_lds = smem + buf * AT_K_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < AT_KSTEPS; ks++) kf[ks] = lds_get(k_lds, k_frag[ks]);
+    };
+    auto read_v = [&](u32x2_t (&vf)[AT_D / 32][2], int buf, int sl) {  // one 16-key slice
+        const char *v_lds = smem + 2 * AT_K_BYTES + buf * AT_V_BYTES;
+#pragma unroll
+        for (int j = 0; j < AT_D / 32; j++) {
+            vf[j][0] = lds_get_tr<2>(v_lds, v_mn[j] + (sl * 16) * (AT_D * 2));
+            vf[j][1] = lds_get_tr<2>(v_lds, v_mn[j] + (sl * 16 + 4) * (AT_D * 2));
+        }
+    };
+    // S = Q K^T: steps [from, to) of the chain over the head dim
+    auto scores = [&](const u32x4_t (&kf)[AT_KSTEPS], acc_t &sc, int from, int to) {
+#pragma unroll
+        for (int ks = from; ks < to; ks++) Cmp::mma(kf[ks], qf[ks], sc);
+    };
+    auto zero = [&](acc_t &sc) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) sc[e] = 0.f;
+    };
+    auto mask = [&](acc_t &sc, int kb) {
+        const int key0 = kb * AT_BK + kh * 32;
+        const int limit = a.causal && my_row < a.sk - 1 ? my_row : a.sk - 1;  // last key the row attends
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) sc[4 * q + e] = key0 + 8 * q + 4 * lh + e > limit ? -INFINITY : sc[4 * q + e];
+    };
+    // The reference value m_run of a row (exponents are taken relative to it) follows the running maximum lazily: it
+    // moves only when a block's maximum exceeds it by more than 8 in the base-2 exponent, so P stays below 2^8 --
+    // harmless in f32 sums and in the 16-bit operand, whose precision is relative -- and the 64 accumulator
+    // registers are rescaled on the first block and then almost never, instead of whenever one of the wavefront's
+    // 32 rows meets a new maximum (which with 32 rows is nearly every block).  The result is the same quotient.
+    // Returns true if some row's accumulators need the rescale.
+    float rescale, neg_mc;
+    auto row_max = [&](const acc_t &sc) {
+        float m_blk = sc[0];
+#pragma unroll
+        for (int e = 1; e < 16; e++) m_blk = __builtin_fmaxf(m_blk, sc[e]);
+        m_blk = __builtin_fmaxf(m_blk, partner(m_blk));
+        // true from -inf (first unmasked key); false for -inf - -inf = NaN (nothing unmasked yet)
+        const bool up = (m_blk - m_run) * a.scale_log2e > 8.f;
+        const float m_new = up ? m_blk : m_run;
+        // a row of the second key half may not have met an unmasked key yet: its reference is still -inf, and
+        // exp2(-inf) = 0 keeps its sums at zero instead of producing inf - inf
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        rescale = up ? __builtin_amdgcn_exp2f((m_run - m_use) * a.scale_log2e) : 1.0f;  // 0 from m_run = -inf
+        neg_mc = -m_use * a.scale_log2e;
+        m_run = m_new;
+        return __builtin_amdgcn_ballot_w64(up) != 0;
+    };
+    // (in place, through the assembler: written as C++ the conditional product makes the compiler keep two copies of
+    // the 64 accumulator registers around the branch and move one onto the other in every iteration)
+    auto rescale_o = [&]() {
+#pragma unroll
+        for (int j = 0; j < AT_D / 32; j++)
+            asm volatile("v_mul_f32 %0, %16, %0\n\tv_mul_f32 %1, %16, %1\n\tv_mul_f32 %2, %16, %2\n\tv_mul_f32 %3, %16, %3\n\t"
+                         "v_mul_f32 %4, %16, %4\n\tv_mul_f32 %5, %16, %5\n\tv_mul_f32 %6, %16, %6\n\tv_mul_f32 %7, %16, %7\n\t"
+                         "v_mul_f32 %8, %16, %8\n\tv_mul_f32 %9, %16, %9\n\tv_mul_f32 %10, %16, %10\n\tv_mul_f32 %11, %16, %11\n\t"
+                         "v_mul_f32 %12, %16, %12\n\tv_mul_f32 %13, %16, %13\n\tv_mul_f32 %14, %16, %14\n\tv_mul_f32 %15, %16, %15"
+                         : "+v"(o_acc[j][0]), "+v"(o_acc[j][1]), "+v"(o_acc[j][2]), "+v"(o_acc[j][3]), "+v"(o_acc[j][4]),
+                           "+v"(o_acc[j][5]), "+v"(o_acc[j][6]), "+v"(o_acc[j][7]), "+v"(o_acc[j][8]), "+v"(o_acc[j][9]),
+                           "+v"(o_acc[j][10]), "+v"(o_acc[j][11]), "+v"(o_acc[j][12]), "+v"(o_acc[j][13]),
+                           "+v"(o_acc[j][14]), "+v"(o_acc[j][15])
+                         : "v"(rescale));
+    };
+    // P of one 16-key slice (groups q = 2 sl and 2 sl + 1) in operand layout; adds the slice's row sums to l_blk
+    auto probs = [&](const acc_t &sc, int sl, float &l_blk) {
+        uint32_t pk[4];  // [2 * (q - 2 sl) + pair]: keys 8 * q + 4 * lh + {0, 1} and {2, 3}
+#pragma unroll
+        for (int qq = 0; qq < 2; qq++) {
+            float p[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                // exp(scale * (s - m)) as one fused multiply-add and a base-2 exponential; 0 for masked keys
+                p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[4 * (2 * sl + qq) + e], a.scale_log2e, neg_mc));
+                l_blk += p[e];
+            }
+            pk[2 * qq] = Narrow<CK>::pack(p[0], p[1]);
+            pk[2 * qq + 1] = Narrow<CK>::pack(p[2], p[3]);
+        }
+        // lane lh = 0 keeps group 2 sl and receives the partner's; lane lh = 1 receives the partner's group 2 sl + 1
+        // and keeps its own: one swap per packed register
+        const auto w0 = __builtin_amdgcn_permlane32_swap(pk[0], pk[2], false, false);
+        const auto w1 = __builtin_amdgcn_permlane32_swap(pk[1], pk[3], false, false);
+        return u32x4_t{w0[0], w1[0], w0[1], w1[1]};
+    };
+    auto pv = [&](const u32x2_t (&vf)[AT_D / 32][2], const u32x4_t &pf) {  // O += P V for one slice
+#pragma unroll
+        for (int j = 0; j < AT_D / 32; j++) Cmp::mma(u32x4_t{vf[j][0].x, vf[j][0].y, vf[j][1].x, vf[j][1].y}, pf, o_acc[j]);
+    };
+    // (l_run is the lane's share of the row sum; the two lanes of a row add up at the end)
+    auto finish_row_sum = [&](float l_blk) { l_run = l_run * rescale + l_blk; };
+
+    // ---- prologue: the first block's scores ----
+    __builtin_amdgcn_s_waitcnt(mfma::waitcnt_vm_lgkm0(0));
+    // (the Q registers are pinned so that the compiler's wait-count tracking knows, on every path into the loop,
+    // that their loads have returned; otherwise it waits for them, i.e. for every load in flight, inside the loop)
+#pragma unroll
+    for (int ks = 0; ks < AT_KSTEPS; ks++) asm volatile("" : "+v"(qf[ks]));
+    __syncthreads();
+    acc_t s_cur;
+    zero(s_cur);
+    {
+        u32x4_t kf[AT_KSTEPS];
+        read_k(kf, 0);
+        scores(kf, s_cur, 0, AT_KSTEPS);  // (the second key half's result is not used where its block 0 is idle)
+    }
+    __syncthreads();  // K buffer 0 may be overwritten
+
+    // The leading blocks of a wavefront need neither the mask nor a test for idleness (both only ever begin to
+    // apply, towards the diagonal and the ragged end).  They run in a loop of their own, whose body is two straight
+    // blocks around the rarely taken rescale: the matrix cores compute the next block's scores while the vector ALU
+    // runs this block's softmax.  The remaining blocks take the general body.  Every wavefront meets one barrier per
+    // block either way.
+    int n_fast = 0;
+    auto loads_whole = [&](int kb) {  // what block kb's iteration loads lies wholly inside the keys
+        return (kb + 2 >= n_blocks || (kb + 3) * AT_BK <= a.sk) && (kb + 1 >= n_blocks || (kb + 2) * AT_BK <= a.sk);
+    };
+    while (n_fast < n_blocks && !idle_in(n_fast) && !idle_in(n_fast + 1) && !edge_in(n_fast) && loads_whole(n_fast)) n_fast++;
+    auto next_loads = [&](int kb) {
+        // K of the block after next into the buffer S(kb) was read from (behind a barrier), V of the next block into
+        // the buffer P V of the previous block was read from (behind the same barrier)
+        if (kb + 2 < n_blocks) dma_k(kb + 2, kb & 1);
+        if (kb + 1 < n_blocks) dma_v(kb + 1, (kb + 1) & 1);
+    };
+    auto publish = [&]() {
+        __builtin_amdgcn_s_waitcnt(mfma::waitcnt_vm_lgkm0(0));  // this wavefront's part of the next loads has landed
+        __syncthreads();  // everybody's has; what this iteration read may be overwritten
+    };
+    int kb = 0;
+    for (; kb < n_fast; kb++) {
+        if (kb + 2 < n_blocks) dma_k_full(kb + 2, kb & 1);
+        if (kb + 1 < n_blocks) dma_v_full(kb + 1, (kb + 1) & 1);
+        u32x4_t kf[AT_KSTEPS];
+        u32x2_t vf0[AT_D / 32][2], vf1[AT_D / 32][2];
+        read_k(kf, (kb + 1) & 1);
+        read_v(vf0, kb & 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        acc_t s_next;
+        zero(s_next);
+        scores(kf, s_next, 0, 3);
+        if (row_max(s_cur)) rescale_o();
+        scores(kf, s_next, 3, AT_KSTEPS);
+        float l_blk = 0.f;
+        const u32x4_t pf0 = probs(s_cur, 0, l_blk);
+        read_v(vf1, kb & 1, 1);
+        pv(vf0, pf0);
+        const u32x4_t pf1 = probs(s_cur, 1, l_blk);
+        pv(vf1, pf1);
+        finish_row_sum(l_blk);
+        s_cur = s_next;
+        publish();
+    }
+    for (; kb < n_blocks; kb++) {
+        next_loads(kb);
+        acc_t s_next;
+        zero(s_next);
+        if (!idle_in(kb + 1)) {
+            u32x4_t kf[AT_KSTEPS];
+            read_k(kf, (kb + 1) & 1);
+            scores(kf, s_next, 0, AT_KSTEPS);
+        }
+        if (!idle_in(kb)) {
+            u32x2_t vf0[AT_D / 32][2], vf1[AT_D / 32][2];
+            read_v(vf0, kb & 1, 0);
+            read_v(vf1, kb & 1, 1);
+            mask(s_cur, kb);
+            if (row_max(s_cur)) rescale_o();
+            float l_blk = 0.f;
+            const u32x4_t pf0 = probs(s_cur, 0, l_blk);
+            pv(vf0, pf0);
+            const u32x4_t pf1 = probs(s_cur, 1, l_blk);
+            pv(vf1, pf1);
+            finish_row_sum(l_blk);
+        }
+        s_cur = s_next;
+        publish();
+    }
+
+    // ---- the two key halves of a row group meet: the second half hands (m, l, O) over through LDS, one float per
+    // lane and register so that a wavefront's store covers 64 consecutive words (every K / V read is behind the
+    // loop's last barrier) ----
+    float *mg = reinterpret_cast<float *>(smem) + qg * ((2 + AT_D / 2) * 64) + lane;
+    l_run += partner(l_run);
+    if (kh == 1) {
+        mg[0] = m_run;
+        mg[64] = l_run;
+#pragma unroll
+        for (int j = 0; j < AT_D / 32; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) mg[(2 + 16 * j + e) * 64] = o_acc[j][e];
     }
     __syncthreads();
-    const int wave_row0 = q0 + wave * 32;  // the wavefront's first query row
-    for (int kb = 0; kb < n_blocks; kb++) {
-        const char *k_lds = smem + (kb & 1) * AT_BUF, *v_lds = k_lds + AT_K_BYTES;
-
-        // ---- S = Q K^T: two 32-key tiles, their accumulation chains interleaved ----
-        acc_t s_acc[AT_BK / 32];
+    if (kh == 1) return;
+    {
+        // the first half has seen key 0, which no row masks: its reference is finite; the second half's may be -inf
+        // (w2 = 0).  Any common reference gives the same quotient.
+        const float m2 = mg[0], l2 = mg[64];
+        const float m = __builtin_fmaxf(m2, m_run);
+        const float w1 = __builtin_amdgcn_exp2f((m_run - m) * a.scale_log2e), w2 = __builtin_amdgcn_exp2f((m2 - m) * a.scale_log2e);
+        l_run = l_run * w1 + l2 * w2;
 #pragma unroll
-        for (int t = 0; t < AT_BK / 32; t++)
+        for (int j = 0; j < AT_D / 32; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) s_acc[t][e] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < AT_KSTEPS; ks++)
-#pragma unroll
-            for (int t = 0; t < AT_BK / 32; t++) Cmp::mma(lds_get(k_lds, k_frag[ks] + t * 32 * 128), qf[ks], s_acc[t]);
-
-        // the next block's K and V have had the S phase to arrive: into the other buffer (nobody reads it: the
-        // barrier at the end of the previous iteration came after its last read), then fetch the one after
-        if (kb + 1 < n_blocks) {
-            commit_to(smem + ((kb + 1) & 1) * AT_BUF);
-            if (kb + 2 < n_blocks) fetch(kb + 2);
-        }
-
-        // ---- scale (base-2 logits), mask, running maximum ----
-        // a block needs the per-element mask only at the ragged end of the keys or where it meets the diagonal
-        const bool edge = (kb + 1) * AT_BK > a.sk || (a.causal && (kb + 1) * AT_BK - 1 > wave_row0);
-        float m_blk = -INFINITY;
-#pragma unroll
-        for (int t = 0; t < AT_BK / 32; t++)
-#pragma unroll
-            for (int q = 0; q < 4; q++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float sv = s_acc[t][4 * q + e] * a.scale_log2e;
-                    if (edge) {
-                        const int key = kb * AT_BK + t * 32 + 8 * q + 4 * lh + e;
-                        if (key >= a.sk || (a.causal && key > my_row)) sv = -INFINITY;
-                    }
-                    s_acc[t][4 * q + e] = sv;
-                    m_blk = sv > m_blk ? sv : m_blk;
-                }
-        const float m_other = partner(m_blk);
-        m_blk = m_other > m_blk ? m_other : m_blk;
-        const float m_new = m_blk > m_run ? m_blk : m_run;
-        // every row has at least key 0 unmasked in its first block, so m_new is finite from the first block on
-        const float rescale = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first block (m_run = -inf)
-        m_run = m_new;
-        float l_blk = 0.f;
-        uint32_t p_pack[AT_BK / 32][8];  // [tile][2 * q + pair]: keys 8 * q + 4 * lh + {0, 1} and {2, 3}
-#pragma unroll
-        for (int t = 0; t < AT_BK / 32; t++)
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                float p[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    p[e] = __builtin_amdgcn_exp2f(s_acc[t][4 * q + e] - m_new);  // exp2(-inf) = 0 for masked keys
-                    l_blk += p[e];
-                }
-                p_pack[t][2 * q] = Narrow<CK>::pack(p[0], p[1]);
-                p_pack[t][2 * q + 1] = Narrow<CK>::pack(p[2], p[3]);
-            }
-        l_blk += partner(l_blk);
-        l_run = l_run * rescale + l_blk;
-        // the running maximum settles after a few blocks: the accumulators are rescaled only while some row's moves
-        if (__builtin_amdgcn_ballot_w64(rescale != 1.0f) != 0) {
-#pragma unroll
-            for (int j = 0; j < AT_D / 32; j++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) o_acc[j][e] *= rescale;
-        }
-
-        // ---- O += P V: four 16-key slices ----
-#pragma unroll
-        for (int sl = 0; sl < AT_BK / 16; sl++) {
-            const int t = sl >> 1, qe = 2 * (sl & 1);  // the slice's keys are groups q = qe and qe + 1 of tile t
-            // lane lh = 0 keeps group qe and receives the partner's group qe; lane lh = 1 receives the partner's
-            // group qe + 1 and keeps its own: one swap per packed register
-            const auto w0 = __builtin_amdgcn_permlane32_swap(p_pack[t][2 * qe], p_pack[t][2 * qe + 2], false, false);
-            const auto w1 = __builtin_amdgcn_permlane32_swap(p_pack[t][2 * qe + 1], p_pack[t][2 * qe + 3], false, false);
-            const u32x4_t pf = {w0[0], w1[0], w0[1], w1[1]};
-#pragma unroll
-            for (int j = 0; j < AT_D / 32; j++) {
-                const u32x2_t lo = lds_get_tr<2>(v_lds, v_mn[j] + (sl * 16) * (AT_D * 2));
-                const u32x2_t hi = lds_get_tr<2>(v_lds, v_mn[j] + (sl * 16 + 4) * (AT_D * 2));
-                Cmp::mma(u32x4_t{lo.x, lo.y, hi.x, hi.y}, pf, o_acc[j]);
-            }
-        }
-        __syncthreads();  // this block's buffer may be overwritten, the next one's is complete
+            for (int e = 0; e < 16; e++) o_acc[j][e] = o_acc[j][e] * w1 + mg[(2 + 16 * j + e) * 64] * w2;
     }
 
     // ---- O / l, one rounding, 8-byte stores: lane (lr, lh) holds row lr, head-dim columns 32 j + 8 q + 4 lh + e ----
@@ -289,6 +464,8 @@ int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k
                      const AttentionArgs &g) {
     if (dtype != HODU_BF16 && dtype != HODU_F16) return HODU_ROCM_UNSUPPORTED;
     if (g.d != AT_D || g.sq < 1 || g.sk < 1 || g.batches < 1) return HODU_ROCM_UNSUPPORTED;
+    // the row maximum is taken before the scale is applied: the scale must be positive (and finite)
+    if (!(g.scale > 0.f) || !(g.scale < INFINITY)) return HODU_ROCM_UNSUPPORTED;
     if (g.nb > kKernelBatchDims) return HODU_ROCM_UNSUPPORTED;
     // 16-byte loads of 8 elements: rows, offsets, batch strides and bases aligned to 8 elements / 16 bytes
     auto al = [](long e) { return e % 8 == 0; };
@@ -323,11 +500,11 @@ int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k
     }
     if (dtype == HODU_BF16) {
         ctx->last_kernel = "attention_fwd_bf16";
-        hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_BF16>, dim3((unsigned)blocks), dim3(256), AT_LDS, ctx->stream,
+        hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_BF16>, dim3((unsigned)blocks), dim3(AT_NT), AT_LDS, ctx->stream,
                            (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, (uint16_t *)out, a);
     } else {
         ctx->last_kernel = "attention_fwd_f16";
-        hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_F16>, dim3((unsigned)blocks), dim3(256), AT_LDS, ctx->stream,
+        hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_F16>, dim3((unsigned)blocks), dim3(AT_NT), AT_LDS, ctx->stream,
                            (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, (uint16_t *)out, a);
     }
     HODU_HIP(hipGetLastError());

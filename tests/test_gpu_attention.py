@@ -2,7 +2,9 @@
 float64 on the exactly widened inputs, with the scale the kernel receives (the scalar in the storage type).
 Tolerance: the output is a convex combination of v rows delivered in bf16 / f16; probabilities are rounded to the
 storage type once as the second product's operand (relative 2^-9 / 2^-11) and the output once more, so the bar is the
-products' 2e-2, relative to max(|want|, mean |v| / sqrt(keys attended)) -- the floor of a sum that may cancel."""
+products' 2e-2, relative to max(|want|, mean |v| / sqrt(n_eff)) with n_eff = 1 / sum p^2 the effective number of keys
+the row attends -- the size of a sum of n_eff weighted v rows that may cancel, which is what a relative error of
+every p scales with."""
 import numpy as np
 import pytest
 
@@ -32,17 +34,33 @@ def reference(q, k, v, scale, causal):
         s = np.where(j > i, -np.inf, s)
     e = np.exp(s - s.max(-1, keepdims=True))
     p = e / e.sum(-1, keepdims=True)
-    return p @ v, (p > 0).sum(-1)
+    return p @ v, 1.0 / (p * p).sum(-1)  # the effective number of keys a row attends
 
 
-def check_attention(ctx, dt, batch, sq, sk, causal, seed=0, qv=None, kv=None, vv=None, vscale=1.0):
+def narrow(dt, x):
+    return (H.f32_to_bf16_rne if dt == "bf16" else H.f16_bits)(np.ascontiguousarray(x, dtype=np.float32))
+
+
+def check_attention(ctx, dt, batch, sq, sk, causal, seed=0, qv=None, kv=None, vv=None, vscale=1.0, qscale=1.0, ramp=None):
+    """ramp: logits that grow along the keys (contiguous operands only) -- q rows all point along one direction and
+    key j is that direction times ramp * f(j), f rising from 0 to 1 (or falling, ramp < 0), plus noise"""
     d = 128
     qv = qv or V(list(batch) + [sq, d])
     kv = kv or V(list(batch) + [sk, d])
     vv = vv or V(list(batch) + [sk, d])
-    q = H.random_storage(dt, qv.span(), 100 + seed, 1.0)
+    q = H.random_storage(dt, qv.span(), 100 + seed, qscale)
     k = H.random_storage(dt, kv.span(), 200 + seed, 1.0)
     v = H.random_storage(dt, vv.span(), 300 + seed, vscale)
+    if ramp is not None:
+        rng = np.random.default_rng(400 + seed)
+        u = np.ones(d, np.float32)
+        qa = u + 0.1 * rng.standard_normal((int(np.prod(batch, dtype=int)) * sq, d)).astype(np.float32)
+        f = np.arange(sk, dtype=np.float32) / max(sk - 1, 1)
+        f = f if ramp > 0 else 1.0 - f
+        # q . k_j * d^-1/2 ~ sqrt(d) * |ramp| * f(j)
+        ka = (abs(ramp) * f)[:, None] * u[None, :] + 0.1 * rng.standard_normal((sk, d)).astype(np.float32)
+        q = narrow(dt, qa).reshape(-1)
+        k = narrow(dt, np.tile(ka, (int(np.prod(batch, dtype=int)), 1))).reshape(-1)
     scale_bits = (H.f32_to_bf16_rne if dt == "bf16" else H.f16_bits)(np.array([1.0 / np.sqrt(d)], dtype=np.float32))
     scale = float(H.widen(dt, scale_bits)[0])
     n_out = int(np.prod(list(batch) + [sq, d]))
@@ -93,6 +111,17 @@ def test_large_logits_and_values(ctx):
     check_attention(ctx, "bf16", [2], 128, 192, False, seed=10, vscale=100.0)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_maxima_that_keep_moving(ctx, causal):
+    """the exponent reference of a row follows its maximum lazily (it moves only when a block exceeds it by 2^8): logits
+    that climb a little with every block (below the threshold per block, far above it in total), that climb steeply,
+    and that fall from a large first value; and logits with a large spread"""
+    check_attention(ctx, "bf16", [2], 160, 1024, causal, seed=11, ramp=6.0)     # ~ +2 per 32 keys, 68 in total
+    check_attention(ctx, "bf16", [2], 160, 512, causal, seed=12, ramp=40.0)     # ~ +28 per 32 keys
+    check_attention(ctx, "f16", [1], 96, 512, causal, seed=13, ramp=-10.0)      # the first keys dominate
+    check_attention(ctx, "bf16", [2], 128, 640, causal, seed=14, qscale=6.0)    # random logits of std ~ 6
+
+
 def test_unsupported_calls_are_refused(ctx):
     q, out = ctx.upload(np.zeros(64 * 64, np.uint16)), ctx.alloc(64 * 64 * 2)
     one = np.array([0x3F80], np.uint16)
@@ -102,4 +131,8 @@ def test_unsupported_calls_are_refused(ctx):
         ctx.attention("bf16", q, q, q, out, attention_md([], 8, 8, 128, V([8, 128], [1, 8]), V([8, 128]), V([8, 128])), one)
     with pytest.raises(ffi.HoduRocmError, match="words"):
         ctx.attention("bf16", q, q, q, out, [0, 8, 8, 128, 128, 1], one)
+    ok = attention_md([], 8, 8, 128, V([8, 128]), V([8, 128]), V([8, 128]))
+    for bits in (0xBF80, 0x0000, 0x7F80, 0x7FC0):  # -1, 0, inf, nan: the kernel takes the row maximum before scaling
+        with pytest.raises(ffi.HoduRocmError, match="positive finite scale"):
+            ctx.attention("bf16", q, q, q, out, ok, np.array([bits], np.uint16))
     q.free(); out.free()
