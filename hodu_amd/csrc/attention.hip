@@ -232,10 +232,10 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     };
 
     // ---- the phases ----
-    auto read_k = [&](u32x4_t (&kf)[AT_KSTEPS], int buf) {
+    auto read_k = [&](u32x4_t (&kf)[AT_KSTEPS], int buf, int from = 0, int to = AT_KSTEPS) {
         const char *k_lds = smem + buf * AT_K_BYTES;
 #pragma unroll
-        for (int ks = 0; ks < AT_KSTEPS; ks++) kf[ks] = lds_get(k_lds, k_frag[ks]);
+        for (int ks = from; ks < to; ks++) kf[ks] = lds_get(k_lds, k_frag[ks]);
     };
     auto read_v = [&](u32x2_t (&vf)[AT_D / 32][2], int buf, int sl) {  // one 16-key slice
         const char *v_lds = smem + 2 * AT_K_BYTES + buf * AT_V_BYTES;
@@ -364,29 +364,37 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
         __builtin_amdgcn_s_waitcnt(mfma::waitcnt_vm_lgkm0(0));  // this wavefront's part of the next loads has landed
         __syncthreads();  // everybody's has; what this iteration read may be overwritten
     };
-    int kb = 0;
-    for (; kb < n_fast; kb++) {
-        if (kb + 2 < n_blocks) dma_k_full(kb + 2, kb & 1);
-        if (kb + 1 < n_blocks) dma_v_full(kb + 1, (kb + 1) & 1);
+    // one fast iteration for a block of parity P (a literal at both call sites, so that ring slots become immediate
+    // offsets of the LDS instructions instead of an address add per read): S(kb) in s_in, S(kb + 1) into s_out
+    auto fast_block = [&](int kb, const int P, acc_t &s_in, acc_t &s_out) {
+        if (kb + 2 < n_blocks) dma_k_full(kb + 2, P);
+        if (kb + 1 < n_blocks) dma_v_full(kb + 1, 1 - P);
         u32x4_t kf[AT_KSTEPS];
         u32x2_t vf0[AT_D / 32][2], vf1[AT_D / 32][2];
-        read_k(kf, (kb + 1) & 1);
-        read_v(vf0, kb & 1, 0);
+        read_k(kf, 1 - P, 0, 4);
+        read_v(vf0, P, 0);
         __builtin_amdgcn_sched_barrier(0);
-        acc_t s_next;
-        zero(s_next);
-        scores(kf, s_next, 0, 3);
-        if (row_max(s_cur)) rescale_o();
-        scores(kf, s_next, 3, AT_KSTEPS);
+        read_k(kf, 1 - P, 4, AT_KSTEPS);
+        zero(s_out);
+        scores(kf, s_out, 0, 3);
+        if (row_max(s_in)) rescale_o();
+        scores(kf, s_out, 3, AT_KSTEPS);
         float l_blk = 0.f;
-        const u32x4_t pf0 = probs(s_cur, 0, l_blk);
-        read_v(vf1, kb & 1, 1);
+        const u32x4_t pf0 = probs(s_in, 0, l_blk);
+        read_v(vf1, P, 1);
         pv(vf0, pf0);
-        const u32x4_t pf1 = probs(s_cur, 1, l_blk);
+        const u32x4_t pf1 = probs(s_in, 1, l_blk);
         pv(vf1, pf1);
         finish_row_sum(l_blk);
-        s_cur = s_next;
         publish();
+    };
+    int kb = 0;
+    {
+        acc_t s_odd;  // the scores ping-pong between two register sets instead of being copied
+        for (; kb + 1 < n_fast; kb += 2) {
+            fast_block(kb, 0, s_cur, s_odd);
+            fast_block(kb + 1, 1, s_odd, s_cur);
+        }
     }
     for (; kb < n_blocks; kb++) {
         next_loads(kb);
