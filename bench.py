@@ -205,6 +205,10 @@ def time_case(ctx, case, steps, warmup, graph=False):
     # the K timed launches are issued back to back from C (hodu_rocm_debug_time_product) so that a
     # 3 us GEMV is not hidden behind the interpreter's per-call cost; HIP events on the same stream
     ms = ctx.time_product(case.op, case.name, a, ws, out, md, steps, graph=graph, steps=fused_steps)
+    # spread: ten more batches of the same launches (outside the K timed steps), each timed the same way
+    batch = steps
+    spread = sorted(ctx.time_product(case.op, case.name, a, ws, out, md, batch, graph=graph, steps=fused_steps) * 1e3 / batch
+                    for _ in range(10))
     for buf in [a, out] + ws + ([bias] if bias else []):
         buf.free()
     per_launch_s = ms / 1e3 / steps
@@ -218,7 +222,9 @@ def time_case(ctx, case, steps, warmup, graph=False):
     roof["traffic"] = MEASURED_TRAFFIC.get(f"{kernel}@{case.key}")
     roof["kernel"] = kernel
     return {"config": case.key, "label": case.label, "kernel": kernel, "us_per_launch": per_launch_s * 1e6,
-            "tflops": tflops, "algorithmic_gbs": gbs, "weight_buffers_rotated": copies, "roofline": roof}
+            "tflops": tflops, "algorithmic_gbs": gbs, "weight_buffers_rotated": copies, "roofline": roof,
+            "us_batches": {"launches_per_batch": batch, "p10": spread[1], "median": 0.5 * (spread[4] + spread[5]),
+                           "p90": spread[8]}}
 
 
 def attention_probe(ctx, steps):
@@ -266,6 +272,37 @@ def attention_probe(ctx, steps):
     res["fused_one_kernel"]["tflops_useful"] = flops / 2 / res["fused_one_kernel"]["us"] / 1e6
     return {"config": "attention", "shape": f"bf16 q,k,v [{heads},{s_len},{d}], causal", "us_three_launches": total,
             "us_fused": res["fused_one_kernel"]["us"], "legs": res}
+
+
+def host_buffers_probe(ctx, reps=5):
+    """config 2 with the operands starting and the result ending in host memory (pageable numpy arrays through
+    hodu_rocm_memcpy_h2d / _d2h, buffers allocated beforehand): what a caller pays who hands host buffers over per
+    product instead of keeping tensors on the device.  Never the headline value."""
+    import time
+    case = build_cases(["c2"])[0]
+    md, obytes = out_bytes(case)
+    a_host, b_host = np.ascontiguousarray(case.make_a()), np.ascontiguousarray(case.make_b())
+    a, b, out = ctx.alloc(a_host.nbytes), ctx.alloc(b_host.nbytes), ctx.alloc(obytes)
+    res = np.empty(obytes // 2, dtype=np.uint16)
+
+    def once():
+        ctx._check(ctx.lib.hodu_rocm_memcpy_h2d(ctx.handle, a.ptr, a_host.ctypes.data, a_host.nbytes))
+        ctx._check(ctx.lib.hodu_rocm_memcpy_h2d(ctx.handle, b.ptr, b_host.ctypes.data, b_host.nbytes))
+        ctx.product(case.op, case.name, a, b, out, md)
+        ctx._check(ctx.lib.hodu_rocm_memcpy_d2h(ctx.handle, res.ctypes.data, out.ptr, res.nbytes))
+
+    once()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        once()
+    ctx.sync()
+    s_per = (time.perf_counter() - t0) / reps
+    for buf in (a, b, out):
+        buf.free()
+    moved = a_host.nbytes + b_host.nbytes + res.nbytes
+    return {"config": "c2_host_buffers", "ms_per_product": s_per * 1e3, "tflops": case.flops / s_per / 1e12,
+            "bytes_over_pcie": moved, "gbs_over_pcie": moved / s_per / 1e9, "host_memory": "pageable"}
 
 
 def read_floor_probe(ctx):
@@ -395,6 +432,10 @@ def main():
         return
     if args.only == "attention":
         print(json.dumps(attention_probe(ctx, args.steps)))
+        ctx.close()
+        return
+    if args.only == "pcie":
+        print(json.dumps(host_buffers_probe(ctx)))
         ctx.close()
         return
     if args.only == "clock":
