@@ -405,8 +405,8 @@ def main():
     ap.add_argument("--force-splitk", type=int, default=-1, help="testing hook: pin the number of K ranges")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU; every GPU box here has one GPU and no collective or sharded "
-              "path exists in this round (the design for sharding is in DESIGN.md). Re-run with --gpus 1.",
+        print("bench.py: this build measures one GPU: it has no collective or sharded path, and `value` is the one "
+              "GPU's throughput. Re-run with --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
 

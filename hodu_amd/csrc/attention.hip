@@ -498,14 +498,9 @@ int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k
     a.q_blocks = (int)((g.sq + AT_BQ - 1) / AT_BQ);
     const long blocks = g.batches * a.q_blocks;
     if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
-    static bool configured = false;  // benign race: the attribute calls are idempotent
-    if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_BF16>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, AT_LDS));
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_F16>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, AT_LDS));
-        configured = true;
-    }
+    const void *kernel = dtype == HODU_BF16 ? reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_BF16>)
+                                            : reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_F16>);
+    if (int rc = ensure_dynamic_lds(ctx, kernel, AT_LDS)) return rc;
     if (dtype == HODU_BF16) {
         ctx->last_kernel = "attention_fwd_bf16";
         hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_BF16>, dim3((unsigned)blocks), dim3(AT_NT), AT_LDS, ctx->stream,

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <mutex>
+#include <unordered_set>
 
 #include <cstddef>
 #include <cstdint>
@@ -34,6 +35,9 @@ struct hodu_rocm_ctx {
     int force_tile = -1;    // testing hook: pins the MFMA tile size
     int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
     char kernel_name[96] = {0};  // storage for a composed last_kernel name
+    // kernels whose dynamic-LDS limit has been raised on THIS context's device (the attribute belongs to a
+    // function on a device; a second context on another device has to set it again)
+    std::unordered_set<const void *> lds_configured;
     // every entry point that launches kernels holds this for the call: the workspace, the arrival counters, the
     // testing hooks and last_kernel belong to the context, and launches of one context go to one stream anyway
     std::recursive_mutex mu;
@@ -55,6 +59,14 @@ int fail(int code, const char *fmt, ...);
             return ::hodu::fail(_e == hipErrorOutOfMemory ? HODU_ROCM_OOM : HODU_ROCM_HIP_ERROR, \
                                 "%s: %s", #expr, hipGetErrorString(_e));                       \
     } while (0)
+
+// raises a kernel's dynamic-LDS limit once per context (called with ctx->mu held, like every launch)
+inline int ensure_dynamic_lds(hodu_rocm_ctx *ctx, const void *kernel, int bytes) {
+    if (ctx->lds_configured.count(kernel)) return HODU_ROCM_OK;
+    HODU_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    ctx->lds_configured.insert(kernel);
+    return HODU_ROCM_OK;
+}
 
 // grows ctx->workspace to at least `bytes`
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes);

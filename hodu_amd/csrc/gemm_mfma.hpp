@@ -698,15 +698,8 @@ inline int pick_mode(const void *base, long off, long row_stride, long k_stride,
 }
 
 template <class Cfg> int launch_config(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
-    static bool configured = false;  // benign race: the attribute call is idempotent
     auto kernel = g.epi.n != 0 ? mfma_product_kernel<Cfg, true> : mfma_product_kernel<Cfg, false>;
-    if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_product_kernel<Cfg, true>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_product_kernel<Cfg, false>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
-        configured = true;
-    }
+    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     const long total = g.batches * tiles_m * tiles_n;
     if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);

@@ -246,13 +246,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
 
 template <class Cfg>
 int launch_pipe_f8(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g, int splits) {
-    static bool configured = false;  // benign race: the attribute call is idempotent
     auto kernel = mfma_pipe_f8_kernel<Cfg>;
-    if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     Cfg::LDS_BYTES));
-        configured = true;
-    }
+    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     const long total = g.batches * tiles_m * tiles_n;
     if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);

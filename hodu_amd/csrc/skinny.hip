@@ -381,11 +381,8 @@ int launch_splitk(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, con
     if (rc == HODU_ROCM_OK) rc = ensure_arrival(ctx);
     if (rc != HODU_ROCM_OK) return rc;
     auto kernel = skinny_splitk_kernel<CK, SKB, OUT>;
-    static bool configured = false;  // benign race: the attribute call is idempotent
-    if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SK_XBYTES + 16 * 16));
-        configured = true;
-    }
+    rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), SK_XBYTES + 16 * 16);
+    if (rc != HODU_ROCM_OK) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(n_blocks * slices)), dim3(512), lds, ctx->stream, (const char *)x, (const char *)w,
                        (typename Out<OUT>::T *)y, (acc_t *)ctx->workspace.ptr, ctx->arrival, g, n_blocks, slices, k_per_slice,
                        x_pitch);
@@ -407,12 +404,7 @@ int launch_shape(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, cons
     const int x_pitch = (g.M * pitch <= X_LDS_LIMIT) ? (int)pitch : 0;
     const size_t lds = x_pitch > 0 ? (size_t)g.M * x_pitch : 0;
     auto kernel = skinny_kdense_kernel<CK, SKB, OUT, NBLK, KW>;
-    static bool configured = false;  // benign race: the attribute call is idempotent
-    if (!configured) {
-        HODU_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     X_LDS_LIMIT));
-        configured = true;
-    }
+    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), X_LDS_LIMIT)) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NBLK * KW * 64), lds, ctx->stream, (const char *)x,
                        (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave, x_pitch);
     HODU_HIP(hipGetLastError());
