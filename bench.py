@@ -274,6 +274,55 @@ def attention_probe(ctx, steps):
             "us_fused": res["fused_one_kernel"]["us"], "legs": res}
 
 
+def cast_cases():
+    """the to_dtype / contiguous passes the path takes when a cast is NOT deferred into the product, at the sizes of
+    the BASELINE configurations: (key, label, src, dst, view, elements)"""
+    import helpers as H
+    V = H.View
+    return [
+        ("cast_f8e4m3_bf16_c3w", "to_dtype f8e4m3 -> bf16, config 3's weight [4096,4096]", "f8e4m3", "bf16", V([4096 * 4096])),
+        ("cast_f8e4m3_bf16_c5w", "to_dtype f8e4m3 -> bf16, config 5's weight [4096,14336]", "f8e4m3", "bf16", V([4096 * 14336])),
+        ("cast_i8_i32_c4", "to_dtype i8 -> i32, one operand of config 4 [2048,2048]", "i8", "i32", V([2048 * 2048])),
+        ("contiguous_bf16_c2_bt", "contiguous of config 2's transposed operand [16,1024,1024]^T", "bf16", "bf16",
+         V([16, 1024, 1024]).t()),
+        ("contiguous_bf16_c5_wdown", "contiguous of config 5's W_down view [4096,14336]^T", "bf16", "bf16",
+         V([4096, 14336]).t()),
+    ]
+
+
+def time_cast_case(ctx, key, label, src, dst, view, steps, warmup):
+    """HBM-bound: algorithmic bytes = elements x (source + destination element size); inputs and outputs rotate
+    through enough buffer pairs to exceed three times the Infinity Cache"""
+    import helpers as H
+    from hodu_amd import ffi
+    n = int(np.prod(view.shape))
+    in_bytes, out_bytes_ = view.span() * ffi.DTYPE_SIZE[src], n * ffi.DTYPE_SIZE[dst]
+    pairs = max(2, int(3 * INFINITY_CACHE_BYTES // (in_bytes + out_bytes_)) + 1)
+    host = np.random.default_rng(77).integers(0, 120, size=in_bytes, dtype=np.uint8)  # finite in every dtype used here
+    ins = [ctx.upload(host)]
+    for _ in range(1, pairs):
+        extra = ctx.alloc(in_bytes)
+        ctx.lib.hodu_rocm_memcpy_d2d(ctx.handle, extra.ptr, ins[0].ptr, in_bytes)
+        ins.append(extra)
+    outs = [ctx.alloc(out_bytes_) for _ in range(pairs)]
+    md = H.cast_md(view)
+    ctx.time_cast(src, dst, ins, outs, md, max(warmup, 1))
+    kernel = ctx.last_kernel()
+    ms = ctx.time_cast(src, dst, ins, outs, md, steps)
+    spread = sorted(ctx.time_cast(src, dst, ins, outs, md, steps) * 1e3 / steps for _ in range(10))
+    for b in ins + outs:
+        b.free()
+    s_per = ms / 1e3 / steps
+    alg = n * (ffi.DTYPE_SIZE[src] + ffi.DTYPE_SIZE[dst])
+    gbs = alg / s_per / 1e9
+    return {"config": key, "label": label, "kernel": kernel, "us_per_launch": s_per * 1e6, "tflops": 0.0,
+            "algorithmic_gbs": gbs, "weight_buffers_rotated": pairs,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": None, "kernel": kernel},
+            "us_batches": {"launches_per_batch": steps, "p10": spread[1], "median": 0.5 * (spread[4] + spread[5]),
+                           "p90": spread[8]}}
+
+
 def host_buffers_probe(ctx, reps=5):
     """config 2 with the operands starting and the result ending in host memory (pageable numpy arrays through
     hodu_rocm_memcpy_h2d / _d2h, buffers allocated beforehand): what a caller pays who hands host buffers over per
@@ -397,7 +446,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,fused,bwd")
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,fused,bwd,casts")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
@@ -442,6 +491,10 @@ def main():
         print(json.dumps({"config": "clock", "register_only_mfma": mfma_clock_probe(ctx), "streaming_read": read_floor_probe(ctx)}))
         ctx.close()
         return
+    if args.only in [c[0] for c in cast_cases()]:
+        print(json.dumps(time_cast_case(ctx, *next(c for c in cast_cases() if c[0] == args.only), args.steps, args.warmup)))
+        ctx.close()
+        return
     if args.only:
         case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "fused", "bwd"}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
@@ -456,6 +509,11 @@ def main():
               f"{results[-1]['algorithmic_gbs']:.0f} GB/s  [{results[-1]['kernel']}] "
               f"{100 * results[-1]['roofline']['frac']:.1f}% of {results[-1]['roofline']['bound']} peak",
               file=sys.stderr, flush=True)
+    if "casts" in which:
+        for cc in cast_cases():
+            results.append(time_cast_case(ctx, *cc, args.steps, args.warmup))
+            print(f"# {results[-1]['label']}: {results[-1]['us_per_launch']:.1f} us  {results[-1]['algorithmic_gbs']:.0f} GB/s  "
+                  f"[{results[-1]['kernel']}] {100 * results[-1]['roofline']['frac']:.1f}% of hbm peak", file=sys.stderr, flush=True)
     head = next(r for r in results if r["config"] == "c2")
     # the headline is re-timed with exactly the requested step count
     case2 = [c for c in build_cases({"c2"})][0]

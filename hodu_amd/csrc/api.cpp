@@ -307,6 +307,38 @@ int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *o
     return launch_cast(ctx, src, dst, in, out, s);
 }
 
+int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *const *in_list, void *const *out_list,
+                              size_t n_buffers, const size_t *md, size_t len, int iters, float *elapsed_ms) {
+    clear_error();
+    if (!ctx || !in_list || !out_list || n_buffers == 0 || !elapsed_ms || iters < 1)
+        return fail(HODU_ROCM_INVALID_ARG, "time_cast: bad argument");
+    if (dtype_size(src) == 0 || dtype_size(dst) == 0)
+        return fail(HODU_ROCM_UNSUPPORTED, "time_cast: unknown dtype id (%d -> %d)", src, dst);
+    for (size_t i = 0; i < n_buffers; i++)
+        if (!in_list[i] || !out_list[i] || in_list[i] == out_list[i]) return fail(HODU_ROCM_INVALID_ARG, "time_cast: bad buffer %zu", i);
+    Strided s;
+    int rc = parse_cast_metadata(md, len, &s);
+    if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    HODU_HIP(hipSetDevice(ctx->device));
+    hipEvent_t t0, t1;
+    HODU_HIP(hipEventCreate(&t0));
+    HODU_HIP(hipEventCreate(&t1));
+    HODU_HIP(hipEventRecord(t0, ctx->stream));
+    for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++) {
+        const size_t j = (size_t)i % n_buffers;
+        rc = src == dst ? launch_gather(ctx, src, in_list[j], out_list[j], s) : launch_cast(ctx, src, dst, in_list[j], out_list[j], s);
+    }
+    hipError_t e = hipEventRecord(t1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_cast: %s", hipGetErrorString(e));
+    return HODU_ROCM_OK;
+}
+
 int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "sum: context is null");

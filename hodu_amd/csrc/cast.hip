@@ -13,6 +13,8 @@
 // One deliberate difference: f8e4m3 is DECODED as OCP E4M3FN (exponent 15 is finite up to 448),
 // which is what hodu's Rust F8E4M3 type and the gfx950 matrix cores implement; the reference's C
 // decoder (t_f8e4m3.h:34-38) reads those 14 codes as inf/NaN.
+#include <utility>
+
 #include "common.hpp"
 #include "device_types.hpp"
 #include "epilogue.hpp"  // ref_f32_to_f16
@@ -201,6 +203,120 @@ __global__ __launch_bounds__(256) void cast_strided_kernel(const typename Src<S>
     }
 }
 
+// strided source whose unit stride sits on a dim J other than the last one (a transposed view): 64 x 64 tiles over
+// (J, last dim L) go through LDS, read along J and written along L, so that both sides move whole cache lines.
+// What contiguous() of a transposed operand costs in the reference is this gather (ops_memory.c:78-83, one thread).
+struct DevTranspose {
+    int n_outer;                                       // the remaining dims, walked by the tile index
+    long outer_shape[16], outer_in[16], outer_out[16];
+    long n_j, n_l, in_l, out_j;                        // extents; source stride of L, destination stride of J
+    long tiles_j, tiles_l;
+};
+constexpr int TT = 64;
+
+template <int S, int D>
+__global__ __launch_bounds__(256) void cast_transpose_kernel(const typename Src<S>::T *__restrict__ in,
+                                                            typename Dst<D>::T *__restrict__ out, DevTranspose t) {
+    typedef typename Dst<D>::T TD;
+    // a row of 64 elements plus padding of one 4-byte bank (at least one element): the column reads of the second
+    // phase then fall into different banks
+    constexpr int PAD = sizeof(TD) >= 4 ? 1 : 4 / (int)sizeof(TD);
+    __shared__ TD tile[TT][TT + PAD];
+    long b = blockIdx.x;
+    const long tl = b % t.tiles_l; b /= t.tiles_l;
+    const long tj = b % t.tiles_j; b /= t.tiles_j;
+    long in_off = 0, out_off = 0;
+    for (int d = t.n_outer - 1; d >= 0; d--) {
+        const long i = b % t.outer_shape[d];
+        b /= t.outer_shape[d];
+        in_off += i * t.outer_in[d];
+        out_off += i * t.outer_out[d];
+    }
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const long j0 = tj * TT, l0 = tl * TT;
+    {   // lanes along J (source stride 1)
+        const long j = j0 + tx;
+        typename Src<S>::T x[TT / 4];  // all 16 loads in flight before the first conversion
+#pragma unroll
+        for (int i = 0; i < TT / 4; i++) {
+            const long l = l0 + ty + 4 * i;
+            if (j < t.n_j && l < t.n_l) x[i] = in[in_off + j + l * t.in_l];
+        }
+#pragma unroll
+        for (int i = 0; i < TT / 4; i++) {
+            const long l = l0 + ty + 4 * i;
+            if (j < t.n_j && l < t.n_l) tile[ty + 4 * i][tx] = Convert<S, D>::run(x[i]);
+        }
+    }
+    __syncthreads();
+    {   // lanes along L (destination stride 1)
+        const long l = l0 + tx;
+#pragma unroll
+        for (int r = ty; r < TT; r += 4) {
+            const long j = j0 + r;
+            if (j < t.n_j && l < t.n_l) out[out_off + j * t.out_j + l] = tile[tx][r];
+        }
+    }
+}
+
+// the same with V elements per lane on both sides (8 bytes of the wider type): a wavefront reads 64 * V elements of
+// one source row and writes 64 / V lanes * V elements of each destination row; tiles are (64 * V) x 64.  The launcher
+// checks that every address involved is a multiple of V elements.
+template <int S, int D, int V>
+__global__ __launch_bounds__(256) void cast_transpose_vec_kernel(const typename Src<S>::T *__restrict__ in,
+                                                                typename Dst<D>::T *__restrict__ out, DevTranspose t) {
+    typedef typename Src<S>::T TS;
+    typedef typename Dst<D>::T TD;
+    constexpr int TJ = TT * V;
+    constexpr int PAD = sizeof(TD) >= 4 ? 1 : 4 / (int)sizeof(TD);  // row pitch = an odd number of 4-byte banks
+    __shared__ TD tile[TT][TJ + PAD];
+    long b = blockIdx.x;
+    const long tl = b % t.tiles_l; b /= t.tiles_l;
+    const long tj = b % t.tiles_j; b /= t.tiles_j;
+    long in_off = 0, out_off = 0;
+    for (int d = t.n_outer - 1; d >= 0; d--) {
+        const long i = b % t.outer_shape[d];
+        b /= t.outer_shape[d];
+        in_off += i * t.outer_in[d];
+        out_off += i * t.outer_out[d];
+    }
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const long j0 = tj * TJ, l0 = tl * TT;
+    {
+        const long j = j0 + tx * V;
+        Pack<TS, V> x[TT / 4];  // all loads in flight before the first conversion
+#pragma unroll
+        for (int i = 0; i < TT / 4; i++) {
+            const long l = l0 + ty + 4 * i;
+            if (j < t.n_j && l < t.n_l) x[i] = *reinterpret_cast<const Pack<TS, V> *>(in + in_off + j + l * t.in_l);
+        }
+#pragma unroll
+        for (int i = 0; i < TT / 4; i++) {
+            const long l = l0 + ty + 4 * i;
+            if (j < t.n_j && l < t.n_l) {
+#pragma unroll
+                for (int v = 0; v < V; v++) tile[ty + 4 * i][tx * V + v] = Convert<S, D>::run(x[i].v[v]);
+            }
+        }
+    }
+    __syncthreads();
+    {
+        constexpr int LPR = TT / V;  // lanes per destination row
+        const int lx = threadIdx.x % LPR, jy = threadIdx.x / LPR;
+        const long l = l0 + lx * V;
+#pragma unroll 4
+        for (int r = jy; r < TJ; r += 256 / LPR) {
+            const long j = j0 + r;
+            if (j < t.n_j && l < t.n_l) {
+                Pack<TD, V> y;
+#pragma unroll
+                for (int v = 0; v < V; v++) y.v[v] = tile[lx * V + v][r];
+                *reinterpret_cast<Pack<TD, V> *>(out + out_off + j * t.out_j + l) = y;
+            }
+        }
+    }
+}
+
 inline unsigned grid_for(long work_items, const hodu_rocm_ctx *ctx) {
     long blocks = (work_items + 255) / 256;
     const long cap = (long)ctx->props.multiProcessorCount * 16;  // grid-stride beyond this
@@ -217,6 +333,7 @@ int run_cast(hodu_rocm_ctx *ctx, const void *in_v, void *out_v, const Strided &s
     TD *out = (TD *)out_v;
     if (s.contiguous) {
         const bool aligned = ((uintptr_t)in % (sizeof(TS) * VEC) == 0) && ((uintptr_t)out % (sizeof(TD) * VEC) == 0);
+        ctx->last_kernel = aligned ? "cast_dense_vec" : "cast_dense";
         if (aligned) {
             hipLaunchKernelGGL((cast_dense_kernel<S, D>), dim3(grid_for((s.n + VEC - 1) / VEC, ctx)), dim3(256), 0,
                                ctx->stream, in, out, s.n);
@@ -240,6 +357,61 @@ int run_cast(hodu_rocm_ctx *ctx, const void *in_v, void *out_v, const Strided &s
             }
         }
         d.nd = nd;
+        // a transposed view: the last dim is strided and some other dim has the unit stride
+        int dj = -1;
+        if (nd >= 2 && d.strides[nd - 1] != 1 && d.shape[nd - 1] >= 16)
+            for (int i = 0; i < nd - 1; i++)
+                if (d.strides[i] == 1 && d.shape[i] >= 16) dj = i;
+        if (dj >= 0) {
+            DevTranspose t{};
+            long out_stride = 1, outer = 1;
+            for (int i = nd - 1; i >= 0; i--) {  // destination strides: row-major over the merged dims
+                if (i == dj) {
+                    t.out_j = out_stride;
+                } else if (i != nd - 1) {
+                    // collected innermost first; the kernel walks them in the same order
+                    t.outer_shape[t.n_outer] = d.shape[i];
+                    t.outer_in[t.n_outer] = d.strides[i];
+                    t.outer_out[t.n_outer] = out_stride;
+                    t.n_outer++;
+                    outer *= d.shape[i];
+                }
+                out_stride *= d.shape[i];
+            }
+            // the kernel peels outer dims from index n_outer - 1 down as the fastest-varying first: reverse so that
+            // the innermost outer dim varies fastest
+            for (int a = 0, b = t.n_outer - 1; a < b; a++, b--) {
+                std::swap(t.outer_shape[a], t.outer_shape[b]);
+                std::swap(t.outer_in[a], t.outer_in[b]);
+                std::swap(t.outer_out[a], t.outer_out[b]);
+            }
+            t.n_j = d.shape[dj];
+            t.n_l = d.shape[nd - 1];
+            t.in_l = d.strides[nd - 1];
+            t.tiles_l = (t.n_l + TT - 1) / TT;
+            // V elements per lane: 8 bytes of the wider type, if every address stays a multiple of V elements
+            constexpr int V = 8 / (int)(sizeof(TS) > sizeof(TD) ? sizeof(TS) : sizeof(TD));
+            bool vec = V >= 2 && t.n_j % V == 0 && t.n_l % V == 0 && t.in_l % V == 0 &&
+                       (uintptr_t)in % (V * sizeof(TS)) == 0 && (uintptr_t)out % (V * sizeof(TD)) == 0;
+            for (int i = 0; i < t.n_outer; i++) vec = vec && t.outer_in[i] % V == 0;
+            t.tiles_j = (t.n_j + (vec ? TT * V : TT) - 1) / (vec ? TT * V : TT);
+            const long blocks = outer * t.tiles_j * t.tiles_l;
+            if (blocks <= 0x7FFFFFFFL) {
+                if constexpr (V >= 2) {
+                    if (vec) {
+                        ctx->last_kernel = "cast_transpose_vec";
+                        hipLaunchKernelGGL((cast_transpose_vec_kernel<S, D, V>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, out, t);
+                        HODU_HIP(hipGetLastError());
+                        return HODU_ROCM_OK;
+                    }
+                }
+                ctx->last_kernel = "cast_transpose";
+                hipLaunchKernelGGL((cast_transpose_kernel<S, D>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, out, t);
+                HODU_HIP(hipGetLastError());
+                return HODU_ROCM_OK;
+            }
+        }
+        ctx->last_kernel = "cast_strided";
         hipLaunchKernelGGL((cast_strided_kernel<S, D>), dim3(grid_for(s.n, ctx)), dim3(256), 0, ctx->stream, in, out,
                            s.n, d);
     }

@@ -114,6 +114,8 @@ def load() -> ctypes.CDLL:
             getattr(lib, f"hodu_rocm_{op}_{dt}_ex").argtypes = [vp, vp, vp, vp, szp, sz, ctypes.POINTER(EpilogueStep), sz]
     lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz,
                                                     ctypes.POINTER(EpilogueStep), sz, ci, ctypes.POINTER(ctypes.c_float)]
+    lib.hodu_rocm_debug_time_cast.argtypes = [vp, ci, ci, ctypes.POINTER(vp), ctypes.POINTER(vp), sz, szp, sz, ci,
+                                              ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, ctypes.POINTER(ctypes.c_float),
                                                ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.hodu_rocm_debug_read_floor.argtypes = [vp, ctypes.POINTER(vp), sz, sz, ci, ctypes.POINTER(ctypes.c_float),
@@ -353,6 +355,21 @@ class Context:
         fn = self.lib.hodu_rocm_debug_time_product_graph if graph else self.lib.hodu_rocm_debug_time_product
         self._check(fn(self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr,
                        n, int(iters), ctypes.byref(ms)))
+        return float(ms.value)
+
+    def time_cast(self, src: str, dst: str, ins, outs, md, iters: int) -> float:
+        """back-to-back cast (src != dst) or contiguous (src == dst) launches issued from C over the buffer pairs in
+        turn, HIP-event timed on the context's stream; total ms"""
+        if len(ins) != len(outs) or not ins:
+            raise HoduRocmError(INVALID_ARG, "time_cast: need as many outputs as inputs, at least one")
+        for x, out in zip(ins, outs):
+            self._check_strided(f"time_cast_{src}_to_{dst}", DTYPE_SIZE[src], DTYPE_SIZE[dst], x, out, md)
+        arr, n = _md_array(md)
+        pin = (ctypes.c_void_p * len(ins))(*[b.ptr for b in ins])
+        pout = (ctypes.c_void_p * len(outs))(*[b.ptr for b in outs])
+        ms = ctypes.c_float()
+        self._check(self.lib.hodu_rocm_debug_time_cast(self.handle, DTYPE_ID[src], DTYPE_ID[dst], pin, pout, len(ins), arr, n,
+                                                       int(iters), ctypes.byref(ms)))
         return float(ms.value)
 
     def mfma_clock(self, kind: int, operands: DeviceBuffer, iters: int = 20000) -> dict:

@@ -215,6 +215,12 @@ HODU_ROCM_DECL_PRODUCT_EX(i32)
 HODU_ROCM_DECL_PRODUCT_EX(i64)
 HODU_ROCM_DECL_PRODUCT_EX(bf16_f8e4m3w) /* vector / scalar in bf16 */
 HODU_ROCM_DECL_PRODUCT_EX(i32_i8i8)     /* vector / scalar in i32 */
+/* measurement hook: `iters` back-to-back launches of hodu_rocm_cast (src != dst) or hodu_rocm_contiguous (src == dst)
+ * on one metadata array, walking through n_buffers input / output pairs (so that a stream larger than the last-level
+ * cache comes from memory), HIP-event timed on the context's stream. */
+int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src_dtype, int dst_dtype, const void *const *in_list,
+                              void *const *out_list, size_t n_buffers, const size_t *metadata, size_t metadata_len,
+                              int iters, float *elapsed_ms);
 /* measurement hook: hodu_rocm_debug_time_product with fused steps */
 int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
                                     const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,

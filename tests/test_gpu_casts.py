@@ -125,6 +125,35 @@ def test_contiguous_all_sizes(ctx):
             assert same(gpu_cast(ctx, "contiguous", dt, x, H.cast_md(v)), oracle.contiguous(dt, x, H.cast_md(v)), dt)
 
 
+def test_transposed_views_go_through_the_tiled_kernel(ctx):
+    """a view whose unit stride is not on the last dim (a transpose, a permutation) is gathered in 64 x 64 tiles
+    through LDS: ragged tiles, several outer dims (one of them broadcast), an offset, casts that change the element size"""
+    views = [V([130, 70]).t(), V([3, 65, 200], offset=5).t(1, 2), V([33, 4, 129]).t(0, 2),
+             V([100, 48]).t().broadcast_to([3, 48, 100]), V([2, 3, 64, 64]).t(2, 3), V([17, 300]).t()]
+    for n, v in enumerate(views):
+        for dt in ("u8", "bf16", "f32", "i64"):
+            x = H.random_storage(dt, v.span(), 40 + n)
+            assert same(gpu_cast(ctx, "contiguous", dt, x, H.cast_md(v)), oracle.contiguous(dt, x, H.cast_md(v)), dt), (n, dt)
+            assert ctx.last_kernel().startswith("cast_transpose"), (n, dt, ctx.last_kernel())
+        for src, dst in (("f8e4m3", "bf16"), ("i8", "i32"), ("f32", "bf16"), ("bf16", "f32"), ("f64", "i16")):
+            x = H.random_storage(src, v.span(), 60 + n, 20.0)
+            md = H.cast_md(v)
+            assert same(gpu_cast(ctx, src, dst, x, md), oracle.cast(src, dst, x, md, decode=oracle.F8_OCP), dst), (n, src, dst)
+            assert ctx.last_kernel().startswith("cast_transpose")
+    # 8 bytes per lane where every address stays a multiple of the vector, one element per lane otherwise
+    for v, dt, name in ((V([2, 3, 64, 64]).t(2, 3), "bf16", "cast_transpose_vec"), (V([256, 512]).t(), "u8", "cast_transpose_vec"),
+                        (V([130, 70]).t(), "bf16", "cast_transpose"), (V([64, 64], offset=1).t(), "f32", "cast_transpose"),
+                        (V([64, 64]).t(), "i64", "cast_transpose")):
+        x = H.random_storage(dt, v.span(), 3)
+        assert same(gpu_cast(ctx, "contiguous", dt, x, H.cast_md(v)), oracle.contiguous(dt, x, H.cast_md(v)), dt)
+        assert ctx.last_kernel() == name, (dt, ctx.last_kernel(), name)
+    # too thin for tiles, or the last dim already dense: the flat-index kernel
+    for v in (V([8, 300]).t(), V([300, 8]).t(), V([40, 50]).slice(1, 0, 50, 2)):
+        x = H.random_storage("bf16", v.span(), 9)
+        assert same(gpu_cast(ctx, "contiguous", "bf16", x, H.cast_md(v)), oracle.contiguous("bf16", x, H.cast_md(v)), "bf16")
+        assert ctx.last_kernel() == "cast_strided", ctx.last_kernel()
+
+
 def test_config_sized_casts(ctx):
     """C3/C4-sized casts (16.8 M f8e4m3 -> bf16, 4.2 M i8 -> i32) against the oracle"""
     w = H.rng(301).integers(0, 256, 4096 * 4096, dtype=np.uint8)
