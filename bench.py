@@ -323,6 +323,46 @@ def time_cast_case(ctx, key, label, src, dst, view, steps, warmup):
                            "p90": spread[8]}}
 
 
+def sum_cases():
+    """sum_to_shape of the backward pass at the sizes of configuration 5: (key, label, view, reduced dims)"""
+    import helpers as H
+    V = H.View
+    return [
+        ("sum_bias_grad_c5_up", "sum_to_shape: bias gradient of C5 up, bf16 [8,512,14336] -> [14336]", V([8, 512, 14336]), [0, 1]),
+        ("sum_bias_grad_c5_down", "sum_to_shape: bias gradient of C5 down, bf16 [8,512,4096] -> [4096]", V([8, 512, 4096]), [0, 1]),
+        ("sum_rows_c5", "row sums, bf16 [4096,14336] -> [4096]", V([4096, 14336]), [1]),
+    ]
+
+
+def time_sum_case(ctx, key, label, view, dims, steps, warmup):
+    """HBM-bound: algorithmic bytes = (input + output elements) x element size; buffers rotate past the Infinity Cache"""
+    import helpers as H
+    n = int(np.prod(view.shape))
+    n_out = n // int(np.prod([view.shape[d] for d in dims]))
+    pairs = max(2, int(3 * INFINITY_CACHE_BYTES // (2 * (n + n_out))) + 1)
+    ins = [ctx.upload(bf16(normal(61, n)))]
+    for _ in range(1, pairs):
+        extra = ctx.alloc(2 * n)
+        ctx.lib.hodu_rocm_memcpy_d2d(ctx.handle, extra.ptr, ins[0].ptr, 2 * n)
+        ins.append(extra)
+    outs = [ctx.alloc(2 * n_out) for _ in range(pairs)]
+    md = H.reduce_md(view, dims, False)
+    ctx.time_sum("bf16", ins, outs, md, max(warmup, 1))
+    kernel = ctx.last_kernel()
+    ms = ctx.time_sum("bf16", ins, outs, md, steps)
+    spread = sorted(ctx.time_sum("bf16", ins, outs, md, steps) * 1e3 / steps for _ in range(10))
+    for b in ins + outs:
+        b.free()
+    s_per = ms / 1e3 / steps
+    gbs = 2 * (n + n_out) / s_per / 1e9
+    return {"config": key, "label": label, "kernel": kernel, "us_per_launch": s_per * 1e6, "tflops": 0.0,
+            "algorithmic_gbs": gbs, "weight_buffers_rotated": pairs,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": None, "kernel": kernel},
+            "us_batches": {"launches_per_batch": steps, "p10": spread[1], "median": 0.5 * (spread[4] + spread[5]),
+                           "p90": spread[8]}}
+
+
 def host_buffers_probe(ctx, reps=5):
     """config 2 with the operands starting and the result ending in host memory (pageable numpy arrays through
     hodu_rocm_memcpy_h2d / _d2h, buffers allocated beforehand): what a caller pays who hands host buffers over per
@@ -491,6 +531,10 @@ def main():
         print(json.dumps({"config": "clock", "register_only_mfma": mfma_clock_probe(ctx), "streaming_read": read_floor_probe(ctx)}))
         ctx.close()
         return
+    if args.only in [c[0] for c in sum_cases()]:
+        print(json.dumps(time_sum_case(ctx, *next(c for c in sum_cases() if c[0] == args.only), args.steps, args.warmup)))
+        ctx.close()
+        return
     if args.only in [c[0] for c in cast_cases()]:
         print(json.dumps(time_cast_case(ctx, *next(c for c in cast_cases() if c[0] == args.only), args.steps, args.warmup)))
         ctx.close()
@@ -512,6 +556,11 @@ def main():
     if "casts" in which:
         for cc in cast_cases():
             results.append(time_cast_case(ctx, *cc, args.steps, args.warmup))
+            print(f"# {results[-1]['label']}: {results[-1]['us_per_launch']:.1f} us  {results[-1]['algorithmic_gbs']:.0f} GB/s  "
+                  f"[{results[-1]['kernel']}] {100 * results[-1]['roofline']['frac']:.1f}% of hbm peak", file=sys.stderr, flush=True)
+    if "bwd" in which:
+        for sc in sum_cases():
+            results.append(time_sum_case(ctx, *sc, args.steps, args.warmup))
             print(f"# {results[-1]['label']}: {results[-1]['us_per_launch']:.1f} us  {results[-1]['algorithmic_gbs']:.0f} GB/s  "
                   f"[{results[-1]['kernel']}] {100 * results[-1]['roofline']['frac']:.1f}% of hbm peak", file=sys.stderr, flush=True)
     head = next(r for r in results if r["config"] == "c2")

@@ -339,6 +339,34 @@ int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *
     return HODU_ROCM_OK;
 }
 
+int hodu_rocm_debug_time_sum(hodu_rocm_ctx *ctx, int dtype, const void *const *in_list, void *const *out_list,
+                             size_t n_buffers, const size_t *md, size_t len, int iters, float *elapsed_ms) {
+    clear_error();
+    if (!ctx || !in_list || !out_list || n_buffers == 0 || !elapsed_ms || iters < 1)
+        return fail(HODU_ROCM_INVALID_ARG, "time_sum: bad argument");
+    if (dtype_size(dtype) == 0 || dtype == HODU_BOOL) return fail(HODU_ROCM_UNSUPPORTED, "time_sum: dtype id %d has no sum kernel", dtype);
+    for (size_t i = 0; i < n_buffers; i++)
+        if (!in_list[i] || !out_list[i] || in_list[i] == out_list[i]) return fail(HODU_ROCM_INVALID_ARG, "time_sum: bad buffer %zu", i);
+    Reduction r;
+    int rc = parse_reduce_metadata(md, len, &r);
+    if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    HODU_HIP(hipSetDevice(ctx->device));
+    hipEvent_t t0, t1;
+    HODU_HIP(hipEventCreate(&t0));
+    HODU_HIP(hipEventCreate(&t1));
+    HODU_HIP(hipEventRecord(t0, ctx->stream));
+    for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++) rc = launch_sum(ctx, dtype, in_list[(size_t)i % n_buffers], out_list[(size_t)i % n_buffers], r);
+    hipError_t e = hipEventRecord(t1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_sum: %s", hipGetErrorString(e));
+    return HODU_ROCM_OK;
+}
+
 int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "sum: context is null");

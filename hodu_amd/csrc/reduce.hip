@@ -6,12 +6,17 @@
 // Arithmetic as for the products: narrow floats and f32 accumulate in f32 and round once on store (the reference
 // re-rounds its bf16 / f16 / f8 accumulator after every add), f64 in f64, integers wrap.
 //
-// Two kernels, chosen by where the unit stride is:
+// Kernels, chosen by where the unit stride is and by how many outputs there are:
 //   * the outputs' last dim is dense (leading dims are summed: the sum_to_shape case): a thread owns V neighbouring
 //     outputs and walks the reduced dims; neighbouring threads read neighbouring addresses, 16 bytes per lane when
 //     alignment allows.  HBM-bound, every input element is read once;
-//   * the innermost reduced dim is dense (a row sum): a wavefront owns an output, its lanes stride over that dim,
-//     and the lane sums meet in a butterfly.
+//   * the same with few outputs and a long reduction (the gradient of a bias: [batch * rows, features] summed to
+//     [features]): one thread per output vector would leave most of the chip idle, so the reduced index space is cut
+//     into chunks, one workgroup per (64 output vectors, chunk), its four wavefronts taking every fourth row; the
+//     chunks' partial sums (in the accumulate type) go through the context's workspace and a second kernel adds
+//     them in chunk order and rounds once;
+//   * the innermost reduced dim is dense (a row sum): a wavefront owns an output, its lanes stride over that dim
+//     (16 bytes per lane when alignment allows), and the lane sums meet in a butterfly.
 #include "common.hpp"
 #include "device_types.hpp"
 #include "elem.hpp"
@@ -84,6 +89,77 @@ __global__ __launch_bounds__(256) void sum_by_output_kernel(const typename E::st
     }
 }
 
+// flattened index over ALL reduced dims -> element offset
+__device__ __forceinline__ long red_offset(const DevReduction &r, long i) {
+    long off = 0;
+    for (int d = r.red_n - 1; d >= 0; d--) {
+        off += (i % r.red_shape[d]) * r.red_stride[d];
+        i /= r.red_shape[d];
+    }
+    return off;
+}
+
+// few outputs, long reduction: workgroup (x, y) sums chunk y of the reduced index space for output vectors
+// 64 x .. 64 x + 63; wavefront w takes indices chunk_begin + w, + 4, ..; partial[y][output] in the accumulate type
+template <class E, int V>
+__global__ __launch_bounds__(256) void sum_chunks_kernel(const typename E::storage *__restrict__ in,
+                                                        typename E::acc *__restrict__ partial, DevReduction r,
+                                                        long per_chunk) {
+    typedef typename E::storage S;
+    typedef typename E::acc A;
+    __shared__ A meet[3][64][V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long o = ((long)blockIdx.x * 64 + lane) * V;
+    const long begin = (long)blockIdx.y * per_chunk;
+    const long end = begin + per_chunk < r.reduce_size ? begin + per_chunk : r.reduce_size;
+    A acc[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) acc[v] = (A)0;
+    if (o < r.n_out) {
+        const S *base = in + r.offset + kept_offset(r, o);
+        for (long i = begin + wave; i < end; i += 4) {
+            const S *p = base + red_offset(r, i);
+            if constexpr (V == 1) {
+                acc[0] += E::load(p[0]);
+            } else {
+                struct alignas(sizeof(S) * V) Vec { S e[V]; };
+                const Vec x = *reinterpret_cast<const Vec *>(p);
+#pragma unroll
+                for (int v = 0; v < V; v++) acc[v] += E::load(x.e[v]);
+            }
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int v = 0; v < V; v++) meet[wave - 1][lane][v] = acc[v];
+    }
+    __syncthreads();
+    if (wave == 0 && o < r.n_out) {
+#pragma unroll
+        for (int v = 0; v < V; v++)
+            partial[(long)blockIdx.y * r.n_out + o + v] = acc[v] + meet[0][lane][v] + meet[1][lane][v] + meet[2][lane][v];
+    }
+}
+
+// out[o] = round(sum over chunks of partial[chunk][o]): a workgroup owns 64 outputs, its four wavefronts take every
+// fourth chunk (several loads in flight each) and meet in LDS; the order of the additions is fixed
+template <class E>
+__global__ __launch_bounds__(256) void sum_finish_kernel(const typename E::acc *__restrict__ partial,
+                                                        typename E::storage *__restrict__ out, long n_out, int chunks) {
+    typedef typename E::acc A;
+    __shared__ A meet[3][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long o = (long)blockIdx.x * 64 + lane;
+    A acc = (A)0;
+    if (o < n_out) {
+#pragma unroll 8
+        for (int c = wave; c < chunks; c += 4) acc += partial[(long)c * n_out + o];
+    }
+    if (wave > 0) meet[wave - 1][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && o < n_out) out[o] = E::store(acc + meet[0][lane] + meet[1][lane] + meet[2][lane]);
+}
+
 template <class A> __device__ __forceinline__ A lanes_sum(A v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
@@ -91,7 +167,8 @@ template <class A> __device__ __forceinline__ A lanes_sum(A v) {
 }
 
 // one wavefront per output; the innermost reduced dim has stride 1
-template <class E>
+// V > 1: every row start is a multiple of V elements and 16 bytes (the launcher checks), a lane reads V at a time
+template <class E, int V>
 __global__ __launch_bounds__(256) void sum_by_row_kernel(const typename E::storage *__restrict__ in,
                                                         typename E::storage *__restrict__ out, DevReduction r) {
     typedef typename E::storage S;
@@ -104,7 +181,18 @@ __global__ __launch_bounds__(256) void sum_by_row_kernel(const typename E::stora
     A acc = (A)0;
     for (long i = 0; i < outer; i++) {
         const S *p = base + outer_red_offset(r, i);
-        for (long j = lane; j < inner; j += 64) acc += E::load(p[j]);
+        if constexpr (V == 1) {
+            for (long j = lane; j < inner; j += 64) acc += E::load(p[j]);
+        } else {
+            struct alignas(sizeof(S) * V) Vec { S e[V]; };
+            const long whole = inner / V;
+            for (long j = lane; j < whole; j += 64) {
+                const Vec x = reinterpret_cast<const Vec *>(p)[j];
+#pragma unroll
+                for (int v = 0; v < V; v++) acc += E::load(x.e[v]);
+            }
+            for (long j = whole * V + lane; j < inner; j += 64) acc += E::load(p[j]);
+        }
     }
     acc = lanes_sum(acc);
     if (lane == 0) out[o] = E::store(acc);
@@ -137,22 +225,61 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
     }
     const bool row_dense = r.red_n > 0 && r.red_stride[r.red_n - 1] == 1 && r.red_shape[r.red_n - 1] >= 128;
     const bool out_dense = r.kept_n > 0 && r.kept_stride[r.kept_n - 1] == 1;
+    constexpr int V = 16 / (int)sizeof(S);
     if (row_dense && !out_dense) {
         const long blocks = (r.n_out + 3) / 4;
         if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "sum needs %ld workgroups", blocks);
-        ctx->last_kernel = "sum_by_row";
-        hipLaunchKernelGGL(sum_by_row_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, r);
+        // 16 bytes per lane: every row must start on a vector boundary
+        bool vec = V > 1 && r.offset % V == 0 && (uintptr_t)in % 16 == 0;
+        for (int d = 0; d < r.kept_n; d++) vec = vec && r.kept_stride[d] % V == 0;
+        for (int d = 0; d + 1 < r.red_n; d++) vec = vec && r.red_stride[d] % V == 0;
+        if (vec) {
+            ctx->last_kernel = "sum_by_row_vec";
+            hipLaunchKernelGGL((sum_by_row_kernel<E, V>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, r);
+        } else {
+            ctx->last_kernel = "sum_by_row";
+            hipLaunchKernelGGL((sum_by_row_kernel<E, 1>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, r);
+        }
         HODU_HIP(hipGetLastError());
         return HODU_ROCM_OK;
     }
     // V outputs per thread as one 16-byte load: the outputs' last dim must be dense, a whole number of vectors
     // long, and every other stride, the offset and both bases must keep a vector aligned
-    constexpr int V = 16 / (int)sizeof(S);
     bool vec = V > 1 && out_dense && r.kept_shape[r.kept_n - 1] % V == 0 && r.offset % V == 0 &&
                (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0;
     for (int d = 0; d + 1 < r.kept_n; d++) vec = vec && r.kept_stride[d] % V == 0;
     for (int d = 0; d < r.red_n; d++) vec = vec && r.red_stride[d] % V == 0;
     const long threads = vec ? r.n_out / V : r.n_out;
+    // few outputs and a long reduction: cut the reduced index space into chunks (see the top of the file)
+    const long cus = ctx->props.multiProcessorCount;
+    if (out_dense && threads < cus * 256 && r.reduce_size >= 64) {
+        typedef typename E::acc A;
+        const long xblocks = (threads + 63) / 64;
+        long chunks = (4 * cus + xblocks - 1) / xblocks;           // about four workgroups per CU
+        if (chunks > r.reduce_size / 8) chunks = r.reduce_size / 8;  // at least 8 indices per chunk
+        if (chunks > 65535) chunks = 65535;
+        if (chunks >= 2 && xblocks <= 0x7FFFFFFFL) {
+            const long per_chunk = (r.reduce_size + chunks - 1) / chunks;
+            chunks = (r.reduce_size + per_chunk - 1) / per_chunk;
+            int rc = ensure_workspace(ctx, (size_t)chunks * r.n_out * sizeof(A));
+            if (rc != HODU_ROCM_OK) return rc;
+            A *partial = (A *)ctx->workspace.ptr;
+            if (vec) {
+                ctx->last_kernel = "sum_chunks_vec";
+                hipLaunchKernelGGL((sum_chunks_kernel<E, V>), dim3((unsigned)xblocks, (unsigned)chunks), dim3(256), 0, ctx->stream,
+                                   (const S *)in, partial, r, per_chunk);
+            } else {
+                ctx->last_kernel = "sum_chunks";
+                hipLaunchKernelGGL((sum_chunks_kernel<E, 1>), dim3((unsigned)xblocks, (unsigned)chunks), dim3(256), 0, ctx->stream,
+                                   (const S *)in, partial, r, per_chunk);
+            }
+            HODU_HIP(hipGetLastError());
+            hipLaunchKernelGGL(sum_finish_kernel<E>, dim3((unsigned)((r.n_out + 63) / 64)), dim3(256), 0, ctx->stream,
+                               (const A *)partial, (S *)out, r.n_out, (int)chunks);
+            HODU_HIP(hipGetLastError());
+            return HODU_ROCM_OK;
+        }
+    }
     const long blocks = (threads + 255) / 256;
     if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "sum needs %ld workgroups", blocks);
     if (vec) {

@@ -116,6 +116,8 @@ def load() -> ctypes.CDLL:
                                                     ctypes.POINTER(EpilogueStep), sz, ci, ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_debug_time_cast.argtypes = [vp, ci, ci, ctypes.POINTER(vp), ctypes.POINTER(vp), sz, szp, sz, ci,
                                               ctypes.POINTER(ctypes.c_float)]
+    lib.hodu_rocm_debug_time_sum.argtypes = [vp, ci, ctypes.POINTER(vp), ctypes.POINTER(vp), sz, szp, sz, ci,
+                                             ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, ctypes.POINTER(ctypes.c_float),
                                                ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.hodu_rocm_debug_read_floor.argtypes = [vp, ctypes.POINTER(vp), sz, sz, ci, ctypes.POINTER(ctypes.c_float),
@@ -370,6 +372,19 @@ class Context:
         ms = ctypes.c_float()
         self._check(self.lib.hodu_rocm_debug_time_cast(self.handle, DTYPE_ID[src], DTYPE_ID[dst], pin, pout, len(ins), arr, n,
                                                        int(iters), ctypes.byref(ms)))
+        return float(ms.value)
+
+    def time_sum(self, dt: str, ins, outs, md, iters: int) -> float:
+        """back-to-back hodu_rocm_sum launches issued from C over the buffer pairs in turn; total ms (the caller sizes
+        the buffers for the metadata, as for Context.sum)"""
+        if len(ins) != len(outs) or not ins:
+            raise HoduRocmError(INVALID_ARG, "time_sum: need as many outputs as inputs, at least one")
+        arr, n = _md_array(md)
+        pin = (ctypes.c_void_p * len(ins))(*[b.ptr for b in ins])
+        pout = (ctypes.c_void_p * len(outs))(*[b.ptr for b in outs])
+        ms = ctypes.c_float()
+        self._check(self.lib.hodu_rocm_debug_time_sum(self.handle, DTYPE_ID[dt], pin, pout, len(ins), arr, n, int(iters),
+                                                      ctypes.byref(ms)))
         return float(ms.value)
 
     def mfma_clock(self, kind: int, operands: DeviceBuffer, iters: int = 20000) -> dict:

@@ -221,6 +221,9 @@ HODU_ROCM_DECL_PRODUCT_EX(i32_i8i8)     /* vector / scalar in i32 */
 int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src_dtype, int dst_dtype, const void *const *in_list,
                               void *const *out_list, size_t n_buffers, const size_t *metadata, size_t metadata_len,
                               int iters, float *elapsed_ms);
+/* measurement hook: the same for hodu_rocm_sum */
+int hodu_rocm_debug_time_sum(hodu_rocm_ctx *ctx, int dtype, const void *const *in_list, void *const *out_list,
+                             size_t n_buffers, const size_t *metadata, size_t metadata_len, int iters, float *elapsed_ms);
 /* measurement hook: hodu_rocm_debug_time_product with fused steps */
 int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
                                     const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
