@@ -5,7 +5,8 @@
 // masked_fill(-inf) (:40-48, mask[i][j] = j > i, :73-86).
 //
 // Here a row is read once: a wavefront owns a row whose dim is dense and at most 4096 long and keeps it in
-// registers (max, exp, sum, scale without touching memory again); longer or strided rows take three passes from
+// registers (max, exp, sum, scale without touching memory again); a longer dense row belongs to a workgroup, which
+// reads it twice (an online maximum / sum pass, then the pass that writes); strided rows take three passes from
 // memory with a thread per row.  Arithmetic: elements widened exactly to f32 (f64 stays f64), exp and the sum in that
 // type, one rounding (RNE) on store.  With `causal` the entries j > i of each [Sq, Sk] matrix count as -inf: they
 // come out as exact zeros, and the mask tensor is never built.
@@ -40,17 +41,18 @@ template <class W> __device__ __forceinline__ W wexp(W x);
 template <> __device__ __forceinline__ float wexp<float>(float x) { return expf(x); }
 template <> __device__ __forceinline__ double wexp<double>(double x) { return exp(x); }
 
-template <class W> __device__ __forceinline__ W lanes_max(W v) {
+// over groups of LANES neighbouring lanes (a power of two)
+template <class W, int LANES = 64> __device__ __forceinline__ W lanes_max(W v) {
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
+    for (int m = LANES / 2; m >= 1; m >>= 1) {
         const W o = __shfl_xor(v, m, 64);
         v = o > v ? o : v;
     }
     return v;
 }
-template <class W> __device__ __forceinline__ W lanes_add(W v) {
+template <class W, int LANES = 64> __device__ __forceinline__ W lanes_add(W v) {
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    for (int m = LANES / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
     return v;
 }
 
@@ -91,15 +93,16 @@ __global__ __launch_bounds__(256) void softmax_row_kernel(const typename E::stor
 
 // the same with 16-byte accesses: a lane holds NV vectors of V neighbouring entries (len a multiple of V, rows and
 // bases 16-byte aligned)
-template <class E, int NV, int V>
+// LPR lanes per row: short rows share a wavefront (64 / LPR of them) instead of leaving most of its lanes idle
+template <class E, int NV, int V, int LPR = 64>
 __global__ __launch_bounds__(256) void softmax_row_vec_kernel(const typename E::storage *__restrict__ in,
                                                              typename E::storage *__restrict__ out, DevSoftmax s) {
     typedef typename E::acc W;
     typedef typename E::storage S;
     struct alignas(16) Vec { S e[V]; };
-    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    if (row >= s.rows) return;
+    const long row = (long)blockIdx.x * (256 / LPR) + (threadIdx.x / LPR);
+    const int lane = threadIdx.x % LPR;
+    if (row >= s.rows) return;  // (whole groups of LPR lanes leave together; the shuffles stay inside a group)
     const S *x = in + s.offset + row_offset(s, row);
     const long limit = s.causal ? (row % s.sq) + 1 : s.len;
     const W ninf = -(W)INFINITY;
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(256) void softmax_row_vec_kernel(const typename E::
     W m = ninf;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        const long j0 = (lane + 64L * i) * V;
+        const long j0 = (lane + (long)LPR * i) * V;
         Vec raw;
         if (j0 < s.len && j0 < limit) raw = *reinterpret_cast<const Vec *>(x + j0);
 #pragma unroll
@@ -116,7 +119,7 @@ __global__ __launch_bounds__(256) void softmax_row_vec_kernel(const typename E::
             m = v[i][e] > m ? v[i][e] : m;
         }
     }
-    m = lanes_max(m);
+    m = lanes_max<W, LPR>(m);
     W sum = (W)0;
 #pragma unroll
     for (int i = 0; i < NV; i++)
@@ -125,16 +128,89 @@ __global__ __launch_bounds__(256) void softmax_row_vec_kernel(const typename E::
             v[i][e] = v[i][e] == ninf ? (W)0 : wexp<W>(v[i][e] - m);
             sum += v[i][e];
         }
-    sum = lanes_add(sum);
+    sum = lanes_add<W, LPR>(sum);
     S *y = out + row * s.len;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        const long j0 = (lane + 64L * i) * V;
+        const long j0 = (lane + (long)LPR * i) * V;
         if (j0 >= s.len) continue;
         Vec o;
 #pragma unroll
         for (int e = 0; e < V; e++) o.e[e] = E::store(v[i][e] / sum);
         *reinterpret_cast<Vec *>(y + j0) = o;
+    }
+}
+
+// a dense row of any length: a workgroup per row, two passes.  Pass 1 keeps, per thread, a running maximum m and the
+// sum l of exp(x - m) over its entries (rescaled when m moves), then the 256 pairs meet: (m, l) + (m', l') =
+// (M = max(m, m'), l exp(m - M) + l' exp(m' - M)).  Pass 2 reads the row again (from L2 for all but very long rows)
+// and writes exp(x - M) / L.  V > 1: 16 bytes per lane (len a multiple of V, rows and bases 16-byte aligned).
+template <class W> __device__ __forceinline__ void meet(W &m, W &l, W m2, W l2) {
+    const W big = m2 > m ? m2 : m;
+    if (big == -(W)INFINITY) return;  // both empty: l stays 0
+    l = l * wexp<W>(m - big) + l2 * wexp<W>(m2 - big);
+    m = big;
+}
+
+template <class E, int V>
+__global__ __launch_bounds__(256) void softmax_long_kernel(const typename E::storage *__restrict__ in,
+                                                          typename E::storage *__restrict__ out, DevSoftmax s) {
+    typedef typename E::acc W;
+    typedef typename E::storage S;
+    struct alignas(sizeof(S) * V) Vec { S e[V]; };
+    __shared__ W wave_m[4], wave_l[4];
+    const long row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const S *x = in + s.offset + row_offset(s, row);
+    long limit = s.causal ? (row % s.sq) + 1 : s.len;
+    limit = limit < s.len ? limit : s.len;
+    const W ninf = -(W)INFINITY;
+    W m = ninf, l = (W)0;
+    for (long j0 = (long)tid * V; j0 < limit; j0 += 256L * V) {
+        W v[V];
+        if constexpr (V == 1) {
+            v[0] = (W)E::load(x[j0]);
+        } else {
+            const Vec raw = *reinterpret_cast<const Vec *>(x + j0);
+#pragma unroll
+            for (int e = 0; e < V; e++) v[e] = j0 + e < limit ? (W)E::load(raw.e[e]) : ninf;
+        }
+        W vm = v[0];
+#pragma unroll
+        for (int e = 1; e < V; e++) vm = v[e] > vm ? v[e] : vm;
+        if (vm > m) {
+            l *= wexp<W>(m - vm);  // exp(-inf) = 0 on the first entries
+            m = vm;
+        }
+        if (m != ninf) {
+#pragma unroll
+            for (int e = 0; e < V; e++) l += wexp<W>(v[e] - m);
+        }
+    }
+#pragma unroll
+    for (int k = 32; k >= 1; k >>= 1) meet(m, l, (W)__shfl_xor(m, k, 64), (W)__shfl_xor(l, k, 64));
+    if ((tid & 63) == 0) { wave_m[tid >> 6] = m; wave_l[tid >> 6] = l; }
+    __syncthreads();
+    m = wave_m[0]; l = wave_l[0];
+#pragma unroll
+    for (int w = 1; w < 4; w++) meet(m, l, wave_m[w], wave_l[w]);
+    const W inv = (W)1 / l;
+    S *y = out + row * s.len;
+    for (long j0 = (long)tid * V; j0 < s.len; j0 += 256L * V) {
+        if constexpr (V == 1) {
+            y[j0] = E::store(j0 < limit ? wexp<W>((W)E::load(x[j0]) - m) * inv : (W)0);
+        } else {
+            Vec o;
+            if (j0 < limit) {
+                const Vec raw = *reinterpret_cast<const Vec *>(x + j0);
+#pragma unroll
+                for (int e = 0; e < V; e++) o.e[e] = E::store(j0 + e < limit ? wexp<W>((W)E::load(raw.e[e]) - m) * inv : (W)0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; e++) o.e[e] = E::store((W)0);
+            }
+            *reinterpret_cast<Vec *>(y + j0) = o;
+        }
     }
 }
 
@@ -172,11 +248,15 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
             ctx->last_kernel = "softmax_row_vec";
             const long vecs = s.len / V;
 #define LAUNCHV(NV) hipLaunchKernelGGL((softmax_row_vec_kernel<E, NV, V>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s)
-            if (vecs <= 64) LAUNCHV(1);
+#define LAUNCHS(LPR) hipLaunchKernelGGL((softmax_row_vec_kernel<E, 1, V, LPR>), dim3((unsigned)((s.rows + 256 / LPR - 1) / (256 / LPR))), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s)
+            if (vecs <= 16) LAUNCHS(16);
+            else if (vecs <= 32) LAUNCHS(32);
+            else if (vecs <= 64) LAUNCHV(1);
             else if (vecs <= 128) LAUNCHV(2);
             else if (vecs <= 256) LAUNCHV(4);
             else if (vecs <= 512) LAUNCHV(8);
             else LAUNCHV(64 / V);  // up to 4096 entries
+#undef LAUNCHS
 #undef LAUNCHV
             HODU_HIP(hipGetLastError());
             return HODU_ROCM_OK;
@@ -193,6 +273,20 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
         return HODU_ROCM_OK;
     }
     if (!dim_is_last) return fail(HODU_ROCM_UNSUPPORTED, "softmax: only the last dim is supported");
+    if (s.stride == 1 && s.rows <= 0x7FFFFFFFL) {
+        constexpr int V = 16 / (int)sizeof(S);
+        bool vec = s.len % V == 0 && s.offset % V == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0;
+        for (int d = 0; d < s.kept_n; d++) vec = vec && s.kept_stride[d] % V == 0;
+        if (vec) {
+            ctx->last_kernel = "softmax_long_vec";
+            hipLaunchKernelGGL((softmax_long_kernel<E, V>), dim3((unsigned)s.rows), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s);
+        } else {
+            ctx->last_kernel = "softmax_long";
+            hipLaunchKernelGGL((softmax_long_kernel<E, 1>), dim3((unsigned)s.rows), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s);
+        }
+        HODU_HIP(hipGetLastError());
+        return HODU_ROCM_OK;
+    }
     const long blocks = (s.rows + 255) / 256;
     if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "softmax needs %ld workgroups", blocks);
     ctx->last_kernel = "softmax_strided";

@@ -57,6 +57,15 @@ def test_rows_in_registers(ctx, dt):
     assert ctx.last_kernel() == "softmax_row"       # misaligned base
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64"])
+def test_short_rows_share_a_wavefront(ctx, dt):
+    """rows of at most 16 (32) vectors are handled 4 (2) to a wavefront; row counts that leave a wavefront or a
+    workgroup partly empty"""
+    for n, (rows, length) in enumerate(((1, 8), (37, 64), (101, 128), (9, 256), (1030, 32), (5, 16))):
+        check_softmax(ctx, dt, V([rows, length]), 1, seed=60 + n, expect_kernel="softmax_row_vec")
+    check_softmax(ctx, dt, V([3, 50, 64]), 2, causal=True, seed=70, expect_kernel="softmax_row_vec")
+
+
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 def test_causal_mask(ctx, dt):
     """attention.rs:40-48 with create_causal_mask (:73-86): row i of each [Sq, Sk] matrix keeps entries j <= i"""
@@ -68,7 +77,11 @@ def test_causal_mask(ctx, dt):
 
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 def test_long_and_strided_rows(ctx, dt):
-    check_softmax(ctx, dt, V([3, 5000]), 1, seed=40, expect_kernel="softmax_strided")
+    check_softmax(ctx, dt, V([3, 5000]), 1, seed=40, expect_kernel="softmax_long_vec")     # a workgroup per row
+    check_softmax(ctx, dt, V([2, 4099]), 1, seed=44, expect_kernel="softmax_long")         # no whole vectors
+    check_softmax(ctx, dt, V([3, 40000]), 1, seed=45, scale=3.0, expect_kernel="softmax_long_vec")
+    check_softmax(ctx, dt, V([2, 3, 5000], offset=8).t(0, 1), 2, seed=46, expect_kernel="softmax_long_vec")
+    check_softmax(ctx, dt, V([2, 6000, 6000]), 2, causal=True, seed=47, expect_kernel="softmax_long_vec")
     check_softmax(ctx, dt, V([6, 90]).slice(1, 1, 90, 3), 1, seed=41, expect_kernel="softmax_strided")
     check_softmax(ctx, dt, V([5, 8, 40], offset=3).t(0, 1), 2, seed=42, expect_kernel="softmax_row")  # rows still dense
     check_softmax(ctx, dt, V([6, 50]).slice(1, 0, 50, 2), 1, causal=True, seed=43, expect_kernel="softmax_strided")
