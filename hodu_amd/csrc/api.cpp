@@ -20,6 +20,10 @@ int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const v
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     rc = launch_skinny(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    if (ctx->force_tile < 0) {  // (a pinned tile variant means the caller wants that kernel)
+        rc = launch_gemv_rows(ctx, kind, dtype, a, b, c, g);
+        if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    }
     rc = launch_mfma(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     ctx->last_kernel = "generic";

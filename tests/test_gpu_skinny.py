@@ -131,3 +131,39 @@ def test_gemv_batch_folding_and_fallbacks(ctx, kind):
     # K not a multiple of the 16-byte vector: falls through
     k = 72 if "f8" in kind else 68
     check_product(ctx, "dot", kind, V([1, k]), V([16, k]).t(), seed=3, rscale=rs, expect_kernel="")
+
+
+ROWS_KINDS = {"bf16": ("gemv_rows_bf16", 4), "f16": ("gemv_rows_f16", 4), "f32": ("gemv_rows_f32", 16)}
+
+
+@pytest.mark.parametrize("kind", list(ROWS_KINDS))
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 13, 16])
+def test_row_dense_weight(ctx, kind, m):
+    """x [m, K] times W stored [K, N] (N contiguous): the kernel that sums weight rows, K cut into chunks -- f32 up to 16
+    rows, bf16 / f16 up to 4 (beyond, and for the other kinds, the tile kernels); K that leaves a ragged last chunk, N
+    that leaves a partly empty last workgroup, a column-strided x"""
+    name, m_max = ROWS_KINDS[kind]
+    expect = name if m <= m_max else "mfma_"
+    check_product(ctx, "dot", kind, V([m, 1000]), V([1000, 320]), seed=m, expect_kernel=expect)
+    k = 2048 if kind == "f32" else 4096  # (f32 against the sequential-k oracle at 1e-5: the orders differ, keep K moderate)
+    check_product(ctx, "dot", kind, V([m, k]), V([k, 1024]), seed=20 + m, expect_kernel=expect)
+    check_product(ctx, "dot", kind, V([m, 200]).slice(1, 0, 200, 2), V([100, 64]), seed=40 + m, expect_kernel=expect)
+
+
+@pytest.mark.parametrize("kind", list(ROWS_KINDS))
+def test_row_dense_weight_views_and_fallbacks(ctx, kind):
+    name, _ = ROWS_KINDS[kind]
+    # a column slice of a wider weight (row pitch > N) at an aligned offset
+    check_product(ctx, "dot", kind, V([4, 256]), V([256, 512], offset=64).slice(1, 64, 320), seed=1, expect_kernel=name)
+    # N not a multiple of the 8-byte vector, a misaligned offset, a batch: other kernels take these
+    check_product(ctx, "dot", kind, V([2, 256]), V([256, 100 + 3]), seed=2)
+    assert not ctx.last_kernel().startswith("gemv_rows")
+    check_product(ctx, "dot", kind, V([2, 256]), V([256, 128], offset=1), seed=3)
+    assert not ctx.last_kernel().startswith("gemv_rows")
+    check_product(ctx, "matmul", kind, V([3, 2, 256]), V([3, 256, 128]), seed=4)
+    assert not ctx.last_kernel().startswith("gemv_rows")
+
+
+def test_row_dense_weight_other_kinds_keep_the_tile_kernels(ctx):
+    check_product(ctx, "dot", "bf16_f8e4m3w", V([1, 256]), V([256, 64]), seed=4, rscale=2.0, expect_kernel="mfma_")
+    check_product(ctx, "dot", "i32_i8i8", V([2, 256]), V([256, 64]), seed=5, expect_kernel="mfma_")
