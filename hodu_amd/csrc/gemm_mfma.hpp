@@ -596,10 +596,13 @@ __device__ __forceinline__ void compute_stage(const char *As, const char *Bs, ac
 // LDS-DMA loads are tracked by vmcnt; wait for them before the barrier that publishes the stage
 __device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// steps_per_split > 0 (kernels without fused steps only): K is cut into ranges of that many K steps, one per
+// blockIdx.y, and the range's sums go to partials[blockIdx.y] in the accumulate type; a second kernel adds them
 template <class Cfg, bool EPI>
 __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                typename Out<Cfg::OUT>::T *__restrict__ C,
-                                                               DevProduct g, int tiles_m, int tiles_n) {
+                                                               DevProduct g, int tiles_m, int tiles_n, int steps_per_split,
+                                                               void *__restrict__ partials) {
     extern __shared__ __align__(16) char smem[];
     typedef typename Compute32<Cfg::CK>::acc_t acc_t;
     typedef typename Cfg::LoaderA LoaderA;
@@ -631,23 +634,30 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
     LoaderA la;
     LoaderB lb;
     const int KT_full = g.K / BK;             // K steps that lie fully inside K
-    const int KT = (g.K + BK - 1) / BK;       // plus the ragged one, if any
-    if (KT_full > 0) {
-        la.issue_full(opA, m0, 0, tid, smem);
-        lb.issue_full(opB, n0, 0, tid, smem + Cfg::A_BYTES);
+    const int KT_all = (g.K + BK - 1) / BK;   // plus the ragged one, if any
+    int kt0 = 0, KT = KT_all;                 // this workgroup's range of K steps
+    if constexpr (!EPI) {
+        if (steps_per_split > 0) {
+            kt0 = blockIdx.y * steps_per_split;
+            KT = kt0 + steps_per_split < KT_all ? kt0 + steps_per_split : KT_all;
+        }
+    }
+    if (kt0 < KT_full) {
+        la.issue_full(opA, m0, kt0 * BK, tid, smem);
+        lb.issue_full(opB, n0, kt0 * BK, tid, smem + Cfg::A_BYTES);
         la.commit_full(smem, tid);
         lb.commit_full(smem + Cfg::A_BYTES, tid);
         wait_vm();
     } else {
-        la.tail(opA, m0, 0, tid, smem);
-        lb.tail(opB, n0, 0, tid, smem + Cfg::A_BYTES);
+        la.tail(opA, m0, kt0 * BK, tid, smem);
+        lb.tail(opB, n0, kt0 * BK, tid, smem + Cfg::A_BYTES);
     }
     __syncthreads();
 
     const int a_row = wave_m * TM * 32 + lr, b_row = wave_n * TN * 32 + lr;
-    for (int kt = 0; kt < KT; kt++) {
-        char *cur = smem + (kt & 1) * Cfg::STAGE_BYTES;
-        char *nxt = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
+    for (int kt = kt0; kt < KT; kt++) {
+        char *cur = smem + ((kt - kt0) & 1) * Cfg::STAGE_BYTES;
+        char *nxt = smem + ((kt - kt0 + 1) & 1) * Cfg::STAGE_BYTES;
         const bool more_full = kt + 1 < KT_full;
         if (more_full) {  // in flight while the matrix cores work on the current stage
             la.issue_full(opA, m0, (kt + 1) * BK, tid, nxt);
@@ -665,8 +675,22 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
         __syncthreads();
     }
 
-    out_t *Cb = C + batch * (long)g.M * g.N;
     const bool vec_ok = (g.N & 3) == 0;
+    if constexpr (!EPI) {
+        if (steps_per_split > 0) {
+            constexpr int ACC = Cfg::CK == CK_I8 ? OUT_I32 : OUT_F32;
+            typedef typename Out<ACC>::T part_t;
+            part_t *Pb = reinterpret_cast<part_t *>(partials) + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    store_tile32<ACC, false>(Pb, acc[i][j], m0 + wave_m * TM * 32 + i * 32 + lr, n0 + wave_n * TN * 32 + j * 32, lh,
+                                             g.M, g.N, vec_ok, g.epi);
+            return;
+        }
+    }
+    out_t *Cb = C + batch * (long)g.M * g.N;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -674,6 +698,41 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
             store_tile32<Cfg::OUT, EPI>(Cb, acc[i][j], m0 + wave_m * TM * 32 + i * 32 + lr, n0 + wave_n * TN * 32 + j * 32, lh,
                                    g.M, g.N, vec_ok, g.epi);
 }
+
+// out[i] = round(partials[0][i] + partials[1][i] + ...), the slabs added in index order: bit-reproducible
+template <int OUT, class part_t>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const part_t *__restrict__ partials,
+                                                           typename Out<OUT>::T *__restrict__ out, long elems, int splits,
+                                                           int N, DevEpilogue epi) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= elems) return;
+    // column of element i + e, for the fused element-wise steps (rows are N long, outputs contiguous)
+    long col[4] = {0, 0, 0, 0};
+    if (epi.n != 0) {
+        col[0] = i % N;
+#pragma unroll
+        for (int e = 1; e < 4; e++) col[e] = col[e - 1] + 1 == N ? 0 : col[e - 1] + 1;
+    }
+    if (i + 3 < elems) {
+        struct alignas(16) Quad { part_t q[4]; };
+        Quad s = *reinterpret_cast<const Quad *>(partials + i);
+        for (int k = 1; k < splits; k++) {
+            const Quad t = *reinterpret_cast<const Quad *>(partials + (long)k * elems + i);
+#pragma unroll
+            for (int e = 0; e < 4; e++) s.q[e] += t.q[e];
+        }
+        struct alignas(sizeof(typename Out<OUT>::T) * 4) OutQuad { typename Out<OUT>::T q[4]; };
+        *reinterpret_cast<OutQuad *>(out + i) = OutQuad{{finish<OUT>(epi, s.q[0], col[0]), finish<OUT>(epi, s.q[1], col[1]),
+                                                       finish<OUT>(epi, s.q[2], col[2]), finish<OUT>(epi, s.q[3], col[3])}};
+    } else {
+        for (long j = i; j < elems; j++) {
+            part_t s = partials[j];
+            for (int k = 1; k < splits; k++) s += partials[(long)k * elems + j];
+            out[j] = finish<OUT>(epi, s, col[j - i]);
+        }
+    }
+}
+
 
 // ------------------------------------------------------------------------------------------------
 // host side: load-mode selection and launch
@@ -697,14 +756,42 @@ inline int pick_mode(const void *base, long off, long row_stride, long k_stride,
     return LM_SCALAR;
 }
 
-template <class Cfg> int launch_config(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
-    auto kernel = g.epi.n != 0 ? mfma_product_kernel<Cfg, true> : mfma_product_kernel<Cfg, false>;
-    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
+// splits > 1: K is cut into that many ranges of whole K steps (grid.y); the partial sums go through the context's
+// workspace and splitk_reduce_kernel (which also applies the fused steps); batches * M * N must be a multiple of 4
+template <class Cfg> int launch_config(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
+                                       int splits = 1) {
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     const long total = g.batches * tiles_m * tiles_n;
     if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a,
-                       (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n);
+    const long elems = g.batches * (long)g.M * g.N;
+    const int KT = (g.K + Cfg::BK - 1) / Cfg::BK;
+    int per = 0;
+    if (splits > 1 && elems % 4 == 0) {
+        per = (KT + splits - 1) / splits;
+        splits = (KT + per - 1) / per;
+    }
+    if (splits <= 1 || per == 0) {
+        auto kernel = g.epi.n != 0 ? mfma_product_kernel<Cfg, true> : mfma_product_kernel<Cfg, false>;
+        if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a,
+                           (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n, 0, (void *)nullptr);
+        HODU_HIP(hipGetLastError());
+        return HODU_ROCM_OK;
+    }
+    auto kernel = mfma_product_kernel<Cfg, false>;
+    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
+    if (int rc = ensure_workspace(ctx, (size_t)splits * elems * 4)) return rc;
+    void *partials = ctx->workspace.ptr;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)total, (unsigned)splits), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream,
+                       (const char *)a, (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n, per, partials);
+    HODU_HIP(hipGetLastError());
+    const unsigned blocks = (unsigned)((elems + 1023) / 1024);
+    if (Cfg::CK == CK_I8)
+        hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, int32_t>), dim3(blocks), dim3(256), 0, ctx->stream,
+                           (const int32_t *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits, g.N, g.epi);
+    else
+        hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, float>), dim3(blocks), dim3(256), 0, ctx->stream,
+                           (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits, g.N, g.epi);
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }

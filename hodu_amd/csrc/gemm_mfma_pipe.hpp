@@ -565,40 +565,6 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         store_band_via_lds<Cfg::OUT, TN, true>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
 }
 
-// out[i] = round(partials[0][i] + partials[1][i] + ...), the slabs added in index order: bit-reproducible
-template <int OUT, class part_t>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const part_t *__restrict__ partials,
-                                                           typename Out<OUT>::T *__restrict__ out, long elems, int splits,
-                                                           int N, DevEpilogue epi) {
-    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= elems) return;
-    // column of element i + e, for the fused element-wise steps (rows are N long, outputs contiguous)
-    long col[4] = {0, 0, 0, 0};
-    if (epi.n != 0) {
-        col[0] = i % N;
-#pragma unroll
-        for (int e = 1; e < 4; e++) col[e] = col[e - 1] + 1 == N ? 0 : col[e - 1] + 1;
-    }
-    if (i + 3 < elems) {
-        struct alignas(16) Quad { part_t q[4]; };
-        Quad s = *reinterpret_cast<const Quad *>(partials + i);
-        for (int k = 1; k < splits; k++) {
-            const Quad t = *reinterpret_cast<const Quad *>(partials + (long)k * elems + i);
-#pragma unroll
-            for (int e = 0; e < 4; e++) s.q[e] += t.q[e];
-        }
-        struct alignas(sizeof(typename Out<OUT>::T) * 4) OutQuad { typename Out<OUT>::T q[4]; };
-        *reinterpret_cast<OutQuad *>(out + i) = OutQuad{{finish<OUT>(epi, s.q[0], col[0]), finish<OUT>(epi, s.q[1], col[1]),
-                                                       finish<OUT>(epi, s.q[2], col[2]), finish<OUT>(epi, s.q[3], col[3])}};
-    } else {
-        for (long j = i; j < elems; j++) {
-            part_t s = partials[j];
-            for (int k = 1; k < splits; k++) s += partials[(long)k * elems + j];
-            out[j] = finish<OUT>(epi, s, col[j - i]);
-        }
-    }
-}
-
 // splits > 1: K is cut into that many ranges of whole stages, each range a workgroup of its own (grid.y);
 // the partial sums go through the context's workspace (splits x batches x M x N accumulators, which requires
 // batches * M * N to be a multiple of 4 for the vectorised second pass -- the caller checks)
