@@ -30,6 +30,17 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64
     const int forced = ctx->force_tile;
     int size = forced >= 0 ? forced % 10 : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 2 : 3;
+    if (forced < 0) {
+        // many small matrices (a batch of 128 x 128 or 16 x 16 products) fill the chip with tiles that are mostly
+        // padding: step down while the smaller tile wastes markedly less (fraction of a tile's outputs that exist)
+        auto used = [&](long bm) {
+            return (double)g.M * g.N / ((double)((g.M + bm - 1) / bm * bm) * (double)((g.N + bm - 1) / bm * bm));
+        };
+        if (size == 0 && used(256) < 0.75 * used(128)) size = 2;
+        // (the 64 x 64 kernels are the plainest ones: only when they waste less than half as much; bf16
+        // [64, 512, 512] x [64, 512, 64] measured 11.3 us with 128 x 128 tiles against 14.3 us with 64 x 64)
+        if (size == 2 && used(128) < 0.5 * used(64)) size = 3;
+    }
     // A product too small to fill the machine with 128x128 tiles is cut along K instead of shrinking the tile
     // further (pipelined kernels only): same HBM traffic, four times fewer bytes through LDS per flop.
     const int stages = (int)((long)g.K * ES / 128);
