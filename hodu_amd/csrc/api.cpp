@@ -16,7 +16,9 @@ int check_ptrs(const char *op, hodu_rocm_ctx *ctx, const void *a, const void *b,
 // Picks the kernel family for one launch-sized product.
 int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                  const DevProduct &g) {
-    int rc = ctx->force_tile == 30 ? HODU_ROCM_UNSUPPORTED : launch_gemv(ctx, kind, dtype, a, b, c, g);
+    int rc = ctx->force_tile >= 0 ? HODU_ROCM_UNSUPPORTED : launch_inner_product(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    rc = ctx->force_tile == 30 ? HODU_ROCM_UNSUPPORTED : launch_gemv(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     rc = launch_skinny(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;

@@ -167,6 +167,8 @@ int launch_mfma(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const vo
 int launch_gemv(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g);
 int launch_skinny(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                   const DevProduct &g);
+// [1, K] x [K, 1] with a long K (reduce.hip)
+int launch_inner_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g);
 // at most 16 rows against a row-dense right operand (gemv_rows.hip)
 int launch_gemv_rows(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g);
 

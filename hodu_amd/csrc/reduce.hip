@@ -16,7 +16,10 @@
 //     chunks' partial sums (in the accumulate type) go through the context's workspace and a second kernel adds
 //     them in chunk order and rounds once;
 //   * the innermost reduced dim is dense (a row sum): a wavefront owns an output, its lanes stride over that dim
-//     (16 bytes per lane when alignment allows), and the lane sums meet in a butterfly.
+//     (16 bytes per lane when alignment allows), and the lane sums meet in a butterfly; few long rows (sum_all of a
+//     large tensor is one) are cut into chunks across workgroups in the same two-kernel way.
+// The same file holds the product of two long vectors (Tensor::matmul of two 1-D tensors is mul + sum_all in the
+// reference): chunks of sum_k a[k] b[k] across workgroups, then the same second kernel.
 #include "common.hpp"
 #include "device_types.hpp"
 #include "elem.hpp"
@@ -87,6 +90,12 @@ __global__ __launch_bounds__(256) void sum_by_output_kernel(const typename E::st
         for (int v = 0; v < V; v++) y.e[v] = E::store(acc[v]);
         *reinterpret_cast<Vec *>(out + o) = y;
     }
+}
+
+template <class A> __device__ __forceinline__ A lanes_sum(A v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
 }
 
 // flattened index over ALL reduced dims -> element offset
@@ -160,11 +169,6 @@ __global__ __launch_bounds__(256) void sum_finish_kernel(const typename E::acc *
     if (wave == 0 && o < n_out) out[o] = E::store(acc + meet[0][lane] + meet[1][lane] + meet[2][lane]);
 }
 
-template <class A> __device__ __forceinline__ A lanes_sum(A v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
 
 // one wavefront per output; the innermost reduced dim has stride 1
 // V > 1: every row start is a multiple of V elements and 16 bytes (the launcher checks), a lane reads V at a time
@@ -196,6 +200,77 @@ __global__ __launch_bounds__(256) void sum_by_row_kernel(const typename E::stora
     }
     acc = lanes_sum(acc);
     if (lane == 0) out[o] = E::store(acc);
+}
+
+// sum of the 256 threads' values, in thread 0 (fixed order: butterfly inside a wavefront, then the four wavefronts)
+template <class A> __device__ __forceinline__ A block_sum(A v, A *meet4) {
+    v = lanes_sum(v);
+    if ((threadIdx.x & 63) == 0) meet4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return meet4[0] + meet4[1] + meet4[2] + meet4[3];
+}
+
+// few outputs, each a long dense row (sum_all of a large tensor is one such row): a workgroup sums chunk y of row x,
+// 16 bytes per lane when V > 1 (rows start on vector boundaries), and leaves partial[y][x] for sum_finish_kernel
+template <class E, int V>
+__global__ __launch_bounds__(256) void sum_row_chunks_kernel(const typename E::storage *__restrict__ in,
+                                                            typename E::acc *__restrict__ partial, DevReduction r,
+                                                            long per_chunk) {
+    typedef typename E::storage S;
+    typedef typename E::acc A;
+    __shared__ A meet4[4];
+    const long o = blockIdx.x;
+    const long inner = r.red_shape[r.red_n - 1], outer = r.reduce_size / inner;
+    const long begin = (long)blockIdx.y * per_chunk;  // a multiple of V
+    const long end = begin + per_chunk < inner ? begin + per_chunk : inner;
+    const S *base = in + r.offset + kept_offset(r, o);
+    A acc = (A)0;
+    for (long i = 0; i < outer; i++) {
+        const S *p = base + outer_red_offset(r, i);
+        if constexpr (V == 1) {
+            for (long j = begin + threadIdx.x; j < end; j += 256) acc += E::load(p[j]);
+        } else {
+            struct alignas(sizeof(S) * V) Vec { S e[V]; };
+            const long whole = begin + (end - begin) / V * V;
+            for (long j = begin + (long)threadIdx.x * V; j < whole; j += 256L * V) {
+                const Vec x = *reinterpret_cast<const Vec *>(p + j);
+#pragma unroll
+                for (int v = 0; v < V; v++) acc += E::load(x.e[v]);
+            }
+            for (long j = whole + threadIdx.x; j < end; j += 256) acc += E::load(p[j]);
+        }
+    }
+    acc = block_sum(acc, meet4);
+    if (threadIdx.x == 0) partial[(long)blockIdx.y * r.n_out + o] = acc;
+}
+
+// the product of two vectors (Tensor::matmul of two 1-D tensors: mul, then sum_all in the reference,
+// crates/hodu_core/src/tensor/ops/matrix.rs:38-47): chunk y of sum_k a[k] b[k], as above
+template <class E, int V>
+__global__ __launch_bounds__(256) void inner_product_kernel(const typename E::storage *__restrict__ a,
+                                                           const typename E::storage *__restrict__ b,
+                                                           typename E::acc *__restrict__ partial, long K, long a_k, long b_k,
+                                                           long per_chunk) {
+    typedef typename E::storage S;
+    typedef typename E::acc A;
+    __shared__ A meet4[4];
+    const long begin = (long)blockIdx.x * per_chunk;
+    const long end = begin + per_chunk < K ? begin + per_chunk : K;
+    A acc = (A)0;
+    if constexpr (V == 1) {
+        for (long k = begin + threadIdx.x; k < end; k += 256) acc += E::load(a[k * a_k]) * E::load(b[k * b_k]);
+    } else {  // both dense and aligned
+        struct alignas(sizeof(S) * V) Vec { S e[V]; };
+        const long whole = begin + (end - begin) / V * V;
+        for (long k = begin + (long)threadIdx.x * V; k < whole; k += 256L * V) {
+            const Vec x = *reinterpret_cast<const Vec *>(a + k), y = *reinterpret_cast<const Vec *>(b + k);
+#pragma unroll
+            for (int v = 0; v < V; v++) acc += E::load(x.e[v]) * E::load(y.e[v]);
+        }
+        for (long k = whole + threadIdx.x; k < end; k += 256) acc += E::load(a[k]) * E::load(b[k]);
+    }
+    acc = block_sum(acc, meet4);
+    if (threadIdx.x == 0) partial[blockIdx.x] = acc;
 }
 
 template <class S> __global__ __launch_bounds__(256) void zero_kernel(S *out, long n) {
@@ -233,6 +308,37 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
         bool vec = V > 1 && r.offset % V == 0 && (uintptr_t)in % 16 == 0;
         for (int d = 0; d < r.kept_n; d++) vec = vec && r.kept_stride[d] % V == 0;
         for (int d = 0; d + 1 < r.red_n; d++) vec = vec && r.red_stride[d] % V == 0;
+        // few long rows (sum_all of a large tensor is one row): a wavefront per row would leave the chip idle
+        const long cus = ctx->props.multiProcessorCount;
+        const long inner = r.red_shape[r.red_n - 1];
+        if (r.n_out < 2 * cus && inner >= 16384 && r.n_out <= 0x7FFFFFFFL) {
+            typedef typename E::acc A;
+            long chunks = (4 * cus + r.n_out - 1) / r.n_out;
+            if (chunks > inner / 4096) chunks = inner / 4096;  // at least 4096 entries per chunk
+            if (chunks > 65535) chunks = 65535;
+            if (chunks >= 2) {
+                long per_chunk = (inner + chunks - 1) / chunks;
+                per_chunk = (per_chunk + 63) / 64 * 64;  // chunks start on vector boundaries
+                chunks = (inner + per_chunk - 1) / per_chunk;
+                int rc = ensure_workspace(ctx, (size_t)chunks * r.n_out * sizeof(A));
+                if (rc != HODU_ROCM_OK) return rc;
+                A *partial = (A *)ctx->workspace.ptr;
+                if (vec) {
+                    ctx->last_kernel = "sum_row_chunks_vec";
+                    hipLaunchKernelGGL((sum_row_chunks_kernel<E, V>), dim3((unsigned)r.n_out, (unsigned)chunks), dim3(256), 0,
+                                       ctx->stream, (const S *)in, partial, r, per_chunk);
+                } else {
+                    ctx->last_kernel = "sum_row_chunks";
+                    hipLaunchKernelGGL((sum_row_chunks_kernel<E, 1>), dim3((unsigned)r.n_out, (unsigned)chunks), dim3(256), 0,
+                                       ctx->stream, (const S *)in, partial, r, per_chunk);
+                }
+                HODU_HIP(hipGetLastError());
+                hipLaunchKernelGGL(sum_finish_kernel<E>, dim3((unsigned)((r.n_out + 63) / 64)), dim3(256), 0, ctx->stream,
+                                   (const A *)partial, (S *)out, r.n_out, (int)chunks);
+                HODU_HIP(hipGetLastError());
+                return HODU_ROCM_OK;
+            }
+        }
         if (vec) {
             ctx->last_kernel = "sum_by_row_vec";
             hipLaunchKernelGGL((sum_by_row_kernel<E, V>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, r);
@@ -294,6 +400,51 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
 }
 
 }  // namespace
+
+namespace {
+template <class E> int run_inner(hodu_rocm_ctx *ctx, const void *a_v, const void *b_v, void *out, long K, long a_k, long b_k,
+                                 long a_off, long b_off) {
+    typedef typename E::storage S;
+    typedef typename E::acc A;
+    const S *a = (const S *)a_v + a_off, *b = (const S *)b_v + b_off;
+    const long cus = ctx->props.multiProcessorCount;
+    long chunks = 4 * cus;
+    if (chunks > K / 4096) chunks = K / 4096;
+    if (chunks < 1) chunks = 1;
+    long per_chunk = (K + chunks - 1) / chunks;
+    per_chunk = (per_chunk + 63) / 64 * 64;
+    chunks = (K + per_chunk - 1) / per_chunk;
+    int rc = ensure_workspace(ctx, (size_t)chunks * sizeof(A));
+    if (rc != HODU_ROCM_OK) return rc;
+    A *partial = (A *)ctx->workspace.ptr;
+    constexpr int V = 16 / (int)sizeof(S);
+    const bool vec = V > 1 && a_k == 1 && b_k == 1 && (uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0;
+    if (vec) {
+        ctx->last_kernel = "inner_product_vec";
+        hipLaunchKernelGGL((inner_product_kernel<E, V>), dim3((unsigned)chunks), dim3(256), 0, ctx->stream, a, b, partial, K, a_k, b_k, per_chunk);
+    } else {
+        ctx->last_kernel = "inner_product";
+        hipLaunchKernelGGL((inner_product_kernel<E, 1>), dim3((unsigned)chunks), dim3(256), 0, ctx->stream, a, b, partial, K, a_k, b_k, per_chunk);
+    }
+    HODU_HIP(hipGetLastError());
+    hipLaunchKernelGGL(sum_finish_kernel<E>, dim3(1), dim3(256), 0, ctx->stream, (const A *)partial, (S *)out, 1L, (int)chunks);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+}  // namespace
+
+// [1, K] x [K, 1] with a long K: returns HODU_ROCM_UNSUPPORTED (no error text) for anything else
+int launch_inner_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
+    if (kind != PK_SAME || g.M != 1 || g.N != 1 || g.batches != 1 || g.K < 16384 || g.epi.n != 0) return HODU_ROCM_UNSUPPORTED;
+    switch (dtype) {
+#define CASE(ID) case ID: return run_inner<Elem<ID>>(ctx, a, b, c, g.K, g.a_k, g.b_k, g.a_off, g.b_off);
+        CASE(HODU_F8E4M3) CASE(HODU_F8E5M2) CASE(HODU_BF16) CASE(HODU_F16) CASE(HODU_F32) CASE(HODU_F64)
+        CASE(HODU_U8) CASE(HODU_U16) CASE(HODU_U32) CASE(HODU_U64) CASE(HODU_I8) CASE(HODU_I16) CASE(HODU_I32)
+        CASE(HODU_I64)
+#undef CASE
+    default: return HODU_ROCM_UNSUPPORTED;
+    }
+}
 
 int launch_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r) {
     switch (dtype) {

@@ -85,6 +85,8 @@ def check_product(ctx, op, name, lv, rv, seed=0, scale=1.0, rscale=None, expect_
         assert np.all(err <= step * np.abs(want[fin]) + tiny + 1e-3 * oabs[fin] / np.sqrt(k)), f"{op} {name}"
         return
     tol = FLOAT_TOL[out_dt]
-    want = o64 if out_dt == "f64" else o32.astype(np.float64)
+    # (a sequential f32 sum over more than a few thousand k is itself off by about sqrt(k) * 2^-24 relative to the
+    # floor: products with a very long K, which the device adds in chunks, are held to the float64 value)
+    want = o64 if (out_dt == "f64" or (out_dt == "f32" and k > 16384)) else o32.astype(np.float64)
     rel = H.rel_err(gotf[fin], want[fin], oabs[fin], k)
     assert rel.size == 0 or rel.max() <= tol, f"{op} {name}: max rel err {rel.max():.3e} > {tol}"

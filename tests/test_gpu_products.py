@@ -88,6 +88,18 @@ def test_integer_golden_fixtures_bit_exact(ctx):
     assert n >= 40
 
 
+@pytest.mark.parametrize("dt", ffi.PRODUCT_DTYPES)
+def test_product_of_two_long_vectors(ctx, dt):
+    """[1, K] x [K, 1] (what Tensor::matmul makes of two 1-D tensors): K is cut into chunks across workgroups; dense
+    and strided vectors, a K that leaves a ragged last chunk"""
+    scale = 0.25 if dt in ("f8e4m3", "f8e5m2") else 1.0
+    check_product(ctx, "dot", dt, V([1, 1 << 17]), V([1 << 17, 1]), seed=1, scale=scale, expect_kernel="inner_product_vec")
+    check_product(ctx, "dot", dt, V([1, 100003]), V([100003, 1]), seed=2, scale=scale, expect_kernel="inner_product")
+    check_product(ctx, "dot", dt, V([1, 40000], [0, 2]), V([40000, 1], [3, 0]), seed=3, scale=scale, expect_kernel="inner_product")
+    check_product(ctx, "dot", dt, V([1, 9000]), V([9000, 1]), seed=4, scale=scale)  # short: the other kernels
+    assert not ctx.last_kernel().startswith("inner_product")
+
+
 def test_inputs_may_alias_each_other(ctx):
     # a.matmul(a.t()) : lhs and rhs are views of one buffer
     lv = V([24, 40]); rv = lv.t()
