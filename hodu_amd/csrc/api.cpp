@@ -13,9 +13,31 @@ int check_ptrs(const char *op, hodu_rocm_ctx *ctx, const void *a, const void *b,
     return HODU_ROCM_OK;
 }
 
+// the bandwidth-bound families for few rows on the left
+int dispatch_few_rows(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
+    int rc = launch_inner_product(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    rc = launch_gemv(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    rc = launch_skinny(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    return launch_gemv_rows(ctx, kind, dtype, a, b, c, g);
+}
+
 // Picks the kernel family for one launch-sized product.
 int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                  const DevProduct &g) {
+    // A matrix times a vector, [M, K] x [K, 1] (what Tensor::matmul makes of a 2-D and a 1-D tensor,
+    // crates/hodu_core/src/tensor/ops/matrix.rs:50-66), is the transposed problem of one row against the matrix as
+    // the weight, [1, K] x [K, M], and the [M, 1] output is the same memory as [1, M]: the few-rows kernels take it.
+    if (g.N == 1 && g.M > 1 && g.batches == 1 && kind == PK_SAME && g.epi.n == 0 && ctx->force_tile < 0) {
+        DevProduct t = g;
+        t.M = 1; t.N = g.M;
+        t.a_m = g.b_n; t.a_k = g.b_k; t.a_off = g.b_off;
+        t.b_k = g.a_k; t.b_n = g.a_m; t.b_off = g.a_off;
+        const int rc = dispatch_few_rows(ctx, kind, dtype, b, a, c, t);
+        if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    }
     int rc = ctx->force_tile >= 0 ? HODU_ROCM_UNSUPPORTED : launch_inner_product(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     rc = ctx->force_tile == 30 ? HODU_ROCM_UNSUPPORTED : launch_gemv(ctx, kind, dtype, a, b, c, g);

@@ -100,6 +100,17 @@ def test_product_of_two_long_vectors(ctx, dt):
     assert not ctx.last_kernel().startswith("inner_product")
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+def test_matrix_times_vector(ctx, dt):
+    """[M, K] x [K, 1] (Tensor::matmul of a 2-D and a 1-D tensor) runs as the transposed one-row product"""
+    check_product(ctx, "dot", dt, V([300, 1040]), V([1040, 1]), seed=1)
+    assert ctx.last_kernel().startswith(("gemv_", "skinny_")), ctx.last_kernel()
+    check_product(ctx, "dot", dt, V([1040, 300]).t(), V([1040, 1]), seed=2)          # the matrix row-dense in K
+    assert ctx.last_kernel().startswith(("gemv_rows_", "mfma_")), ctx.last_kernel()
+    check_product(ctx, "dot", dt, V([64, 512], offset=8), V([512, 1], [3, 0]), seed=3)  # a strided vector: other kernels
+    check_product(ctx, "dot", dt, V([2, 70000]), V([70000, 1]), seed=4)
+
+
 def test_inputs_may_alias_each_other(ctx):
     # a.matmul(a.t()) : lhs and rhs are views of one buffer
     lv = V([24, 40]); rv = lv.t()
