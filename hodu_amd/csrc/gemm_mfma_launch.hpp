@@ -21,12 +21,27 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     constexpr int ROWVEC = ES == 4 ? 4 : 8;
     const int la = pick_mode(a, g.a_off, g.a_m, g.a_k, g.M, g.K, SA, EPC, ROWVEC, g, g.a_bs);
     const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, SB, EPC, ROWVEC, g, g.b_bs);
-    if (la == LM_SCALAR || lb == LM_SCALAR) {
-        ctx->last_kernel = names[16];
-        return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_SCALAR>>(ctx, a, b, c, g);
-    }
     const long cus = ctx->props.multiProcessorCount;
     auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
+    if (la == LM_SCALAR || lb == LM_SCALAR) {
+        // an operand whose rows or columns do not start on vector boundaries is loaded element by element; the other
+        // one keeps its vector loads (a [K, 2] right operand must not slow down the [M, K] matrix beside it)
+        const int gs = pick_splits(tiles(64, 64), cus, (int)(((long)g.K * ES + 127) / 128), g.batches * (long)g.M * g.N,
+                                   ctx->force_splits);
+        if (gs > 1) {
+            snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_splitk%d", names[16], gs);
+            ctx->last_kernel = ctx->kernel_name;
+        } else {
+            ctx->last_kernel = names[16];
+        }
+        if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
+            if (la == LM_K) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_K, LM_SCALAR>>(ctx, a, b, c, g, gs);
+            if (la == LM_MN) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_MN, LM_SCALAR>>(ctx, a, b, c, g, gs);
+            if (lb == LM_K) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_K>>(ctx, a, b, c, g, gs);
+            if (lb == LM_MN) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_MN>>(ctx, a, b, c, g, gs);
+        }
+        return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_SCALAR>>(ctx, a, b, c, g, gs);
+    }
     // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64
     const int forced = ctx->force_tile;
     int size = forced >= 0 ? forced % 10 : tiles(256, 256) >= cus ? 0 : tiles(128, 128) >= cus ? 2 : 3;
