@@ -17,6 +17,8 @@
 //       LM_MN     the row dim (m of lhs / n of rhs) is dense: loads along the rows for 8 (16-bit
 //                 and 8-bit types) or 4 (f32) consecutive k, transposed in registers with
 //                 v_perm_b32 on the way to LDS -- a transposed view costs no extra HBM traffic
+//       LM_MNU    the row dim is dense but its vectors are not 16-byte aligned, or the row count is no whole
+//                 number of vectors (a [K, N] weight with an odd N): the LM_MN scheme with unaligned loads
 //       LM_SCALAR anything else (odd strides, misaligned, ragged K): element loads with bounds
 //     f8e4m3 storage is widened to bf16 in registers between the global load and the LDS store
 //     (v_cvt_pk_f32_fp8 + v_perm_b32; exact, since e4m3 has 3 mantissa bits), so the weight is
@@ -34,7 +36,7 @@ namespace mfma {
 
 enum { CK_BF16 = 0, CK_F16 = 1, CK_I8 = 2, CK_F32 = 3 };  // compute kind (type held in LDS / fed to MFMA)
 enum { SK_SAME = 0, SK_F8 = 1 };                         // operand storage: compute type, or f8e4m3 -> bf16
-enum { LM_K = 0, LM_MN = 1, LM_SCALAR = 2 };
+enum { LM_K = 0, LM_MN = 1, LM_SCALAR = 2, LM_MNU = 3 };
 enum { OUT_BF16 = 0, OUT_F16 = 1, OUT_F32 = 2, OUT_I32 = 3 };
 
 constexpr int ROW_BYTES = 128;   // bytes of compute type per LDS row per K step
@@ -157,6 +159,9 @@ struct Operand {
 __device__ __forceinline__ u32x4_t zero4() { return u32x4_t{0u, 0u, 0u, 0u}; }
 __device__ __forceinline__ u32x4_t ldg128(const char *p) { return *reinterpret_cast<const u32x4_t *>(p); }
 __device__ __forceinline__ u32x2_t ldg64(const char *p) { return *reinterpret_cast<const u32x2_t *>(p); }
+// 16 bytes from an address that is only known to be a multiple of 2 (one 16-byte load all the same)
+typedef u32x4_t __attribute__((aligned(2))) u32x4_elem_aligned_t;
+__device__ __forceinline__ u32x4_t ldg128_elem_aligned(const char *p) { return *reinterpret_cast<const u32x4_elem_aligned_t *>(p); }
 __device__ __forceinline__ void lds_put(char *lds, int off, const u32x4_t &v) { *reinterpret_cast<u32x4_t *>(lds + off) = v; }
 __device__ __forceinline__ u32x4_t lds_get(const char *lds, int off) { return *reinterpret_cast<const u32x4_t *>(lds + off); }
 
@@ -422,6 +427,55 @@ template <> struct ScalarFetch<SK_F8, CK_BF16> {
     }
 };
 
+// ---- row-dense, unaligned: the registers, the transpose and the LDS layout of LM_MN; every vector is fetched at
+// whatever alignment it has (the hardware takes unaligned vector loads).  A vector of the last row group may reach
+// past the row's end: the extra lanes belong to rows that do not exist and are never stored, so that is harmless as
+// long as the bytes are inside the operand -- the next k-row's.  Where they would not be (the last k-row, or k-rows
+// closer together than a vector) the vector is put together element by element.
+template <class V> __device__ __forceinline__ V ldg_elem_aligned(const char *p) {
+    typedef V __attribute__((aligned(1))) unaligned_t;
+    return *reinterpret_cast<const unaligned_t *>(p);
+}
+template <int SK, int CK, int ROWS, int NT> struct Loader<LM_MNU, SK, CK, ROWS, NT> : Loader<LM_MN, SK, CK, ROWS, NT> {
+    typedef Loader<LM_MN, SK, CK, ROWS, NT> Base;
+    typedef RowDense<SK, CK> RD;
+    static constexpr int RG = RD::RG, VK = RD::VK, SES = RD::SES, GROUPS = Base::GROUPS, UNITS = Base::UNITS;
+    static __device__ __forceinline__ typename RD::vec_t fetch(const Operand &op, int k, int row) {
+        if (row >= op.rows) row = 0;  // a group of the tile's overhang: any readable rows will do
+        const char *p = op.base + ((long)k * op.k_stride + row) * SES;
+        const bool past_end = row + RG > op.rows && (k == op.K - 1 || op.k_stride < RG);
+        if (!past_end) return ldg_elem_aligned<typename RD::vec_t>(p);
+        union { typename RD::vec_t v; unsigned char b[sizeof(typename RD::vec_t)]; } u;
+        u.v = RD::zero();
+        for (int e = 0; e < RG; e++)
+            if (row + e < op.rows)
+                for (int i = 0; i < SES; i++) u.b[e * SES + i] = (unsigned char)p[e * SES + i];
+        return u.v;
+    }
+    __device__ __forceinline__ void issue_full(const Operand &op, int row0, int k0, int tid, char *) {
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const int id = tid + u * NT;
+            const int rg = id % GROUPS, kc = (id / GROUPS) % CHUNKS;
+#pragma unroll
+            for (int j = 0; j < VK; j++) this->r[u][j] = fetch(op, k0 + kc * VK + j, row0 + rg * RG);
+        }
+    }
+    __device__ __forceinline__ void tail(const Operand &op, int row0, int k0, int tid, char *dst) {
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const int id = tid + u * NT;
+            const int rg = id % GROUPS, kc = (id / GROUPS) % CHUNKS;
+#pragma unroll
+            for (int j = 0; j < VK; j++) {
+                const int k = k0 + kc * VK + j;
+                this->r[u][j] = k < op.K ? fetch(op, k, row0 + rg * RG) : RD::zero();
+            }
+        }
+        this->commit_full(dst, tid);
+    }
+};
+
 template <int SK, int CK, int ROWS, int NT> struct Loader<LM_SCALAR, SK, CK, ROWS, NT> {
     static constexpr int ES = Compute<CK>::ES, EPC = 16 / ES;
     static constexpr int UNITS = ROWS * CHUNKS / NT;
@@ -434,6 +488,15 @@ template <int SK, int CK, int ROWS, int NT> struct Loader<LM_SCALAR, SK, CK, ROW
             const int c = tid + u * NT, row = c >> 3, kc = c & 7;
             const int grow = row0 + row;
             uint32_t w[4] = {0u, 0u, 0u, 0u};
+            if constexpr (SK == SK_SAME) {
+                // a k-dense row whose chunk lies inside K: one 16-byte load at whatever alignment the row has (the
+                // hardware takes unaligned vector loads; only their element alignment is guaranteed here).  This is
+                // the case of an odd K or row stride -- a [.., 197, 197] score matrix, K = 4100.
+                if (grow < op.rows && op.k_stride == 1 && k0 + kc * EPC + EPC <= op.K) {
+                    r[u] = ldg128_elem_aligned(op.base + ((long)grow * op.row_stride + k0 + kc * EPC) * ES);
+                    continue;
+                }
+            }
             if (grow < op.rows) {
 #pragma unroll
                 for (int e = 0; e < EPC; e++) {
@@ -753,6 +816,8 @@ inline int pick_mode(const void *base, long off, long row_stride, long k_stride,
         return LM_K;
     if ((row_stride == 1 || rows == 1) && rows % rowvec == 0 && addr % rbytes == 0 && (K == 1 || aligned(k_stride, rbytes)) && batch_r)
         return LM_MN;
+    // row-dense without the alignment (storage type = compute type only; k-rows must not overlap)
+    if (row_stride == 1 && rows > 1 && ses * epc == 16 && (K == 1 || k_stride >= rows)) return LM_MNU;
     return LM_SCALAR;
 }
 

@@ -1,6 +1,8 @@
 // Variant selection and launch for one compute kind of the MFMA tile kernels.
 #pragma once
 
+#include <cstring>
+
 #include "gemm_mfma.hpp"
 #include "gemm_mfma_pipe.hpp"
 
@@ -23,23 +25,38 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, SB, EPC, ROWVEC, g, g.b_bs);
     const long cus = ctx->props.multiProcessorCount;
     auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
-    if (la == LM_SCALAR || lb == LM_SCALAR) {
+    if (la >= LM_SCALAR || lb >= LM_SCALAR) {
         // an operand whose rows or columns do not start on vector boundaries is loaded element by element; the other
         // one keeps its vector loads (a [K, 2] right operand must not slow down the [M, K] matrix beside it)
         const int gs = pick_splits(tiles(64, 64), cus, (int)(((long)g.K * ES + 127) / 128), g.batches * (long)g.M * g.N,
                                    ctx->force_splits);
-        if (gs > 1) {
+        // large products: 128 x 128 tiles (a quarter of the LDS traffic per flop), where they fill the chip
+        const bool big = SKA == SK_SAME && SKB == SK_SAME && ctx->force_tile < 0 && g.M >= 256 && g.N >= 256 &&
+                         tiles(128, 128) >= cus;
+        if (big) {  // "<prefix>_64x64_scalar" -> "<prefix>_128x128_scalar"
+            const char *cut = strstr(names[16], "_64x64_scalar");
+            snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%.*s_128x128_scalar", (int)(cut ? cut - names[16] : 0), names[16]);
+            ctx->last_kernel = ctx->kernel_name;
+        } else if (gs > 1) {
             snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_splitk%d", names[16], gs);
             ctx->last_kernel = ctx->kernel_name;
         } else {
             ctx->last_kernel = names[16];
         }
         if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
-            if (la == LM_K) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_K, LM_SCALAR>>(ctx, a, b, c, g, gs);
-            if (la == LM_MN) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_MN, LM_SCALAR>>(ctx, a, b, c, g, gs);
-            if (lb == LM_K) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_K>>(ctx, a, b, c, g, gs);
-            if (lb == LM_MN) return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_MN>>(ctx, a, b, c, g, gs);
+#define HODU_IRREGULAR(LA, LB)                                                                                         \
+    if (la == LA && lb == LB) {                                                                                        \
+        if (big) return launch_config<Config<CK, SKA, SKB, OUT, 128, 128, 2, 2, LA, LB>>(ctx, a, b, c, g, 1);           \
+        return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LA, LB>>(ctx, a, b, c, g, gs);                     \
+    }
+            HODU_IRREGULAR(LM_K, LM_SCALAR) HODU_IRREGULAR(LM_MN, LM_SCALAR) HODU_IRREGULAR(LM_MNU, LM_SCALAR)
+            HODU_IRREGULAR(LM_SCALAR, LM_K) HODU_IRREGULAR(LM_SCALAR, LM_MN) HODU_IRREGULAR(LM_SCALAR, LM_MNU)
+            HODU_IRREGULAR(LM_K, LM_MNU) HODU_IRREGULAR(LM_MN, LM_MNU) HODU_IRREGULAR(LM_MNU, LM_K)
+            HODU_IRREGULAR(LM_MNU, LM_MN) HODU_IRREGULAR(LM_MNU, LM_MNU)
+            HODU_IRREGULAR(LM_SCALAR, LM_SCALAR)
+#undef HODU_IRREGULAR
         }
+        // (f8e4m3 weight bytes: element loads for both)
         return launch_config<Config<CK, SKA, SKB, OUT, 64, 64, 2, 2, LM_SCALAR, LM_SCALAR>>(ctx, a, b, c, g, gs);
     }
     // size: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4 wavefronts, 2 = 128x128, 3 = 64x64

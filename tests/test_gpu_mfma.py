@@ -135,6 +135,36 @@ def test_scalar_load_variant(ctx, kind):
                   expect_kernel=f"{prefix}_64x64_scalar")
 
 
+@pytest.mark.parametrize("kind", ["bf16", "f16", "f32", "i32_i8i8"])
+def test_unaligned_operands(ctx, kind):
+    """operands whose vectors do not start on 16-byte boundaries: k-dense rows with an odd K or stride or offset (one
+    unaligned vector load per chunk), row-dense operands with an odd row count or offset (the row-dense scheme with
+    unaligned loads and a guarded last vector), both at once, tiny and degenerate extents"""
+    cases = [
+        (V([70, 197]), V([67, 197]).t()),                         # odd K, both k-dense
+        (V([3, 40, 100], offset=1), V([3, 50, 100], offset=3).t()),   # misaligned bases, batched
+        (V([70, 96]), V([96, 67])),                               # right operand row-dense, odd N
+        (V([70, 96]), V([96, 67], offset=1)),
+        (V([96, 71]).t(), V([96, 67])),                           # both row-dense and odd
+        (V([96, 71]).t(), V([61, 96]).t()),                       # left row-dense odd, right k-dense
+        (V([33, 101]), V([101, 3])),                              # fewer columns than one vector holds
+        (V([5, 1]), V([1, 13])),                                  # K = 1
+        (V([64, 200]), V([200, 500]).slice(1, 3, 260)),           # a column slice: row pitch 500, 257 columns
+        (V([2, 45, 130]), V([130, 75]).broadcast_to([2, 130, 75])),
+    ]
+    for n, (lv, rv) in enumerate(cases):
+        check_product(ctx, "matmul" if len(lv.shape) > 2 else "dot", kind, lv, rv, seed=n, expect_kernel="mfma_")
+        assert "scalar" in ctx.last_kernel(), ctx.last_kernel()
+    # large enough for several K steps and workgroups, at the sizes the paths were written for
+    check_product(ctx, "matmul", kind, V([2, 3, 197, 197]), V([2, 3, 197, 64]), seed=20)
+    check_product(ctx, "dot", kind, V([300, 520]), V([520, 1031]), seed=21)
+    # enough 128 x 128 tiles to fill the chip: the large-tile variant of the same loaders
+    check_product(ctx, "dot", kind, V([2048, 264]), V([264, 2051]), seed=22, expect_kernel="mfma_")
+    assert ctx.last_kernel().endswith("_128x128_scalar"), ctx.last_kernel()
+    check_product(ctx, "dot", kind, V([2049, 197]), V([2048, 197]).t(), seed=23, expect_kernel="mfma_")
+    assert ctx.last_kernel().endswith("_128x128_scalar"), ctx.last_kernel()
+
+
 @pytest.mark.parametrize("kind", list(KINDS))
 def test_batched_and_broadcast(ctx, kind):
     prefix, _, _ = KINDS[kind]
