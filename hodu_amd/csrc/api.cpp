@@ -420,11 +420,15 @@ int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, 
     const size_t nd = md[0], out_nd = md[2 + 2 * nd], n_red = md[3 + 2 * nd + out_nd];
     if (n_red != 1) return fail(HODU_ROCM_INVALID_ARG, "softmax: exactly one dim, got %zu", n_red);
     const size_t dim = md[4 + 2 * nd + out_nd];
+    if (dim >= nd) return fail(HODU_ROCM_INVALID_ARG, "softmax: dim %zu of a %zu-d tensor", dim, nd);
     const bool last = dim + 1 == nd;
     if (causal && (!last || nd < 2)) return fail(HODU_ROCM_INVALID_ARG, "softmax: the causal mask needs the last dim of a matrix");
+    long inner = 1;  // extents after the softmax dim
+    for (size_t d = dim + 1; d < nd; d++) inner *= (long)md[1 + d];
+    if (inner == 0) return HODU_ROCM_OK;
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
-    return launch_softmax(ctx, dtype, in, out, r, last, causal ? 1 : 0, nd >= 2 ? (long)md[1 + nd - 2] : 1);
+    return launch_softmax(ctx, dtype, in, out, r, inner, causal ? 1 : 0, nd >= 2 ? (long)md[1 + nd - 2] : 1);
 }
 
 int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,

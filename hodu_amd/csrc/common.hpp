@@ -187,7 +187,7 @@ int parse_reduce_metadata(const size_t *md, size_t len, Reduction *r);
 int launch_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r);
 // softmax over the one reduced dim of `r`; dim_is_last: it is the tensor's last dim; causal: entries j > i of every
 // [sq, len] matrix count as -inf
-int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, bool dim_is_last,
+int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, long inner,
                    int causal, long sq);
 
 // One fused attention call: q [batch.., sq, d], k and v [batch.., sk, d] (batch dims already broadcast, last dim

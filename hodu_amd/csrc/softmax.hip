@@ -7,7 +7,7 @@
 // Here a row is read once: a wavefront owns a row whose dim is dense and at most 4096 long and keeps it in
 // registers (max, exp, sum, scale without touching memory again); a longer dense row belongs to a workgroup, which
 // reads it twice (an online maximum / sum pass, then the pass that writes); strided rows take three passes from
-// memory with a thread per row.  Arithmetic: elements widened exactly to f32 (f64 stays f64), exp and the sum in that
+// memory with a thread per row; a dim other than the last one gets a thread per position of the other dims.  Arithmetic: elements widened exactly to f32 (f64 stays f64), exp and the sum in that
 // type, one rounding (RNE) on store.  With `causal` the entries j > i of each [Sq, Sk] matrix count as -inf: they
 // come out as exact zeros, and the mask tensor is never built.
 #include "common.hpp"
@@ -26,6 +26,7 @@ struct DevSoftmax {
     long kept_shape[16], kept_stride[16];
     int causal;        // 1: mask j > i, i = the row's index along the innermost kept dim (extent sq)
     long sq;
+    long inner;        // product of the extents after the softmax dim (1: it is the last dim)
 };
 
 __device__ __forceinline__ long row_offset(const DevSoftmax &s, long row) {
@@ -214,6 +215,31 @@ __global__ __launch_bounds__(256) void softmax_long_kernel(const typename E::sto
     }
 }
 
+// softmax along a dim that is not the last one: a thread per kept position (neighbouring threads are neighbouring
+// positions of the dims after the softmax dim, so their loads and stores are neighbours in memory), two passes: an
+// online maximum / sum over the dim, then the pass that writes.  The output is contiguous in the input's shape:
+// position (outer, j, inner) at (outer * len + j) * inner_extent + inner.
+template <class E>
+__global__ __launch_bounds__(256) void softmax_cols_kernel(const typename E::storage *__restrict__ in,
+                                                          typename E::storage *__restrict__ out, DevSoftmax s) {
+    typedef typename E::acc W;
+    const long row = (long)blockIdx.x * 256 + threadIdx.x;
+    if (row >= s.rows) return;
+    const typename E::storage *x = in + s.offset + row_offset(s, row);
+    W m = -(W)INFINITY, l = (W)0;
+    for (long j = 0; j < s.len; j++) {
+        const W v = (W)E::load(x[j * s.stride]);
+        if (v > m) {
+            l *= wexp<W>(m - v);  // exp(-inf) = 0 on the first entry
+            m = v;
+        }
+        if (m != -(W)INFINITY) l += wexp<W>(v - m);
+    }
+    const W inv = (W)1 / l;
+    typename E::storage *y = out + (row / s.inner) * s.len * s.inner + row % s.inner;
+    for (long j = 0; j < s.len; j++) y[j * s.inner] = E::store(wexp<W>((W)E::load(x[j * s.stride]) - m) * inv);
+}
+
 // any stride, any length: a thread per row, three passes from memory
 template <class E>
 __global__ __launch_bounds__(256) void softmax_strided_kernel(const typename E::storage *__restrict__ in,
@@ -272,7 +298,14 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
         HODU_HIP(hipGetLastError());
         return HODU_ROCM_OK;
     }
-    if (!dim_is_last) return fail(HODU_ROCM_UNSUPPORTED, "softmax: only the last dim is supported");
+    if (!dim_is_last) {
+        const long blocks = (s.rows + 255) / 256;
+        if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "softmax needs %ld workgroups", blocks);
+        ctx->last_kernel = "softmax_cols";
+        hipLaunchKernelGGL(softmax_cols_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out, s);
+        HODU_HIP(hipGetLastError());
+        return HODU_ROCM_OK;
+    }
     if (s.stride == 1 && s.rows <= 0x7FFFFFFFL) {
         constexpr int V = 16 / (int)sizeof(S);
         bool vec = s.len % V == 0 && s.offset % V == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0;
@@ -297,11 +330,13 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
 
 }  // namespace
 
-// r: the reduction over the softmax dim as parsed from reduce_metadata (one reduced dim); last_dim: that dim is
-// the tensor's last; sq: extent of the dim before it (for the causal mask)
-int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, bool dim_is_last,
+// r: the reduction over the softmax dim as parsed from reduce_metadata (one reduced dim); inner: product of the
+// extents after that dim (1: it is the tensor's last); sq: extent of the dim before it (for the causal mask)
+int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, long inner,
                    int causal, long sq) {
+    const bool dim_is_last = inner == 1;
     DevSoftmax s{};
+    s.inner = inner;
     s.rows = r.n_out;
     s.len = r.reduce_size;
     s.stride = r.red_n > 0 ? r.red_stride[0] : 1;

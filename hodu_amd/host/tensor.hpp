@@ -197,12 +197,12 @@ public:
     }
 
     // ---- attention's middle step and the function around it ---------------------------------------------------
-    // tensor/ops/normalization.rs:4-21, one launch instead of five; only the last dim (what attention uses).
-    // causal: the masked_fill(-inf) of attention.rs:40-48 folded in.
+    // tensor/ops/normalization.rs:4-21, one launch instead of five.
+    // causal: the masked_fill(-inf) of attention.rs:40-48 folded in (last dim only).
     Tensor softmax(int dim, bool causal = false) const {
         const size_t d = layout_.axis(dim);
-        if (d + 1 != layout_.ndim())
-            throw Error(ErrorKind::InvalidArgument, "softmax: only the last dim is supported on this device");
+        if (causal && d + 1 != layout_.ndim())
+            throw Error(ErrorKind::InvalidArgument, "softmax: the causal mask applies to the last dim");
         auto out = std::make_shared<RocmStorage>(storage_->call_ops_softmax(layout_, d, causal));
         return Tensor(out, Layout::from_shape(shape()));
     }

@@ -200,7 +200,7 @@ class Tensor:
         return self._wrap(load().hodu_host_matmul_then(self._h, other._h, arr, len(steps), ctypes.byref(out)), out)
 
     def softmax(self, dim: int = -1, causal: bool = False) -> "Tensor":
-        """Tensor::softmax (tensor/ops/normalization.rs:4-21) as one launch; last dim only.  causal: entries j > i of
+        """Tensor::softmax (tensor/ops/normalization.rs:4-21) as one launch.  causal (last dim only): entries j > i of
         every [.., Sq, Sk] matrix are masked first (attention.rs:40-48)"""
         return self._unary(load().hodu_host_softmax, int(dim), int(causal))
 

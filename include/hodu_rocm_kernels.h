@@ -256,8 +256,9 @@ int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, cons
  * storage type after each.  This is the same function as one kernel with one rounding: elements widened to f32 (f64
  * stays f64), exp and sum in that type, RNE on store.  metadata: reduce_metadata (op_metadatas.rs:525-586) of the
  * input layout with the softmax dim as the one reduced dim -- what the reference hands its max / sum kernels; the
- * output is contiguous in the INPUT's shape.  Only the tensor's last dim is supported (dense rows up to 4096 long
- * stay in registers).  causal != 0 treats entries j > i of every [.., Sq, Sk] matrix as -inf before the softmax:
+ * output is contiguous in the INPUT's shape.  Any dim (dense rows of the last dim up to 4096 long stay in registers,
+ * longer ones take two passes; another dim gets a thread per position of the other dims).  causal != 0 (last dim of
+ * a matrix only) treats entries j > i of every [.., Sq, Sk] matrix as -inf before the softmax:
  * scaled_dot_product_attention's masked_fill with create_causal_mask (crates/hodu_nn/src/modules/attention.rs:40-48,
  * :73-86) without building the mask.  dtypes: bf16, f16, f32, f64. */
 int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *metadata,

@@ -435,14 +435,17 @@ def test_attention_bf16_with_cross_lengths():
     assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), 0.25))
 
 
-def test_softmax_of_a_view_and_its_limits():
+def test_softmax_of_a_view_and_along_other_dims():
     x = H.rng(53).standard_normal(6 * 10).astype(np.float32)
     t = from_f32(x, [6, 10])
     a = x.astype(np.float64).reshape(6, 10)
     e = np.exp(a.T - a.T.max(-1, keepdims=True))
     assert np.allclose(f32_of(t.t().softmax(-1)).reshape(10, 6), e / e.sum(-1, keepdims=True), rtol=1e-5)
+    # along the other dim: columns
+    e0 = np.exp(a - a.max(0, keepdims=True))
+    assert np.allclose(f32_of(t.softmax(0)).reshape(6, 10), e0 / e0.sum(0, keepdims=True), rtol=1e-5)
     with pytest.raises(T.HoduError) as err:
-        t.softmax(0)
+        t.softmax(0, True)  # the causal mask belongs to the last dim
     assert err.value.kind == "InvalidArgument"
 
 

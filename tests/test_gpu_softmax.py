@@ -41,8 +41,8 @@ def check_softmax(ctx, dt, v, dim, causal=False, seed=0, scale=3.0, expect_kerne
     assert np.all(got[want == 0.0] == 0.0)  # masked entries
     err = np.abs(got - want)
     assert np.all(err <= TOL[dt] * np.abs(want) + FLOOR[dt]), f"softmax {dt}: max rel err {(err / np.maximum(np.abs(want), FLOOR[dt])).max():.3e}"
-    rows = got.reshape(-1, v.shape[-1]).sum(axis=1)
-    assert np.allclose(rows, 1.0, atol=4 * TOL[dt])
+    sums = got.reshape(v.shape).sum(axis=dim)
+    assert np.allclose(sums, 1.0, atol=4 * TOL[dt])
 
 
 @pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64"])
@@ -92,10 +92,21 @@ def test_large_logits_do_not_overflow(ctx):
     check_softmax(ctx, "bf16", V([8, 300]), 1, seed=51, scale=200.0)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64"])
+def test_other_dims(ctx, dt):
+    """softmax along a dim that is not the last one: a thread per position of the other dims"""
+    check_softmax(ctx, dt, V([8, 8]), 0, seed=80, expect_kernel="softmax_cols")
+    check_softmax(ctx, dt, V([3, 50, 70]), 1, seed=81, expect_kernel="softmax_cols")
+    check_softmax(ctx, dt, V([5, 300, 2, 9]), 1, seed=82, expect_kernel="softmax_cols")
+    check_softmax(ctx, dt, V([1000, 33]), 0, seed=83, scale=20.0, expect_kernel="softmax_cols")
+    check_softmax(ctx, dt, V([4, 6, 40], offset=5).t(0, 2), 1, seed=84, expect_kernel="softmax_cols")   # strided input
+    check_softmax(ctx, dt, V([7, 9, 1]), 1, seed=85, expect_kernel="softmax_row")                        # nothing after it
+
+
 def test_rejected_calls(ctx):
     x, out = ctx.upload(np.zeros(64, np.float32)), ctx.alloc(256)
-    with pytest.raises(ffi.HoduRocmError, match="last dim"):
-        ctx.softmax("f32", x, out, H.reduce_md(V([8, 8]), [0], True))
+    with pytest.raises(ffi.HoduRocmError, match="causal"):
+        ctx.softmax("f32", x, out, H.reduce_md(V([8, 8]), [0], True), causal=True)
     with pytest.raises(ffi.HoduRocmError, match="exactly one dim"):
         ctx.softmax("f32", x, out, H.reduce_md(V([8, 8]), [0, 1], True))
     with pytest.raises(ffi.HoduRocmError, match="causal"):
