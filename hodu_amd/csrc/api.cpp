@@ -458,7 +458,7 @@ int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void
     HODU_HIP(hipSetDevice(ctx->device));
     rc = launch_attention(ctx, dtype, q, k, v, out, a);
     if (rc == HODU_ROCM_UNSUPPORTED)
-        return fail(HODU_ROCM_UNSUPPORTED, "attention: the fused kernel needs head dim 128, at most %d batch dims, 16-byte aligned rows and a positive finite scale",
+        return fail(HODU_ROCM_UNSUPPORTED, "attention: the fused kernel needs head dim 64 or 128, at most %d batch dims, 16-byte aligned rows and a positive finite scale",
                     kKernelBatchDims);
     return rc;
 }

@@ -47,18 +47,23 @@ using mfma::kd_slot;
 using mfma::lds_get;
 using mfma::lds_get_tr;
 
-constexpr int AT_D = 128;        // head dim
 constexpr int AT_BQ = 128;       // query rows per workgroup (4 groups of 32)
 constexpr int AT_BK = 64;        // keys per step (2 halves of 32, one per wavefront of a row group)
 constexpr int AT_NT = 512;       // 8 wavefronts: wave & 3 = row group, wave >> 2 = key half
-constexpr int AT_KSTEPS = AT_D / 16;
-constexpr int AT_K_BYTES = AT_BK * AT_D * 2;  // 16 KB: K block, two halves of [64 rows][128 bytes]
-constexpr int AT_V_BYTES = AT_BK * AT_D * 2;  // 16 KB: V block, [64 keys][256 bytes]
-constexpr int AT_BUF = AT_K_BYTES + AT_V_BYTES;  // one K block and one V block
-// two of them: the next block is written while this one is read.  The same memory carries, at the end, the second
-// key half's (m, l, O) of every row: 4 row groups x 66 floats x 64 lanes
-constexpr int AT_MERGE = 4 * (2 + AT_D / 2) * 64 * 4;
-constexpr int AT_LDS = AT_MERGE > 2 * AT_BUF ? AT_MERGE : 2 * AT_BUF;
+// per head dim D (64 or 128):
+//   K block: D / 64 halves of [64 keys][128 bytes], chunks XOR-swizzled by (key >> 1) & 7;
+//   V block: [64 keys][2 D bytes], chunks XOR-swizzled so that the four key rows one LDS transpose read touches fall
+//   into different banks: by (key & 3) << 2 for 256-byte rows, by ((key >> 1) & 1) << 2 for 128-byte rows (whose keys k and k + 2 would share banks);
+//   two blocks of each: the next is written while this one is read.  The same memory carries, at the end, the
+//   second key half's (m, l, O) of every row: 4 row groups x (2 + D / 2) floats x 64 lanes.
+template <int D> struct AtGeom {
+    static_assert(D == 64 || D == 128, "head dim");
+    static constexpr int KSTEPS = D / 16, OT = D / 32, NP = D / 64;  // MFMA k steps of S, output tiles, DMAs per wavefront
+    static constexpr int K_BYTES = AT_BK * D * 2, V_BYTES = AT_BK * D * 2, ROW = D * 2;
+    static constexpr int MERGE = 4 * (2 + D / 2) * 64 * 4;
+    static constexpr int LDS = MERGE > 2 * (K_BYTES + V_BYTES) ? MERGE : 2 * (K_BYTES + V_BYTES);
+    static __device__ __forceinline__ int vswz(int key) { return D == 128 ? (key & 3) << 2 : ((key >> 1) & 1) << 2; }
+};
 
 struct DevAttention {
     int sq, sk;
@@ -97,12 +102,14 @@ __device__ __forceinline__ float partner(float v) {
     return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
 }
 
-template <int CK>
+template <int CK, int D>
 __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
                                                                const uint16_t *__restrict__ V, uint16_t *__restrict__ O,
                                                                DevAttention a) {
     typedef Compute32<CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
+    typedef AtGeom<D> G;
+    constexpr int AT_D = D, AT_KSTEPS = G::KSTEPS, AT_K_BYTES = G::K_BYTES, AT_V_BYTES = G::V_BYTES;
     extern __shared__ __align__(16) char smem[];
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
 
@@ -133,26 +140,27 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     const int n_blocks = (k_end + AT_BK - 1) / AT_BK;  // >= 1: Sk >= 1
 
     // ---- global -> LDS without registers in between (global_load_lds_dwordx4: a wavefront's 64 lanes fill 1 KB of
-    // consecutive LDS, so the lane that owns an LDS slot fetches the chunk the swizzle puts there).  16 such
-    // instructions per K block and per V block, two of each per wavefront ----
-    const uint16_t *k_src[2], *v_src[2];   // the lane's source in block 0
-    int k_srow[2], v_srow[2];              // its key row within the block
-    unsigned k_dst[2], v_dst[2];           // LDS byte offset of the instruction within the block's buffer
+    // consecutive LDS, so the lane that owns an LDS slot fetches the chunk the swizzle puts there).  D / 8 such
+    // instructions per K block and per V block, D / 64 of each per wavefront ----
+    const uint16_t *k_src[G::NP], *v_src[G::NP];  // the lane's source in block 0
+    int k_srow[G::NP], v_srow[G::NP];             // its key row within the block
+    unsigned k_dst[G::NP], v_dst[G::NP];          // LDS byte offset of the instruction within the block's buffer
 #pragma unroll
-    for (int p = 0; p < 2; p++) {
+    for (int p = 0; p < G::NP; p++) {
         const int i = wave + 8 * p;
-        // K: two halves of [64 rows][128 bytes]; instruction i fills rows (i % 8) * 8 .. + 7 of half i / 8
+        // K: halves of [64 rows][128 bytes]; instruction i fills rows (i % 8) * 8 .. + 7 of half i / 8
         k_srow[p] = (i & 7) * 8 + (lane >> 3);
         k_src[p] = K + ko + (long)k_srow[p] * a.k_row + (i >> 3) * 64 + ((lane & 7) ^ ((k_srow[p] >> 1) & 7)) * 8;
         k_dst[p] = i * 1024;
-        // V: [64 keys][256 bytes]; instruction i fills keys 4 i .. 4 i + 3
-        v_srow[p] = i * 4 + (lane >> 4);
-        v_src[p] = V + vo + (long)v_srow[p] * a.v_row + ((lane & 15) ^ ((v_srow[p] & 3) << 2)) * 8;
+        // V: [64 keys][2 D bytes]; instruction i fills 1024 / (2 D) keys, a lane one 16-byte chunk of one of them
+        constexpr int CPR = G::ROW / 16;  // chunks per key row
+        v_srow[p] = i * (64 / CPR) + lane / CPR;
+        v_src[p] = V + vo + (long)v_srow[p] * a.v_row + ((lane % CPR) ^ G::vswz(v_srow[p])) * 8;
         v_dst[p] = i * 1024;
     }
     auto dma_k = [&](int kb, int buf) {
 #pragma unroll
-        for (int p = 0; p < 2; p++) {
+        for (int p = 0; p < G::NP; p++) {
             int key = kb * AT_BK + k_srow[p];
             key = key < a.sk ? key : a.sk - 1;  // ragged tail: clamped, masked below
             mfma::dma16_raw(reinterpret_cast<const char *>(k_src[p] + (long)(key - k_srow[p]) * a.k_row),
@@ -161,7 +169,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     };
     auto dma_v = [&](int kb, int buf) {
 #pragma unroll
-        for (int p = 0; p < 2; p++) {
+        for (int p = 0; p < G::NP; p++) {
             int key = kb * AT_BK + v_srow[p];
             key = key < a.sk ? key : a.sk - 1;
             mfma::dma16_raw(reinterpret_cast<const char *>(v_src[p] + (long)(key - v_srow[p]) * a.v_row),
@@ -172,14 +180,14 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     auto dma_k_full = [&](int kb, int buf) {
         const long step = (long)kb * AT_BK * a.k_row;
 #pragma unroll
-        for (int p = 0; p < 2; p++)
+        for (int p = 0; p < G::NP; p++)
             mfma::dma16_raw(reinterpret_cast<const char *>(k_src[p] + step),
                             __builtin_amdgcn_readfirstlane(lds0 + buf * AT_K_BYTES + k_dst[p]));
     };
     auto dma_v_full = [&](int kb, int buf) {
         const long step = (long)kb * AT_BK * a.v_row;
 #pragma unroll
-        for (int p = 0; p < 2; p++)
+        for (int p = 0; p < G::NP; p++)
             mfma::dma16_raw(reinterpret_cast<const char *>(v_src[p] + step),
                             __builtin_amdgcn_readfirstlane(lds0 + 2 * AT_K_BYTES + buf * AT_V_BYTES + v_dst[p]));
     };
@@ -216,7 +224,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
 #pragma unroll
         for (int j = 0; j < AT_D / 32; j++) {
             const int bytes = j * 64 + col_bytes, c = bytes >> 4;
-            v_mn[j] = (kh * 32 + lh * 8 + kq) * (AT_D * 2) + ((c ^ (kq << 2)) << 4) + (bytes & 8);
+            v_mn[j] = (kh * 32 + lh * 8 + kq) * (AT_D * 2) + ((c ^ G::vswz(kq)) << 4) + (bytes & 8);
         }
     }
     const int wave_row0 = q0 + qg * 32;  // the wavefront's first query row
@@ -232,7 +240,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     };
 
     // ---- the phases ----
-    auto read_k = [&](u32x4_t (&kf)[AT_KSTEPS], int buf, int from = 0, int to = AT_KSTEPS) {
+    auto read_k = [&](u32x4_t (&kf)[AT_KSTEPS], int buf, int from = 0, int to = G::KSTEPS) {
         const char *k_lds = smem + buf * AT_K_BYTES;
 #pragma unroll
         for (int ks = from; ks < to; ks++) kf[ks] = lds_get(k_lds, k_frag[ks]);
@@ -371,14 +379,15 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
         if (kb + 1 < n_blocks) dma_v_full(kb + 1, 1 - P);
         u32x4_t kf[AT_KSTEPS];
         u32x2_t vf0[AT_D / 32][2], vf1[AT_D / 32][2];
-        read_k(kf, 1 - P, 0, 4);
+        constexpr int HALF = AT_KSTEPS / 2, HEAD = D == 128 ? 3 : 2;  // MFMAs issued ahead of the row maximum
+        read_k(kf, 1 - P, 0, HALF);
         read_v(vf0, P, 0);
         __builtin_amdgcn_sched_barrier(0);
-        read_k(kf, 1 - P, 4, AT_KSTEPS);
+        read_k(kf, 1 - P, HALF, AT_KSTEPS);
         zero(s_out);
-        scores(kf, s_out, 0, 3);
+        scores(kf, s_out, 0, HEAD);
         if (row_max(s_in)) rescale_o();
-        scores(kf, s_out, 3, AT_KSTEPS);
+        scores(kf, s_out, HEAD, AT_KSTEPS);
         float l_blk = 0.f;
         const u32x4_t pf0 = probs(s_in, 0, l_blk);
         read_v(vf1, P, 1);
@@ -471,7 +480,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
 int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
                      const AttentionArgs &g) {
     if (dtype != HODU_BF16 && dtype != HODU_F16) return HODU_ROCM_UNSUPPORTED;
-    if (g.d != AT_D || g.sq < 1 || g.sk < 1 || g.batches < 1) return HODU_ROCM_UNSUPPORTED;
+    if ((g.d != 64 && g.d != 128) || g.sq < 1 || g.sk < 1 || g.batches < 1) return HODU_ROCM_UNSUPPORTED;
     // the row maximum is taken before the scale is applied: the scale must be positive (and finite)
     if (!(g.scale > 0.f) || !(g.scale < INFINITY)) return HODU_ROCM_UNSUPPORTED;
     if (g.nb > kKernelBatchDims) return HODU_ROCM_UNSUPPORTED;
@@ -498,18 +507,21 @@ int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k
     a.q_blocks = (int)((g.sq + AT_BQ - 1) / AT_BQ);
     const long blocks = g.batches * a.q_blocks;
     if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
-    const void *kernel = dtype == HODU_BF16 ? reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_BF16>)
-                                            : reinterpret_cast<const void *>(attention_fwd_kernel<mfma::CK_F16>);
-    if (int rc = ensure_dynamic_lds(ctx, kernel, AT_LDS)) return rc;
-    if (dtype == HODU_BF16) {
-        ctx->last_kernel = "attention_fwd_bf16";
-        hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_BF16>, dim3((unsigned)blocks), dim3(AT_NT), AT_LDS, ctx->stream,
-                           (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, (uint16_t *)out, a);
-    } else {
-        ctx->last_kernel = "attention_fwd_f16";
-        hipLaunchKernelGGL(attention_fwd_kernel<mfma::CK_F16>, dim3((unsigned)blocks), dim3(AT_NT), AT_LDS, ctx->stream,
-                           (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, (uint16_t *)out, a);
-    }
+    auto launch = [&](auto kernel, int lds, const char *name) -> int {
+        if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), lds)) return rc;
+        ctx->last_kernel = name;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(AT_NT), lds, ctx->stream, (const uint16_t *)q, (const uint16_t *)k,
+                           (const uint16_t *)v, (uint16_t *)out, a);
+        return HODU_ROCM_OK;
+    };
+    int rc;
+    if (g.d == 128)
+        rc = dtype == HODU_BF16 ? launch(attention_fwd_kernel<mfma::CK_BF16, 128>, AtGeom<128>::LDS, "attention_fwd_bf16")
+                                : launch(attention_fwd_kernel<mfma::CK_F16, 128>, AtGeom<128>::LDS, "attention_fwd_f16");
+    else
+        rc = dtype == HODU_BF16 ? launch(attention_fwd_kernel<mfma::CK_BF16, 64>, AtGeom<64>::LDS, "attention_fwd_bf16_d64")
+                                : launch(attention_fwd_kernel<mfma::CK_F16, 64>, AtGeom<64>::LDS, "attention_fwd_f16_d64");
+    if (rc != HODU_ROCM_OK) return rc;
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }

@@ -208,7 +208,7 @@ public:
     }
 
     // the whole of scaled_dot_product_attention as one launch, where the fused kernel takes the call (bf16 / f16,
-    // head dim 128, dense aligned rows): *taken says whether it did.  md: hodu_rocm_attention's metadata.
+    // head dim 64 or 128, dense aligned rows): *taken says whether it did.  md: hodu_rocm_attention's metadata.
     RocmStorage call_ops_attention(const RocmStorage &k, const RocmStorage &v, const Layout &ql, const Layout &kl, const Layout &vl,
                                    const Metadata &md, size_t out_elems, const unsigned char scale[8], bool causal,
                                    bool *taken) const {

@@ -245,7 +245,7 @@ public:
 
     // scaled_dot_product_attention (hodu_nn/src/modules/attention.rs:25-70) without attn_mask and dropout:
     // softmax(Q K^T / sqrt(d_k) [+ causal mask]) V.  One launch where the fused kernel applies (bf16 / f16, head dim
-    // 128, dense aligned rows); otherwise three -- the scale rides in the first product's store, the mask and the
+    // 64 or 128, dense aligned rows); otherwise three -- the scale rides in the first product's store, the mask and the
     // five softmax kernels are one kernel, the second product is plain.
     static Tensor scaled_dot_product_attention(const Tensor &q, const Tensor &k, const Tensor &v, bool is_causal) {
         if (q.layout().ndim() < 2) throw Error(ErrorKind::InvalidArgument, "attention: query needs at least two dimensions");

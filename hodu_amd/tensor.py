@@ -277,7 +277,7 @@ def scalar_bits(dtype: str, value: float) -> np.ndarray:
 
 def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False) -> Tensor:
     """hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) without attn_mask and
-    dropout: one launch where the fused kernel applies (bf16 / f16, head dim 128), otherwise three (product with the
+    dropout: one launch where the fused kernel applies (bf16 / f16, head dim 64 or 128), otherwise three (product with the
     scale in its store, masked softmax, product)"""
     out = ctypes.c_void_p()
     rc = load().hodu_host_attention(q._h, k._h, v._h, int(is_causal), ctypes.byref(out))

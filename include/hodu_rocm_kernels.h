@@ -269,7 +269,7 @@ int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, 
  * scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) computes with a batched matmul,
  * mul_scalar, masked_fill, the five softmax kernels and a second batched matmul, without attn_mask and dropout.  The
  * scores never leave the chip: scores and probabilities stay in f32 (the reference rounds them to the storage type
- * after every kernel), the output is rounded once.  Takes bf16 / f16, D = 128, dense head dims, rows / offsets /
+ * after every kernel), the output is rounded once.  Takes bf16 / f16, D = 64 or 128, dense head dims, rows / offsets /
  * batch strides that are multiples of 8 elements, a positive finite scale (the row maximum is taken before the scale
  * is applied); returns HODU_ROCM_UNSUPPORTED otherwise, and the caller runs the
  * three launches (hodu_rocm_matmul_<dt>_ex with MUL_SCALAR, hodu_rocm_softmax, hodu_rocm_matmul_<dt>).

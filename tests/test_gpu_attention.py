@@ -41,10 +41,9 @@ def narrow(dt, x):
     return (H.f32_to_bf16_rne if dt == "bf16" else H.f16_bits)(np.ascontiguousarray(x, dtype=np.float32))
 
 
-def check_attention(ctx, dt, batch, sq, sk, causal, seed=0, qv=None, kv=None, vv=None, vscale=1.0, qscale=1.0, ramp=None):
+def check_attention(ctx, dt, batch, sq, sk, causal, seed=0, qv=None, kv=None, vv=None, vscale=1.0, qscale=1.0, ramp=None, d=128):
     """ramp: logits that grow along the keys (contiguous operands only) -- q rows all point along one direction and
     key j is that direction times ramp * f(j), f rising from 0 to 1 (or falling, ramp < 0), plus noise"""
-    d = 128
     qv = qv or V(list(batch) + [sq, d])
     kv = kv or V(list(batch) + [sk, d])
     vv = vv or V(list(batch) + [sk, d])
@@ -68,7 +67,7 @@ def check_attention(ctx, dt, batch, sq, sk, causal, seed=0, qv=None, kv=None, vv
     dout = ctx.alloc(n_out * 2)
     ctx.fill(dout, 0xFF)
     ctx.attention(dt, dq, dk, dv, dout, attention_md(batch, sq, sk, d, qv, kv, vv), scale_bits, causal)
-    assert ctx.last_kernel().startswith("attention_fwd")
+    assert ctx.last_kernel() == f"attention_fwd_{dt}" + ("_d64" if d == 64 else "")
     got = H.widen(dt, ctx.download(dout, np.uint16, n_out)).reshape(list(batch) + [sq, d])
     for b in (dq, dk, dv, dout):
         b.free()
@@ -122,11 +121,30 @@ def test_maxima_that_keep_moving(ctx, causal):
     check_attention(ctx, "bf16", [2], 128, 640, causal, seed=14, qscale=6.0)    # random logits of std ~ 6
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_head_dim_64(ctx, dt, causal):
+    check_attention(ctx, dt, [2], 128, 128, causal, seed=20, d=64)
+    check_attention(ctx, dt, [3], 77, 203, causal, seed=21, d=64)      # ragged rows and keys
+    check_attention(ctx, dt, [2, 2], 300, 1000, causal, seed=22, d=64)  # many key blocks: the fast loop and its tail
+    check_attention(ctx, dt, [1], 1, 1, causal, seed=23, d=64)
+    check_attention(ctx, dt, [2], 128, 640, causal, seed=24, qscale=6.0, d=64)
+    check_attention(ctx, dt, [1], 200, 777, causal, seed=25, ramp=2.0, d=64)  # the reference maximum keeps moving
+
+
+def test_head_dim_64_strided_views(ctx):
+    sq, sk = 130, 190
+    qv = V([sq, 4, 64], offset=64).t(0, 1)  # [4, sq, 64] with row stride 4 * 64
+    kv = V([sk, 4, 64]).t(0, 1)
+    vv = V([sk, 4, 64], offset=128).t(0, 1)
+    check_attention(ctx, "bf16", [4], sq, sk, True, seed=26, qv=qv, kv=kv, vv=vv, d=64)
+
+
 def test_unsupported_calls_are_refused(ctx):
     q, out = ctx.upload(np.zeros(64 * 64, np.uint16)), ctx.alloc(64 * 64 * 2)
     one = np.array([0x3F80], np.uint16)
-    with pytest.raises(ffi.HoduRocmError, match="head dim 128"):
-        ctx.attention("bf16", q, q, q, out, attention_md([], 64, 64, 64, V([64, 64]), V([64, 64]), V([64, 64])), one)
+    with pytest.raises(ffi.HoduRocmError, match="head dim 64 or 128"):
+        ctx.attention("bf16", q, q, q, out, attention_md([], 64, 64, 32, V([64, 32]), V([64, 32]), V([64, 32])), one)
     with pytest.raises(ffi.HoduRocmError, match="dense"):
         ctx.attention("bf16", q, q, q, out, attention_md([], 8, 8, 128, V([8, 128], [1, 8]), V([8, 128]), V([8, 128])), one)
     with pytest.raises(ffi.HoduRocmError, match="words"):

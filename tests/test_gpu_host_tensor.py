@@ -502,8 +502,8 @@ def test_attention_takes_the_fused_kernel_at_head_dim_128(causal):
     assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), floor))
     # a head dim the kernel does not take goes down the three-launch path, same function
     T.stats(reset=True)
-    q64 = T.Tensor.from_bits(q[:2 * 3 * 72 * 64], "bf16", [2, 3, 72, 64])
-    k64 = T.Tensor.from_bits(k[:90 * 64], "bf16", [90, 64])
-    T.scaled_dot_product_attention(q64, k64, k64, causal)
+    q32 = T.Tensor.from_bits(q[:2 * 3 * 72 * 32], "bf16", [2, 3, 72, 32])
+    k32 = T.Tensor.from_bits(k[:90 * 32], "bf16", [90, 32])
+    T.scaled_dot_product_attention(q32, k32, k32, causal)
     s = T.stats()
     assert s["attention_kernels"] == 0 and s["product_kernels"] == 2 and s["softmax_kernels"] == 1
