@@ -131,8 +131,12 @@ def test_scalar_load_variant(ctx, kind):
     # odd K, odd strides, odd offsets: nothing is vector-loadable
     lv = V([45, 77], offset=1)
     rv = V([77, 2 * 31]).slice(1, 1, 62, 2)
-    check_product(ctx, "dot", kind, lv, rv, seed=3, rscale=2.0 if "f8" in kind else None,
-                  expect_kernel=f"{prefix}_64x64_scalar")
+    ctx.force_tile(3)  # (a small f32 product would go to the kernel that needs no vector loads at all)
+    try:
+        check_product(ctx, "dot", kind, lv, rv, seed=3, rscale=2.0 if "f8" in kind else None,
+                      expect_kernel=f"{prefix}_64x64_scalar")
+    finally:
+        ctx.force_tile(-1)
 
 
 @pytest.mark.parametrize("kind", ["bf16", "f16", "f32", "i32_i8i8"])
@@ -152,9 +156,13 @@ def test_unaligned_operands(ctx, kind):
         (V([64, 200]), V([200, 500]).slice(1, 3, 260)),           # a column slice: row pitch 500, 257 columns
         (V([2, 45, 130]), V([130, 75]).broadcast_to([2, 130, 75])),
     ]
-    for n, (lv, rv) in enumerate(cases):
-        check_product(ctx, "matmul" if len(lv.shape) > 2 else "dot", kind, lv, rv, seed=n, expect_kernel="mfma_")
-        assert "scalar" in ctx.last_kernel(), ctx.last_kernel()
+    ctx.force_tile(3 if kind == "f32" else -1)  # (small f32 products have a kernel of their own: pin the tile kernel)
+    try:
+        for n, (lv, rv) in enumerate(cases):
+            check_product(ctx, "matmul" if len(lv.shape) > 2 else "dot", kind, lv, rv, seed=n, expect_kernel="mfma_")
+            assert "scalar" in ctx.last_kernel(), ctx.last_kernel()
+    finally:
+        ctx.force_tile(-1)
     # large enough for several K steps and workgroups, at the sizes the paths were written for
     check_product(ctx, "matmul", kind, V([2, 3, 197, 197]), V([2, 3, 197, 64]), seed=20)
     check_product(ctx, "dot", kind, V([300, 520]), V([520, 1031]), seed=21)
@@ -169,22 +177,26 @@ def test_unaligned_operands(ctx, kind):
 def test_batched_and_broadcast(ctx, kind):
     prefix, _, _ = KINDS[kind]
     rs = 2.0 if "f8" in kind else None
-    # strided batch on both sides, rhs a transposed view (BASELINE config 2 in small)
-    check_product(ctx, "matmul", kind, V([3, 72, 64]), V([3, 80, 64]).t(), seed=11, rscale=rs, expect_kernel=prefix)
-    # weight shared across the batch (stride 0) and transposed: folds into one tall product
-    check_product(ctx, "matmul", kind, V([4, 40, 96]), V([56, 96]).t().broadcast_to([4, 96, 56]), seed=12, rscale=rs,
-                  expect_kernel=prefix)
-    # 2-D rhs, two batch dims on the lhs
-    check_product(ctx, "matmul", kind, V([2, 3, 24, 32]), V([32, 40]), seed=13, rscale=rs, expect_kernel=prefix)
-    # lhs broadcast over the batch, batched rhs (cannot fold: stays batched with a stride-0 operand)
-    check_product(ctx, "matmul", kind, V([24, 32]).broadcast_to([3, 24, 32]), V([3, 32, 40]), seed=14, rscale=rs,
-                  expect_kernel=prefix)
-    # aligned offsets into larger buffers
-    check_product(ctx, "dot", kind, V([40, 64], offset=64), V([64, 48], offset=128), seed=15, rscale=rs,
-                  expect_kernel=prefix)
-    # row slices: leading dimension larger than the extent
-    check_product(ctx, "dot", kind, V([40, 128]).slice(1, 32, 96), V([64, 96]).slice(1, 16, 64), seed=16, rscale=rs,
-                  expect_kernel=prefix)
+    ctx.force_tile(2 if kind == "f32" else -1)  # (small f32 products have a kernel of their own: pin the tile kernel)
+    try:
+        # strided batch on both sides, rhs a transposed view (BASELINE config 2 in small)
+        check_product(ctx, "matmul", kind, V([3, 72, 64]), V([3, 80, 64]).t(), seed=11, rscale=rs, expect_kernel=prefix)
+        # weight shared across the batch (stride 0) and transposed: folds into one tall product
+        check_product(ctx, "matmul", kind, V([4, 40, 96]), V([56, 96]).t().broadcast_to([4, 96, 56]), seed=12, rscale=rs,
+                      expect_kernel=prefix)
+        # 2-D rhs, two batch dims on the lhs
+        check_product(ctx, "matmul", kind, V([2, 3, 24, 32]), V([32, 40]), seed=13, rscale=rs, expect_kernel=prefix)
+        # lhs broadcast over the batch, batched rhs (cannot fold: stays batched with a stride-0 operand)
+        check_product(ctx, "matmul", kind, V([24, 32]).broadcast_to([3, 24, 32]), V([3, 32, 40]), seed=14, rscale=rs,
+                      expect_kernel=prefix)
+        # aligned offsets into larger buffers
+        check_product(ctx, "dot", kind, V([40, 64], offset=64), V([64, 48], offset=128), seed=15, rscale=rs,
+                      expect_kernel=prefix)
+        # row slices: leading dimension larger than the extent
+        check_product(ctx, "dot", kind, V([40, 128]).slice(1, 32, 96), V([64, 96]).slice(1, 16, 64), seed=16, rscale=rs,
+                      expect_kernel=prefix)
+    finally:
+        ctx.force_tile(-1)
 
 
 def test_deep_k_accumulation(ctx):
@@ -216,7 +228,7 @@ def test_split_k(ctx, kind, splits):
         ctx.force_splitk(-1)
         K = 32 * 128 // es
         check_product(ctx, "dot", kind, V([256, K]), V([384, K]).t(), seed=5, rscale=rs,
-                      expect_kernel=f"{prefix}_pipe128x128_KK_splitk")
+                      expect_kernel="small_f32_KK" if kind == "f32" else f"{prefix}_pipe128x128_KK_splitk")
     finally:
         ctx.force_tile(-1)
         ctx.force_splitk(-1)
