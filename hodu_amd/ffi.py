@@ -220,17 +220,28 @@ class Context:
     def alloc(self, nbytes: int) -> DeviceBuffer:
         return DeviceBuffer(self, nbytes)
 
+    def upload_into(self, buf: DeviceBuffer, host: np.ndarray, first_byte: int = 0):
+        """copy a host array into an existing buffer at a byte offset (large operands are filled piece by piece)"""
+        host = np.ascontiguousarray(host)
+        if first_byte < 0 or first_byte + host.nbytes > buf.nbytes:
+            raise HoduRocmError(INVALID_ARG, "upload_into: the range lies outside the buffer")
+        self._check(self.lib.hodu_rocm_memcpy_h2d(self.handle, buf.ptr + int(first_byte), host.ctypes.data, host.nbytes))
+
     def upload(self, host: np.ndarray) -> DeviceBuffer:
         host = np.ascontiguousarray(host)
         buf = DeviceBuffer(self, host.nbytes)
         self._check(self.lib.hodu_rocm_memcpy_h2d(self.handle, buf.ptr, host.ctypes.data, host.nbytes))
         return buf
 
-    def download(self, buf: DeviceBuffer, dtype, count: Optional[int] = None) -> np.ndarray:
+    def download(self, buf: DeviceBuffer, dtype, count: Optional[int] = None, first: int = 0) -> np.ndarray:
+        """`count` elements of `dtype` starting at element `first` of the buffer (default: all of it)"""
         dtype = np.dtype(dtype)
-        n = buf.nbytes // dtype.itemsize if count is None else int(count)
+        first = int(first)
+        n = buf.nbytes // dtype.itemsize - first if count is None else int(count)
+        if first < 0 or n < 0 or (first + n) * dtype.itemsize > buf.nbytes:
+            raise HoduRocmError(INVALID_ARG, "download: the range lies outside the buffer")
         out = np.empty(n, dtype=dtype)
-        self._check(self.lib.hodu_rocm_memcpy_d2h(self.handle, out.ctypes.data, buf.ptr, out.nbytes))
+        self._check(self.lib.hodu_rocm_memcpy_d2h(self.handle, out.ctypes.data, buf.ptr + first * dtype.itemsize, out.nbytes))
         return out
 
     def fill(self, buf: DeviceBuffer, byte: int):
