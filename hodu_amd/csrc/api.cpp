@@ -50,6 +50,8 @@ int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const v
     }
     rc = launch_small_f32(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    rc = launch_gemm_f64(ctx, kind, dtype, a, b, c, g);
+    if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     rc = launch_mfma(ctx, kind, dtype, a, b, c, g);
     if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     ctx->last_kernel = "generic";

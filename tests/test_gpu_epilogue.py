@@ -91,13 +91,19 @@ SPECS = [LINEAR, [("mul",)], [("relu",)], [("mul",), ("add", 2, 3), ("relu",)], 
 @pytest.mark.parametrize("dt", ffi.EPILOGUE_DTYPES)
 def test_generic_kernel_every_dtype(ctx, dt):
     """column-strided operands: the generic kernel, the tile kernel's scalar-load variant for bf16 / f16, the
-    small-product kernel for f32"""
+    small-product kernel for f32, the f64 matrix-core kernel"""
     lv, rv = V([37, 50]).slice(1, 1, 49, 2), V([24, 70]).slice(1, 0, 70, 2)
-    family = "mfma_" if dt in ("bf16", "f16") else "small_f32" if dt == "f32" else "generic"
+    family = "mfma_" if dt in ("bf16", "f16") else "small_f32" if dt == "f32" else "mfma_f64" if dt == "f64" else "generic"
     for n, spec in enumerate(SPECS):
         if dt not in FLOATS and ("relu",) in spec:
             continue
         check_fused(ctx, "dot", dt, lv, rv, spec, seed=n, expect_kernel=family)
+        if dt == "f64":  # (and the generic kernel, which keeps the f64 products thinner than a matrix-core tile)
+            ctx.force_tile(3)
+            try:
+                check_fused(ctx, "dot", dt, lv, rv, spec, seed=n, expect_kernel="generic")
+            finally:
+                ctx.force_tile(-1)
     check_fused(ctx, "matmul", dt, V([3, 2, 9, 12]), V([12, 7], [1, 12]).broadcast_to([3, 2, 12, 7]), LINEAR, seed=9)
 
 
