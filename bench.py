@@ -33,7 +33,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 # published MI355X peaks (dense)
-PEAK = {"bf16": 2500.0, "f16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}  # TFLOP/s or TOP/s
+PEAK = {"bf16": 2500.0, "f16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3, "f64": 78.6}  # TFLOP/s or TOP/s
 HBM_PEAK_GBS = 8000.0
 INFINITY_CACHE_BYTES = 256 << 20
 
@@ -124,6 +124,12 @@ def build_cases(which):
         cases.append(Case("f8_4096", "f8e4m3 dot 4096^3 (native fp8 MFMA), rhs a transposed view", "dot", "f8e4m3",
                           V([n, n]), V([n, n]).t(), lambda n=n: fp8_weights(601, n * n, top=8.0),
                           lambda n=n: fp8_weights(602, n * n, top=8.0), 2.0 * n ** 3, 3 * n * n, "mfma", "fp8"))
+    if "f64" in which:
+        # not a BASELINE configuration: hodu's f64 dot at 2048^3 on the f64 matrix instruction
+        n = 2048
+        cases.append(Case("f64_2048", "f64 dot 2048^3 (not a BASELINE config)", "dot", "f64", V([n, n]), V([n, n]),
+                          lambda n=n: normal(701, n * n).astype(np.float64), lambda n=n: normal(702, n * n).astype(np.float64),
+                          2.0 * n ** 3, 3 * n * n * 8, "mfma", "f64"))
     if "c4" in which:
         n = 2048
         ints = lambda seed, n=n: np.random.default_rng(seed).integers(-127, 128, n * n).astype(np.int8)  # noqa: E731
@@ -166,7 +172,7 @@ def out_bytes(case):
     import helpers as H
     md = H.dot_md(case.lv, case.rv) if case.op == "dot" else H.matmul_md(case.lv, case.rv)
     n = md[0] * md[2] if case.op == "dot" else md[0]
-    return md, n * {"f32": 4, "bf16": 2, "bf16_f8e4m3w": 2, "i32_i8i8": 4, "f8e4m3": 1}[case.name]
+    return md, n * {"f32": 4, "f64": 8, "bf16": 2, "bf16_f8e4m3w": 2, "i32_i8i8": 4, "f8e4m3": 1}[case.name]
 
 
 def time_case(ctx, case, steps, warmup, graph=False):
@@ -486,7 +492,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,fused,bwd,casts")
+    ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,f64,fused,bwd,casts")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
     ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
