@@ -1,7 +1,8 @@
-// f8e4m3 x f8e4m3 -> f8e4m3 on the 8-bit matrix instruction (gemm_mfma_pipe_f8.hpp): applicability and launch.
+// f8e4m3 x f8e4m3 -> f8e4m3 and f8e5m2 x f8e5m2 -> f8e5m2 on the 8-bit matrix instruction (gemm_mfma_pipe_f8.hpp):
+// applicability and launch.
 #include "gemm_mfma_pipe_f8.hpp"
 namespace hodu {
-int launch_mfma_f8(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
+int launch_mfma_f8(hodu_rocm_ctx *ctx, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
     using namespace mfma;
     // both operands k-dense with every 16-byte chunk aligned, K a whole number of 128-byte stages;
     // anything else stays with the generic kernel
@@ -17,12 +18,18 @@ int launch_mfma_f8(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, co
     int splits = 1;
     if (ctx->force_splits >= 1) splits = pick_splits(1, cus, stages, elems, ctx->force_splits);
     else if (!big) splits = pick_splits(tiles(128, 128), cus, stages, elems, -1);
-    const char *base = big ? "mfma_f8e4m3_pipe256x256_KK" : "mfma_f8e4m3_pipe128x128_KK";
+    const bool e5m2 = dtype == HODU_F8E5M2;
+    const char *base = e5m2 ? (big ? "mfma_f8e5m2_pipe256x256_KK" : "mfma_f8e5m2_pipe128x128_KK")
+                            : (big ? "mfma_f8e4m3_pipe256x256_KK" : "mfma_f8e4m3_pipe128x128_KK");
     if (splits > 1) {
         snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_splitk%d", base, splits);
         ctx->last_kernel = ctx->kernel_name;
     } else {
         ctx->last_kernel = base;
+    }
+    if (e5m2) {
+        if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E5M2, 256, 256>>(ctx, a, b, c, g, splits);
+        return launch_pipe_f8<PipeF8Config<OUT_F8E5M2, 128, 128>>(ctx, a, b, c, g, splits);
     }
     if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 256, 256>>(ctx, a, b, c, g, splits);
     return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 128, 128>>(ctx, a, b, c, g, splits);

@@ -1,9 +1,9 @@
-// f8e4m3 x f8e4m3 products on the native gfx950 8-bit MFMA (v_mfma_scale_f32_32x32x64_f8f6f4 with
-// unit scales: 64 k per instruction, twice the arithmetic of the bf16 instruction for the same
-// operand bytes).  hodu's own f8e4m3 matmul / dot (lhs, rhs and result all f8e4m3;
-// crates/hodu_cpu_kernels/kernels/ops_matrix.c:353, :715) lands here when both operands are k-dense
+// f8e4m3 x f8e4m3 and f8e5m2 x f8e5m2 products on the native gfx950 8-bit MFMA (v_mfma_scale_f32_32x32x64_f8f6f4
+// with unit scales: 64 k per instruction, twice the arithmetic of the bf16 instruction for the same
+// operand bytes; the instruction's format fields select e4m3 or e5m2).  hodu's own f8 matmul / dot (lhs, rhs and
+// result all of one f8 type; crates/hodu_cpu_kernels/kernels/ops_matrix.c:353-354, :715-716) lands here when both operands are k-dense
 // and K is a multiple of 128; products accumulate in f32 and are narrowed once, round-to-nearest-even
-// and saturating at +-448 like every other f8e4m3 product of this library (the reference re-rounds
+// and saturating at +-448 (e5m2: +-57344) like every other f8 product of this library (the reference re-rounds
 // its f8 accumulator after every k, ops_matrix.c:572-573).
 //
 // Same feeding scheme as gemm_mfma_pipe.hpp -- whole 128-byte rows by LDS-DMA into a two-stage ring,
@@ -21,7 +21,7 @@
 namespace hodu {
 namespace mfma {
 
-enum { OUT_F8E4M3 = 4 };
+enum { OUT_F8E4M3 = 4, OUT_F8E5M2 = 5 };
 
 template <> struct Out<OUT_F8E4M3> {
     static constexpr int DT = HODU_F8E4M3;
@@ -30,15 +30,22 @@ template <> struct Out<OUT_F8E4M3> {
     static __device__ __forceinline__ T cvt(float v) { return f32_to_f8e4m3_sat(v); }
 };
 
+template <> struct Out<OUT_F8E5M2> {
+    static constexpr int DT = HODU_F8E5M2;
+    typedef uint8_t T;
+    static __device__ __forceinline__ T cvt(float v) { return f32_to_f8e5m2_sat(v); }
+};
+
 struct FragF8 {
     u32x4_t lo, hi;  // 32 consecutive bytes of k
 };
 typedef int i32x8_t __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ void mma_f8(const FragF8 &a, const FragF8 &b, f32x16_t &c) {
+// FMT: the instruction's operand format code, 0 = e4m3, 1 = e5m2 (both operands alike)
+template <int FMT> __device__ __forceinline__ void mma_f8(const FragF8 &a, const FragF8 &b, f32x16_t &c) {
     const i32x8_t av = {(int)a.lo.x, (int)a.lo.y, (int)a.lo.z, (int)a.lo.w, (int)a.hi.x, (int)a.hi.y, (int)a.hi.z, (int)a.hi.w};
     const i32x8_t bv = {(int)b.lo.x, (int)b.lo.y, (int)b.lo.z, (int)b.lo.w, (int)b.hi.x, (int)b.hi.y, (int)b.hi.z, (int)b.hi.w};
-    // cbsz = blgp = 0: both operands e4m3; scale bytes 0x7F = 2^0
-    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    // cbsz = blgp = FMT; scale bytes 0x7F = 2^0
+    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
 
 template <int OUT_, int BM_, int BN_> struct PipeF8Config {
@@ -179,7 +186,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
             }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                mma_f8(fbw[CUR][j], fa[i & 1], acc[i][j]);
+                mma_f8<Cfg::OUT == OUT_F8E5M2 ? 1 : 0>(fbw[CUR][j], fa[i & 1], acc[i][j]);
                 // DMA: in a LATE window only behind the barrier; otherwise spread over all MFMAs
                 constexpr int SLOTS = LATE ? TN : TM * TN;
                 const int pos = LATE ? j : i * TN + j;

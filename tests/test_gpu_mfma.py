@@ -234,25 +234,27 @@ def test_split_k(ctx, kind, splits):
         ctx.force_splitk(-1)
 
 
+@pytest.mark.parametrize("dt", ["f8e4m3", "f8e5m2"])
 @pytest.mark.parametrize("tile,name", [(11, "pipe256x256"), (12, "pipe128x128")])
-def test_native_f8_products(ctx, tile, name):
-    """f8e4m3 x f8e4m3 -> f8e4m3 on the 8-bit matrix instruction: 1 to 5 stages of 128 k, ragged M and N, batches,
+def test_native_f8_products(ctx, dt, tile, name):
+    """f8e4m3 x f8e4m3 -> f8e4m3 (and the same for f8e5m2) on the 8-bit matrix instruction: 1 to 5 stages of 128 k, ragged M
+    and N, batches,
     row slices and offsets; K not a multiple of 128 or a row-dense operand stay with the generic kernel"""
     ctx.force_tile(tile)
     try:
         for K in (128, 256, 384, 640):
-            check_product(ctx, "dot", "f8e4m3", V([296, K]), V([200, K]).t(), seed=K, scale=0.5,
-                          expect_kernel=f"mfma_f8e4m3_{name}_KK")
-        check_product(ctx, "matmul", "f8e4m3", V([3, 72, 512]).slice(2, 128, 384), V([3, 80, 256], offset=64).t(), seed=7,
-                      scale=0.5, expect_kernel=f"mfma_f8e4m3_{name}_KK")
-        check_product(ctx, "matmul", "f8e4m3", V([4, 40, 256]), V([56, 256]).t().broadcast_to([4, 256, 56]), seed=8, scale=0.5,
-                      expect_kernel=f"mfma_f8e4m3_{name}_KK")
+            check_product(ctx, "dot", dt, V([296, K]), V([200, K]).t(), seed=K, scale=0.5,
+                          expect_kernel=f"mfma_{dt}_{name}_KK")
+        check_product(ctx, "matmul", dt, V([3, 72, 512]).slice(2, 128, 384), V([3, 80, 256], offset=64).t(), seed=7,
+                      scale=0.5, expect_kernel=f"mfma_{dt}_{name}_KK")
+        check_product(ctx, "matmul", dt, V([4, 40, 256]), V([56, 256]).t().broadcast_to([4, 256, 56]), seed=8, scale=0.5,
+                      expect_kernel=f"mfma_{dt}_{name}_KK")
         ctx.force_splitk(3)
-        check_product(ctx, "dot", "f8e4m3", V([296, 1280]), V([200, 1280]).t(), seed=9, scale=0.3,
-                      expect_kernel=f"mfma_f8e4m3_{name}_KK_splitk3")
+        check_product(ctx, "dot", dt, V([296, 1280]), V([200, 1280]).t(), seed=9, scale=0.3,
+                      expect_kernel=f"mfma_{dt}_{name}_KK_splitk3")
         ctx.force_splitk(-1)
-        check_product(ctx, "dot", "f8e4m3", V([64, 200]), V([48, 200]).t(), seed=10, scale=0.5, expect_kernel="generic")
-        check_product(ctx, "dot", "f8e4m3", V([64, 256]), V([256, 48]), seed=11, scale=0.5, expect_kernel="generic")
+        check_product(ctx, "dot", dt, V([64, 200]), V([48, 200]).t(), seed=10, scale=0.5, expect_kernel="generic")
+        check_product(ctx, "dot", dt, V([64, 256]), V([256, 48]), seed=11, scale=0.5, expect_kernel="generic")
     finally:
         ctx.force_tile(-1)
         ctx.force_splitk(-1)
