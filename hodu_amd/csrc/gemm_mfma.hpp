@@ -37,7 +37,7 @@ namespace mfma {
 enum { CK_BF16 = 0, CK_F16 = 1, CK_I8 = 2, CK_F32 = 3 };  // compute kind (type held in LDS / fed to MFMA)
 enum { SK_SAME = 0, SK_F8 = 1 };                         // operand storage: compute type, or f8e4m3 -> bf16
 enum { LM_K = 0, LM_MN = 1, LM_SCALAR = 2, LM_MNU = 3 };
-enum { OUT_BF16 = 0, OUT_F16 = 1, OUT_F32 = 2, OUT_I32 = 3 };
+enum { OUT_BF16 = 0, OUT_F16 = 1, OUT_F32 = 2, OUT_I32 = 3, OUT_I8 = 6, OUT_U8 = 7 };  // (4, 5: the f8 outputs)
 
 constexpr int ROW_BYTES = 128;   // bytes of compute type per LDS row per K step
 constexpr int ROW_PITCH = 144;   // padded: 16 consecutive rows at one chunk hit 64 distinct banks
@@ -546,6 +546,20 @@ template <> struct Out<OUT_I32> {
     static constexpr int DT = HODU_I32;
     typedef int32_t T;
     static __device__ __forceinline__ T cvt(int v) { return v; }
+};
+
+// i8 x i8 -> i8 and u8 x u8 -> u8 (hodu's own 8-bit integer products, which wrap): the low byte of the exact i32 sum.
+// The matrix core reads the bytes as signed; for u8 that changes each factor by a multiple of 256, so the low byte of
+// the sum is the same.
+template <> struct Out<OUT_I8> {
+    static constexpr int DT = HODU_I8;
+    typedef int8_t T;
+    static __device__ __forceinline__ T cvt(int v) { return (int8_t)v; }
+};
+template <> struct Out<OUT_U8> {
+    static constexpr int DT = HODU_U8;
+    typedef uint8_t T;
+    static __device__ __forceinline__ T cvt(int v) { return (uint8_t)v; }
 };
 
 // accumulator -> stored element: the product's own rounding, then the fused element-wise steps for column n

@@ -1,7 +1,7 @@
 // f8e4m3 x f8e4m3 and f8e5m2 x f8e5m2 products on the native gfx950 8-bit MFMA (v_mfma_scale_f32_32x32x64_f8f6f4
 // with unit scales: 64 k per instruction, twice the arithmetic of the bf16 instruction for the same
 // operand bytes; the instruction's format fields select e4m3 or e5m2).  hodu's own f8 matmul / dot (lhs, rhs and
-// result all of one f8 type; crates/hodu_cpu_kernels/kernels/ops_matrix.c:353-354, :715-716) lands here when both operands are k-dense
+// result all of one f8 type; crates/hodu_cpu_kernels/kernels/ops_matrix.c:351-352, :713-714) lands here when both operands are k-dense
 // and K is a multiple of 128; products accumulate in f32 and are narrowed once, round-to-nearest-even
 // and saturating at +-448 (e5m2: +-57344) like every other f8 product of this library (the reference re-rounds
 // its f8 accumulator after every k, ops_matrix.c:572-573).

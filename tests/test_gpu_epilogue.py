@@ -90,10 +90,11 @@ SPECS = [LINEAR, [("mul",)], [("relu",)], [("mul",), ("add", 2, 3), ("relu",)], 
 
 @pytest.mark.parametrize("dt", ffi.EPILOGUE_DTYPES)
 def test_generic_kernel_every_dtype(ctx, dt):
-    """column-strided operands: the generic kernel, the tile kernel's scalar-load variant for bf16 / f16, the
-    small-product kernel for f32, the f64 matrix-core kernel"""
+    """column-strided operands: the generic kernel, the tile kernel's scalar-load variant for bf16 / f16 / i8 / u8,
+    the small-product kernel for f32, the f64 matrix-core kernel"""
     lv, rv = V([37, 50]).slice(1, 1, 49, 2), V([24, 70]).slice(1, 0, 70, 2)
-    family = "mfma_" if dt in ("bf16", "f16") else "small_f32" if dt == "f32" else "mfma_f64" if dt == "f64" else "generic"
+    family = ("mfma_" if dt in ("bf16", "f16", "i8", "u8") else "small_f32" if dt == "f32" else "mfma_f64" if dt == "f64"
+              else "generic")
     for n, spec in enumerate(SPECS):
         if dt not in FLOATS and ("relu",) in spec:
             continue

@@ -258,3 +258,43 @@ def test_native_f8_products(ctx, dt, tile, name):
     finally:
         ctx.force_tile(-1)
         ctx.force_splitk(-1)
+
+
+@pytest.mark.parametrize("dt", ["i8", "u8"])
+def test_eight_bit_integer_products_wrap(ctx, dt):
+    """hodu's own i8 x i8 -> i8 and u8 x u8 -> u8 products (the accumulator has the operands' type and wraps) on the i8
+    matrix instruction: the low byte of the exact sum, bit for bit the reference's result -- every tile variant, row-dense
+    and unaligned operands, batches, K cut across workgroups"""
+    prefix = f"mfma_{dt}_"
+    for tile in (10, 11, 12, 13, 0, 2, 3):
+        ctx.force_tile(tile)
+        try:
+            check_product(ctx, "dot", dt, V([296, 384]), V([200, 384]).t(), seed=tile, expect_kernel=prefix)
+            check_product(ctx, "dot", dt, V([150, 128]), V([128, 272]), seed=20 + tile, expect_kernel=prefix)
+        finally:
+            ctx.force_tile(-1)
+    check_product(ctx, "matmul", dt, V([3, 72, 256]), V([3, 80, 256]).t(), seed=40, expect_kernel=prefix)
+    check_product(ctx, "matmul", dt, V([4, 40, 96]), V([56, 96]).t().broadcast_to([4, 96, 56]), seed=41, expect_kernel=prefix)
+    check_product(ctx, "dot", dt, V([70, 197]), V([67, 197]).t(), seed=42, expect_kernel=prefix)          # odd K
+    check_product(ctx, "dot", dt, V([33, 101], offset=1), V([101, 35]), seed=43, expect_kernel=prefix)    # odd everything
+    check_product(ctx, "dot", dt, V([256, 4096]), V([384, 4096]).t(), seed=44, expect_kernel=prefix)      # cut along K
+    assert "splitk" in ctx.last_kernel(), ctx.last_kernel()
+    check_product(ctx, "dot", dt, V([2, 512]), V([64, 512]).t(), seed=45, expect_kernel=prefix)           # two rows
+
+
+@pytest.mark.parametrize("dt", ["i8", "u8"])
+def test_eight_bit_integer_products_full_range(ctx, dt):
+    """every byte value on both sides (u8 values from 128 up are negative numbers to the matrix core: the low byte of
+    the sum does not care), against the reference-faithful oracle bit for bit"""
+    from gpu_util import run_product
+    import oracle
+    np_dt = np.int8 if dt == "i8" else np.uint8
+    g = H.rng(77)
+    for (m, k, n), rt in (((200, 384, 136), True), ((96, 1000, 72), False)):
+        a = g.integers(0, 256, m * k).astype(np.uint8).view(np_dt)
+        b = g.integers(0, 256, k * n).astype(np.uint8).view(np_dt)
+        a[:256] = np.arange(256, dtype=np.uint8).view(np_dt)
+        md = H.dot_md(V([m, k]), V([n, k]).t() if rt else V([k, n]))
+        got = run_product(ctx, "dot", dt, a, b, md)
+        assert ctx.last_kernel().startswith(f"mfma_{dt}_")
+        assert np.array_equal(got, oracle.dot_asis(dt, a, b, md))
