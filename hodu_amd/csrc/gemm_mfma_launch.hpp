@@ -85,19 +85,21 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     } else if (forced < 0 && size == 3) {
         splits = pick_splits(tiles(128, 128), cus, stages, elems, ctx->force_splits);
         if (splits > 1) size = 2;
-        if constexpr (SKA == SK_SAME && SKB == SK_SAME && ES <= 2) {
+        if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
             // Cutting K costs a second kernel and the partial sums' trip through memory, which a short K does not
             // earn back.  Measured (bf16, one workgroup per CU or fewer; microseconds): a 128 x 128 workgroup takes
             // 5 + 0.42 per stage, a 64 x 64 one (both operands k-dense) 4.5 + 0.25 per stage, the second pass
             // 3 + 8 bytes per output and range at 4 TB/s.  [1024, 1024] x [1024, 1024]^T: 18.3 us cut four ways,
             // 11.8 on 128 x 128 tiles as it is, 8.1 on 64 x 64 tiles; [512, 4096] x [4096, 512]: 15.3 cut eight ways,
-            // 19.3 / 30.1 uncut.
+            // 19.3 / 30.1 uncut.  f32 (a stage is 32 k, and the f32 matrix instruction is eight times slower per
+            // k): 2.05 and 0.65 per stage; [1024, 1024] x [1024, 1024]^T 31.5 us cut four ways, 24.5 on 64 x 64 tiles.
             if (ctx->force_splits < 0 && tiles(128, 128) < cus) {
+                constexpr double S128 = ES == 4 ? 2.05 : 0.42, S64 = ES == 4 ? 0.65 : 0.25;
                 const bool kk = la == LM_K && lb == LM_K;
-                const double t_cut = splits > 1 ? 8.0 + 0.42 * ((stages + splits - 1) / splits) + (double)elems * splits * 8 / 4e6 : 1e30;
-                const double t_128 = g.M >= 64 && g.N >= 64 ? 5.0 + 0.42 * stages : 1e30;
+                const double t_cut = splits > 1 ? 8.0 + S128 * ((stages + splits - 1) / splits) + (double)elems * splits * 8 / 4e6 : 1e30;
+                const double t_128 = g.M >= 64 && g.N >= 64 ? 5.0 + S128 * stages : 1e30;
                 const double waves64 = (double)tiles(64, 64) / cus;
-                const double t_64 = kk ? 4.5 + 0.25 * stages * (waves64 > 1 ? waves64 : 1) : 1e30;
+                const double t_64 = kk ? 4.5 + S64 * stages * (waves64 > 1 ? waves64 : 1) : 1e30;
                 if (t_64 <= t_cut && t_64 <= t_128) {
                     size = 3;
                     splits = 1;
