@@ -162,6 +162,21 @@ __device__ __forceinline__ u32x2_t ldg64(const char *p) { return *reinterpret_ca
 // 16 bytes from an address that is only known to be a multiple of 2 (one 16-byte load all the same)
 typedef u32x4_t __attribute__((aligned(2))) u32x4_elem_aligned_t;
 __device__ __forceinline__ u32x4_t ldg128_elem_aligned(const char *p) { return *reinterpret_cast<const u32x4_elem_aligned_t *>(p); }
+// and the stores: BYTES at an address that is only known to be a multiple of ALIGN (the element size) -- one store
+// instruction all the same, which is what an output with an odd row length needs ([.., 197, 197] scores)
+template <int BYTES, int ALIGN> struct UnderAligned;
+#define HODU_UNDER_ALIGNED(BYTES, ALIGN, BASE) \
+    template <> struct UnderAligned<BYTES, ALIGN> { typedef BASE Base; typedef BASE __attribute__((aligned(ALIGN))) T; };
+HODU_UNDER_ALIGNED(16, 1, u32x4_t)
+HODU_UNDER_ALIGNED(16, 2, u32x4_t)
+HODU_UNDER_ALIGNED(16, 4, u32x4_t)
+HODU_UNDER_ALIGNED(8, 2, u32x2_t)
+HODU_UNDER_ALIGNED(4, 1, uint32_t)
+#undef HODU_UNDER_ALIGNED
+template <int BYTES, int ALIGN> __device__ __forceinline__ void stg_elem_aligned(void *dst, const void *src) {
+    typedef UnderAligned<BYTES, ALIGN> U;
+    *reinterpret_cast<typename U::T *>(dst) = *reinterpret_cast<const typename U::Base *>(src);
+}
 __device__ __forceinline__ void lds_put(char *lds, int off, const u32x4_t &v) { *reinterpret_cast<u32x4_t *>(lds + off) = v; }
 __device__ __forceinline__ u32x4_t lds_get(const char *lds, int off) { return *reinterpret_cast<const u32x4_t *>(lds + off); }
 
@@ -594,9 +609,12 @@ __device__ __forceinline__ void store_tile32(typename Out<OUT>::T *Cb, const acc
             else v[e] = Out<OUT>::cvt(acc[4 * q + e]);
         }
         out_t *dst = Cb + (long)m * N + n;
+        struct alignas(sizeof(out_t) * 4) Quad { out_t q[4]; };
         if (vec_ok && n + 3 < N) {
-            struct alignas(sizeof(out_t) * 4) Quad { out_t q[4]; };
             *reinterpret_cast<Quad *>(dst) = Quad{{v[0], v[1], v[2], v[3]}};
+        } else if (n + 3 < N) {  // an odd row length: the same store at element alignment
+            const Quad quad{{v[0], v[1], v[2], v[3]}};
+            stg_elem_aligned<sizeof(out_t) * 4, sizeof(out_t)>(dst, &quad);
         } else {
 #pragma unroll
             for (int e = 0; e < 4; e++)

@@ -182,6 +182,8 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
         out_t *dst = Cb + (long)m * N + n;
         if (vec_ok && n + EPV <= N) {
             *reinterpret_cast<u32x4_t *>(dst) = v;
+        } else if (n + EPV <= N) {  // an odd row length: the same store at element alignment
+            stg_elem_aligned<16, OS>(dst, &v);
         } else {
             const out_t *e = reinterpret_cast<const out_t *>(&v);
 #pragma unroll
