@@ -7,7 +7,8 @@
 // and nothing has to be transposed.  Operands therefore go from memory straight into the MFMA's registers -- no LDS, no
 // barriers:
 //   * a workgroup is 2 x 2 wavefronts, a wavefront owns TM x TN tiles of 16 x 16 outputs (64 x 64 for large products,
-//     32 x 32 for small ones; neighbouring wavefronts share operand rows through the caches);
+//     32 x 32 and 16 x 16 for smaller ones, so that every compute unit gets a workgroup; neighbouring wavefronts share
+//     operand rows through the caches);
 //   * k is fed in chunks of 8: lane (r, q) takes k0 + 2 q and k0 + 2 q + 1 of row r -- one 16-byte load where the
 //     operand is k-dense, two 8-byte loads (16 lanes = one 128-byte line) where it is row-dense; both operands use
 //     the same order, which is all the sum needs;
@@ -159,15 +160,18 @@ int run_f64(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const Dev
 // Every f64 product with at least a tile's worth of rows and columns; the generic kernel keeps the thin ones.
 int launch_gemm_f64(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
     if (kind != PK_SAME || dtype != HODU_F64 || g.M < 1 || g.N < 1 || g.K < 1 || g.batches < 1) return HODU_ROCM_UNSUPPORTED;
-    if (ctx->force_tile >= 0 && ctx->force_tile != 41 && ctx->force_tile != 42) return HODU_ROCM_UNSUPPORTED;
+    if (ctx->force_tile >= 0 && (ctx->force_tile < 41 || ctx->force_tile > 43)) return HODU_ROCM_UNSUPPORTED;
     if (ctx->force_tile < 0 && (g.M < 16 || g.N < 16)) return HODU_ROCM_UNSUPPORTED;
     static const char *const big[4] = {"mfma_f64_128x128_KK", "mfma_f64_128x128_KM", "mfma_f64_128x128_MK", "mfma_f64_128x128_MM"};
     static const char *const small[4] = {"mfma_f64_64x64_KK", "mfma_f64_64x64_KM", "mfma_f64_64x64_MK", "mfma_f64_64x64_MM"};
+    static const char *const tiny[4] = {"mfma_f64_32x32_KK", "mfma_f64_32x32_KM", "mfma_f64_32x32_MK", "mfma_f64_32x32_MM"};
     const int cus = ctx->props.multiProcessorCount;
-    const long big_tiles = g.batches * ((g.M + 127) / 128) * ((g.N + 127) / 128);
-    const bool use_big = ctx->force_tile == 41 || (ctx->force_tile < 0 && big_tiles >= cus);
-    if (use_big) return run_f64<4, 4, 2>(ctx, a, b, c, g, big);
-    return run_f64<2, 2, 4>(ctx, a, b, c, g, small);
+    auto tiles = [&](long bm) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bm - 1) / bm); };
+    // the largest tile that still gives every compute unit a workgroup
+    const int size = ctx->force_tile >= 0 ? ctx->force_tile - 41 : tiles(128) >= cus ? 0 : tiles(64) >= cus ? 1 : 2;
+    if (size == 0) return run_f64<4, 4, 2>(ctx, a, b, c, g, big);
+    if (size == 1) return run_f64<2, 2, 4>(ctx, a, b, c, g, small);
+    return run_f64<1, 1, 8>(ctx, a, b, c, g, tiny);
 }
 
 }  // namespace hodu

@@ -84,8 +84,8 @@ const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
  * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
  * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; 14 = the pipelined 256x128 tile;
  * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
- * variant that cuts K across workgroups wherever it applies; 40 = the small-product f32 kernel at any size; 41 / 42 = the f64 matrix-core kernel with
- * 128 x 128 / 64 x 64 tiles;
+ * variant that cuts K across workgroups wherever it applies; 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
+ * 128 x 128 / 64 x 64 / 32 x 32 tiles;
  * -1 = automatic) so that every compiled variant
  * can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);

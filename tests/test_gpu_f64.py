@@ -25,7 +25,7 @@ LAYOUTS = {
 }
 
 
-@pytest.mark.parametrize("tile,size", [(41, "128x128"), (42, "64x64")])
+@pytest.mark.parametrize("tile,size", [(41, "128x128"), (42, "64x64"), (43, "32x32")])
 @pytest.mark.parametrize("layout", list(LAYOUTS))
 def test_layouts_and_edges(ctx, tile, size, layout):
     ctx.force_tile(tile)
@@ -44,12 +44,13 @@ def test_layouts_and_edges(ctx, tile, size, layout):
 def test_views_batches_and_selection(ctx):
     # row-sliced operands at odd offsets, a column-strided x
     check_product(ctx, "dot", "f64", V([48, 300], offset=3).slice(1, 5, 261), V([256, 131], offset=1).slice(1, 0, 99),
-                  seed=1, expect_kernel="mfma_f64_64x64_KM")
-    check_product(ctx, "dot", "f64", V([48, 400]).slice(1, 0, 400, 2), V([200, 64]), seed=2, expect_kernel="mfma_f64_64x64_MM")
+                  seed=1, expect_kernel="mfma_f64_32x32_KM")
+    check_product(ctx, "dot", "f64", V([48, 400]).slice(1, 0, 400, 2), V([200, 64]), seed=2, expect_kernel="mfma_f64_32x32_MM")
     # batched; one operand shared across the batch
     check_product(ctx, "matmul", "f64", V([3, 2, 40, 64]), V([64, 72]).broadcast_to([3, 2, 64, 72]), seed=3,
-                  expect_kernel="mfma_f64_64x64_KM")
-    check_product(ctx, "matmul", "f64", V([5, 96, 128]), V([5, 80, 128]).t(1, 2), seed=4, expect_kernel="mfma_f64_64x64_KK")
+                  expect_kernel="mfma_f64_32x32_KM")
+    check_product(ctx, "matmul", "f64", V([5, 96, 128]), V([5, 80, 128]).t(1, 2), seed=4, expect_kernel="mfma_f64_32x32_KK")
+    check_product(ctx, "dot", "f64", V([1024, 40]), V([40, 1100]), seed=8, expect_kernel="mfma_f64_64x64_KM")
     # enough 128 x 128 tiles to fill the chip: the large tile
     check_product(ctx, "dot", "f64", V([2048, 40]), V([40, 2048]), seed=5, expect_kernel="mfma_f64_128x128_KM")
     # thinner than a tile: the generic kernel keeps these
