@@ -126,16 +126,22 @@ __global__ __launch_bounds__(256) void sum_chunks_kernel(const typename E::stora
     for (int v = 0; v < V; v++) acc[v] = (A)0;
     if (o < r.n_out) {
         const S *base = in + r.offset + kept_offset(r, o);
-        for (long i = begin + wave; i < end; i += 4) {
-            const S *p = base + red_offset(r, i);
-            if constexpr (V == 1) {
-                acc[0] += E::load(p[0]);
-            } else {
-                struct alignas(sizeof(S) * V) Vec { S e[V]; };
-                const Vec x = *reinterpret_cast<const Vec *>(p);
+        struct alignas(sizeof(S) * V) Vec { S e[V]; };
+        constexpr int IF = 4;  // loads in flight per lane: the additions keep their order (index by index)
+        long i = begin + wave;
+        for (; i + 4 * (IF - 1) < end; i += 4 * IF) {
+            Vec x[IF];
 #pragma unroll
-                for (int v = 0; v < V; v++) acc[v] += E::load(x.e[v]);
-            }
+            for (int u = 0; u < IF; u++) x[u] = *reinterpret_cast<const Vec *>(base + red_offset(r, i + 4 * u));
+#pragma unroll
+            for (int u = 0; u < IF; u++)
+#pragma unroll
+                for (int v = 0; v < V; v++) acc[v] += E::load(x[u].e[v]);
+        }
+        for (; i < end; i += 4) {
+            const Vec x = *reinterpret_cast<const Vec *>(base + red_offset(r, i));
+#pragma unroll
+            for (int v = 0; v < V; v++) acc[v] += E::load(x.e[v]);
         }
     }
     if (wave > 0) {
