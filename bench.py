@@ -233,14 +233,14 @@ def time_case(ctx, case, steps, warmup, graph=False):
                            "p90": spread[8]}}
 
 
-def attention_probe(ctx, steps):
-    """not a BASELINE configuration: hodu_nn's scaled_dot_product_attention (causal, bf16, 32 heads x 2048 x 128) as
+def attention_probe(ctx, steps, d=128):
+    """not a BASELINE configuration: hodu_nn's scaled_dot_product_attention (causal, bf16, 32 heads x 2048 x d) as
     the one fused kernel, and as the three launches the host mirror falls back to -- Q K^T with the scale in its
     store, masked softmax, P V -- each timed with HIP events around `steps` back-to-back launches"""
     import helpers as H
     from hodu_amd import ffi
     V = H.View
-    heads, s_len, d = 32, 2048, 128
+    heads, s_len = 32, 2048
     q, k, v = (ctx.upload(bf16(normal(950 + i, heads * s_len * d))) for i in range(3))
     scores, probs = ctx.alloc(heads * s_len * s_len * 2), ctx.alloc(heads * s_len * s_len * 2)
     out = ctx.alloc(heads * s_len * d * 2)
@@ -525,8 +525,8 @@ def main():
                           "launches": args.steps}))
         ctx.close()
         return
-    if args.only == "attention":
-        print(json.dumps(attention_probe(ctx, args.steps)))
+    if args.only in ("attention", "attention_d64"):
+        print(json.dumps(attention_probe(ctx, args.steps, 64 if args.only == "attention_d64" else 128)))
         ctx.close()
         return
     if args.only == "pcie":
