@@ -169,7 +169,7 @@ int launch_gemv(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const vo
 // it): returns HODU_ROCM_UNSUPPORTED when the product is not f32 or is large enough for the tiled kernels
 int launch_small_f32(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g);
 // f64 products on the f64 matrix-core instruction, operands straight from memory: returns HODU_ROCM_UNSUPPORTED for
-// other dtypes and for products thinner than one 16 x 16 tile
+// other dtypes
 int launch_gemm_f64(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g);
 int launch_skinny(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                   const DevProduct &g);

@@ -157,11 +157,12 @@ int run_f64(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const Dev
 
 }  // namespace
 
-// Every f64 product with at least a tile's worth of rows and columns; the generic kernel keeps the thin ones.
+// Every f64 product: thin ones (a few rows or columns, a matrix times a vector) included -- their tiles are mostly
+// padding, but the operands still arrive as whole cache lines, [1, 4096] x [4096, 4096] in 58 us where the generic
+// kernel takes 664.
 int launch_gemm_f64(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
     if (kind != PK_SAME || dtype != HODU_F64 || g.M < 1 || g.N < 1 || g.K < 1 || g.batches < 1) return HODU_ROCM_UNSUPPORTED;
     if (ctx->force_tile >= 0 && (ctx->force_tile < 41 || ctx->force_tile > 43)) return HODU_ROCM_UNSUPPORTED;
-    if (ctx->force_tile < 0 && (g.M < 16 || g.N < 16)) return HODU_ROCM_UNSUPPORTED;
     static const char *const big[4] = {"mfma_f64_128x128_KK", "mfma_f64_128x128_KM", "mfma_f64_128x128_MK", "mfma_f64_128x128_MM"};
     static const char *const small[4] = {"mfma_f64_64x64_KK", "mfma_f64_64x64_KM", "mfma_f64_64x64_MK", "mfma_f64_64x64_MM"};
     static const char *const tiny[4] = {"mfma_f64_32x32_KK", "mfma_f64_32x32_KM", "mfma_f64_32x32_MK", "mfma_f64_32x32_MM"};

@@ -53,5 +53,8 @@ def test_views_batches_and_selection(ctx):
     check_product(ctx, "dot", "f64", V([1024, 40]), V([40, 1100]), seed=8, expect_kernel="mfma_f64_64x64_KM")
     # enough 128 x 128 tiles to fill the chip: the large tile
     check_product(ctx, "dot", "f64", V([2048, 40]), V([40, 2048]), seed=5, expect_kernel="mfma_f64_128x128_KM")
-    # thinner than a tile: the generic kernel keeps these
-    check_product(ctx, "dot", "f64", V([4, 256]), V([256, 64]), seed=6, expect_kernel="generic")
+    # thinner than a tile, a matrix times a vector, a single output
+    check_product(ctx, "dot", "f64", V([4, 256]), V([256, 64]), seed=6, expect_kernel="mfma_f64_32x32_KM")
+    check_product(ctx, "dot", "f64", V([1, 1000]), V([333, 1000]).t(), seed=9, expect_kernel="mfma_f64_32x32_KK")
+    check_product(ctx, "dot", "f64", V([77, 130]), V([130, 1]), seed=10, expect_kernel="mfma_f64_32x32")
+    check_product(ctx, "dot", "f64", V([1, 50]), V([50, 1]), seed=11, expect_kernel="mfma_f64_32x32")
