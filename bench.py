@@ -546,7 +546,7 @@ def main():
         ctx.close()
         return
     if args.only:
-        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "fused", "bwd"}) if c.key == args.only)
+        case = next(c for c in build_cases({"c1", "c2", "c3", "c4", "c5", "f8", "f64", "fused", "bwd"}) if c.key == args.only)
         print(json.dumps(time_case(ctx, case, args.steps, args.warmup, graph=args.graph)))
         ctx.close()
         return
