@@ -17,6 +17,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "_build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libhodu_rocm_kernels.so")
+DEBUG_SRC = os.path.join(HERE, "csrc_debug")
+DEBUG_LIB = os.path.join(LIB_DIR, "libhodu_rocm_debug.so")
 HOST_DIR = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIB_DIR, "libhodu_rocm_host.so")
 
@@ -39,8 +41,18 @@ def hipcc() -> str:
     return path
 
 
+_ONLY_CHANGED = False  # `python -m hodu_amd.build --changed`: keep objects newer than their source and every header
+
+
+def _headers_mtime() -> float:
+    dirs = [CSRC, DEBUG_SRC, os.path.join(ROOT, "include")]
+    return max(os.path.getmtime(os.path.join(d, f)) for d in dirs for f in os.listdir(d) if f.endswith((".hpp", ".h")))
+
+
 def _compile(src: str) -> str:
-    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+    obj = os.path.join(OBJ, os.path.basename(os.path.dirname(src)) + "_" + os.path.basename(src) + ".o")
+    if _ONLY_CHANGED and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _headers_mtime()):
+        return obj
     cmd = [hipcc(), *FLAGS, "-c", src, "-o", obj]
     if src.endswith(".cpp"):
         cmd[1:1] = ["-x", "hip"]
@@ -68,8 +80,26 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     os.replace(tmp, LIB)
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
+    build_debug(verbose, jobs)
     build_host(verbose)
     return LIB
+
+
+def build_debug(verbose: bool = True, jobs: int = 8) -> str:
+    """The test and measurement hooks (include/hodu_rocm_debug.h): a library of their own on top of the kernel
+    library, so that the kernel library exports the boundary and nothing else."""
+    srcs = sorted(os.path.join(DEBUG_SRC, f) for f in os.listdir(DEBUG_SRC) if f.endswith((".hip", ".cpp")))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, srcs))
+    tmp = DEBUG_LIB + ".tmp"
+    r = subprocess.run([hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs, f"-L{LIB_DIR}",
+                        "-lhodu_rocm_kernels", "-Wl,-rpath,$ORIGIN"], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link of the hooks library failed:\n{r.stderr[-4000:]}")
+    os.replace(tmp, DEBUG_LIB)
+    if verbose:
+        print(f"built {DEBUG_LIB} from {len(srcs)} sources", file=sys.stderr)
+    return DEBUG_LIB
 
 
 def build_host(verbose: bool = True) -> str:
@@ -88,4 +118,5 @@ def build_host(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    _ONLY_CHANGED = "--changed" in sys.argv
     build()

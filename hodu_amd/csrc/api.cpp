@@ -245,85 +245,6 @@ HODU_ROCM_DEF_PRODUCT_EX(i64, PK_SAME, HODU_I64)
 HODU_ROCM_DEF_PRODUCT_EX(bf16_f8e4m3w, PK_BF16_F8W, HODU_BF16)
 HODU_ROCM_DEF_PRODUCT_EX(i32_i8i8, PK_I32_I8I8, HODU_I32)
 
-static int time_product_impl(bool graph, hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                 const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
-                                 int iters, float *elapsed_ms, const hodu_rocm_epilogue_step *steps = nullptr,
-                                 size_t n_steps = 0) {
-    clear_error();
-    if (!ctx || !rhs_list || n_rhs == 0 || !elapsed_ms || iters <= 0)
-        return fail(HODU_ROCM_INVALID_ARG, "time_product: bad argument");
-    if (kind < PK_SAME || kind > PK_I32_I8I8) return fail(HODU_ROCM_INVALID_ARG, "time_product: kind %d", kind);
-    for (size_t i = 0; i < n_rhs; i++) {
-        int rc = check_ptrs("time_product", ctx, lhs, rhs_list[i], out);
-        if (rc) return rc;
-    }
-    Product p;
-    int rc = is_matmul ? parse_matmul_metadata(md, len, &p) : parse_dot_metadata(md, len, &p);
-    if (rc) return rc;
-    DevEpilogue epi;
-    rc = build_epilogue("time_product", kind, dtype, out, steps, n_steps, &epi);
-    if (rc) return rc;
-    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
-    HODU_HIP(hipSetDevice(ctx->device));
-    hipEvent_t t0, t1;
-    HODU_HIP(hipEventCreate(&t0));
-    HODU_HIP(hipEventCreate(&t1));
-    hipGraph_t g = nullptr;
-    hipGraphExec_t exec = nullptr;
-    if (graph) {
-        // the launches are recorded once (kernel nodes only) and replayed as one graph: what a decode loop
-        // that cannot afford a host round trip per product would do
-        HODU_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
-        for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
-            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p, epi);
-        hipError_t ce = hipStreamEndCapture(ctx->stream, &g);
-        if (rc == HODU_ROCM_OK && ce != hipSuccess) rc = fail(HODU_ROCM_HIP_ERROR, "graph capture: %s", hipGetErrorString(ce));
-        if (rc == HODU_ROCM_OK && hipGraphInstantiate(&exec, g, nullptr, nullptr, 0) != hipSuccess)
-            rc = fail(HODU_ROCM_HIP_ERROR, "graph instantiate failed");
-        if (rc == HODU_ROCM_OK) {  // one untimed replay uploads the graph
-            (void)hipGraphLaunch(exec, ctx->stream);
-            (void)hipStreamSynchronize(ctx->stream);
-        }
-    }
-    HODU_HIP(hipEventRecord(t0, ctx->stream));
-    if (graph) {
-        if (rc == HODU_ROCM_OK && hipGraphLaunch(exec, ctx->stream) != hipSuccess)
-            rc = fail(HODU_ROCM_HIP_ERROR, "graph launch failed");
-    } else {
-        for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++)
-            rc = run_product(ctx, kind, dtype, lhs, rhs_list[(size_t)i % n_rhs], out, p, epi);
-    }
-    hipError_t e = hipEventRecord(t1, ctx->stream);
-    if (e == hipSuccess) e = hipEventSynchronize(t1);
-    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    if (exec) (void)hipGraphExecDestroy(exec);
-    if (g) (void)hipGraphDestroy(g);
-    if (rc) return rc;
-    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_product: %s", hipGetErrorString(e));
-    return HODU_ROCM_OK;
-}
-
-int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                 const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
-                                 int iters, float *elapsed_ms) {
-    return time_product_impl(false, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms);
-}
-
-int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                       const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md,
-                                       size_t len, int iters, float *elapsed_ms) {
-    return time_product_impl(true, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms);
-}
-
-int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                    const void *const *rhs_list, size_t n_rhs, void *out, const size_t *md, size_t len,
-                                    const hodu_rocm_epilogue_step *steps, size_t n_steps, int iters, float *elapsed_ms) {
-    return time_product_impl(false, ctx, is_matmul, kind, dtype, lhs, rhs_list, n_rhs, out, md, len, iters, elapsed_ms,
-                             steps, n_steps);
-}
-
 int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const size_t *md, size_t len) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "cast: context is null");
@@ -337,66 +258,6 @@ int hodu_rocm_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *o
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
     return launch_cast(ctx, src, dst, in, out, s);
-}
-
-int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *const *in_list, void *const *out_list,
-                              size_t n_buffers, const size_t *md, size_t len, int iters, float *elapsed_ms) {
-    clear_error();
-    if (!ctx || !in_list || !out_list || n_buffers == 0 || !elapsed_ms || iters < 1)
-        return fail(HODU_ROCM_INVALID_ARG, "time_cast: bad argument");
-    if (dtype_size(src) == 0 || dtype_size(dst) == 0)
-        return fail(HODU_ROCM_UNSUPPORTED, "time_cast: unknown dtype id (%d -> %d)", src, dst);
-    for (size_t i = 0; i < n_buffers; i++)
-        if (!in_list[i] || !out_list[i] || in_list[i] == out_list[i]) return fail(HODU_ROCM_INVALID_ARG, "time_cast: bad buffer %zu", i);
-    Strided s;
-    int rc = parse_cast_metadata(md, len, &s);
-    if (rc) return rc;
-    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
-    HODU_HIP(hipSetDevice(ctx->device));
-    hipEvent_t t0, t1;
-    HODU_HIP(hipEventCreate(&t0));
-    HODU_HIP(hipEventCreate(&t1));
-    HODU_HIP(hipEventRecord(t0, ctx->stream));
-    for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++) {
-        const size_t j = (size_t)i % n_buffers;
-        rc = src == dst ? launch_gather(ctx, src, in_list[j], out_list[j], s) : launch_cast(ctx, src, dst, in_list[j], out_list[j], s);
-    }
-    hipError_t e = hipEventRecord(t1, ctx->stream);
-    if (e == hipSuccess) e = hipEventSynchronize(t1);
-    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    if (rc) return rc;
-    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_cast: %s", hipGetErrorString(e));
-    return HODU_ROCM_OK;
-}
-
-int hodu_rocm_debug_time_sum(hodu_rocm_ctx *ctx, int dtype, const void *const *in_list, void *const *out_list,
-                             size_t n_buffers, const size_t *md, size_t len, int iters, float *elapsed_ms) {
-    clear_error();
-    if (!ctx || !in_list || !out_list || n_buffers == 0 || !elapsed_ms || iters < 1)
-        return fail(HODU_ROCM_INVALID_ARG, "time_sum: bad argument");
-    if (dtype_size(dtype) == 0 || dtype == HODU_BOOL) return fail(HODU_ROCM_UNSUPPORTED, "time_sum: dtype id %d has no sum kernel", dtype);
-    for (size_t i = 0; i < n_buffers; i++)
-        if (!in_list[i] || !out_list[i] || in_list[i] == out_list[i]) return fail(HODU_ROCM_INVALID_ARG, "time_sum: bad buffer %zu", i);
-    Reduction r;
-    int rc = parse_reduce_metadata(md, len, &r);
-    if (rc) return rc;
-    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
-    HODU_HIP(hipSetDevice(ctx->device));
-    hipEvent_t t0, t1;
-    HODU_HIP(hipEventCreate(&t0));
-    HODU_HIP(hipEventCreate(&t1));
-    HODU_HIP(hipEventRecord(t0, ctx->stream));
-    for (int i = 0; i < iters && rc == HODU_ROCM_OK; i++) rc = launch_sum(ctx, dtype, in_list[(size_t)i % n_buffers], out_list[(size_t)i % n_buffers], r);
-    hipError_t e = hipEventRecord(t1, ctx->stream);
-    if (e == hipSuccess) e = hipEventSynchronize(t1);
-    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    if (rc) return rc;
-    if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "time_sum: %s", hipGetErrorString(e));
-    return HODU_ROCM_OK;
 }
 
 int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {

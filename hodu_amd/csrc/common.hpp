@@ -4,7 +4,6 @@
 #include <hip/hip_runtime.h>
 
 #include <mutex>
-#include <unordered_set>
 
 #include <cstddef>
 #include <cstdint>
@@ -36,8 +35,10 @@ struct hodu_rocm_ctx {
     int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
     char kernel_name[96] = {0};  // storage for a composed last_kernel name
     // kernels whose dynamic-LDS limit has been raised on THIS context's device (the attribute belongs to a
-    // function on a device; a second context on another device has to set it again)
-    std::unordered_set<const void *> lds_configured;
+    // function on a device; a second context on another device has to set it again).  A fixed open-addressed
+    // table: recording a kernel allocates nothing, so entry points that must not allocate can share it.
+    static constexpr int kLdsSlots = 1024;
+    const void *lds_configured[kLdsSlots] = {};
     // every entry point that launches kernels holds this for the call: the workspace, the arrival counters, the
     // testing hooks and last_kernel belong to the context, and launches of one context go to one stream anyway
     std::recursive_mutex mu;
@@ -62,13 +63,19 @@ int fail(int code, const char *fmt, ...);
 
 // raises a kernel's dynamic-LDS limit once per context (called with ctx->mu held, like every launch)
 inline int ensure_dynamic_lds(hodu_rocm_ctx *ctx, const void *kernel, int bytes) {
-    if (ctx->lds_configured.count(kernel)) return HODU_ROCM_OK;
+    constexpr int N = hodu_rocm_ctx::kLdsSlots;
+    unsigned h = (unsigned)(((uintptr_t)kernel >> 4) * 2654435761u) % N;
+    for (int probe = 0; probe < N; probe++, h = (h + 1) % N) {
+        if (ctx->lds_configured[h] == kernel) return HODU_ROCM_OK;
+        if (ctx->lds_configured[h] == nullptr) break;
+    }
     HODU_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-    ctx->lds_configured.insert(kernel);
+    if (ctx->lds_configured[h] == nullptr) ctx->lds_configured[h] = kernel;  // a full table only repeats the call
     return HODU_ROCM_OK;
 }
 
-// grows ctx->workspace to at least `bytes`
+// grows ctx->workspace to at least `bytes` (refused, with an error text, while the context's stream is being
+// captured into a graph and it would have to grow)
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes);
 // allocates (once) and zeroes ctx->arrival; kernels that use a counter leave it at zero again
 constexpr int kArrivalSlots = 4096;

@@ -27,8 +27,25 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+namespace {
+
+__global__ __launch_bounds__(1024) void clear_words_kernel(int *__restrict__ p, int n) {
+    const int i = blockIdx.x * 1024 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+}  // namespace
+
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
     if (ctx->workspace.bytes >= bytes) return HODU_ROCM_OK;
+    if (stream_is_capturing(ctx->stream))
+        return fail(HODU_ROCM_SCRATCH, "the workspace would have to grow to %zu bytes while the stream is being "
+                    "captured: run the product once outside the capture first", bytes);
     if (ctx->workspace.ptr) {
         HODU_HIP(hipStreamSynchronize(ctx->stream));
         HODU_HIP(hipFree(ctx->workspace.ptr));
@@ -42,8 +59,14 @@ int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
 
 int ensure_arrival(hodu_rocm_ctx *ctx) {
     if (ctx->arrival) return HODU_ROCM_OK;
+    if (stream_is_capturing(ctx->stream))
+        return fail(HODU_ROCM_SCRATCH, "the arrival counters would be allocated while the stream is being "
+                    "captured: run the product once outside the capture first");
     HODU_HIP(hipMalloc((void **)&ctx->arrival, kArrivalSlots * sizeof(int)));
-    HODU_HIP(hipMemsetAsync(ctx->arrival, 0, kArrivalSlots * sizeof(int), ctx->stream));
+    // zeroed by a kernel, in stream order, before any kernel of this context can count on them
+    hipLaunchKernelGGL(clear_words_kernel, dim3((kArrivalSlots + 1023) / 1024), dim3(1024), 0, ctx->stream, ctx->arrival,
+                       kArrivalSlots);
+    HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }
 
@@ -172,24 +195,6 @@ int hodu_rocm_sync(hodu_rocm_ctx *ctx) {
 const char *hodu_rocm_last_error(hodu_rocm_ctx *) { return get_error(); }
 
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
-
-int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
-    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
-    const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 14) || tile == 30 || tile == 31 ||
-                    tile == 32 || tile == 34 || (tile >= 35 && tile <= 38) || (tile >= 40 && tile <= 43);
-    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..14, 30, 31, 32, 34..38, 40..43", tile);
-    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
-    ctx->force_tile = tile;
-    return HODU_ROCM_OK;
-}
-
-int hodu_rocm_debug_force_splitk(hodu_rocm_ctx *ctx, int splits) {
-    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
-    if (splits < -1 || splits == 0 || splits > 64) return fail(HODU_ROCM_INVALID_ARG, "splits %d not in -1, 1..64", splits);
-    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
-    ctx->force_splits = splits;
-    return HODU_ROCM_OK;
-}
 
 int hodu_rocm_device_info(hodu_rocm_ctx *ctx, char *name, size_t name_len, int *cus, int *clock_khz,
                           size_t *total_mem) {

@@ -196,17 +196,37 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
 // values are one 16-byte store) and bumps its column block's arrival counter; the workgroup that arrives last
 // adds the slices in slice order -- so the result does not depend on who was last --, rounds once, stores, and
 // zeroes the counter for the next launch.
-// 16-byte accesses at device scope (sc1): the store goes through to memory, the load does not take a line that this
-// compute unit's cache complex may hold from an earlier launch
-template <typename V>
-__device__ __forceinline__ void st16_device(V *p, const V &v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+//
+// How the partial sums cross from one workgroup to another (they run on different XCDs, each with an L2 of its
+// own that is not kept coherent with the others for ordinary accesses):
+//   * every partial sum is written and read with 16-byte buffer accesses that carry the sc1 bit, the encoding the
+//     gfx942 / gfx950 memory model gives an agent-scope atomic store / load: the store writes through the XCD's L2
+//     to memory, the load is served from the point all XCDs share and cannot hit a stale line this XCD kept from
+//     an earlier launch.  They are compiler builtins, so the wait-count bookkeeping of every load is the
+//     compiler's own;
+//   * release: each thread waits for its own stores (s_waitcnt vmcnt(0): a write-through store is acknowledged once
+//     it is visible at agent scope), the workgroup barrier follows, and only then does thread 0 increment the
+//     counter.  A release FENCE at agent scope would add a write-back of the whole L2 (buffer_wbl2), which exists
+//     for dirty lines of ordinary stores; there are none to publish here -- everything published was written
+//     through -- and it measured 7 us per launch;
+//   * acquire: the workgroup that finds slices - 1 in the counter has, by the counter's atomicity, been preceded by
+//     every other slice's increment and therefore by their completed stores; it passes its own barrier and reads
+//     with the sc1 loads above, which do not depend on an invalidate of this XCD's caches (buffer_inv, the other
+//     half of an acquire fence, is for ordinary loads).
+// The counter itself is a relaxed agent-scope read-modify-write, executed where all XCDs see it.
+constexpr int AUX_SC1 = 16;  // cache-policy bit of the raw buffer builtins that sets sc1 on gfx942 / gfx950
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t agent_buffer(void *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, bytes, 0x00020000);  // raw buffer: no stride, 32-bit format
 }
 template <typename V>
-__device__ __forceinline__ V ld16_device(const V *p) {
-    V v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(p) : "memory");
-    return v;
+__device__ __forceinline__ void store16_agent(__amdgpu_buffer_rsrc_t r, unsigned byte_off, const V &v) {
+    static_assert(sizeof(V) == 16, "one 16-byte access");
+    __builtin_amdgcn_raw_buffer_store_b128(bitcast<u32x4_t>(v), r, byte_off, 0, AUX_SC1);
+}
+template <typename V>
+__device__ __forceinline__ V load16_agent(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    static_assert(sizeof(V) == 16, "one 16-byte access");
+    return bitcast<V>(__builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, AUX_SC1));
 }
 
 constexpr int SK_ROWS = 128;  // weight rows per workgroup
@@ -297,11 +317,11 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
             }
         }
     }
-    // lane holds y[m = 4*lg + e][n] for e = 0..3: one 16-byte store into [slice][n][16]
-    // written THROUGH the cache at device scope, and waited for: the sums are then visible to every compute unit
-    // without a cache write-back (which costs 7 us per launch here when the counter update carries one)
-    if (n_ok) st16_device(&partials[((long)ks * g.N + n) * 4 + lg], acc);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // lane holds y[m = 4*lg + e][n] for e = 0..3: 16 consecutive bytes of [slice][n][16], written through at agent
+    // scope and waited for before the barrier
+    const __amdgpu_buffer_rsrc_t part = agent_buffer(partials, (unsigned)slices * (unsigned)g.N * 64u);
+    if (n_ok) store16_agent(part, (((unsigned)ks * g.N + n) * 4 + lg) * 16u, acc);
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0): this thread's stores are visible at agent scope
 
     // every thread's sums have landed before the barrier; thread 0 then counts this workgroup in.  Whoever sees
     // slices - 1 in the counter is last.
@@ -312,23 +332,19 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
     }
     __syncthreads();
     if (!last_flag) return;
-    // 128 columns x 4 quads of m: thread -> (column, quad); the other workgroups' sums are read at device scope
-    // (a plain load could be served from a line this compute unit cached during an earlier launch)
+    // 128 columns x 4 quads of m: thread -> (column, quad); the other workgroups' sums are read at agent scope
+    // (a plain load could be served from a line this XCD cached during an earlier launch)
     const int col = nb * SK_ROWS + (tid >> 2), quad = tid & 3;
     if (col < g.N) {
         acc_t s = acc_t{0, 0, 0, 0};
-        for (int k0 = 0; k0 < slices; k0 += 8) {  // eight loads in flight
+        for (int k0 = 0; k0 < slices; k0 += 8) {  // eight slices' loads in flight, added in slice order
             acc_t v[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                v[j] = acc_t{0, 0, 0, 0};
-                if (k0 + j < slices) v[j] = ld16_device(&partials[((long)(k0 + j) * g.N + col) * 4 + quad]);
+                // past the last slice: the last slice again (a valid address), its value unused
+                const int ksl = k0 + j < slices ? k0 + j : slices - 1;
+                v[j] = load16_agent<acc_t>(part, (((unsigned)ksl * g.N + col) * 4 + quad) * 16u);
             }
-            // the loaded registers are operands of the wait, so that no use of them can be scheduled ahead of it
-            asm volatile("s_waitcnt vmcnt(0)"
-                         : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
-                         :
-                         : "memory");
 #pragma unroll
             for (int j = 0; j < 8; j++)
                 if (k0 + j < slices) s += v[j];
@@ -353,7 +369,7 @@ int launch_splitk(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, con
     constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB, STEP = CHUNK * 4 * EPL;
     if (g.batches != 1 || g.M <= 4 || g.N < 8 * SK_ROWS || g.K < 4 * STEP) return HODU_ROCM_UNSUPPORTED;
     const int n_blocks = (g.N + SK_ROWS - 1) / SK_ROWS;
-    if (n_blocks > kArrivalSlots) return HODU_ROCM_UNSUPPORTED;
+    if (n_blocks > kArrivalSlots || (long)g.N * 64 * 64 > 0xFFFFFFFFL) return HODU_ROCM_UNSUPPORTED;  // 32-bit buffer offsets
     // Measured against the one-pass kernel (f8 and bf16 weights, M = 5..16): the arrival counter and the last
     // workgroup's second look at the sums cost about 2 us, which pays off once the weights take 16 MB and x is
     // half as large as a workgroup's share of them, or 32 MB whatever M is, or when N is too small to give the

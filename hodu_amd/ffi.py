@@ -12,9 +12,11 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libhodu_rocm_kernels.so")
+# test and measurement hooks (include/hodu_rocm_debug.h): a library of their own, not part of the boundary
+DEBUG_LIB_PATH = os.path.join(_HERE, "lib", "libhodu_rocm_debug.so")
 
-OK, INVALID_ARG, UNSUPPORTED, HIP_ERROR, OOM = 0, 1, 2, 3, 4
-_STATUS = {1: "INVALID_ARG", 2: "UNSUPPORTED", 3: "HIP_ERROR", 4: "OOM"}
+OK, INVALID_ARG, UNSUPPORTED, HIP_ERROR, OOM, SCRATCH = 0, 1, 2, 3, 4, 5
+_STATUS = {1: "INVALID_ARG", 2: "UNSUPPORTED", 3: "HIP_ERROR", 4: "OOM", 5: "SCRATCH"}
 
 # dtype ids: crates/hodu_core/src/types/dtype.rs:6-28
 DTYPE_ID = {
@@ -35,6 +37,7 @@ class HoduRocmError(RuntimeError):
 
 
 _lib: Optional[ctypes.CDLL] = None
+_debug_lib: Optional[ctypes.CDLL] = None
 
 
 class EpilogueStep(ctypes.Structure):
@@ -95,11 +98,6 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_last_error.restype = ctypes.c_char_p
     lib.hodu_rocm_last_kernel.argtypes = [vp]
     lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
-    lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
-    lib.hodu_rocm_debug_force_splitk.argtypes = [vp, ci]
-    lib.hodu_rocm_debug_time_product.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz, ci,
-                                                 ctypes.POINTER(ctypes.c_float)]
-    lib.hodu_rocm_debug_time_product_graph.argtypes = lib.hodu_rocm_debug_time_product.argtypes
     lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
                                           ctypes.POINTER(sz)]
     lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
@@ -112,22 +110,39 @@ def load() -> ctypes.CDLL:
     for dt in EPILOGUE_DTYPES + list(FUSED_PRODUCTS):
         for op in ("matmul", "dot"):
             getattr(lib, f"hodu_rocm_{op}_{dt}_ex").argtypes = [vp, vp, vp, vp, szp, sz, ctypes.POINTER(EpilogueStep), sz]
-    lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, ctypes.POINTER(vp), sz, vp, szp, sz,
-                                                    ctypes.POINTER(EpilogueStep), sz, ci, ctypes.POINTER(ctypes.c_float)]
-    lib.hodu_rocm_debug_time_cast.argtypes = [vp, ci, ci, ctypes.POINTER(vp), ctypes.POINTER(vp), sz, szp, sz, ci,
-                                              ctypes.POINTER(ctypes.c_float)]
-    lib.hodu_rocm_debug_time_sum.argtypes = [vp, ci, ctypes.POINTER(vp), ctypes.POINTER(vp), sz, szp, sz, ci,
-                                             ctypes.POINTER(ctypes.c_float)]
-    lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, ctypes.POINTER(ctypes.c_float),
-                                               ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
-    lib.hodu_rocm_debug_read_floor.argtypes = [vp, ctypes.POINTER(vp), sz, sz, ci, ctypes.POINTER(ctypes.c_float),
-                                               ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
     lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
     _lib = lib
+    return lib
+
+
+def load_debug() -> ctypes.CDLL:
+    """Load the hooks library (include/hodu_rocm_debug.h); it links against the kernel library."""
+    global _debug_lib
+    if _debug_lib is not None:
+        return _debug_lib
+    load()
+    if not os.path.exists(DEBUG_LIB_PATH):
+        raise ImportError(f"{DEBUG_LIB_PATH} is missing: build it first (python -m hodu_amd.build)")
+    lib = ctypes.CDLL(DEBUG_LIB_PATH)
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    szp, fp = ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_float)
+    vpp = ctypes.POINTER(vp)
+    lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
+    lib.hodu_rocm_debug_force_splitk.argtypes = [vp, ci]
+    lib.hodu_rocm_debug_time_product.argtypes = [vp, ci, ci, ci, vp, vpp, sz, vp, szp, sz, ci, fp]
+    lib.hodu_rocm_debug_time_product_graph.argtypes = lib.hodu_rocm_debug_time_product.argtypes
+    lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, vpp, sz, vp, szp, sz,
+                                                    ctypes.POINTER(EpilogueStep), sz, ci, fp]
+    lib.hodu_rocm_debug_time_cast.argtypes = [vp, ci, ci, vpp, vpp, sz, szp, sz, ci, fp]
+    lib.hodu_rocm_debug_time_sum.argtypes = [vp, ci, vpp, vpp, sz, szp, sz, ci, fp]
+    lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, fp, ctypes.POINTER(ctypes.c_double),
+                                               ctypes.POINTER(ctypes.c_double)]
+    lib.hodu_rocm_debug_read_floor.argtypes = [vp, vpp, sz, sz, ci, fp, fp]
+    _debug_lib = lib
     return lib
 
 
@@ -206,6 +221,11 @@ class Context:
         if rc != 0:
             raise HoduRocmError(rc, self.lib.hodu_rocm_last_error(None).decode())
         self.device = device
+
+    @property
+    def debug(self) -> ctypes.CDLL:
+        """the hooks library, loaded on first use (tests and bench.py only)"""
+        return load_debug()
 
     def close(self):
         if self.handle is not None:
@@ -361,11 +381,11 @@ class Context:
         ms = ctypes.c_float()
         if steps:
             sarr, ns = _steps_array(steps)
-            self._check(self.lib.hodu_rocm_debug_time_product_ex(
+            self._check(self.debug.hodu_rocm_debug_time_product_ex(
                 self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr, n,
                 sarr, ns, int(iters), ctypes.byref(ms)))
             return float(ms.value)
-        fn = self.lib.hodu_rocm_debug_time_product_graph if graph else self.lib.hodu_rocm_debug_time_product
+        fn = self.debug.hodu_rocm_debug_time_product_graph if graph else self.debug.hodu_rocm_debug_time_product
         self._check(fn(self.handle, 1 if op == "matmul" else 0, kind, dtype, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr,
                        n, int(iters), ctypes.byref(ms)))
         return float(ms.value)
@@ -381,7 +401,7 @@ class Context:
         pin = (ctypes.c_void_p * len(ins))(*[b.ptr for b in ins])
         pout = (ctypes.c_void_p * len(outs))(*[b.ptr for b in outs])
         ms = ctypes.c_float()
-        self._check(self.lib.hodu_rocm_debug_time_cast(self.handle, DTYPE_ID[src], DTYPE_ID[dst], pin, pout, len(ins), arr, n,
+        self._check(self.debug.hodu_rocm_debug_time_cast(self.handle, DTYPE_ID[src], DTYPE_ID[dst], pin, pout, len(ins), arr, n,
                                                        int(iters), ctypes.byref(ms)))
         return float(ms.value)
 
@@ -394,7 +414,7 @@ class Context:
         pin = (ctypes.c_void_p * len(ins))(*[b.ptr for b in ins])
         pout = (ctypes.c_void_p * len(outs))(*[b.ptr for b in outs])
         ms = ctypes.c_float()
-        self._check(self.lib.hodu_rocm_debug_time_sum(self.handle, DTYPE_ID[dt], pin, pout, len(ins), arr, n, int(iters),
+        self._check(self.debug.hodu_rocm_debug_time_sum(self.handle, DTYPE_ID[dt], pin, pout, len(ins), arr, n, int(iters),
                                                       ctypes.byref(ms)))
         return float(ms.value)
 
@@ -403,7 +423,7 @@ class Context:
         if operands.nbytes < 16384:
             raise HoduRocmError(INVALID_ARG, "mfma_clock: operands must hold 16 KB")
         ms, tf, mhz = ctypes.c_float(), ctypes.c_double(), ctypes.c_double()
-        self._check(self.lib.hodu_rocm_debug_mfma_clock(self.handle, int(kind), operands.ptr, int(iters), ctypes.byref(ms),
+        self._check(self.debug.hodu_rocm_debug_mfma_clock(self.handle, int(kind), operands.ptr, int(iters), ctypes.byref(ms),
                                                         ctypes.byref(tf), ctypes.byref(mhz)))
         return {"ms": ms.value, "tflops": tf.value, "shader_mhz": mhz.value}
 
@@ -413,18 +433,18 @@ class Context:
             raise HoduRocmError(INVALID_ARG, "read_floor: a buffer is smaller than nbytes")
         ptrs = (ctypes.c_void_p * len(buffers))(*[b.ptr for b in buffers])
         r, e = ctypes.c_float(), ctypes.c_float()
-        self._check(self.lib.hodu_rocm_debug_read_floor(self.handle, ptrs, len(buffers), int(nbytes), int(iters),
+        self._check(self.debug.hodu_rocm_debug_read_floor(self.handle, ptrs, len(buffers), int(nbytes), int(iters),
                                                         ctypes.byref(r), ctypes.byref(e)))
         return {"read_us": r.value, "empty_us": e.value}
 
     def force_tile(self, tile: int):
         """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, 10..14 the pipelined
         kernel's tiles, 30..34 the GEMV kernel's shapes, 35..38 the M <= 16 kernel's, -1 = automatic"""
-        self._check(self.lib.hodu_rocm_debug_force_tile(self.handle, int(tile)))
+        self._check(self.debug.hodu_rocm_debug_force_tile(self.handle, int(tile)))
 
     def force_splitk(self, splits: int):
         """testing hook: K ranges of the pipelined kernels (-1 automatic, 1 never, n forced)"""
-        self._check(self.lib.hodu_rocm_debug_force_splitk(self.handle, int(splits)))
+        self._check(self.debug.hodu_rocm_debug_force_splitk(self.handle, int(splits)))
 
     def last_kernel(self) -> str:
         return self.lib.hodu_rocm_last_kernel(self.handle).decode()

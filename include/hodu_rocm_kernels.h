@@ -46,7 +46,9 @@ enum {
     HODU_ROCM_INVALID_ARG = 1, /* null pointer, malformed or inconsistent metadata */
     HODU_ROCM_UNSUPPORTED = 2, /* dtype / rank outside what the device implements */
     HODU_ROCM_HIP_ERROR = 3,   /* a HIP runtime call failed; see hodu_rocm_last_error */
-    HODU_ROCM_OOM = 4          /* device allocation failed */
+    HODU_ROCM_OOM = 4,         /* device allocation failed */
+    HODU_ROCM_SCRATCH = 5      /* the call may not allocate (its stream is under graph capture) and its kernels need
+                                  more scratch than is there */
 };
 
 /* dtype ids, equal to hodu's repr(u8) DType (crates/hodu_core/src/types/dtype.rs:6-28) */
@@ -80,49 +82,6 @@ int hodu_rocm_timer_stop(hodu_rocm_ctx *ctx, void *timer, float *elapsed_ms); /*
 int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
 /* name of the kernel family the last matmul/dot call on this context dispatched to (diagnostics) */
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
-/* testing hook: pin the MFMA tile variant (0 = 256x256 with 8 wavefronts, 1 = 256x256 with 4,
- * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
- * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; 14 = the pipelined 256x128 tile;
- * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
- * variant that cuts K across workgroups wherever it applies; 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
- * 128 x 128 / 64 x 64 / 32 x 32 tiles;
- * -1 = automatic) so that every compiled variant
- * can be exercised at small sizes */
-int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
-/* testing hook: number of K ranges the pipelined tile kernels cut a product into (each range a workgroup of its
- * own, partial sums added in a fixed order by a second kernel): -1 = automatic (only products too small to
- * fill the machine are cut), 1 = never, n = n ranges wherever the kernel can */
-int hodu_rocm_debug_force_splitk(hodu_rocm_ctx *ctx, int splits);
-/* measurement hook: issues the same product `iters` times back to back from C (no per-launch
- * interpreter overhead), cycling through `n_rhs` right-hand buffers so a small operand cannot sit
- * in the Infinity Cache, bracketed by HIP events on the context's stream; *elapsed_ms is the total.
- * is_matmul selects the metadata format; kind: 0 = plain `dtype`, 1 = bf16 x f8e4m3, 2 = i8 x i8 -> i32 */
-int hodu_rocm_debug_time_product(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                 const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
-                                 size_t metadata_len, int iters, float *elapsed_ms);
-/* the same, with the `iters` launches captured once into a HIP graph (kernel nodes only) and replayed as
- * one graph launch inside the timed region: the per-launch time a caller sees who replays a recorded
- * decode step instead of paying a host round trip per product */
-int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                       const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
-                                       size_t metadata_len, int iters, float *elapsed_ms);
-
-/* measurement hook: the rate and shader clock of a register-only MFMA loop (no LDS, no memory traffic) on
- * caller-supplied operand bits, two workgroups per compute unit.  kind 0: bf16 32x32x16; kind 1: f8e4m3 32x32x64
- * with unit scales.  `operands`: 16 KB of device memory (1024 x 16 bytes: per lane the a and b fragments, twice).
- * *tflops is what the loop sustained, *shader_mhz the clock one wavefront saw (shader-clock counter over the
- * 100 MHz counter).  Under full MFMA load the clock depends on the data, so this is the ceiling a GEMM kernel can
- * approach on that data. */
-int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
-                               double *tflops, double *shader_mhz);
-
-/* measurement hook: `iters` launches of a flat streaming read (16 bytes per lane, eight loads in flight, nothing
- * else) of `bytes` from each of the `n_src` device buffers in turn, and `iters` launches of an empty kernel, each
- * bracketed by HIP events on the context's stream.  *read_us: time per read launch; *empty_us: time per empty launch
- * (the launch cadence).  What the memory system and the launch path allow a kernel that moves `bytes`. */
-int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const *src_list, size_t n_src, size_t bytes, int iters,
-                               float *read_us, float *empty_us);
-
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>
  * (kernels/ops_matrix.c:423, :581).  Narrow floats accumulate in f32 and round once on store.   */
@@ -161,7 +120,6 @@ int hodu_rocm_matmul_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void
                               void *out_i32, const size_t *metadata, size_t metadata_len);
 int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void *rhs_i8,
                            void *out_i32, const size_t *metadata, size_t metadata_len);
-
 /* ---- matmul / dot with the caller's next element-wise kernels fused into the store -------------- *
  * The reference's callers of the product launch an element-wise kernel on its output straight away:
  *   Linear::forward (crates/hodu_nn/src/modules/linear.rs:40-46): matmul, then add(bias)
@@ -217,21 +175,6 @@ HODU_ROCM_DECL_PRODUCT_EX(i32)
 HODU_ROCM_DECL_PRODUCT_EX(i64)
 HODU_ROCM_DECL_PRODUCT_EX(bf16_f8e4m3w) /* vector / scalar in bf16 */
 HODU_ROCM_DECL_PRODUCT_EX(i32_i8i8)     /* vector / scalar in i32 */
-/* measurement hook: `iters` back-to-back launches of hodu_rocm_cast (src != dst) or hodu_rocm_contiguous (src == dst)
- * on one metadata array, walking through n_buffers input / output pairs (so that a stream larger than the last-level
- * cache comes from memory), HIP-event timed on the context's stream. */
-int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src_dtype, int dst_dtype, const void *const *in_list,
-                              void *const *out_list, size_t n_buffers, const size_t *metadata, size_t metadata_len,
-                              int iters, float *elapsed_ms);
-/* measurement hook: the same for hodu_rocm_sum */
-int hodu_rocm_debug_time_sum(hodu_rocm_ctx *ctx, int dtype, const void *const *in_list, void *const *out_list,
-                             size_t n_buffers, const size_t *metadata, size_t metadata_len, int iters, float *elapsed_ms);
-/* measurement hook: hodu_rocm_debug_time_product with fused steps */
-int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind, int dtype, const void *lhs,
-                                    const void *const *rhs_list, size_t n_rhs, void *out, const size_t *metadata,
-                                    size_t metadata_len, const hodu_rocm_epilogue_step *steps, size_t n_steps,
-                                    int iters, float *elapsed_ms);
-
 /* ---- casts and strided gather ------------------------------------------------------------------ *
  * replaces hodu_cpu_cast_<src>_to_<dst> (kernels/ops_cast.c:53, table :108-388) and
  * hodu_cpu_contiguous_<dt> (kernels/ops_memory.c:36).  One entry point taking dtype ids stands

@@ -66,8 +66,7 @@ def check_product(ctx, op, name, lv, rv, seed=0, scale=1.0, rscale=None, expect_
         A = np.abs(lv.broadcast_to(bshape + lv.shape[-2:]).take(a)); B = np.abs(rv.broadcast_to(bshape + rv.shape[-2:]).take(b))
         oabs = (A @ B).ravel()
         assert np.all(np.isfinite(got))
-        rel = H.rel_err(got, want, oabs, k)
-        assert rel.max() <= 1e-12, f"{op} f64: max rel err {rel.max():.3e}"
+        H.assert_close(got, want, oabs, k, 1e-12, f"{op} f64", eps_acc=H.EPS_F64)
         return
     fn = oracle.dot_spec if op == "dot" else oracle.matmul_spec
     o32, o64, oabs = fn(l_dt, r_dt, a, b, md)
@@ -88,5 +87,4 @@ def check_product(ctx, op, name, lv, rv, seed=0, scale=1.0, rscale=None, expect_
     # (a sequential f32 sum over more than a few thousand k is itself off by about sqrt(k) * 2^-24 relative to the
     # floor: products with a very long K, which the device adds in chunks, are held to the float64 value)
     want = o64 if (out_dt == "f64" or (out_dt == "f32" and k > 16384)) else o32.astype(np.float64)
-    rel = H.rel_err(gotf[fin], want[fin], oabs[fin], k)
-    assert rel.size == 0 or rel.max() <= tol, f"{op} {name}: max rel err {rel.max():.3e} > {tol}"
+    H.assert_close(gotf[fin], want[fin], oabs[fin], k, tol, f"{op} {name}")

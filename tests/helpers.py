@@ -228,18 +228,58 @@ def widen(dt: str, x: np.ndarray, ocp=True) -> np.ndarray:
     return x.astype(np.float64)
 
 
-def rel_err(got: np.ndarray, want: np.ndarray, sumabs: np.ndarray, k: int) -> np.ndarray:
-    """Per-element relative error with a floor under the denominator.
+# unit round-off of the accumulator a product is summed in
+EPS_F32, EPS_F64 = 2.0 ** -24, 2.0 ** -53
+# Constant of the rounding-model floor.  A sum of K products accumulated in a type of unit round-off eps, in any
+# order, is off by a random walk of about 0.5 * eps * sum|a b| (standard deviation: each partial sum of zero-mean
+# terms is ~ sqrt(k) terms large and is rounded once); the largest of 10^7 such errors is ~ 3 * eps * sum|a b|, and
+# the comparator's own f32 sum carries the same.  8 leaves a factor of two above that.
+FLOOR_C = 8.0
 
-    A sum of K zero-mean products can cancel to (almost) zero while every rounding step still
-    contributes an absolute error proportional to sum|a_k b_k|; dividing by |want| alone then
-    reports arbitrarily large 'relative' errors for a correct kernel (of 10^7 outputs a few are
-    10^-6 of the typical magnitude).  The denominator is therefore
-        max(|want|, sum_k|a_k b_k| / sqrt(K)),
-    i.e. an output that cancelled below the magnitude a random-sign sum of its own products
-    would have is judged relative to that magnitude.  Outputs of ordinary size are judged
-    against |want| alone.
-    """
-    den = np.maximum(np.abs(want), np.asarray(sumabs, dtype=np.float64) / np.sqrt(max(int(k), 1)))
+
+def rel_floor(sumabs, k: int, tol: float, eps_acc: float = EPS_F32) -> np.ndarray:
+    """The least denominator an element is judged against: the smaller of
+      * sum|a b| / sqrt(K): the magnitude a random-sign sum of the element's own products would have (no element is
+        ever judged against something larger than an ordinary output), and
+      * FLOOR_C * eps_acc * sum|a b| / tol: the accumulation error of a correct kernel expressed in units of `tol`,
+        so that an element which cancelled to (almost) zero is allowed exactly that absolute error and no more.
+    For bf16 / f16 / fp8 outputs at tol = 2e-2 the second is the smaller by two to three orders of magnitude
+    (2.4e-5 * sum|a b| against 1.6e-2 * sum|a b| at K = 4096); for f32 outputs at 1e-5 the two are comparable."""
+    sumabs = np.asarray(sumabs, dtype=np.float64)
+    return np.minimum(sumabs / np.sqrt(max(int(k), 1)), FLOOR_C * eps_acc * sumabs / tol)
+
+
+def rel_err(got: np.ndarray, want: np.ndarray, sumabs: np.ndarray, k: int, tol: float,
+            eps_acc: float = EPS_F32) -> np.ndarray:
+    """Per-element relative error |got - want| / max(|want|, rel_floor).
+
+    Dividing by |want| alone reports arbitrarily large 'relative' errors for a correct kernel on the few of 10^7
+    zero-mean sums that cancel to ~0; the floor (rel_floor) is what the accumulator's rounding alone can contribute
+    there, expressed in units of the tolerance the caller is about to apply.  An element of ordinary size is judged
+    against |want| alone: at bf16 tolerances and K = 4096 that is every element above ~0.1 % of the typical output
+    magnitude."""
+    den = np.maximum(np.abs(want), rel_floor(sumabs, k, tol, eps_acc))
     den = np.where(den == 0, 1.0, den)
-    return np.abs(got.astype(np.float64) - want) / den
+    return np.abs(np.asarray(got, dtype=np.float64) - want) / den
+
+
+def floor_fraction(want, sumabs, k: int, tol: float, eps_acc: float = EPS_F32) -> float:
+    """fraction of elements whose denominator is the floor rather than |want|"""
+    want = np.asarray(want, dtype=np.float64)
+    return float(np.mean(np.abs(want) < rel_floor(sumabs, k, tol, eps_acc))) if want.size else 0.0
+
+
+def assert_close(got, want, sumabs, k: int, tol: float, what: str = "", eps_acc: float = EPS_F32):
+    """asserts rel_err <= tol for every element; the message names the worst element and how many elements were
+    judged on the floor"""
+    got = np.asarray(got, dtype=np.float64).ravel()
+    want = np.asarray(want, dtype=np.float64).ravel()
+    sumabs = np.asarray(sumabs, dtype=np.float64).ravel()
+    if got.size == 0:
+        return
+    rel = rel_err(got, want, sumabs, k, tol, eps_acc)
+    worst = int(np.argmax(rel))
+    assert rel[worst] <= tol, (
+        f"{what}: max rel err {rel[worst]:.3e} > {tol:g} at element {worst} (got {got[worst]!r}, want {want[worst]!r}, "
+        f"sum|ab| {sumabs[worst]!r}); {int((rel > tol).sum())} of {rel.size} elements fail; "
+        f"{100 * floor_fraction(want, sumabs, k, tol, eps_acc):.2f} % of elements are judged on the floor")

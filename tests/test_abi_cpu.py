@@ -11,11 +11,18 @@ from hodu_amd import ffi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "hodu_rocm_kernels.h")
+DEBUG_HEADER = os.path.join(ROOT, "include", "hodu_rocm_debug.h")
 
 
-def declared_symbols():
-    text = subprocess.check_output(["gcc", "-E", "-P", HEADER], text=True)
+def declared_symbols(header=HEADER):
+    text = subprocess.check_output(["gcc", "-E", "-P", f"-I{ROOT}/include", header], text=True)
     return sorted(set(re.findall(r"\b(hodu_rocm_\w+)\s*\(", text)))
+
+
+def exported_symbols(path):
+    out = subprocess.check_output(["nm", "-D", "--defined-only", path], text=True)
+    return sorted({line.split()[-1] for line in out.splitlines() if " T " in line and "hodu_rocm_" in line
+                   and not line.split()[-1].startswith("_Z")})
 
 
 def test_library_exports_every_declared_symbol():
@@ -27,6 +34,20 @@ def test_library_exports_every_declared_symbol():
             assert f"hodu_rocm_{op}_{dt}" in names
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
+    # and nothing else: the kernel library is the drop-in boundary, so every extern "C" hodu_rocm_* symbol it
+    # exports is one the header declares (test and measurement hooks live in the hooks library)
+    assert not [n for n in names if "debug" in n]
+    extra = sorted(set(exported_symbols(ffi.LIB_PATH)) - set(names))
+    assert not extra, extra
+
+
+def test_hooks_library_exports_what_its_header_declares():
+    lib = ffi.load_debug()
+    names = sorted(set(declared_symbols(DEBUG_HEADER)) - set(declared_symbols()))
+    assert names and all(n.startswith("hodu_rocm_debug_") for n in names), names
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert sorted(exported_symbols(ffi.DEBUG_LIB_PATH)) == names
 
 
 def test_header_compiles_as_c_and_cxx(tmp_path):

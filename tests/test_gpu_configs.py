@@ -34,8 +34,7 @@ def check_rows(got_rows, l_dt, r_dt, a, b, md_rows, k, tol):
     o32, o64, oabs = oracle.dot_spec(l_dt, r_dt, a, b, md_rows)
     gotf = H.bf16_to_f32(got_rows).astype(np.float64) if got_rows.dtype == np.uint16 else got_rows.astype(np.float64)
     assert np.all(np.isfinite(gotf)) and np.all(np.isfinite(o32))
-    rel = H.rel_err(gotf, o32.astype(np.float64), oabs, k)
-    assert rel.max() <= tol, f"max rel err {rel.max():.3e}"
+    H.assert_close(gotf, o32.astype(np.float64), oabs, k, tol, f"{l_dt} x {r_dt}, K = {k}")
 
 
 def test_config1_f32_512(ctx):
@@ -46,11 +45,11 @@ def test_config1_f32_512(ctx):
     assert ctx.last_kernel() == "small_f32_KM"
     want = oracle.dot_asis("f32", a, b, md)  # sequential-k f32, the reference's fallback arithmetic
     _, o64, oabs = oracle.dot_spec("f32", "f32", a, b, md)
-    assert H.rel_err(got, want.astype(np.float64), oabs, 512).max() <= 1e-5
-    assert H.rel_err(got, o64, oabs, 512).max() <= 1e-5
+    H.assert_close(got, want.astype(np.float64), oabs, 512, 1e-5, "config 1 against the sequential-k f32 sum")
+    H.assert_close(got, o64, oabs, 512, 1e-5, "config 1 against float64")
     # the OpenBLAS flavour of the reference (cblas_sgemm) through numpy's bundled OpenBLAS
     blas = (a.reshape(512, 512) @ b.reshape(512, 512)).ravel()
-    assert H.rel_err(got, blas.astype(np.float64), oabs, 512).max() <= 1e-5
+    H.assert_close(got, blas.astype(np.float64), oabs, 512, 1e-5, "config 1 against sgemm")
 
 
 def test_config2_bf16_batched_transposed(ctx):

@@ -1,0 +1,118 @@
+"""Exact-valued products, compared bit for bit.
+
+Small-integer operands (bf16 activations in [-4, 4], f8e4m3 / bf16 weights in [-8, 8]) make every product and every
+partial sum an integer below 2^24, so an f32 accumulator holds the exact sum whatever the order of addition, and
+the one rounding to bf16 is the same on every correct kernel: the float kernels that have no integer twin (the
+row-streaming GEMV, the M <= 16 kernel and its split-K form, the f8e4m3-weight pipelined tile kernel, split-K through
+the workspace) are held to equality here, where the tolerance tests allow 2e-2.  A dropped or doubled k-term, a
+wrong decode of one f8 code or a stale partial sum changes the integer and fails.
+"""
+import numpy as np
+import pytest
+
+import helpers as H
+from hodu_amd import ffi
+
+pytestmark = pytest.mark.gpu
+V = H.View
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = ffi.Context(0)
+    yield c
+    c.force_tile(-1)
+    c.force_splitk(-1)
+    c.close()
+
+
+def int_bf16(seed, n, top):
+    return H.f32_to_bf16_rne(H.rng(seed).integers(-top, top + 1, n).astype(np.float32))
+
+
+def int_f8(seed, n, top=8):
+    codes = H.f32_to_ocp_e4m3_rne(H.rng(seed).integers(-top, top + 1, n).astype(np.float64))
+    assert np.array_equal(H.ocp_e4m3_decode(codes), np.round(H.ocp_e4m3_decode(codes)))  # integers survive the encoding
+    return codes
+
+
+def run_exact(ctx, op, name, lv, rv, seed, expect_kernel):
+    l_dt, r_dt = ("bf16", "f8e4m3") if name == "bf16_f8e4m3w" else ("bf16", "bf16")
+    a = int_bf16(100 + seed, max(lv.span(), 1), 4)
+    b = int_f8(200 + seed, max(rv.span(), 1)) if r_dt == "f8e4m3" else int_bf16(200 + seed, max(rv.span(), 1), 8)
+    md = H.dot_md(lv, rv) if op == "dot" else H.matmul_md(lv, rv)
+    n_out = int(md[0]) if op == "matmul" else int(md[0]) * int(md[2])
+    da, db, dout = ctx.upload(a), ctx.upload(b), ctx.alloc(2 * n_out)
+    ctx.fill(dout, 0xFF)
+    ctx.product(op, name, da, db, dout, md)
+    got = ctx.download(dout, np.uint16, n_out)
+    kernel = ctx.last_kernel()
+    for d in (da, db, dout):
+        d.free()
+    assert kernel.startswith(expect_kernel), (kernel, expect_kernel)
+    bshape = list(np.broadcast_shapes(tuple(lv.shape[:-2]), tuple(rv.shape[:-2])))
+    A = H.widen(l_dt, lv.broadcast_to(bshape + lv.shape[-2:]).take(a))
+    B = H.widen(r_dt, rv.broadcast_to(bshape + rv.shape[-2:]).take(b))
+    exact = A @ B  # float64 of integers: exact
+    assert np.abs(exact).max() < 2 ** 24
+    want = H.f32_to_bf16_rne(exact.astype(np.float32).ravel())
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, f"{kernel}: {bad.size} of {got.size} outputs differ, first at {bad[:5]}"
+    return kernel
+
+
+@pytest.mark.parametrize("name", ["bf16_f8e4m3w", "bf16"])
+@pytest.mark.parametrize("m", [1, 2, 4])
+def test_row_streaming_gemv(ctx, name, m):
+    pre = "gemv_bf16_f8w" if name == "bf16_f8e4m3w" else "gemv_bf16"
+    run_exact(ctx, "dot", name, V([m, 4096]), V([1024, 4096]).t(), m, pre)
+    run_exact(ctx, "dot", name, V([m, 4112]), V([203, 4112]).t(), 10 + m, pre)
+
+
+@pytest.mark.parametrize("name", ["bf16_f8e4m3w", "bf16"])
+@pytest.mark.parametrize("m", [5, 16])
+def test_one_pass_and_split_k_skinny(ctx, name, m):
+    pre = "skinny_bf16_f8w" if name == "bf16_f8e4m3w" else "skinny_bf16"
+    for shape in (35, 36, 37):
+        ctx.force_tile(shape)
+        run_exact(ctx, "dot", name, V([m, 4096]), V([1040, 4096]).t(), m, pre)
+    ctx.force_tile(38)
+    for _ in range(2):
+        k = run_exact(ctx, "dot", name, V([m, 4224]), V([1100, 4224]).t(), 20 + m, pre)
+        assert k.endswith("_splitk")
+    ctx.force_tile(-1)
+
+
+def test_config3_m16_takes_the_split_k_kernel_exactly(ctx):
+    k = run_exact(ctx, "dot", "bf16_f8e4m3w", V([16, 4096]), V([4096, 4096]).t(), 3, "skinny_bf16_f8w")
+    assert k.endswith("_splitk")
+
+
+@pytest.mark.parametrize("tile", [10, 11, 12, 14])
+@pytest.mark.parametrize("combo", ["KK", "KM"])
+def test_f8_weight_pipelined_tiles(ctx, tile, combo):
+    """every tile shape of the pipelined kernel on f8e4m3 weights, k-dense ([N, K]^T view) and row-dense ([K, N])"""
+    rv = V([384, 1024]).t() if combo == "KK" else V([1024, 384])
+    ctx.force_tile(tile)
+    try:
+        run_exact(ctx, "dot", "bf16_f8e4m3w", V([296, 1024]), rv, tile, "mfma_bf16_f8w_pipe")
+        run_exact(ctx, "dot", "bf16", V([296, 1024]), V([384, 1024]).t() if combo == "KK" else V([1024, 384]), tile,
+                  "mfma_bf16_pipe")
+    finally:
+        ctx.force_tile(-1)
+
+
+@pytest.mark.parametrize("splits", [2, 4, 7])
+def test_pipelined_split_k_through_the_workspace(ctx, splits):
+    ctx.force_splitk(splits)
+    try:
+        for name in ("bf16_f8e4m3w", "bf16"):
+            k = run_exact(ctx, "dot", name, V([256, 4096]), V([512, 4096]).t(), splits, "mfma_bf16")
+            assert "splitk" in k, k
+    finally:
+        ctx.force_splitk(-1)
+
+
+def test_batched_and_broadcast_exact(ctx):
+    run_exact(ctx, "matmul", "bf16", V([3, 160, 512]), V([3, 136, 512]).t(), 1, "mfma_bf16")
+    run_exact(ctx, "matmul", "bf16_f8e4m3w", V([4, 128, 512]), V([512, 256]).broadcast_to([4, 512, 256]), 2, "mfma_bf16_f8w")

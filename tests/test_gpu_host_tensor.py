@@ -131,7 +131,7 @@ def test_f8_weight_cast_is_deferred_and_fused():
     lv, rv = H.View([m, k]), H.View([n, k]).t()
     want32, _, sumabs = oracle.dot_spec("bf16", "f8e4m3", xb, w8, H.dot_md(lv, rv), decode=oracle.F8_OCP)
     got = H.bf16_to_f32(y.to_bits())
-    assert H.rel_err(got, want32, sumabs, k).max() <= 2e-2  # bf16 output, f32 accumulate
+    H.assert_close(got, want32, sumabs, k, 2e-2, "bf16 output, f32 accumulate")
     # reading the deferred tensor materialises the cast: bit-exact with the cast oracle (OCP decode)
     want_bits = oracle.cast("f8e4m3", "bf16", w8, H.cast_md(H.View([n, k])), decode=oracle.F8_OCP)
     assert np.array_equal(wb.to_bits(), want_bits)
@@ -139,7 +139,7 @@ def test_f8_weight_cast_is_deferred_and_fused():
     wt_dense = w.t().to_dtype("bf16")  # non-dense input: materialised, [k, n] contiguous
     assert wt_dense.physical_dtype == "bf16"
     y2 = x.matmul(wt_dense)
-    assert H.rel_err(H.bf16_to_f32(y2.to_bits()), want32, sumabs, k).max() <= 2e-2
+    H.assert_close(H.bf16_to_f32(y2.to_bits()), want32, sumabs, k, 2e-2, "deferred cast")
 
 
 def test_i8_casts_are_deferred_and_the_product_is_bit_exact():
@@ -185,7 +185,7 @@ def test_reference_mode_copies_and_nocopy_mode_agree_bit_for_bit():
     assert y_ref.shape == [b, s, d] and np.array_equal(y_ref.to_bits(), y_new.to_bits())
     lv, rv = H.View([b, s, f]), H.View([d, f]).t().broadcast_to([b, f, d])
     want32, _, sumabs = oracle.matmul_spec("bf16", "bf16", xb, wb, H.matmul_md(lv, rv))
-    assert H.rel_err(H.bf16_to_f32(y_new.to_bits()), want32, sumabs, f).max() <= 2e-2
+    H.assert_close(H.bf16_to_f32(y_new.to_bits()), want32, sumabs, f, 2e-2, "no-copy mode")
 
 
 def test_to_dtype_of_a_view_matches_the_cast_oracle():
@@ -385,10 +385,11 @@ def test_linear_backward_bf16_against_f32_accumulated_comparator():
             dx, dw = T.matmul_vjp(tx, tw, tg)
         finally:
             T.set_matmul_mode("nocopy")
-        rel = H.rel_err(H.bf16_to_f32(dw.to_bits()).astype(np.float64), want_dw.ravel(), abs_dw.ravel(), 512)
-        assert rel.max() <= 2e-2, (mode, rel.max())
-        rel = H.rel_err(H.bf16_to_f32(dx.to_bits()).astype(np.float64), want_dx.ravel(), abs_dx.ravel(), 192)
-        assert rel.max() <= 2e-2, (mode, rel.max())
+        # the reference sequence rounds every batch's [K, N] product to bf16 before sum_to_shape adds them: its
+        # error on an element that cancels is a bf16 rounding of the per-batch parts, not an f32 accumulation error
+        H.assert_close(H.bf16_to_f32(dw.to_bits()), want_dw.ravel(), abs_dw.ravel(), 512, 2e-2, f"dW, {mode}",
+                       eps_acc=2.0 ** -9 if mode == "reference" else H.EPS_F32)
+        H.assert_close(H.bf16_to_f32(dx.to_bits()), want_dx.ravel(), abs_dx.ravel(), 192, 2e-2, f"dX, {mode}")
 
 
 # ---- attention core (hodu_nn/src/modules/attention.rs:25-70) ----------------------------------------------

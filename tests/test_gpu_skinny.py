@@ -167,3 +167,52 @@ def test_row_dense_weight_views_and_fallbacks(ctx, kind):
 def test_row_dense_weight_other_kinds_keep_the_tile_kernels(ctx):
     check_product(ctx, "dot", "bf16_f8e4m3w", V([1, 256]), V([256, 64]), seed=4, rscale=2.0, expect_kernel="mfma_")
     check_product(ctx, "dot", "i32_i8i8", V([2, 256]), V([256, 64]), seed=5, expect_kernel="mfma_")
+
+
+def test_split_k_arrival_protocol_over_thousands_of_launches(ctx):
+    """Config 3 at M = 16 (the automatic choice is the split-K kernel) 3072 times back to back over 48 weight buffers
+    whose rows are rotated by a different amount each -- so a partial sum left over from the previous launch, or one
+    read before its writer's store was visible, gives a different output -- into a ring of 64 output buffers, every one
+    of them compared bit for bit with the one-pass kernel's result on the unrotated weight, stopping at the first
+    mismatch."""
+    import numpy as np
+    m, n, k = 16, 4096, 4096
+    x = H.random_storage("bf16", m * k, 71)
+    w = H.random_storage("f8e4m3", n * k, 72, 30.0)
+    md = H.dot_md(V([m, k]), V([n, k]).t())
+    dx, dw = ctx.upload(x), ctx.upload(w)
+    ref = ctx.alloc(m * n * 2)
+    ctx.force_tile(36)
+    try:
+        ctx.product("dot", "bf16_f8e4m3w", dx, dw, ref, md)
+        assert not ctx.last_kernel().endswith("_splitk")
+    finally:
+        ctx.force_tile(-1)
+    base = ctx.download(ref, np.uint16).reshape(m, n)
+    copies, ring = 48, 64
+    shifts = [(128 * c + 16 * (c // 32)) % n for c in range(copies)]  # W_c[j] = W[(j + shift_c) % n]
+    ws = []
+    for s in shifts:
+        buf = ctx.alloc(n * k)
+        ctx._check(ctx.lib.hodu_rocm_memcpy_d2d(ctx.handle, buf.ptr, dw.ptr + s * k, (n - s) * k))
+        if s:
+            ctx._check(ctx.lib.hodu_rocm_memcpy_d2d(ctx.handle, buf.ptr + (n - s) * k, dw.ptr, s * k))
+        ws.append(buf)
+    outs = [ctx.alloc(m * n * 2) for _ in range(ring)]
+    launch = 0
+    try:
+        for _ in range(3072 // ring):
+            used = []
+            for slot in range(ring):
+                c = launch % copies
+                ctx.product("dot", "bf16_f8e4m3w", dx, ws[c], outs[slot], md)
+                used.append(c)
+                launch += 1
+            assert ctx.last_kernel() == "skinny_bf16_f8w_splitk"
+            for slot, c in enumerate(used):
+                got = ctx.download(outs[slot], np.uint16).reshape(m, n)
+                want = np.roll(base, -shifts[c], axis=1)
+                assert np.array_equal(got, want), f"launch {launch - ring + slot} (weight copy {c}) differs"
+    finally:
+        for b in [dx, dw, ref] + ws + outs:
+            b.free()

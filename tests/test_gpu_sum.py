@@ -44,7 +44,7 @@ def check_sum(ctx, dt, v, dims, keep, seed=0, expect_kernel=None):
     gotf = H.widen(dt, got)
     assert np.all(np.isfinite(gotf))
     if dt == "f64":
-        assert H.rel_err(gotf, o64, oabs, max(r, 1)).max() <= 1e-12
+        H.assert_close(gotf, o64, oabs, max(r, 1), 1e-12, f"sum {dt}", eps_acc=H.EPS_F64)
     elif dt in ("f8e4m3", "f8e5m2"):
         step, lim, tiny = (2.0 ** -3, 448.0, 2.0 ** -9) if dt == "f8e4m3" else (2.0 ** -2, 57344.0, 2.0 ** -16)
         want = np.clip(o64, -lim, lim)
@@ -55,8 +55,7 @@ def check_sum(ctx, dt, v, dims, keep, seed=0, expect_kernel=None):
         # floor used here (1e-5 at r = 10^5); the device adds in chunks and trees, so long f32 reductions are held to
         # the exact (float64) sum instead of to the sequential f32 one
         want = o64 if (dt == "f32" and r > 4096) else o32.astype(np.float64)
-        rel = H.rel_err(gotf, want, oabs, max(r, 1))
-        assert rel.max() <= tol, f"sum {dt}: max rel err {rel.max():.3e} > {tol}"
+        H.assert_close(gotf, want, oabs, max(r, 1), tol, f"sum {dt}")
 
 
 @pytest.mark.parametrize("dt", oracle.MATMUL_DTYPES)
