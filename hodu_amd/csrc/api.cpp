@@ -221,6 +221,36 @@ int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, voi
     return dot_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
 }
 
+// The one entry point that allocates nothing: hodu_rocm_dot_bf16_f8e4m3w with the partial sums and arrival counters
+// of its split-K kernels in the device's static scratch array instead of the context's workspace.  For the length
+// of the call the context's workspace / counters are pointed at that array and marked fixed, so a kernel choice that
+// needs more is refused (ensure_workspace) rather than grown; the counters are zeroed by a kernel first, because the
+// array is shared by every call on this GPU and keeps whatever the last one left.
+int hodu_rocm_dot_bf16_f8e4m3w_noalloc(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,
+                                       size_t n) {
+    clear_error();
+    int rc = check_ptrs("dot", ctx, l, r, o);
+    if (rc) return rc;
+    Product p;
+    rc = parse_dot_metadata(md, n, &p);
+    if (rc) return rc;
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    HODU_HIP(hipSetDevice(ctx->device));
+    if (!ctx->static_scratch) return fail(HODU_ROCM_HIP_ERROR, "dot: the static scratch is not set up on this context");
+    const Workspace saved_ws = ctx->workspace;
+    int *const saved_arrival = ctx->arrival;
+    ctx->workspace.ptr = (char *)ctx->static_scratch + kStaticArrivalBytes;
+    ctx->workspace.bytes = kStaticPartialBytes;
+    ctx->arrival = (int *)ctx->static_scratch;
+    ctx->fixed_scratch = true;
+    rc = clear_static_arrival(ctx);
+    if (rc == HODU_ROCM_OK) rc = run_product(ctx, PK_BF16_F8W, HODU_BF16, l, r, o, p, DevEpilogue{});
+    ctx->workspace = saved_ws;
+    ctx->arrival = saved_arrival;
+    ctx->fixed_scratch = false;
+    return rc;
+}
+
 #define HODU_ROCM_DEF_PRODUCT_EX(dt, KIND, ID)                                                                  \
     int hodu_rocm_matmul_##dt##_ex(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md, \
                                    size_t n, const hodu_rocm_epilogue_step *steps, size_t n_steps) {           \

@@ -30,6 +30,10 @@ struct hodu_rocm_ctx {
     hipDeviceProp_t props{};
     hodu::Workspace workspace;  // split-K partial sums; grown on demand, owned by the context
     int *arrival = nullptr;     // kArrivalSlots zeroed counters for kernels whose last workgroup finishes a reduction
+    // Set for the duration of a call that must not allocate: `workspace` and `arrival` then point into the
+    // device's static scratch array, and a kernel that needs more than it holds is refused instead of grown.
+    bool fixed_scratch = false;
+    void *static_scratch = nullptr;  // this device's copy of the static scratch array (hipGetSymbolAddress)
     const char *last_kernel = "";
     int force_tile = -1;    // testing hook: pins the MFMA tile size
     int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
@@ -74,12 +78,20 @@ inline int ensure_dynamic_lds(hodu_rocm_ctx *ctx, const void *kernel, int bytes)
     return HODU_ROCM_OK;
 }
 
-// grows ctx->workspace to at least `bytes` (refused, with an error text, while the context's stream is being
-// captured into a graph and it would have to grow)
+// grows ctx->workspace to at least `bytes` (refused, with an error text, while ctx->fixed_scratch is set and the
+// static scratch is smaller, or while the context's stream is being captured into a graph and it would have to grow)
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes);
 // allocates (once) and zeroes ctx->arrival; kernels that use a counter leave it at zero again
 constexpr int kArrivalSlots = 4096;
 int ensure_arrival(hodu_rocm_ctx *ctx);
+
+// The static scratch array of the entry point that allocates nothing: kArrivalSlots counters, then partial sums.
+constexpr size_t kStaticArrivalBytes = (size_t)kArrivalSlots * sizeof(int);
+constexpr size_t kStaticPartialBytes = (size_t)8 << 20;
+constexpr size_t kStaticScratchBytes = kStaticArrivalBytes + kStaticPartialBytes;
+// launches the small kernel that zeroes the counters at the head of the static scratch (no memset node: callers may
+// be capturing a graph)
+int clear_static_arrival(hodu_rocm_ctx *ctx);
 
 inline size_t dtype_size(int dt) {
     static const size_t sz[15] = {1, 1, 1, 2, 2, 4, 8, 1, 2, 4, 8, 1, 2, 4, 8};

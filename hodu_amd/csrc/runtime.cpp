@@ -29,6 +29,29 @@ int fail(int code, const char *fmt, ...) {
 
 namespace {
 
+// Scratch of the entry point that allocates nothing: arrival counters first, partial sums behind them.  Every GPU
+// the library runs on holds its own copy of this array until the process ends.  In host code the NAME is only a
+// handle for hipGetSymbolAddress; kernels and copies get the per-device address that call returns.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {};  // per device: where that device keeps its copy of `scratch`
+
+// with `device` current: the device's address of the static scratch array, looked up once per device
+int static_scratch_of(int device, void **ptr) {
+    if (device < 0 || device >= kMaxDevices) return fail(HODU_ROCM_UNSUPPORTED, "device id %d beyond %d", device, kMaxDevices);
+    std::lock_guard<std::mutex> hold(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        HODU_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(HODU_ROCM_HIP_ERROR, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_scratch_ptr[device] = p;
+    }
+    *ptr = g_scratch_ptr[device];
+    return HODU_ROCM_OK;
+}
+
 __global__ __launch_bounds__(1024) void clear_words_kernel(int *__restrict__ p, int n) {
     const int i = blockIdx.x * 1024 + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -43,6 +66,10 @@ bool stream_is_capturing(hipStream_t s) {
 
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
     if (ctx->workspace.bytes >= bytes) return HODU_ROCM_OK;
+    if (ctx->fixed_scratch)
+        return fail(HODU_ROCM_SCRATCH,
+                    "this product needs %zu bytes of partial sums; the static scratch of the entry point that "
+                    "allocates nothing holds %zu", bytes, ctx->workspace.bytes);
     if (stream_is_capturing(ctx->stream))
         return fail(HODU_ROCM_SCRATCH, "the workspace would have to grow to %zu bytes while the stream is being "
                     "captured: run the product once outside the capture first", bytes);
@@ -59,6 +86,7 @@ int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
 
 int ensure_arrival(hodu_rocm_ctx *ctx) {
     if (ctx->arrival) return HODU_ROCM_OK;
+    if (ctx->fixed_scratch) return fail(HODU_ROCM_HIP_ERROR, "static scratch is not set up on this context");
     if (stream_is_capturing(ctx->stream))
         return fail(HODU_ROCM_SCRATCH, "the arrival counters would be allocated while the stream is being "
                     "captured: run the product once outside the capture first");
@@ -66,6 +94,14 @@ int ensure_arrival(hodu_rocm_ctx *ctx) {
     // zeroed by a kernel, in stream order, before any kernel of this context can count on them
     hipLaunchKernelGGL(clear_words_kernel, dim3((kArrivalSlots + 1023) / 1024), dim3(1024), 0, ctx->stream, ctx->arrival,
                        kArrivalSlots);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
+int clear_static_arrival(hodu_rocm_ctx *ctx) {
+    if (!ctx->static_scratch) return fail(HODU_ROCM_HIP_ERROR, "static scratch is not set up on this context");
+    hipLaunchKernelGGL(clear_words_kernel, dim3((kArrivalSlots + 1023) / 1024), dim3(1024), 0, ctx->stream,
+                       (int *)ctx->static_scratch, kArrivalSlots);
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;
 }
@@ -115,6 +151,13 @@ int hodu_rocm_ctx_create(int device, hodu_rocm_ctx **out) {
         (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return fail(HODU_ROCM_UNSUPPORTED, "device %d is %s; this library carries gfx950 code only", device, arch);
+    }
+    // this device's address of the static scratch array (the device is current): kept for the entry point that
+    // allocates nothing
+    if (int rc = static_scratch_of(device, &ctx->static_scratch)) {
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return rc;
     }
     *out = ctx;
     return HODU_ROCM_OK;

@@ -143,6 +143,16 @@ int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind,
                              steps, n_steps);
 }
 
+int hodu_rocm_debug_time_noalloc(hodu_rocm_ctx *ctx, const void *lhs, const void *const *rhs_list, size_t n_rhs,
+                                 void *out, const size_t *md, size_t len, int iters, int graph, float *elapsed_ms) {
+    clear_error();
+    if (!ctx || !rhs_list || n_rhs == 0 || !elapsed_ms || iters <= 0)
+        return fail(HODU_ROCM_INVALID_ARG, "time_noalloc: bad argument");
+    return timed_loop(ctx, graph != 0, iters, elapsed_ms, [&](int i) {
+        return hodu_rocm_dot_bf16_f8e4m3w_noalloc(ctx, lhs, rhs_list[(size_t)i % n_rhs], out, md, len);
+    });
+}
+
 int hodu_rocm_debug_time_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *const *in_list, void *const *out_list,
                               size_t n_buffers, const size_t *md, size_t len, int iters, float *elapsed_ms) {
     clear_error();

@@ -115,6 +115,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
     lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
+    lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc.argtypes = [vp, vp, vp, vp, szp, sz]
     _lib = lib
     return lib
 
@@ -137,6 +138,7 @@ def load_debug() -> ctypes.CDLL:
     lib.hodu_rocm_debug_time_product_graph.argtypes = lib.hodu_rocm_debug_time_product.argtypes
     lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, vpp, sz, vp, szp, sz,
                                                     ctypes.POINTER(EpilogueStep), sz, ci, fp]
+    lib.hodu_rocm_debug_time_noalloc.argtypes = [vp, vp, vpp, sz, vp, szp, sz, ci, ci, fp]
     lib.hodu_rocm_debug_time_cast.argtypes = [vp, ci, ci, vpp, vpp, sz, szp, sz, ci, fp]
     lib.hodu_rocm_debug_time_sum.argtypes = [vp, ci, vpp, vpp, sz, szp, sz, ci, fp]
     lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, fp, ctypes.POINTER(ctypes.c_double),
@@ -277,6 +279,23 @@ class Context:
         arr, n = _md_array(md)
         fn = getattr(self.lib, f"hodu_rocm_{op}_{name}")
         self._check(fn(self.handle, lhs.ptr, rhs.ptr, out.ptr, arr, n))
+
+    def dot_noalloc(self, lhs: DeviceBuffer, rhs: DeviceBuffer, out: DeviceBuffer, md):
+        """hodu_rocm_dot_bf16_f8e4m3w_noalloc: the fused f8e4m3-weight dot with its scratch in the library's static
+        device array (no device allocation inside the call)"""
+        self._check_extents("dot", "bf16_f8e4m3w", lhs, [rhs], out, md)
+        arr, n = _md_array(md)
+        self._check(self.lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc(self.handle, lhs.ptr, rhs.ptr, out.ptr, arr, n))
+
+    def time_noalloc(self, lhs: DeviceBuffer, rhs_list, out: DeviceBuffer, md, iters: int, graph: bool = False) -> float:
+        """back-to-back calls of the entry point that allocates nothing, HIP-event timed; total ms"""
+        self._check_extents("dot", "bf16_f8e4m3w", lhs, rhs_list, out, md)
+        arr, n = _md_array(md)
+        ptrs = (ctypes.c_void_p * len(rhs_list))(*[b.ptr for b in rhs_list])
+        ms = ctypes.c_float()
+        self._check(self.debug.hodu_rocm_debug_time_noalloc(self.handle, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr, n,
+                                                            int(iters), int(bool(graph)), ctypes.byref(ms)))
+        return float(ms.value)
 
     def product_ex(self, op: str, name: str, lhs: DeviceBuffer, rhs: DeviceBuffer, out: DeviceBuffer, md, steps):
         """hodu_rocm_<op>_<name>_ex: the product with element-wise steps (add_row / mul_scalar / relu) fused into

@@ -73,6 +73,13 @@ int hodu_rocm_debug_time_product_ex(hodu_rocm_ctx *ctx, int is_matmul, int kind,
                                     size_t metadata_len, const hodu_rocm_epilogue_step *steps, size_t n_steps,
                                     int iters, float *elapsed_ms);
 
+/* measurement hook: `iters` calls of hodu_rocm_dot_bf16_f8e4m3w_noalloc, as hodu_rocm_debug_time_product times
+ * the allocating entry point; graph != 0 captures the calls into one HIP graph first (the entry point launches
+ * kernels only, so it may be captured from its first call on) */
+int hodu_rocm_debug_time_noalloc(hodu_rocm_ctx *ctx, const void *lhs, const void *const *rhs_list, size_t n_rhs,
+                                 void *out, const size_t *metadata, size_t metadata_len, int iters, int graph,
+                                 float *elapsed_ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,8 +47,8 @@ enum {
     HODU_ROCM_UNSUPPORTED = 2, /* dtype / rank outside what the device implements */
     HODU_ROCM_HIP_ERROR = 3,   /* a HIP runtime call failed; see hodu_rocm_last_error */
     HODU_ROCM_OOM = 4,         /* device allocation failed */
-    HODU_ROCM_SCRATCH = 5      /* the call may not allocate (its stream is under graph capture) and its kernels need
-                                  more scratch than is there */
+    HODU_ROCM_SCRATCH = 5      /* the call may not allocate (the entry point that allocates nothing, or a stream under
+                                  graph capture) and its kernels need more scratch than is there */
 };
 
 /* dtype ids, equal to hodu's repr(u8) DType (crates/hodu_core/src/types/dtype.rs:6-28) */
@@ -120,6 +120,23 @@ int hodu_rocm_matmul_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void
                               void *out_i32, const size_t *metadata, size_t metadata_len);
 int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void *rhs_i8,
                            void *out_i32, const size_t *metadata, size_t metadata_len);
+
+/* ---- the one entry point that allocates nothing ------------------------------------------------- *
+ * No counterpart in the reference.  It exists for callers that cannot allocate device memory while they call:
+ * code under HIP graph capture, tight decode loops, harnesses that forbid hipMalloc.  Same arguments, same result
+ * (bit for bit) as hodu_rocm_dot_bf16_f8e4m3w, whose kernels for M <= 16 cut K across workgroups and keep partial
+ * sums and arrival counters in a workspace the context allocates and grows on demand; here that scratch is a
+ * file-scope device array inside the library (16 KiB of counters + HODU_ROCM_NOALLOC_PARTIAL_BYTES of partial
+ * sums; every GPU the library runs on holds one copy until the process ends) and the call makes no hipMalloc /
+ * hipFree.  A product whose kernel would need more partial-sum space than that returns HODU_ROCM_SCRATCH with a
+ * message naming both sizes (C3's M = 256 cut four ways needs 16 MiB; M <= 16 against any weight up to
+ * N x slices <= 131072 fits).  All calls on one GPU share the array: the counters are zeroed by a small kernel at
+ * the head of every call, and calls that overlap on one GPU -- two contexts, i.e. two streams -- race on it;
+ * calls on one context are ordered by its stream.  No fused steps. */
+#define HODU_ROCM_NOALLOC_PARTIAL_BYTES ((size_t)8 << 20)
+int hodu_rocm_dot_bf16_f8e4m3w_noalloc(hodu_rocm_ctx *ctx, const void *lhs_bf16, const void *rhs_f8e4m3,
+                                       void *out_bf16, const size_t *metadata, size_t metadata_len);
+
 /* ---- matmul / dot with the caller's next element-wise kernels fused into the store -------------- *
  * The reference's callers of the product launch an element-wise kernel on its output straight away:
  *   Linear::forward (crates/hodu_nn/src/modules/linear.rs:40-46): matmul, then add(bias)
