@@ -44,16 +44,25 @@ def hipcc() -> str:
 _ONLY_CHANGED = False  # `python -m hodu_amd.build --changed`: keep objects newer than their source and every header
 
 
-def _headers_mtime() -> float:
-    dirs = [CSRC, DEBUG_SRC, os.path.join(ROOT, "include")]
-    return max(os.path.getmtime(os.path.join(d, f)) for d in dirs for f in os.listdir(d) if f.endswith((".hpp", ".h")))
+def _deps_mtime(src: str, dep: str) -> float:
+    """newest of the source and the project headers the last compile of it read (the compiler's own -MD list)"""
+    newest = os.path.getmtime(src)
+    try:
+        words = open(dep).read().replace("\\\n", " ").split()
+    except OSError:
+        return float("inf")
+    for w in words[1:]:
+        if w.startswith(ROOT) and os.path.exists(w):
+            newest = max(newest, os.path.getmtime(w))
+    return newest
 
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ, os.path.basename(os.path.dirname(src)) + "_" + os.path.basename(src) + ".o")
-    if _ONLY_CHANGED and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _headers_mtime()):
+    dep = obj + ".d"
+    if _ONLY_CHANGED and os.path.exists(obj) and os.path.getmtime(obj) > _deps_mtime(src, dep):
         return obj
-    cmd = [hipcc(), *FLAGS, "-c", src, "-o", obj]
+    cmd = [hipcc(), *FLAGS, "-MD", "-MF", dep, "-c", src, "-o", obj]
     if src.endswith(".cpp"):
         cmd[1:1] = ["-x", "hip"]
     r = subprocess.run(cmd, capture_output=True, text=True)

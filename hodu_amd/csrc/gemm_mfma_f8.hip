@@ -10,6 +10,7 @@ int launch_mfma_f8(hodu_rocm_ctx *ctx, int dtype, const void *a, const void *b, 
     const int lb = pick_mode(b, g.b_off, g.b_n, g.b_k, g.N, g.K, 1, 16, 16, g, g.b_bs);
     const int forced = ctx->force_tile;
     if (la != LM_K || lb != LM_K || g.K % P_ROW_BYTES != 0 || (forced >= 0 && forced < 10)) return HODU_ROCM_UNSUPPORTED;
+    if (!pipe_offsets_fit(g.a_m, 1) || !pipe_offsets_fit(g.b_n, 1)) return HODU_ROCM_UNSUPPORTED;
     const long cus = ctx->props.multiProcessorCount;
     auto tiles = [&](long bm, long bn) { return g.batches * ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); };
     const bool big = forced >= 10 ? forced != 12 : tiles(256, 256) >= cus;
@@ -28,10 +29,10 @@ int launch_mfma_f8(hodu_rocm_ctx *ctx, int dtype, const void *a, const void *b, 
         ctx->last_kernel = base;
     }
     if (e5m2) {
-        if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E5M2, 256, 256>>(ctx, a, b, c, g, splits);
+        if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E5M2, 256, 256, 25, false, 4>>(ctx, a, b, c, g, splits);
         return launch_pipe_f8<PipeF8Config<OUT_F8E5M2, 128, 128>>(ctx, a, b, c, g, splits);
     }
-    if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 256, 256>>(ctx, a, b, c, g, splits);
+    if (big) return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 256, 256, 25, false, 4>>(ctx, a, b, c, g, splits);
     return launch_pipe_f8<PipeF8Config<OUT_F8E4M3, 128, 128>>(ctx, a, b, c, g, splits);
 }
 }  // namespace hodu

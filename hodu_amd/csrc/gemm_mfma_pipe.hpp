@@ -113,6 +113,12 @@ __device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
 }
 
+// The same with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit byte offset per
+// lane: the form whose per-instruction cost is one M0 write -- no vector arithmetic, no readfirstlane.
+__device__ __forceinline__ void dma16_sbase(const char *sbase, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+
 // 64 bits per lane through the LDS transpose.  Of the 16 lanes that execute together, lane s supplies the
 // address of 8 consecutive bytes.
 //   16-bit elements: lane i receives element (i % 4) of lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4 -- with lanes
@@ -223,7 +229,10 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     typedef RowDenseGeom<ES, ES> GA;
     typedef RowDenseGeom<SB, ES> GB;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wavefront's index as a scalar: what a DMA instruction needs besides the lane's offset inside the tile --
+    // the operand's base address, the LDS destination in M0 -- is then wave-uniform and stays in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
     const int lr = lane & 31, lh = lane >> 5;
 
@@ -244,7 +253,11 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     // row-dense operand: KPI consecutive k-rows of ROWS elements; lane -> (k-row, slot), the slot holds chunk
     // slot ^ swz(k); a chunk that starts past the operand's last row is fetched from the last whole chunk
     // instead (its columns are never stored).
-    const char *gpa[PA], *gpb[PB];    // source address of this lane for stage (buffer) 0
+    // An address is the scalar base of the tile (its first row, or its first column of k-row 0; advanced by a
+    // stage's worth per stage) plus the lane's 32-bit byte offset inside the tile, fixed for the whole launch: an
+    // instruction then costs one M0 write and the load itself, no vector arithmetic.  pipe_offsets_fit() on the
+    // host guarantees that the offsets stay below 4 GB.
+    unsigned offa[PA], offb[PB];      // byte offset of this lane inside the tile, stage (buffer) 0
     unsigned lda[PA], ldb[PB];        // block offset inside a buffer (wave-uniform)
 #pragma unroll
     for (int p = 0; p < PA; p++) {
@@ -253,13 +266,14 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
             int row = m0 + trow;
             row = row < g.M ? row : g.M - 1;
-            gpa[p] = A + (ao + (long)row * g.a_m) * ES + dchunk * 16;
+            offa[p] = (unsigned)((long)(row - m0) * g.a_m * ES) + dchunk * 16;
         } else {
             constexpr int CPR = Cfg::BM / GA::EPC, KPI = 64 / CPR;  // chunks per k-row, k-rows per instruction
             const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ GA::swz(k);
             int col = m0 + c * GA::EPC;
             col = col <= g.M - GA::EPC ? col : g.M - GA::EPC;
-            gpa[p] = A + (ao + (long)k * g.a_k + col) * ES;
+            // (the clamped column may lie left of the tile's first one: the offset is taken from the clamped base)
+            offa[p] = (unsigned)(((long)k * g.a_k + (col - (m0 <= g.M - GA::EPC ? m0 : g.M - GA::EPC))) * ES);
         }
         lda[p] = q * 1024;
     }
@@ -270,16 +284,21 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
             int row = n0 + trow;
             row = row < g.N ? row : g.N - 1;
-            gpb[p] = B + (bo + (long)row * g.b_n) * SB + dchunk * 16;
+            offb[p] = (unsigned)((long)(row - n0) * g.b_n * SB) + dchunk * 16;
         } else {
             constexpr int CPR = Cfg::BN / GB::EPC, KPI = 64 / CPR;
             const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ GB::swz(k);
             int col = n0 + c * GB::EPC;
             col = col <= g.N - GB::EPC ? col : g.N - GB::EPC;
-            gpb[p] = B + (bo + (long)k * g.b_k + col) * SB;
+            offb[p] = (unsigned)(((long)k * g.b_k + (col - (n0 <= g.N - GB::EPC ? n0 : g.N - GB::EPC))) * SB);
         }
         ldb[p] = B_BASE + q * 1024;
     }
+    // scalar bases: k-dense -> first row of the tile; row-dense -> first (clamped) column of the tile in k-row 0
+    const char *base_a = Cfg::LA == LM_K ? A + (ao + (long)m0 * g.a_m) * ES
+                                         : A + (ao + (m0 <= g.M - GA::EPC ? m0 : g.M - GA::EPC)) * ES;
+    const char *base_b = Cfg::LB == LM_K ? B + (bo + (long)n0 * g.b_n) * SB
+                                         : B + (bo + (n0 <= g.N - GB::EPC ? n0 : g.N - GB::EPC)) * SB;
     // bytes a stage advances an operand's source by: 128 bytes of k, or a stage's k-rows; a k-dense f8 buffer
     // is 128 bytes of k as well, but that is two stages
     const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : (long)GA::STAGE_K * g.a_k * ES;
@@ -292,10 +311,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     const int t0 = blockIdx.y * stages_per_split;
     const int T = T_all - t0 < stages_per_split ? T_all - t0 : stages_per_split;  // stages of this workgroup
     const int TB = B_PAIR ? (T + 1) / 2 : T;        // right-operand buffers' worth of k
-#pragma unroll
-    for (int p = 0; p < PA; p++) gpa[p] += t0 * a_adv;
-#pragma unroll
-    for (int p = 0; p < PB; p++) gpb[p] += (B_PAIR ? t0 >> 1 : t0) * b_adv;
+    base_a += t0 * a_adv;
+    base_b += (B_PAIR ? t0 >> 1 : t0) * b_adv;
 
     // What to fetch next, decided at a stage's barrier and carried to the slices that issue it.  Every stage
     // issues a full list -- PA instructions of A, PBS of B -- so that the number of instructions in flight at any
@@ -313,17 +330,16 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     auto dma_element = [&](int e, const Fetch &f) {
 #pragma unroll
         for (int p = 0; p < PA; p++)
-            if (e == p) dma16_raw(gpa[p] + f.a_src * a_adv, __builtin_amdgcn_readfirstlane(lds0 + f.a_dst + lda[p]));
+            if (e == p) dma16_sbase(base_a + f.a_src * a_adv, offa[p], lds0 + f.a_dst + lda[p]);
 #pragma unroll
         for (int p = 0; p < PBS; p++)
             if (e == PA + p && f.b_on) {
-                const char *src = gpb[p];
-                unsigned off = ldb[p];
+                unsigned voff = offb[p], off = ldb[p];
                 if constexpr (B_PAIR) {
-                    src = f.b_half ? gpb[p + PBS] : gpb[p];
+                    voff = f.b_half ? offb[p + PBS] : offb[p];
                     off = f.b_half ? ldb[p + PBS] : ldb[p];
                 }
-                dma16_raw(src + f.b_src * b_adv, __builtin_amdgcn_readfirstlane(lds0 + f.b_dst + off));
+                dma16_sbase(base_b + f.b_src * b_adv, voff, lds0 + f.b_dst + off);
             }
     };
 
@@ -450,10 +466,10 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         const int ta = j < T ? j : T - 1, tb = j < TB ? j : TB - 1;
 #pragma unroll
         for (int p = 0; p < PA; p++)
-            dma16_raw(gpa[p] + ta * a_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)j * Cfg::A_BYTES + lda[p]));
+            dma16_sbase(base_a + ta * a_adv, offa[p], lds0 + (unsigned)j * Cfg::A_BYTES + lda[p]);
 #pragma unroll
         for (int p = 0; p < PB; p++)
-            dma16_raw(gpb[p] + tb * b_adv, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)j * Cfg::B_BYTES + ldb[p]));
+            dma16_sbase(base_b + tb * b_adv, offb[p], lds0 + (unsigned)j * Cfg::B_BYTES + ldb[p]);
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 1) * (PA + PB)));  // group 0 has landed
     __builtin_amdgcn_s_barrier();
@@ -622,9 +638,16 @@ inline int pick_splits(long tiles, long cus, int stages, long elems, int forced)
 
 // K a whole number of 128-byte stages; the row-dense layouts exist for 8- and 16-bit types and fetch whole
 // 16-byte chunks of a k-row; alignment is what pick_mode already established
+// the DMA addresses are a scalar base plus a 32-bit byte offset per lane that spans up to 256 rows (k-dense) or 128
+// k-rows (row-dense) of the operand: the stride that separates them must keep that below 4 GB
+inline bool pipe_offsets_fit(long stride, int elem_bytes) {
+    return stride >= 0 && stride <= ((1L << 32) - 8192) / (256L * elem_bytes);
+}
+
 template <int CK> bool pipe_eligible(int la, int lb, const DevProduct &g) {
     constexpr int ES = Compute<CK>::ES;
     if (g.K <= 0 || ((long)g.K * ES) % P_ROW_BYTES != 0) return false;
+    if (!pipe_offsets_fit(la == LM_K ? g.a_m : g.a_k, ES) || !pipe_offsets_fit(lb == LM_K ? g.b_n : g.b_k, ES)) return false;
     if (la == LM_K && lb == LM_K) return true;
     if (ES > 2 || la == LM_SCALAR || lb == LM_SCALAR) return false;
     constexpr int EPC = 16 / ES;  // a row-dense operand is fetched in whole 16-byte chunks of a k-row
@@ -636,6 +659,7 @@ template <int CK> bool pipe_eligible(int la, int lb, const DevProduct &g) {
 // moves whole 128-byte lines of k, i.e. K is a multiple of 128.
 inline bool pipe_f8_eligible(int la, int lb, const void *b, const DevProduct &g) {
     if (la != LM_K || lb == LM_SCALAR || g.K <= 0 || g.K % 64 != 0) return false;
+    if (!pipe_offsets_fit(g.a_m, 2) || !pipe_offsets_fit(lb == LM_K ? g.b_n : g.b_k, 1)) return false;
     if (((uintptr_t)b + (uintptr_t)g.b_off) % 16 != 0) return false;
     for (int d = 0; d < g.nb; d++)
         if (g.b_bs[d] % 16 != 0) return false;

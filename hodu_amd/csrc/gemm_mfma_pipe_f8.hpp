@@ -48,8 +48,16 @@ template <int FMT> __device__ __forceinline__ void mma_f8(const FragF8 &a, const
     c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
 
-template <int OUT_, int BM_, int BN_> struct PipeF8Config {
-    static constexpr int OUT = OUT_, BM = BM_, BN = BN_, WM = 2, WN = 2, NT = 256, NW = 4, NST = 2;
+// WN_: wavefronts along n (2 along m).  The 256 x 256 tile runs with 2 x 4: two wavefronts share a SIMD, and one's
+// LDS reads and DMA issue overlap the other's MFMAs (measured 2410 against 2540 cycles per 128-k stage with 2 x 2, where
+// a wavefront owns 128 x 128 outputs and has its SIMD to itself; 2048 is the matrix core's own time).
+template <int OUT_, int BM_, int BN_, int PH_ = 50, bool PROBE_ = false, int WN_ = 2> struct PipeF8Config {
+    static constexpr int OUT = OUT_, BM = BM_, BN = BN_, WM = 2, WN = WN_, NT = WM * WN * 64, NW = WM * WN, NST = 2;
+    // share of a stage's DMA list issued right behind the stage's barrier, in the last quarter of the stage, where the
+    // next stage's first fragment reads crowd as well; the rest goes out during the next stage's first half.  Measured
+    // cycles per stage of the 2 x 2 tile: 3409 with 100 %, 2755 with 50 %, 2552 with 25 %, 2594 with none.
+    static constexpr int PH_PERCENT = PH_;
+    static constexpr bool PROBE = PROBE_;    // measurement builds only: per-wavefront cycle stamps around the waits
     static constexpr int A_BYTES = BM * P_ROW_BYTES, B_BYTES = BN * P_ROW_BYTES;
     static constexpr int LDS_BYTES = NST * (A_BYTES + B_BYTES);
     static constexpr int PA = (BM / 8) / NW, PB = (BN / 8) / NW, P = PA + PB;
@@ -69,7 +77,10 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
     constexpr int TM = Cfg::TM, TN = Cfg::TN, PA = Cfg::PA, PB = Cfg::PB, P = Cfg::P;
     constexpr int TILE_BYTES = 32 * P_ROW_BYTES, B_BASE = 2 * Cfg::A_BYTES;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wavefront's index as a scalar: everything a DMA instruction needs besides the lane's row offset -- the
+    // operand's base address, the LDS destination in M0 -- is then wave-uniform and stays in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
     const int lr = lane & 31, lh = lane >> 5;
 
@@ -81,15 +92,18 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
 
-    // DMA plan: one instruction = 8 rows x 128 bytes; the slot of a lane holds chunk slot ^ ((row >> 1) & 7)
-    const char *gpa[PA], *gpb[PB];
+    // DMA plan: one instruction = 8 rows x 128 bytes; the slot of a lane holds chunk slot ^ ((row >> 1) & 7).
+    // Address = scalar base of the tile's first row (advanced 128 bytes per stage) + the lane's 32-bit offset of
+    // its (clamped) row and chunk inside the tile, fixed for the whole launch: a DMA instruction costs one M0
+    // write and the load itself, no vector arithmetic.  (The launcher checks that 256 rows stay below 4 GB.)
+    unsigned offa[PA], offb[PB];
     unsigned lda[PA], ldb[PB];
 #pragma unroll
     for (int p = 0; p < PA; p++) {
         const int q = p * Cfg::NW + wave, trow = q * 8 + (lane >> 3);
         int row = m0 + trow;
         row = row < g.M ? row : g.M - 1;
-        gpa[p] = A + ao + (long)row * g.a_m + kd_slot(trow, lane & 7) * 16;
+        offa[p] = (unsigned)((long)(row - m0) * g.a_m) + kd_slot(trow, lane & 7) * 16;
         lda[p] = q * 1024;
     }
 #pragma unroll
@@ -97,27 +111,23 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
         const int q = p * Cfg::NW + wave, trow = q * 8 + (lane >> 3);
         int row = n0 + trow;
         row = row < g.N ? row : g.N - 1;
-        gpb[p] = B + bo + (long)row * g.b_n + kd_slot(trow, lane & 7) * 16;
+        offb[p] = (unsigned)((long)(row - n0) * g.b_n) + kd_slot(trow, lane & 7) * 16;
         ldb[p] = B_BASE + q * 1024;
     }
     const int T_all = g.K / P_ROW_BYTES;
     const int t0 = blockIdx.y * stages_per_split;
     const int T = T_all - t0 < stages_per_split ? T_all - t0 : stages_per_split;
-#pragma unroll
-    for (int p = 0; p < PA; p++) gpa[p] += (long)t0 * P_ROW_BYTES;
-#pragma unroll
-    for (int p = 0; p < PB; p++) gpb[p] += (long)t0 * P_ROW_BYTES;
+    const char *const base_a = A + ao + (long)m0 * g.a_m + (long)t0 * P_ROW_BYTES;
+    const char *const base_b = B + bo + (long)n0 * g.b_n + (long)t0 * P_ROW_BYTES;
 
     // element e of stage `src`'s issue list (PA of A, then PB of B) into ring slot `slot`
     auto dma_element = [&](int e, int src, int slot) {
 #pragma unroll
         for (int p = 0; p < PA; p++)
-            if (e == p)
-                dma16_raw(gpa[p] + (long)src * P_ROW_BYTES, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)slot * Cfg::A_BYTES + lda[p]));
+            if (e == p) dma16_sbase(base_a + (long)src * P_ROW_BYTES, offa[p], lds0 + (unsigned)slot * Cfg::A_BYTES + lda[p]);
 #pragma unroll
         for (int p = 0; p < PB; p++)
-            if (e == PA + p)
-                dma16_raw(gpb[p] + (long)src * P_ROW_BYTES, __builtin_amdgcn_readfirstlane(lds0 + (unsigned)slot * Cfg::B_BYTES + ldb[p]));
+            if (e == PA + p) dma16_sbase(base_b + (long)src * P_ROW_BYTES, offb[p], lds0 + (unsigned)slot * Cfg::B_BYTES + ldb[p]);
     };
 
     // fragment addresses: window w, lane (lr, lh) reads bytes 64*w + 32*lh .. +31 of row lr = chunks 4w + 2lh, +1
@@ -149,6 +159,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
 
+    unsigned long long probe_wait = 0, probe_barrier = 0;
+    const unsigned long long probe_start = Cfg::PROBE ? __builtin_amdgcn_s_memtime() : 0;
     FragF8 fbw[2][TN];  // right fragments of the current window and of the next
     FragF8 fa[2];       // left fragments: the one multiplying and the one arriving
     typedef std::integral_constant<int, 0> W0;
@@ -172,8 +184,20 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
             const bool last = i == TM - 1;
             if (LATE && last) {
                 // stage t+1 has landed, every read of stage t has returned
-                __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-                __builtin_amdgcn_s_barrier();
+                if constexpr (Cfg::PROBE) {
+                    const unsigned long long c0 = __builtin_amdgcn_s_memtime();
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+                    const unsigned long long c1 = __builtin_amdgcn_s_memtime();
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+                    __builtin_amdgcn_s_barrier();
+                    const unsigned long long c2 = __builtin_amdgcn_s_memtime();
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+                    probe_wait += c1 - c0;
+                    probe_barrier += c2 - c1;
+                } else {
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+                    __builtin_amdgcn_s_barrier();
+                }
                 asm volatile("" ::: "memory");
             }
             if (!last) fa[(i + 1) & 1] = read_a(slot_cur, WC{}, i + 1);
@@ -199,7 +223,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    constexpr int PH = P / 2;  // issued behind the barrier of the stage; the rest during the next stage's first window
+    constexpr int PH = P * Cfg::PH_PERCENT / 100;  // issued behind the barrier of the stage; the rest during the next stage's first window
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, PH> DH;
     typedef std::integral_constant<int, P - PH> DR;
@@ -236,9 +260,19 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
     // the clamped re-fetches still write LDS: wait for them, then for everybody's, before LDS is reused
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
+    if constexpr (Cfg::PROBE) {
+        // measurement builds: `partials` is the stamp buffer, four words per wavefront
+        if (lane == 0) {
+            unsigned long long *w = (unsigned long long *)partials + ((long)blockIdx.x * Cfg::NW + wave) * 4;
+            w[0] = __builtin_amdgcn_s_memtime() - probe_start;
+            w[1] = probe_wait;
+            w[2] = probe_barrier;
+            w[3] = (unsigned long long)T;
+        }
+    }
 
     char *patch = smem + wave * (32 * (TN * 32 * 4 + 16));
-    if (gridDim.y > 1) {
+    if (!Cfg::PROBE && gridDim.y > 1) {
         float *Pb = (float *)partials + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
 #pragma unroll
         for (int i = 0; i < TM; i++)
