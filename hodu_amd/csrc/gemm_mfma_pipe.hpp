@@ -45,7 +45,21 @@
 
 #include <type_traits>
 
+#include "agent_scope.hpp"
 #include "gemm_mfma.hpp"
+
+// Measurement builds only (never the library's): HODU_PIPE_STAMPS makes every workgroup record the 100 MHz
+// real-time counter at a few points into the buffer whose address the third fused-step slot carries.
+#ifdef HODU_PIPE_STAMPS
+#define HODU_STAMP(i)                                                                                              \
+    do {                                                                                                           \
+        if (threadIdx.x == 0)                                                                                      \
+            ((unsigned long long *)g.epi.step[2].vec)[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] =   \
+                __builtin_amdgcn_s_memrealtime();                                                                  \
+    } while (0)
+#else
+#define HODU_STAMP(i) do { } while (0)
+#endif
 
 namespace hodu {
 namespace mfma {
@@ -115,6 +129,13 @@ __device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
 
 // The same with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit byte offset per
 // lane: the form whose per-instruction cost is one M0 write -- no vector arithmetic, no readfirstlane.
+// (a pointer the compiler can hold in scalar registers: both halves through readfirstlane, which is free for a value
+// that already is uniform and makes the "s" constraints below hold where the uniformity analysis gives up)
+__device__ __forceinline__ const char *uniform_ptr(const char *p) {
+    const unsigned long long v = (unsigned long long)(uintptr_t)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (const char *)(uintptr_t)(((unsigned long long)hi << 32) | lo);
+}
 __device__ __forceinline__ void dma16_sbase(const char *sbase, unsigned voff, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
@@ -140,6 +161,7 @@ __device__ __forceinline__ u32x2_t lds_get64(const char *lds, int off) { return 
 
 // 8 f8e4m3 -> 8 bf16 (exact)
 __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
+
     return u32x4_t{f8pair_to_bf16pair(v.x, false), f8pair_to_bf16pair(v.x, true), f8pair_to_bf16pair(v.y, false),
                    f8pair_to_bf16pair(v.y, true)};
 }
@@ -214,11 +236,68 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
     asm volatile("" ::: "memory");  // the next band overwrites the patch
 }
 
+// A product cut along K (grid.y ranges): every workgroup of a tile writes its accumulators, unrounded, to its own
+// slab of the workspace -- in the accumulator layout, 16 bytes per lane and instruction, so a slab is written and
+// read in whole 1 KB pieces -- and counts itself in on the tile's arrival counter; the one that arrives last adds all
+// slabs in range order (its own included, from memory: the order, and therefore the rounding, does not depend on who
+// was last) and goes on to store the tile.  One launch instead of two, and the other workgroups' compute units are
+// free as soon as their slab is out.  Returns true in the workgroup that now holds the tile's sums.
+template <int NW, int TM, int TN, class acc_t>
+__device__ __forceinline__ bool splitk_exchange(acc_t (&acc)[TM][TN], void *partials, int *arrival, int *flag, int tid) {
+    typedef decltype(acc_t{}[0]) elem_ref_t;
+    typedef std::remove_cv_t<std::remove_reference_t<elem_ref_t>> elem_t;
+    typedef elem_t quad_t __attribute__((ext_vector_type(4)));
+    constexpr unsigned WAVE_BYTES = TM * TN * 4 * 1024, SLAB = NW * WAVE_BYTES;
+    const int lane = tid & 63, wave = tid >> 6;
+    const unsigned mine = wave * WAVE_BYTES + lane * 16;
+    char *slab0 = (char *)partials + (size_t)blockIdx.x * SLAB;
+    const size_t range_pitch = (size_t)gridDim.x * SLAB;
+    {
+        const __amdgpu_buffer_rsrc_t out = agent_buffer(slab0 + blockIdx.y * range_pitch, SLAB);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    store16_agent(out, mine + ((i * TN + j) * 4 + q) * 1024,
+                                  quad_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]});
+    }
+    if (!arrive_and_check_last(&arrival[blockIdx.x], (int)gridDim.y, flag, tid)) return false;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
+    // The slabs come from memory (a round trip of a microsecond or more) and are added in range order; what hides the
+    // latency is the number of loads in flight: a whole slab's share of this wavefront at a time where the registers
+    // allow it (TM * TN * 4 loads of 16 bytes per lane), half of it otherwise.
+    constexpr int PER = TM * TN * 4, CHUNK = PER <= 32 ? PER : PER / 2;
+    for (unsigned r = 0; r < gridDim.y; r++) {
+        const __amdgpu_buffer_rsrc_t in = agent_buffer(slab0 + r * range_pitch, SLAB);
+#pragma unroll
+        for (int c0 = 0; c0 < PER; c0 += CHUNK) {
+            quad_t v[CHUNK];
+#pragma unroll
+            for (int c = 0; c < CHUNK; c++) v[c] = load16_agent<quad_t>(in, mine + (c0 + c) * 1024);
+#pragma unroll
+            for (int c = 0; c < CHUNK; c++) {
+                const int t = (c0 + c) / 4, q = (c0 + c) % 4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[t / TN][t % TN][4 * q + e] += v[c][e];
+            }
+        }
+    }
+    arrival_reset(&arrival[blockIdx.x], tid);
+    return true;
+}
+
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                             typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                             int tiles_m, int tiles_n, int stages_per_split,
-                                                            void *__restrict__ partials) {
+                                                            void *__restrict__ partials, int *__restrict__ arrival) {
     extern __shared__ __align__(16) char smem[];
     typedef Compute32<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
@@ -229,6 +308,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     typedef RowDenseGeom<ES, ES> GA;
     typedef RowDenseGeom<SB, ES> GB;
 
+    HODU_STAMP(0);
     const int tid = threadIdx.x, lane = tid & 63;
     // the wavefront's index as a scalar: what a DMA instruction needs besides the lane's offset inside the tile --
     // the operand's base address, the LDS destination in M0 -- is then wave-uniform and stays in scalar registers
@@ -311,8 +391,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     const int t0 = blockIdx.y * stages_per_split;
     const int T = T_all - t0 < stages_per_split ? T_all - t0 : stages_per_split;  // stages of this workgroup
     const int TB = B_PAIR ? (T + 1) / 2 : T;        // right-operand buffers' worth of k
-    base_a += t0 * a_adv;
-    base_b += (B_PAIR ? t0 >> 1 : t0) * b_adv;
+    base_a = uniform_ptr(base_a + t0 * a_adv);
+    base_b = uniform_ptr(base_b + (B_PAIR ? t0 >> 1 : t0) * b_adv);
 
     // What to fetch next, decided at a stage's barrier and carried to the slices that issue it.  Every stage
     // issues a full list -- PA instructions of A, PBS of B -- so that the number of instructions in flight at any
@@ -412,6 +492,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         }
     };
     u32x4_t fa[2][TM], fb[2][TN];  // [register set][tile]: slice s lives in set s % 2
+    u32x4_t bwide = u32x4_t{0u, 0u, 0u, 0u};  // f8e4m3 storage: the widened first right fragment of the next slice
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -430,19 +511,33 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         constexpr int SET = decltype(cur_)::value & 1, RD = decltype(rd_)::value;
         constexpr int D0 = decltype(d0_)::value, DN = decltype(dn_)::value;
         constexpr int MF = TM * TN, RN = TM + TN;
-        u32x4_t bcur = fb[SET][0];
+        // f8e4m3 storage: a right fragment is widened to bf16 one group of TM MFMAs AHEAD of its use, right behind an
+        // MFMA that has just been issued, so that the conversions run in that MFMA's shadow; widened in front of
+        // its first use they hold the matrix core up for their own latency once per group, which a wavefront that has
+        // its SIMD to itself cannot hide (measured on 128 x 128 tiles, M = 256: 0.60 -> 0.56 us per 64-k stage; the
+        // four conversions per fragment are full-rate instructions, 16 cycles of issue against 32 per MFMA, so with
+        // one or two MFMAs per fragment the wavefront's own instruction issue stays the limit: 0.45 us without any
+        // conversion, 0.39 us with bf16 weights).  `bwide` carries the first fragment of the next slice across the call.
+        u32x4_t bcur = B_F8 ? bwide : fb[SET][0], bnext = bcur;
 #pragma unroll
         for (int idx = 0; idx < MF; idx++) {
 #pragma unroll
             for (int r = 0; r < RN; r++) {
                 if (r * MF / RN != idx) continue;
                 typedef std::integral_constant<int, RD> RS;
-                if (r < TM) fa[RD & 1][r] = read_a(rd_a, RS{}, r);
-                else fb[RD & 1][r - TM] = read_b(rd_b, rd_second, RS{}, r - TM);
+                // (f8e4m3: the next slice's first right fragment is needed first, by the conversion at the end of this one)
+                const bool b_turn = B_F8 ? (r == 0 || r > TM) : r >= TM;
+                const int bi = B_F8 ? (r == 0 ? 0 : r - TM) : r - TM, ai = B_F8 ? r - 1 : r;
+                if (!b_turn) fa[RD & 1][ai] = read_a(rd_a, RS{}, ai);
+                else fb[RD & 1][bi] = read_b(rd_b, rd_second, RS{}, bi);
             }
-            if (idx % TM == 0) bcur = B_F8 ? widen_f8x8(u32x2_t{fb[SET][idx / TM].x, fb[SET][idx / TM].y}) : fb[SET][idx / TM];
+            if (idx % TM == 0 && idx > 0) bcur = B_F8 ? bnext : fb[SET][idx / TM];
             // operands swapped: the accumulator then holds, per lane, runs of 4 consecutive n of one m
             Cmp::mma(bcur, fa[SET][idx % TM], acc[idx % TM][idx / TM]);
+            if constexpr (B_F8) {
+                if (idx % TM == 0 && idx / TM + 1 < TN) bnext = widen_f8x8(u32x2_t{fb[SET][idx / TM + 1].x, fb[SET][idx / TM + 1].y});
+                if (idx == MF - 1) bwide = widen_f8x8(u32x2_t{fb[RD & 1][0].x, fb[RD & 1][0].y});
+            }
 #pragma unroll
             for (int d = 0; d < DN; d++) {
                 if (d * MF / (DN > 0 ? DN : 1) != idx) continue;
@@ -473,11 +568,13 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 1) * (PA + PB)));  // group 0 has landed
     __builtin_amdgcn_s_barrier();
+    HODU_STAMP(1);
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int i = 0; i < TM; i++) fa[0][i] = read_a(0u, I0{}, i);
 #pragma unroll
     for (int j = 0; j < TN; j++) fb[0][j] = read_b(0u, 0, I0{}, j);
+    if constexpr (B_F8) bwide = widen_f8x8(u32x2_t{fb[0][0].x, fb[0][0].y});
 
     // Instructions that may still be in flight at the barrier of stage t without touching what stage t+1 reads:
     // the NST - 2 youngest issue groups.  Groups, oldest first: the NST groups of the prologue (PA + PB each), then
@@ -567,8 +664,17 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
     out_t *Cb;
     // every wavefront's DMA has landed before any wavefront reuses LDS for its epilogue
     __syncthreads();
+    HODU_STAMP(2);
     char *patch = smem + wave * (32 * (TN * 32 * 4 + 16));  // sized for 4-byte outputs, the largest
-    if (gridDim.y > 1) {
+    if (gridDim.y > 1 && arrival != nullptr) {
+        // cut along K, summed here: only the workgroup that arrives last stores the tile
+        if (!splitk_exchange<Cfg::NW, TM, TN>(acc, partials, arrival, reinterpret_cast<int *>(smem + Cfg::LDS_BYTES - 16), tid)) {
+            HODU_STAMP(3);
+            return;
+        }
+        __syncthreads();  // (the flag word lies outside every wavefront's patch; the barrier orders LDS reuse all the same)
+        HODU_STAMP(4);
+    } else if (gridDim.y > 1) {
         constexpr int ACC = Cfg::CK == CK_I8 ? OUT_I32 : OUT_F32;
         typedef typename Out<ACC>::T part_t;
         part_t *Pb = (part_t *)partials + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
@@ -581,6 +687,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
 #pragma unroll
     for (int i = 0; i < TM; i++)
         store_band_via_lds<Cfg::OUT, TN, true>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
+    HODU_STAMP(5);
 }
 
 // splits > 1: K is cut into that many ranges of whole stages, each range a workgroup of its own (grid.y);
@@ -602,16 +709,23 @@ template <class Cfg> int launch_pipe(hodu_rocm_ctx *ctx, const void *a, const vo
         splits = (T + per - 1) / per;
     }
     const long elems = g.batches * (long)g.M * g.N;
+    // the ranges of a tile meet inside the kernel (one arrival counter per tile) wherever there is a counter for every
+    // tile; a product with more tiles than that -- it does not need cutting -- keeps the second kernel
+    const bool in_kernel = splits > 1 && total <= kArrivalSlots;
+    int *arrival = nullptr;
     if (splits > 1) {
-        int rc = ensure_workspace(ctx, (size_t)splits * elems * 4);
+        const size_t bytes = in_kernel ? (size_t)splits * total * Cfg::BM * Cfg::BN * 4 : (size_t)splits * elems * 4;
+        int rc = ensure_workspace(ctx, bytes);
+        if (rc == HODU_ROCM_OK && in_kernel) rc = ensure_arrival(ctx);
         if (rc != HODU_ROCM_OK) return rc;
         partials = ctx->workspace.ptr;
+        if (in_kernel) arrival = ctx->arrival;
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)total, (unsigned)(splits > 1 ? splits : 1)), dim3(Cfg::NT), Cfg::LDS_BYTES,
                        ctx->stream, (const char *)a, (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n,
-                       per, partials);
+                       per, partials, arrival);
     HODU_HIP(hipGetLastError());
-    if (splits > 1) {
+    if (splits > 1 && !in_kernel) {
         const unsigned blocks = (unsigned)((elems + 1023) / 1024);
         if (Cfg::CK == CK_I8)
             hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, int32_t>), dim3(blocks), dim3(256), 0, ctx->stream,

@@ -71,7 +71,7 @@ template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                int tiles_m, int tiles_n, int stages_per_split,
-                                                               void *__restrict__ partials) {
+                                                               void *__restrict__ partials, int *__restrict__ arrival) {
     extern __shared__ __align__(16) char smem[];
     typedef typename Out<Cfg::OUT>::T out_t;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, PA = Cfg::PA, PB = Cfg::PB, P = Cfg::P;
@@ -117,8 +117,8 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
     const int T_all = g.K / P_ROW_BYTES;
     const int t0 = blockIdx.y * stages_per_split;
     const int T = T_all - t0 < stages_per_split ? T_all - t0 : stages_per_split;
-    const char *const base_a = A + ao + (long)m0 * g.a_m + (long)t0 * P_ROW_BYTES;
-    const char *const base_b = B + bo + (long)n0 * g.b_n + (long)t0 * P_ROW_BYTES;
+    const char *const base_a = uniform_ptr(A + ao + (long)m0 * g.a_m + (long)t0 * P_ROW_BYTES);
+    const char *const base_b = uniform_ptr(B + bo + (long)n0 * g.b_n + (long)t0 * P_ROW_BYTES);
 
     // element e of stage `src`'s issue list (PA of A, then PB of B) into ring slot `slot`
     auto dma_element = [&](int e, int src, int slot) {
@@ -272,7 +272,11 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
     }
 
     char *patch = smem + wave * (32 * (TN * 32 * 4 + 16));
-    if (!Cfg::PROBE && gridDim.y > 1) {
+    if (!Cfg::PROBE && gridDim.y > 1 && arrival != nullptr) {
+        // cut along K, summed here: only the workgroup that arrives last stores the tile
+        if (!splitk_exchange<Cfg::NW, TM, TN>(acc, partials, arrival, reinterpret_cast<int *>(smem + Cfg::LDS_BYTES - 16), tid)) return;
+        __syncthreads();
+    } else if (!Cfg::PROBE && gridDim.y > 1) {
         float *Pb = (float *)partials + ((long)blockIdx.y * g.batches + batch) * (long)g.M * g.N;
 #pragma unroll
         for (int i = 0; i < TM; i++)
@@ -300,16 +304,21 @@ int launch_pipe_f8(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, co
         splits = (T + per - 1) / per;
     }
     const long elems = g.batches * (long)g.M * g.N;
+    const bool in_kernel = splits > 1 && total <= kArrivalSlots;  // as in launch_pipe
+    int *arrival = nullptr;
     if (splits > 1) {
-        int rc = ensure_workspace(ctx, (size_t)splits * elems * 4);
+        const size_t bytes = in_kernel ? (size_t)splits * total * Cfg::BM * Cfg::BN * 4 : (size_t)splits * elems * 4;
+        int rc = ensure_workspace(ctx, bytes);
+        if (rc == HODU_ROCM_OK && in_kernel) rc = ensure_arrival(ctx);
         if (rc != HODU_ROCM_OK) return rc;
         partials = ctx->workspace.ptr;
+        if (in_kernel) arrival = ctx->arrival;
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)total, (unsigned)(splits > 1 ? splits : 1)), dim3(Cfg::NT), Cfg::LDS_BYTES,
                        ctx->stream, (const char *)a, (const char *)b, (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n,
-                       per, partials);
+                       per, partials, arrival);
     HODU_HIP(hipGetLastError());
-    if (splits > 1) {
+    if (splits > 1 && !in_kernel) {
         const unsigned blocks = (unsigned)((elems + 1023) / 1024);
         hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::OUT, float>), dim3(blocks), dim3(256), 0, ctx->stream,
                            (const float *)partials, (typename Out<Cfg::OUT>::T *)c, elems, splits, g.N, g.epi);

@@ -17,6 +17,7 @@
 #include "common.hpp"
 #include "device_types.hpp"
 #include "gemm_mfma.hpp"
+#include "agent_scope.hpp"
 
 namespace hodu {
 namespace {
@@ -196,39 +197,7 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
 // values are one 16-byte store) and bumps its column block's arrival counter; the workgroup that arrives last
 // adds the slices in slice order -- so the result does not depend on who was last --, rounds once, stores, and
 // zeroes the counter for the next launch.
-//
-// How the partial sums cross from one workgroup to another (they run on different XCDs, each with an L2 of its
-// own that is not kept coherent with the others for ordinary accesses):
-//   * every partial sum is written and read with 16-byte buffer accesses that carry the sc1 bit, the encoding the
-//     gfx942 / gfx950 memory model gives an agent-scope atomic store / load: the store writes through the XCD's L2
-//     to memory, the load is served from the point all XCDs share and cannot hit a stale line this XCD kept from
-//     an earlier launch.  They are compiler builtins, so the wait-count bookkeeping of every load is the
-//     compiler's own;
-//   * release: each thread waits for its own stores (s_waitcnt vmcnt(0): a write-through store is acknowledged once
-//     it is visible at agent scope), the workgroup barrier follows, and only then does thread 0 increment the
-//     counter.  A release FENCE at agent scope would add a write-back of the whole L2 (buffer_wbl2), which exists
-//     for dirty lines of ordinary stores; there are none to publish here -- everything published was written
-//     through -- and it measured 7 us per launch;
-//   * acquire: the workgroup that finds slices - 1 in the counter has, by the counter's atomicity, been preceded by
-//     every other slice's increment and therefore by their completed stores; it passes its own barrier and reads
-//     with the sc1 loads above, which do not depend on an invalidate of this XCD's caches (buffer_inv, the other
-//     half of an acquire fence, is for ordinary loads).
-// The counter itself is a relaxed agent-scope read-modify-write, executed where all XCDs see it.
-constexpr int AUX_SC1 = 16;  // cache-policy bit of the raw buffer builtins that sets sc1 on gfx942 / gfx950
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t agent_buffer(void *base, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(base, 0, bytes, 0x00020000);  // raw buffer: no stride, 32-bit format
-}
-template <typename V>
-__device__ __forceinline__ void store16_agent(__amdgpu_buffer_rsrc_t r, unsigned byte_off, const V &v) {
-    static_assert(sizeof(V) == 16, "one 16-byte access");
-    __builtin_amdgcn_raw_buffer_store_b128(bitcast<u32x4_t>(v), r, byte_off, 0, AUX_SC1);
-}
-template <typename V>
-__device__ __forceinline__ V load16_agent(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
-    static_assert(sizeof(V) == 16, "one 16-byte access");
-    return bitcast<V>(__builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, AUX_SC1));
-}
-
+// How the partial sums cross from one workgroup to another: agent_scope.hpp.
 constexpr int SK_ROWS = 128;  // weight rows per workgroup
 constexpr int SK_XVEC = 8;    // 16-byte vectors of x per thread: 512 threads x 8 x 16 B = 64 KB covers M = 16 x 2048 k of bf16
 constexpr int SK_XBYTES = SK_XVEC * 512 * 16;
@@ -321,17 +290,8 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
     // scope and waited for before the barrier
     const __amdgpu_buffer_rsrc_t part = agent_buffer(partials, (unsigned)slices * (unsigned)g.N * 64u);
     if (n_ok) store16_agent(part, (((unsigned)ks * g.N + n) * 4 + lg) * 16u, acc);
-    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0): this thread's stores are visible at agent scope
-
-    // every thread's sums have landed before the barrier; thread 0 then counts this workgroup in.  Whoever sees
-    // slices - 1 in the counter is last.
-    __syncthreads();
-    if (tid == 0) {
-        const int before = __hip_atomic_fetch_add(&arrival[nb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        last_flag = before == slices - 1;
-    }
-    __syncthreads();
-    if (!last_flag) return;
+    // every thread's sums have landed before thread 0 counts this workgroup in; whoever finds slices - 1 is last
+    if (!arrive_and_check_last(&arrival[nb], slices, &last_flag, tid)) return;
     // 128 columns x 4 quads of m: thread -> (column, quad); the other workgroups' sums are read at agent scope
     // (a plain load could be served from a line this XCD cached during an earlier launch)
     const int col = nb * SK_ROWS + (tid >> 2), quad = tid & 3;
@@ -359,7 +319,7 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
             if (m < g.M) Y[(long)m * g.N + col] = v;
         }
     }
-    if (tid == 0) __hip_atomic_store(&arrival[nb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrival_reset(&arrival[nb], tid);
 }
 
 // applicable when one product (no batch) is wide and deep enough to be cut; returns UNSUPPORTED otherwise
