@@ -47,8 +47,19 @@ INFINITY_CACHE_BYTES = 256 << 20
 # HBM bytes per launch from the rocprofv3 --pmc runs summarised under profiles/ (FETCH_SIZE + WRITE_SIZE, each scaled
 # by what the counter reads for a plain copy of known size).  A figure is reported only for the (kernel, configuration)
 # pair it was measured on, together with the file that holds the measurement; anything else reports null.
+_TRAFFIC_FILE = "profiles/traffic_counters_all_bench_rows.txt"
 MEASURED_TRAFFIC = {
-    # "kernel@config": (bytes per launch, summary file)
+    # "kernel@config": (bytes per launch: FETCH_SIZE + WRITE_SIZE, each scaled by what it reads for a plain copy; summary file)
+    "mfma_bf16_pipe256x256w8_KK@c5_down_bf16": (734.54e6, _TRAFFIC_FILE),
+    "mfma_bf16_pipe256x256w8_KM@c5_up_bf16": (884.05e6, _TRAFFIC_FILE),
+    "mfma_bf16_f8w_pipe256x256w8_KK@c3_m4096": (200.41e6, _TRAFFIC_FILE),
+    "mfma_bf16_f8w_pipe128x128_KK_splitk4@c3_m256": (69.03e6, _TRAFFIC_FILE),
+    "skinny_bf16_f8w_splitk@c3_m16": (22.19e6, _TRAFFIC_FILE),
+    "gemv_bf16_f8w@c3_m1": (16.83e6, _TRAFFIC_FILE),
+    "gemv_bf16_f8w@gemv_14336x4096": (58.60e6, _TRAFFIC_FILE),
+    "mfma_f8e4m3_pipe256x256_KK@f8_4096": (116.96e6, _TRAFFIC_FILE),
+    "mfma_i32_i8i8_pipe128x128_KM@c4": (41.82e6, _TRAFFIC_FILE),
+    "mfma_bf16_pipe256x256w8_KK@c2": (100.24e6, _TRAFFIC_FILE),
 }
 
 
@@ -526,12 +537,12 @@ def time_sum_case(ctx, key, label, view, dims, steps, warmup):
                            "median": 0.5 * (spread[4] + spread[5]), "p90": spread[-2]}}
 
 
-def host_buffers_probe(ctx, reps=5):
-    """config 2 with the operands starting and the result ending in host memory (pageable numpy arrays through
+def host_buffers_probe(ctx, key, reps=5):
+    """one configuration with the operands starting and the result ending in host memory (pageable numpy arrays through
     hodu_rocm_memcpy_h2d / _d2h, buffers allocated beforehand): what a caller pays who hands host buffers over per
     product instead of keeping tensors on the device.  Never the headline value."""
     import time
-    case = build_cases(["c2"])[0]
+    case = next(c for c in build_cases({"c2", "c5"}) if c.key == key)
     md, obytes = out_bytes(case)
     a_host, b_host = np.ascontiguousarray(case.make_a()), np.ascontiguousarray(case.make_b())
     a, b, out = ctx.alloc(a_host.nbytes), ctx.alloc(b_host.nbytes), ctx.alloc(obytes)
@@ -553,7 +564,7 @@ def host_buffers_probe(ctx, reps=5):
     for buf in (a, b, out):
         buf.free()
     moved = a_host.nbytes + b_host.nbytes + res.nbytes
-    return {"config": "c2_host_buffers", "ms_per_product": s_per * 1e3, "tflops": case.flops / s_per / 1e12,
+    return {"config": key + "_host_buffers", "ms_per_product": s_per * 1e3, "tflops": case.flops / s_per / 1e12,
             "bytes_over_pcie": moved, "gbs_over_pcie": moved / s_per / 1e9, "host_memory": "pageable"}
 
 
@@ -839,7 +850,7 @@ def main():
         ctx.close()
         return
     if args.only == "pcie":
-        print(json.dumps(host_buffers_probe(ctx)))
+        print(json.dumps({"config": "pcie", "rows": [host_buffers_probe(ctx, k) for k in ("c5_down_bf16", "c2")]}))
         ctx.close()
         return
     if args.only == "clock":

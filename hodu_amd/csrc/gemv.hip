@@ -11,10 +11,12 @@
 // pairs (v_cvt_scalef32_pk_bf16_fp8, exact) and v_dot2_f32_bf16 accumulates in f32; the 64 partial
 // sums of an output meet through DPP row operations, and the sum is rounded once to bf16.
 //
-// Measured alternatives that did not pay on 4096 x 4096 f8e4m3 weights (5.1 us as built): staging the
+// Measured alternatives that did not pay on 4096 x 4096 f8e4m3 weights (4.9 us as built): staging the
 // activations in LDS (+0.7 us: a barrier in front of the first multiply), renumbering workgroups so
-// that one XCD writes whole output lines (+0.1 us), four rows per wavefront (+0.3 us).  Of the 5.1 us,
-// 2.5 us is the launch cadence of an empty kernel and about 0.3 us the acknowledged output store.
+// that one XCD writes whole output lines (+0.1 us), four rows per wavefront (+0.3 us).  Non-temporal
+// weight loads did pay (5.1 -> 4.9 us).  A kernel that only reads the same 16.8 MB, in any of five
+// shapes of grid and loads in flight, takes 3.9-4.3 us, an empty kernel launches every 1.3-2.4 us
+// (it varies from machine to machine), and about 0.3 us is the acknowledged output store.
 #include "common.hpp"
 #include "device_types.hpp"
 #include "gemm_mfma.hpp"
@@ -100,7 +102,9 @@ __global__ __launch_bounds__(NW * 64, (M <= 2 ? 4 : 2)) void gemv_rowstream_kern
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 wv[r][c] = u32x4_t{0u, 0u, 0u, 0u};
-                if (k < K) wv[r][c] = *reinterpret_cast<const u32x4_t *>(wrow[r] + (long)k * SB);
+                // (read once, by this wavefront alone: the non-temporal hint keeps the weight stream from evicting the
+                // activations every wavefront re-reads out of L2)
+                if (k < K) wv[r][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(wrow[r] + (long)k * SB));
             }
         }
     };

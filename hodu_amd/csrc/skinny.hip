@@ -36,6 +36,9 @@ constexpr int CHUNK = 8;                 // weight vectors in flight per lane (8
 constexpr int X_LDS_LIMIT = 144 * 1024;  // bytes of LDS the staged left operand may take
 
 __device__ __forceinline__ u32x4_t ldg16(const char *p) { return *reinterpret_cast<const u32x4_t *>(p); }
+// a weight vector: read once by one wavefront, so with the non-temporal hint (the stream then does not push the
+// activations, which every workgroup re-reads, out of L2)
+__device__ __forceinline__ u32x4_t ldg16_stream(const char *p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p)); }
 
 // 16 f8e4m3 -> two chunks of 8 bf16 (exact)
 __device__ __forceinline__ void widen_f8x16(const u32x4_t &w, u32x4_t &lo, u32x4_t &hi) {
@@ -108,7 +111,7 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
 #pragma unroll
     for (int u = 0; u < CHUNK; u++) {
         const int k = kbeg + (u * 4 + lg) * EPL;
-        wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+        wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
     }
     if (x_pitch > 0) {
 #pragma unroll
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
 #pragma unroll
             for (int u = 0; u < CHUNK; u++) {
                 const int k = kb + (u * 4 + lg) * EPL;
-                wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+                wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
             }
         }
 #pragma unroll
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
 #pragma unroll
     for (int u = 0; u < CHUNK; u++) {
         const int k = kbeg + (u * 4 + lg) * EPL;
-        wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+        wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
     }
 #pragma unroll
     for (int i = 0; i < XB; i++) {
@@ -264,7 +267,7 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
 #pragma unroll
             for (int u = 0; u < CHUNK; u++) {
                 const int k = kb + (u * 4 + lg) * EPL;
-                wv[u] = k < kend ? ldg16(wrow + (long)k * SB) : mfma::zero4();
+                wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
             }
         }
 #pragma unroll

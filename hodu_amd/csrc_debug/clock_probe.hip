@@ -9,6 +9,8 @@
 #include "common.hpp"
 #include "device_types.hpp"
 
+#include <type_traits>
+
 namespace hodu {
 namespace {
 
@@ -56,14 +58,15 @@ __global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restri
 
 // the simplest possible reader: every lane loads PER 16-byte vectors, all in flight at once, and folds them into a
 // value that is (almost) never stored
-template <int PER>
+template <int PER, bool NT>
 __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t *__restrict__ src, unsigned *__restrict__ sink, long n_vec) {
     const long base = (long)blockIdx.x * PER * 256 + threadIdx.x;
     u32x4_t v[PER];
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const long j = base + (long)i * 256;
-        v[i] = j < n_vec ? src[j] : u32x4_t{0u, 0u, 0u, 0u};
+        v[i] = u32x4_t{0u, 0u, 0u, 0u};
+        if (j < n_vec) v[i] = NT ? __builtin_nontemporal_load(src + j) : src[j];
     }
     unsigned x = 0;
 #pragma unroll
@@ -90,10 +93,8 @@ extern "C" int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const 
         if (!src_list[i] || (uintptr_t)src_list[i] % 16 != 0) return fail(HODU_ROCM_INVALID_ARG, "read_floor: bad buffer %zu", i);
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
-    constexpr int PER = 8;
     const long n_vec = (long)(bytes / 16);
-    const long blocks = (n_vec + PER * 256 - 1) / (PER * 256);
-    if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "read_floor: buffer too large");
+    if ((n_vec + 4 * 256 - 1) / (4 * 256) > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "read_floor: buffer too large");
     unsigned *sink = nullptr;
     HODU_HIP(hipMalloc((void **)&sink, 256 * sizeof(unsigned)));
     hipEvent_t t0, t1;
@@ -109,10 +110,25 @@ extern "C" int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const 
         if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
         *us = ms * 1e3f / (float)iters;
     };
-    timed([&](int i) {
-        hipLaunchKernelGGL(stream_read_kernel<PER>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
-                           (const u32x4_t *)src_list[(size_t)i % n_src], sink, n_vec);
-    }, read_us);
+    // the fastest of several shapes of the same read -- 4, 8 or 16 loads in flight per lane, plain and with the
+    // non-temporal hint -- so that the figure is a floor of the memory system and not of one kernel shape
+    *read_us = 1e30f;
+    auto shape = [&](auto per_, auto nt_) {
+        constexpr int PER = decltype(per_)::value;
+        constexpr bool NT = decltype(nt_)::value;
+        const unsigned blocks = (unsigned)((n_vec + PER * 256 - 1) / (PER * 256));
+        float us = 0.f;
+        timed([&](int i) {
+            hipLaunchKernelGGL((stream_read_kernel<PER, NT>), dim3(blocks), dim3(256), 0, ctx->stream,
+                               (const u32x4_t *)src_list[(size_t)i % n_src], sink, n_vec);
+        }, &us);
+        if (us < *read_us) *read_us = us;
+    };
+    shape(std::integral_constant<int, 8>{}, std::false_type{});
+    shape(std::integral_constant<int, 8>{}, std::true_type{});
+    shape(std::integral_constant<int, 4>{}, std::false_type{});
+    shape(std::integral_constant<int, 16>{}, std::false_type{});
+    shape(std::integral_constant<int, 16>{}, std::true_type{});
     timed([&](int) { hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, ctx->stream); }, empty_us);
     (void)hipEventDestroy(t0);
     (void)hipEventDestroy(t1);

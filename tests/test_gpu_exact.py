@@ -116,3 +116,53 @@ def test_pipelined_split_k_through_the_workspace(ctx, splits):
 def test_batched_and_broadcast_exact(ctx):
     run_exact(ctx, "matmul", "bf16", V([3, 160, 512]), V([3, 136, 512]).t(), 1, "mfma_bf16")
     run_exact(ctx, "matmul", "bf16_f8e4m3w", V([4, 128, 512]), V([512, 256]).broadcast_to([4, 512, 256]), 2, "mfma_bf16_f8w")
+
+
+def narrow_e5m2_rne(x):
+    """round-to-nearest-even of values that float16 holds exactly (|x| < 2048 integers) to f8e5m2 codes"""
+    h = np.asarray(x, dtype=np.float16)
+    assert np.array_equal(h.astype(np.float64), x)
+    bits = h.view(np.uint16).astype(np.uint32)
+    return ((bits + 0x7F + ((bits >> 8) & 1)) >> 8).astype(np.uint8)
+
+
+@pytest.mark.parametrize("dt", ["f8e4m3", "f8e5m2"])
+@pytest.mark.parametrize("tile", [11, 12])
+def test_native_f8_products_narrow_the_exact_sum_once(ctx, dt, tile):
+    """f8 x f8 -> f8 on the 8-bit matrix instruction: operands in {-2 .. 2} (exact in both formats), so the f32 sum is
+    the exact integer in any order and the stored code must be its round-to-nearest-even, saturating at 448 for
+    f8e4m3 -- bit for bit, across the ties (sums like 17, 18, 20 ... fall between f8e4m3 codes) and, uncut and cut
+    three ways along K"""
+    g = H.rng(300 + tile)
+    enc = (lambda v: H.f32_to_ocp_e4m3_rne(v.astype(np.float64))) if dt == "f8e4m3" else narrow_e5m2_rne
+    ctx.force_tile(tile)
+    try:
+        for (m, n, k), splits, top in (((296, 200, 640), -1, 2), ((296, 200, 1280), 3, 2), ((130, 264, 2048), -1, 6 if dt == "f8e4m3" else 3)):
+            av = g.integers(-top, top + 1, m * k).astype(np.float64)
+            bv = g.integers(-top, top + 1, n * k).astype(np.float64)
+            a, b = enc(av), enc(bv)
+            assert np.array_equal(H.widen(dt, a), av) and np.array_equal(H.widen(dt, b), bv)
+            md = H.dot_md(V([m, k]), V([n, k]).t())
+            da, db, dout = ctx.upload(a), ctx.upload(b), ctx.alloc(m * n)
+            ctx.fill(dout, 0xFF)
+            ctx.force_splitk(splits)
+            ctx.product("dot", dt, da, db, dout, md)
+            got = ctx.download(dout, np.uint8, m * n)
+            kernel = ctx.last_kernel()
+            for d in (da, db, dout):
+                d.free()
+            assert kernel.startswith(f"mfma_{dt}_pipe") and (splits < 0 or "splitk" in kernel), kernel
+            exact = (av.reshape(m, k) @ bv.reshape(n, k).T).ravel()
+            if dt == "f8e4m3":
+                want = H.f32_to_ocp_e4m3_rne(np.clip(exact, -448.0, 448.0))
+                assert np.abs(exact).max() > 448 or top == 2  # the wide-range case saturates in places
+            else:
+                assert np.abs(exact).max() < 2048
+                want = narrow_e5m2_rne(exact)
+            # +0 and -0 are one value: an exact zero sum is stored as +0
+            bad = np.flatnonzero(got != want)
+            assert bad.size == 0, f"{kernel}: {bad.size} of {got.size} codes differ, first at {bad[:5]}: " \
+                                  f"{got[bad[:5]]} for sums {exact[bad[:5]]}"
+    finally:
+        ctx.force_tile(-1)
+        ctx.force_splitk(-1)
