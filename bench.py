@@ -55,8 +55,6 @@ MEASURED_TRAFFIC = {
     "mfma_bf16_f8w_pipe256x256w8_KK@c3_m4096": (200.41e6, _TRAFFIC_FILE),
     "mfma_bf16_f8w_pipe128x128_KK_splitk4@c3_m256": (69.03e6, _TRAFFIC_FILE),
     "skinny_bf16_f8w_splitk@c3_m16": (22.19e6, _TRAFFIC_FILE),
-    "gemv_bf16_f8w@c3_m1": (16.83e6, _TRAFFIC_FILE),
-    "gemv_bf16_f8w@gemv_14336x4096": (58.60e6, _TRAFFIC_FILE),
     "mfma_f8e4m3_pipe256x256_KK@f8_4096": (116.96e6, _TRAFFIC_FILE),
     "mfma_i32_i8i8_pipe128x128_KM@c4": (41.82e6, _TRAFFIC_FILE),
     "mfma_bf16_pipe256x256w8_KK@c2": (100.24e6, _TRAFFIC_FILE),

@@ -17,7 +17,8 @@ extern "C" {
 
 /* testing hook: pin the MFMA tile variant (0 = 256x256 with 8 wavefronts, 1 = 256x256 with 4,
  * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
- * GEMV kernel, 31/32/34 = that kernel with 1/2/4 weight rows per wavefront; 14 = the pipelined 256x128 tile;
+ * GEMV kernel, 31/32/34 = that kernel as one-shot wavefronts (4 x 1, 4 x 2, 8 x 2 wavefronts x weight rows per workgroup),
+ * 33 = its row-walking form (one wavefront per SIMD, the default from 16 weight rows per compute unit); 14 = the pipelined 256x128 tile;
  * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
  * variant that cuts K across workgroups wherever it applies; 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
  * 128 x 128 / 64 x 64 / 32 x 32 tiles;

@@ -67,6 +67,9 @@ def test_row_streaming_gemv(ctx, name, m):
     pre = "gemv_bf16_f8w" if name == "bf16_f8e4m3w" else "gemv_bf16"
     run_exact(ctx, "dot", name, V([m, 4096]), V([1024, 4096]).t(), m, pre)
     run_exact(ctx, "dot", name, V([m, 4112]), V([203, 4112]).t(), 10 + m, pre)
+    # from 4096 weight rows on a wavefront walks several row groups; K of one pass and of several
+    run_exact(ctx, "dot", name, V([m, 4096]), V([4610, 4096]).t(), 20 + m, pre)
+    run_exact(ctx, "dot", name, V([m, 9216]), V([4100, 9216]).t(), 30 + m, pre)
 
 
 @pytest.mark.parametrize("name", ["bf16_f8e4m3w", "bf16"])
@@ -166,3 +169,4 @@ def test_native_f8_products_narrow_the_exact_sum_once(ctx, dt, tile):
     finally:
         ctx.force_tile(-1)
         ctx.force_splitk(-1)
+

@@ -101,7 +101,7 @@ def test_not_applicable_layouts_fall_through(ctx):
 # ---- row-streaming GEMV kernel (M <= 4, bf16 activations, bf16 or f8e4m3 weights) ---------------------
 @pytest.mark.parametrize("kind", list(GEMV_KINDS))
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
-@pytest.mark.parametrize("rows", [-1, 31, 32, 34])
+@pytest.mark.parametrize("rows", [-1, 31, 32, 33, 34])
 def test_gemv_rowstream(ctx, kind, m, rows):
     rs = 2.0 if "f8" in kind else None
     name = GEMV_KINDS[kind]
@@ -116,6 +116,12 @@ def test_gemv_rowstream(ctx, kind, m, rows):
         # row-sliced weight and activations (leading dimension > K) at aligned offsets
         check_product(ctx, "dot", kind, V([m, 512]).slice(1, 128, 384), V([24, 512], offset=64).slice(1, 64, 320).t(),
                       seed=30 + m, rscale=rs, expect_kernel=name)
+        if rows in (-1, 33):
+            # more row groups than wavefronts in the grid: a wavefront walks up to three groups, the last round ragged
+            # (from 4096 rows on this is the kernel chosen without a pin); K of one pass, of a long pass, of several
+            check_product(ctx, "dot", kind, V([m, 1040]), V([5001, 1040]).t(), seed=40 + m, rscale=rs, expect_kernel=name + "_walk")
+            check_product(ctx, "dot", kind, V([m, 4112]), V([4100, 4112]).t(), seed=50 + m, rscale=rs, expect_kernel=name + "_walk")
+            check_product(ctx, "dot", kind, V([m, 8720]), V([4099, 8720]).t(), seed=60 + m, rscale=rs, expect_kernel=name + "_walk")
     finally:
         ctx.force_tile(-1)
 
