@@ -51,7 +51,7 @@ def test_two_calls_in_a_row_the_second_smaller(ctx):
 
 
 def test_shapes_without_scratch(ctx):
-    both(ctx, 1, 4096, 4096, 5, expect="gemv_bf16_f8w")
+    both(ctx, 1, 4096, 4096, 5, expect="gemv_bf16_f8w_walk")
     both(ctx, 8, 640, 1024, 7)
     both(ctx, 512, 512, 1024, 9)
 
