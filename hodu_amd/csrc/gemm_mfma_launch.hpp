@@ -73,6 +73,14 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
         // [64, 512, 512] x [64, 512, 64] measured 11.3 us with 128 x 128 tiles against 14.3 us with 64 x 64)
         if (size == 2 && used(128) < 0.5 * used(64)) size = 3;
     }
+    // 16-bit operands of one type: the 256 x 256 tile on four wavefronts (one per SIMD, 128 x 128 outputs each) reads
+    // a third fewer fragment bytes out of LDS than on eight and measured 2 % ahead (config 5 down 335 against 341 us,
+    // up 368 against 376); with f8e4m3 weights, whose widening wants a second wavefront on the SIMD to hide behind,
+    // eight stay ahead (349 against 355 us), and so they do when element-wise steps ride on the store (config 2 with the
+    // attention scale: 38 against 44 us)
+    if constexpr (SKA == SK_SAME && SKB == SK_SAME && ES == 2) {
+        if (forced < 0 && size == 0 && g.epi.n == 0) size = 1;
+    }
     // A product too small to fill the machine with 128x128 tiles is cut along K instead of shrinking the tile
     // further (pipelined kernels only): same HBM traffic, four times fewer bytes through LDS per flop.
     const int stages = (int)((long)g.K * ES / 128);

@@ -540,7 +540,10 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
             }
 #pragma unroll
             for (int d = 0; d < DN; d++) {
-                if (d * MF / (DN > 0 ? DN : 1) != idx) continue;
+                // (in the gaps BETWEEN those that take a fragment read where the spacing allows it: a read and a DMA
+                // instruction behind the same MFMA take longer to issue than the MFMA runs, and the next one starts late)
+                constexpr int GAP = DN > 0 ? MF / DN : 1;
+                if (d * MF / (DN > 0 ? DN : 1) + (GAP > 1 ? GAP / 2 : 0) != idx) continue;
                 if (do_dma) dma_element(D0 + d, f);
             }
             __builtin_amdgcn_sched_barrier(0);
