@@ -59,7 +59,11 @@
  * as for the products, the GPU is gated against the f32 comparator, not against that chain.
  *
  * Parity unpinned: float->integer casts of out-of-range or NaN inputs are undefined behaviour
- * in the reference C ((T)x) and are not checked.
+ * in the reference C ((T)x) and are not checked.  The stored code of an f8 x f8 -> f8 product: the reference
+ * narrows an accumulator that it re-rounded to f8 after every k with float_to_f8e4m3 (t_f8e4m3.h:52-85); the device
+ * rounds the f32 sum once, to nearest even, saturating.  No fixture of the reference holds an f8 product, so the
+ * device's f8 outputs are checked against the SPEC value narrowed by an independent round-to-nearest-even encoder
+ * (bit for bit on exactly representable sums, tests/test_gpu_exact.py), not against the reference's bytes.
  */
 #include <math.h>
 #include <stdbool.h>
