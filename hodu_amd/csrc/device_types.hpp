@@ -24,11 +24,15 @@ typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void batch_offsets(const DevProduct &g, long batch, long &ao, long &bo) {
     ao = g.a_off;
     bo = g.b_off;
+    // (a batch index is below 2^31 -- a grid has no more workgroups than that -- and 32-bit unsigned division is a
+    // fraction of the instructions of the 64-bit signed one)
+    unsigned rest = (unsigned)batch;
 #pragma unroll
     for (int d = kKernelBatchDims - 1; d >= 0; d--) {
         if (d < g.nb) {
-            const long i = batch % g.bshape[d];
-            batch /= g.bshape[d];
+            const unsigned extent = (unsigned)g.bshape[d], q = rest / extent;
+            const long i = (long)(rest - q * extent);
+            rest = q;
             ao += i * g.a_bs[d];
             bo += i * g.b_bs[d];
         }

@@ -29,6 +29,7 @@
 
 #include "common.hpp"
 #include "device_types.hpp"
+#include "tile_walk.hpp"
 #include "epilogue.hpp"
 
 namespace hodu {
@@ -642,20 +643,13 @@ template <int CK_, int SKA_, int SKB_, int OUT_, int BM_, int BN_, int WM_, int 
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
 
-// maps the linear workgroup id to (batch, tile_m, tile_n): ids that land on one XCD (id % 8) get
-// neighbouring tiles, and tiles are walked in groups of 8 tile-rows so that the A and B panels a
-// group shares stay in that XCD's L2
+// maps the linear workgroup id to (batch, tile_m, tile_n): tile_walk.hpp
 __device__ __forceinline__ void tile_of(long pid, long total, int tiles_m, int tiles_n, long &batch, int &tm, int &tn) {
-    if (total % 8 == 0) pid = (pid % 8) * (total / 8) + pid / 8;
-    const long per_batch = (long)tiles_m * tiles_n;
-    batch = pid / per_batch;
-    const int t = (int)(pid % per_batch);
-    constexpr int GROUP = 8;
-    const int width = GROUP * tiles_n;
-    const int first_m = (t / width) * GROUP;
-    const int gsize = (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
-    tm = first_m + (t % width) % gsize;
-    tn = (t % width) / gsize;
+    unsigned b, m, n;
+    tile_walk((unsigned)pid, (unsigned)total, (unsigned)tiles_m, (unsigned)tiles_n, b, m, n);
+    batch = b;
+    tm = (int)m;
+    tn = (int)n;
 }
 
 // One K step (128 bytes of K = four 32-byte slices) out of LDS.  The fragments of slice s+1 are read
