@@ -166,30 +166,43 @@ __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
                    f8pair_to_bf16pair(v.y, true)};
 }
 
-// Epilogue for one 32-row band of a wavefront's tile (TN accumulator tiles side by side): the values go through a
+// Epilogue for one band of a wavefront's tile (TN accumulator tiles side by side; 32 rows, or 16 with TS = 16): the values go through a
 // wavefront-private patch of LDS so that they leave as whole rows -- 16 contiguous bytes per lane, a row of the
 // band per 2..16 lanes -- instead of the accumulator layout's 8-byte pieces of 32 different rows per instruction
 // (measured: 13 us of a 37 us launch spent storing a 256 x 256 bf16 tile that way).
 //   acc layout (operands swapped): lane (lr, lh) holds row lr, columns 32*j + 8*q + 4*lh + e of the band.
 // EPI: the values are final outputs and take the fused element-wise steps (partial sums of a K range do not).
-template <int OUT, int TN, bool EPI, class acc_t>
+// TS = 16: bands of 16 rows out of 16 x 16 accumulators, where lane (r = lane % 16, g = lane / 16) holds row r,
+// columns 16*j + 4*g + e.
+template <int OUT, int TN, bool EPI, class acc_t, int TS = 32>
 __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,
                                                    int n_base, int lane, int M, int N, const DevEpilogue &epi) {
     typedef typename Out<OUT>::T out_t;
-    constexpr int OS = sizeof(out_t), ROWB = TN * 32 * OS, PITCH = ROWB + 16, EPV = 16 / OS;
+    constexpr int OS = sizeof(out_t), ROWB = TN * TS * OS, PITCH = ROWB + 16, EPV = 16 / OS;
     constexpr int CPR = ROWB / 16, RPP = 64 / CPR;  // 16-byte chunks per row, rows per pass of the wavefront
-    static_assert(CPR <= 64 && 32 % RPP == 0, "band geometry");
-    const int lr = lane & 31, lh = lane >> 5;
+    static_assert((TS == 32 || TS == 16) && CPR <= 64 && TS % RPP == 0, "band geometry");
+    struct alignas(OS * 4) Quad { out_t v[4]; };
+    if constexpr (TS == 32) {
+        const int lr = lane & 31, lh = lane >> 5;
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            struct alignas(OS * 4) Quad { out_t v[4]; };
+            for (int q = 0; q < 4; q++) {
+                Quad w;
+#pragma unroll
+                for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][4 * q + e]);
+                *reinterpret_cast<Quad *>(patch + lr * PITCH + (j * 32 + 8 * q + 4 * lh) * OS) = w;
+            }
+    } else {
+        const int r16 = lane & 15, g4 = lane >> 4;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
             Quad w;
 #pragma unroll
-            for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][4 * q + e]);
-            *reinterpret_cast<Quad *>(patch + lr * PITCH + (j * 32 + 8 * q + 4 * lh) * OS) = w;
+            for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][e]);
+            *reinterpret_cast<Quad *>(patch + r16 * PITCH + (j * 16 + 4 * g4) * OS) = w;
         }
+    }
     // the same wavefront reads what it wrote: the LDS operations of one wavefront complete in order, and the
     // compiler is told not to move the differently-typed accesses across each other
     asm volatile("" ::: "memory");
@@ -224,14 +237,14 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
         // instructions per element, inlined once per band this way instead of once per pass
         if constexpr (Out<OUT>::DT == HODU_F16) {
 #pragma unroll 1
-            for (int pass = 0; pass < 32 / RPP; pass++) row_chunk(pass, std::true_type{});
+            for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::true_type{});
         } else {
 #pragma unroll
-            for (int pass = 0; pass < 32 / RPP; pass++) row_chunk(pass, std::true_type{});
+            for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::true_type{});
         }
     } else {
 #pragma unroll
-        for (int pass = 0; pass < 32 / RPP; pass++) row_chunk(pass, std::false_type{});
+        for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::false_type{});
     }
     asm volatile("" ::: "memory");  // the next band overwrites the patch
 }

@@ -16,7 +16,9 @@ namespace {
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-// KIND 0: v_mfma_f32_32x32x16_bf16; KIND 1: v_mfma_scale_f32_32x32x64_f8f6f4 on f8e4m3 with unit scales
+// KIND 0: v_mfma_f32_32x32x16_bf16; KIND 1: v_mfma_scale_f32_32x32x64_f8f6f4 on f8e4m3 with unit scales;
+// KIND 2: v_mfma_f32_16x16x32_bf16 (half the flop per instruction of KIND 0, a quarter of the accumulator registers)
+typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
 template <int KIND>
 __global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restrict__ operands, float *__restrict__ sink,
                                                         unsigned long long *__restrict__ clocks, int iters) {
@@ -28,6 +30,30 @@ __global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restri
     for (int i = 0; i < NACC; i++)
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[i][e] = 0.f;
+    if constexpr (KIND == 2) {
+        // eight independent 16 x 16 accumulators, two instructions per accumulator and trip: the same flop per
+        // trip as KIND 0
+        f32x4_acc_t small[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) small[i] = f32x4_acc_t{0.f, 0.f, 0.f, 0.f};
+        const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                // (written out: left to the register allocator, the eight accumulators rotate through copies)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(small[i]) : "v"(a0), "v"(b0));
+        }
+        const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) v += small[i][0] + small[i][1] + small[i][2] + small[i][3];
+        sink[blockIdx.x * 256 + t] = v + a1.x + b1.x;
+        if (blockIdx.x == 0 && t == 0) {
+            clocks[0] = c1 - c0;
+            clocks[1] = r1 - r0;
+        }
+        return;
+    }
     const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
     for (int it = 0; it < iters; it++) {
 #pragma unroll
@@ -140,7 +166,7 @@ extern "C" int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const 
 extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
                                           double *tflops, double *shader_mhz) {
     clear_error();
-    if (!ctx || !operands || iters <= 0 || !elapsed_ms || !tflops || !shader_mhz || kind < 0 || kind > 1)
+    if (!ctx || !operands || iters <= 0 || !elapsed_ms || !tflops || !shader_mhz || kind < 0 || kind > 2)
         return fail(HODU_ROCM_INVALID_ARG, "mfma_clock: bad argument");
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
@@ -155,6 +181,8 @@ extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const vo
     auto launch = [&](int n) {
         if (kind == 0)
             hipLaunchKernelGGL(mfma_clock_kernel<0>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
+        else if (kind == 2)
+            hipLaunchKernelGGL(mfma_clock_kernel<2>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
         else
             hipLaunchKernelGGL(mfma_clock_kernel<1>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
     };
@@ -177,9 +205,9 @@ extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const vo
     (void)hipFree(sink);
     (void)hipFree(clocks);
     if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "mfma_clock: %s", hipGetErrorString(e));
-    // flop per MFMA: 32 x 32 x k x 2 with k = 16 (bf16) or 64 (f8)
-    const double per_mfma = kind == 0 ? 32768.0 : 131072.0;
-    *tflops = (double)blocks * 4 /* wavefronts */ * 4 /* accumulators */ * (double)iters * per_mfma / (*elapsed_ms * 1e-3) / 1e12;
+    // flop per trip of the loop: four 32 x 32 x k x 2 instructions with k = 16 (bf16) or 64 (f8), or eight 16 x 16 x 32 x 2
+    const double per_trip = kind == 0 ? 4 * 32768.0 : kind == 2 ? 8 * 16384.0 : 4 * 131072.0;
+    *tflops = (double)blocks * 4 /* wavefronts */ * (double)iters * per_trip / (*elapsed_ms * 1e-3) / 1e12;
     *shader_mhz = h[1] ? (double)h[0] / (double)h[1] * 100.0 : 0.0;
     return HODU_ROCM_OK;
 }

@@ -18,7 +18,8 @@ extern "C" {
 /* testing hook: pin the MFMA tile variant (0 = 256x256 with 8 wavefronts, 1 = 256x256 with 4,
  * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
  * GEMV kernel, 31/32/34 = that kernel as one-shot wavefronts (4 x 1, 4 x 2, 8 x 2 wavefronts x weight rows per workgroup),
- * 33 = its row-walking form (one wavefront per SIMD, the default from 16 weight rows per compute unit); 14 = the pipelined 256x128 tile;
+ * 33 = its row-walking form (one wavefront per SIMD, the default from 16 weight rows per compute unit); 14 = the pipelined 256x128 tile,
+ * 15 = the pipelined 256x256 tile on the 16x16x32 instruction (two k-dense 16-bit operands; 11 pins the 32x32x16 one);
  * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
  * variant that cuts K across workgroups wherever it applies; 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
  * 128 x 128 / 64 x 64 / 32 x 32 tiles;
@@ -45,7 +46,7 @@ int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int ki
 
 /* measurement hook: the rate and shader clock of a register-only MFMA loop (no LDS, no memory traffic) on
  * caller-supplied operand bits, two workgroups per compute unit.  kind 0: bf16 32x32x16; kind 1: f8e4m3 32x32x64
- * with unit scales.  `operands`: 16 KB of device memory (1024 x 16 bytes: per lane the a and b fragments, twice).
+ * with unit scales; kind 2: bf16 16x16x32.  `operands`: 16 KB of device memory (1024 x 16 bytes: per lane the a and b fragments, twice).
  * *tflops is what the loop sustained, *shader_mhz the clock one wavefront saw (shader-clock counter over the
  * 100 MHz counter).  Under full MFMA load the clock depends on the data, so this is the ceiling a GEMM kernel can
  * approach on that data. */

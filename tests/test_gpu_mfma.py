@@ -70,6 +70,24 @@ def test_pipelined_kk_variants(ctx, kind, tile, name):
     ctx.force_tile(-1)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+def test_pipelined_kk_16x16_instruction(ctx, kind):
+    """the 256 x 256 tile on the 16 x 16 x 32 matrix instruction (two k-dense 16-bit operands): the shapes of
+    test_pipelined_kk_variants"""
+    prefix = KINDS[kind][0]
+    ctx.force_tile(15)
+    try:
+        for stages in (1, 2, 3, 4, 5, 11):
+            K = stages * 64
+            check_product(ctx, "dot", kind, V([296, K]), V([200, K]).t(), seed=stages, expect_kernel=f"{prefix}_pipe256x256mi16_KK")
+        K = 6 * 64
+        check_product(ctx, "matmul", kind, V([3, 72, 2 * K]).slice(2, K, 2 * K), V([3, 80, K], offset=64).t(), seed=7,
+                      expect_kernel=f"{prefix}_pipe256x256mi16_KK")
+        check_product(ctx, "dot", kind, V([1000, 1024]), V([777, 1024]).t(), seed=8, expect_kernel=f"{prefix}_pipe256x256mi16_KK")
+    finally:
+        ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("kind", ["bf16", "f16", "i32_i8i8"])
 @pytest.mark.parametrize("tile,name", [(10, "pipe256x256w8"), (11, "pipe256x256"), (12, "pipe128x128")])
 @pytest.mark.parametrize("combo", ["KM", "MK", "MM"])
