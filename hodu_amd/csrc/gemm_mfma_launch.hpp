@@ -15,7 +15,7 @@ namespace mfma {
 // type -- the software-pipelined kernels of gemm_mfma_pipe.hpp: KK at four tile shapes and, for the
 // 16-bit types, KM / MK / MM at the three larger ones.  The tile is the largest that still yields at
 // least one workgroup per compute unit.
-constexpr int kVariants = 33;
+constexpr int kVariants = 34;
 template <int CK, int SKA, int SKB, int OUT>
 int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
                 const char *const names[kVariants]) {
@@ -129,11 +129,14 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     };
     const int combo = (la == LM_MN ? 2 : 0) + (lb == LM_MN ? 1 : 0);
     if constexpr (SKA == SK_SAME && SKB == SK_SAME && ES == 2 && CK != CK_I8) {
-        // two k-dense 16-bit operands on the 256 x 256 tile of four wavefronts: the 16 x 16 x 32 instruction, which
+        // 16-bit operands on the 256 x 256 tile of four wavefronts: the 16 x 16 x 32 instruction, which
         // leaves the power-limited part a higher clock than the 32 x 32 x 16 one (hook value 15 pins it, 11 the other)
-        if (pipe_ok && combo == 0 && splits == 1 && ((forced < 0 && size == 1) || size == 5)) {
-            ctx->last_kernel = names[32];
-            return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
+        // (a k-dense left operand: with a row-dense one the per-tile fragment addresses no longer fit beside 128
+        // fragment registers, and the compiler spills inside the loop)
+        if (pipe_ok && combo <= 1 && splits == 1 && ((forced < 0 && size == 1) || size == 5)) {
+            ctx->last_kernel = names[32 + combo];
+            if (combo == 0) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
+            return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
         }
     }
     if (size == 5) return HODU_ROCM_UNSUPPORTED;
@@ -234,7 +237,7 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
      P "_pipe256x256w8_KM", P "_pipe256x256_KM", P "_pipe128x128_KM",                                              \
      P "_pipe256x256w8_MK", P "_pipe256x256_MK", P "_pipe128x128_MK",                                              \
      P "_pipe256x256w8_MM", P "_pipe256x256_MM", P "_pipe128x128_MM",                                              \
-     P "_pipe256x128_KK", P "_pipe256x128_KM", P "_pipe256x256mi16_KK"}
+     P "_pipe256x128_KK", P "_pipe256x128_KM", P "_pipe256x256mi16_KK", P "_pipe256x256mi16_KM"}
 
 }  // namespace mfma
 }  // namespace hodu

@@ -1,5 +1,5 @@
-// The pipelined tile kernel of gemm_mfma_pipe.hpp on the 16 x 16 x 32 matrix instruction, for 16-bit operands that are
-// both k-dense.  Same feeding scheme -- whole 128-byte rows by LDS-DMA into a two-stage ring, source-side XOR swizzle,
+// The pipelined tile kernel of gemm_mfma_pipe.hpp on the 16 x 16 x 32 matrix instruction, for 16-bit operands, k-dense
+// or row-dense.  Same feeding scheme -- whole 128-byte rows by LDS-DMA into a two-stage ring, source-side XOR swizzle,
 // one barrier per 64-k stage, the tile leaving through LDS as whole rows -- and the same sums in the same order per
 // output (k ascending in blocks of 32 instead of 16, which an f32 accumulator of exact products does not see; the
 // bit-for-bit tests on exact-valued operands hold both variants to one result).
@@ -11,7 +11,8 @@
 //
 // What differs from the 32 x 32 kernel:
 //   * a wavefront's 128 x 128 outputs are 8 x 8 accumulators of 4 registers; a fragment is 16 rows x 32 k, 16 bytes per
-//     lane: lane (r = lane % 16, g = lane / 16) reads chunk 4 * slice + g of row r, one ds_read_b128;
+//     lane: lane (r = lane % 16, g = lane / 16) reads chunk 4 * slice + g of row r, one ds_read_b128 (k-dense), or
+//     takes its 8 k of column r out of the k-major stage through two transpose reads of 4 k-rows each (row-dense);
 //   * a stage is TWO slices of 32 k, 64 MFMAs of 16 cycles each.  Slice 0 multiplies while the 16 fragments of slice 1
 //     are read (all issued in its first three quarters, so that they have returned at the barrier that follows it);
 //     behind the barrier slice 1 multiplies while the next stage's slice 0 is read and the whole DMA list of the
@@ -27,26 +28,38 @@ namespace mfma {
 
 typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
 
+// The instruction is written out with the accumulator tied to itself and held in the accumulation registers: left to
+// the register allocator, a kernel with 64 four-register accumulators and 128 fragment registers came out with the
+// accumulators rotating through copies inside the loop (twice the time).  What the compiler then no longer knows about
+// the instruction: an accumulator is next touched 64 MFMAs later (or, behind the loop, after a barrier), and its other
+// operands come from LDS reads the compiler waits for as for any use of a register.
 template <int CK> struct Compute16;
 template <> struct Compute16<CK_BF16> {
     typedef f32x4_acc_t acc_t;
     static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<bf16x8_t>(a), bitcast<bf16x8_t>(b), c, 0, 0, 0);
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 template <> struct Compute16<CK_F16> {
     typedef f32x4_acc_t acc_t;
     static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
-        c = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<f16x8_t>(a), bitcast<f16x8_t>(b), c, 0, 0, 0);
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 
-// Cfg: a PipeConfig with both operands k-dense, stored in the compute type, and a ring of two stages
+// Row-dense stages: chunk c of k-row k sits at slot c ^ rd16_swz(k).  A transpose read is served 32 lanes at a time;
+// the two groups of 16 among them read k-rows 8 apart, columns alike, so besides the (k % 4) << 2 that spreads the
+// four k-rows of one group, bit 3 of k moves a row by two chunks (32 bytes): the 32 lanes then touch every bank once.
+__device__ __forceinline__ int rd16_swz(int k) { return ((k & 3) << 2) ^ (((k >> 3) & 1) << 1); }
+
+// Cfg: a PipeConfig with operands stored in the compute type and a ring of two stages
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                               typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                               int tiles_m, int tiles_n) {
-    static_assert(Cfg::LA == LM_K && Cfg::LB == LM_K && !Cfg::B_F8 && Cfg::ES == 2 && Cfg::NST == 2, "k-dense 16-bit operands, two stages");
+    static_assert(!Cfg::B_F8 && Cfg::ES == 2 && Cfg::NST == 2, "16-bit operands stored in the compute type, two stages");
+    // (a row-dense left operand compiles, but with register spills inside the loop: the launcher does not use it)
+    typedef RowDenseGeom<Cfg::ES, Cfg::ES> G;
     extern __shared__ __align__(16) char smem[];
     typedef Compute16<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
@@ -78,38 +91,70 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
     // plus the lane's 32-bit byte offset inside the tile (the launcher checks that 256 rows stay below 4 GB).
     unsigned offa[PA], offb[PB];
     unsigned lda[PA], ldb[PB];
+    // row-dense operand: an instruction writes KPI consecutive k-rows of the tile's ROWS contiguous elements; lane ->
+    // (k-row, slot), the slot holds chunk slot ^ swz(k); a chunk that starts past the operand's last row is fetched
+    // from the last whole chunk instead (its columns are never stored), and the scalar base is the tile's first
+    // (clamped) column of k-row 0, advanced by a stage's k-rows per stage.
 #pragma unroll
     for (int p = 0; p < PA; p++) {
-        const int q = p * Cfg::NW + wave, trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
-        int row = m0 + trow;
-        row = row < g.M ? row : g.M - 1;
-        offa[p] = (unsigned)((long)(row - m0) * g.a_m * ES) + dchunk * 16;
+        const int q = p * Cfg::NW + wave;
+        if constexpr (Cfg::LA == LM_K) {
+            const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
+            int row = m0 + trow;
+            row = row < g.M ? row : g.M - 1;
+            offa[p] = (unsigned)((long)(row - m0) * g.a_m * ES) + dchunk * 16;
+        } else {
+            constexpr int CPR = Cfg::BM / G::EPC, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ rd16_swz(k);
+            int col = m0 + c * G::EPC;
+            col = col <= g.M - G::EPC ? col : g.M - G::EPC;
+            offa[p] = (unsigned)(((long)k * g.a_k + (col - (m0 <= g.M - G::EPC ? m0 : g.M - G::EPC))) * ES);
+        }
         lda[p] = q * 1024;
     }
 #pragma unroll
     for (int p = 0; p < PB; p++) {
-        const int q = p * Cfg::NW + wave, trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
-        int row = n0 + trow;
-        row = row < g.N ? row : g.N - 1;
-        offb[p] = (unsigned)((long)(row - n0) * g.b_n * ES) + dchunk * 16;
+        const int q = p * Cfg::NW + wave;
+        if constexpr (Cfg::LB == LM_K) {
+            const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
+            int row = n0 + trow;
+            row = row < g.N ? row : g.N - 1;
+            offb[p] = (unsigned)((long)(row - n0) * g.b_n * ES) + dchunk * 16;
+        } else {
+            constexpr int CPR = Cfg::BN / G::EPC, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ rd16_swz(k);
+            int col = n0 + c * G::EPC;
+            col = col <= g.N - G::EPC ? col : g.N - G::EPC;
+            offb[p] = (unsigned)(((long)k * g.b_k + (col - (n0 <= g.N - G::EPC ? n0 : g.N - G::EPC))) * ES);
+        }
         ldb[p] = B_BASE + q * 1024;
     }
     const int T = g.K * ES / P_ROW_BYTES;  // stages
-    const char *const base_a = uniform_ptr(A + (ao + (long)m0 * g.a_m) * ES);
-    const char *const base_b = uniform_ptr(B + (bo + (long)n0 * g.b_n) * ES);
+    const char *const base_a = uniform_ptr(Cfg::LA == LM_K ? A + (ao + (long)m0 * g.a_m) * ES
+                                                           : A + (ao + (m0 <= g.M - G::EPC ? m0 : g.M - G::EPC)) * ES);
+    const char *const base_b = uniform_ptr(Cfg::LB == LM_K ? B + (bo + (long)n0 * g.b_n) * ES
+                                                           : B + (bo + (n0 <= g.N - G::EPC ? n0 : g.N - G::EPC)) * ES);
+    // bytes a stage advances an operand's source by: 128 bytes of k, or a stage's k-rows
+    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : (long)G::STAGE_K * g.a_k * ES;
+    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : (long)G::STAGE_K * g.b_k * ES;
 
     // element e of the list that fetches stage `src` (already clamped to T - 1) into ring slot `slot`
     auto dma_element = [&](int e, int src, int slot) {
 #pragma unroll
         for (int p = 0; p < PA; p++)
-            if (e == p) dma16_sbase(base_a + (long)src * P_ROW_BYTES, offa[p], lds0 + (unsigned)slot * Cfg::A_BYTES + lda[p]);
+            if (e == p) dma16_sbase(base_a + src * a_adv, offa[p], lds0 + (unsigned)slot * Cfg::A_BYTES + lda[p]);
 #pragma unroll
         for (int p = 0; p < PB; p++)
-            if (e == PA + p) dma16_sbase(base_b + (long)src * P_ROW_BYTES, offb[p], lds0 + (unsigned)slot * Cfg::B_BYTES + ldb[p]);
+            if (e == PA + p) dma16_sbase(base_b + src * b_adv, offb[p], lds0 + (unsigned)slot * Cfg::B_BYTES + ldb[p]);
     };
 
-    // fragment addresses: lane (r16, g4) reads chunk 4 * slice + g4 of row r16 of a 16-row tile; every tile starts on
-    // a multiple of 16 rows, so the swizzle term (row >> 1) & 7 is the lane's own
+    // fragment addresses.  k-dense: lane (r16, g4) reads chunk 4 * slice + g4 of row r16 of a 16-row tile; every tile
+    // starts on a multiple of 16 rows, so the swizzle term (row >> 1) & 7 is the lane's own, and the tiles are
+    // immediates.  row-dense: the lane needs k = 32 * slice + 8 * g4 .. + 7 of column r16 of the tile; a transpose
+    // read hands each of 16 lanes 4 consecutive k of its own column out of 4 k-rows, for which lane s of the 16
+    // supplies the address of 4 columns (8 bytes) of k-row (that start) + s / 4.  k % 4 == s / 4 and bit 3 of k is
+    // bit 0 of g4 whatever the slice and the half, so the swizzle is a per-lane constant and slices and halves are immediates; tiles are not (the
+    // swizzle is an XOR on the chunk index), so there is an address per tile.
     constexpr int TILE_BYTES = 16 * P_ROW_BYTES;
     int a_frag[2], b_frag[2];
 #pragma unroll
@@ -117,6 +162,20 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
         const int at = r16 * P_ROW_BYTES + (kd_slot(r16, 4 * sl + g4) << 4);
         a_frag[sl] = (wave_m * TM) * TILE_BYTES + at;
         b_frag[sl] = B_BASE + (wave_n * TN) * TILE_BYTES + at;
+    }
+    int a_mn[TM], b_mn[TN];
+    {
+        const int kq = r16 >> 2, sub = r16 & 3;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int bytes = (wave_m * TM + i) * 16 * ES + sub * 8, c = bytes >> 4;
+            a_mn[i] = (g4 * 8 + kq) * Cfg::BM * ES + ((c ^ rd16_swz(g4 * 8 + kq)) << 4) + (bytes & 8);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int bytes = (wave_n * TN + j) * 16 * ES + sub * 8, c = bytes >> 4;
+            b_mn[j] = B_BASE + (g4 * 8 + kq) * Cfg::BN * ES + ((c ^ rd16_swz(g4 * 8 + kq)) << 4) + (bytes & 8);
+        }
     }
     u32x4_t fa[2][TM], fb[2][TN];  // [slice][tile]
     acc_t acc[TM][TN];
@@ -129,8 +188,25 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
     // then the right operand's
     auto read_fragment = [&](auto sl_, int r, int slot) {
         constexpr int SL = decltype(sl_)::value;
-        if (r < TM) fa[SL][r] = lds_get(smem + slot * Cfg::A_BYTES, a_frag[SL] + r * TILE_BYTES);
-        else fb[SL][r - TM] = lds_get(smem + slot * Cfg::B_BYTES, b_frag[SL] + (r - TM) * TILE_BYTES);
+        if (r < TM) {
+            const char *buf = smem + slot * Cfg::A_BYTES;
+            if constexpr (Cfg::LA == LM_K) {
+                fa[SL][r] = lds_get(buf, a_frag[SL] + r * TILE_BYTES);
+            } else {
+                const u32x2_t lo = lds_get_tr<ES>(buf, a_mn[r] + (SL * 32) * Cfg::BM * ES);
+                const u32x2_t hi = lds_get_tr<ES>(buf, a_mn[r] + (SL * 32 + 4) * Cfg::BM * ES);
+                fa[SL][r] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+            }
+        } else {
+            const char *buf = smem + slot * Cfg::B_BYTES;
+            if constexpr (Cfg::LB == LM_K) {
+                fb[SL][r - TM] = lds_get(buf, b_frag[SL] + (r - TM) * TILE_BYTES);
+            } else {
+                const u32x2_t lo = lds_get_tr<ES>(buf, b_mn[r - TM] + (SL * 32) * Cfg::BN * ES);
+                const u32x2_t hi = lds_get_tr<ES>(buf, b_mn[r - TM] + (SL * 32 + 4) * Cfg::BN * ES);
+                fb[SL][r - TM] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+            }
+        }
     };
     // One slice of work in a pinned order: the MFMAs of slice CUR with the reads of slice 1 - CUR (from ring slot
     // rd_slot) and, in slice 1 -- behind the barrier --, the DMA list between them.  A read goes behind MFMAs 1, 4, 7, ..,

@@ -17,7 +17,8 @@ namespace {
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 // KIND 0: v_mfma_f32_32x32x16_bf16; KIND 1: v_mfma_scale_f32_32x32x64_f8f6f4 on f8e4m3 with unit scales;
-// KIND 2: v_mfma_f32_16x16x32_bf16 (half the flop per instruction of KIND 0, a quarter of the accumulator registers)
+// KIND 2: v_mfma_f32_16x16x32_bf16 (half the flop per instruction of KIND 0, a quarter of the accumulator registers);
+// KIND 3: v_mfma_scale_f32_16x16x128_f8f6f4, the same relation to KIND 1
 typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
 template <int KIND>
 __global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restrict__ operands, float *__restrict__ sink,
@@ -48,6 +49,32 @@ __global__ __launch_bounds__(256) void mfma_clock_kernel(const u32x4_t *__restri
 #pragma unroll
         for (int i = 0; i < 8; i++) v += small[i][0] + small[i][1] + small[i][2] + small[i][3];
         sink[blockIdx.x * 256 + t] = v + a1.x + b1.x;
+        if (blockIdx.x == 0 && t == 0) {
+            clocks[0] = c1 - c0;
+            clocks[1] = r1 - r0;
+        }
+        return;
+    }
+    if constexpr (KIND == 3) {
+        // v_mfma_scale_f32_16x16x128_f8f6f4 on f8e4m3 with unit scales: eight accumulators, the flop per trip of KIND 1
+        f32x4_acc_t small[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) small[i] = f32x4_acc_t{0.f, 0.f, 0.f, 0.f};
+        const i32x8_t a = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+        const i32x8_t b = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+        const int unit = 0x7F7F7F7F;
+        const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]"
+                             : "+v"(small[i]) : "v"(a), "v"(b), "v"(unit));
+        }
+        const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) v += small[i][0] + small[i][1] + small[i][2] + small[i][3];
+        sink[blockIdx.x * 256 + t] = v;
         if (blockIdx.x == 0 && t == 0) {
             clocks[0] = c1 - c0;
             clocks[1] = r1 - r0;
@@ -166,7 +193,7 @@ extern "C" int hodu_rocm_debug_read_floor(hodu_rocm_ctx *ctx, const void *const 
 extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const void *operands, int iters, float *elapsed_ms,
                                           double *tflops, double *shader_mhz) {
     clear_error();
-    if (!ctx || !operands || iters <= 0 || !elapsed_ms || !tflops || !shader_mhz || kind < 0 || kind > 2)
+    if (!ctx || !operands || iters <= 0 || !elapsed_ms || !tflops || !shader_mhz || kind < 0 || kind > 3)
         return fail(HODU_ROCM_INVALID_ARG, "mfma_clock: bad argument");
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
@@ -181,6 +208,8 @@ extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const vo
     auto launch = [&](int n) {
         if (kind == 0)
             hipLaunchKernelGGL(mfma_clock_kernel<0>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
+        else if (kind == 3)
+            hipLaunchKernelGGL(mfma_clock_kernel<3>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
         else if (kind == 2)
             hipLaunchKernelGGL(mfma_clock_kernel<2>, dim3(blocks), dim3(256), 0, ctx->stream, (const u32x4_t *)operands, sink, clocks, n);
         else
@@ -206,7 +235,7 @@ extern "C" int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *ctx, int kind, const vo
     (void)hipFree(clocks);
     if (e != hipSuccess) return fail(HODU_ROCM_HIP_ERROR, "mfma_clock: %s", hipGetErrorString(e));
     // flop per trip of the loop: four 32 x 32 x k x 2 instructions with k = 16 (bf16) or 64 (f8), or eight 16 x 16 x 32 x 2
-    const double per_trip = kind == 0 ? 4 * 32768.0 : kind == 2 ? 8 * 16384.0 : 4 * 131072.0;
+    const double per_trip = kind == 0 ? 4 * 32768.0 : kind == 2 ? 8 * 16384.0 : kind == 3 ? 8 * 65536.0 : 4 * 131072.0;
     *tflops = (double)blocks * 4 /* wavefronts */ * (double)iters * per_trip / (*elapsed_ms * 1e-3) / 1e12;
     *shader_mhz = h[1] ? (double)h[0] / (double)h[1] * 100.0 : 0.0;
     return HODU_ROCM_OK;

@@ -46,7 +46,7 @@ int hodu_rocm_debug_time_product_graph(hodu_rocm_ctx *ctx, int is_matmul, int ki
 
 /* measurement hook: the rate and shader clock of a register-only MFMA loop (no LDS, no memory traffic) on
  * caller-supplied operand bits, two workgroups per compute unit.  kind 0: bf16 32x32x16; kind 1: f8e4m3 32x32x64
- * with unit scales; kind 2: bf16 16x16x32.  `operands`: 16 KB of device memory (1024 x 16 bytes: per lane the a and b fragments, twice).
+ * with unit scales; kind 2: bf16 16x16x32; kind 3: f8e4m3 16x16x128.  `operands`: 16 KB of device memory (1024 x 16 bytes: per lane the a and b fragments, twice).
  * *tflops is what the loop sustained, *shader_mhz the clock one wavefront saw (shader-clock counter over the
  * 100 MHz counter).  Under full MFMA load the clock depends on the data, so this is the ceiling a GEMM kernel can
  * approach on that data. */

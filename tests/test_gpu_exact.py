@@ -106,8 +106,8 @@ def test_f8_weight_pipelined_tiles(ctx, tile, combo):
 
 
 def test_16x16_instruction_tile_is_exact_and_equals_the_32x32_one(ctx):
-    """the 256 x 256 tile of two k-dense bf16 operands on the 16 x 16 x 32 matrix instruction (hook value 15, the default
-    for large products): exact sums on ragged shapes, a batch, and a full-size tile grid"""
+    """the 256 x 256 bf16 tile on the 16 x 16 x 32 matrix instruction (hook value 15, the default for large products;
+    right operand k-dense or row-dense): exact sums on ragged shapes, a batch, and a full-size tile grid"""
     for tile in (15, 11):
         ctx.force_tile(tile)
         try:
@@ -117,10 +117,16 @@ def test_16x16_instruction_tile_is_exact_and_equals_the_32x32_one(ctx):
             run_exact(ctx, "dot", "bf16", V([17, 192]), V([5, 192]).t(), 5, name)             # less than one fragment of rows
             run_exact(ctx, "matmul", "bf16", V([3, 160, 512]), V([3, 136, 512]).t(), 6, name)
             run_exact(ctx, "dot", "bf16", V([1024, 2048 + 64]).slice(1, 64, 2048 + 64), V([768, 2048], offset=128).t(), 7, name)
+            # the right operand row-dense ([K, N] row-major)
+            km = name.replace("_KK", "_KM")
+            run_exact(ctx, "dot", "bf16", V([296, 1024]), V([1024, 384]), 9, km)
+            run_exact(ctx, "dot", "bf16", V([520, 64]), V([64, 264]), 10, km)
+            run_exact(ctx, "matmul", "bf16", V([2, 160, 512]), V([512, 520]).broadcast_to([2, 512, 520]), 11, km)
         finally:
             ctx.force_tile(-1)
     # what the launcher picks by itself for a product that fills the chip with 256 x 256 tiles
     assert run_exact(ctx, "dot", "bf16", V([4096, 256]), V([4096, 256]).t(), 8, "mfma_bf16_pipe256x256mi16_KK")
+    assert run_exact(ctx, "dot", "bf16", V([4096, 128]), V([128, 4096]), 12, "mfma_bf16_pipe256x256mi16_KM")
 
 
 @pytest.mark.parametrize("splits", [2, 4, 7])

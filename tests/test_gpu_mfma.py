@@ -84,6 +84,17 @@ def test_pipelined_kk_16x16_instruction(ctx, kind):
         check_product(ctx, "matmul", kind, V([3, 72, 2 * K]).slice(2, K, 2 * K), V([3, 80, K], offset=64).t(), seed=7,
                       expect_kernel=f"{prefix}_pipe256x256mi16_KK")
         check_product(ctx, "dot", kind, V([1000, 1024]), V([777, 1024]).t(), seed=8, expect_kernel=f"{prefix}_pipe256x256mi16_KK")
+        # a row-dense right operand ([K, N] row-major, read through the LDS transpose): the shapes of
+        # test_pipelined_row_dense_variants
+        km = f"{prefix}_pipe256x256mi16_KM"
+        for stages in (1, 2, 3, 5):
+            K = stages * 64
+            check_product(ctx, "dot", kind, V([19 * 16 - 8, K]), V([K, 13 * 16 - 8]), seed=stages, expect_kernel=km)
+        check_product(ctx, "dot", kind, V([24, 128]), V([128, 40]), seed=9, expect_kernel=km)
+        check_product(ctx, "matmul", kind, V([3, 72, 128], offset=64), V([128, 80], offset=128).broadcast_to([3, 128, 80]), seed=10,
+                      expect_kernel=km)
+        check_product(ctx, "dot", kind, V([72, 128]), V([128, 160]).slice(1, 16, 16 + 6 * 16), seed=11, expect_kernel=km)
+        check_product(ctx, "dot", kind, V([1000, 512]), V([512, 776]), seed=12, expect_kernel=km)
     finally:
         ctx.force_tile(-1)
 
