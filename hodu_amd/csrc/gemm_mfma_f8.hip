@@ -1,6 +1,7 @@
 // f8e4m3 x f8e4m3 -> f8e4m3 and f8e5m2 x f8e5m2 -> f8e5m2 on the 8-bit matrix instruction (gemm_mfma_pipe_f8.hpp):
 // applicability and launch.
 #include "gemm_mfma_pipe_f8.hpp"
+#include "gemm_mfma_pipe_f8_16.hpp"
 namespace hodu {
 int launch_mfma_f8(hodu_rocm_ctx *ctx, int dtype, const void *a, const void *b, void *c, const DevProduct &g) {
     using namespace mfma;
@@ -20,6 +21,14 @@ int launch_mfma_f8(hodu_rocm_ctx *ctx, int dtype, const void *a, const void *b, 
     if (ctx->force_splits >= 1) splits = pick_splits(1, cus, stages, elems, ctx->force_splits);
     else if (!big) splits = pick_splits(tiles(128, 128), cus, stages, elems, -1);
     const bool e5m2 = dtype == HODU_F8E5M2;
+    // the 256 x 256 tile of an uncut product: four wavefronts on the 16 x 16 x 128 form of the instruction (hook value 15
+    // pins it, 11 the eight wavefronts on the 32 x 32 x 64 form)
+    if (big && splits == 1 && (forced < 0 || forced == 15)) {
+        ctx->last_kernel = e5m2 ? "mfma_f8e5m2_pipe256x256mi16_KK" : "mfma_f8e4m3_pipe256x256mi16_KK";
+        if (e5m2) return launch_pipe_f8x16<PipeF8x16Config<OUT_F8E5M2, 256, 256>>(ctx, a, b, c, g);
+        return launch_pipe_f8x16<PipeF8x16Config<OUT_F8E4M3, 256, 256>>(ctx, a, b, c, g);
+    }
+    if (forced == 15) return HODU_ROCM_UNSUPPORTED;
     const char *base = e5m2 ? (big ? "mfma_f8e5m2_pipe256x256_KK" : "mfma_f8e5m2_pipe128x128_KK")
                             : (big ? "mfma_f8e4m3_pipe256x256_KK" : "mfma_f8e4m3_pipe128x128_KK");
     if (splits > 1) {

@@ -212,8 +212,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
     // rd_slot) and, in slice 1 -- behind the barrier --, the DMA list between them.  A read goes behind MFMAs 1, 4, 7, ..,
     // so that the last one is out a quarter of a slice before the slice ends (in slice 0 the barrier's wait for the
     // reads follows, in slice 1 the loop's back edge, where the compiler waits for every read in flight); a DMA
-    // instruction goes behind one of the MFMAs 4, 7, 10, .. (the compiler moves a read in front of the MFMA it is
-    // grouped with, so the reads sit in the gaps behind MFMAs 0, 3, 6, .. and the DMA instructions in gaps of their own).
+    // instruction goes behind one of the MFMAs 3, 6, 9, .., never into the gap that already took a read.
     auto slice_step = [&](auto cur_, int rd_slot, int dma_src, int dma_slot) {
         constexpr int CUR = decltype(cur_)::value;
         typedef std::integral_constant<int, 1 - CUR> RS;
@@ -227,7 +226,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
             if constexpr (CUR == 1) {
 #pragma unroll
                 for (int d = 0; d < P; d++)
-                    if (3 * (1 + d * DSLOTS / P) + 1 == idx) dma_element(d, dma_src, dma_slot);
+                    if (3 * (1 + d * DSLOTS / P) == idx) dma_element(d, dma_src, dma_slot);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
