@@ -139,6 +139,14 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
             return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
         }
     }
+    if constexpr (SKA == SK_SAME && SKB == SK_F8) {
+        // f8e4m3 weights, both operands k-dense: the same tile and instruction with the widening in front of the MFMA
+        // (K a multiple of 128: the weight's lines move whole)
+        if (pipe_ok && combo == 0 && splits == 1 && g.K % 128 == 0 && ((forced < 0 && size == 0) || size == 5)) {
+            ctx->last_kernel = names[32];
+            return launch_pipe16_f8w<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_F8, 2>>(ctx, a, b, c, g);
+        }
+    }
     if (size == 5) return HODU_ROCM_UNSUPPORTED;
     if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
         // testing hook values 10..13 pin the pipelined kernel's tile, 0..3 the general kernel's

@@ -129,6 +129,21 @@ def test_16x16_instruction_tile_is_exact_and_equals_the_32x32_one(ctx):
     assert run_exact(ctx, "dot", "bf16", V([4096, 128]), V([128, 4096]), 12, "mfma_bf16_pipe256x256mi16_KM")
 
 
+def test_16x16_instruction_tile_with_f8_weights_is_exact(ctx):
+    """the same tile with f8e4m3 weights widened in front of the MFMA (pairs of stages per weight buffer): 1 to 9 pairs,
+    ragged shapes, a batch sharing the weight, and what the launcher picks for a product that fills the chip"""
+    name = "mfma_bf16_f8w_pipe256x256mi16_KK"
+    ctx.force_tile(15)
+    try:
+        for k in (128, 256, 384, 1024, 2304):
+            run_exact(ctx, "dot", "bf16_f8e4m3w", V([296, k]), V([384, k]).t(), k, name)
+        run_exact(ctx, "dot", "bf16_f8e4m3w", V([17, 256]), V([5, 256]).t(), 5, name)
+        run_exact(ctx, "matmul", "bf16_f8e4m3w", V([2, 160, 512]), V([520, 512]).t().broadcast_to([2, 512, 520]), 6, name)
+    finally:
+        ctx.force_tile(-1)
+    assert run_exact(ctx, "dot", "bf16_f8e4m3w", V([4096, 256]), V([4096, 256]).t(), 8, name)
+
+
 @pytest.mark.parametrize("splits", [2, 4, 7])
 def test_pipelined_split_k_through_the_workspace(ctx, splits):
     ctx.force_splitk(splits)

@@ -154,6 +154,24 @@ def test_pipelined_f8_weight_variants(ctx, tile, name, combo):
         ctx.force_tile(-1)
 
 
+def test_pipelined_f8_weight_16x16_instruction(ctx):
+    """fused f8e4m3 weights on the 256 x 256 tile of the 16 x 16 x 32 instruction (both operands k-dense; hook value 15, the
+    default for large products): 1, 2, 3 and 5 pairs of stages, ragged and tiny M and N, a shared weight at an offset
+    with a leading dimension larger than its extent, a full grid of tiles"""
+    kind, prefix = "bf16_f8e4m3w", KINDS["bf16_f8e4m3w"][0]
+    name = f"{prefix}_pipe256x256mi16_KK"
+    ctx.force_tile(15)
+    try:
+        for K in (128, 256, 384, 640):
+            check_product(ctx, "dot", kind, V([296, K]), V([208, K]).t(), seed=K, rscale=2.0, expect_kernel=name)
+        check_product(ctx, "dot", kind, V([24, 256]), V([48, 256]).t(), seed=9, rscale=2.0, expect_kernel=name)
+        w = V([80, 512], offset=64).slice(1, 128, 384).t().broadcast_to([3, 256, 80])
+        check_product(ctx, "matmul", kind, V([3, 72, 256]), w, seed=10, rscale=2.0, expect_kernel=name)
+        check_product(ctx, "dot", kind, V([1000, 1024]), V([777, 1024]).t(), seed=11, rscale=2.0, expect_kernel=name)
+    finally:
+        ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("kind", list(KINDS))
 def test_scalar_load_variant(ctx, kind):
     prefix, _, _ = KINDS[kind]
