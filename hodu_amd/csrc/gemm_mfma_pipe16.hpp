@@ -271,22 +271,26 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
                                                           g.M, g.N, g.epi);
 }
 
-// The same tile with f8e4m3 weights (the fused to_dtype of the right operand), both operands k-dense.  The weight's
-// bytes move as they are -- whole 128-byte lines, i.e. 128 k, the k of TWO stages of the bf16 left operand, so a
-// right-operand buffer holds a pair of stages and the ring two pairs -- and are widened to bf16 between the fragment
-// read (8 bytes per lane) and the MFMA, one fragment ahead of its use, in the shadow of the MFMAs of the fragment
-// before.  A pair's buffer is free behind the barrier of the pair's second stage and is needed four stages on, so its
-// refill goes out in two halves, behind that barrier and behind the next one: every stage issues 8 + 4 DMA instructions.
+// The same tile with f8e4m3 weights (the fused to_dtype of the right operand): the weight's bytes move as they are and
+// are widened to bf16 between the fragment read (8 bytes per lane) and the MFMA, one fragment ahead of its use, in the
+// shadow of the MFMAs of the fragment before.
+//   k-dense weights ([N, K] bytes): whole 128-byte lines, i.e. 128 k, the k of TWO stages of the bf16 left operand, so
+//     a right-operand buffer holds a pair of stages and the ring two pairs.  A pair's buffer is free behind the barrier
+//     of the pair's second stage and is needed four stages on, so its refill goes out in two halves, behind that
+//     barrier and behind the next one: every stage issues 8 + 4 DMA instructions.
+//   row-dense weights ([K, N] bytes): a stage is 64 k-rows of the tile's 256 bytes, in a ring of two like the left
+//     operand's (8 + 4 instructions per stage as well); a fragment is one 8-bit transpose read of 8 k-rows.
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                   typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                   int tiles_m, int tiles_n) {
-    static_assert(Cfg::LA == LM_K && Cfg::LB == LM_K && Cfg::B_PAIR && Cfg::NST == 2, "bf16 x f8e4m3, both k-dense, two stages");
+    static_assert(Cfg::LA == LM_K && Cfg::B_F8 && Cfg::NST == 2, "bf16 x f8e4m3, the left operand k-dense, two stages");
     extern __shared__ __align__(16) char smem[];
     typedef Compute16<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;
-    constexpr int ES = Cfg::ES, PA = Cfg::PA, PB = Cfg::PB, PBH = PB / 2, P = PA + PBH;
+    constexpr bool PAIR = Cfg::B_PAIR;  // k-dense weights
+    constexpr int ES = Cfg::ES, PA = Cfg::PA, PB = Cfg::PB, PBS = Cfg::PBS, P = PA + PBS;
     constexpr int TM = Cfg::BM / Cfg::WM / 16, TN = Cfg::BN / Cfg::WN / 16;
     constexpr int MF = TM * TN;
     static_assert(TM == 8 && TN == 8 && P <= 19, "the schedule below is written for 128 x 128 outputs per wavefront");
@@ -303,13 +307,16 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
     batch_offsets(g, batch, ao, bo);
     const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
 
-    // LDS: two stages of A (64 k of bf16 each), then two pair buffers of B (128 k of f8e4m3 each)
+    // LDS: two stages of A (64 k of bf16 each), then two buffers of B (k-dense: 128 k each; row-dense: 64 k-rows each)
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
     constexpr int B_BASE = 2 * Cfg::A_BYTES;
 
-    // DMA plan: an instruction writes 8 rows x 128 bytes; lane -> (row, slot), the slot holds chunk
+    // DMA plan.  k-dense: an instruction writes 8 rows x 128 bytes; lane -> (row, slot), the slot holds chunk
     // slot ^ ((row >> 1) & 7); rows past the operand's last one re-fetch the last one.  Address = scalar base of the
     // tile's first row (advanced 128 bytes per stage of A, per pair of B) + the lane's 32-bit offset inside the tile.
+    // row-dense weights: an instruction writes 4 k-rows of 256 bytes; lane -> (k-row, slot), the slot holds chunk
+    // slot ^ (k % 16) (a transpose read serves 32 lanes at a time, 16 k-rows of 16 bytes: the swizzle spreads them over
+    // all banks); a chunk that starts past the last column is fetched from the last whole chunk instead.
     unsigned offa[PA], offb[PB];
     unsigned lda[PA], ldb[PB];
 #pragma unroll
@@ -322,40 +329,64 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
     }
 #pragma unroll
     for (int p = 0; p < PB; p++) {
-        const int q = p * Cfg::NW + wave, trow = q * 8 + (lane >> 3);
-        int row = n0 + trow;
-        row = row < g.N ? row : g.N - 1;
-        offb[p] = (unsigned)((long)(row - n0) * g.b_n) + kd_slot(trow, lane & 7) * 16;
+        const int q = p * Cfg::NW + wave;
+        if constexpr (PAIR) {
+            const int trow = q * 8 + (lane >> 3);
+            int row = n0 + trow;
+            row = row < g.N ? row : g.N - 1;
+            offb[p] = (unsigned)((long)(row - n0) * g.b_n) + kd_slot(trow, lane & 7) * 16;
+        } else {
+            constexpr int CPR = Cfg::BN / 16, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ (k & 15);
+            int col = n0 + c * 16;
+            col = col <= g.N - 16 ? col : g.N - 16;
+            offb[p] = (unsigned)((long)k * g.b_k + (col - (n0 <= g.N - 16 ? n0 : g.N - 16)));
+        }
         ldb[p] = B_BASE + q * 1024;
     }
-    const int T = g.K * ES / P_ROW_BYTES;  // stages (even: K is a multiple of 128)
-    const int TB = T / 2;                  // pairs
+    const int T = g.K * ES / P_ROW_BYTES;  // stages (k-dense weights: even, K is a multiple of 128)
+    const int TB = PAIR ? T / 2 : T;       // right-operand buffers' worth of k
     const char *const base_a = uniform_ptr(A + (ao + (long)m0 * g.a_m) * ES);
-    const char *const base_b = uniform_ptr(B + bo + (long)n0 * g.b_n);
+    const char *const base_b = uniform_ptr(PAIR ? B + bo + (long)n0 * g.b_n : B + bo + (n0 <= g.N - 16 ? n0 : g.N - 16));
+    const long b_adv = PAIR ? P_ROW_BYTES : 64L * g.b_k;
 
     auto dma_a = [&](int e, int src, int slot) {
 #pragma unroll
         for (int p = 0; p < PA; p++)
             if (e == p) dma16_sbase(base_a + (long)src * P_ROW_BYTES, offa[p], lds0 + (unsigned)slot * Cfg::A_BYTES + lda[p]);
     };
-    // element e of half `half` of pair `pair`'s list into pair buffer `buf`
-    auto dma_b = [&](int e, int pair, int buf, int half) {
+    // element e of a stage's share of the list that fetches buffer's worth `src` of B into buffer `buf` (k-dense: half
+    // `half` of the pair's rows)
+    auto dma_b = [&](int e, int src, int buf, int half) {
 #pragma unroll
-        for (int p = 0; p < PBH; p++)
+        for (int p = 0; p < PBS; p++)
             if (e == p) {
-                const unsigned voff = half ? offb[p + PBH] : offb[p], off = half ? ldb[p + PBH] : ldb[p];
-                dma16_sbase(base_b + (long)pair * P_ROW_BYTES, voff, lds0 + (unsigned)buf * Cfg::B_BYTES + off);
+                unsigned voff = offb[p], off = ldb[p];
+                if constexpr (PAIR) {
+                    voff = half ? offb[p + PBS] : offb[p];
+                    off = half ? ldb[p + PBS] : ldb[p];
+                }
+                dma16_sbase(base_b + src * b_adv, voff, lds0 + (unsigned)buf * Cfg::B_BYTES + off);
             }
     };
 
-    // fragment addresses.  A: lane (r16, g4) reads chunk 4 * slice + g4 of row r16 (16 bytes).  B: the lane's 8 k are
-    // 8 bytes: half g4 % 2 of chunk 4 * (stage % 2) + 2 * slice + g4 / 2 of the row's 128-byte line; slice and stage
-    // flip bits 5 and 6 of the byte offset (the swizzle is an XOR on the chunk index).
+    // fragment addresses.  A: lane (r16, g4) reads chunk 4 * slice + g4 of row r16 (16 bytes).  B k-dense: the lane's
+    // 8 k are 8 bytes: half g4 % 2 of chunk 4 * (stage % 2) + 2 * slice + g4 / 2 of the row's 128-byte line; slice and
+    // stage flip bits 5 and 6 of the byte offset (the swizzle is an XOR on the chunk index).  B row-dense: the 16 lanes
+    // of group g4 take their 8 k of column r16 out of k-rows 32 * slice + 8 * g4 .. + 7 through one transpose read, for
+    // which lane s of the 16 supplies the address of 8 columns of k-row (that start) + s / 2; k % 16 is
+    // 8 * (g4 % 2) + s / 2 whatever the slice, so the swizzle is the lane's own and slices are immediates; tiles are not.
     constexpr int TILE_BYTES = 16 * P_ROW_BYTES;
     int a_frag[2];
 #pragma unroll
     for (int sl = 0; sl < 2; sl++) a_frag[sl] = (wave_m * TM) * TILE_BYTES + r16 * P_ROW_BYTES + (kd_slot(r16, 4 * sl + g4) << 4);
     const int b_frag = B_BASE + (wave_n * TN) * TILE_BYTES + r16 * P_ROW_BYTES + (kd_slot(r16, g4 >> 1) << 4) + (g4 & 1) * 8;
+    int b_mn[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int kq = r16 >> 1, bytes = (wave_n * TN + j) * 16 + (r16 & 1) * 8, c = bytes >> 4, k = 8 * g4 + kq;
+        b_mn[j] = B_BASE + k * Cfg::BN + ((c ^ (k & 15)) << 4) + (bytes & 8);
+    }
 
     u32x4_t fa[2][TM];
     u32x2_t fb[2][TN];  // raw bytes
@@ -365,21 +396,23 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
 #pragma unroll
         for (int j = 0; j < TN; j++) acc[i][j] = acc_t{0.f, 0.f, 0.f, 0.f};
 
-    // the r-th fragment read of slice SL of stage `st` (A from ring slot a_slot): the left operand's tiles, then the right's
-    auto read_fragment = [&](auto sl_, int r, int a_slot, int st) {
+    // the r-th fragment read of slice SL of stage `st` (ring slot st % 2): the left operand's tiles, then the right's
+    auto read_fragment = [&](auto sl_, int r, int st) {
         constexpr int SL = decltype(sl_)::value;
         if (r < TM) {
-            fa[SL][r] = lds_get(smem + a_slot * Cfg::A_BYTES, a_frag[SL] + r * TILE_BYTES);
-        } else {
+            fa[SL][r] = lds_get(smem + (st & 1) * Cfg::A_BYTES, a_frag[SL] + r * TILE_BYTES);
+        } else if constexpr (PAIR) {
             const int at = (b_frag ^ (SL << 5) ^ ((st & 1) << 6)) + (r - TM) * TILE_BYTES;
             fb[SL][r - TM] = lds_get64(smem + ((st >> 1) & 1) * Cfg::B_BYTES, at);
+        } else {
+            fb[SL][r - TM] = lds_get_tr<1>(smem + (st & 1) * Cfg::B_BYTES, b_mn[r - TM] + SL * 32 * Cfg::BN);
         }
     };
     u32x4_t bwide = u32x4_t{0u, 0u, 0u, 0u};  // the widened first right fragment of the next slice
     // One slice in a pinned order, as in mfma_pipe16_kernel: a read behind MFMAs 1, 4, 7, .., in slice 1 a DMA instruction
     // behind MFMAs 3, 6, 9, ..; the right fragment of the next group of TM MFMAs is widened behind the first MFMA of
     // the current group, the first fragment of the next slice behind this slice's last MFMA.
-    auto slice_step = [&](auto cur_, int rd_slot, int rd_stage, int a_src, int a_slot, int b_pair, int b_buf, int b_half) {
+    auto slice_step = [&](auto cur_, int rd_stage, int a_src, int a_slot, int b_src, int b_buf, int b_half) {
         constexpr int CUR = decltype(cur_)::value;
         typedef std::integral_constant<int, 1 - CUR> RS;
         constexpr int DSLOTS = (MF - 4) / 3;
@@ -390,13 +423,13 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
             if (idx % TM == 0 && idx > 0) bcur = bnext;
             Cmp::mma(bcur, fa[CUR][idx % TM], acc[idx % TM][idx / TM]);
             if (idx % TM == 0 && idx / TM + 1 < TN) bnext = widen_f8x8(fb[CUR][idx / TM + 1]);
-            if (idx % 3 == 1 && idx / 3 < TM + TN) read_fragment(RS{}, idx / 3, rd_slot, rd_stage);
+            if (idx % 3 == 1 && idx / 3 < TM + TN) read_fragment(RS{}, idx / 3, rd_stage);
             if constexpr (CUR == 1) {
 #pragma unroll
                 for (int d = 0; d < P; d++)
                     if (3 * (1 + d * DSLOTS / P) == idx) {
                         if (d < PA) dma_a(d, a_src, a_slot);
-                        else dma_b(d - PA, b_pair, b_buf, b_half);
+                        else dma_b(d - PA, b_src, b_buf, b_half);
                     }
             }
             if (idx == MF - 1) bwide = widen_f8x8(fb[1 - CUR][0]);
@@ -406,38 +439,43 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, 1> I1;
 
-    // prologue: stage 0 of A and pair 0 of B, then stage 1 of A and the first half of pair 1 (clamped)
+    // prologue: stage 0 of A and buffer 0 of B, then stage 1 of A and (k-dense: the first half of) buffer 1 of B (clamped)
 #pragma unroll
     for (int e = 0; e < PA; e++) dma_a(e, 0, 0);
 #pragma unroll
-    for (int e = 0; e < PBH; e++) dma_b(e, 0, 0, 0);
+    for (int e = 0; e < PBS; e++) dma_b(e, 0, 0, 0);
+    if constexpr (PAIR) {
 #pragma unroll
-    for (int e = 0; e < PBH; e++) dma_b(e, 0, 0, 1);
+        for (int e = 0; e < PBS; e++) dma_b(e, 0, 0, 1);
+    }
 #pragma unroll
     for (int e = 0; e < PA; e++) dma_a(e, 1 < T ? 1 : T - 1, 1);
 #pragma unroll
-    for (int e = 0; e < PBH; e++) dma_b(e, 1 < TB ? 1 : TB - 1, 1, 0);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA + PBH));  // stage 0 and pair 0 have landed
+    for (int e = 0; e < PBS; e++) dma_b(e, 1 < TB ? 1 : TB - 1, 1, 0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA + PBS));  // stage 0 and buffer 0 have landed
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < TM + TN; r++) read_fragment(I0{}, r, 0, 0);
+    for (int r = 0; r < TM + TN; r++) read_fragment(I0{}, r, 0);
     bwide = widen_f8x8(fb[0][0]);
 
-    // Past the last stage the reads fetch LDS bytes nobody uses and the lists re-fetch the last stage and pair into
+    // Past the last stage the reads fetch LDS bytes nobody uses and the lists re-fetch the last stage (pair) into
     // buffers nobody reads: harmless, and the number of instructions in flight stays what the waits assume.
-    int slot = 0;
     for (int t = 0; t < T; t++) {
-        slice_step(I0{}, slot, t, 0, 0, 0, 0, 0);
-        // stage t + 1 and its pair have landed and every read of stage t has returned
+        slice_step(I0{}, t, 0, 0, 0, 0, 0);
+        // stage t + 1 (and its pair) has landed and every read of stage t has returned
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        // A: stage t + 2 into the slot of stage t.  B: odd t has just finished pair t / 2 and sends the first half of
-        // pair t / 2 + 2 into its buffer; the next (even) stage sends the second half of that pair
-        const int pair = (t & 1) ? (t + 3) >> 1 : (t + 2) >> 1;
-        slice_step(I1{}, slot ^ 1, t + 1, t + 2 < T ? t + 2 : T - 1, slot, pair < TB ? pair : TB - 1, pair & 1, (t & 1) ? 0 : 1);
-        slot ^= 1;
+        // A: stage t + 2 into the slot of stage t.  B row-dense: likewise.  B k-dense: odd t has just finished pair
+        // t / 2 and sends the first half of pair t / 2 + 2 into its buffer; the next (even) stage sends the second half
+        const int a_src = t + 2 < T ? t + 2 : T - 1;
+        if constexpr (PAIR) {
+            const int pair = (t & 1) ? (t + 3) >> 1 : (t + 2) >> 1;
+            slice_step(I1{}, t + 1, a_src, t & 1, pair < TB ? pair : TB - 1, pair & 1, (t & 1) ? 0 : 1);
+        } else {
+            slice_step(I1{}, t + 1, a_src, t & 1, a_src, t & 1, 0);
+        }
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the re-fetches of the last stages are still writing LDS
     __syncthreads();
@@ -457,7 +495,7 @@ template <class Cfg> int launch_pipe16_f8w(hodu_rocm_ctx *ctx, const void *a, co
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
     const long total = g.batches * tiles_m * tiles_n;
     if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);
-    if (g.K <= 0 || g.K % 128 != 0) return fail(HODU_ROCM_UNSUPPORTED, "K is not a whole number of 128-byte weight lines");
+    if (g.K <= 0 || g.K % (Cfg::B_PAIR ? 128 : 64) != 0) return fail(HODU_ROCM_UNSUPPORTED, "K is not a whole number of stages");
     hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a, (const char *)b,
                        (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n);
     HODU_HIP(hipGetLastError());

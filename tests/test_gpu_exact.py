@@ -139,9 +139,14 @@ def test_16x16_instruction_tile_with_f8_weights_is_exact(ctx):
             run_exact(ctx, "dot", "bf16_f8e4m3w", V([296, k]), V([384, k]).t(), k, name)
         run_exact(ctx, "dot", "bf16_f8e4m3w", V([17, 256]), V([5, 256]).t(), 5, name)
         run_exact(ctx, "matmul", "bf16_f8e4m3w", V([2, 160, 512]), V([520, 512]).t().broadcast_to([2, 512, 520]), 6, name)
+        km = name.replace("_KK", "_KM")  # row-dense weights
+        for k in (64, 192, 1024):
+            run_exact(ctx, "dot", "bf16_f8e4m3w", V([296, k]), V([k, 384]), k + 1, km)
+        run_exact(ctx, "matmul", "bf16_f8e4m3w", V([2, 160, 512]), V([512, 528]).broadcast_to([2, 512, 528]), 7, km)
     finally:
         ctx.force_tile(-1)
     assert run_exact(ctx, "dot", "bf16_f8e4m3w", V([4096, 256]), V([4096, 256]).t(), 8, name)
+    assert run_exact(ctx, "dot", "bf16_f8e4m3w", V([4096, 128]), V([128, 4096]), 9, name.replace("_KK", "_KM"))
 
 
 @pytest.mark.parametrize("splits", [2, 4, 7])

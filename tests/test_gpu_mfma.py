@@ -155,8 +155,8 @@ def test_pipelined_f8_weight_variants(ctx, tile, name, combo):
 
 
 def test_pipelined_f8_weight_16x16_instruction(ctx):
-    """fused f8e4m3 weights on the 256 x 256 tile of the 16 x 16 x 32 instruction (both operands k-dense; hook value 15, the
-    default for large products): 1, 2, 3 and 5 pairs of stages, ragged and tiny M and N, a shared weight at an offset
+    """fused f8e4m3 weights on the 256 x 256 tile of the 16 x 16 x 32 instruction (hook value 15, the default for large
+    products): 1, 2, 3 and 5 pairs of stages, ragged and tiny M and N, a shared weight at an offset
     with a leading dimension larger than its extent, a full grid of tiles"""
     kind, prefix = "bf16_f8e4m3w", KINDS["bf16_f8e4m3w"][0]
     name = f"{prefix}_pipe256x256mi16_KK"
@@ -168,6 +168,14 @@ def test_pipelined_f8_weight_16x16_instruction(ctx):
         w = V([80, 512], offset=64).slice(1, 128, 384).t().broadcast_to([3, 256, 80])
         check_product(ctx, "matmul", kind, V([3, 72, 256]), w, seed=10, rscale=2.0, expect_kernel=name)
         check_product(ctx, "dot", kind, V([1000, 1024]), V([777, 1024]).t(), seed=11, rscale=2.0, expect_kernel=name)
+        # row-dense weights ([K, N] bytes, read through the 8-bit LDS transpose): odd and even stage counts
+        km = f"{prefix}_pipe256x256mi16_KM"
+        for K in (64, 128, 192, 320):
+            check_product(ctx, "dot", kind, V([296, K]), V([K, 208]), seed=K, rscale=2.0, expect_kernel=km)
+        check_product(ctx, "dot", kind, V([24, 256]), V([256, 48]), seed=12, rscale=2.0, expect_kernel=km)
+        w = V([256, 160], offset=32).slice(1, 16, 112).broadcast_to([3, 256, 96])
+        check_product(ctx, "matmul", kind, V([3, 72, 256]), w, seed=13, rscale=2.0, expect_kernel=km)
+        check_product(ctx, "dot", kind, V([1000, 512]), V([512, 784]), seed=14, rscale=2.0, expect_kernel=km)
     finally:
         ctx.force_tile(-1)
 
