@@ -133,7 +133,11 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
         // leaves the power-limited part a higher clock than the 32 x 32 x 16 one (hook value 15 pins it, 11 the other)
         // (a k-dense left operand: with a row-dense one the per-tile fragment addresses no longer fit beside 128
         // fragment registers, and the compiler spills inside the loop)
-        if (pipe_ok && combo <= 1 && splits == 1 && ((forced < 0 && size == 1) || size == 5)) {
+        // (with element-wise steps on the store, which four wavefronts take 5 us longer over than eight, from 64 stages
+        // on: config 5 up with bias and ReLU 408 against 420 us, config 2 with the attention scale -- 16 stages -- 43
+        // against 38)
+        const bool fused_long = size == 0 && g.epi.n != 0 && stages >= 64;
+        if (pipe_ok && combo <= 1 && splits == 1 && ((forced < 0 && (size == 1 || fused_long)) || size == 5)) {
             ctx->last_kernel = names[32 + combo];
             if (combo == 0) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
             return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
