@@ -633,12 +633,14 @@ def read_floor_probe(ctx):
 
 def mfma_clock_probe(ctx):
     """what the matrix cores sustain from registers (no LDS, no memory traffic), and at which shader clock, on
-    constant and on N(0,1) operands: the clock under full MFMA load depends on the data"""
+    constant and on N(0,1) operands, for both shapes of the bf16 and of the f8 instruction: the clock under full MFMA
+    load depends on the data and on the instruction's shape"""
     import helpers as H
     out = []
-    for kind, name, peak in ((0, "bf16 32x32x16", PEAK["bf16"]), (1, "f8e4m3 32x32x64 (unit scales)", PEAK["fp8"])):
+    for kind, name, peak in ((0, "bf16 32x32x16", PEAK["bf16"]), (2, "bf16 16x16x32", PEAK["bf16"]),
+                             (1, "f8e4m3 32x32x64 (unit scales)", PEAK["fp8"]), (3, "f8e4m3 16x16x128 (unit scales)", PEAK["fp8"])):
         for data in ("constant", "normal"):
-            if kind == 0:
+            if kind in (0, 2):
                 bits = bf16(np.full(8192, 0.0111, dtype=np.float32) if data == "constant" else normal(900, 8192))
             else:
                 vals = np.full(16384, 0.5, dtype=np.float32) if data == "constant" else normal(901, 16384)

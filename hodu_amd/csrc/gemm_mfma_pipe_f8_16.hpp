@@ -109,12 +109,15 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8x16_kernel(const char *__
             if (e == PA + p) dma16_sbase(base_b + (long)src * P_ROW_BYTES, offb[p], lds0 + (unsigned)slot * Cfg::B_BYTES + ldb[p]);
     };
 
-    // fragment addresses: lane (r16, g4) reads bytes 32 * g4 .. + 31 of row r16 of a 16-row tile = chunks 2 * g4 and
-    // 2 * g4 + 1; tiles start on multiples of 16 rows, so the swizzle term is the lane's own and tiles are immediates
+    // fragment addresses: the instruction wants 32 k per lane, the same 32 in both operands -- which 32 is free, the
+    // sum runs over all 128 either way.  Lane (r16, g4) takes chunks g4 and g4 + 4 of row r16 of a 16-row tile: each of
+    // the two reads then has the four lane groups on four neighbouring chunks, the pattern of the 16-bit kernel's
+    // reads (with chunks 2 * g4 and 2 * g4 + 1 the counters showed every read conflicting two ways).  Tiles start on
+    // multiples of 16 rows, so the swizzle term is the lane's own and tiles are immediates.
     int a_fr[2], b_fr[2];
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        const int at = r16 * P_ROW_BYTES + (kd_slot(r16, 2 * g4 + h) << 4);
+        const int at = r16 * P_ROW_BYTES + (kd_slot(r16, g4 + 4 * h) << 4);
         a_fr[h] = (wave_m * TM) * TILE_BYTES + at;
         b_fr[h] = B_BASE + (wave_n * TN) * TILE_BYTES + at;
     }
