@@ -159,11 +159,12 @@ template <int SB> __device__ __forceinline__ u32x2_t lds_get_tr(const char *lds,
 }
 __device__ __forceinline__ u32x2_t lds_get64(const char *lds, int off) { return *reinterpret_cast<const u32x2_t *>(lds + off); }
 
-// 8 f8e4m3 -> 8 bf16 (exact)
+// 8 f8e4m3 -> 8 bf16 (exact), two per instruction (v_cvt_scalef32_pk_bf16_fp8 with a unit scale)
 __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
-
-    return u32x4_t{f8pair_to_bf16pair(v.x, false), f8pair_to_bf16pair(v.x, true), f8pair_to_bf16pair(v.y, false),
-                   f8pair_to_bf16pair(v.y, true)};
+    return u32x4_t{bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, false)),
+                   bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, true)),
+                   bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, false)),
+                   bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, true))};
 }
 
 // Epilogue for one band of a wavefront's tile (TN accumulator tiles side by side; 32 rows, or 16 with TS = 16): the values go through a

@@ -271,14 +271,6 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
                                                           g.M, g.N, g.epi);
 }
 
-// 8 f8e4m3 -> 8 bf16 (exact), two per instruction
-__device__ __forceinline__ u32x4_t widen16_f8x8(const u32x2_t &v) {
-    return u32x4_t{bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, false)),
-                   bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, true)),
-                   bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, false)),
-                   bitcast<uint32_t>(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, true))};
-}
-
 // The same tile with f8e4m3 weights (the fused to_dtype of the right operand): the weight's bytes move as they are and
 // are widened to bf16 between the fragment read (8 bytes per lane) and the MFMA, one fragment ahead of its use, in the
 // shadow of the MFMAs of the fragment before.
@@ -430,7 +422,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
         for (int idx = 0; idx < MF; idx++) {
             if (idx % TM == 0 && idx > 0) bcur = bnext;
             Cmp::mma(bcur, fa[CUR][idx % TM], acc[idx % TM][idx / TM]);
-            if (idx % TM == 0 && idx / TM + 1 < TN) bnext = widen16_f8x8(fb[CUR][idx / TM + 1]);
+            if (idx % TM == 0 && idx / TM + 1 < TN) bnext = widen_f8x8(fb[CUR][idx / TM + 1]);
             if (idx % 3 == 1 && idx / 3 < TM + TN) read_fragment(RS{}, idx / 3, rd_stage);
             if constexpr (CUR == 1) {
 #pragma unroll
@@ -440,7 +432,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
                         else dma_b(d - PA, b_src, b_buf, b_half);
                     }
             }
-            if (idx == MF - 1) bwide = widen16_f8x8(fb[1 - CUR][0]);
+            if (idx == MF - 1) bwide = widen_f8x8(fb[1 - CUR][0]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -465,7 +457,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int r = 0; r < TM + TN; r++) read_fragment(I0{}, r, 0);
-    bwide = widen16_f8x8(fb[0][0]);
+    bwide = widen_f8x8(fb[0][0]);
 
     // Past the last stage the reads fetch LDS bytes nobody uses and the lists re-fetch the last stage (pair) into
     // buffers nobody reads: harmless, and the number of instructions in flight stays what the waits assume.
