@@ -410,19 +410,31 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
     };
     u32x4_t bwide = u32x4_t{0u, 0u, 0u, 0u};  // the widened first right fragment of the next slice
     // One slice in a pinned order, as in mfma_pipe16_kernel: a read behind MFMAs 1, 4, 7, .., in slice 1 a DMA instruction
-    // behind MFMAs 3, 6, 9, ..; the right fragment of the next group of TM MFMAs is widened behind the first MFMA of
-    // the current group, the first fragment of the next slice behind this slice's last MFMA.
+    // behind MFMAs 3, 6, 9, ..; the right fragment of the next group of TM MFMAs is widened behind the first four
+    // MFMAs of the current group, the first fragment of the next slice behind this slice's last four.
     auto slice_step = [&](auto cur_, int rd_stage, int a_src, int a_slot, int b_src, int b_buf, int b_half) {
         constexpr int CUR = decltype(cur_)::value;
         typedef std::integral_constant<int, 1 - CUR> RS;
         constexpr int DSLOTS = (MF - 4) / 3;
         static_assert(DSLOTS >= P, "a gap of its own for every DMA instruction");
         u32x4_t bcur = bwide, bnext = bcur;
+        // one conversion (two values) behind each of the first four MFMAs of a group: four in a row take longer to
+        // issue than the MFMA in front of them runs
+        auto widen_part = [&](u32x4_t &dst, const u32x2_t &raw, int part) {
+            const uint32_t w = part < 2 ? raw.x : raw.y;
+            const uint32_t v = bitcast<uint32_t>(part & 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                                                          : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+            if (part == 0) dst.x = v;
+            else if (part == 1) dst.y = v;
+            else if (part == 2) dst.z = v;
+            else dst.w = v;
+        };
 #pragma unroll
         for (int idx = 0; idx < MF; idx++) {
             if (idx % TM == 0 && idx > 0) bcur = bnext;
             Cmp::mma(bcur, fa[CUR][idx % TM], acc[idx % TM][idx / TM]);
-            if (idx % TM == 0 && idx / TM + 1 < TN) bnext = widen_f8x8(fb[CUR][idx / TM + 1]);
+            if (idx % TM < 4 && idx / TM + 1 < TN) widen_part(bnext, fb[CUR][idx / TM + 1], idx % TM);
+            if (idx >= MF - 4) widen_part(bwide, fb[1 - CUR][0], idx - (MF - 4));
             if (idx % 3 == 1 && idx / 3 < TM + TN) read_fragment(RS{}, idx / 3, rd_stage);
             if constexpr (CUR == 1) {
 #pragma unroll
@@ -432,7 +444,6 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
                         else dma_b(d - PA, b_src, b_buf, b_half);
                     }
             }
-            if (idx == MF - 1) bwide = widen_f8x8(fb[1 - CUR][0]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
