@@ -15,7 +15,7 @@ namespace mfma {
 // type -- the software-pipelined kernels of gemm_mfma_pipe.hpp: KK at four tile shapes and, for the
 // 16-bit types, KM / MK / MM at the three larger ones.  The tile is the largest that still yields at
 // least one workgroup per compute unit.
-constexpr int kVariants = 34;
+constexpr int kVariants = 36;
 template <int CK, int SKA, int SKB, int OUT>
 int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g,
                 const char *const names[kVariants]) {
@@ -131,16 +131,16 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     if constexpr (SKA == SK_SAME && SKB == SK_SAME && ES == 2 && CK != CK_I8) {
         // 16-bit operands on the 256 x 256 tile of four wavefronts: the 16 x 16 x 32 instruction, which
         // leaves the power-limited part a higher clock than the 32 x 32 x 16 one (hook value 15 pins it, 11 the other)
-        // (a k-dense left operand: with a row-dense one the per-tile fragment addresses no longer fit beside 128
-        // fragment registers, and the compiler spills inside the loop)
         // (with element-wise steps on the store, which four wavefronts take 5 us longer over than eight, from 64 stages
         // on: config 5 up with bias and ReLU 408 against 420 us, config 2 with the attention scale -- 16 stages -- 43
         // against 38)
         const bool fused_long = size == 0 && g.epi.n != 0 && stages >= 64;
-        if (pipe_ok && combo <= 1 && splits == 1 && ((forced < 0 && (size == 1 || fused_long)) || size == 5)) {
+        if (pipe_ok && splits == 1 && ((forced < 0 && (size == 1 || fused_long)) || size == 5)) {
             ctx->last_kernel = names[32 + combo];
             if (combo == 0) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
-            return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
+            if (combo == 1) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
+            if (combo == 2) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_MN, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
+            return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_MN, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
         }
     }
     if constexpr (SKA == SK_SAME && SKB == SK_F8) {
@@ -249,7 +249,8 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
      P "_pipe256x256w8_KM", P "_pipe256x256_KM", P "_pipe128x128_KM",                                              \
      P "_pipe256x256w8_MK", P "_pipe256x256_MK", P "_pipe128x128_MK",                                              \
      P "_pipe256x256w8_MM", P "_pipe256x256_MM", P "_pipe128x128_MM",                                              \
-     P "_pipe256x128_KK", P "_pipe256x128_KM", P "_pipe256x256mi16_KK", P "_pipe256x256mi16_KM"}
+     P "_pipe256x128_KK", P "_pipe256x128_KM", P "_pipe256x256mi16_KK", P "_pipe256x256mi16_KM",                \
+     P "_pipe256x256mi16_MK", P "_pipe256x256mi16_MM"}
 
 }  // namespace mfma
 }  // namespace hodu

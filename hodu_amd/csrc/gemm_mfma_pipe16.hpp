@@ -58,7 +58,6 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
                                                               typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                               int tiles_m, int tiles_n) {
     static_assert(!Cfg::B_F8 && Cfg::ES == 2 && Cfg::NST == 2, "16-bit operands stored in the compute type, two stages");
-    // (a row-dense left operand compiles, but with register spills inside the loop: the launcher does not use it)
     typedef RowDenseGeom<Cfg::ES, Cfg::ES> G;
     extern __shared__ __align__(16) char smem[];
     typedef Compute16<Cfg::CK> Cmp;

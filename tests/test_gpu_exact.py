@@ -122,6 +122,9 @@ def test_16x16_instruction_tile_is_exact_and_equals_the_32x32_one(ctx):
             run_exact(ctx, "dot", "bf16", V([296, 1024]), V([1024, 384]), 9, km)
             run_exact(ctx, "dot", "bf16", V([520, 64]), V([64, 264]), 10, km)
             run_exact(ctx, "matmul", "bf16", V([2, 160, 512]), V([512, 520]).broadcast_to([2, 512, 520]), 11, km)
+            # the left operand row-dense (a transposed view)
+            run_exact(ctx, "dot", "bf16", V([1024, 296]).t(), V([384, 1024]).t(), 13, name.replace("_KK", "_MK"))
+            run_exact(ctx, "dot", "bf16", V([192, 520]).t(), V([192, 264]), 14, name.replace("_KK", "_MM"))
         finally:
             ctx.force_tile(-1)
     # what the launcher picks by itself for a product that fills the chip with 256 x 256 tiles

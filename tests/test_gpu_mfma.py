@@ -95,6 +95,16 @@ def test_pipelined_kk_16x16_instruction(ctx, kind):
                       expect_kernel=km)
         check_product(ctx, "dot", kind, V([72, 128]), V([128, 160]).slice(1, 16, 16 + 6 * 16), seed=11, expect_kernel=km)
         check_product(ctx, "dot", kind, V([1000, 512]), V([512, 776]), seed=12, expect_kernel=km)
+        # a row-dense left operand (a transposed view), against both kinds of right operand
+        for combo in ("MK", "MM"):
+            name = f"{prefix}_pipe256x256mi16_{combo}"
+            for stages in (1, 2, 3, 5):
+                lv, rv = views(combo, 19 * 16 - 8, stages * 64, 13 * 16 - 8)
+                check_product(ctx, "dot", kind, lv, rv, seed=stages, expect_kernel=name)
+            lv, rv = views(combo, 24, 128, 40)
+            check_product(ctx, "dot", kind, lv, rv, seed=9, expect_kernel=name)
+            lv, rv = views(combo, 1000, 512, 776)
+            check_product(ctx, "dot", kind, lv, rv, seed=13, expect_kernel=name)
     finally:
         ctx.force_tile(-1)
 
