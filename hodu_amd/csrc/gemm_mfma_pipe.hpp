@@ -175,9 +175,22 @@ __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
 // EPI: the values are final outputs and take the fused element-wise steps (partial sums of a K range do not).
 // TS = 16: bands of 16 rows out of 16 x 16 accumulators, where lane (r = lane % 16, g = lane / 16) holds row r,
 // columns 16*j + 4*g + e.
-template <int OUT, int TN, bool EPI, class acc_t, int TS = 32>
+// What the fused steps need for the columns a lane stores in a band of TN tiles of TS columns (the same columns in
+// every pass of every band of a wavefront's tile): fetched once per tile by the caller and handed to every band --
+// fetched per band, a bias vector's entries cost a trip to memory eight times per tile (config 5 up with bias and
+// ReLU: 46 us more than the plain product; once per tile: 28).
+template <int OUT, int TN, int TS>
+__device__ __forceinline__ EpiPrepared<Out<OUT>::DT, 16 / (int)sizeof(typename Out<OUT>::T)> band_columns_prepare(const DevEpilogue &epi, int n_base,
+                                                                                                                  int lane, int N) {
+    constexpr int OS = sizeof(typename Out<OUT>::T), EPV = 16 / OS, CPR = TN * TS * OS / 16;
+    const int n = n_base + (lane % CPR) * EPV;
+    return epilogue_prepare<Out<OUT>::DT, EPV>(epi, n < N ? n : N - 1, N);
+}
+
+template <int OUT, int TN, bool EPI, class acc_t, int TS = 32, bool READY = false>
 __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,
-                                                   int n_base, int lane, int M, int N, const DevEpilogue &epi) {
+                                                   int n_base, int lane, int M, int N, const DevEpilogue &epi,
+                                                   const EpiPrepared<Out<OUT>::DT, 16 / (int)sizeof(typename Out<OUT>::T)> &ready) {
     typedef typename Out<OUT>::T out_t;
     constexpr int OS = sizeof(out_t), ROWB = TN * TS * OS, PITCH = ROWB + 16, EPV = 16 / OS;
     constexpr int CPR = ROWB / 16, RPP = 64 / CPR;  // 16-byte chunks per row, rows per pass of the wavefront
@@ -212,8 +225,12 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
     // of one row -- the same columns in every pass, so what the steps need for them is fetched once
     EpiPrepared<Out<OUT>::DT, EPV> prepared;
     if (EPI && epi.n != 0) {
-        const int n = n_base + (lane % CPR) * EPV;
-        prepared = epilogue_prepare<Out<OUT>::DT, EPV>(epi, n < N ? n : N - 1, N);
+        if constexpr (READY) {
+            prepared = ready;
+        } else {
+            const int n = n_base + (lane % CPR) * EPV;
+            prepared = epilogue_prepare<Out<OUT>::DT, EPV>(epi, n < N ? n : N - 1, N);
+        }
     }
     auto row_chunk = [&](int pass, auto fused) {
         const int row = pass * RPP + lane / CPR, chunk = lane % CPR;
@@ -248,6 +265,12 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
         for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::false_type{});
     }
     asm volatile("" ::: "memory");  // the next band overwrites the patch
+}
+template <int OUT, int TN, bool EPI, class acc_t, int TS = 32>
+__device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,
+                                                   int n_base, int lane, int M, int N, const DevEpilogue &epi) {
+    const EpiPrepared<Out<OUT>::DT, 16 / (int)sizeof(typename Out<OUT>::T)> none{};
+    store_band_via_lds<OUT, TN, EPI, acc_t, TS, false>(patch, Cb, acc, m_base, n_base, lane, M, N, epi, none);
 }
 
 // A product cut along K (grid.y ranges): every workgroup of a tile writes its accumulators, unrounded, to its own
@@ -701,9 +724,12 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
         return;
     }
     Cb = C + batch * (long)g.M * g.N;
+    EpiPrepared<Out<Cfg::OUT>::DT, 16 / (int)sizeof(out_t)> steps{};
+    if (g.epi.n != 0) steps = band_columns_prepare<Cfg::OUT, TN, 32>(g.epi, n0 + wave_n * TN * 32, lane, g.N);
 #pragma unroll
     for (int i = 0; i < TM; i++)
-        store_band_via_lds<Cfg::OUT, TN, true>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M, g.N, g.epi);
+        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 32, true>(patch, Cb, acc[i], m0 + wave_m * TM * 32 + i * 32, n0 + wave_n * TN * 32, lane, g.M,
+                                                                g.N, g.epi, steps);
     HODU_STAMP(5);
 }
 

@@ -264,10 +264,12 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
     // epilogue: bands of 16 rows through a wavefront-private patch of LDS
     char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));
     out_t *Cb = C + batch * (long)g.M * g.N;
+    EpiPrepared<Out<Cfg::OUT>::DT, 16 / (int)sizeof(out_t)> steps{};
+    if (g.epi.n != 0) steps = band_columns_prepare<Cfg::OUT, TN, 16>(g.epi, n0 + wave_n * TN * 16, lane, g.N);
 #pragma unroll
     for (int i = 0; i < TM; i++)
-        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
-                                                          g.M, g.N, g.epi);
+        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16, true>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
+                                                                g.M, g.N, g.epi, steps);
 }
 
 // The same tile with f8e4m3 weights (the fused to_dtype of the right operand): the weight's bytes move as they are and
@@ -492,10 +494,12 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
 
     char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));
     out_t *Cb = C + batch * (long)g.M * g.N;
+    EpiPrepared<Out<Cfg::OUT>::DT, 16 / (int)sizeof(out_t)> steps{};
+    if (g.epi.n != 0) steps = band_columns_prepare<Cfg::OUT, TN, 16>(g.epi, n0 + wave_n * TN * 16, lane, g.N);
 #pragma unroll
     for (int i = 0; i < TM; i++)
-        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
-                                                          g.M, g.N, g.epi);
+        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16, true>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
+                                                                g.M, g.N, g.epi, steps);
 }
 
 template <class Cfg> int launch_pipe16_f8w(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
