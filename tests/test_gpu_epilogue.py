@@ -145,6 +145,28 @@ def test_pipelined_kernels(ctx, name, tile):
         ctx.force_tile(-1)
 
 
+@pytest.mark.parametrize("name", ["bf16", "f16", "bf16_f8e4m3w"])
+def test_16x16_instruction_tiles(ctx, name):
+    """the 256 x 256 tile on the 16 x 16 x 32 instruction (bands of 16 rows leave through LDS; the steps' column data is
+    fetched once per tile): every step combination, N ragged against the 16-byte store, row-dense operands, batches"""
+    ctx.force_tile(15)
+    try:
+        rs = 2.0 if "f8" in name else None
+        for n, spec in enumerate(SPECS):
+            check_fused(ctx, "dot", name, V([150, 512]), V([133, 512]).t(), spec, seed=n, rscale=rs, expect_kernel="mfma_")
+            assert "mi16_KK" in ctx.last_kernel(), ctx.last_kernel()
+        n_km = 528 if "f8" in name else 520  # (row-dense f8e4m3 weights move in 16-byte chunks: N a multiple of 16)
+        check_fused(ctx, "dot", name, V([300, 256]), V([256, n_km]), [("mul",), ("add", 2, 3), ("relu",)], seed=8, rscale=rs)
+        assert "mi16_KM" in ctx.last_kernel(), ctx.last_kernel()
+        check_fused(ctx, "matmul", name, V([3, 70, 512]), V([3, 72, 512]).t(), [("mul",), ("add", 1, 1)], seed=7, rscale=rs)
+        assert "mi16_KK" in ctx.last_kernel(), ctx.last_kernel()
+        if name != "bf16_f8e4m3w":
+            check_fused(ctx, "dot", name, V([256, 296]).t(), V([256, 264]), [("add", 1, 0), ("relu",)], seed=9)
+            assert "mi16_MM" in ctx.last_kernel(), ctx.last_kernel()
+    finally:
+        ctx.force_tile(-1)
+
+
 @pytest.mark.parametrize("name", ["bf16", "f32", "bf16_f8e4m3w", "i32_i8i8"])
 def test_pipelined_kernels_with_k_cut(ctx, name):
     """partial sums of the K ranges carry no steps; the second pass that adds them applies the steps once"""
