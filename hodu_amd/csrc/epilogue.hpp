@@ -187,6 +187,46 @@ __device__ __forceinline__ void epilogue_apply_prepared(const EpiPrepared<DT, EP
     }
 }
 
+// The same for G pieces at once (the same columns of G rows): the steps are the outer loop, so a launch's choice
+// of operation is branched on once per step and group instead of once per step and piece, and each step is G * EPV
+// independent operations.  Between steps a value is narrowed and widened again, exactly what storing it and loading
+// it for the next step would do (for bf16 that is one AND).
+template <int DT, int EPV, int G>
+__device__ __forceinline__ void epilogue_apply_prepared_group(const EpiPrepared<DT, EPV> &p, typename EpiElem<DT>::T (&v)[G][EPV]) {
+#pragma clang fp contract(off)
+    typedef EpiElem<DT> E;
+    typedef typename E::W W;
+    W r[G][EPV];
+#pragma unroll
+    for (int q = 0; q < G; q++)
+#pragma unroll
+        for (int k = 0; k < EPV; k++) r[q][k] = E::widen(v[q][k]);
+#pragma unroll
+    for (int i = 0; i < kMaxEpilogueSteps; i++) {
+        if (i >= p.n) break;
+        if (p.op[i] == EPI_ADD_ROW) {
+#pragma unroll
+            for (int q = 0; q < G; q++)
+#pragma unroll
+                for (int k = 0; k < EPV; k++) r[q][k] = E::widen(E::narrow((W)(r[q][k] + p.k[i][k])));
+        } else if (p.op[i] == EPI_MUL_SCALAR) {
+#pragma unroll
+            for (int q = 0; q < G; q++)
+#pragma unroll
+                for (int k = 0; k < EPV; k++) r[q][k] = E::widen(E::narrow((W)(r[q][k] * p.k[i][0])));
+        } else if (E::floating) {  // EPI_RELU
+#pragma unroll
+            for (int q = 0; q < G; q++)
+#pragma unroll
+                for (int k = 0; k < EPV; k++) r[q][k] = E::widen(E::narrow(r[q][k] > (W)0 ? r[q][k] : (W)0));
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < G; q++)
+#pragma unroll
+        for (int k = 0; k < EPV; k++) v[q][k] = E::narrow(r[q][k]);
+}
+
 // the same behind a call, for kernels whose accumulator layout makes for hundreds of store sites per lane
 template <int DT>
 __device__ __attribute__((noinline)) typename EpiElem<DT>::T epilogue_apply_call(const DevEpilogue &e, typename EpiElem<DT>::T v,

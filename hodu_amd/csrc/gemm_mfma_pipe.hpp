@@ -178,7 +178,8 @@ __device__ __forceinline__ u32x4_t widen_f8x8(const u32x2_t &v) {
 // What the fused steps need for the columns a lane stores in a band of TN tiles of TS columns (the same columns in
 // every pass of every band of a wavefront's tile): fetched once per tile by the caller and handed to every band --
 // fetched per band, a bias vector's entries cost a trip to memory eight times per tile (config 5 up with bias and
-// ReLU: 46 us more than the plain product; once per tile: 28).
+// ReLU: 46 us more than the plain product; once per tile: 28; with four passes' pieces taking each step together,
+// one branch on the step's kind per group instead of per piece: 26).
 template <int OUT, int TN, int TS>
 __device__ __forceinline__ EpiPrepared<Out<OUT>::DT, 16 / (int)sizeof(typename Out<OUT>::T)> band_columns_prepare(const DevEpilogue &epi, int n_base,
                                                                                                                   int lane, int N) {
@@ -232,12 +233,14 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
             prepared = epilogue_prepare<Out<OUT>::DT, EPV>(epi, n < N ? n : N - 1, N);
         }
     }
-    auto row_chunk = [&](int pass, auto fused) {
+    auto patch_chunk = [&](int pass) {
         const int row = pass * RPP + lane / CPR, chunk = lane % CPR;
-        u32x4_t v = *reinterpret_cast<const u32x4_t *>(patch + row * PITCH + chunk * 16);
+        return *reinterpret_cast<const u32x4_t *>(patch + row * PITCH + chunk * 16);
+    };
+    auto store_chunk = [&](int pass, u32x4_t v) {
+        const int row = pass * RPP + lane / CPR, chunk = lane % CPR;
         const int m = m_base + row, n = n_base + chunk * EPV;
         if (m >= M || n >= N) return;
-        if constexpr (decltype(fused)::value) epilogue_apply_prepared<Out<OUT>::DT, EPV>(prepared, reinterpret_cast<out_t *>(&v));
         out_t *dst = Cb + (long)m * N + n;
         if (vec_ok && n + EPV <= N) {
             *reinterpret_cast<u32x4_t *>(dst) = v;
@@ -255,14 +258,35 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
         // instructions per element, inlined once per band this way instead of once per pass
         if constexpr (Out<OUT>::DT == HODU_F16) {
 #pragma unroll 1
-            for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::true_type{});
+            for (int pass = 0; pass < TS / RPP; pass++) {
+                u32x4_t v = patch_chunk(pass);
+                epilogue_apply_prepared<Out<OUT>::DT, EPV>(prepared, reinterpret_cast<out_t *>(&v));
+                store_chunk(pass, v);
+            }
         } else {
+            // up to four passes' pieces at a time: their steps are applied together
+            constexpr int NP = TS / RPP, GRP = NP < 4 ? NP : 4;
+            static_assert(NP % GRP == 0, "whole groups of passes");
 #pragma unroll
-            for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::true_type{});
+            for (int p0 = 0; p0 < NP; p0 += GRP) {
+                out_t e[GRP][EPV];
+#pragma unroll
+                for (int q = 0; q < GRP; q++) {
+                    const u32x4_t v = patch_chunk(p0 + q);
+                    __builtin_memcpy(e[q], &v, 16);
+                }
+                epilogue_apply_prepared_group<Out<OUT>::DT, EPV, GRP>(prepared, e);
+#pragma unroll
+                for (int q = 0; q < GRP; q++) {
+                    u32x4_t v;
+                    __builtin_memcpy(&v, e[q], 16);
+                    store_chunk(p0 + q, v);
+                }
+            }
         }
     } else {
 #pragma unroll
-        for (int pass = 0; pass < TS / RPP; pass++) row_chunk(pass, std::false_type{});
+        for (int pass = 0; pass < TS / RPP; pass++) store_chunk(pass, patch_chunk(pass));
     }
     asm volatile("" ::: "memory");  // the next band overwrites the patch
 }
