@@ -67,5 +67,16 @@ __device__ __forceinline__ uint8_t f32_to_f8e5m2_sat(float f) {
     f = (f != f) ? f : fminf(fmaxf(f, -57344.0f), 57344.0f);
     return (uint8_t)(__builtin_amdgcn_cvt_pk_bf8_f32(f, f, 0, false) & 0xFF);
 }
+// the same narrowing of four values into the four bytes of a dword (a first, in the low byte): the conversion
+// instruction takes two values and fills the half of the dword it is told to
+__device__ __forceinline__ float clamp_keep_nan(float f, float lim) { return (f != f) ? f : __builtin_amdgcn_fmed3f(f, -lim, lim); }
+__device__ __forceinline__ uint32_t f32x4_to_f8e4m3_sat(float a, float b, float c, float d) {
+    const int lo = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_keep_nan(a, 448.0f), clamp_keep_nan(b, 448.0f), 0, false);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(clamp_keep_nan(c, 448.0f), clamp_keep_nan(d, 448.0f), lo, true);
+}
+__device__ __forceinline__ uint32_t f32x4_to_f8e5m2_sat(float a, float b, float c, float d) {
+    const int lo = __builtin_amdgcn_cvt_pk_bf8_f32(clamp_keep_nan(a, 57344.0f), clamp_keep_nan(b, 57344.0f), 0, false);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(clamp_keep_nan(c, 57344.0f), clamp_keep_nan(d, 57344.0f), lo, true);
+}
 
 }  // namespace hodu

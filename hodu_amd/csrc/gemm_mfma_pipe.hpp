@@ -188,6 +188,10 @@ __device__ __forceinline__ EpiPrepared<Out<OUT>::DT, 16 / (int)sizeof(typename O
     return epilogue_prepare<Out<OUT>::DT, EPV>(epi, n < N ? n : N - 1, N);
 }
 
+// an output type that narrows four accumulators into one dword at once (Out<OUT>::cvt4; the 8-bit floats)
+template <class O, class = void> struct OutHasCvt4 : std::false_type {};
+template <class O> struct OutHasCvt4<O, std::void_t<decltype(&O::cvt4)>> : std::true_type {};
+
 template <int OUT, int TN, bool EPI, class acc_t, int TS = 32, bool READY = false>
 __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,
                                                    int n_base, int lane, int M, int N, const DevEpilogue &epi,
@@ -204,8 +208,13 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 Quad w;
+                if constexpr (OutHasCvt4<Out<OUT>>::value) {
+                    const uint32_t bits = Out<OUT>::cvt4(acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]);
+                    __builtin_memcpy(&w, &bits, 4);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][4 * q + e]);
+                    for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][4 * q + e]);
+                }
                 *reinterpret_cast<Quad *>(patch + lr * PITCH + (j * 32 + 8 * q + 4 * lh) * OS) = w;
             }
     } else {
@@ -213,8 +222,13 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             Quad w;
+            if constexpr (OutHasCvt4<Out<OUT>>::value) {
+                const uint32_t bits = Out<OUT>::cvt4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+                __builtin_memcpy(&w, &bits, 4);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][e]);
+                for (int e = 0; e < 4; e++) w.v[e] = Out<OUT>::cvt(acc[j][e]);
+            }
             *reinterpret_cast<Quad *>(patch + r16 * PITCH + (j * 16 + 4 * g4) * OS) = w;
         }
     }

@@ -28,12 +28,14 @@ template <> struct Out<OUT_F8E4M3> {
     typedef uint8_t T;
     // same narrowing as the generic kernel's f8e4m3 products: round to nearest even, saturating at +-448
     static __device__ __forceinline__ T cvt(float v) { return f32_to_f8e4m3_sat(v); }
+    static __device__ __forceinline__ uint32_t cvt4(float a, float b, float c, float d) { return f32x4_to_f8e4m3_sat(a, b, c, d); }
 };
 
 template <> struct Out<OUT_F8E5M2> {
     static constexpr int DT = HODU_F8E5M2;
     typedef uint8_t T;
     static __device__ __forceinline__ T cvt(float v) { return f32_to_f8e5m2_sat(v); }
+    static __device__ __forceinline__ uint32_t cvt4(float a, float b, float c, float d) { return f32x4_to_f8e5m2_sat(a, b, c, d); }
 };
 
 struct FragF8 {

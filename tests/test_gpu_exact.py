@@ -219,3 +219,53 @@ def test_native_f8_products_narrow_the_exact_sum_once(ctx, dt, tile):
         ctx.force_tile(-1)
         ctx.force_splitk(-1)
 
+
+
+@pytest.mark.parametrize("dt", ["f8e4m3", "f8e5m2"])
+@pytest.mark.parametrize("tile", [11, 12, 15])
+def test_native_f8_products_keep_nan_and_saturate_infinity(ctx, dt, tile):
+    """what the narrowing does where the f32 sum is not finite: a NaN operand makes its whole output row NaN, an
+    infinite f8e5m2 operand makes sums of +-inf, stored as the largest finite code of that sign (the narrowing
+    saturates), and inf * 0 is NaN; every other output is the exact small sum"""
+    m, n, k = 272, 208, 256
+    g = H.rng(900 + tile)
+    one = 0x38 if dt == "f8e4m3" else 0x3C
+    a = np.where(g.integers(0, 2, m * k) == 1, one, 0).astype(np.uint8).reshape(m, k)
+    b = np.full((n, k), one, dtype=np.uint8)
+    nan_code = 0x7F if dt == "f8e4m3" else 0x7E
+    a[3, 17] = nan_code
+    a[200, 255] = nan_code | 0x80
+    if dt == "f8e5m2":
+        a[5, :] = 0
+        a[5, 9] = 0x7C   # +inf
+        a[130, :] = 0
+        a[130, 77] = 0xFC  # -inf
+        b[40, 9] = 0     # inf * 0
+    ctx.force_tile(tile)
+    try:
+        md = H.dot_md(V([m, k]), V([n, k]).t())
+        da, db, dout = ctx.upload(a.ravel()), ctx.upload(b.ravel()), ctx.alloc(m * n)
+        ctx.fill(dout, 0x11)
+        ctx.product("dot", dt, da, db, dout, md)
+        got = ctx.download(dout, np.uint8, m * n).reshape(m, n)
+        kernel = ctx.last_kernel()
+        for d in (da, db, dout):
+            d.free()
+    finally:
+        ctx.force_tile(-1)
+    assert kernel.startswith(f"mfma_{dt}_pipe"), kernel
+    is_nan = (lambda c: (c & 0x7F) == 0x7F) if dt == "f8e4m3" else (lambda c: ((c & 0x7C) == 0x7C) & ((c & 3) != 0))
+    assert is_nan(got[3]).all() and is_nan(got[200]).all()
+    plain = np.ones(m, dtype=bool)
+    plain[[3, 200]] = False
+    if dt == "f8e5m2":
+        plain[[5, 130]] = False
+        cols = np.arange(n) != 40
+        assert (got[5, cols] == 0x7B).all() and (got[130] == 0xFB).all(), (got[5, :4], got[130, :4])
+        assert is_nan(got[5, 40])
+    # each output of a plain row: the number of ones in the row (column 40 of the f8e5m2 case misses k = 9)
+    sums = np.repeat((a[plain] == one).sum(axis=1).astype(np.float64)[:, None], n, axis=1)
+    if dt == "f8e5m2":
+        sums[:, 40] -= a[plain, 9] == one
+    want = H.f32_to_ocp_e4m3_rne(sums.ravel()) if dt == "f8e4m3" else narrow_e5m2_rne(sums.ravel())
+    assert np.array_equal(got[plain].ravel(), want)
