@@ -77,8 +77,8 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     // 16-bit operands of one type: the 256 x 256 tile on four wavefronts (one per SIMD, 128 x 128 outputs each) reads
     // a third fewer fragment bytes out of LDS than on eight and measured 2 % ahead (config 5 down 335 against 341 us,
     // up 368 against 376); with f8e4m3 weights, whose widening wants a second wavefront on the SIMD to hide behind,
-    // eight stay ahead (349 against 355 us), and so they do when element-wise steps ride on the store (config 2 with the
-    // attention scale: 38 against 44 us)
+    // eight stay ahead (349 against 355 us), and so they do on the 32 x 32 x 16 kernels when element-wise steps ride on
+    // the store (config 2 with the attention scale: 38 against 44 us)
     if constexpr (SKA == SK_SAME && SKB == SK_SAME && ES == 2) {
         if (forced < 0 && size == 0 && g.epi.n == 0) size = 1;
     }
@@ -131,11 +131,10 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     if constexpr (SKA == SK_SAME && SKB == SK_SAME && ES == 2 && CK != CK_I8) {
         // 16-bit operands on the 256 x 256 tile of four wavefronts: the 16 x 16 x 32 instruction, which
         // leaves the power-limited part a higher clock than the 32 x 32 x 16 one (hook value 15 pins it, 11 the other)
-        // (with element-wise steps on the store, which four wavefronts take 5 us longer over than eight, from 64 stages
-        // on: config 5 up with bias and ReLU 408 against 420 us, config 2 with the attention scale -- 16 stages -- 43
-        // against 38)
-        const bool fused_long = size == 0 && g.epi.n != 0 && stages >= 64;
-        if (pipe_ok && splits == 1 && ((forced < 0 && (size == 1 || fused_long)) || size == 5)) {
+        // (with element-wise steps on the store as well: config 5 up with bias and ReLU 375 against 420 us on eight
+        // wavefronts of the 32 x 32 x 16 kernel, config 2 with the attention scale 36.5-38.5 against 38.5-39.3)
+        const bool fused = size == 0 && g.epi.n != 0;
+        if (pipe_ok && splits == 1 && ((forced < 0 && (size == 1 || fused)) || size == 5)) {
             ctx->last_kernel = names[32 + combo];
             if (combo == 0) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
             if (combo == 1) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
