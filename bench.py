@@ -50,16 +50,16 @@ INFINITY_CACHE_BYTES = 256 << 20
 _TRAFFIC_FILE = "profiles/traffic_counters_all_bench_rows.txt"
 MEASURED_TRAFFIC = {
     # "kernel@config": (bytes per launch: FETCH_SIZE + WRITE_SIZE, each scaled by what it reads for a plain copy; summary file)
-    "mfma_bf16_pipe256x256mi16_KK@c5_down_bf16": (734.64e6, _TRAFFIC_FILE),
-    "mfma_bf16_pipe256x256mi16_KM@c5_up_bf16": (884.07e6, _TRAFFIC_FILE),
-    "mfma_bf16_f8w_pipe256x256mi16_KK@c3_m4096": (200.58e6, _TRAFFIC_FILE),
-    "mfma_bf16_f8w_pipe128x128_KK_splitk4@c3_m256": (68.98e6, _TRAFFIC_FILE),
+    "mfma_bf16_pipe256x256mi16_KK@c5_down_bf16": (734.63e6, _TRAFFIC_FILE),
+    "mfma_bf16_pipe256x256mi16_KM@c5_up_bf16": (884.02e6, _TRAFFIC_FILE),
+    "mfma_bf16_f8w_pipe256x256mi16_KK@c3_m4096": (200.56e6, _TRAFFIC_FILE),
+    "mfma_bf16_f8w_pipe128x128_KK_splitk4@c3_m256": (68.94e6, _TRAFFIC_FILE),
     "skinny_bf16_f8w_splitk@c3_m16": (22.19e6, _TRAFFIC_FILE),
     "gemv_bf16_f8w_walk@c3_m1": (16.89e6, _TRAFFIC_FILE),
     "gemv_bf16_f8w_walk@gemv_14336x4096": (58.67e6, _TRAFFIC_FILE),
-    "mfma_f8e4m3_pipe256x256mi16_KK@f8_4096": (117.15e6, _TRAFFIC_FILE),
-    "mfma_i32_i8i8_pipe128x128_KM@c4": (41.79e6, _TRAFFIC_FILE),
-    "mfma_bf16_pipe256x256mi16_KK@c2": (100.45e6, _TRAFFIC_FILE),
+    "mfma_f8e4m3_pipe256x256mi16_KK@f8_4096": (117.08e6, _TRAFFIC_FILE),
+    "mfma_i32_i8i8_pipe128x128_KM@c4": (41.78e6, _TRAFFIC_FILE),
+    "mfma_bf16_pipe256x256mi16_KK@c2": (100.43e6, _TRAFFIC_FILE),
 }
 
 
