@@ -53,12 +53,14 @@ __device__ __forceinline__ void widen_f8x16(const u32x4_t &w, u32x4_t &lo, u32x4
 }
 
 // CK: type fed to the matrix core; SKB: weight storage (CK itself, or f8e4m3 widened to bf16).
-// x_pitch > 0: the left operand (M x K, a few KB) is first copied to LDS, rows x_pitch bytes apart,
+// STAGE: the left operand (M x K, a few KB) is first copied to LDS, rows x_pitch bytes apart,
 // so that the MFMA's left fragments come from LDS instead of nearly-empty global loads (for M = 1
-// only 4 of 64 lanes carry a left-operand row).  x_pitch == 0: it does not fit; read it from global.
+// only 4 of 64 lanes carry a left-operand row).  !STAGE: a wavefront's left fragments come straight from memory
+// (cache hits), issued together with the weight loads they meet in the MFMA -- for a left operand that does not
+// fit in LDS, and where copying all of it into every workgroup costs more than reading it in place.
 // NBLK blocks of 16 weight rows per workgroup, KW wavefronts splitting K for each: the staged copy of x is shared
 // by all of them, so a larger NBLK means proportionally fewer copies of x through the memory pipeline
-template <int CK, int SKB, int OUT, int NBLK, int KW>
+template <int CK, int SKB, int OUT, int NBLK, int KW, bool STAGE = true>
 __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const char *__restrict__ X,
                                                                   const char *__restrict__ W,
                                                                   typename Out<OUT>::T *__restrict__ Y, DevProduct g,
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
     // finishes while the weights are still on their way.  (Issued after the weights, every load of the copy
     // loop waited for all of them, and the loop made one cache round trip per iteration.)
     constexpr int XB = 16;  // vectors of x a thread keeps in flight
-    const int vec_per_row = g.K * ES / 16, x_vecs = x_pitch > 0 ? g.M * vec_per_row : 0;
+    const int vec_per_row = g.K * ES / 16, x_vecs = STAGE ? g.M * vec_per_row : 0;
     u32x4_t xr[XB];
 #pragma unroll
     for (int i = 0; i < XB; i++) {
@@ -108,12 +110,26 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
         }
     }
     u32x4_t wv[CHUNK];
+    // !STAGE: the left fragments of a block of CHUNK weight vectors (two per vector of 16 f8 weights)
+    u32x4_t xa[STAGE ? 1 : CHUNK], xb[STAGE || SKB != SK_F8 ? 1 : CHUNK];
+    auto load_block = [&](int kb) {
 #pragma unroll
-    for (int u = 0; u < CHUNK; u++) {
-        const int k = kbeg + (u * 4 + lg) * EPL;
-        wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
-    }
-    if (x_pitch > 0) {
+        for (int u = 0; u < CHUNK; u++) {
+            const int k = kb + (u * 4 + lg) * EPL;
+            wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
+        }
+        if constexpr (!STAGE) {
+#pragma unroll
+            for (int u = 0; u < CHUNK; u++) {
+                const int k = kb + (u * 4 + lg) * EPL;
+                const bool ok = k < kend && has_x;
+                xa[u] = ok ? ldg16(xrow + (long)k * ES) : mfma::zero4();
+                if constexpr (SKB == SK_F8) xb[u] = ok ? ldg16(xrow + (long)(k + 8) * ES) : mfma::zero4();
+            }
+        }
+    };
+    load_block(kbeg);
+    if constexpr (STAGE) {
 #pragma unroll
         for (int i = 0; i < XB; i++) {
             const int v = tid + i * NT;
@@ -132,34 +148,27 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
 
     acc_t acc = acc_t{0, 0, 0, 0};
     for (int kb = kbeg; kb < kend; kb += CHUNK * 4 * EPL) {
-        if (kb != kbeg) {
-#pragma unroll
-            for (int u = 0; u < CHUNK; u++) {
-                const int k = kb + (u * 4 + lg) * EPL;
-                wv[u] = k < kend ? ldg16_stream(wrow + (long)k * SB) : mfma::zero4();
-            }
-        }
+        if (kb != kbeg) load_block(kb);
 #pragma unroll
         for (int u = 0; u < CHUNK; u++) {
             const int k = kb + (u * 4 + lg) * EPL;
-            const bool ok = k < kend && has_x;
-            u32x4_t xa = mfma::zero4(), xb = mfma::zero4();
-            if (x_pitch > 0) {
-                if (ok) {
-                    xa = *reinterpret_cast<const u32x4_t *>(xl + k * ES);
-                    if (SKB == SK_F8) xb = *reinterpret_cast<const u32x4_t *>(xl + (k + 8) * ES);
+            u32x4_t fa = mfma::zero4(), fb = mfma::zero4();
+            if constexpr (STAGE) {
+                if (k < kend && has_x) {
+                    fa = *reinterpret_cast<const u32x4_t *>(xl + k * ES);
+                    if (SKB == SK_F8) fb = *reinterpret_cast<const u32x4_t *>(xl + (k + 8) * ES);
                 }
-            } else if (ok) {
-                xa = ldg16(xrow + (long)k * ES);
-                if (SKB == SK_F8) xb = ldg16(xrow + (long)(k + 8) * ES);
+            } else {
+                fa = xa[u];
+                if constexpr (SKB == SK_F8) fb = xb[u];
             }
             if (SKB == SK_F8) {
                 u32x4_t lo, hi;
                 widen_f8x16(wv[u], lo, hi);
-                Cmp::mma(xa, lo, acc);
-                Cmp::mma(xb, hi, acc);
+                Cmp::mma(fa, lo, acc);
+                Cmp::mma(fb, hi, acc);
             } else {
-                Cmp::mma(xa, wv[u], acc);
+                Cmp::mma(fa, wv[u], acc);
             }
         }
     }
@@ -369,6 +378,22 @@ int launch_splitk(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, con
     return HODU_ROCM_OK;
 }
 
+// the one-pass kernel with the left operand read in place: one block of 16 weight rows per workgroup
+template <int CK, int SKB, int OUT>
+int launch_unstaged(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g) {
+    constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB, KW = 8;
+    (void)ES;
+    const int tiles_n = (g.N + 15) / 16;
+    const long blocks = g.batches * tiles_n;
+    if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
+    const int step = 4 * EPL;
+    const int k_per_wave = ((g.K + KW - 1) / KW + step - 1) / step * step;
+    hipLaunchKernelGGL((skinny_kdense_kernel<CK, SKB, OUT, 1, KW, false>), dim3((unsigned)blocks), dim3(KW * 64), 0, ctx->stream,
+                       (const char *)x, (const char *)w, (typename Out<OUT>::T *)y, g, tiles_n, k_per_wave, 0);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
 template <int CK, int SKB, int OUT, int NBLK, int KW>
 int launch_shape(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const DevProduct &g) {
     constexpr int ES = Compute<CK>::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB;
@@ -380,8 +405,9 @@ int launch_shape(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, cons
     // rows of the staged left operand are padded by 16 bytes so that the 16 row slots of a fragment
     // read hit different LDS banks
     const long pitch = (long)g.K * ES + 16;
-    const int x_pitch = (g.M * pitch <= X_LDS_LIMIT) ? (int)pitch : 0;
-    const size_t lds = x_pitch > 0 ? (size_t)g.M * x_pitch : 0;
+    if (g.M * pitch > X_LDS_LIMIT) return launch_unstaged<CK, SKB, OUT>(ctx, x, w, y, g);  // it does not fit
+    const int x_pitch = (int)pitch;
+    const size_t lds = (size_t)g.M * x_pitch;
     auto kernel = skinny_kdense_kernel<CK, SKB, OUT, NBLK, KW>;
     if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), X_LDS_LIMIT)) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NBLK * KW * 64), lds, ctx->stream, (const char *)x,
@@ -410,6 +436,7 @@ int run_kdense(hodu_rocm_ctx *ctx, const void *x, const void *w, void *y, const 
     if (ctx->force_tile == 36) shape = 1;
     if (ctx->force_tile == 37) shape = 2;
     ctx->last_kernel = name;
+    if (ctx->force_tile == 39) return launch_unstaged<CK, SKB, OUT>(ctx, x, w, y, g);
     if (ctx->force_tile < 35 || ctx->force_tile > 37) {  // the hook values 35..37 pin the one-pass kernel's shape, 38 this one
         const int rc = launch_splitk<CK, SKB, OUT>(ctx, x, w, y, g);
         if (rc != HODU_ROCM_UNSUPPORTED) {

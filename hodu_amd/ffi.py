@@ -458,7 +458,7 @@ class Context:
 
     def force_tile(self, tile: int):
         """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, 10..15 the pipelined
-        kernel's tiles (15: the 16x16x32 instruction), 30..34 the GEMV kernel's shapes, 35..38 the M <= 16 kernel's, -1 = automatic"""
+        kernel's tiles (15: the 16x16x32 instruction), 30..34 the GEMV kernel's shapes, 35..39 the M <= 16 kernel's, -1 = automatic"""
         self._check(self.debug.hodu_rocm_debug_force_tile(self.handle, int(tile)))
 
     def force_splitk(self, splits: int):

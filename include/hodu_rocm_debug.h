@@ -21,7 +21,8 @@ extern "C" {
  * 33 = its row-walking form (one wavefront per SIMD, the default from 16 weight rows per compute unit); 14 = the pipelined 256x128 tile,
  * 15 = the pipelined 256x256 tile on the 16x16x32 instruction (two k-dense 16-bit operands; 11 pins the 32x32x16 one);
  * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
- * variant that cuts K across workgroups wherever it applies; 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
+ * variant that cuts K across workgroups wherever it applies, 39 = one block per workgroup with the left operand read
+ * in place instead of staged in LDS (what a left operand too large for LDS gets); 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
  * 128 x 128 / 64 x 64 / 32 x 32 tiles;
  * -1 = automatic) so that every compiled variant
  * can be exercised at small sizes */

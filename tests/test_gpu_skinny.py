@@ -55,9 +55,10 @@ def test_batched_rows_fold_or_stay_batched(no_gemv, kind):
 
 
 @pytest.mark.parametrize("kind", list(KINDS))
-@pytest.mark.parametrize("shape", [35, 36, 37])
+@pytest.mark.parametrize("shape", [35, 36, 37, 39])
 def test_workgroup_shapes(ctx, kind, shape):
-    """1, 2 or 4 blocks of 16 weight rows per workgroup: N ragged against all of them, M from 5 to 16"""
+    """1, 2 or 4 blocks of 16 weight rows per workgroup, and (39) one block with the left operand read in place
+    instead of staged in LDS: N ragged against all of them, M from 5 to 16"""
     rs = 2.0 if "f8" in kind else None
     ctx.force_tile(shape)
     try:
@@ -66,6 +67,15 @@ def test_workgroup_shapes(ctx, kind, shape):
         check_product(ctx, "matmul", kind, V([3, 9, 256]), V([3, 40, 256]).t(), seed=2, rscale=rs, expect_kernel=KINDS[kind])
     finally:
         ctx.force_tile(-1)
+
+
+@pytest.mark.parametrize("kind", list(KINDS))
+def test_left_operand_too_large_for_lds(ctx, kind):
+    """16 rows of 9216 k do not fit the staging buffer: the one-pass kernel reads its left fragments in place (the
+    path hook value 39 pins at any size); K leaves an uneven split over the wavefronts, N is ragged"""
+    rs = 2.0 if "f8" in kind else None
+    check_product(ctx, "dot", kind, V([16, 9232]), V([40, 9232]).t(), seed=3, scale=0.5, rscale=rs, expect_kernel=KINDS[kind])
+    check_product(ctx, "dot", kind, V([13, 18432]), V([21, 18432]).t(), seed=4, scale=0.5, rscale=rs, expect_kernel=KINDS[kind])
 
 
 @pytest.mark.parametrize("kind", list(KINDS))
