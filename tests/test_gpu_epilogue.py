@@ -234,3 +234,52 @@ def test_rejected_steps(ctx):
         ctx.product_ex("dot", "i32", a, b, out, md, [ffi.add_row(out)])
     for d in (a, b, out, vec):
         d.free()
+
+
+@pytest.mark.parametrize("tile", [15, 11, 12, 2, -1])
+def test_steps_on_zero_nan_and_infinite_sums(ctx, tile):
+    """bf16 product whose plain output holds exact +0 (a zero row), NaN (a NaN in the row), +inf and -inf beside
+    ordinary small integers: a negative scalar turns +0 into -0 and the infinities round, ReLU turns -0, NaN and
+    -inf into +0 -- the reference's `(x > 0) ? x : 0` -- and the fused launch equals the reference's kernels on the
+    plain output bit for bit, on the 16 x 16 x 32 tile, the 32 x 32 x 16 ones, the general tile kernel and whatever
+    the automatic choice is"""
+    m, n, k = 272, 208, 256
+    g = H.rng(70 + tile)
+    af = g.integers(-3, 4, (m, k)).astype(np.float32)
+    bf = g.integers(1, 4, (n, k)).astype(np.float32)  # positive: an infinite operand gives an infinite sum, not NaN
+    af[0] = 0.0
+    af[17] = 0.0
+    af[1, 5] = np.nan
+    af[2, 100] = np.inf
+    af[3, 200] = -np.inf
+    af[4, 7], af[4, 9] = np.inf, -np.inf  # inf - inf
+    a, b = H.f32_to_bf16_rne(af.ravel()), H.f32_to_bf16_rne(bf.ravel())
+    lv, rv = V([m, k]), V([n, k]).t()
+    md = H.dot_md(lv, rv)
+    bias = H.f32_to_bf16_rne(g.integers(-4, 5, n).astype(np.float32))
+    bias[::7] = 0x8000  # -0
+    scalar = H.f32_to_bf16_rne(np.array([-1.5], dtype=np.float32))
+    ctx.force_tile(tile)
+    try:
+        plain = run_product(ctx, "dot", "bf16", a, b, md)
+        kernel = ctx.last_kernel()
+        p = plain.reshape(m, n)
+        assert (p[0] == 0).all() and (p[17] == 0).all() and ((p[1] & 0x7FFF) > 0x7F80).all()
+        assert (p[2] == 0x7F80).all() and (p[3] == 0xFF80).all() and ((p[4] & 0x7FFF) > 0x7F80).all()
+        for spec in ([("mul",)], [("relu",)], [("mul",), ("relu",)], [("add", 1, 0), ("relu",)],
+                     [("mul",), ("add", 1, 0), ("relu",)], [("relu",), ("mul",)]):
+            da, db, dbias = ctx.upload(a), ctx.upload(b), ctx.upload(bias)
+            dout = ctx.alloc(m * n * 2)
+            ctx.fill(dout, 0xFF)
+            steps = [ffi.add_row(dbias, s[1], s[2]) if s[0] == "add" else ffi.mul_scalar(scalar) if s[0] == "mul" else ffi.relu()
+                     for s in spec]
+            ctx.product_ex("dot", "bf16", da, db, dout, md, steps)
+            assert ctx.last_kernel() == kernel
+            got = ctx.download(dout, np.uint16, m * n)
+            for d in (da, db, dbias, dout):
+                d.free()
+            want = oracle_chain("bf16", plain, [m, n], spec, bias, scalar)
+            bad = np.flatnonzero(got != want)
+            assert bad.size == 0, (kernel, spec, bad[:5], got[bad[:5]], want[bad[:5]], plain[bad[:5]])
+    finally:
+        ctx.force_tile(-1)
