@@ -130,6 +130,20 @@ def test_k_zero_writes_zeros(ctx):
     assert np.all(got == 0)
 
 
+def test_empty_outputs_launch_nothing(ctx):
+    """M = 0, N = 0 or an empty batch: the call succeeds and the (one-element) output buffer keeps its bytes"""
+    a = ctx.upload(np.ones(16, np.float32)); b = ctx.upload(np.ones(16, np.float32)); o = ctx.alloc(4)
+    ctx.fill(o, 0x5A)
+    for md in ([0, 4, 3, 4, 1, 3, 1, 0, 0], [3, 4, 0, 4, 1, 1, 1, 0, 0]):  # dot: [M, K, N, ls_m, ls_k, rs_k, rs_n, l_off, r_off]
+        ctx.product("dot", "f32", a, b, o, md)
+    # matmul with batch [0]: [num_els, l_nd, r_nd, b_nd, l_shape, r_shape, batch_shape, l_strides, r_strides, l_off, r_off, M, K, N]
+    ctx.product("matmul", "f32", a, b, o, [0, 3, 3, 1, 0, 2, 4, 0, 4, 2, 0, 8, 4, 1, 8, 2, 1, 0, 0, 2, 4, 2])
+    ctx.sync()
+    assert ctx.download(o, np.uint8, 4).tolist() == [0x5A] * 4
+    for d in (a, b, o):
+        d.free()
+
+
 def test_errors_are_status_codes(ctx):
     a = ctx.upload(np.zeros(16, np.float32)); b = ctx.upload(np.zeros(16, np.float32)); o = ctx.alloc(64)
     with pytest.raises(ffi.HoduRocmError) as e:
