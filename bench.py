@@ -360,19 +360,16 @@ def time_case(ctx, case, steps, warmup, graph=False, exact_steps=False, verify=T
 
 
 def compact_row(r):
-    """one row of roofline.per_config: the median over the extra batches is the figure, p10 / p90 its spread"""
+    """one row of roofline.per_config: the median over the extra batches is the figure"""
     us = r["us_batches"]["median"]
     roof = r["roofline"]
     if roof["bound"] == "hbm":
         ach = r["alg_bytes"] / us / 1e3 if "alg_bytes" in r else roof["achieved"]
     else:
         ach = r["flops"] / us / 1e6 if "flops" in r else roof["achieved"]
-    row = {"key": r["config"], "us": round(us, 2), "p10": round(r["us_batches"]["p10"], 2), "p90": round(r["us_batches"]["p90"], 2),
-           "launches": r["us_batches"]["launches_per_batch"] * r["us_batches"]["batches"],
-           "bound": roof["bound"], "achieved": round(ach, 1), "unit": roof["unit"], "peak": roof["peak"],
+    # unit is TFLOP/s (TOP/s for integers) where bound is mfma, GB/s where it is hbm; p10 / p90 are in bench_full.json
+    row = {"key": r["config"], "us": round(us, 2), "bound": roof["bound"], "achieved": round(ach, 1), "peak": roof["peak"],
            "frac": round(ach / roof["peak"], 4), "kernel": r["kernel"]}
-    if r.get("parity") is not None:
-        row["parity"] = "ok"
     return row
 
 
@@ -945,65 +942,100 @@ def main():
         for sc in sum_cases():
             results.append(time_sum_case(ctx, *sc, args.steps, args.warmup))
             note(results[-1])
-    by_key = {r["config"]: r for r in results}
-    # the headline: exactly --warmup untimed launches, then exactly --steps timed ones, taken inside the HEAD row's call
-    head = by_key[HEAD]
-    head_us = head["headline_ms_total"] * 1e3 / args.steps
-    head_tflops = head_case.flops / head_us / 1e6
+    head = next(r for r in results if r["config"] == HEAD)
+    probes = {"register_only_mfma": mfma_clock_probe(ctx), "streaming_read": read_floor_probe(ctx), "device": info}
+    ctx.close()
+    cpu_rows, cpu_head = (None, None) if args.no_cpu else cpu_baselines(which, HEAD)
+    line, full = assemble_line(args.steps, args.warmup, HEAD, head_case.flops, head_case.alg_bytes, results, cpu_rows,
+                               cpu_head, probes)
+    # what does not fit the one-line contract (every row in full, the probes, the CPU rows' descriptions) goes to a file
+    try:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_full.json"), "w") as f:
+            json.dump(full, f)
+    except OSError as e:
+        print(f"# bench_full.json not written: {e}", file=sys.stderr)
+    text = json.dumps(line, separators=(",", ":"))
+    assert len(text) < LINE_LIMIT, f"the bench line is {len(text)} characters; its reader needs it under {LINE_LIMIT}"
+    sys.stderr.flush()
+    print(text, flush=True)
 
-    def target(key, need):
-        r = by_key.get(key)
-        if r is None:
-            return None
-        row = compact_row(r)
-        return {"key": key, "us": row["us"], "achieved": row["achieved"], "unit": row["unit"], "peak": row["peak"],
-                "frac": row["frac"], "target_frac": need, "met": row["frac"] >= need, "kernel": row["kernel"]}
+
+ROW_COLUMNS = ("key", "us", "bound", "achieved", "peak", "frac", "kernel")
+LINE_LIMIT = 6000  # characters of the final stdout line: what reads it keeps only a tail of stdout
+
+
+def _target(by_key, key, need):
+    r = by_key.get(key)
+    if r is None:
+        return None
+    row = compact_row(r)
+    return {"key": key, "us": row["us"], "frac": row["frac"], "target": need, "met": row["frac"] >= need}
+
+
+def assemble_line(steps, warmup, head_key, head_flops, head_bytes, results, cpu_rows, cpu_head, probes=None):
+    """(line, full): `line` is the one JSON object printed last on stdout -- the contract's scalar keys, the workload,
+    the headline's roofline with one compact row per measured configuration, and the CPU baseline with one short row
+    per configuration -- kept under LINE_LIMIT characters; `full` adds every row unabridged, the probe tables and the
+    CPU rows' descriptions, and is written to gpurun_out/bench_full.json."""
+    by_key = {r["config"]: r for r in results}
+    head = by_key[head_key]
+    head_us = head["headline_ms_total"] * 1e3 / steps
+    head_tflops = head_flops / head_us / 1e6
     line = {
         "metric": "TFLOP/s & % MFMA peak per dtype; M=1 GEMV GB/s & % HBM peak",
-        "value": head_tflops,
+        "value": round(head_tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": head_us / 1e3,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(head_us / 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE configs[4], the largest: transformer-MLP-shaped broadcast matmul, down projection with bf16 "
-                               "weights: X[8,512,14336] bf16 N(0,0.3) x W_down, a transposed view of bf16 N(0,0.02) [4096,14336] "
-                               "broadcast over the batch (stride 0), f32 accumulate, bf16 out; one matmul call per step",
-                   "flop_per_step": head_case.flops, "algorithmic_bytes_per_step": head_case.alg_bytes,
-                   "parity_checked_in_this_run": head["parity"],
-                   # the three rows the targets are stated on (bf16-rate 4096^3-class GEMM, native fp8 4096^3, M = 1 GEMV)
-                   "north_star": [t for t in (target("c3_m4096", 0.60), target("c5_down_bf16", 0.60), target("c5_up_bf16", 0.60),
-                                              target("bf16_4096", 0.60), target("f8_4096", 0.60), target("c3_m1", 0.70)) if t]},
-        "roofline": {"bound": "mfma", "achieved": head_tflops, "peak": PEAK["bf16"], "unit": "TFLOP/s",
-                     "frac": head_tflops / PEAK["bf16"], "traffic": head["roofline"]["traffic"],
+        "config": {"workload": "BASELINE configs[4] (largest), down projection: X[8,512,14336] bf16 x W_down = transposed "
+                               "view of bf16 [4096,14336] broadcast over the batch; f32 accumulate, bf16 out; 1 matmul per step",
+                   "flop_per_step": head_flops, "algorithmic_bytes_per_step": head_bytes,
+                   "parity_checked_in_this_run": bool(head.get("parity")),
+                   # `value` is timed on a warm clock; the first batch after host-side work runs on a ramping clock
+                   "cold_first_batch_us": round(head["first_batch_us"], 1),
+                   # the rows the targets are stated on (bf16-rate 4096^3-class GEMM, native fp8 4096^3, M = 1 GEMV)
+                   "north_star": [t for t in (_target(by_key, "c3_m4096", 0.60), _target(by_key, "c5_down_bf16", 0.60),
+                                              _target(by_key, "c5_up_bf16", 0.60), _target(by_key, "bf16_4096", 0.60),
+                                              _target(by_key, "f8_4096", 0.60), _target(by_key, "c3_m1", 0.70)) if t]},
+        "roofline": {"bound": "mfma", "achieved": round(head_tflops, 2), "peak": PEAK["bf16"], "unit": "TFLOP/s",
+                     "frac": round(head_tflops / PEAK["bf16"], 4), "traffic": head["roofline"]["traffic"],
                      "traffic_source": head["roofline"]["traffic_source"], "kernel": head["kernel"],
-                     "launch_us": head_us, "first_batch_us": head["first_batch_us"],
-                     # every configuration of this run: us = median over 10 batches of `launches / 10` back-to-back launches
-                     "per_config": [compact_row(r) for r in results]},
-        "dominant_kernel": head["kernel"],
-        # not part of the roofline (whose peak is the datasheet's): the rate a register-only MFMA loop sustains on
-        # this box, by operand data
-        "register_only_mfma": mfma_clock_probe(ctx),
-        # likewise for the HBM-bound rows: a kernel that only reads, at the M = 1 configurations' sizes
-        "streaming_read": read_floor_probe(ctx),
-        "device": info,
-        "all_configs": results,
+                     "launch_us": round(head_us, 2),
+                     # rows whose timed output buffer was compared with the oracle inside this run (a mismatch aborts)
+                     "parity_rows_ok": sum(1 for r in results if r.get("parity") is not None), "rows": len(results),
+                     # every configuration of this run, one array per row in the order of per_config_columns:
+                     # us = median over 10 batches of back-to-back launches; achieved and peak in TFLOP/s (TOP/s for
+                     # integers) where bound is mfma, in GB/s where it is hbm
+                     "per_config_columns": list(ROW_COLUMNS),
+                     "per_config": [[compact_row(r)[c] for c in ROW_COLUMNS] for r in results]},
     }
-    ctx.close()
-    if not args.no_cpu:
-        rows, head_row = cpu_baselines(which, HEAD)
-        line["cpu_baseline"] = {"value": head_row["value"], "unit": "TFLOP/s", "cores": head_row["cores"], "kind": head_row["kind"],
-                                "sample": f"{head_row['path']}: {head_row['sample']}; {head_row['seconds_sampled']} s of CPU work; "
-                                          f"the whole step would take {head_row['whole_job_seconds']} s ({head_row['whole_job_is']})",
-                                "host_cores_online": head_row["host_cores_online"],
-                                "f32_comparator_sgemm_tflops": head_row.get("f32_comparator_sgemm_tflops"),
-                                "per_config": rows}
-    print(json.dumps(line))
+    full = dict(line)
+    full["all_configs"] = results
+    if probes:
+        full.update(probes)
+    if cpu_rows is not None:
+        how = lambda r: "measured" if r["whole_job_is"] == "measured" else "extrapolated"  # noqa: E731
+        line["cpu_baseline"] = {
+            "value": float(f"{cpu_head['value']:.4g}"), "unit": "TFLOP/s", "cores": cpu_head["cores"], "kind": cpu_head["kind"],
+            "sample": (f"hodu_cpu_matmul_bf16, {cpu_head['sample']}: {cpu_head['seconds_sampled']} s of CPU work; "
+                       f"whole step {cpu_head['whole_job_seconds']} s ({how(cpu_head)})")[:200],
+            "host_cores_online": cpu_head["host_cores_online"],
+            "f32_comparator_sgemm_tflops": round(cpu_head.get("f32_comparator_sgemm_tflops") or 0.0, 2),
+            "per_config": [{"key": r["key"], "value": float(f"{r['value']:.4g}"), "cores": r["cores"], "kind": r["kind"],
+                            "whole_job_is": how(r)} for r in cpu_rows]}
+        full["cpu_baseline"] = dict(line["cpu_baseline"], per_config=cpu_rows,
+                                    sample=f"{cpu_head['path']}: {cpu_head['sample']}; {cpu_head['seconds_sampled']} s of CPU "
+                                           f"work; the whole step would take {cpu_head['whole_job_seconds']} s "
+                                           f"({cpu_head['whole_job_is']})")
+    return line, full
 
 
 if __name__ == "__main__":
