@@ -134,6 +134,14 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
         // (with element-wise steps on the store as well: config 5 up with bias and ReLU 375 against 420 us on eight
         // wavefronts of the 32 x 32 x 16 kernel, config 2 with the attention scale 36.5-38.5 against 38.5-39.3)
         const bool fused = size == 0 && g.epi.n != 0;
+        if (pipe_ok && splits == 1 && size == 6 && pipe16r_stages_ok(g.K, ES)) {
+            snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_r", names[32 + combo]);
+            ctx->last_kernel = ctx->kernel_name;
+            if (combo == 0) return launch_pipe16r<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
+            if (combo == 1) return launch_pipe16r<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
+            if (combo == 2) return launch_pipe16r<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_MN, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
+            return launch_pipe16r<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_MN, LM_MN, SK_SAME, 2>>(ctx, a, b, c, g);
+        }
         if (pipe_ok && splits == 1 && ((forced < 0 && (size == 1 || fused)) || size == 5)) {
             ctx->last_kernel = names[32 + combo];
             if (combo == 0) return launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_SAME, 2>>(ctx, a, b, c, g);
@@ -150,7 +158,7 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
             return launch_pipe16_f8w<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_F8, 2>>(ctx, a, b, c, g);
         }
     }
-    if (size == 5) return HODU_ROCM_UNSUPPORTED;
+    if (size == 5 || size == 6) return HODU_ROCM_UNSUPPORTED;
     if constexpr (SKA == SK_SAME && SKB == SK_SAME) {
         // testing hook values 10..13 pin the pipelined kernel's tile, 0..3 the general kernel's
         if (pipe_ok && size == 4 && combo <= 1) {

@@ -120,6 +120,12 @@ struct PipeConfig {
                   "row-dense operands: 8- and 16-bit types, tiles of at least 128 rows");
 };
 
+// Kernels that write their MFMAs out in assembly hide them from the compiler's hazard recogniser, which therefore
+// inserts nothing between the last matrix instruction and the first read of an accumulator behind the loop.  The
+// hardware wants idle wait states there -- up to 18 when a 16-pass instruction's result is read by a vector
+// instruction, fewer for the 4- and 8-pass instructions used here -- and does not interlock: these are they.
+__device__ __forceinline__ void mfma_results_settle() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
+
 // issued through inline assembly so that the compiler's own wait-count bookkeeping (which would put
 // an s_waitcnt vmcnt(0) in front of the next LDS read) stays out of the way; completion is awaited
 // explicitly before the barrier that publishes the stage

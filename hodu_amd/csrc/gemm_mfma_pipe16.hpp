@@ -28,6 +28,14 @@ namespace mfma {
 
 typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
 
+// f(integral_constant<int, 0>) .. f(integral_constant<int, N - 1>), in order: a loop whose index is a constant expression
+template <int N, int I = 0, class F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 // The instruction is written out with the accumulator tied to itself and held in the accumulation registers: left to
 // the register allocator, a kernel with 64 four-register accumulators and 128 fragment registers came out with the
 // accumulators rotating through copies inside the loop (twice the time).  What the compiler then no longer knows about
@@ -259,6 +267,269 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
         slot ^= 1;
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the re-fetches of the last stages are still writing LDS
+    mfma_results_settle();                      // the accumulators are read next
+    __syncthreads();
+
+    // epilogue: bands of 16 rows through a wavefront-private patch of LDS
+    char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));
+    out_t *Cb = C + batch * (long)g.M * g.N;
+    EpiPrepared<Out<Cfg::OUT>::DT, 16 / (int)sizeof(out_t)> steps{};
+    if (g.epi.n != 0) steps = band_columns_prepare<Cfg::OUT, TN, 16>(g.epi, n0 + wave_n * TN * 16, lane, g.N);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16, true>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
+                                                                g.M, g.N, g.epi, steps);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same kernel with the loop's non-MFMA instructions spaced by issue slots.
+//
+// One wavefront per SIMD issues everything in order, one instruction per four cycles; a 16 x 16 x 32 MFMA occupies
+// the matrix core for 16, so a gap between two MFMAs has room for three other instructions and every one beyond
+// that idles the matrix core for four cycles.  What the first kernel spent there: each LDS-DMA instruction with its
+// own M0 computation and write (s_add, s_mov m0, s_nop, load: four slots in one gap), and the compiler's address
+// arithmetic for sixteen of them gathered in a single gap.  Here
+//   * a wavefront's DMA instructions of an operand write 1 KB pieces that lie 1 KB apart in LDS, so the instruction's
+//     immediate offset (added to the global AND the LDS address) steps through four of them under one M0 value: the
+//     lane's global offset carries the opposite of that step, and base pointer and lane offsets are biased by 4 KB so
+//     that no offset goes below zero.  Four M0 writes per stage instead of sixteen, each a single s_add_u32 of a
+//     literal to a per-wavefront base, placed one gap ahead of the first load that needs it;
+//   * the stage loop is unrolled by two with the ring slot a literal, so every LDS address of a fragment read is an
+//     immediate on one of four registers and no M0 value needs arithmetic;
+//   * the source pointers advance by one add per operand and stage; the last two stages, which fetch nothing, are
+//     a copy of the loop body without the DMA list instead of re-fetching a clamped stage.
+// Needs an even number of stages (K a multiple of 128 elements), at least two; anything else takes the first kernel.
+template <int IMM> __device__ __forceinline__ void dma16_imm(const char *sbase, unsigned voff) {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(voff), "s"(sbase), "n"(IMM) : "memory");
+}
+// M0 = base + literal.  M0 stays as written until the next call: nothing else in these loops reads or writes it (LDS
+// reads need no M0 on this target), and at least the MFMA that follows separates the write from the DMA that uses it.
+template <int LIT> __device__ __forceinline__ void m0_set(unsigned base) {
+    asm volatile("s_add_u32 m0, %0, %1" ::"s"(base), "n"(LIT) : "scc");
+}
+
+// an even number of 128-byte stages, at least two
+inline bool pipe16r_stages_ok(long K, int elem_bytes) { return K > 0 && (K * elem_bytes) % (2 * P_ROW_BYTES) == 0; }
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_kernel(const char *__restrict__ A, const char *__restrict__ B,
+                                                               typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
+                                                               int tiles_m, int tiles_n) {
+    static_assert(!Cfg::B_F8 && Cfg::ES == 2 && Cfg::NST == 2, "16-bit operands stored in the compute type, two stages");
+    typedef RowDenseGeom<Cfg::ES, Cfg::ES> G;
+    extern __shared__ __align__(16) char smem[];
+    typedef Compute16<Cfg::CK> Cmp;
+    typedef typename Cmp::acc_t acc_t;
+    typedef typename Out<Cfg::OUT>::T out_t;
+    constexpr int ES = Cfg::ES, PA = Cfg::PA, PB = Cfg::PB, P = PA + PB;
+    constexpr int TM = Cfg::BM / Cfg::WM / 16, TN = Cfg::BN / Cfg::WN / 16;
+    constexpr int MF = TM * TN, RN = TM + TN;
+    constexpr int GRP = 4, BIAS = 4096;  // DMA instructions per M0 value; what keeps the lane offsets non-negative
+    static_assert(PA % GRP == 0 && PB % GRP == 0 && 3 * RN + 1 <= MF, "DMA groups of four; a gap for every fragment read");
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    long batch;
+    int tm, tn;
+    tile_of(blockIdx.x, (long)gridDim.x, tiles_m, tiles_n, batch, tm, tn);
+    long ao, bo;
+    batch_offsets(g, batch, ao, bo);
+    const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+
+    // LDS: two stages of A, then two of B.  Piece q (1 KB: 8 rows of 128 bytes, or KPI k-rows of a row-dense tile) of
+    // a stage is fetched by wavefront q / PA as its instruction q % PA.
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
+    constexpr int B_BASE = 2 * Cfg::A_BYTES;
+    unsigned offa[PA], offb[PB];
+#pragma unroll
+    for (int p = 0; p < PA; p++) {
+        const int q = wave * PA + p;
+        unsigned off;
+        if constexpr (Cfg::LA == LM_K) {
+            const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
+            int row = m0 + trow;
+            row = row < g.M ? row : g.M - 1;
+            off = (unsigned)((long)(row - m0) * g.a_m * ES) + dchunk * 16;
+        } else {
+            constexpr int CPR = Cfg::BM / G::EPC, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ rd16_swz(k);
+            int col = m0 + c * G::EPC;
+            col = col <= g.M - G::EPC ? col : g.M - G::EPC;
+            off = (unsigned)(((long)k * g.a_k + (col - (m0 <= g.M - G::EPC ? m0 : g.M - G::EPC))) * ES);
+        }
+        offa[p] = off + BIAS - (p % GRP) * 1024;
+    }
+#pragma unroll
+    for (int p = 0; p < PB; p++) {
+        const int q = wave * PB + p;
+        unsigned off;
+        if constexpr (Cfg::LB == LM_K) {
+            const int trow = q * 8 + (lane >> 3), dchunk = kd_slot(trow, lane & 7);
+            int row = n0 + trow;
+            row = row < g.N ? row : g.N - 1;
+            off = (unsigned)((long)(row - n0) * g.b_n * ES) + dchunk * 16;
+        } else {
+            constexpr int CPR = Cfg::BN / G::EPC, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ rd16_swz(k);
+            int col = n0 + c * G::EPC;
+            col = col <= g.N - G::EPC ? col : g.N - G::EPC;
+            off = (unsigned)(((long)k * g.b_k + (col - (n0 <= g.N - G::EPC ? n0 : g.N - G::EPC))) * ES);
+        }
+        offb[p] = off + BIAS - (p % GRP) * 1024;
+    }
+    const unsigned wbase_a = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * (PA * 1024));
+    const unsigned wbase_b = __builtin_amdgcn_readfirstlane(lds0 + B_BASE + (unsigned)wave * (PB * 1024));
+    const int T = g.K * ES / P_ROW_BYTES;  // stages: even, at least two (the launcher checks)
+    const long a_adv = Cfg::LA == LM_K ? P_ROW_BYTES : (long)G::STAGE_K * g.a_k * ES;
+    const long b_adv = Cfg::LB == LM_K ? P_ROW_BYTES : (long)G::STAGE_K * g.b_k * ES;
+    // source of the stage the next DMA list fetches, less the bias the lane offsets carry
+    const char *pa = uniform_ptr((Cfg::LA == LM_K ? A + (ao + (long)m0 * g.a_m) * ES
+                                                  : A + (ao + (m0 <= g.M - G::EPC ? m0 : g.M - G::EPC)) * ES) - BIAS);
+    const char *pb = uniform_ptr((Cfg::LB == LM_K ? B + (bo + (long)n0 * g.b_n) * ES
+                                                  : B + (bo + (n0 <= g.N - G::EPC ? n0 : g.N - G::EPC)) * ES) - BIAS);
+
+    // element d of the DMA list of a stage into ring slot SLOT: the left operand's pieces, then the right one's
+    auto dma_element = [&](auto slot_, auto d_) {
+        constexpr int SLOT = decltype(slot_)::value, D = decltype(d_)::value;
+        if constexpr (D < PA) dma16_imm<(D % GRP) * 1024>(pa, offa[D]);
+        else dma16_imm<((D - PA) % GRP) * 1024>(pb, offb[D - PA]);
+        (void)SLOT;
+    };
+    // the M0 value the group of list element d needs
+    auto dma_m0 = [&](auto slot_, auto d_) {
+        constexpr int SLOT = decltype(slot_)::value, D = decltype(d_)::value;
+        if constexpr (D < PA) m0_set<SLOT * Cfg::A_BYTES + (D / GRP) * GRP * 1024>(wbase_a);
+        else m0_set<SLOT * Cfg::B_BYTES + ((D - PA) / GRP) * GRP * 1024>(wbase_b);
+    };
+
+    constexpr int TILE_BYTES = 16 * P_ROW_BYTES;
+    int a_frag[2], b_frag[2];
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++) {
+        const int at = r16 * P_ROW_BYTES + (kd_slot(r16, 4 * sl + g4) << 4);
+        a_frag[sl] = (wave_m * TM) * TILE_BYTES + at;
+        b_frag[sl] = B_BASE + (wave_n * TN) * TILE_BYTES + at;
+    }
+    int a_mn[TM], b_mn[TN];
+    {
+        const int kq = r16 >> 2, sub = r16 & 3;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int bytes = (wave_m * TM + i) * 16 * ES + sub * 8, c = bytes >> 4;
+            a_mn[i] = (g4 * 8 + kq) * Cfg::BM * ES + ((c ^ rd16_swz(g4 * 8 + kq)) << 4) + (bytes & 8);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int bytes = (wave_n * TN + j) * 16 * ES + sub * 8, c = bytes >> 4;
+            b_mn[j] = B_BASE + (g4 * 8 + kq) * Cfg::BN * ES + ((c ^ rd16_swz(g4 * 8 + kq)) << 4) + (bytes & 8);
+        }
+    }
+    u32x4_t fa[2][TM], fb[2][TN];  // [slice][tile]
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = acc_t{0.f, 0.f, 0.f, 0.f};
+
+    // the r-th fragment read of slice SL from ring slot SLOT, in the order of first use
+    auto read_fragment = [&](auto sl_, auto slot_, int r) {
+        constexpr int SL = decltype(sl_)::value, SLOT = decltype(slot_)::value;
+        if (r < TM) {
+            const char *buf = smem + SLOT * Cfg::A_BYTES;
+            if constexpr (Cfg::LA == LM_K) {
+                fa[SL][r] = lds_get(buf, a_frag[SL] + r * TILE_BYTES);
+            } else {
+                const u32x2_t lo = lds_get_tr<ES>(buf, a_mn[r] + (SL * 32) * Cfg::BM * ES);
+                const u32x2_t hi = lds_get_tr<ES>(buf, a_mn[r] + (SL * 32 + 4) * Cfg::BM * ES);
+                fa[SL][r] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+            }
+        } else {
+            const char *buf = smem + SLOT * Cfg::B_BYTES;
+            if constexpr (Cfg::LB == LM_K) {
+                fb[SL][r - TM] = lds_get(buf, b_frag[SL] + (r - TM) * TILE_BYTES);
+            } else {
+                const u32x2_t lo = lds_get_tr<ES>(buf, b_mn[r - TM] + (SL * 32) * Cfg::BN * ES);
+                const u32x2_t hi = lds_get_tr<ES>(buf, b_mn[r - TM] + (SL * 32 + 4) * Cfg::BN * ES);
+                fb[SL][r - TM] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+            }
+        }
+    };
+    // One slice in a pinned order: the MFMAs of slice CUR; behind MFMAs 1, 4, 7, .. a read of slice 1 - CUR from ring
+    // slot RSLOT (none when READ is off: the last slice of the tile); in slice 1 with DMA on, list element d behind MFMA
+    // 3 * (1 + d * DSLOTS / P) -- a gap that holds nothing else -- and the M0 write of a group of four in the gap
+    // before its first element.
+    constexpr int DSLOTS = (MF - 4) / 3;
+    static_assert(DSLOTS >= P, "a gap of its own for every DMA instruction");
+    auto slice_step = [&](auto cur_, auto rslot_, auto read_, auto dma_, auto dslot_) {
+        constexpr int CUR = decltype(cur_)::value;
+        constexpr bool READ = decltype(read_)::value, DMA = decltype(dma_)::value;
+        typedef std::integral_constant<int, 1 - CUR> RS;
+        static_for<MF>([&](auto idx_) {
+            constexpr int idx = decltype(idx_)::value;
+            // operands swapped: a lane's accumulator then holds 4 consecutive n of one m
+            Cmp::mma(fb[CUR][idx / TM], fa[CUR][idx % TM], acc[idx % TM][idx / TM]);
+            if constexpr (READ && idx % 3 == 1 && idx / 3 < RN) read_fragment(RS{}, rslot_, idx / 3);
+            if constexpr (DMA) {
+                static_for<P>([&](auto d_) {
+                    constexpr int d = decltype(d_)::value;
+                    if constexpr (3 * (1 + d * DSLOTS / P) == idx) dma_element(dslot_, d_);
+                    if constexpr (d % GRP == 0 && 3 * (1 + d * DSLOTS / P) - 1 == idx) dma_m0(dslot_, d_);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    typedef std::true_type Yes;
+    typedef std::false_type No;
+
+    // prologue: stage 0 into slot 0, stage 1 into slot 1
+    static_for<2>([&](auto j_) {
+        static_for<P>([&](auto d_) {
+            constexpr int d = decltype(d_)::value;
+            if constexpr (d % GRP == 0) {
+                dma_m0(j_, d_);
+                asm volatile("s_nop 0");
+            }
+            dma_element(j_, d_);
+        });
+        pa += a_adv;
+        pb += b_adv;
+    });
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(P));  // slot 0 has landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int r = 0; r < RN; r++) read_fragment(I0{}, I0{}, r);
+
+    // stage t out of ring slot SLOT: slice 0 multiplies while slice 1's fragments are read; behind the barrier (stage
+    // t + 1 has landed, every read of stage t has returned) slice 1 multiplies while the next stage's slice 0 is read
+    // from the other slot and, with DMA on, stage t + 2 is sent for into the slot the barrier has just freed
+    auto stage = [&](auto slot_, auto dma_, auto last_) {
+        constexpr int SLOT = decltype(slot_)::value;
+        typedef std::integral_constant<int, 1 - SLOT> Other;
+        typedef std::integral_constant<bool, !decltype(last_)::value> ReadNext;
+        slice_step(I0{}, slot_, Yes{}, No{}, slot_);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        slice_step(I1{}, Other{}, ReadNext{}, dma_, slot_);
+        if constexpr (decltype(dma_)::value) {
+            pa += a_adv;
+            pb += b_adv;
+        }
+    };
+    for (int t = 0; t + 2 < T; t += 2) {
+        stage(I0{}, Yes{}, No{});
+        stage(I1{}, Yes{}, No{});
+    }
+    stage(I0{}, No{}, No{});
+    stage(I1{}, No{}, Yes{});
+    mfma_results_settle();  // the accumulators are read next
     __syncthreads();
 
     // epilogue: bands of 16 rows through a wavefront-private patch of LDS
@@ -490,6 +761,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
         }
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the re-fetches of the last stages are still writing LDS
+    mfma_results_settle();                      // the accumulators are read next
     __syncthreads();
 
     char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));
@@ -510,6 +782,20 @@ template <class Cfg> int launch_pipe16_f8w(hodu_rocm_ctx *ctx, const void *a, co
     const long total = g.batches * tiles_m * tiles_n;
     if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);
     if (g.K <= 0 || g.K % (Cfg::B_PAIR ? 128 : 64) != 0) return fail(HODU_ROCM_UNSUPPORTED, "K is not a whole number of stages");
+    hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a, (const char *)b,
+                       (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
+template <class Cfg> int launch_pipe16r(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
+    auto kernel = mfma_pipe16r_kernel<Cfg>;
+    static_assert(Cfg::NW * 16 * ((Cfg::BN / Cfg::WN) * 4 + 16) <= Cfg::LDS_BYTES, "the epilogue's patches fit the ring");
+    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
+    const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
+    const long total = g.batches * tiles_m * tiles_n;
+    if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);
+    if (!pipe16r_stages_ok(g.K, Cfg::ES)) return fail(HODU_ROCM_UNSUPPORTED, "K is not an even number of stages");
     hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a, (const char *)b,
                        (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n);
     HODU_HIP(hipGetLastError());

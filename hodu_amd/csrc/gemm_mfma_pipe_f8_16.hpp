@@ -191,6 +191,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8x16_kernel(const char *__
     if (t < T) stage(S0{}, 0, T - 1);
     // the re-fetches of the last stages still write LDS: wait for them, then for everybody's, before LDS is reused
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    mfma_results_settle();  // the accumulators are read next
     __syncthreads();
 
     char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));

@@ -108,9 +108,9 @@ extern "C" {
 
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
-    const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 15) || tile == 30 || tile == 31 ||
+    const bool ok = tile == -1 || (tile >= 0 && tile <= 3) || (tile >= 10 && tile <= 16) || tile == 30 || tile == 31 ||
                     (tile >= 32 && tile <= 34) || (tile >= 35 && tile <= 39) || (tile >= 40 && tile <= 43);
-    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..15, 30..39, 40..43", tile);
+    if (!ok) return fail(HODU_ROCM_INVALID_ARG, "tile %d not in -1..3, 10..16, 30..39, 40..43", tile);
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     ctx->force_tile = tile;
     return HODU_ROCM_OK;
