@@ -66,9 +66,8 @@ size_t out_elem_size(int kind, int dtype) {
 
 // Splits a parsed product into launches: the innermost kKernelBatchDims merged batch dims go to
 // the kernel, any further outer dims are walked here.
-int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p,
-                const DevEpilogue &epi) {
-    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+int run_product_launches(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p,
+                         const DevEpilogue &epi) {
     HODU_HIP(hipSetDevice(ctx->device));
     if (p.M > 0x7FFFFFFFL || p.N > 0x7FFFFFFFL || p.K > 0x7FFFFFFFL)
         return fail(HODU_ROCM_UNSUPPORTED, "matrix extent exceeds 2^31-1");
@@ -105,6 +104,16 @@ int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const vo
         if (rc != HODU_ROCM_OK) return rc;
     }
     return HODU_ROCM_OK;
+}
+
+int run_product(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c, const Product &p,
+                const DevEpilogue &epi) {
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    const int rc = run_product_launches(ctx, kind, dtype, a, b, c, p, epi);
+    // A launch that failed may have left arrival counters half counted (a kernel cut along K puts its counter back
+    // to zero only when its last workgroup finishes): zero them before the next kernel that relies on them.
+    if (rc == HODU_ROCM_HIP_ERROR || rc == HODU_ROCM_OOM) ctx->arrival_stale = true;
+    return rc;
 }
 
 // Validates the caller's fused steps for an output of `dtype` and turns them into what the kernels read.
@@ -224,8 +233,10 @@ int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, voi
 // The one entry point that allocates nothing: hodu_rocm_dot_bf16_f8e4m3w with the partial sums and arrival counters
 // of its split-K kernels in the device's static scratch array instead of the context's workspace.  For the length
 // of the call the context's workspace / counters are pointed at that array and marked fixed, so a kernel choice that
-// needs more is refused (ensure_workspace) rather than grown; the counters are zeroed by a kernel first, because the
-// array is shared by every call on this GPU and keeps whatever the last one left.
+// needs more is refused (ensure_workspace) rather than grown.  The array is shared by every call on this GPU and
+// keeps whatever the last one left, so its counters are marked stale: the kernel that counts on them zeroes them first
+// (ensure_arrival, one small launch), and a product whose kernel uses no counter -- the M <= 4 decode shapes -- pays
+// nothing for them.
 int hodu_rocm_dot_bf16_f8e4m3w_noalloc(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md,
                                        size_t n) {
     clear_error();
@@ -242,11 +253,13 @@ int hodu_rocm_dot_bf16_f8e4m3w_noalloc(hodu_rocm_ctx *ctx, const void *l, const 
     ctx->workspace.ptr = (char *)ctx->static_scratch + kStaticArrivalBytes;
     ctx->workspace.bytes = kStaticPartialBytes;
     ctx->arrival = (int *)ctx->static_scratch;
+    const bool saved_stale = ctx->arrival_stale;
     ctx->fixed_scratch = true;
-    rc = clear_static_arrival(ctx);
-    if (rc == HODU_ROCM_OK) rc = run_product(ctx, PK_BF16_F8W, HODU_BF16, l, r, o, p, DevEpilogue{});
+    ctx->arrival_stale = true;
+    rc = run_product(ctx, PK_BF16_F8W, HODU_BF16, l, r, o, p, DevEpilogue{});
     ctx->workspace = saved_ws;
     ctx->arrival = saved_arrival;
+    ctx->arrival_stale = saved_stale;
     ctx->fixed_scratch = false;
     return rc;
 }

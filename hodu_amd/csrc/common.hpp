@@ -30,6 +30,10 @@ struct hodu_rocm_ctx {
     hipDeviceProp_t props{};
     hodu::Workspace workspace;  // split-K partial sums; grown on demand, owned by the context
     int *arrival = nullptr;     // kArrivalSlots zeroed counters for kernels whose last workgroup finishes a reduction
+    // The counters `arrival` points at may hold something other than zeros (fresh memory; a launch that failed part
+    // way; the shared static array, which keeps what the last call on this GPU left): ensure_arrival zeroes them, by
+    // a kernel in stream order, before the next kernel that counts on them -- and only then.
+    bool arrival_stale = false;
     // Set for the duration of a call that must not allocate: `workspace` and `arrival` then point into the
     // device's static scratch array, and a kernel that needs more than it holds is refused instead of grown.
     bool fixed_scratch = false;
@@ -81,7 +85,9 @@ inline int ensure_dynamic_lds(hodu_rocm_ctx *ctx, const void *kernel, int bytes)
 // grows ctx->workspace to at least `bytes` (refused, with an error text, while ctx->fixed_scratch is set and the
 // static scratch is smaller, or while the context's stream is being captured into a graph and it would have to grow)
 int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes);
-// allocates (once) and zeroes ctx->arrival; kernels that use a counter leave it at zero again
+// allocates ctx->arrival (once) and zeroes the counters whenever ctx->arrival_stale says they may not be zero; a
+// kernel that uses a counter leaves it at zero again, so a launch that runs to completion keeps them clean.  Every
+// kernel that counts arrivals calls this right before its launch.
 constexpr int kArrivalSlots = 4096;
 int ensure_arrival(hodu_rocm_ctx *ctx);
 
@@ -89,9 +95,6 @@ int ensure_arrival(hodu_rocm_ctx *ctx);
 constexpr size_t kStaticArrivalBytes = (size_t)kArrivalSlots * sizeof(int);
 constexpr size_t kStaticPartialBytes = (size_t)8 << 20;
 constexpr size_t kStaticScratchBytes = kStaticArrivalBytes + kStaticPartialBytes;
-// launches the small kernel that zeroes the counters at the head of the static scratch (no memset node: callers may
-// be capturing a graph)
-int clear_static_arrival(hodu_rocm_ctx *ctx);
 
 inline size_t dtype_size(int dt) {
     static const size_t sz[15] = {1, 1, 1, 2, 2, 4, 8, 1, 2, 4, 8, 1, 2, 4, 8};

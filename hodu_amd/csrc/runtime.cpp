@@ -85,24 +85,21 @@ int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
 }
 
 int ensure_arrival(hodu_rocm_ctx *ctx) {
-    if (ctx->arrival) return HODU_ROCM_OK;
-    if (ctx->fixed_scratch) return fail(HODU_ROCM_HIP_ERROR, "static scratch is not set up on this context");
-    if (stream_is_capturing(ctx->stream))
-        return fail(HODU_ROCM_SCRATCH, "the arrival counters would be allocated while the stream is being "
-                    "captured: run the product once outside the capture first");
-    HODU_HIP(hipMalloc((void **)&ctx->arrival, kArrivalSlots * sizeof(int)));
-    // zeroed by a kernel, in stream order, before any kernel of this context can count on them
-    hipLaunchKernelGGL(clear_words_kernel, dim3((kArrivalSlots + 1023) / 1024), dim3(1024), 0, ctx->stream, ctx->arrival,
-                       kArrivalSlots);
-    HODU_HIP(hipGetLastError());
-    return HODU_ROCM_OK;
-}
-
-int clear_static_arrival(hodu_rocm_ctx *ctx) {
-    if (!ctx->static_scratch) return fail(HODU_ROCM_HIP_ERROR, "static scratch is not set up on this context");
-    hipLaunchKernelGGL(clear_words_kernel, dim3((kArrivalSlots + 1023) / 1024), dim3(1024), 0, ctx->stream,
-                       (int *)ctx->static_scratch, kArrivalSlots);
-    HODU_HIP(hipGetLastError());
+    if (!ctx->arrival) {
+        if (ctx->fixed_scratch) return fail(HODU_ROCM_HIP_ERROR, "static scratch is not set up on this context");
+        if (stream_is_capturing(ctx->stream))
+            return fail(HODU_ROCM_SCRATCH, "the arrival counters would be allocated while the stream is being "
+                        "captured: run the product once outside the capture first");
+        HODU_HIP(hipMalloc((void **)&ctx->arrival, kArrivalSlots * sizeof(int)));
+        ctx->arrival_stale = true;
+    }
+    if (ctx->arrival_stale) {
+        // by a kernel, in stream order (never a memset node: the caller may be capturing a graph)
+        hipLaunchKernelGGL(clear_words_kernel, dim3((kArrivalSlots + 1023) / 1024), dim3(1024), 0, ctx->stream, ctx->arrival,
+                           kArrivalSlots);
+        HODU_HIP(hipGetLastError());
+        ctx->arrival_stale = false;
+    }
     return HODU_ROCM_OK;
 }
 

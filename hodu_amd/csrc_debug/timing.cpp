@@ -116,6 +116,15 @@ int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile) {
     return HODU_ROCM_OK;
 }
 
+int hodu_rocm_debug_scratch_state(hodu_rocm_ctx *ctx, size_t *workspace_bytes, int *arrival_allocated, int *in_fixed_mode) {
+    if (!ctx || !workspace_bytes || !arrival_allocated || !in_fixed_mode) return fail(HODU_ROCM_INVALID_ARG, "null argument");
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    *workspace_bytes = ctx->workspace.ptr ? ctx->workspace.bytes : 0;
+    *arrival_allocated = ctx->arrival != nullptr;
+    *in_fixed_mode = ctx->fixed_scratch || (ctx->static_scratch && ctx->arrival == (int *)ctx->static_scratch);
+    return HODU_ROCM_OK;
+}
+
 int hodu_rocm_debug_force_splitk(hodu_rocm_ctx *ctx, int splits) {
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "context is null");
     if (splits < -1 || splits == 0 || splits > 64) return fail(HODU_ROCM_INVALID_ARG, "splits %d not in -1, 1..64", splits);

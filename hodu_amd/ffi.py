@@ -134,6 +134,7 @@ def load_debug() -> ctypes.CDLL:
     vpp = ctypes.POINTER(vp)
     lib.hodu_rocm_debug_force_tile.argtypes = [vp, ci]
     lib.hodu_rocm_debug_force_splitk.argtypes = [vp, ci]
+    lib.hodu_rocm_debug_scratch_state.argtypes = [vp, szp, ctypes.POINTER(ci), ctypes.POINTER(ci)]
     lib.hodu_rocm_debug_time_product.argtypes = [vp, ci, ci, ci, vp, vpp, sz, vp, szp, sz, ci, fp]
     lib.hodu_rocm_debug_time_product_graph.argtypes = lib.hodu_rocm_debug_time_product.argtypes
     lib.hodu_rocm_debug_time_product_ex.argtypes = [vp, ci, ci, ci, vp, vpp, sz, vp, szp, sz,
@@ -457,13 +458,20 @@ class Context:
         return {"read_us": r.value, "empty_us": e.value}
 
     def force_tile(self, tile: int):
-        """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, 10..15 the pipelined
-        kernel's tiles (15: the 16x16x32 instruction), 30..34 the GEMV kernel's shapes, 35..39 the M <= 16 kernel's, -1 = automatic"""
+        """testing hook: 0 = 256x256 / 8 wavefronts, 1 = 256x256 / 4, 2 = 128x128, 3 = 64x64, 10..16 the pipelined
+        kernel's tiles (15: the 16x16x32 instruction, 16: its respaced-issue form), 30..34 the GEMV kernel's shapes, 35..39 the M <= 16 kernel's, -1 = automatic"""
         self._check(self.debug.hodu_rocm_debug_force_tile(self.handle, int(tile)))
 
     def force_splitk(self, splits: int):
         """testing hook: K ranges of the pipelined kernels (-1 automatic, 1 never, n forced)"""
         self._check(self.debug.hodu_rocm_debug_force_splitk(self.handle, int(splits)))
+
+    def scratch_state(self) -> dict:
+        """testing hook: what this context has allocated for its kernels' scratch, and whether it is pointed at the
+        static scratch of the entry point that allocates nothing (never, between calls)"""
+        ws, arr, fixed = ctypes.c_size_t(), ctypes.c_int(), ctypes.c_int()
+        self._check(self.debug.hodu_rocm_debug_scratch_state(self.handle, ctypes.byref(ws), ctypes.byref(arr), ctypes.byref(fixed)))
+        return {"workspace_bytes": ws.value, "arrival_allocated": bool(arr.value), "fixed": bool(fixed.value)}
 
     def last_kernel(self) -> str:
         return self.lib.hodu_rocm_last_kernel(self.handle).decode()

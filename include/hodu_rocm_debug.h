@@ -19,7 +19,8 @@ extern "C" {
  * 2 = 128x128, 3 = 64x64; 10..13 the same tiles of the software-pipelined kernel; 30 = no row-streaming
  * GEMV kernel, 31/32/34 = that kernel as one-shot wavefronts (4 x 1, 4 x 2, 8 x 2 wavefronts x weight rows per workgroup),
  * 33 = its row-walking form (one wavefront per SIMD, the default from 16 weight rows per compute unit); 14 = the pipelined 256x128 tile,
- * 15 = the pipelined 256x256 tile on the 16x16x32 instruction (two k-dense 16-bit operands; 11 pins the 32x32x16 one);
+ * 15 = the pipelined 256x256 tile on the 16x16x32 instruction (two k-dense 16-bit operands; 11 pins the 32x32x16 one),
+ * 16 = the same tile with the loop's LDS-DMA and address instructions spaced by issue slots (an even number of stages);
  * 35/36/37 = the one-pass kernel for M <= 16 with 1/2/4 blocks of 16 weight rows per workgroup, 38 = its
  * variant that cuts K across workgroups wherever it applies, 39 = one block per workgroup with the left operand read
  * in place instead of staged in LDS (what a left operand too large for LDS gets); 40 = the small-product f32 kernel at any size; 41 / 42 / 43 = the f64 matrix-core kernel with
@@ -27,6 +28,10 @@ extern "C" {
  * -1 = automatic) so that every compiled variant
  * can be exercised at small sizes */
 int hodu_rocm_debug_force_tile(hodu_rocm_ctx *ctx, int tile);
+/* testing hook: what the context itself has allocated for its kernels' scratch -- bytes of its partial-sum workspace
+ * (0 = never allocated), whether its arrival counters exist -- and whether it is (still) pointed at the static
+ * scratch of the entry point that allocates nothing, which must never be the case between calls */
+int hodu_rocm_debug_scratch_state(hodu_rocm_ctx *ctx, size_t *workspace_bytes, int *arrival_allocated, int *in_fixed_mode);
 /* testing hook: number of K ranges the pipelined tile kernels cut a product into (each range a workgroup of its
  * own, partial sums added in a fixed order by a second kernel): -1 = automatic (only products too small to
  * fill the machine are cut), 1 = never, n = n ranges wherever the kernel can */

@@ -130,9 +130,11 @@ int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *lhs_i8, const void *r
  * sums; every GPU the library runs on holds one copy until the process ends) and the call makes no hipMalloc /
  * hipFree.  A product whose kernel would need more partial-sum space than that returns HODU_ROCM_SCRATCH with a
  * message naming both sizes (C3's M = 256 cut four ways needs 16 MiB; M <= 16 against any weight up to
- * N x slices <= 131072 fits).  All calls on one GPU share the array: the counters are zeroed by a small kernel at
- * the head of every call, and calls that overlap on one GPU -- two contexts, i.e. two streams -- race on it;
- * calls on one context are ordered by its stream.  No fused steps. */
+ * N x slices <= 131072 fits).  All calls on one GPU share the array and it keeps what the last call left: a call
+ * whose kernel counts arrivals zeroes the counters first (one small kernel in front of it, never a memset: the call
+ * may be under capture), a call whose kernel uses no scratch (M <= 4) launches nothing extra.  Calls that overlap
+ * on one GPU -- two contexts, i.e. two streams -- race on the array; calls on one context are ordered by its
+ * stream.  No fused steps. */
 #define HODU_ROCM_NOALLOC_PARTIAL_BYTES ((size_t)8 << 20)
 int hodu_rocm_dot_bf16_f8e4m3w_noalloc(hodu_rocm_ctx *ctx, const void *lhs_bf16, const void *rhs_f8e4m3,
                                        void *out_bf16, const size_t *metadata, size_t metadata_len);

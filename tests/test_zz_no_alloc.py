@@ -50,6 +50,42 @@ def test_two_calls_in_a_row_the_second_smaller(ctx):
     both(ctx, 16, 4096, 4096, 1, expect="skinny_bf16_f8w_splitk")   # and the first again, after the smaller one
 
 
+def test_a_fresh_context_allocates_nothing_for_it():
+    """the split-K shapes on a context that has never run a product: after the calls the context still owns no
+    partial-sum workspace and no arrival counters (had the entry point grown them, they would be there), while the
+    allocating entry point on the same context does grow them"""
+    fresh = ffi.Context(0)
+    try:
+        assert fresh.scratch_state() == {"workspace_bytes": 0, "arrival_allocated": False, "fixed": False}
+        m, n, k = 16, 4096, 4096
+        x = H.random_storage("bf16", m * k, 31)
+        w = H.random_storage("f8e4m3", n * k, 32, 30.0)
+        md = H.dot_md(V([m, k]), V([n, k]).t())
+        dx, dw, out_a, out_b = fresh.upload(x), fresh.upload(w), fresh.alloc(m * n * 2), fresh.alloc(m * n * 2)
+        for _ in range(2):
+            fresh.fill(out_b, 0xEE)
+            fresh.dot_noalloc(dx, dw, out_b, md)
+            assert fresh.last_kernel() == "skinny_bf16_f8w_splitk"
+            assert fresh.scratch_state() == {"workspace_bytes": 0, "arrival_allocated": False, "fixed": False}
+        fresh.force_splitk(4)
+        x2 = H.random_storage("bf16", 128 * k, 33)
+        dx2, out2 = fresh.upload(x2), fresh.alloc(128 * 512 * 2)
+        fresh.dot_noalloc(dx2, dw, out2, H.dot_md(V([128, k]), V([512, k]).t()))  # the pipelined kernel cut along K
+        assert "splitk" in fresh.last_kernel()
+        assert fresh.scratch_state() == {"workspace_bytes": 0, "arrival_allocated": False, "fixed": False}
+        fresh.force_splitk(-1)
+        got_b = fresh.download(out_b, np.uint16)
+        fresh.product("dot", "bf16_f8e4m3w", dx, dw, out_a, md)
+        state = fresh.scratch_state()
+        assert state["workspace_bytes"] > 0 and state["arrival_allocated"] and not state["fixed"]
+        assert np.array_equal(fresh.download(out_a, np.uint16), got_b)
+        for d in (dx, dw, out_a, out_b, dx2, out2):
+            d.free()
+    finally:
+        fresh.force_splitk(-1)
+        fresh.close()
+
+
 def test_shapes_without_scratch(ctx):
     both(ctx, 1, 4096, 4096, 5, expect="gemv_bf16_f8w_walk")
     both(ctx, 8, 640, 1024, 7)
@@ -77,8 +113,11 @@ def test_scratch_beyond_the_limit_is_refused(ctx):
             ctx.dot_noalloc(dx, dw, out, md)
         assert e.value.status == ffi.SCRATCH
         assert "16777216" in e.value.message and "8388608" in e.value.message
+        assert not ctx.scratch_state()["fixed"]  # the refused call put the context's own scratch pointers back
         ctx.product("dot", "bf16_f8e4m3w", dx, dw, out, md)  # the allocating entry point still takes it
         ctx.sync()
+        ctx.force_splitk(-1)
+        both(ctx, 16, 4096, 4096, 1, expect="skinny_bf16_f8w_splitk")  # and a split-K product after the refusal matches
     finally:
         ctx.force_splitk(-1)
         for d in (dx, dw, out):
