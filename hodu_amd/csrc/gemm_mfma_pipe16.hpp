@@ -311,7 +311,9 @@ template <int LIT> __device__ __forceinline__ void m0_set(unsigned base) {
 // an even number of 128-byte stages, at least two
 inline bool pipe16r_stages_ok(long K, int elem_bytes) { return K > 0 && (K * elem_bytes) % (2 * P_ROW_BYTES) == 0; }
 
-template <class Cfg>
+// STEPS: the instantiation that applies fused element-wise steps where the rows leave (the plain product's carries
+// none of their registers)
+template <class Cfg, bool STEPS>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                int tiles_m, int tiles_n) {
@@ -535,12 +537,18 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_kernel(const char *__res
     // epilogue: bands of 16 rows through a wavefront-private patch of LDS
     char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));
     out_t *Cb = C + batch * (long)g.M * g.N;
-    EpiPrepared<Out<Cfg::OUT>::DT, 16 / (int)sizeof(out_t)> steps{};
-    if (g.epi.n != 0) steps = band_columns_prepare<Cfg::OUT, TN, 16>(g.epi, n0 + wave_n * TN * 16, lane, g.N);
+    if constexpr (STEPS) {
+        const auto steps = band_columns_prepare<Cfg::OUT, TN, 16>(g.epi, n0 + wave_n * TN * 16, lane, g.N);
 #pragma unroll
-    for (int i = 0; i < TM; i++)
-        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16, true>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
-                                                                g.M, g.N, g.epi, steps);
+        for (int i = 0; i < TM; i++)
+            store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16, true>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16,
+                                                                    n0 + wave_n * TN * 16, lane, g.M, g.N, g.epi, steps);
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            store_band_via_lds<Cfg::OUT, TN, false, acc_t, 16>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16,
+                                                               n0 + wave_n * TN * 16, lane, g.M, g.N, g.epi);
+    }
 }
 
 // The same tile with f8e4m3 weights (the fused to_dtype of the right operand): the weight's bytes move as they are and
@@ -789,7 +797,7 @@ template <class Cfg> int launch_pipe16_f8w(hodu_rocm_ctx *ctx, const void *a, co
 }
 
 template <class Cfg> int launch_pipe16r(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
-    auto kernel = mfma_pipe16r_kernel<Cfg>;
+    auto kernel = g.epi.n != 0 ? mfma_pipe16r_kernel<Cfg, true> : mfma_pipe16r_kernel<Cfg, false>;
     static_assert(Cfg::NW * 16 * ((Cfg::BN / Cfg::WN) * 4 + 16) <= Cfg::LDS_BYTES, "the epilogue's patches fit the ring");
     if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
