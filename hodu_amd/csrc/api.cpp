@@ -339,6 +339,36 @@ int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, 
     return launch_softmax(ctx, dtype, in, out, r, inner, causal ? 1 : 0, nd >= 2 ? (long)md[1 + nd - 2] : 1);
 }
 
+int hodu_rocm_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len,
+                             int causal, const void *mask, int mask_dtype, const size_t *mask_layout, size_t mask_layout_len) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "softmax: context is null");
+    if (!in || !out || !mask) return fail(HODU_ROCM_INVALID_ARG, "softmax: null operand pointer");
+    if (in == out || mask == out) return fail(HODU_ROCM_INVALID_ARG, "softmax: out aliases an input");
+    if (mask_dtype != HODU_BOOL && mask_dtype != HODU_U8 && mask_dtype != HODU_I8)
+        return fail(HODU_ROCM_UNSUPPORTED, "softmax: the mask is one byte per element (bool, u8 or i8), got dtype id %d", mask_dtype);
+    Reduction r;
+    int rc = parse_reduce_metadata(md, len, &r);
+    if (rc) return rc;
+    const size_t nd = md[0], out_nd = md[2 + 2 * nd], n_red = md[3 + 2 * nd + out_nd];
+    if (nd < 1 || n_red != 1 || md[4 + 2 * nd + out_nd] + 1 != nd)
+        return fail(HODU_ROCM_INVALID_ARG, "softmax: a mask applies to the last dim of the input");
+    if (!mask_layout || mask_layout_len != nd + 2 || mask_layout[0] != nd)
+        return fail(HODU_ROCM_INVALID_ARG, "softmax: the mask layout is [nd, strides (nd).., offset] over the input's %zu dims", nd);
+    long shape[16], in_strides[16], mask_strides[16];
+    for (size_t d = 0; d < nd; d++) {
+        if (mask_layout[1 + d] > 0x7FFFFFFFFFFFL) return fail(HODU_ROCM_INVALID_ARG, "softmax: mask stride %zu out of range", d);
+        shape[d] = (long)md[1 + d];
+        in_strides[d] = (long)md[1 + nd + d];
+        mask_strides[d] = (long)mask_layout[1 + d];
+    }
+    if (mask_layout[1 + nd] > 0x7FFFFFFFFFFFL) return fail(HODU_ROCM_INVALID_ARG, "softmax: mask offset out of range");
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    HODU_HIP(hipSetDevice(ctx->device));
+    return launch_softmax_masked(ctx, dtype, in, out, mask, (int)nd, shape, in_strides, (long)md[1 + 2 * nd], mask_strides,
+                                 (long)mask_layout[1 + nd], causal ? 1 : 0);
+}
+
 int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
                         const size_t *md, size_t len, const void *scale, int causal) {
     clear_error();

@@ -218,6 +218,12 @@ int launch_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const R
 int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Reduction &r, long inner,
                    int causal, long sq);
 
+// softmax along the last dim with an attention mask (one byte per element, 0 = masked, own strides over the input's
+// shape) applied the way the reference's masked_fill + softmax applies it; causal as above
+int launch_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const void *mask, int nd,
+                          const long *shape, const long *in_strides, long in_off, const long *mask_strides, long mask_off,
+                          int causal);
+
 // One fused attention call: q [batch.., sq, d], k and v [batch.., sk, d] (batch dims already broadcast, last dim
 // dense), out contiguous [batch.., sq, d]
 struct AttentionArgs {

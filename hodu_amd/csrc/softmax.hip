@@ -260,6 +260,71 @@ __global__ __launch_bounds__(256) void softmax_strided_kernel(const typename E::
     for (long j = 0; j < s.len; j++) y[j] = E::store(j < limit ? wexp<W>((W)E::load(x[j * s.stride]) - m) / sum : (W)0);
 }
 
+// Softmax along the last dim with scaled_dot_product_attention's attn_mask (crates/hodu_nn/src/modules/attention.rs:
+// 50-56) and, optionally, its causal mask folded in.  The reference fills masked scores with get_neg_inf(dtype)
+// (:88-96) through masked_fill and then runs the softmax over ALL entries: -inf in f32 / f64, a finite stand-in in the
+// 16-bit types (-65504 converted to the dtype).  This kernel substitutes the same fill for a masked entry and computes
+// the same function, so a masked entry of a row with an open one is an exact zero, a row masked entirely is uniform
+// in bf16 / f16 and NaN in f32 / f64.  The mask (one byte per element, 0 = masked) keeps its own strides over the
+// input's shape -- 0 where it is broadcast -- and is never expanded.  One wavefront per row, three passes over it
+// (maximum, sum, write): the second and third read what the first brought into L2.
+struct DevMaskedSoftmax {
+    long rows, len;
+    long in_stride, in_off;         // element stride of the softmax dim in the input, offset of the input layout
+    long mask_stride, mask_off;     // the same for the mask
+    int lead_n;                     // dims in front of the softmax dim
+    long lead_shape[16], in_lead[16], mask_lead[16];
+    int causal;
+    long sq;
+    double fill;                    // what a masked score counts as
+};
+
+template <class E>
+__global__ __launch_bounds__(256) void softmax_masked_kernel(const typename E::storage *__restrict__ in,
+                                                            typename E::storage *__restrict__ out,
+                                                            const unsigned char *__restrict__ mask, DevMaskedSoftmax s) {
+    typedef typename E::acc W;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= s.rows) return;  // (whole wavefronts leave together: the shuffles below stay complete)
+    long xo = s.in_off, mo = s.mask_off, rem = row;
+    for (int d = s.lead_n - 1; d >= 0; d--) {
+        const long i = rem % s.lead_shape[d];
+        rem /= s.lead_shape[d];
+        xo += i * s.in_lead[d];
+        mo += i * s.mask_lead[d];
+    }
+    const typename E::storage *x = in + xo;
+    const unsigned char *mk = mask + mo;
+    long limit = s.causal ? (row % s.sq) + 1 : s.len;
+    limit = limit < s.len ? limit : s.len;
+    const W fill = (W)s.fill;
+    auto value = [&](long j) -> W { return (j < limit && mk[j * s.mask_stride] != 0) ? (W)E::load(x[j * s.in_stride]) : fill; };
+    W m = -(W)INFINITY;
+    for (long j = lane; j < s.len; j += 64) {
+        const W v = value(j);
+        m = v > m ? v : m;
+    }
+    m = lanes_max(m);
+    W sum = (W)0;
+    for (long j = lane; j < s.len; j += 64) sum += wexp<W>(value(j) - m);
+    sum = lanes_add(sum);
+    typename E::storage *y = out + row * s.len;
+    for (long j = lane; j < s.len; j += 64) y[j] = E::store(wexp<W>(value(j) - m) / sum);
+}
+
+template <class E> int run_masked(hodu_rocm_ctx *ctx, const void *in, void *out, const void *mask, const DevMaskedSoftmax &s) {
+    typedef typename E::storage S;
+    if (s.rows == 0 || s.len == 0) return HODU_ROCM_OK;
+    const long blocks = (s.rows + 3) / 4;
+    if (blocks > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "softmax needs %ld workgroups", blocks);
+    ctx->last_kernel = "softmax_masked";
+    hipLaunchKernelGGL(softmax_masked_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const S *)in, (S *)out,
+                       (const unsigned char *)mask, s);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
 template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const DevSoftmax &s, bool dim_is_last) {
     typedef typename E::storage S;
     if (s.rows == 0 || s.len == 0) return HODU_ROCM_OK;
@@ -353,6 +418,37 @@ int launch_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, con
     case HODU_F16: return run<Elem<HODU_F16>>(ctx, in, out, s, dim_is_last);
     case HODU_F32: return run<Elem<HODU_F32>>(ctx, in, out, s, dim_is_last);
     case HODU_F64: return run<Elem<HODU_F64>>(ctx, in, out, s, dim_is_last);
+    default: return fail(HODU_ROCM_UNSUPPORTED, "softmax: dtype id %d is not bf16 / f16 / f32 / f64", dtype);
+    }
+}
+
+// shape / in_strides / mask_strides: the input's nd extents and the two layouts' element strides over them (softmax dim
+// last, nd >= 1); the output is contiguous in that shape
+int launch_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const void *mask, int nd,
+                          const long *shape, const long *in_strides, long in_off, const long *mask_strides, long mask_off,
+                          int causal) {
+    DevMaskedSoftmax s{};
+    s.len = shape[nd - 1];
+    s.in_stride = in_strides[nd - 1];
+    s.mask_stride = mask_strides[nd - 1];
+    s.in_off = in_off;
+    s.mask_off = mask_off;
+    s.lead_n = nd - 1;
+    s.rows = 1;
+    for (int d = 0; d < 16; d++) {
+        s.lead_shape[d] = d < nd - 1 ? shape[d] : 1;
+        s.in_lead[d] = d < nd - 1 ? in_strides[d] : 0;
+        s.mask_lead[d] = d < nd - 1 ? mask_strides[d] : 0;
+        s.rows *= s.lead_shape[d];
+    }
+    s.causal = causal;
+    s.sq = nd >= 2 ? shape[nd - 2] : 1;
+    if (s.sq <= 0) s.sq = 1;
+    switch (dtype) {
+    case HODU_BF16: s.fill = -65536.0; return run_masked<Elem<HODU_BF16>>(ctx, in, out, mask, s);
+    case HODU_F16: s.fill = -65504.0; return run_masked<Elem<HODU_F16>>(ctx, in, out, mask, s);
+    case HODU_F32: s.fill = -(double)INFINITY; return run_masked<Elem<HODU_F32>>(ctx, in, out, mask, s);
+    case HODU_F64: s.fill = -(double)INFINITY; return run_masked<Elem<HODU_F64>>(ctx, in, out, mask, s);
     default: return fail(HODU_ROCM_UNSUPPORTED, "softmax: dtype id %d is not bf16 / f16 / f32 / f64", dtype);
     }
 }

@@ -114,6 +114,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
     lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
+    lib.hodu_rocm_softmax_masked.argtypes = [vp, ci, vp, vp, szp, sz, ci, vp, ci, szp, sz]
     lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
     lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc.argtypes = [vp, vp, vp, vp, szp, sz]
     _lib = lib
@@ -367,6 +368,26 @@ class Context:
                 raise HoduRocmError(INVALID_ARG, f"softmax_{dt}: metadata reaches past a device buffer")
         arr, n_md = _md_array(md)
         self._check(self.lib.hodu_rocm_softmax(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n_md, int(bool(causal))))
+
+    def softmax_masked(self, dt: str, x: DeviceBuffer, out: DeviceBuffer, md, mask: DeviceBuffer, mask_strides,
+                       mask_offset: int = 0, causal: bool = False, mask_dt: str = "u8"):
+        """hodu_rocm_softmax_masked: softmax along the last dim with attention's attn_mask (one byte per element, 0 =
+        masked; mask_strides in elements over the input's shape, 0 where the mask is broadcast) and optionally the
+        causal mask folded in"""
+        m = [int(v) for v in md]
+        nd = m[0] if m else 0
+        strides = [int(v) for v in mask_strides]
+        if len(m) < 2 + 2 * nd or len(strides) != nd:
+            raise HoduRocmError(INVALID_ARG, f"softmax_masked_{dt}: the mask layout needs one stride per input dim")
+        span = _view_span(m[1:1 + nd], m[1 + nd:1 + 2 * nd], m[1 + 2 * nd])
+        n = int(np.prod(m[1:1 + nd], dtype=np.int64)) if nd else 1
+        mask_span = _view_span(m[1:1 + nd], strides, int(mask_offset))
+        if span * DTYPE_SIZE[dt] > x.nbytes or n * DTYPE_SIZE[dt] > out.nbytes or mask_span > mask.nbytes:
+            raise HoduRocmError(INVALID_ARG, f"softmax_masked_{dt}: a layout reaches past a device buffer")
+        arr, n_md = _md_array(md)
+        larr, n_l = _md_array([nd] + strides + [int(mask_offset)])
+        self._check(self.lib.hodu_rocm_softmax_masked(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n_md, int(bool(causal)),
+                                                      mask.ptr, DTYPE_ID[mask_dt], larr, n_l))
 
     def attention(self, dt: str, q: DeviceBuffer, k: DeviceBuffer, v: DeviceBuffer, out: DeviceBuffer, md, scale, causal=False):
         """hodu_rocm_attention; md = [nb, batch_shape.., Sq, Sk, D, q_strides.., k_strides.., v_strides.., q_off, k_off,

@@ -98,6 +98,13 @@ long hodu_host_stats_attention_kernels(void) { return stats().attention_kernels;
 int hodu_host_softmax(const hodu_host_tensor *t, int dim, int causal, hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(T(t)->softmax(dim, causal != 0))); });
 }
+int hodu_host_softmax_masked(const hodu_host_tensor *t, const hodu_host_tensor *mask, int causal, hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(T(t)->softmax_masked(*T(mask), causal != 0))); });
+}
+int hodu_host_attention_masked(const hodu_host_tensor *q, const hodu_host_tensor *k, const hodu_host_tensor *v,
+                               const hodu_host_tensor *mask, int is_causal, hodu_host_tensor **out) {
+    return guarded([&] { *out = H(box(Tensor::scaled_dot_product_attention(*T(q), *T(k), *T(v), is_causal != 0, T(mask)))); });
+}
 int hodu_host_attention(const hodu_host_tensor *q, const hodu_host_tensor *k, const hodu_host_tensor *v, int is_causal,
                         hodu_host_tensor **out) {
     return guarded([&] { *out = H(box(Tensor::scaled_dot_product_attention(*T(q), *T(k), *T(v), is_causal != 0))); });

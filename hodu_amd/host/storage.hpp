@@ -207,6 +207,31 @@ public:
         return out;
     }
 
+    // softmax(-1) with attention's attn_mask folded in (crates/hodu_nn/src/modules/attention.rs:50-56): the mask's
+    // storage is read through `mask_layout` -- already broadcast to the scores' shape, stride 0 where it repeats -- and
+    // is never expanded.  One byte per element (bool / u8 / i8), 0 = masked out.
+    RocmStorage call_ops_softmax_masked(const Layout &layout, bool causal, const RocmStorage &mask, const Layout &mask_layout) const {
+        check_span(layout, "softmax");
+        mask.check_span(mask_layout, "softmax mask");
+        if (deferred()) return gather(layout).call_ops_softmax_masked(Layout::from_shape(layout.shape()), causal, mask, mask_layout);
+        if (mask.deferred() || dtype_size(mask.dtype()) != 1)
+            throw Error(ErrorKind::UnsupportedDTypeForOp, "softmax: the mask is a bool / u8 / i8 tensor (cast it with to_dtype first)");
+        if (dev_->id() != mask.dev_->id()) throw Error(ErrorKind::DeviceMismatch, "softmax: the mask lives on another device");
+        if (layout.ndim() == 0 || mask_layout.shape() != layout.shape())
+            throw Error(ErrorKind::InvalidArgument, "softmax: the mask layout is not broadcast to the input's shape");
+        const Metadata md = reduce_metadata(layout, {layout.ndim() - 1}, true);
+        Metadata ml{layout.ndim()};
+        ml.insert(ml.end(), mask_layout.strides().begin(), mask_layout.strides().end());
+        ml.push_back(mask_layout.offset());
+        RocmStorage out = fresh(dtype_, layout.size());
+        if (layout.size() == 0) return out;
+        dev_->check(hodu_rocm_softmax_masked(dev_->ctx(), (int)dtype_, ptr(), (void *)out.ptr(), md.data(), md.size(), causal ? 1 : 0,
+                                             mask.ptr(), (int)mask.dtype(), ml.data(), ml.size()),
+                    "softmax (masked)");
+        stats().softmax_kernels++;
+        return out;
+    }
+
     // the whole of scaled_dot_product_attention as one launch, where the fused kernel takes the call (bf16 / f16,
     // head dim 64 or 128, dense aligned rows): *taken says whether it did.  md: hodu_rocm_attention's metadata.
     RocmStorage call_ops_attention(const RocmStorage &k, const RocmStorage &v, const Layout &ql, const Layout &kl, const Layout &vl,

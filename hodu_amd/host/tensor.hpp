@@ -207,6 +207,15 @@ public:
         return Tensor(out, Layout::from_shape(shape()));
     }
 
+    // softmax(-1) of masked_fill(mask.eq_scalar(0), get_neg_inf(dtype)) (attention.rs:50-56, :88-96) as one launch: the
+    // mask broadcasts against the scores the way masked_fill's where3 broadcasts it (right-aligned, extent 1 repeats)
+    Tensor softmax_masked(const Tensor &mask, bool causal = false) const {
+        if (layout_.ndim() == 0) throw Error(ErrorKind::InvalidArgument, "softmax: a scalar has no last dim");
+        const Layout ml = mask.layout().broadcast_to(shape());
+        auto out = std::make_shared<RocmStorage>(storage_->call_ops_softmax_masked(layout_, causal, *mask.storage_, ml));
+        return Tensor(out, Layout::from_shape(shape()));
+    }
+
     // `value` as a scalar of dtype `dt`, round-to-nearest-even (what Scalar::to_dtype does through the `half` crate's
     // from_f32 for bf16 / f16: scalar.rs:391-404); only the floating dtypes
     static size_t scalar_bits(DType dt, double value, unsigned char out[8]) {
@@ -243,15 +252,22 @@ public:
         }
     }
 
-    // scaled_dot_product_attention (hodu_nn/src/modules/attention.rs:25-70) without attn_mask and dropout:
+    // scaled_dot_product_attention (hodu_nn/src/modules/attention.rs:25-70) without dropout:
     // softmax(Q K^T / sqrt(d_k) [+ causal mask]) V.  One launch where the fused kernel applies (bf16 / f16, head dim
     // 64 or 128, dense aligned rows); otherwise three -- the scale rides in the first product's store, the mask and the
     // five softmax kernels are one kernel, the second product is plain.
-    static Tensor scaled_dot_product_attention(const Tensor &q, const Tensor &k, const Tensor &v, bool is_causal) {
+    static Tensor scaled_dot_product_attention(const Tensor &q, const Tensor &k, const Tensor &v, bool is_causal,
+                                               const Tensor *attn_mask = nullptr) {
         if (q.layout().ndim() < 2) throw Error(ErrorKind::InvalidArgument, "attention: query needs at least two dimensions");
         const double scale = 1.0 / std::sqrt((double)q.shape().back());
         unsigned char bits[8];
         const size_t n = scalar_bits(q.dtype(), scale, bits);
+        if (attn_mask) {
+            // with an attn_mask (1 = attend, 0 = mask out; attention.rs:50-56) the function is three launches: the one
+            // kernel has no mask operand.  The mask is read in place by the softmax, broadcast over batch and heads.
+            const Tensor scores = q.matmul_then(k.transpose(-2, -1), {Then::mul_scalar(bits, n)});
+            return scores.softmax_masked(*attn_mask, is_causal).matmul(v);
+        }
         // one kernel where it applies: q [.., Sq, D], k and v [.., Sk, D] with the batch dims broadcast the way the
         // two matmuls would broadcast them
         const size_t qn = q.layout().ndim(), kn = k.layout().ndim(), vn = v.layout().ndim();

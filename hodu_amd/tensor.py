@@ -68,6 +68,8 @@ def load() -> ctypes.CDLL:
     lib.hodu_host_stats_attention_kernels.restype = ctypes.c_long
     lib.hodu_host_softmax.argtypes = [vp, ci, ci, vpp]
     lib.hodu_host_attention.argtypes = [vp, vp, vp, ci, vpp]
+    lib.hodu_host_softmax_masked.argtypes = [vp, vp, ci, vpp]
+    lib.hodu_host_attention_masked.argtypes = [vp, vp, vp, vp, ci, vpp]
     lib.hodu_host_scalar_bits.argtypes = [ci, ctypes.c_double, ctypes.POINTER(ctypes.c_ubyte), szp]
     lib.hodu_host_sum.argtypes = [vp, ctypes.POINTER(ci), sz, ci, vpp]
     lib.hodu_host_sum_to_shape.argtypes = [vp, szp, sz, vpp]
@@ -204,6 +206,11 @@ class Tensor:
         every [.., Sq, Sk] matrix are masked first (attention.rs:40-48)"""
         return self._unary(load().hodu_host_softmax, int(dim), int(causal))
 
+    def softmax_masked(self, mask: "Tensor", causal: bool = False) -> "Tensor":
+        """softmax(-1) of masked_fill(mask == 0, the dtype's -inf stand-in) (attention.rs:50-56) as one launch; the mask
+        (bool / u8 / i8) broadcasts against the scores and is read in place"""
+        return self._unary(load().hodu_host_softmax_masked, mask._h, int(causal))
+
     def sum(self, dims: Sequence[int] = (), keep_dim: bool = False) -> "Tensor":
         """Tensor::sum (tensor/ops/reduce.rs:11-13): no dims = all of them"""
         arr = (ctypes.c_int * max(1, len(dims)))(*dims)
@@ -275,11 +282,15 @@ def scalar_bits(dtype: str, value: float) -> np.ndarray:
     return np.frombuffer(bytes(buf[:n.value]), dtype=_BITS[n.value]).copy()
 
 
-def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False) -> Tensor:
-    """hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) without attn_mask and
-    dropout: one launch where the fused kernel applies (bf16 / f16, head dim 64 or 128), otherwise three (product with the
-    scale in its store, masked softmax, product)"""
+def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False,
+                                 attn_mask: Optional[Tensor] = None) -> Tensor:
+    """hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) without dropout: one launch
+    where the fused kernel applies (bf16 / f16, head dim 64 or 128, no attn_mask), otherwise three (product with the
+    scale in its store, masked softmax, product).  attn_mask: 1 = attend, 0 = mask out, broadcast against the scores."""
     out = ctypes.c_void_p()
+    if attn_mask is not None:
+        rc = load().hodu_host_attention_masked(q._h, k._h, v._h, attn_mask._h, int(is_causal), ctypes.byref(out))
+        return Tensor._wrap(rc, out)
     rc = load().hodu_host_attention(q._h, k._h, v._h, int(is_causal), ctypes.byref(out))
     return Tensor._wrap(rc, out)
 

@@ -228,6 +228,18 @@ int hodu_rocm_sum(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, cons
 int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *metadata,
                       size_t metadata_len, int causal);
 
+/* The same along the last dim with scaled_dot_product_attention's attn_mask (crates/hodu_nn/src/modules/attention.rs:
+ * 50-56: masked_fill(mask.eq_scalar(0), get_neg_inf(dtype)) in front of the softmax) folded in; causal as above, both
+ * may be given.  mask: device storage of a bool / u8 / i8 tensor, 0 = masked out; mask_layout (host): [nd, strides
+ * (nd).., offset] in elements over the INPUT's shape, stride 0 where the mask is broadcast (a [B, 1, 1, Sk] padding
+ * mask, a [Sq, Sk] mask shared by every head) -- the mask is read in place, never expanded.  Masked scores count as
+ * what the reference fills them with: -inf in f32 / f64, the dtype's rounding of -65504 in f16 / bf16 (:88-96), so a
+ * masked entry of a row that has an open one is an exact zero, a row masked entirely is uniform (16-bit types) or NaN
+ * (f32 / f64).  A mask of another dtype is cast by the caller (hodu_rocm_cast to u8) or compared on its side. */
+int hodu_rocm_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *metadata,
+                             size_t metadata_len, int causal, const void *mask, int mask_dtype,
+                             const size_t *mask_layout, size_t mask_layout_len);
+
 /* ---- attention as one kernel --------------------------------------------------------------------------- *
  * out = softmax(q k^T * scale [causal]) v for q [batch.., Sq, D], k and v [batch.., Sk, D]: what
  * scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) computes with a batched matmul,

@@ -196,6 +196,22 @@ def softmax_spec(dt: str, x: np.ndarray, md, causal: bool = False):
     return o32, o64
 
 
+def softmax_masked_spec(dt: str, x: np.ndarray, md, mask: np.ndarray, mask_strides, mask_offset: int = 0, causal: bool = False):
+    """(f32, f64) softmax along the last dim with attention's masks applied as the reference applies them (masked_fill
+    with the dtype's stand-in for -inf, then the softmax over every entry).  mask: one byte per element, 0 = masked;
+    mask_strides: element strides of the mask over the input's shape (0 where it is broadcast)."""
+    md = _md(md)
+    nd = int(md[0])
+    n = int(np.prod([int(v) for v in md[1:1 + nd]], dtype=np.int64)) if nd else 1
+    o32, o64 = np.empty(n, np.float32), np.empty(n, np.float64)
+    ms = _md(mask_strides)
+    assert len(ms) == nd
+    mask = np.ascontiguousarray(mask).view(np.uint8)
+    _check(lib().oracle_softmax_masked_spec(DTYPE_ID[dt], _ptr(x), _ptr(md), int(causal), _ptr(mask), _ptr(ms),
+                                            ctypes.c_size_t(int(mask_offset)), _ptr(o32), _ptr(o64)), "softmax_masked_spec")
+    return o32, o64
+
+
 def f8e4m3_table(decode: int) -> np.ndarray:
     """All 256 decoded values as f32."""
     return np.array([lib().oracle_f8e4m3_to_f32(b, decode) for b in range(256)], dtype=np.float32)

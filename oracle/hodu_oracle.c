@@ -20,7 +20,8 @@
  *            dims walked innermost first, accumulator in the storage type -- bf16 / f16 / f8 re-round after every
  *            add, :127-130), :133-237 (f32; a lane-wise SIMD order only when the last, dense dim alone is reduced)
  *   softmax  crates/hodu_core/src/tensor/ops/normalization.rs:4-21 (max(keep_dim), sub, exp, sum(keep_dim), div) with
- *            the causal masked_fill(-inf) of crates/hodu_nn/src/modules/attention.rs:40-48, :73-86 (mask j > i)
+ *            the causal masked_fill(-inf) of crates/hodu_nn/src/modules/attention.rs:40-48, :73-86 (mask j > i) and
+ *            the attn_mask masked_fill of :50-56 with get_neg_inf (:88-96)
  *   mul_scalar, relu
  *            crates/hodu_cpu_kernels/kernels/ops_unary.c:138-200, :352-386 (scalar arrives in the storage type),
  *            :648-697, :1233, :1319, :1404, :1484 ((x > 0) ? x : 0 in f32)
@@ -56,7 +57,12 @@
  * between); it is held against a float64 numpy softmax, against sum-to-one and shift invariance, and -- for f32 --
  * against the five-kernel chain run through oracle/_ref (hodu_cpu_max / sub / exp / sum / div), which it matches to
  * rounding.  The reference's bf16 / f16 chain rounds after every kernel and accumulates the sum in the narrow type;
- * as for the products, the GPU is gated against the f32 comparator, not against that chain.
+ * as for the products, the GPU is gated against the f32 comparator, not against that chain.  The masked form is
+ * held against the softmax of each row's unmasked entries (what it must equal whenever a row has one), against the
+ * unmasked function for a mask of ones, against the explicit fill-then-softmax in numpy, and -- for f32 -- against the
+ * reference's five-kernel chain run on a numpy masked_fill of the scores.  The conversion of -65504 to bf16 (-65536 by
+ * round-to-nearest) is the Rust `half` crate's, not under /root/reference: parity unpinned; it only shows in the
+ * maximum of a row masked entirely, whose result (uniform) does not depend on it.
  *
  * Parity unpinned: float->integer casts of out-of-range or NaN inputs are undefined behaviour
  * in the reference C ((T)x) and are not checked.  The stored code of an f8 x f8 -> f8 product: the reference
@@ -875,6 +881,54 @@ int oracle_softmax_spec(int dt, const void *in, const size_t *md, int causal, fl
             if (out64) out64[q] = j < limit ? exp(v - m64) / s64 : 0.0;
             if (out32) out32[q] = j < limit ? expf((float)v - m32) / s32 : 0.0f;
         }
+    }
+    return 0;
+}
+
+/* The same with scaled_dot_product_attention's attn_mask (crates/hodu_nn/src/modules/attention.rs:40-56): the causal
+ * mask (j > i) and the attention mask (mask element == 0; `mask.eq_scalar(0)`) are both applied by masked_fill with
+ * get_neg_inf(dtype) (attention.rs:88-96: -inf for f32 / f64, -65504 for f16 / bf16), the scalar converted to the
+ * tensor's dtype by full_like (tensor/ops/selection.rs:20-24; round to nearest: -65504 in f16, -65536 in bf16), and the
+ * softmax runs over ALL entries of the row, filled ones included.  So a masked entry of a row that has an unmasked one
+ * comes out as exp(fill - max) = 0; a row masked entirely comes out uniform (1 / len) in the 16-bit types and NaN in
+ * f32 / f64 (-inf - -inf).  mask: one byte per element; mask_strides: nd element strides over the INPUT's shape (0
+ * where the mask is broadcast), softmax dim last. */
+int oracle_softmax_masked_spec(int dt, const void *in, const size_t *md, int causal, const unsigned char *mask,
+                               const size_t *mask_strides, size_t mask_off, float *out32, double *out64) {
+    if (dt != DT_BF16 && dt != DT_F16 && dt != DT_F32 && dt != DT_F64) return -1;
+    reduce_space r;
+    reduce_space_from(md, &r);
+    if (r.n_red != 1 || r.red[0] + 1 != r.nd) return -1;
+    const size_t len = r.dims[r.nd - 1];
+    const size_t sq = r.nd >= 2 ? r.dims[r.nd - 2] : 1;
+    const double fill = dt == DT_F16 ? -65504.0 : dt == DT_BF16 ? -65536.0 : -INFINITY;
+    _Pragma("omp parallel for schedule(static)")
+    for (size_t o = 0; o < r.n_out; o++) {
+        /* o counts the rows in row-major order of the leading dims */
+        size_t mrow = mask_off, rem = o;
+        for (size_t d = r.nd - 1; d-- > 0;) {
+            mrow += (rem % r.dims[d]) * mask_strides[d];
+            rem /= r.dims[d];
+        }
+        const size_t limit = causal ? ((o % sq) + 1 < len ? (o % sq) + 1 : len) : len;
+        double m64 = -INFINITY, s64 = 0.0;
+        float m32 = -INFINITY, s32 = 0.0f;
+        for (int pass = 0; pass < 3; pass++)
+            for (size_t j = 0; j < len; j++) {
+                const size_t pos = reduce_pos(&r, o, j);
+                const int open = j < limit && mask[mrow + j * mask_strides[r.nd - 1]] != 0;
+                const double v = !open ? fill : dt == DT_F64 ? ((const double *)in)[pos] : (double)widen_any(dt, in, pos, F8_DECODE_OCP);
+                if (pass == 0) {
+                    if (v > m64) m64 = v;
+                    if ((float)v > m32) m32 = (float)v;
+                } else if (pass == 1) {
+                    s64 += exp(v - m64);
+                    s32 += expf((float)v - m32);
+                } else {
+                    if (out64) out64[o * len + j] = exp(v - m64) / s64;
+                    if (out32) out32[o * len + j] = expf((float)v - m32) / s32;
+                }
+            }
     }
     return 0;
 }
