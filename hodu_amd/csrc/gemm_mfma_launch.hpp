@@ -152,6 +152,12 @@ int launch_kind(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const
     }
     if constexpr (SKA == SK_SAME && SKB == SK_F8) {
         // f8e4m3 weights, k-dense or row-dense: the same tile and instruction with the widening in front of the MFMA
+        if (pipe_ok && combo <= 1 && splits == 1 && size == 6) {
+            snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_r", names[32 + combo]);
+            ctx->last_kernel = ctx->kernel_name;
+            if (combo == 0) return launch_pipe16r_f8w<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_F8, 2>>(ctx, a, b, c, g);
+            return launch_pipe16r_f8w<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_MN, SK_F8, 2>>(ctx, a, b, c, g);
+        }
         if (pipe_ok && combo <= 1 && splits == 1 && ((forced < 0 && size == 0) || size == 5)) {
             ctx->last_kernel = names[32 + combo];
             if (combo == 0) return launch_pipe16_f8w<PipeConfig<CK, OUT, 256, 256, 2, 2, LM_K, LM_K, SK_F8, 2>>(ctx, a, b, c, g);

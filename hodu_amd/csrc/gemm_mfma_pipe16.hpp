@@ -782,8 +782,274 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
                                                                 g.M, g.N, g.epi, steps);
 }
 
+// mfma_pipe16_f8w_kernel with its LDS-DMA spaced by issue slots, as mfma_pipe16r_kernel does for 16-bit operands: a
+// wavefront's pieces of an operand lie 1 KB apart in LDS and four of them share one M0 write (two groups for a stage of
+// the left operand, one for a stage's share of the right one), each M0 write -- a single s_add_u32 of a literal to a
+// base that depends on the ring slot -- in the gap before its group's first load and every load alone with the
+// conversion or fragment read its gap already holds.  Everything else is that kernel: the weight's bytes move as they are and
+// are widened to bf16 between the fragment read (8 bytes per lane) and the MFMA, one fragment ahead of its use, in the
+// shadow of the MFMAs of the fragment before.
+//   k-dense weights ([N, K] bytes): whole 128-byte lines, i.e. 128 k, the k of TWO stages of the bf16 left operand, so
+//     a right-operand buffer holds a pair of stages and the ring two pairs.  A pair's buffer is free behind the barrier
+//     of the pair's second stage and is needed four stages on, so its refill goes out in two halves, behind that
+//     barrier and behind the next one: every stage issues 8 + 4 DMA instructions.
+//   row-dense weights ([K, N] bytes): a stage is 64 k-rows of the tile's 256 bytes, in a ring of two like the left
+//     operand's (8 + 4 instructions per stage as well); a fragment is one 8-bit transpose read of 8 k-rows.
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_f8w_kernel(const char *__restrict__ A, const char *__restrict__ B,
+                                                                  typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
+                                                                  int tiles_m, int tiles_n) {
+    static_assert(Cfg::LA == LM_K && Cfg::B_F8 && Cfg::NST == 2, "bf16 x f8e4m3, the left operand k-dense, two stages");
+    extern __shared__ __align__(16) char smem[];
+    typedef Compute16<Cfg::CK> Cmp;
+    typedef typename Cmp::acc_t acc_t;
+    typedef typename Out<Cfg::OUT>::T out_t;
+    constexpr bool PAIR = Cfg::B_PAIR;  // k-dense weights
+    constexpr int ES = Cfg::ES, PA = Cfg::PA, PB = Cfg::PB, PBS = Cfg::PBS, P = PA + PBS;
+    constexpr int TM = Cfg::BM / Cfg::WM / 16, TN = Cfg::BN / Cfg::WN / 16;
+    constexpr int MF = TM * TN;
+    static_assert(TM == 8 && TN == 8 && P <= 19, "the schedule below is written for 128 x 128 outputs per wavefront");
+    constexpr int GRP = 4, BIAS = 4096;  // DMA instructions per M0 value; what keeps the biased lane offsets non-negative
+    static_assert(PA % GRP == 0 && PBS == GRP, "groups of four: two for a stage of A, one for a stage's share of B");
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    long batch;
+    int tm, tn;
+    tile_of(blockIdx.x, (long)gridDim.x, tiles_m, tiles_n, batch, tm, tn);
+    long ao, bo;
+    batch_offsets(g, batch, ao, bo);
+    const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+
+    // LDS: two stages of A (64 k of bf16 each), then two buffers of B (k-dense: 128 k each; row-dense: 64 k-rows each)
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
+    constexpr int B_BASE = 2 * Cfg::A_BYTES;
+
+    // DMA plan.  k-dense: an instruction writes 8 rows x 128 bytes; lane -> (row, slot), the slot holds chunk
+    // slot ^ ((row >> 1) & 7); rows past the operand's last one re-fetch the last one.  Address = scalar base of the
+    // tile's first row (advanced 128 bytes per stage of A, per pair of B) + the lane's 32-bit offset inside the tile.
+    // row-dense weights: an instruction writes 4 k-rows of 256 bytes; lane -> (k-row, slot), the slot holds chunk
+    // slot ^ (k % 16) (a transpose read serves 32 lanes at a time, 16 k-rows of 16 bytes: the swizzle spreads them over
+    // all banks); a chunk that starts past the last column is fetched from the last whole chunk instead.
+    // (piece q of a buffer is instruction q % PA -- q % PB -- of wavefront q / PA -- q / PB --; a lane's offset carries the
+    // bias and the opposite of the immediate offset its instruction adds back to the global and the LDS address)
+    unsigned offa[PA], offb[PB];
+#pragma unroll
+    for (int p = 0; p < PA; p++) {
+        const int q = wave * PA + p, trow = q * 8 + (lane >> 3);
+        int row = m0 + trow;
+        row = row < g.M ? row : g.M - 1;
+        offa[p] = (unsigned)((long)(row - m0) * g.a_m * ES) + kd_slot(trow, lane & 7) * 16 + BIAS - (p % GRP) * 1024;
+    }
+#pragma unroll
+    for (int p = 0; p < PB; p++) {
+        const int q = wave * PB + p;
+        if constexpr (PAIR) {
+            const int trow = q * 8 + (lane >> 3);
+            int row = n0 + trow;
+            row = row < g.N ? row : g.N - 1;
+            offb[p] = (unsigned)((long)(row - n0) * g.b_n) + kd_slot(trow, lane & 7) * 16 + BIAS - (p % GRP) * 1024;
+        } else {
+            constexpr int CPR = Cfg::BN / 16, KPI = 64 / CPR;
+            const int k = q * KPI + lane / CPR, c = (lane % CPR) ^ (k & 15);
+            int col = n0 + c * 16;
+            col = col <= g.N - 16 ? col : g.N - 16;
+            offb[p] = (unsigned)((long)k * g.b_k + (col - (n0 <= g.N - 16 ? n0 : g.N - 16))) + BIAS - (p % GRP) * 1024;
+        }
+    }
+    const unsigned wbase_a = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * (PA * 1024));
+    const unsigned wbase_b = __builtin_amdgcn_readfirstlane(lds0 + B_BASE + (unsigned)wave * (PB * 1024));
+    const int T = g.K * ES / P_ROW_BYTES;  // stages (k-dense weights: even, K is a multiple of 128)
+    const int TB = PAIR ? T / 2 : T;       // right-operand buffers' worth of k
+    const char *const base_a = uniform_ptr(A + (ao + (long)m0 * g.a_m) * ES - BIAS);
+    const char *const base_b = uniform_ptr((PAIR ? B + bo + (long)n0 * g.b_n : B + bo + (n0 <= g.N - 16 ? n0 : g.N - 16)) - BIAS);
+    const long b_adv = PAIR ? P_ROW_BYTES : 64L * g.b_k;
+
+    // list element e of a stage: the left operand's PA pieces of stage `src` (M0 of its group set beforehand from the
+    // ring slot), then the stage's PBS pieces of the right operand (k-dense: half `half` of the pair's rows)
+    auto dma_a = [&](auto e_, int src) {
+        constexpr int E = decltype(e_)::value;
+        dma16_imm<(E % GRP) * 1024>(base_a + (long)src * P_ROW_BYTES, offa[E]);
+    };
+    auto dma_b = [&](auto e_, int src, int half) {
+        constexpr int E = decltype(e_)::value;
+        unsigned voff = offb[E];
+        if constexpr (PAIR) voff = half ? offb[E + PBS] : offb[E];
+        dma16_imm<(E % GRP) * 1024>(base_b + src * b_adv, voff);
+    };
+    // M0 for group `grp` of the left operand's pieces into ring slot `slot`, and for the right operand's share
+    auto m0_a = [&](auto grp_, int slot) {
+        m0_set<decltype(grp_)::value * GRP * 1024>(wbase_a + (unsigned)slot * Cfg::A_BYTES);
+    };
+    auto m0_b = [&](int buf, int half) {
+        m0_set<0>(wbase_b + (unsigned)buf * Cfg::B_BYTES + (PAIR ? (unsigned)half * (PBS * 1024) : 0u));
+    };
+
+    // fragment addresses.  A: lane (r16, g4) reads chunk 4 * slice + g4 of row r16 (16 bytes).  B k-dense: the lane's
+    // 8 k are 8 bytes: half g4 % 2 of chunk 4 * (stage % 2) + 2 * slice + g4 / 2 of the row's 128-byte line; slice and
+    // stage flip bits 5 and 6 of the byte offset (the swizzle is an XOR on the chunk index).  B row-dense: the 16 lanes
+    // of group g4 take their 8 k of column r16 out of k-rows 32 * slice + 8 * g4 .. + 7 through one transpose read, for
+    // which lane s of the 16 supplies the address of 8 columns of k-row (that start) + s / 2; k % 16 is
+    // 8 * (g4 % 2) + s / 2 whatever the slice, so the swizzle is the lane's own and slices are immediates; tiles are not.
+    constexpr int TILE_BYTES = 16 * P_ROW_BYTES;
+    int a_frag[2];
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++) a_frag[sl] = (wave_m * TM) * TILE_BYTES + r16 * P_ROW_BYTES + (kd_slot(r16, 4 * sl + g4) << 4);
+    const int b_frag = B_BASE + (wave_n * TN) * TILE_BYTES + r16 * P_ROW_BYTES + (kd_slot(r16, g4 >> 1) << 4) + (g4 & 1) * 8;
+    int b_mn[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int kq = r16 >> 1, bytes = (wave_n * TN + j) * 16 + (r16 & 1) * 8, c = bytes >> 4, k = 8 * g4 + kq;
+        b_mn[j] = B_BASE + k * Cfg::BN + ((c ^ (k & 15)) << 4) + (bytes & 8);
+    }
+
+    u32x4_t fa[2][TM];
+    u32x2_t fb[2][TN];  // raw bytes
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = acc_t{0.f, 0.f, 0.f, 0.f};
+
+    // the r-th fragment read of slice SL of stage `st` (ring slot st % 2): the left operand's tiles, then the right's
+    auto read_fragment = [&](auto sl_, int r, int st) {
+        constexpr int SL = decltype(sl_)::value;
+        if (r < TM) {
+            fa[SL][r] = lds_get(smem + (st & 1) * Cfg::A_BYTES, a_frag[SL] + r * TILE_BYTES);
+        } else if constexpr (PAIR) {
+            const int at = (b_frag ^ (SL << 5) ^ ((st & 1) << 6)) + (r - TM) * TILE_BYTES;
+            fb[SL][r - TM] = lds_get64(smem + ((st >> 1) & 1) * Cfg::B_BYTES, at);
+        } else {
+            fb[SL][r - TM] = lds_get_tr<1>(smem + (st & 1) * Cfg::B_BYTES, b_mn[r - TM] + SL * 32 * Cfg::BN);
+        }
+    };
+    u32x4_t bwide = u32x4_t{0u, 0u, 0u, 0u};  // the widened first right fragment of the next slice
+    // One slice in a pinned order, as in mfma_pipe16_kernel: a read behind MFMAs 1, 4, 7, .., in slice 1 a DMA instruction
+    // behind MFMAs 3, 6, 9, ..; the right fragment of the next group of TM MFMAs is widened behind the first four
+    // MFMAs of the current group, the first fragment of the next slice behind this slice's last four.
+    auto slice_step = [&](auto cur_, int rd_stage, int a_src, int a_slot, int b_src, int b_buf, int b_half) {
+        constexpr int CUR = decltype(cur_)::value;
+        typedef std::integral_constant<int, 1 - CUR> RS;
+        constexpr int DSLOTS = (MF - 4) / 3;
+        static_assert(DSLOTS >= P, "a gap of its own for every DMA instruction");
+        u32x4_t bcur = bwide, bnext = bcur;
+        // one conversion (two values) behind each of the first four MFMAs of a group: four in a row take longer to
+        // issue than the MFMA in front of them runs
+        auto widen_part = [&](u32x4_t &dst, const u32x2_t &raw, int part) {
+            const uint32_t w = part < 2 ? raw.x : raw.y;
+            const uint32_t v = bitcast<uint32_t>(part & 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                                                          : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+            if (part == 0) dst.x = v;
+            else if (part == 1) dst.y = v;
+            else if (part == 2) dst.z = v;
+            else dst.w = v;
+        };
+#pragma unroll
+        for (int idx = 0; idx < MF; idx++) {
+            if (idx % TM == 0 && idx > 0) bcur = bnext;
+            Cmp::mma(bcur, fa[CUR][idx % TM], acc[idx % TM][idx / TM]);
+            if (idx % TM < 4 && idx / TM + 1 < TN) widen_part(bnext, fb[CUR][idx / TM + 1], idx % TM);
+            if (idx >= MF - 4) widen_part(bwide, fb[1 - CUR][0], idx - (MF - 4));
+            if (idx % 3 == 1 && idx / 3 < TM + TN) read_fragment(RS{}, idx / 3, rd_stage);
+            if constexpr (CUR == 1) {
+                static_for<P>([&](auto d_) {
+                    constexpr int d = decltype(d_)::value;
+                    if (3 * (1 + d * DSLOTS / P) == idx) {
+                        if constexpr (d < PA) dma_a(d_, a_src);
+                        else dma_b(std::integral_constant<int, (d < PA ? 0 : d - PA)>{}, b_src, b_half);
+                    }
+                    // the group's M0 one gap ahead of its first load
+                    if (d % GRP == 0 && 3 * (1 + d * DSLOTS / P) - 1 == idx) {
+                        if constexpr (d < PA) m0_a(std::integral_constant<int, d / GRP>{}, a_slot);
+                        else m0_b(b_buf, b_half);
+                    }
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+
+    // prologue: stage 0 of A and buffer 0 of B, then stage 1 of A and (k-dense: the first half of) buffer 1 of B (clamped)
+    auto fetch_a = [&](int src, int slot) {
+        static_for<PA>([&](auto e_) {
+            constexpr int E = decltype(e_)::value;
+            if constexpr (E % GRP == 0) {
+                m0_a(std::integral_constant<int, E / GRP>{}, slot);
+                asm volatile("s_nop 0");
+            }
+            dma_a(e_, src);
+        });
+    };
+    auto fetch_b = [&](int src, int buf, int half) {
+        m0_b(buf, half);
+        asm volatile("s_nop 0");
+        static_for<PBS>([&](auto e_) { dma_b(e_, src, half); });
+    };
+    fetch_a(0, 0);
+    fetch_b(0, 0, 0);
+    if constexpr (PAIR) fetch_b(0, 0, 1);
+    fetch_a(1 < T ? 1 : T - 1, 1);
+    fetch_b(1 < TB ? 1 : TB - 1, 1, 0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(PA + PBS));  // stage 0 and buffer 0 have landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int r = 0; r < TM + TN; r++) read_fragment(I0{}, r, 0);
+    bwide = widen_f8x8(fb[0][0]);
+
+    // Past the last stage the reads fetch LDS bytes nobody uses and the lists re-fetch the last stage (pair) into
+    // buffers nobody reads: harmless, and the number of instructions in flight stays what the waits assume.
+    for (int t = 0; t < T; t++) {
+        slice_step(I0{}, t, 0, 0, 0, 0, 0);
+        // stage t + 1 (and its pair) has landed and every read of stage t has returned
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // A: stage t + 2 into the slot of stage t.  B row-dense: likewise.  B k-dense: odd t has just finished pair
+        // t / 2 and sends the first half of pair t / 2 + 2 into its buffer; the next (even) stage sends the second half
+        const int a_src = t + 2 < T ? t + 2 : T - 1;
+        if constexpr (PAIR) {
+            const int pair = (t & 1) ? (t + 3) >> 1 : (t + 2) >> 1;
+            slice_step(I1{}, t + 1, a_src, t & 1, pair < TB ? pair : TB - 1, pair & 1, (t & 1) ? 0 : 1);
+        } else {
+            slice_step(I1{}, t + 1, a_src, t & 1, a_src, t & 1, 0);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the re-fetches of the last stages are still writing LDS
+    mfma_results_settle();                      // the accumulators are read next
+    __syncthreads();
+
+    char *patch = smem + wave * (16 * (TN * 16 * 4 + 16));
+    out_t *Cb = C + batch * (long)g.M * g.N;
+    EpiPrepared<Out<Cfg::OUT>::DT, 16 / (int)sizeof(out_t)> steps{};
+    if (g.epi.n != 0) steps = band_columns_prepare<Cfg::OUT, TN, 16>(g.epi, n0 + wave_n * TN * 16, lane, g.N);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+        store_band_via_lds<Cfg::OUT, TN, true, acc_t, 16, true>(patch, Cb, acc[i], m0 + (wave_m * TM + i) * 16, n0 + wave_n * TN * 16, lane,
+                                                                g.M, g.N, g.epi, steps);
+}
+
 template <class Cfg> int launch_pipe16_f8w(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
     auto kernel = mfma_pipe16_f8w_kernel<Cfg>;
+    static_assert(Cfg::NW * 16 * ((Cfg::BN / Cfg::WN) * 4 + 16) <= Cfg::LDS_BYTES, "the epilogue's patches fit the ring");
+    if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
+    const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;
+    const long total = g.batches * tiles_m * tiles_n;
+    if (total > 0x7FFFFFFFL) return fail(HODU_ROCM_UNSUPPORTED, "product needs %ld workgroups", total);
+    if (g.K <= 0 || g.K % (Cfg::B_PAIR ? 128 : 64) != 0) return fail(HODU_ROCM_UNSUPPORTED, "K is not a whole number of stages");
+    hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, ctx->stream, (const char *)a, (const char *)b,
+                       (typename Out<Cfg::OUT>::T *)c, g, tiles_m, tiles_n);
+    HODU_HIP(hipGetLastError());
+    return HODU_ROCM_OK;
+}
+
+template <class Cfg> int launch_pipe16r_f8w(hodu_rocm_ctx *ctx, const void *a, const void *b, void *c, const DevProduct &g) {
+    auto kernel = mfma_pipe16r_f8w_kernel<Cfg>;
     static_assert(Cfg::NW * 16 * ((Cfg::BN / Cfg::WN) * 4 + 16) <= Cfg::LDS_BYTES, "the epilogue's patches fit the ring");
     if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES)) return rc;
     const int tiles_m = (g.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (g.N + Cfg::BN - 1) / Cfg::BN;

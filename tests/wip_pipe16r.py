@@ -69,3 +69,23 @@ def test_respaced_is_exact_on_exact_operands(ctx):
         run_exact(ctx, "dot", "bf16", V([4096, 128]), V([128, 4096]), 12, "mfma_bf16_pipe256x256mi16_KM_r")
     finally:
         ctx.force_tile(-1)
+
+
+def test_respaced_f8_weight_tile_is_exact(ctx):
+    """mfma_pipe16r_f8w_kernel: the shapes of test_16x16_instruction_tile_with_f8_weights_is_exact"""
+    name = "mfma_bf16_f8w_pipe256x256mi16_KK_r"
+    ctx.force_tile(16)
+    try:
+        for k in (128, 256, 384, 1024, 2304):
+            run_exact(ctx, "dot", "bf16_f8e4m3w", V([296, k]), V([384, k]).t(), k, name)
+        run_exact(ctx, "dot", "bf16_f8e4m3w", V([17, 256]), V([5, 256]).t(), 5, name)
+        run_exact(ctx, "matmul", "bf16_f8e4m3w", V([2, 160, 512]), V([520, 512]).t().broadcast_to([2, 512, 520]), 6, name)
+        km = name.replace("_KK_r", "_KM_r")  # row-dense weights
+        for k in (64, 192, 1024):
+            run_exact(ctx, "dot", "bf16_f8e4m3w", V([296, k]), V([k, 384]), k + 1, km)
+        run_exact(ctx, "matmul", "bf16_f8e4m3w", V([2, 160, 512]), V([512, 528]).broadcast_to([2, 512, 528]), 7, km)
+        run_exact(ctx, "dot", "bf16_f8e4m3w", V([4096, 256]), V([4096, 256]).t(), 8, name)
+        # N(0,1) data against the comparator as well
+        check_product(ctx, "dot", "bf16_f8e4m3w", V([1000, 1024]), V([777, 1024]).t(), seed=8, rscale=2.0, expect_kernel=name)
+    finally:
+        ctx.force_tile(-1)
