@@ -10,6 +10,29 @@
 namespace hodu {
 namespace mfma {
 
+// The 256 x 256 tile on the 16 x 16 x 32 instruction (both generations, four layout pairs, two 16-bit types) is compiled
+// in translation units of its own, gemm_mfma_mi16_{bf16,f16}.hip, so that the build's longest compile stays short:
+// everywhere else these launchers are only declared.
+#ifdef HODU_MI16_DEFINE_HERE
+#define HODU_MI16_LINKAGE
+#else
+#define HODU_MI16_LINKAGE extern
+#endif
+#define HODU_MI16_ONE(CK, OUT, LA, LB)                                                                                     \
+    HODU_MI16_LINKAGE template int launch_pipe16<PipeConfig<CK, OUT, 256, 256, 2, 2, LA, LB, SK_SAME, 2>>(                   \
+        hodu_rocm_ctx *, const void *, const void *, void *, const DevProduct &);                                            \
+    HODU_MI16_LINKAGE template int launch_pipe16r<PipeConfig<CK, OUT, 256, 256, 2, 2, LA, LB, SK_SAME, 2>>(                  \
+        hodu_rocm_ctx *, const void *, const void *, void *, const DevProduct &);
+#define HODU_MI16_ALL(CK, OUT)                                                                                             \
+    HODU_MI16_ONE(CK, OUT, LM_K, LM_K) HODU_MI16_ONE(CK, OUT, LM_K, LM_MN) HODU_MI16_ONE(CK, OUT, LM_MN, LM_K)               \
+    HODU_MI16_ONE(CK, OUT, LM_MN, LM_MN)
+#if !defined(HODU_MI16_DEFINE_HERE) || HODU_MI16_DEFINE_HERE == 0
+HODU_MI16_ALL(CK_BF16, OUT_BF16)
+#endif
+#if !defined(HODU_MI16_DEFINE_HERE) || HODU_MI16_DEFINE_HERE == 1
+HODU_MI16_ALL(CK_F16, OUT_F16)
+#endif
+
 // One compute kind: {KK, KM, MK, MM} x {256x256 with 4 wavefronts, 128x128, 64x64}, {KK, KM} x 256x256
 // with 8 wavefronts, a scalar-load 64x64 kernel, and -- when both operands are stored in the compute
 // type -- the software-pipelined kernels of gemm_mfma_pipe.hpp: KK at four tile shapes and, for the
