@@ -1,5 +1,5 @@
 //! An owning handle on one device's library context, and device buffers that free themselves.
-use crate::error::{Result, RocmKernelError};
+use crate::error::{Result, RocmKernelError, Status};
 use crate::ffi;
 use core::ffi::{c_int, c_void};
 use std::ffi::CStr;
@@ -19,7 +19,7 @@ impl Context {
         let mut raw = core::ptr::null_mut();
         let rc = unsafe { ffi::hodu_rocm_ctx_create(device as c_int, &mut raw) };
         if rc != ffi::HODU_ROCM_OK || raw.is_null() {
-            return Err(RocmKernelError::LaunchError(format!("hodu_rocm_ctx_create({device}) failed with status {rc}")));
+            return Err(RocmKernelError::new(Status::from_code(rc), format!("hodu_rocm_ctx_create({device}) failed")));
         }
         Ok(Arc::new(Self { raw, device }))
     }
@@ -35,13 +35,7 @@ impl Context {
             let p = ffi::hodu_rocm_last_error(self.raw);
             if p.is_null() { String::new() } else { CStr::from_ptr(p).to_string_lossy().into_owned() }
         };
-        Err(match rc {
-            ffi::HODU_ROCM_INVALID_ARG => RocmKernelError::InvalidInput(msg),
-            ffi::HODU_ROCM_UNSUPPORTED => RocmKernelError::Unsupported(msg),
-            ffi::HODU_ROCM_HIP_ERROR => RocmKernelError::LaunchError(msg),
-            ffi::HODU_ROCM_OOM | ffi::HODU_ROCM_SCRATCH => RocmKernelError::MemoryError(msg),
-            _ => RocmKernelError::Message(format!("status {rc}: {msg}")),
-        })
+        Err(RocmKernelError::new(Status::from_code(rc), msg))
     }
 
     /// uninitialised device memory, like CpuDevice::allocate (crates/hodu_core/src/be_cpu/device.rs:19-24): a kernel

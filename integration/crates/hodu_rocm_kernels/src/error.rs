@@ -1,32 +1,54 @@
-//! Error type of the ROCm kernel crate (same shape as CudaKernelError, crates/hodu_cuda_kernels/src/error.rs:7-18).
-use std::fmt;
+//! What a failed call of the kernel library looks like on the Rust side: the library's status code and the message it
+//! left for the calling thread (`hodu_rocm_last_error`).  hodu_core turns it into `HoduError::RocmKernelError(String)`.
+use core::ffi::c_int;
 
-#[derive(Debug, Clone)]
-pub enum RocmKernelError {
-    /// no kernel of that name
-    InvalidKernel(String),
-    /// HODU_ROCM_INVALID_ARG: bad metadata or arguments
-    InvalidInput(String),
-    /// HODU_ROCM_UNSUPPORTED: no kernel takes the request (the caller may fall back)
-    Unsupported(String),
-    /// HODU_ROCM_HIP_ERROR: a HIP call failed
-    LaunchError(String),
-    /// HODU_ROCM_OOM, or HODU_ROCM_SCRATCH (internal scratch could not be obtained)
-    MemoryError(String),
-    Message(String),
+/// the status codes of include/hodu_rocm_kernels.h, plus one for a kernel name this crate does not know
+#[derive(Debug, Clone, Copy, PartialEq, Eq)]
+pub enum Status {
+    InvalidArg,
+    /// no kernel takes the request: the caller may fall back (e.g. attention -> three launches)
+    Unsupported,
+    Hip,
+    OutOfMemory,
+    /// internal scratch could not be obtained (stream under capture, or the no-alloc entry point beyond its limit)
+    Scratch,
+    UnknownKernel,
+    Other(c_int),
 }
 
-impl fmt::Display for RocmKernelError {
-    fn fmt(&self, f: &mut fmt::Formatter<'_>) -> fmt::Result {
-        match self {
-            Self::InvalidKernel(m) => write!(f, "invalid kernel: {m}"),
-            Self::InvalidInput(m) => write!(f, "invalid input: {m}"),
-            Self::Unsupported(m) => write!(f, "unsupported: {m}"),
-            Self::LaunchError(m) => write!(f, "launch error: {m}"),
-            Self::MemoryError(m) => write!(f, "memory error: {m}"),
-            Self::Message(m) => write!(f, "{m}"),
+impl Status {
+    pub fn from_code(rc: c_int) -> Self {
+        match rc {
+            1 => Status::InvalidArg,
+            2 => Status::Unsupported,
+            3 => Status::Hip,
+            4 => Status::OutOfMemory,
+            5 => Status::Scratch,
+            other => Status::Other(other),
         }
     }
 }
+
+#[derive(Debug, Clone)]
+pub struct RocmKernelError {
+    pub status: Status,
+    pub message: String,
+}
+
+impl RocmKernelError {
+    pub fn new(status: Status, message: impl Into<String>) -> Self {
+        Self { status, message: message.into() }
+    }
+    pub fn is_unsupported(&self) -> bool {
+        self.status == Status::Unsupported
+    }
+}
+
+impl core::fmt::Display for RocmKernelError {
+    fn fmt(&self, f: &mut core::fmt::Formatter<'_>) -> core::fmt::Result {
+        write!(f, "hodu_rocm_kernels [{:?}]: {}", self.status, self.message)
+    }
+}
 impl std::error::Error for RocmKernelError {}
-pub type Result<T> = std::result::Result<T, RocmKernelError>;
+
+pub type Result<T> = core::result::Result<T, RocmKernelError>;

@@ -2,7 +2,7 @@
 //! (crates/hodu_cpu_kernels/src/kernels/ops_matrix.rs:56-68, :102-114; ops_cast.rs:70-81): a `Kernel` is a static
 //! name "hodu_rocm_<op>_<dtype>", the metadata is hodu's `&[usize]`, a non-zero status becomes an error.
 use crate::context::{Context, DeviceBuf};
-use crate::error::{Result, RocmKernelError};
+use crate::error::{Result, RocmKernelError, Status};
 use crate::ffi::{self, ProductExFn, ProductFn};
 use core::ffi::c_int;
 
@@ -65,10 +65,10 @@ product_ex_table!(dot; bf16, f16, f32, f64, u8, u16, u32, u64, i8, i16, i32, i64
 fn run_product(ctx: &Context, plain: Option<ProductFn>, ex: Option<ProductExFn>, kernel: Kernel, lhs: &DeviceBuf,
                rhs: &DeviceBuf, out: &DeviceBuf, metadata: &[usize], steps: &[ffi::hodu_rocm_epilogue_step]) -> Result<()> {
     let rc = if steps.is_empty() {
-        let f = plain.ok_or_else(|| RocmKernelError::InvalidKernel(kernel.0.to_string()))?;
+        let f = plain.ok_or_else(|| RocmKernelError::new(Status::UnknownKernel, kernel.0))?;
         unsafe { f(ctx.raw(), lhs.as_ptr(), rhs.as_ptr(), out.as_mut_ptr(), metadata.as_ptr(), metadata.len()) }
     } else {
-        let f = ex.ok_or_else(|| RocmKernelError::InvalidKernel(format!("{} takes no fused steps", kernel.0)))?;
+        let f = ex.ok_or_else(|| RocmKernelError::new(Status::UnknownKernel, format!("{} takes no fused steps", kernel.0)))?;
         unsafe { f(ctx.raw(), lhs.as_ptr(), rhs.as_ptr(), out.as_mut_ptr(), metadata.as_ptr(), metadata.len(), steps.as_ptr(), steps.len()) }
     };
     ctx.check(rc)

@@ -7,4 +7,4 @@ pub mod ffi;
 pub mod kernels;
 
 pub use context::{Context, DeviceBuf};
-pub use error::{Result, RocmKernelError};
+pub use error::{Result, RocmKernelError, Status};
