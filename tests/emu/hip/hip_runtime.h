@@ -1,0 +1,159 @@
+// Test infrastructure, not a HIP runtime: a CPU stand-in for the few pieces of <hip/hip_runtime.h> that the plain
+// (no matrix-core, no LDS-DMA) kernels of hodu_amd/csrc use, so that a kernel's UNMODIFIED source can be compiled
+// for the host and run there -- a CPU build for checking indexing, masks and reductions without a GPU.
+//
+// Execution model: a launch runs its workgroups one after the other; the threads of a workgroup are real host
+// threads (so __shared__ can be a plain static), grouped into wavefronts of 64 whose cross-lane operations
+// (__shfl_xor) exchange through a per-wavefront buffer between two barriers.  Arithmetic is the host's: expf / exp
+// are libm's, bf16 / f16 conversions the host compiler's (round to nearest even), so results agree with the device
+// to rounding, not to the bit.  Nothing here knows about MFMA, DPP, LDS-DMA or buffer instructions.
+#pragma once
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <condition_variable>
+#include <cstring>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+#define __global__
+#define __device__
+#define __host__
+#define __forceinline__ inline __attribute__((always_inline))
+#define __launch_bounds__(...)
+#define __shared__ static
+
+struct dim3 {
+    unsigned x, y, z;
+    dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+struct emu_uint3 { unsigned x = 0, y = 0, z = 0; };
+
+typedef void *hipStream_t;
+typedef int hipError_t;
+constexpr hipError_t hipSuccess = 0, hipErrorOutOfMemory = 2;
+struct hipDeviceProp_t { int multiProcessorCount = 256; };
+inline hipError_t hipGetLastError() { return hipSuccess; }
+inline hipError_t hipSetDevice(int) { return hipSuccess; }
+inline const char *hipGetErrorString(hipError_t) { return "emulated"; }
+enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize = 8 };
+inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { return hipSuccess; }
+
+namespace emu {
+constexpr int kWave = 64, kMaxBlock = 1024;
+
+// a barrier whose parties may leave for good: a thread that returns from the kernel no longer counts, as on the GPU
+class Barrier {
+public:
+    void reset(unsigned parties) { parties_ = parties; waiting_ = 0; phase_ = 0; }
+    void wait() {
+        std::unique_lock<std::mutex> hold(mu_);
+        const unsigned my = phase_;
+        if (++waiting_ >= parties_) {
+            waiting_ = 0;
+            phase_++;
+            cv_.notify_all();
+            return;
+        }
+        cv_.wait(hold, [&] { return phase_ != my; });
+    }
+    void leave() {
+        std::unique_lock<std::mutex> hold(mu_);
+        parties_--;
+        if (parties_ > 0 && waiting_ >= parties_) {
+            waiting_ = 0;
+            phase_++;
+            cv_.notify_all();
+        }
+    }
+private:
+    std::mutex mu_;
+    std::condition_variable cv_;
+    unsigned parties_ = 0, waiting_ = 0, phase_ = 0;
+};
+
+struct Block {
+    Barrier all;                       // __syncthreads
+    Barrier wave[kMaxBlock / kWave];   // cross-lane exchanges
+    alignas(16) unsigned char xchg[kMaxBlock / kWave][kWave][16];
+};
+inline Block *&current() { static Block *b = nullptr; return b; }
+inline thread_local emu_uint3 t_idx, b_idx, b_dim, g_dim;
+
+template <class K, class... Args> void launch(K kernel, dim3 grid, dim3 block, Args... args) {
+    const unsigned nthreads = block.x * block.y * block.z;
+    if (nthreads == 0 || nthreads > (unsigned)kMaxBlock || nthreads % kWave != 0) {
+        fprintf(stderr, "emu: a workgroup of %u threads is not whole wavefronts\n", nthreads);
+        abort();
+    }
+    Block blk;
+    current() = &blk;
+    for (unsigned bz = 0; bz < grid.z; bz++)
+        for (unsigned by = 0; by < grid.y; by++)
+            for (unsigned bx = 0; bx < grid.x; bx++) {
+                blk.all.reset(nthreads);
+                for (unsigned w = 0; w < nthreads / kWave; w++) blk.wave[w].reset(kWave);
+                std::vector<std::thread> pool;
+                pool.reserve(nthreads);
+                for (unsigned t = 0; t < nthreads; t++)
+                    pool.emplace_back([=, &blk] {
+                        t_idx.x = t % block.x; t_idx.y = (t / block.x) % block.y; t_idx.z = t / (block.x * block.y);
+                        b_idx.x = bx; b_idx.y = by; b_idx.z = bz;
+                        b_dim.x = block.x; b_dim.y = block.y; b_dim.z = block.z;
+                        g_dim.x = grid.x; g_dim.y = grid.y; g_dim.z = grid.z;
+                        kernel(args...);
+                        blk.wave[t / kWave].leave();
+                        blk.all.leave();
+                    });
+                for (auto &th : pool) th.join();
+            }
+    current() = nullptr;
+}
+inline unsigned flat_tid() { return t_idx.x + b_dim.x * (t_idx.y + b_dim.y * t_idx.z); }
+}  // namespace emu
+
+#define threadIdx (emu::t_idx)
+#define blockIdx (emu::b_idx)
+#define blockDim (emu::b_dim)
+#define gridDim (emu::g_dim)
+// the parenthesised kernel name of a template instantiation arrives as one macro argument
+#define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) emu::launch(kernel, grid, block, __VA_ARGS__)
+
+inline void __syncthreads() { emu::current()->all.wait(); }
+
+// every lane of the wavefront that is still running calls it; a lane that has returned from the kernel is not waited
+// for (its slot keeps what it wrote last)
+template <class T> inline T __shfl_xor(T v, int lane_mask, int width = 64) {
+    static_assert(sizeof(T) <= 16, "exchange slot");
+    (void)width;
+    emu::Block *b = emu::current();
+    const unsigned tid = emu::flat_tid(), w = tid / emu::kWave, lane = tid % emu::kWave;
+    memcpy(b->xchg[w][lane], &v, sizeof(T));
+    b->wave[w].wait();
+    T out;
+    memcpy(&out, b->xchg[w][(lane ^ (unsigned)lane_mask) % emu::kWave], sizeof(T));
+    b->wave[w].wait();
+    return out;
+}
+
+// HIP's device headers put the classification functions at global scope
+using std::isinf;
+using std::isnan;
+using std::isfinite;
+
+inline float __uint_as_float(unsigned u) { float f; memcpy(&f, &u, 4); return f; }
+inline unsigned __float_as_uint(float f) { unsigned u; memcpy(&u, &f, 4); return u; }
+
+// The conversion and median builtins of gfx950 that the shared headers mention (the 8-bit float conversions): no CPU
+// stand-in -- a kernel that reaches one counts it here and goes on with zeros, and the test that ran it fails on the count.
+namespace emu {
+inline int &no_such_instruction_hits() { static int n = 0; return n; }
+inline int no_such_instruction() { return ++no_such_instruction_hits(); }
+}  // namespace emu
+#define __builtin_amdgcn_cvt_f32_fp8(a, b) ((void)emu::no_such_instruction(), 0.f)
+#define __builtin_amdgcn_cvt_f32_bf8(a, b) ((void)emu::no_such_instruction(), 0.f)
+#define __builtin_amdgcn_cvt_pk_fp8_f32(a, b, c, d) ((void)emu::no_such_instruction(), 0)
+#define __builtin_amdgcn_cvt_pk_bf8_f32(a, b, c, d) ((void)emu::no_such_instruction(), 0)
+#define __builtin_amdgcn_fmed3f(a, b, c) ((void)emu::no_such_instruction(), 0.f)
