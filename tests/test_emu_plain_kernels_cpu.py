@@ -131,3 +131,44 @@ def test_generic_product_floats_and_fused_cast_entries(emu):
     got = np.zeros(45 * 33, dtype=np.int32)
     emu.product("dot", "i32_i8i8", a8, b8, got, md)
     assert np.array_equal(got, oracle.dot_asis("i32", a8.astype(np.int32), b8.astype(np.int32), md))
+
+
+def test_reference_known_answers_and_edge_shapes(emu):
+    """the reference's own known-answer tests (crates/hodu_cpu_kernels/tests/ops_matrix.rs:8-147) through the entry
+    points of the CPU build; K = 0 writes zeros; an empty output writes nothing"""
+    a = np.arange(1, 7, dtype=np.float32)
+    b = np.arange(7, 13, dtype=np.float32)
+    out = np.zeros(4, np.float32)
+    emu.product("dot", "f32", a, b, out, [2, 3, 2, 3, 1, 2, 1, 0, 0])
+    assert out.tolist() == [58, 64, 139, 154]
+    out = np.zeros(4, np.float32)
+    emu.product("matmul", "f32", a, b, out, [4, 2, 2, 0, 2, 3, 3, 2, 3, 1, 2, 1, 0, 0, 2, 3, 2])
+    assert out.tolist() == [58, 64, 139, 154]
+    out = np.full(35, 7, np.int32)
+    emu.product("dot", "i32", np.zeros(1, np.int32), np.zeros(1, np.int32), out, [5, 0, 7, 0, 1, 7, 1, 0, 0])
+    assert np.all(out == 0)
+    keep = np.full(1, 0x5A5A5A5A, np.uint32)
+    ones = np.ones(16, np.float32)
+    for md in ([0, 4, 3, 4, 1, 3, 1, 0, 0], [3, 4, 0, 4, 1, 1, 1, 0, 0]):
+        emu.product("dot", "f32", ones, ones, keep.view(np.float32), md)
+    emu.product("matmul", "f32", ones, ones, keep.view(np.float32), [0, 3, 3, 1, 0, 2, 4, 0, 4, 2, 0, 8, 4, 1, 8, 2, 1, 0, 0, 2, 4, 2])
+    assert keep[0] == 0x5A5A5A5A
+
+
+def test_errors_are_status_codes_not_launches(emu):
+    a, b, o = np.zeros(16, np.float32), np.zeros(16, np.float32), np.zeros(16, np.float32)
+    bad = [
+        ("dot", a, b, o, [2, 3, 2, 3, 1, 2, 1, 0]),                                     # 8 words
+        ("matmul", a, b, o, [4, 2, 2, 0, 2, 3, 4, 2, 3, 1, 2, 1, 0, 0, 2, 3, 2]),       # K mismatch
+        ("matmul", a, b, o, [4, 1, 2, 0, 3, 3, 2, 1, 2, 1, 0, 0, 2, 3, 2]),             # 1-D operand
+        ("matmul", a, b, o, [5, 2, 2, 0, 2, 3, 3, 2, 3, 1, 2, 1, 0, 0, 2, 3, 2]),       # num_els inconsistent
+        ("dot", a, b, a, [2, 3, 2, 3, 1, 2, 1, 0, 0]),                                  # out aliases an input
+    ]
+    for op, x, y, out, md in bad:
+        with pytest.raises(RuntimeError, match="status 1"):
+            emu.product(op, "f32", x, y, out, md)
+    with pytest.raises(RuntimeError, match="status 1"):
+        emu.cast("f32", "bf16", a, o.view(np.uint16), [4, 1, 5, 1, 0])                  # num_els != prod(shape)
+    with pytest.raises(RuntimeError, match="status 2"):
+        emu._check(emu.lib.hodu_rocm_cast(emu.ctx, 99, 3, a.ctypes.data, o.ctypes.data, *emu._md([4, 1, 4, 1, 0])), "cast")
+    emu.product("dot", "f32", a, b, o, [2, 3, 2, 3, 1, 2, 1, 0, 0])                     # the context is still usable
