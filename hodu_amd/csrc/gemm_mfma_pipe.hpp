@@ -47,6 +47,7 @@
 
 #include "agent_scope.hpp"
 #include "gemm_mfma.hpp"
+#include "gfx950_insn.hpp"
 
 // Measurement builds only (never the library's): HODU_PIPE_STAMPS makes every workgroup record the 100 MHz
 // real-time counter at a few points into the buffer whose address the third fused-step slot carries.
@@ -120,30 +121,13 @@ struct PipeConfig {
                   "row-dense operands: 8- and 16-bit types, tiles of at least 128 rows");
 };
 
-// Kernels that write their MFMAs out in assembly hide them from the compiler's hazard recogniser, which therefore
-// inserts nothing between the last matrix instruction and the first read of an accumulator behind the loop.  The
-// hardware wants idle wait states there -- up to 18 when a 16-pass instruction's result is read by a vector
-// instruction, fewer for the 4- and 8-pass instructions used here -- and does not interlock: these are they.
-__device__ __forceinline__ void mfma_results_settle() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
-
-// issued through inline assembly so that the compiler's own wait-count bookkeeping (which would put
-// an s_waitcnt vmcnt(0) in front of the next LDS read) stays out of the way; completion is awaited
-// explicitly before the barrier that publishes the stage
-__device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
-}
-
-// The same with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit byte offset per
-// lane: the form whose per-instruction cost is one M0 write -- no vector arithmetic, no readfirstlane.
-// (a pointer the compiler can hold in scalar registers: both halves through readfirstlane, which is free for a value
-// that already is uniform and makes the "s" constraints below hold where the uniformity analysis gives up)
+// A pointer the compiler can hold in scalar registers (the base of dma16_sbase / dma16_imm): both halves through
+// readfirstlane, which is free for a value that already is uniform and makes the "s" constraints of those
+// instructions hold where the uniformity analysis gives up.
 __device__ __forceinline__ const char *uniform_ptr(const char *p) {
     const unsigned long long v = (unsigned long long)(uintptr_t)p;
     const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
     return (const char *)(uintptr_t)(((unsigned long long)hi << 32) | lo);
-}
-__device__ __forceinline__ void dma16_sbase(const char *sbase, unsigned voff, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 
 // 64 bits per lane through the LDS transpose.  Of the 16 lanes that execute together, lane s supplies the

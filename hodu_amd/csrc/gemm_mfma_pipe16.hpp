@@ -26,8 +26,6 @@
 namespace hodu {
 namespace mfma {
 
-typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
-
 // f(integral_constant<int, 0>) .. f(integral_constant<int, N - 1>), in order: a loop whose index is a constant expression
 template <int N, int I = 0, class F> __device__ __forceinline__ void static_for(F &&f) {
     if constexpr (I < N) {
@@ -36,22 +34,18 @@ template <int N, int I = 0, class F> __device__ __forceinline__ void static_for(
     }
 }
 
-// The instruction is written out with the accumulator tied to itself and held in the accumulation registers: left to
-// the register allocator, a kernel with 64 four-register accumulators and 128 fragment registers came out with the
-// accumulators rotating through copies inside the loop (twice the time).  What the compiler then no longer knows about
-// the instruction: an accumulator is next touched 64 MFMAs later (or, behind the loop, after a barrier), and its other
-// operands come from LDS reads the compiler waits for as for any use of a register.
+// (the instruction itself, with its accumulator tied: gfx950_insn.hpp)
 template <int CK> struct Compute16;
 template <> struct Compute16<CK_BF16> {
     typedef f32x4_acc_t acc_t;
     static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        mfma16x16x32_bf16(a, b, c);
     }
 };
 template <> struct Compute16<CK_F16> {
     typedef f32x4_acc_t acc_t;
     static __device__ __forceinline__ void mma(const u32x4_t &a, const u32x4_t &b, acc_t &c) {
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        mfma16x16x32_f16(a, b, c);
     }
 };
 
@@ -299,15 +293,6 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
 //   * the source pointers advance by one add per operand and stage; the last two stages, which fetch nothing, are
 //     a copy of the loop body without the DMA list instead of re-fetching a clamped stage.
 // Needs an even number of stages (K a multiple of 128 elements), at least two; anything else takes the first kernel.
-template <int IMM> __device__ __forceinline__ void dma16_imm(const char *sbase, unsigned voff) {
-    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(voff), "s"(sbase), "n"(IMM) : "memory");
-}
-// M0 = base + literal.  M0 stays as written until the next call: nothing else in these loops reads or writes it (LDS
-// reads need no M0 on this target), and at least the MFMA that follows separates the write from the DMA that uses it.
-template <int LIT> __device__ __forceinline__ void m0_set(unsigned base) {
-    asm volatile("s_add_u32 m0, %0, %1" ::"s"(base), "n"(LIT) : "scc");
-}
-
 // an even number of 128-byte stages, at least two
 inline bool pipe16r_stages_ok(long K, int elem_bytes) { return K > 0 && (K * elem_bytes) % (2 * P_ROW_BYTES) == 0; }
 
@@ -495,7 +480,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_kernel(const char *__res
             constexpr int d = decltype(d_)::value;
             if constexpr (d % GRP == 0) {
                 dma_m0(j_, d_);
-                asm volatile("s_nop 0");
+                m0_wait_state();
             }
             dma_element(j_, d_);
         });
@@ -980,14 +965,14 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_f8w_kernel(const char *_
             constexpr int E = decltype(e_)::value;
             if constexpr (E % GRP == 0) {
                 m0_a(std::integral_constant<int, E / GRP>{}, slot);
-                asm volatile("s_nop 0");
+                m0_wait_state();
             }
             dma_a(e_, src);
         });
     };
     auto fetch_b = [&](int src, int buf, int half) {
         m0_b(buf, half);
-        asm volatile("s_nop 0");
+        m0_wait_state();
         static_for<PBS>([&](auto e_) { dma_b(e_, src, half); });
     };
     fetch_a(0, 0);

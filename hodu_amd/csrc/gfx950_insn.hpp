@@ -1,0 +1,65 @@
+// The gfx950 instructions these kernels write out in assembly, one small function each: the matrix instruction with
+// a tied accumulator, the LDS-DMA load in its three addressing forms, the M0 writes that go with it, and the wait
+// states the hardware wants and the compiler cannot insert for instructions it does not see.
+//
+// Kept apart from the kernels so that a CPU build of the kernels for tests (tests/emu) can put stand-ins with the
+// same names in their place: it defines HODU_GFX950_INSN_PROVIDED before this file is reached.  The product never
+// does.
+#pragma once
+#ifndef HODU_GFX950_INSN_PROVIDED
+
+#include "device_types.hpp"
+
+namespace hodu {
+namespace mfma {
+
+typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
+
+// v_mfma_f32_16x16x32_{bf16,f16} with the accumulator tied to itself and held in the accumulation registers: left to
+// the register allocator, a kernel with 64 four-register accumulators and 128 fragment registers came out with the
+// accumulators rotating through copies inside the loop (twice the time).  What the compiler then no longer knows about
+// the instruction: an accumulator is next touched 64 MFMAs later (or, behind the loop, after a barrier), and its other
+// operands come from LDS reads the compiler waits for as for any use of a register.
+__device__ __forceinline__ void mfma16x16x32_bf16(const u32x4_t &a, const u32x4_t &b, f32x4_acc_t &c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma16x16x32_f16(const u32x4_t &a, const u32x4_t &b, f32x4_acc_t &c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+// Kernels that write their MFMAs out in assembly hide them from the compiler's hazard recogniser, which therefore
+// inserts nothing between the last matrix instruction and the first read of an accumulator behind the loop.  The
+// hardware wants idle wait states there -- up to 18 when a 16-pass instruction's result is read by a vector
+// instruction, fewer for the 4- and 8-pass instructions used here -- and does not interlock: these are they.
+__device__ __forceinline__ void mfma_results_settle() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
+
+// LDS-DMA: 16 bytes per lane from global memory straight into LDS at M0 + lane * 16 (+ the immediate offset, which
+// moves the global and the LDS address alike).  Issued through inline assembly so that the compiler's own wait-count
+// bookkeeping (which would put an s_waitcnt vmcnt(0) in front of the next LDS read) stays out of the way; completion
+// is awaited explicitly before the barrier that publishes the stage.
+//   dma16_raw    a full 64-bit address per lane
+//   dma16_sbase  a wave-uniform 64-bit base (scalar registers) + a 32-bit byte offset per lane: the form whose
+//                per-instruction cost is one M0 write -- no vector arithmetic, no readfirstlane
+//   dma16_imm    the same with M0 written beforehand (m0_set) and an immediate offset, so that one M0 value serves
+//                several instructions
+__device__ __forceinline__ void dma16_raw(const char *gptr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void dma16_sbase(const char *sbase, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+template <int IMM> __device__ __forceinline__ void dma16_imm(const char *sbase, unsigned voff) {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(voff), "s"(sbase), "n"(IMM) : "memory");
+}
+// M0 = base + literal.  M0 stays as written until the next call: nothing else in these loops reads or writes it (LDS
+// reads need no M0 on this target).  An instruction has to separate the write from the DMA that uses it: the MFMA
+// that follows in a loop, m0_wait_state() where there is none.
+template <int LIT> __device__ __forceinline__ void m0_set(unsigned base) {
+    asm volatile("s_add_u32 m0, %0, %1" ::"s"(base), "n"(LIT) : "scc");
+}
+__device__ __forceinline__ void m0_wait_state() { asm volatile("s_nop 0"); }
+
+}  // namespace mfma
+}  // namespace hodu
+
+#endif  // HODU_GFX950_INSN_PROVIDED
