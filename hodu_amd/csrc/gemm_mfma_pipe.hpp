@@ -224,7 +224,7 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
     }
     // the same wavefront reads what it wrote: the LDS operations of one wavefront complete in order, and the
     // compiler is told not to move the differently-typed accesses across each other
-    asm volatile("" ::: "memory");
+    wave_lds_fence();
     const bool vec_ok = ((long)N * OS) % 16 == 0;
     // the fused element-wise steps work on the rounded values, here where a lane holds EPV neighbouring columns
     // of one row -- the same columns in every pass, so what the steps need for them is fetched once
@@ -292,7 +292,7 @@ __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT
 #pragma unroll
         for (int pass = 0; pass < TS / RPP; pass++) store_chunk(pass, patch_chunk(pass));
     }
-    asm volatile("" ::: "memory");  // the next band overwrites the patch
+    wave_lds_fence();  // the next band overwrites the patch
 }
 template <int OUT, int TN, bool EPI, class acc_t, int TS = 32>
 __device__ __forceinline__ void store_band_via_lds(char *patch, typename Out<OUT>::T *Cb, const acc_t (&acc)[TN], int m_base,

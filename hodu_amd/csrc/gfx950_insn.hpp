@@ -59,6 +59,11 @@ template <int LIT> __device__ __forceinline__ void m0_set(unsigned base) {
 }
 __device__ __forceinline__ void m0_wait_state() { asm volatile("s_nop 0"); }
 
+// Between a wavefront's LDS writes and its own reads of what other lanes of it wrote (or the other way round): the
+// lanes of a wavefront execute together and one wavefront's LDS operations complete in order, so no instruction is
+// needed -- only the compiler must not move the accesses across this point.
+__device__ __forceinline__ void wave_lds_fence() { asm volatile("" ::: "memory"); }
+
 }  // namespace mfma
 }  // namespace hodu
 

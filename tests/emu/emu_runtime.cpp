@@ -33,11 +33,31 @@ int ensure_workspace(hodu_rocm_ctx *ctx, size_t bytes) {
     ctx->workspace.bytes = ctx->workspace.ptr ? bytes : 0;
     return ctx->workspace.ptr ? HODU_ROCM_OK : fail(HODU_ROCM_OOM, "workspace of %zu bytes", bytes);
 }
+#ifdef EMU_WITH_MFMA
+int ensure_arrival(hodu_rocm_ctx *ctx) {
+    if (!ctx->arrival) ctx->arrival = (int *)calloc(kArrivalSlots, sizeof(int));
+    if (ctx->arrival && ctx->arrival_stale) memset(ctx->arrival, 0, kArrivalSlots * sizeof(int));
+    ctx->arrival_stale = false;
+    return ctx->arrival ? HODU_ROCM_OK : fail(HODU_ROCM_OOM, "arrival counters");
+}
+#else
 int ensure_arrival(hodu_rocm_ctx *) { return fail(HODU_ROCM_UNSUPPORTED, "no arrival counters in the CPU build"); }
+#endif
 
 #define NO_CPU_BUILD(name) \
     int name(hodu_rocm_ctx *, int, int, const void *, const void *, void *, const DevProduct &) { return HODU_ROCM_UNSUPPORTED; }
+#ifndef EMU_WITH_MFMA
 NO_CPU_BUILD(launch_mfma)
+#else
+// the tile kernels of the 16-bit types and of f8e4m3 weights are built (gfx950_insn_emu.hpp); the other kinds are not
+#define NO_CPU_BUILD_KIND(name) \
+    int name(hodu_rocm_ctx *, const void *, const void *, void *, const DevProduct &) { return HODU_ROCM_UNSUPPORTED; }
+NO_CPU_BUILD_KIND(launch_mfma_i8)
+NO_CPU_BUILD_KIND(launch_mfma_f32)
+NO_CPU_BUILD_KIND(launch_mfma_i8_out)
+NO_CPU_BUILD_KIND(launch_mfma_u8_out)
+int launch_mfma_f8(hodu_rocm_ctx *, int, const void *, const void *, void *, const DevProduct &) { return HODU_ROCM_UNSUPPORTED; }
+#endif
 NO_CPU_BUILD(launch_gemv)
 NO_CPU_BUILD(launch_small_f32)
 NO_CPU_BUILD(launch_gemm_f64)
@@ -48,14 +68,39 @@ int launch_attention(hodu_rocm_ctx *, int, const void *, const void *, const voi
 }
 }  // namespace hodu
 
+#ifdef EMU_WITH_MFMA
+// LDS of the workgroup that is running (workgroups run one at a time): what `extern __shared__ char smem[]` names in
+// the tile kernels, and the model of LDS-DMA arrival
+namespace hodu {
+namespace mfma {
+alignas(256) char smem[emu::kLdsBytes];
+}
+}  // namespace hodu
+namespace emu {
+char *lds_base() { return hodu::mfma::smem; }
+int &dma_lazy() { static int model = 0; return model; }
+}  // namespace emu
+extern "C" void emu_dma_lazy(int model) { emu::dma_lazy() = model; }
+// fills LDS with a pattern, so that a kernel that reads what it has not written does not find the last launch's data
+extern "C" void emu_lds_fill(int byte) { memset(hodu::mfma::smem, byte, sizeof(hodu::mfma::smem)); }
+#endif
+
 extern "C" {
 hodu_rocm_ctx *emu_ctx_create(void) { return new hodu_rocm_ctx; }
 void emu_ctx_destroy(hodu_rocm_ctx *ctx) {
-    if (ctx) free(ctx->workspace.ptr);
+    if (ctx) {
+        free(ctx->workspace.ptr);
+        free(ctx->arrival);
+    }
     delete ctx;
 }
 const char *emu_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+// the testing hooks of the debug library, which has no CPU build
+void emu_force_tile(hodu_rocm_ctx *ctx, int v) { ctx->force_tile = v; }
+void emu_force_splitk(hodu_rocm_ctx *ctx, int v) { ctx->force_splits = v; }
 const char *emu_last_error(void) { return hodu::get_error(); }
 // how often a kernel reached an instruction that has no CPU stand-in (must stay 0 for a result to mean anything)
 int emu_unsupported_hits(void) { return emu::no_such_instruction_hits(); }
+const char *emu_unsupported_first(void) { return emu::no_such_instruction_first(); }
+void emu_unsupported_reset(void) { emu::no_such_instruction_hits() = 0; }
 }

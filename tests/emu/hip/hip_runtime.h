@@ -6,7 +6,9 @@
 // threads (so __shared__ can be a plain static), grouped into wavefronts of 64 whose cross-lane operations
 // (__shfl_xor) exchange through a per-wavefront buffer between two barriers.  Arithmetic is the host's: expf / exp
 // are libm's, bf16 / f16 conversions the host compiler's (round to nearest even), so results agree with the device
-// to rounding, not to the bit.  Nothing here knows about MFMA, DPP, LDS-DMA or buffer instructions.
+// to rounding, not to the bit.  The 8-bit float conversions are written out below.  Nothing here knows about MFMA,
+// DPP, LDS-DMA or buffer instructions; stand-ins for
+// those the tile kernels use are in gfx950_insn_emu.hpp, for the translation units that want them.
 #pragma once
 
 #include <cmath>
@@ -23,7 +25,15 @@
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
+// A kernel's static __shared__ arrays become statics (workgroups run one at a time).  A translation unit whose kernels
+// use the dynamic array instead (`extern __shared__ char smem[]`) defines EMU_DYNAMIC_LDS: the declaration then names an
+// ordinary global the harness provides.
+#ifdef EMU_DYNAMIC_LDS
+#define __shared__
+#else
 #define __shared__ static
+#endif
+#define __align__(n) __attribute__((aligned(n)))
 
 struct dim3 {
     unsigned x, y, z;
@@ -78,6 +88,7 @@ struct Block {
     Barrier all;                       // __syncthreads
     Barrier wave[kMaxBlock / kWave];   // cross-lane exchanges
     alignas(16) unsigned char xchg[kMaxBlock / kWave][kWave][16];
+    alignas(16) unsigned char wide[2][kMaxBlock / kWave][kWave][64];  // operands of wavefront-wide instructions, two sets
 };
 inline Block *&current() { static Block *b = nullptr; return b; }
 inline thread_local emu_uint3 t_idx, b_idx, b_dim, g_dim;
@@ -146,14 +157,58 @@ using std::isfinite;
 inline float __uint_as_float(unsigned u) { float f; memcpy(&f, &u, 4); return f; }
 inline unsigned __float_as_uint(float f) { unsigned u; memcpy(&u, &f, 4); return u; }
 
-// The conversion and median builtins of gfx950 that the shared headers mention (the 8-bit float conversions): no CPU
-// stand-in -- a kernel that reaches one counts it here and goes on with zeros, and the test that ran it fails on the count.
+// An instruction without a CPU stand-in: a kernel that reaches one counts it here and goes on with zeros, and the test
+// that ran it fails on the count.
 namespace emu {
 inline int &no_such_instruction_hits() { static int n = 0; return n; }
-inline int no_such_instruction() { return ++no_such_instruction_hits(); }
+inline const char *&no_such_instruction_first() { static const char *what = ""; return what; }
+inline int no_such_instruction(const char *what = "?") {
+    if (no_such_instruction_hits() == 0) no_such_instruction_first() = what;
+    return ++no_such_instruction_hits();
+}
+
+// The 8-bit float conversions of gfx950 (OCP formats): e4m3 has no infinities and one NaN per sign (0x7F), e5m2 is
+// IEEE-like.  Narrowing rounds to nearest even; what lies beyond the largest finite value becomes NaN (e4m3) or
+// infinity (e5m2) -- the kernels clamp first, so that only matters for non-finite inputs.
+template <int EBITS, int MBITS> inline float f8_decode(unsigned v) {
+    constexpr int BIAS = (1 << (EBITS - 1)) - 1, EMAX = (1 << EBITS) - 1;
+    const unsigned e = (v >> MBITS) & EMAX, m = v & ((1u << MBITS) - 1);
+    const float sign = (v & 0x80u) ? -1.f : 1.f;
+    if (EBITS == 4 ? (e == (unsigned)EMAX && m == (1u << MBITS) - 1) : (e == (unsigned)EMAX && m != 0)) return NAN;
+    if (EBITS == 5 && e == (unsigned)EMAX) return sign * INFINITY;
+    if (e == 0) return sign * std::ldexp((float)m, 1 - BIAS - MBITS);
+    return sign * std::ldexp(1.f + (float)m / (1 << MBITS), (int)e - BIAS);
+}
+template <int EBITS, int MBITS> inline unsigned f8_encode(float f) {
+    constexpr int BIAS = (1 << (EBITS - 1)) - 1, EMAX = (1 << EBITS) - 1;
+    constexpr unsigned NAN_CODE = 0x7F, INF_CODE = EBITS == 5 ? (unsigned)EMAX << MBITS : NAN_CODE;
+    const unsigned sign = std::signbit(f) ? 0x80u : 0u;
+    if (f != f) return sign | NAN_CODE;
+    const double a = std::fabs((double)f);
+    if (std::isinf(a)) return sign | INF_CODE;
+    unsigned code;
+    if (a < std::ldexp(1.0, 1 - BIAS)) {
+        code = (unsigned)std::nearbyint(a * std::ldexp(1.0, BIAS - 1 + MBITS));  // units of the smallest subnormal
+    } else {
+        int e;
+        const double m = std::frexp(a, &e) * 2.0;  // [1, 2)
+        e -= 1;
+        unsigned q = (unsigned)std::nearbyint((m - 1.0) * (1 << MBITS));
+        if (q == (1u << MBITS)) { q = 0; e += 1; }
+        if (e + BIAS > EMAX) return sign | INF_CODE;
+        code = ((unsigned)(e + BIAS) << MBITS) | q;
+    }
+    if (EBITS == 4 ? code >= 0x7F : code >= INF_CODE) return sign | INF_CODE;
+    return sign | code;
+}
+inline int cvt_pk_f8(unsigned lo, unsigned hi_code, int old, bool high_half) {
+    const unsigned pk = lo | (hi_code << 8);
+    return high_half ? (int)(((unsigned)old & 0xFFFFu) | (pk << 16)) : (int)(((unsigned)old & 0xFFFF0000u) | pk);
+}
+inline float fmed3(float a, float b, float c) { return std::fmax(std::fmin(a, b), std::fmin(std::fmax(a, b), c)); }
 }  // namespace emu
-#define __builtin_amdgcn_cvt_f32_fp8(a, b) ((void)emu::no_such_instruction(), 0.f)
-#define __builtin_amdgcn_cvt_f32_bf8(a, b) ((void)emu::no_such_instruction(), 0.f)
-#define __builtin_amdgcn_cvt_pk_fp8_f32(a, b, c, d) ((void)emu::no_such_instruction(), 0)
-#define __builtin_amdgcn_cvt_pk_bf8_f32(a, b, c, d) ((void)emu::no_such_instruction(), 0)
-#define __builtin_amdgcn_fmed3f(a, b, c) ((void)emu::no_such_instruction(), 0.f)
+#define __builtin_amdgcn_cvt_f32_fp8(word, sel) (emu::f8_decode<4, 3>(((unsigned)(word) >> (8 * (sel))) & 0xFFu))
+#define __builtin_amdgcn_cvt_f32_bf8(word, sel) (emu::f8_decode<5, 2>(((unsigned)(word) >> (8 * (sel))) & 0xFFu))
+#define __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, hi) (emu::cvt_pk_f8(emu::f8_encode<4, 3>(a), emu::f8_encode<4, 3>(b), old, hi))
+#define __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, hi) (emu::cvt_pk_f8(emu::f8_encode<5, 2>(a), emu::f8_encode<5, 2>(b), old, hi))
+#define __builtin_amdgcn_fmed3f(a, b, c) (emu::fmed3(a, b, c))

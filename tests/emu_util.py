@@ -2,9 +2,14 @@
 metadata.cpp, softmax.hip, cast.hip, reduce.hip and gemm_generic.hip compiled for the host against a stand-in for
 <hip/hip_runtime.h> that runs a workgroup as host threads.  Test infrastructure: what it proves is indexing, masking,
 reduction structure and the entry points' argument handling -- arithmetic is the host's, so results are compared at the
-parity tolerances, bit for bit only where the kernel's arithmetic is integer or pure bit manipulation.  The matrix-core
-and LDS-DMA kernels have no CPU build; their launchers answer UNSUPPORTED here, which routes every product to the
-generic kernel."""
+parity tolerances, bit for bit only where the kernel's arithmetic is integer or pure bit manipulation.  In that build
+the matrix-core launchers answer UNSUPPORTED, which routes every product to the generic kernel.
+
+A second library (build(mfma=True), Emu(mfma=True)) adds the matrix-core tile kernels of bf16, f16 and f8e4m3 weights --
+gemm_mfma.hip, gemm_mfma_{bf16,f16}.hip, gemm_mfma_mi16_{bf16,f16}.hip, gemm_mfma_w8a16.hip, unmodified -- against the instruction
+models of tests/emu/gfx950_insn_emu.hpp (MFMA lane layouts, LDS-DMA with M0 and the immediate offset, the LDS
+transpose reads, vmcnt).  Those kernels' sums are f32 sums of exact products, so on operands whose partial sums are
+exact the comparison with the oracle is bit for bit."""
 import ctypes
 import os
 import shutil
@@ -20,6 +25,9 @@ CSRC = os.path.join(ROOT, "hodu_amd", "csrc")
 SOURCES = [os.path.join(CSRC, f) for f in ("api.cpp", "metadata.cpp", "softmax.hip", "cast.hip", "reduce.hip", "gemm_generic.hip")] + \
           [os.path.join(EMU, "emu_runtime.cpp")]
 LIB = os.path.join(OUT, "libhodu_emu.so")
+MFMA_SOURCES = [os.path.join(CSRC, f) for f in ("gemm_mfma.hip", "gemm_mfma_bf16.hip", "gemm_mfma_mi16_bf16.hip", "gemm_mfma_w8a16.hip",
+                                                "gemm_mfma_f16.hip", "gemm_mfma_mi16_f16.hip")]
+MFMA_LIB = os.path.join(OUT, "libhodu_emu_mfma.so")
 
 
 def compiler():
@@ -30,36 +38,49 @@ def compiler():
 
 
 def _newest_input():
-    paths = list(SOURCES) + [os.path.join(EMU, "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "hodu_rocm_kernels.h")]
+    paths = list(SOURCES) + list(MFMA_SOURCES) + [os.path.join(EMU, "hip", "hip_runtime.h"), os.path.join(EMU, "gfx950_insn_emu.hpp"),
+                                                  os.path.join(ROOT, "include", "hodu_rocm_kernels.h"), os.path.abspath(__file__)]
     paths += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
     return max(os.path.getmtime(p) for p in paths)
 
 
-def build():
+def build(mfma=False):
     """compiles the CPU build unless it is newer than every input; returns the library's path (None: no host clang)"""
     cxx = compiler()
     if cxx is None:
         return None
-    if os.path.exists(LIB) and os.path.getmtime(LIB) > _newest_input():
-        return LIB
+    lib = MFMA_LIB if mfma else LIB
+    if os.path.exists(lib) and os.path.getmtime(lib) > _newest_input():
+        return lib
     os.makedirs(OUT, exist_ok=True)
     flags = ["-std=c++17", "-O1", "-fPIC", "-x", "c++", f"-I{EMU}", f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
-             "-Wno-unused-function", "-Wno-unknown-attributes"]
+             "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-psabi"]
+    with_models = ["-DEMU_WITH_MFMA", "-DEMU_DYNAMIC_LDS", "-include", os.path.join(EMU, "gfx950_insn_emu.hpp")]
+    jobs = [(src, "", []) for src in SOURCES]
+    if mfma:
+        # the plain kernels keep their static __shared__ arrays; only the runtime and the tile kernels see the models
+        jobs = [(src, ".mfma" if src.endswith("emu_runtime.cpp") else "", with_models if src.endswith("emu_runtime.cpp") else [])
+                for src in SOURCES] + [(src, ".mfma", with_models) for src in MFMA_SOURCES]
 
-    def one(src):
-        obj = os.path.join(OUT, os.path.basename(src) + ".o")
-        r = subprocess.run([cxx, *flags, "-c", src, "-o", obj], capture_output=True, text=True)
+    def one(job):
+        src, tag, extra = job
+        obj = os.path.join(OUT, os.path.basename(src) + tag + ".o")
+        if os.path.exists(obj) and os.path.getmtime(obj) > _newest_input():
+            return obj
+        tmp_obj = obj + f".{os.getpid()}.tmp"
+        r = subprocess.run([cxx, *flags, *extra, "-c", src, "-o", tmp_obj], capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"CPU build of {src} failed:\n{r.stderr[-4000:]}")
+        os.replace(tmp_obj, obj)
         return obj
     with ThreadPoolExecutor(max_workers=7) as ex:
-        objs = list(ex.map(one, SOURCES))
-    tmp = LIB + ".tmp"
+        objs = list(ex.map(one, jobs))
+    tmp = lib + f".{os.getpid()}.tmp"
     r = subprocess.run([cxx, "-shared", "-o", tmp, *objs, "-lpthread"], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link of the CPU build failed:\n{r.stderr[-4000:]}")
-    os.replace(tmp, LIB)
-    return LIB
+    os.replace(tmp, lib)
+    return lib
 
 
 DTYPE_ID = {"bool": 0, "f8e4m3": 1, "f8e5m2": 2, "bf16": 3, "f16": 4, "f32": 5, "f64": 6, "u8": 7, "u16": 8, "u32": 9,
@@ -69,8 +90,8 @@ DTYPE_ID = {"bool": 0, "f8e4m3": 1, "f8e5m2": 2, "bf16": 3, "f16": 4, "f32": 5, 
 class Emu:
     """the entry points of api.cpp as compiled for the host; every pointer argument is a numpy array"""
 
-    def __init__(self):
-        path = build()
+    def __init__(self, mfma=False):
+        path = build(mfma)
         if path is None:
             raise RuntimeError("no host clang++ to build tests/emu with")
         self.lib = lib = ctypes.CDLL(path)
@@ -81,11 +102,17 @@ class Emu:
         lib.emu_last_kernel.restype = ctypes.c_char_p
         lib.emu_last_kernel.argtypes = [vp]
         lib.emu_last_error.restype = ctypes.c_char_p
+        lib.emu_unsupported_first.restype = ctypes.c_char_p
         lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
         lib.hodu_rocm_softmax_masked.argtypes = [vp, ci, vp, vp, szp, sz, ci, vp, ci, szp, sz]
         lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
         lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
         lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
+        if mfma:
+            lib.emu_dma_lazy.argtypes = [ci]
+            lib.emu_lds_fill.argtypes = [ci]
+            lib.emu_force_tile.argtypes = [vp, ci]
+            lib.emu_force_splitk.argtypes = [vp, ci]
         self.ctx = lib.emu_ctx_create()
 
     def close(self):
@@ -100,10 +127,28 @@ class Emu:
     def _check(self, rc, what):
         if rc != 0:
             raise RuntimeError(f"{what}: status {rc}: {self.lib.emu_last_error().decode()}")
-        assert self.lib.emu_unsupported_hits() == 0, f"{what} reached an instruction without a CPU stand-in"
+        if self.lib.emu_unsupported_hits() != 0:
+            first = self.lib.emu_unsupported_first().decode()
+            self.lib.emu_unsupported_reset()
+            raise AssertionError(f"{what} ({self.last_kernel()}) reached an instruction without a CPU stand-in: {first}")
 
     def last_kernel(self):
         return self.lib.emu_last_kernel(self.ctx).decode()
+
+    # the library with the tile kernels only
+    def force_tile(self, v):
+        self.lib.emu_force_tile(self.ctx, v)
+
+    def force_splitk(self, v):
+        self.lib.emu_force_splitk(self.ctx, v)
+
+    def dma_lazy(self, model):
+        """LDS-DMA bytes arrive at issue (0), only when an s_waitcnt vmcnt retires them (1), or one load later than
+        that (2: a model under which a correct kernel must FAIL)"""
+        self.lib.emu_dma_lazy(int(model))
+
+    def lds_fill(self, byte):
+        self.lib.emu_lds_fill(byte)
 
     def softmax(self, dt, x, out, md, causal=False):
         a, n = self._md(md)
@@ -132,3 +177,78 @@ class Emu:
         fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.POINTER(ctypes.c_size_t), ctypes.c_size_t]
         arr, n = self._md(md)
         self._check(fn(self.ctx, a.ctypes.data, b.ctypes.data, out.ctypes.data, arr, n), f"{op}_{name}")
+
+
+# ---- a stand-in for hodu_amd.ffi.Context over the CPU build, so that the GPU tests' helpers run against it unchanged ----
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mmap.restype = ctypes.c_void_p
+_libc.mmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_long]
+_libc.munmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+PAGE = 4096
+
+
+class GuardedBuffer:
+    """`nbytes` of "device" memory between two inaccessible pages: a kernel that reads or writes past either end of an
+    operand takes a segmentation fault here instead of a GPU memory fault there.  `tight` says which end touches its
+    guard page exactly ("end": the last 16-byte unit ends where the guard begins, the way a clamped row or a biased
+    pointer would overrun; "start": the first byte follows the front guard)."""
+
+    def __init__(self, nbytes, tight="end"):
+        body = max((nbytes + PAGE - 1) // PAGE, 1) * PAGE
+        self.total = body + 2 * PAGE
+        base = _libc.mmap(None, self.total, 3, 0x22, -1, 0)  # PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS
+        if base in (None, ctypes.c_void_p(-1).value):
+            raise MemoryError("mmap")
+        self.base = base
+        assert _libc.mprotect(base, PAGE, 0) == 0 and _libc.mprotect(base + PAGE + body, PAGE, 0) == 0
+        self.nbytes = nbytes
+        self.ptr = base + PAGE + (body - (nbytes + 15) // 16 * 16 if tight == "end" else 0)
+
+    def array(self, dtype, count=None):
+        count = self.nbytes // np.dtype(dtype).itemsize if count is None else count
+        return np.ctypeslib.as_array(ctypes.cast(self.ptr, ctypes.POINTER(ctypes.c_uint8)), (self.nbytes,)).view(dtype)[:count]
+
+    def free(self):
+        if self.base:
+            _libc.munmap(self.base, self.total)
+            self.base = None
+
+
+class EmuContext(Emu):
+    """upload / alloc / fill / product / download / last_kernel / force_tile with hodu_amd.ffi.Context's signatures"""
+
+    def __init__(self, tight="end"):
+        super().__init__(mfma=True)
+        self.tight = tight
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        buf = GuardedBuffer(arr.nbytes, self.tight)
+        buf.array(np.uint8)[:] = arr.view(np.uint8).ravel()
+        return buf
+
+    def alloc(self, nbytes):
+        return GuardedBuffer(nbytes, self.tight)
+
+    def fill(self, buf, byte):
+        buf.array(np.uint8)[:] = byte
+
+    def download(self, buf, dtype, count=None):
+        return buf.array(dtype, count).copy()
+
+    def product(self, op, name, a, b, out, md):
+        fn = getattr(self.lib, f"hodu_rocm_{op}_{name}")
+        fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.POINTER(ctypes.c_size_t), ctypes.c_size_t]
+        arr, n = self._md(md)
+        self._check(fn(self.ctx, a.ptr, b.ptr, out.ptr, arr, n), f"{op}_{name}")
+
+    def product_ex(self, op, name, a, b, out, md, steps):
+        """steps: hodu_amd.ffi.EpilogueStep values (ffi.add_row / mul_scalar / relu accept a GuardedBuffer)"""
+        steps = list(steps)
+        fn = getattr(self.lib, f"hodu_rocm_{op}_{name}_ex")
+        fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.POINTER(ctypes.c_size_t), ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t]
+        arr, n = self._md(md)
+        sarr = (type(steps[0]) * len(steps))(*steps) if steps else None
+        self._check(fn(self.ctx, a.ptr, b.ptr, out.ptr, arr, n, ctypes.cast(sarr, ctypes.c_void_p) if steps else None, len(steps)),
+                    f"{op}_{name}_ex")
