@@ -27,6 +27,10 @@ int dispatch_few_rows(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, co
 // Picks the kernel family for one launch-sized product.
 int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                  const DevProduct &g) {
+    if (ctx->reference_sums) {
+        const int rc = launch_reference_sums(ctx, kind, dtype, a, b, c, g);
+        if (rc != HODU_ROCM_UNSUPPORTED) return rc;
+    }
     // A matrix times a vector, [M, K] x [K, 1] (what Tensor::matmul makes of a 2-D and a 1-D tensor,
     // crates/hodu_core/src/tensor/ops/matrix.rs:50-66), is the transposed problem of one row against the matrix as
     // the weight, [1, K] x [K, M], and the [M, 1] output is the same memory as [1, M]: the few-rows kernels take it.
@@ -228,6 +232,14 @@ int hodu_rocm_matmul_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, 
 }
 int hodu_rocm_dot_i32_i8i8(hodu_rocm_ctx *ctx, const void *l, const void *r, void *o, const size_t *md, size_t n) {
     return dot_entry(ctx, PK_I32_I8I8, HODU_I32, l, r, o, md, n);
+}
+
+int hodu_rocm_ctx_set_reference_sums(hodu_rocm_ctx *ctx, int on) {
+    clear_error();
+    if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "set_reference_sums: context is null");
+    std::lock_guard<std::recursive_mutex> hold(ctx->mu);
+    ctx->reference_sums = on != 0;
+    return HODU_ROCM_OK;
 }
 
 // The one entry point that allocates nothing: hodu_rocm_dot_bf16_f8e4m3w with the partial sums and arrival counters

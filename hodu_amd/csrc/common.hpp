@@ -38,6 +38,7 @@ struct hodu_rocm_ctx {
     // device's static scratch array, and a kernel that needs more than it holds is refused instead of grown.
     bool fixed_scratch = false;
     void *static_scratch = nullptr;  // this device's copy of the static scratch array (hipGetSymbolAddress)
+    bool reference_sums = false;  // narrow-float products re-round after every multiply and add, as the reference's do
     const char *last_kernel = "";
     int force_tile = -1;    // testing hook: pins the MFMA tile size
     int force_splits = -1;  // testing hook: pins the number of K ranges of the pipelined kernels (1 = never split)
@@ -182,6 +183,9 @@ enum ProductKind {
 // generic strided kernel: every dtype, any strides; slow, always correct
 int launch_generic(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                    const DevProduct &g);
+// the reference's narrow-type running sum (gemm_refsum.hip): returns HODU_ROCM_UNSUPPORTED for dtypes it is not for
+int launch_reference_sums(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
+                          const DevProduct &g);
 // MFMA tile kernel: returns HODU_ROCM_UNSUPPORTED (without setting an error) when it has no variant
 int launch_mfma(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const void *b, void *c,
                 const DevProduct &g);

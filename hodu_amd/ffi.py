@@ -117,6 +117,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_softmax_masked.argtypes = [vp, ci, vp, vp, szp, sz, ci, vp, ci, szp, sz]
     lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
     lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc.argtypes = [vp, vp, vp, vp, szp, sz]
+    lib.hodu_rocm_ctx_set_reference_sums.argtypes = [vp, ci]
     _lib = lib
     return lib
 
@@ -298,6 +299,11 @@ class Context:
         self._check(self.debug.hodu_rocm_debug_time_noalloc(self.handle, lhs.ptr, ptrs, len(rhs_list), out.ptr, arr, n,
                                                             int(iters), int(bool(graph)), ctypes.byref(ms)))
         return float(ms.value)
+
+    def set_reference_sums(self, on: bool):
+        """hodu_rocm_ctx_set_reference_sums: narrow-float products in the reference's own arithmetic (the running sum
+        re-rounded to the dtype after every multiply and add), byte for byte hodu's CPU result; slow"""
+        self._check(self.lib.hodu_rocm_ctx_set_reference_sums(self.handle, int(bool(on))))
 
     def product_ex(self, op: str, name: str, lhs: DeviceBuffer, rhs: DeviceBuffer, out: DeviceBuffer, md, steps):
         """hodu_rocm_<op>_<name>_ex: the product with element-wise steps (add_row / mul_scalar / relu) fused into

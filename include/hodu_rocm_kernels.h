@@ -82,6 +82,16 @@ int hodu_rocm_timer_stop(hodu_rocm_ctx *ctx, void *timer, float *elapsed_ms); /*
 int hodu_rocm_timer_destroy(hodu_rocm_ctx *ctx, void *timer);
 /* name of the kernel family the last matmul/dot call on this context dispatched to (diagnostics) */
 const char *hodu_rocm_last_kernel(hodu_rocm_ctx *ctx);
+/* The reference's own arithmetic for products of the narrow float dtypes, for a caller that needs hodu's CPU bytes.
+ * hodu_cpu_matmul_<dt> / hodu_cpu_dot_<dt> for f8e4m3, f8e5m2, bf16 and f16 keep the running sum in the narrow type,
+ * sum = add(sum, mul(a, b)) with both results narrowed by the type's routine (kernels/ops_matrix.c:196-240, :351-354,
+ * :556-600, :713-716; t_bf16.h:27-55, t_f16.h:27-84, t_f8e4m3.h:27-101, t_f8e5m2.h:27-100).  With `on` != 0 every
+ * later product of those four dtypes on this context (plain and _ex, and the bf16_f8e4m3w kind as this library's
+ * cast of the weight followed by the bf16 product) is computed that way, k ascending, and stores the reference's bytes
+ * bit for bit -- at the rate of one scalar loop per output element.  Off (the default) they accumulate in f32 and
+ * round once, which is what the rest of this header documents.  Other dtypes are not affected: integers and f64 are
+ * the reference's arithmetic already, f32 goes to a BLAS there.                                                   */
+int hodu_rocm_ctx_set_reference_sums(hodu_rocm_ctx *ctx, int on);
 /* ---- matmul / dot: lhs, rhs and out share one dtype (utils/valid.rs:50-76) -------------------- *
  * replaces hodu_cpu_matmul_<dt> (kernels/ops_matrix.c:70, :221) and hodu_cpu_dot_<dt>
  * (kernels/ops_matrix.c:423, :581).  Narrow floats accumulate in f32 and round once on store.   */

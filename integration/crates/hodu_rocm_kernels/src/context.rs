@@ -61,6 +61,12 @@ impl Context {
         Ok(out)
     }
     pub fn sync(&self) -> Result<()> { self.check(unsafe { ffi::hodu_rocm_sync(self.raw) }) }
+    /// Products of f8e4m3 / f8e5m2 / bf16 / f16 in the CPU backend's arithmetic (the running sum re-rounded to the dtype
+    /// after every multiply and add): byte for byte what `hodu_cpu_matmul_<dt>` stores, at a scalar loop's speed.  For
+    /// tests that compare devices bit for bit; off by default.
+    pub fn set_reference_sums(&self, on: bool) -> Result<()> {
+        self.check(unsafe { ffi::hodu_rocm_ctx_set_reference_sums(self.raw, on as c_int) })
+    }
 }
 
 impl Drop for Context {

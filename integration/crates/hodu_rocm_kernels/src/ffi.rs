@@ -47,6 +47,7 @@ extern "C" {
     pub fn hodu_rocm_memcpy_d2d(ctx: *mut hodu_rocm_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn hodu_rocm_sync(ctx: *mut hodu_rocm_ctx) -> c_int;
     pub fn hodu_rocm_last_error(ctx: *mut hodu_rocm_ctx) -> *const c_char;
+    pub fn hodu_rocm_ctx_set_reference_sums(ctx: *mut hodu_rocm_ctx, on: c_int) -> c_int;
 
     pub fn hodu_rocm_cast(ctx: *mut hodu_rocm_ctx, src_dtype: c_int, dst_dtype: c_int, input: *const c_void,
                           out: *mut c_void, metadata: *const usize, metadata_len: usize) -> c_int;

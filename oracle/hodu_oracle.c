@@ -69,7 +69,9 @@
  * narrows an accumulator that it re-rounded to f8 after every k with float_to_f8e4m3 (t_f8e4m3.h:52-85); the device
  * rounds the f32 sum once, to nearest even, saturating.  No fixture of the reference holds an f8 product, so the
  * device's f8 outputs are checked against the SPEC value narrowed by an independent round-to-nearest-even encoder
- * (bit for bit on exactly representable sums, tests/test_gpu_exact.py), not against the reference's bytes.
+ * (bit for bit on exactly representable sums, tests/test_gpu_exact.py), not against the reference's bytes.  (The
+ * library's optional reference-sum mode, hodu_rocm_ctx_set_reference_sums, IS held to the reference's bytes: against
+ * the asis products here and against oracle/_ref, tests/test_emu_reference_sums_cpu.py.)
  */
 #include <math.h>
 #include <stdbool.h>

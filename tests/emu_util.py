@@ -1,5 +1,5 @@
 """Builds and loads the CPU build of the library's plain kernels (tests/emu): the unmodified sources of api.cpp,
-metadata.cpp, softmax.hip, cast.hip, reduce.hip and gemm_generic.hip compiled for the host against a stand-in for
+metadata.cpp, softmax.hip, cast.hip, reduce.hip, gemm_generic.hip and gemm_refsum.hip compiled for the host against a stand-in for
 <hip/hip_runtime.h> that runs a workgroup as host threads.  Test infrastructure: what it proves is indexing, masking,
 reduction structure and the entry points' argument handling -- arithmetic is the host's, so results are compared at the
 parity tolerances, bit for bit only where the kernel's arithmetic is integer or pure bit manipulation.  In that build
@@ -22,7 +22,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EMU = os.path.join(ROOT, "tests", "emu")
 OUT = os.path.join(EMU, "_build")
 CSRC = os.path.join(ROOT, "hodu_amd", "csrc")
-SOURCES = [os.path.join(CSRC, f) for f in ("api.cpp", "metadata.cpp", "softmax.hip", "cast.hip", "reduce.hip", "gemm_generic.hip")] + \
+SOURCES = [os.path.join(CSRC, f) for f in ("api.cpp", "metadata.cpp", "softmax.hip", "cast.hip", "reduce.hip", "gemm_generic.hip", "gemm_refsum.hip")] + \
           [os.path.join(EMU, "emu_runtime.cpp")]
 LIB = os.path.join(OUT, "libhodu_emu.so")
 MFMA_SOURCES = [os.path.join(CSRC, f) for f in ("gemm_mfma.hip", "gemm_mfma_bf16.hip", "gemm_mfma_mi16_bf16.hip", "gemm_mfma_w8a16.hip",
@@ -134,6 +134,10 @@ class Emu:
 
     def last_kernel(self):
         return self.lib.emu_last_kernel(self.ctx).decode()
+
+    def set_reference_sums(self, on):
+        self.lib.hodu_rocm_ctx_set_reference_sums.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        assert self.lib.hodu_rocm_ctx_set_reference_sums(self.ctx, int(on)) == 0
 
     # the library with the tile kernels only
     def force_tile(self, v):
