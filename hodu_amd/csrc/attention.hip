@@ -110,7 +110,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     typedef typename Cmp::acc_t acc_t;
     typedef AtGeom<D> G;
     constexpr int AT_D = D, AT_KSTEPS = G::KSTEPS, AT_K_BYTES = G::K_BYTES, AT_V_BYTES = G::V_BYTES;
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, lh = lane >> 5;

@@ -7,6 +7,12 @@
 
 #include "common.hpp"
 
+// The workgroup's dynamically sized LDS as a char array called `name`, 16-byte aligned.  (A macro so that a CPU build
+// of the kernels for tests, where LDS is an ordinary array, can say it its own way: it defines the macro first.)
+#ifndef HODU_DYNAMIC_LDS
+#define HODU_DYNAMIC_LDS(name) extern __shared__ __align__(16) char name[]
+#endif
+
 namespace hodu {
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));

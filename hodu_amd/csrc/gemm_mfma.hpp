@@ -692,7 +692,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_product_kernel(const char *__res
                                                                typename Out<Cfg::OUT>::T *__restrict__ C,
                                                                DevProduct g, int tiles_m, int tiles_n, int steps_per_split,
                                                                void *__restrict__ partials) {
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef typename Compute32<Cfg::CK>::acc_t acc_t;
     typedef typename Cfg::LoaderA LoaderA;
     typedef typename Cfg::LoaderB LoaderB;

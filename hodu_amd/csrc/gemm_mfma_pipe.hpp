@@ -363,7 +363,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_kernel(const char *__restri
                                                             typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                             int tiles_m, int tiles_n, int stages_per_split,
                                                             void *__restrict__ partials, int *__restrict__ arrival) {
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef Compute32<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;

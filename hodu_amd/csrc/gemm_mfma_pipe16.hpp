@@ -61,7 +61,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_kernel(const char *__rest
                                                               int tiles_m, int tiles_n) {
     static_assert(!Cfg::B_F8 && Cfg::ES == 2 && Cfg::NST == 2, "16-bit operands stored in the compute type, two stages");
     typedef RowDenseGeom<Cfg::ES, Cfg::ES> G;
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef Compute16<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_kernel(const char *__res
                                                                int tiles_m, int tiles_n) {
     static_assert(!Cfg::B_F8 && Cfg::ES == 2 && Cfg::NST == 2, "16-bit operands stored in the compute type, two stages");
     typedef RowDenseGeom<Cfg::ES, Cfg::ES> G;
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef Compute16<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;
@@ -550,7 +550,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16_f8w_kernel(const char *__
                                                                   typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                   int tiles_m, int tiles_n) {
     static_assert(Cfg::LA == LM_K && Cfg::B_F8 && Cfg::NST == 2, "bf16 x f8e4m3, the left operand k-dense, two stages");
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef Compute16<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;
@@ -785,7 +785,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe16r_f8w_kernel(const char *_
                                                                   typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                   int tiles_m, int tiles_n) {
     static_assert(Cfg::LA == LM_K && Cfg::B_F8 && Cfg::NST == 2, "bf16 x f8e4m3, the left operand k-dense, two stages");
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef Compute16<Cfg::CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef typename Out<Cfg::OUT>::T out_t;

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8_kernel(const char *__res
                                                                typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                int tiles_m, int tiles_n, int stages_per_split,
                                                                void *__restrict__ partials, int *__restrict__ arrival) {
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef typename Out<Cfg::OUT>::T out_t;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, PA = Cfg::PA, PB = Cfg::PB, P = Cfg::P;
     constexpr int TILE_BYTES = 32 * P_ROW_BYTES, B_BASE = 2 * Cfg::A_BYTES;

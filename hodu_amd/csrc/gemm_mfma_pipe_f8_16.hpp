@@ -26,17 +26,10 @@ namespace mfma {
 
 typedef float f32x4_f8acc_t __attribute__((ext_vector_type(4)));
 
-// FMT: the instruction's operand format code, 0 = e4m3, 1 = e5m2 (both operands alike).  Written out with the
-// accumulator tied to itself in the accumulation registers (left to the register allocator, kernels with this many
-// small accumulators came out with copies inside the loop); an accumulator is next touched 64 MFMAs later, the other
-// operands come from LDS reads the compiler waits for as for any use of a register.
+// FMT: the instruction's operand format code, 0 = e4m3, 1 = e5m2 (both operands alike).  The instruction itself,
+// written out with its accumulator tied: mfma16x16x128_f8 of gfx950_insn.hpp.
 template <int FMT> __device__ __forceinline__ void mma_f8_16(const i32x8_t &a, const i32x8_t &b, f32x4_f8acc_t &c) {
-    const int unit = 0x7F7F7F7F;  // scale bytes 0x7F = 2^0
-    if constexpr (FMT == 0)
-        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]" : "+a"(c) : "v"(a), "v"(b), "v"(unit));
-    else
-        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0] cbsz:1 blgp:1"
-                     : "+a"(c) : "v"(a), "v"(b), "v"(unit));
+    mfma16x16x128_f8<FMT>(a, b, c);
 }
 
 template <int OUT_, int BM_, int BN_> struct PipeF8x16Config {
@@ -53,7 +46,7 @@ template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void mfma_pipe_f8x16_kernel(const char *__restrict__ A, const char *__restrict__ B,
                                                                   typename Out<Cfg::OUT>::T *__restrict__ C, DevProduct g,
                                                                   int tiles_m, int tiles_n) {
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     typedef typename Out<Cfg::OUT>::T out_t;
     typedef f32x4_f8acc_t acc_t;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, PA = Cfg::PA, PB = Cfg::PB, P = Cfg::P, HALF = TM / 2;

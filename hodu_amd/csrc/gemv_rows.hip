@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const typename T::XS *__
     typedef typename T::A A;
     typedef typename T::WS WS;
     struct alignas(sizeof(WS) * V) Vec { WS e[V]; };
-    extern __shared__ __align__(16) char smem[];
+    HODU_DYNAMIC_LDS(smem);
     A *xs = reinterpret_cast<A *>(smem);  // [per_chunk][MT]; later [3][64][MT * V] for the wavefronts to meet
     // weight rows a wavefront has loads out for at a time: deep where the accumulators leave the registers for it
     constexpr int RIF = MT * V <= 32 ? 8 : 4;

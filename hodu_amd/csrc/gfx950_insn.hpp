@@ -27,6 +27,19 @@ __device__ __forceinline__ void mfma16x16x32_f16(const u32x4_t &a, const u32x4_t
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
+// v_mfma_scale_f32_16x16x128_f8f6f4 with unit scales (scale bytes 0x7F = 2^0), both operands of one 8-bit float format
+// (FMT 0 = e4m3, 1 = e5m2: the instruction's cbsz / blgp fields), the accumulator tied as above -- left to the register
+// allocator, kernels with this many small accumulators came out with copies inside the loop; an accumulator is next
+// touched 64 MFMAs later, the other operands come from LDS reads the compiler waits for as for any use of a register.
+template <int FMT> __device__ __forceinline__ void mfma16x16x128_f8(const i32x8_t &a, const i32x8_t &b, f32x4_acc_t &c) {
+    const int unit = 0x7F7F7F7F;
+    if constexpr (FMT == 0)
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]" : "+a"(c) : "v"(a), "v"(b), "v"(unit));
+    else
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0] cbsz:1 blgp:1"
+                     : "+a"(c) : "v"(a), "v"(b), "v"(unit));
+}
+
 // Kernels that write their MFMAs out in assembly hide them from the compiler's hazard recogniser, which therefore
 // inserts nothing between the last matrix instruction and the first read of an accumulator behind the loop.  The
 // hardware wants idle wait states there -- up to 18 when a 16-pass instruction's result is read by a vector

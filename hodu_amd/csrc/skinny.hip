@@ -71,7 +71,7 @@ __global__ __launch_bounds__(NBLK * KW * 64) void skinny_kdense_kernel(const cha
     constexpr int ES = Cmp::ES;                         // bytes per element of x (and of W unless f8)
     constexpr int SB = SKB == SK_F8 ? 1 : ES;           // bytes per stored weight element
     constexpr int EPL = 16 / SB;                        // weight elements per lane per load
-    extern __shared__ __align__(16) char xs[];
+    HODU_DYNAMIC_LDS(xs);
     constexpr int NT = NBLK * KW * 64;
     __shared__ acc_t red[NBLK * KW][64];
 
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const char *__restri
     typedef typename Cmp::acc_t acc_t;
     typedef decltype(acc_t{}.x) part_t;
     constexpr int ES = Cmp::ES, SB = SKB == SK_F8 ? 1 : ES, EPL = 16 / SB;
-    extern __shared__ __align__(16) char xs[];
+    HODU_DYNAMIC_LDS(xs);
     __shared__ int last_flag;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

@@ -4,6 +4,7 @@
 // LDS-DMA and therefore have no CPU build (the long inner product of reduce.hip does).  "Device" pointers are host pointers here.
 #include <cstdarg>
 #include <cstdlib>
+#include <cstring>
 
 #include "common.hpp"
 
@@ -48,41 +49,32 @@ int ensure_arrival(hodu_rocm_ctx *) { return fail(HODU_ROCM_UNSUPPORTED, "no arr
     int name(hodu_rocm_ctx *, int, int, const void *, const void *, void *, const DevProduct &) { return HODU_ROCM_UNSUPPORTED; }
 #ifndef EMU_WITH_MFMA
 NO_CPU_BUILD(launch_mfma)
-#else
-// the tile kernels of the 16-bit types and of f8e4m3 weights are built (gfx950_insn_emu.hpp); the other kinds are not
-#define NO_CPU_BUILD_KIND(name) \
-    int name(hodu_rocm_ctx *, const void *, const void *, void *, const DevProduct &) { return HODU_ROCM_UNSUPPORTED; }
-NO_CPU_BUILD_KIND(launch_mfma_i8)
-NO_CPU_BUILD_KIND(launch_mfma_f32)
-NO_CPU_BUILD_KIND(launch_mfma_i8_out)
-NO_CPU_BUILD_KIND(launch_mfma_u8_out)
-int launch_mfma_f8(hodu_rocm_ctx *, int, const void *, const void *, void *, const DevProduct &) { return HODU_ROCM_UNSUPPORTED; }
-#endif
 NO_CPU_BUILD(launch_gemv)
 NO_CPU_BUILD(launch_small_f32)
 NO_CPU_BUILD(launch_gemm_f64)
 NO_CPU_BUILD(launch_skinny)
 NO_CPU_BUILD(launch_gemv_rows)
+#endif
 int launch_attention(hodu_rocm_ctx *, int, const void *, const void *, const void *, void *, const AttentionArgs &) {
     return HODU_ROCM_UNSUPPORTED;
 }
 }  // namespace hodu
 
-#ifdef EMU_WITH_MFMA
-// LDS of the workgroup that is running (workgroups run one at a time): what `extern __shared__ char smem[]` names in
-// the tile kernels, and the model of LDS-DMA arrival
-namespace hodu {
-namespace mfma {
-alignas(256) char smem[emu::kLdsBytes];
-}
-}  // namespace hodu
+// LDS of the workgroup that is running (workgroups run one at a time): what HODU_DYNAMIC_LDS names in the kernels
 namespace emu {
-char *lds_base() { return hodu::mfma::smem; }
+namespace {
+alignas(256) char g_lds[kLdsBytes];
+}
+char *lds_base() { return g_lds; }
+}  // namespace emu
+// fills LDS with a pattern, so that a kernel that reads what it has not written does not find the last launch's data
+extern "C" void emu_lds_fill(int byte) { memset(emu::lds_base(), byte, emu::kLdsBytes); }
+#ifdef EMU_WITH_MFMA
+// the model of LDS-DMA arrival (gfx950_insn_emu.hpp)
+namespace emu {
 int &dma_lazy() { static int model = 0; return model; }
 }  // namespace emu
 extern "C" void emu_dma_lazy(int model) { emu::dma_lazy() = model; }
-// fills LDS with a pattern, so that a kernel that reads what it has not written does not find the last launch's data
-extern "C" void emu_lds_fill(int byte) { memset(hodu::mfma::smem, byte, sizeof(hodu::mfma::smem)); }
 #endif
 
 extern "C" {

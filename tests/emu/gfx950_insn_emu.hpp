@@ -1,7 +1,6 @@
 // Test infrastructure: CPU stand-ins for the instruction wrappers of hodu_amd/csrc/gfx950_insn.hpp and for the gfx950
 // builtins the matrix-core kernel headers use, so that the tile kernels' unmodified source runs in the CPU build
-// (tests/emu/hip/hip_runtime.h).  A translation unit gets this file through -include, ahead of everything else, with
-// EMU_DYNAMIC_LDS defined.
+// (tests/emu/hip/hip_runtime.h).  A translation unit gets this file through -include, ahead of everything else.
 //
 // What is modelled, as this repository understands the hardware (the kernels that have run on a GPU and pass their
 // tests there are the evidence for the model; a kernel that has not is checked against the model, not against the
@@ -10,6 +9,11 @@
 //     first operand and of column r of the second; it then holds D[4 g + e][r], e = 0..3, added to its accumulator;
 //   * v_mfma_f32_32x32x16_{bf16,f16}: lane (r = lane % 32, h = lane / 32) supplies k = 8 h .. 8 h + 7 of row / column r;
 //     it then holds D[8 (e / 4) + 4 h + e % 4][r], e = 0..15;
+//   * the other shapes alike, with the k a lane supplies: one (f32 32 x 32 x 2 and 16 x 16 x 4, f64 16 x 16 x 4), 16
+//     bytes (i8 32 x 32 x 32 and 16 x 16 x 64), 32 bytes (the 8-bit float forms 32 x 32 x 64 and 16 x 16 x 128 with
+//     unit scales);
+//   * v_dot2_f32_bf16, v_readlane, v_mov with the DPP controls quad_perm / row_mirror / row_half_mirror, ballot,
+//     v_permlane32_swap;
 //     both sum in f32 with k ascending (the hardware's order inside one instruction is not architected; the tests that
 //     compare bit for bit use operands whose products and partial sums are exact);
 //   * global_load_lds_dwordx4: lane l copies 16 bytes from (base + lane offset + immediate) to LDS at M0 + immediate
@@ -40,8 +44,6 @@
 #include <vector>
 
 namespace emu {
-constexpr unsigned kLdsBytes = 160 * 1024;
-char *lds_base();    // the array the kernels' `smem` names
 int &dma_lazy();     // the model of LDS-DMA arrival: 0 at issue, 1 as late as allowed, 2 later than allowed by one
 inline char *lds_at(unsigned addr32, unsigned bytes) {
     const unsigned off = addr32 - (unsigned)(uintptr_t)lds_base();
@@ -100,24 +102,115 @@ typedef unsigned vu32x4 __attribute__((ext_vector_type(4)));
 typedef float vf32x4 __attribute__((ext_vector_type(4)));
 typedef float vf32x16 __attribute__((ext_vector_type(16)));
 
-// D (ROWS x ROWS) += A (ROWS x K) * B (K x ROWS), 8 k per lane, K = 8 * 64 / ROWS
-template <int ROWS, class Acc, class Widen> inline void mfma_8k(const vu32x4 &a, const vu32x4 &b, Acc &c, Widen widen) {
-    struct Ops { vu32x4 a, b; };
+// D (ROWS x ROWS) += A (ROWS x K) * B (K x ROWS) for every MFMA shape used here: a lane supplies KPL consecutive k
+// (OPB bytes) of row / column r = lane % ROWS, starting at k = KPL * (lane / ROWS); it then holds column r of D rows
+//   4 g + e                    (16 x 16: e = 0..3, g = lane / 16)
+//   8 (e / 4) + 4 g + e % 4    (32 x 32: e = 0..15, g = lane / 32)
+//   4 e + g                    (the f64 16 x 16 x 4 form, F64ROWS: its registers step through the rows by four)
+// `term(pa, pb, k)` is one product in the accumulate type, from the two lanes' raw operand bytes.
+template <int ROWS, int KPL, int OPB, class AccT, bool F64ROWS = false, class Acc, class Term>
+inline void mfma_model(const void *a, const void *b, Acc &c, Term term) {
+    static_assert(2 * OPB <= kWideBytes, "both operands in one exchange slot");
+    struct Ops { unsigned char a[OPB], b[OPB]; };
     constexpr int KG = 64 / ROWS, NE = ROWS * ROWS / 64;
-    const Ops mine{a, b};
+    Ops mine;
+    memcpy(mine.a, a, OPB);
+    memcpy(mine.b, b, OPB);
     const auto slots = wave_deposit(mine);
     const unsigned lane = lane_id(), r = lane % ROWS, g = lane / ROWS;
     for (int e = 0; e < NE; e++) {
-        const unsigned i = ROWS == 16 ? 4 * g + e : 8 * (e / 4) + 4 * g + e % 4;  // row of D; column r
-        float sum = 0.f;
+        const unsigned i = F64ROWS ? 4 * e + g : ROWS == 16 ? 4 * g + e : 8 * (e / 4) + 4 * g + e % 4;
+        AccT sum = 0;
         for (unsigned kg = 0; kg < (unsigned)KG; kg++) {
-            uint16_t pa[8], pb[8];
-            memcpy(pa, slots[ROWS * kg + i], 16);        // lane (i, kg): A[i][8 kg ..], its first operand
-            memcpy(pb, slots[ROWS * kg + r] + 16, 16);   // lane (r, kg): B[8 kg ..][r], its second operand
-            for (int k = 0; k < 8; k++) sum += widen(pa[k]) * widen(pb[k]);
+            const unsigned char *pa = slots[ROWS * kg + i];        // lane (i, kg): A[i][KPL kg ..], its first operand
+            const unsigned char *pb = slots[ROWS * kg + r] + OPB;  // lane (r, kg): B[KPL kg ..][r], its second operand
+            for (int k = 0; k < KPL; k++) sum += term(pa, pb, k);
         }
         c[e] += sum;
     }
+}
+template <int ROWS, class Acc, class Widen> inline void mfma_8k(const vu32x4 &a, const vu32x4 &b, Acc &c, Widen widen) {
+    mfma_model<ROWS, 8, 16, float>(&a, &b, c, [&](const unsigned char *pa, const unsigned char *pb, int k) {
+        uint16_t x, y;
+        memcpy(&x, pa + 2 * k, 2);
+        memcpy(&y, pb + 2 * k, 2);
+        return widen(x) * widen(y);
+    });
+}
+template <int ROWS, class Acc> inline Acc mfma_f32(float a, float b, Acc c) {
+    mfma_model<ROWS, 1, 4, float>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int) {
+        float x, y;
+        memcpy(&x, pa, 4);
+        memcpy(&y, pb, 4);
+        return x * y;
+    });
+    return c;
+}
+template <class Acc> inline Acc mfma_f64_16(double a, double b, Acc c) {
+    mfma_model<16, 1, 8, double, true>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int) {
+        double x, y;
+        memcpy(&x, pa, 8);
+        memcpy(&y, pb, 8);
+        return x * y;
+    });
+    return c;
+}
+template <int ROWS, class Vec, class Acc> inline Acc mfma_i8(const Vec &a, const Vec &b, Acc c) {
+    static_assert(sizeof(Vec) == 16, "16 bytes of k per lane");
+    mfma_model<ROWS, 16, 16, int>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int k) {
+        return (int)(int8_t)pa[k] * (int)(int8_t)pb[k];
+    });
+    return c;
+}
+// the 8-bit float forms (v_mfma_scale_f32_*_f8f6f4 with unit scales): 32 bytes of k per lane; FMT 0 = e4m3, 1 = e5m2
+template <int ROWS, int FMT, class Vec, class Acc> inline void mfma_f8(const Vec &a, const Vec &b, Acc &c) {
+    static_assert(sizeof(Vec) == 32, "32 bytes of k per lane");
+    mfma_model<ROWS, 32, 32, float>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int k) {
+        return FMT == 0 ? f8_decode<4, 3>(pa[k]) * f8_decode<4, 3>(pb[k]) : f8_decode<5, 2>(pa[k]) * f8_decode<5, 2>(pb[k]);
+    });
+}
+
+// v_dot2_f32_bf16: c + a.x * b.x + a.y * b.y
+inline float fdot2_bf16(unsigned a, unsigned b, float c) {
+    return c + widen_bf16((uint16_t)(a & 0xFFFF)) * widen_bf16((uint16_t)(b & 0xFFFF)) + widen_bf16((uint16_t)(a >> 16)) * widen_bf16((uint16_t)(b >> 16));
+}
+// what every lane of the wavefront holds in `v`, by lane
+inline const unsigned char (*wave_values(unsigned v))[kWideBytes] { return wave_deposit(v); }
+inline unsigned slot_u32(const unsigned char (*slots)[kWideBytes], unsigned lane) {
+    unsigned v;
+    memcpy(&v, slots[lane], 4);
+    return v;
+}
+inline int readlane(int v, int lane) { return (int)slot_u32(wave_values((unsigned)v), (unsigned)lane & 63u); }
+// v_mov_b32 with a DPP control, all rows and banks enabled: the controls these kernels use
+inline int update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+    (void)old; (void)bound_ctrl;
+    if (row_mask != 0xF || bank_mask != 0xF) (void)no_such_instruction("DPP with a row or bank mask");
+    const auto slots = wave_values((unsigned)src);
+    const unsigned l = lane_id();
+    unsigned from;
+    if (ctrl >= 0 && ctrl <= 0xFF) from = (l & ~3u) + (((unsigned)ctrl >> (2 * (l & 3u))) & 3u);  // quad_perm
+    else if (ctrl == 0x140) from = (l & ~15u) + (15u - (l & 15u));                                 // row_mirror
+    else if (ctrl == 0x141) from = (l & ~7u) + (7u - (l & 7u));                                    // row_half_mirror
+    else { (void)no_such_instruction("DPP control"); from = l; }
+    return (int)slot_u32(slots, from);
+}
+inline unsigned long long ballot(bool pred) {
+    const auto slots = wave_values(pred ? 1u : 0u);
+    unsigned long long m = 0;
+    for (unsigned l = 0; l < 64; l++) m |= (unsigned long long)(slot_u32(slots, l) & 1u) << l;
+    return m;
+}
+// v_permlane32_swap: lanes 0..31 of `hi_src` change places with lanes 32..63 of `lo_src`; returns {lo_src', hi_src'}
+typedef unsigned vu32x2 __attribute__((ext_vector_type(2)));
+inline vu32x2 permlane32_swap(unsigned a, unsigned b) {
+    struct Pair { unsigned a, b; };
+    const auto slots = wave_deposit(Pair{a, b});
+    const unsigned l = lane_id();
+    Pair other;
+    memcpy(&other, slots[l ^ 32u], sizeof(Pair));
+    // vdst (a) keeps its lower half and takes the partner's src (b) lower half in its upper lanes; src the reverse
+    return l < 32 ? vu32x2{a, other.a} : vu32x2{other.b, b};
 }
 
 template <int ELEM_BYTES, class R> inline R ds_read_tr(const void *lds_ptr) {
@@ -151,11 +244,12 @@ inline uint16_t f8e4m3_to_bf16_bits(uint8_t v) {
     }
     return (uint16_t)(sign | ((e - 7 + 127) << 7) | (m << 4));
 }
-typedef unsigned short vu16x2 __attribute__((ext_vector_type(2)));
-inline vu16x2 cvt_pk_bf16_fp8(unsigned word, float scale, bool hi) {
+typedef __bf16 vbf16x2 __attribute__((ext_vector_type(2)));
+inline vbf16x2 cvt_pk_bf16_fp8(unsigned word, float scale, bool hi) {
     if (scale != 1.0f) (void)no_such_instruction("cvt_scalef32_pk_bf16_fp8 with a scale");
     const unsigned half = hi ? word >> 16 : word & 0xFFFFu;
-    return vu16x2{f8e4m3_to_bf16_bits((uint8_t)(half & 0xFF)), f8e4m3_to_bf16_bits((uint8_t)(half >> 8))};
+    const unsigned both = (unsigned)f8e4m3_to_bf16_bits((uint8_t)(half & 0xFF)) | ((unsigned)f8e4m3_to_bf16_bits((uint8_t)(half >> 8)) << 16);
+    return __builtin_bit_cast(vbf16x2, both);
 }
 
 // v_perm_b32: result byte i is byte sel[i] of the eight bytes {s1 (0..3), s0 (4..7)}; selectors above 7 (sign fills and
@@ -220,10 +314,21 @@ struct Any {
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) EMU_MFMA(32, emu::widen_f16, a, b, c)
 #define __builtin_amdgcn_perm(s0, s1, sel) (emu::perm_b32(s0, s1, sel))
 #define __builtin_amdgcn_cvt_pk_f32_fp8(word, hi) (emu::cvt_pk_f32_fp8((unsigned)(word), hi))
-#define __builtin_amdgcn_mfma_f32_32x32x2f32(...) (emu::Any{"mfma_f32_32x32x2f32"})
-#define __builtin_amdgcn_mfma_f32_16x16x4f32(...) (emu::Any{"mfma_f32_16x16x4f32"})
-#define __builtin_amdgcn_mfma_i32_32x32x32_i8(...) (emu::Any{"mfma_i32_32x32x32_i8"})
-#define __builtin_amdgcn_mfma_i32_16x16x64_i8(...) (emu::Any{"mfma_i32_16x16x64_i8"})
+#define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) (emu::mfma_f32<32>(a, b, c))
+#define __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, x, y, z) (emu::mfma_f32<16>(a, b, c))
+#define __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, x, y, z) (emu::mfma_f64_16(a, b, c))
+#define __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, x, y, z) (emu::mfma_i8<32>(a, b, c))
+#define __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, x, y, z) (emu::mfma_i8<16>(a, b, c))
+#define __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, fa, fb, sa, scale_a, sb, scale_b) \
+    ([&] { auto acc_ = (c); if ((fa) != (fb) || (fa) > 1 || (scale_a) != 0x7F7F7F7F || (scale_b) != 0x7F7F7F7F) (void)emu::no_such_instruction("scaled MFMA beyond unit scales of one 8-bit format"); \
+           if ((fa) == 0) emu::mfma_f8<32, 0>(a, b, acc_); else emu::mfma_f8<32, 1>(a, b, acc_); return acc_; }())
+#define __builtin_amdgcn_fdot2_f32_bf16(a, b, c, clamp) (emu::fdot2_bf16(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b), c))
+#define __builtin_amdgcn_readlane(v, lane) (emu::readlane(v, lane))
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, rm, bm, bc) (emu::update_dpp(old, src, ctrl, rm, bm, bc))
+#define __builtin_amdgcn_ballot_w64(p) (emu::ballot(p))
+#define __builtin_amdgcn_exp2f(x) (exp2f(x))
+#define __builtin_amdgcn_permlane32_swap(a, b, fi, bc) (emu::permlane32_swap(a, b))
+#define __builtin_amdgcn_s_memtime() 0ull
 
 namespace hodu {
 namespace mfma {
@@ -233,6 +338,8 @@ typedef unsigned emu_u32x4 __attribute__((ext_vector_type(4)));
 
 inline void mfma16x16x32_bf16(const emu_u32x4 &a, const emu_u32x4 &b, f32x4_acc_t &c) { emu::mfma_8k<16>(a, b, c, emu::widen_bf16); }
 inline void mfma16x16x32_f16(const emu_u32x4 &a, const emu_u32x4 &b, f32x4_acc_t &c) { emu::mfma_8k<16>(a, b, c, emu::widen_f16); }
+typedef int emu_i32x8 __attribute__((ext_vector_type(8)));
+template <int FMT> inline void mfma16x16x128_f8(const emu_i32x8 &a, const emu_i32x8 &b, f32x4_acc_t &c) { emu::mfma_f8<16, FMT>(a, b, c); }
 inline void mfma_results_settle() {}
 
 inline void emu_set_m0(unsigned v) { emu::m0 = v; emu::m0_written = true; }

@@ -25,14 +25,14 @@
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
-// A kernel's static __shared__ arrays become statics (workgroups run one at a time).  A translation unit whose kernels
-// use the dynamic array instead (`extern __shared__ char smem[]`) defines EMU_DYNAMIC_LDS: the declaration then names an
-// ordinary global the harness provides.
-#ifdef EMU_DYNAMIC_LDS
-#define __shared__
-#else
+// A kernel's static __shared__ arrays become statics (workgroups run one at a time).  The dynamically sized LDS
+// (HODU_DYNAMIC_LDS(name) in the kernels) is one 160 KiB array that belongs to the workgroup that is running.
 #define __shared__ static
-#endif
+namespace emu {
+constexpr unsigned kLdsBytes = 160 * 1024;
+char *lds_base();
+}  // namespace emu
+#define HODU_DYNAMIC_LDS(name) char *const name = emu::lds_base()
 #define __align__(n) __attribute__((aligned(n)))
 
 struct dim3 {
