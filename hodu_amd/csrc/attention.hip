@@ -37,6 +37,7 @@
 #include "common.hpp"
 #include "device_types.hpp"
 #include "gemm_mfma_pipe.hpp"
+#include "gfx950_insn.hpp"
 
 namespace hodu {
 namespace {
@@ -298,15 +299,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     auto rescale_o = [&]() {
 #pragma unroll
         for (int j = 0; j < AT_D / 32; j++)
-            asm volatile("v_mul_f32 %0, %16, %0\n\tv_mul_f32 %1, %16, %1\n\tv_mul_f32 %2, %16, %2\n\tv_mul_f32 %3, %16, %3\n\t"
-                         "v_mul_f32 %4, %16, %4\n\tv_mul_f32 %5, %16, %5\n\tv_mul_f32 %6, %16, %6\n\tv_mul_f32 %7, %16, %7\n\t"
-                         "v_mul_f32 %8, %16, %8\n\tv_mul_f32 %9, %16, %9\n\tv_mul_f32 %10, %16, %10\n\tv_mul_f32 %11, %16, %11\n\t"
-                         "v_mul_f32 %12, %16, %12\n\tv_mul_f32 %13, %16, %13\n\tv_mul_f32 %14, %16, %14\n\tv_mul_f32 %15, %16, %15"
-                         : "+v"(o_acc[j][0]), "+v"(o_acc[j][1]), "+v"(o_acc[j][2]), "+v"(o_acc[j][3]), "+v"(o_acc[j][4]),
-                           "+v"(o_acc[j][5]), "+v"(o_acc[j][6]), "+v"(o_acc[j][7]), "+v"(o_acc[j][8]), "+v"(o_acc[j][9]),
-                           "+v"(o_acc[j][10]), "+v"(o_acc[j][11]), "+v"(o_acc[j][12]), "+v"(o_acc[j][13]),
-                           "+v"(o_acc[j][14]), "+v"(o_acc[j][15])
-                         : "v"(rescale));
+            mfma::scale16_in_place(o_acc[j], rescale);
     };
     // P of one 16-key slice (groups q = 2 sl and 2 sl + 1) in operand layout; adds the slice's row sums to l_blk
     auto probs = [&](const acc_t &sc, int sl, float &l_blk) {

@@ -72,6 +72,19 @@ template <int LIT> __device__ __forceinline__ void m0_set(unsigned base) {
 }
 __device__ __forceinline__ void m0_wait_state() { asm volatile("s_nop 0"); }
 
+// v[e] *= s for the 16 registers of an accumulator, in place.  Through the assembler because, written as C++ inside a
+// conditional, the product makes the compiler keep two copies of the accumulators around the branch and move one onto
+// the other in every iteration.
+template <class V16> __device__ __forceinline__ void scale16_in_place(V16 &v, float s) {
+    asm volatile("v_mul_f32 %0, %16, %0\n\tv_mul_f32 %1, %16, %1\n\tv_mul_f32 %2, %16, %2\n\tv_mul_f32 %3, %16, %3\n\t"
+                 "v_mul_f32 %4, %16, %4\n\tv_mul_f32 %5, %16, %5\n\tv_mul_f32 %6, %16, %6\n\tv_mul_f32 %7, %16, %7\n\t"
+                 "v_mul_f32 %8, %16, %8\n\tv_mul_f32 %9, %16, %9\n\tv_mul_f32 %10, %16, %10\n\tv_mul_f32 %11, %16, %11\n\t"
+                 "v_mul_f32 %12, %16, %12\n\tv_mul_f32 %13, %16, %13\n\tv_mul_f32 %14, %16, %14\n\tv_mul_f32 %15, %16, %15"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                   "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15])
+                 : "v"(s));
+}
+
 // Between a wavefront's LDS writes and its own reads of what other lanes of it wrote (or the other way round): the
 // lanes of a wavefront execute together and one wavefront's LDS operations complete in order, so no instruction is
 // needed -- only the compiler must not move the accesses across this point.

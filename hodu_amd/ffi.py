@@ -72,6 +72,26 @@ def _steps_array(steps):
     return (EpilogueStep * max(1, len(steps)))(*steps), len(steps)
 
 
+def declare_compute(lib: ctypes.CDLL):
+    """argument types of the compute entry points (everything in include/hodu_rocm_kernels.h that launches kernels)"""
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    szp = ctypes.POINTER(ctypes.c_size_t)
+    for dt in PRODUCT_DTYPES + list(FUSED_PRODUCTS):
+        for op in ("matmul", "dot"):
+            getattr(lib, f"hodu_rocm_{op}_{dt}").argtypes = [vp, vp, vp, vp, szp, sz]
+    for dt in EPILOGUE_DTYPES + list(FUSED_PRODUCTS):
+        for op in ("matmul", "dot"):
+            getattr(lib, f"hodu_rocm_{op}_{dt}_ex").argtypes = [vp, vp, vp, vp, szp, sz, ctypes.POINTER(EpilogueStep), sz]
+    lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
+    lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
+    lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
+    lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
+    lib.hodu_rocm_softmax_masked.argtypes = [vp, ci, vp, vp, szp, sz, ci, vp, ci, szp, sz]
+    lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
+    lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc.argtypes = [vp, vp, vp, vp, szp, sz]
+    lib.hodu_rocm_ctx_set_reference_sums.argtypes = [vp, ci]
+
+
 def load() -> ctypes.CDLL:
     """Load the built HIP library; raises if it is missing (build with `python -m hodu_amd.build`)."""
     global _lib
@@ -104,20 +124,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_rocm_timer_start.argtypes = [vp, vp]
     lib.hodu_rocm_timer_stop.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
     lib.hodu_rocm_timer_destroy.argtypes = [vp, vp]
-    for dt in PRODUCT_DTYPES + list(FUSED_PRODUCTS):
-        for op in ("matmul", "dot"):
-            getattr(lib, f"hodu_rocm_{op}_{dt}").argtypes = [vp, vp, vp, vp, szp, sz]
-    for dt in EPILOGUE_DTYPES + list(FUSED_PRODUCTS):
-        for op in ("matmul", "dot"):
-            getattr(lib, f"hodu_rocm_{op}_{dt}_ex").argtypes = [vp, vp, vp, vp, szp, sz, ctypes.POINTER(EpilogueStep), sz]
-    lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
-    lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
-    lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
-    lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
-    lib.hodu_rocm_softmax_masked.argtypes = [vp, ci, vp, vp, szp, sz, ci, vp, ci, szp, sz]
-    lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
-    lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc.argtypes = [vp, vp, vp, vp, szp, sz]
-    lib.hodu_rocm_ctx_set_reference_sums.argtypes = [vp, ci]
+    declare_compute(lib)
     _lib = lib
     return lib
 

@@ -17,8 +17,8 @@
 //     both sum in f32 with k ascending (the hardware's order inside one instruction is not architected; the tests that
 //     compare bit for bit use operands whose products and partial sums are exact);
 //   * global_load_lds_dwordx4: lane l copies 16 bytes from (base + lane offset + immediate) to LDS at M0 + immediate
-//     + 16 l: the immediate moves both addresses.  M0 is a per-wavefront register, kept per lane thread here (every
-//     lane writes the same value); a DMA before any M0 write aborts;
+//     + 16 l: the immediate moves both addresses.  M0 is a per-wavefront register, kept per lane here (every lane
+//     writes the same value); a DMA before any M0 write aborts;
 //   * when a DMA's bytes arrive is the hardware's business between the issue and the s_waitcnt vmcnt(n) that leaves at
 //     most n of the wavefront's loads outstanding.  Two models, chosen by emu_dma_lazy(): at issue (0, the default),
 //     and as late as allowed (1) -- queued per lane and written by the s_waitcnt that retires them, oldest first; what
@@ -53,30 +53,31 @@ inline char *lds_at(unsigned addr32, unsigned bytes) {
     }
     return lds_base() + off;
 }
-inline thread_local unsigned m0 = 0;
-inline thread_local bool m0_written = false;
-struct PendingDma { const char *src; unsigned lds_addr; };
-inline thread_local std::vector<PendingDma> dma_queue;
+// M0, the flag that it has been written and the queue of loads in flight live in the lane (hip_runtime.h: Lane)
+#define EMU_M0 (emu::t_lane->m0)
+#define EMU_M0_WRITTEN (emu::t_lane->m0_written)
+#define EMU_DMA_QUEUE (emu::t_lane->dma_queue)
 
 inline unsigned lane_id() { return flat_tid() % kWave; }
 inline void dma16_now(const char *src, unsigned lds_addr) { memcpy(lds_at(lds_addr, 16), src, 16); }
 inline void dma16(const char *src, unsigned wave_lds_addr) {
-    if (!m0_written) {
+    if (!EMU_M0_WRITTEN) {
         fprintf(stderr, "emu: LDS-DMA before any M0 write\n");
         abort();
     }
     const unsigned dst = wave_lds_addr + 16 * lane_id();
     (void)lds_at(dst, 16);  // the address is checked at issue under both models
-    if (dma_lazy()) dma_queue.push_back({src, dst});
+    if (dma_lazy()) EMU_DMA_QUEUE.push_back({src, dst});
     else dma16_now(src, dst);
 }
 // s_waitcnt: vmcnt is bits 3:0 and 15:14 of the immediate
 inline void waitcnt(int imm) {
     const size_t vm = (size_t)((imm & 15) | (((imm >> 14) & 3) << 4)) + (dma_lazy() == 2 ? 1 : 0);
-    if (dma_queue.size() > vm) {
-        const size_t retire = dma_queue.size() - vm;
-        for (size_t i = 0; i < retire; i++) dma16_now(dma_queue[i].src, dma_queue[i].lds_addr);
-        dma_queue.erase(dma_queue.begin(), dma_queue.begin() + (long)retire);
+    auto &queue = EMU_DMA_QUEUE;
+    if (queue.size() > vm) {
+        const size_t retire = queue.size() - vm;
+        for (size_t i = 0; i < retire; i++) dma16_now(queue[i].src, queue[i].lds_addr);
+        queue.erase(queue.begin(), queue.begin() + (long)retire);
     }
 }
 
@@ -84,14 +85,13 @@ inline void waitcnt(int imm) {
 // alternate between two sets of slots, so the next exchange's deposits cannot overwrite what a slower lane still
 // reads and one wait per exchange is enough.  All 64 lanes must be running.
 constexpr int kWideBytes = 64;
-inline thread_local unsigned wide_phase = 0;
 template <class T> inline const unsigned char (*wave_deposit(const T &mine))[kWideBytes] {
     static_assert(sizeof(T) <= kWideBytes, "exchange slot");
     Block *b = current();
     const unsigned tid = flat_tid(), w = tid / kWave, lane = tid % kWave;
-    auto slots = b->wide[wide_phase++ & 1][w];
+    auto slots = b->wide[t_lane->wide_phase++ & 1][w];
     memcpy(slots[lane], &mine, sizeof(T));
-    b->wave[w].wait();
+    wave_meet();
     return slots;
 }
 
@@ -106,68 +106,43 @@ typedef float vf32x16 __attribute__((ext_vector_type(16)));
 // (OPB bytes) of row / column r = lane % ROWS, starting at k = KPL * (lane / ROWS); it then holds column r of D rows
 //   4 g + e                    (16 x 16: e = 0..3, g = lane / 16)
 //   8 (e / 4) + 4 g + e % 4    (32 x 32: e = 0..15, g = lane / 32)
-//   4 e + g                    (the f64 16 x 16 x 4 form, F64ROWS: its registers step through the rows by four)
-// `term(pa, pb, k)` is one product in the accumulate type, from the two lanes' raw operand bytes.
-template <int ROWS, int KPL, int OPB, class AccT, bool F64ROWS = false, class Acc, class Term>
-inline void mfma_model(const void *a, const void *b, Acc &c, Term term) {
+//   4 e + g                    (the f64 16 x 16 x 4 form: its registers step through the rows by four)
+// The sums themselves are in emu_models.cpp (compiled with optimisation; this header is not): products of the two
+// lanes' operand elements in the accumulate type, k ascending.
+enum MfmaKind { kMfmaBf16, kMfmaF16, kMfmaF32, kMfmaF64, kMfmaI8, kMfmaF8E4M3, kMfmaF8E5M2 };
+// slots: what the 64 lanes deposited (first operand at byte 0, second at byte opb); acc: this lane's registers
+void mfma_sums(int rows, int kpl, int opb, MfmaKind kind, bool f64_rows, const unsigned char (*slots)[64], unsigned lane, void *acc);
+
+template <int ROWS, int KPL, int OPB, MfmaKind KIND, bool F64ROWS = false, class Acc>
+inline void mfma_model(const void *a, const void *b, Acc &c) {
     static_assert(2 * OPB <= kWideBytes, "both operands in one exchange slot");
     struct Ops { unsigned char a[OPB], b[OPB]; };
-    constexpr int KG = 64 / ROWS, NE = ROWS * ROWS / 64;
     Ops mine;
     memcpy(mine.a, a, OPB);
     memcpy(mine.b, b, OPB);
     const auto slots = wave_deposit(mine);
-    const unsigned lane = lane_id(), r = lane % ROWS, g = lane / ROWS;
-    for (int e = 0; e < NE; e++) {
-        const unsigned i = F64ROWS ? 4 * e + g : ROWS == 16 ? 4 * g + e : 8 * (e / 4) + 4 * g + e % 4;
-        AccT sum = 0;
-        for (unsigned kg = 0; kg < (unsigned)KG; kg++) {
-            const unsigned char *pa = slots[ROWS * kg + i];        // lane (i, kg): A[i][KPL kg ..], its first operand
-            const unsigned char *pb = slots[ROWS * kg + r] + OPB;  // lane (r, kg): B[KPL kg ..][r], its second operand
-            for (int k = 0; k < KPL; k++) sum += term(pa, pb, k);
-        }
-        c[e] += sum;
-    }
+    mfma_sums(ROWS, KPL, OPB, KIND, F64ROWS, slots, lane_id(), &c);
 }
-template <int ROWS, class Acc, class Widen> inline void mfma_8k(const vu32x4 &a, const vu32x4 &b, Acc &c, Widen widen) {
-    mfma_model<ROWS, 8, 16, float>(&a, &b, c, [&](const unsigned char *pa, const unsigned char *pb, int k) {
-        uint16_t x, y;
-        memcpy(&x, pa + 2 * k, 2);
-        memcpy(&y, pb + 2 * k, 2);
-        return widen(x) * widen(y);
-    });
+template <int ROWS, MfmaKind KIND, class Acc> inline void mfma_8k(const vu32x4 &a, const vu32x4 &b, Acc &c) {
+    mfma_model<ROWS, 8, 16, KIND>(&a, &b, c);
 }
 template <int ROWS, class Acc> inline Acc mfma_f32(float a, float b, Acc c) {
-    mfma_model<ROWS, 1, 4, float>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int) {
-        float x, y;
-        memcpy(&x, pa, 4);
-        memcpy(&y, pb, 4);
-        return x * y;
-    });
+    mfma_model<ROWS, 1, 4, kMfmaF32>(&a, &b, c);
     return c;
 }
 template <class Acc> inline Acc mfma_f64_16(double a, double b, Acc c) {
-    mfma_model<16, 1, 8, double, true>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int) {
-        double x, y;
-        memcpy(&x, pa, 8);
-        memcpy(&y, pb, 8);
-        return x * y;
-    });
+    mfma_model<16, 1, 8, kMfmaF64, true>(&a, &b, c);
     return c;
 }
 template <int ROWS, class Vec, class Acc> inline Acc mfma_i8(const Vec &a, const Vec &b, Acc c) {
     static_assert(sizeof(Vec) == 16, "16 bytes of k per lane");
-    mfma_model<ROWS, 16, 16, int>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int k) {
-        return (int)(int8_t)pa[k] * (int)(int8_t)pb[k];
-    });
+    mfma_model<ROWS, 16, 16, kMfmaI8>(&a, &b, c);
     return c;
 }
 // the 8-bit float forms (v_mfma_scale_f32_*_f8f6f4 with unit scales): 32 bytes of k per lane; FMT 0 = e4m3, 1 = e5m2
 template <int ROWS, int FMT, class Vec, class Acc> inline void mfma_f8(const Vec &a, const Vec &b, Acc &c) {
     static_assert(sizeof(Vec) == 32, "32 bytes of k per lane");
-    mfma_model<ROWS, 32, 32, float>(&a, &b, c, [](const unsigned char *pa, const unsigned char *pb, int k) {
-        return FMT == 0 ? f8_decode<4, 3>(pa[k]) * f8_decode<4, 3>(pb[k]) : f8_decode<5, 2>(pa[k]) * f8_decode<5, 2>(pb[k]);
-    });
+    mfma_model<ROWS, 32, 32, FMT == 0 ? kMfmaF8E4M3 : kMfmaF8E5M2>(&a, &b, c);
 }
 
 // v_dot2_f32_bf16: c + a.x * b.x + a.y * b.y
@@ -305,13 +280,13 @@ struct Any {
 #define __builtin_amdgcn_ds_read_tr8_b64_v2i32(p) (emu::ds_read_tr<1, int __attribute__((ext_vector_type(2)))>((const void *)(p)))
 #define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, scale, hi) emu::cvt_pk_bf16_fp8(w, scale, hi)
 #define __builtin_amdgcn_global_load_lds(g, l, size, off, aux) \
-    (emu::m0_written = true, emu::dma16((const char *)(g), (unsigned)(uintptr_t)(l)))
+    (EMU_M0_WRITTEN = true, emu::dma16((const char *)(g), (unsigned)(uintptr_t)(l)))
 #define EMU_MFMA(ROWS, WIDEN, a, b, c) \
-    ([&] { auto acc_ = (c); emu::mfma_8k<ROWS>(__builtin_bit_cast(emu::vu32x4, a), __builtin_bit_cast(emu::vu32x4, b), acc_, WIDEN); return acc_; }())
-#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) EMU_MFMA(16, emu::widen_bf16, a, b, c)
-#define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) EMU_MFMA(16, emu::widen_f16, a, b, c)
-#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) EMU_MFMA(32, emu::widen_bf16, a, b, c)
-#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) EMU_MFMA(32, emu::widen_f16, a, b, c)
+    ([&] { auto acc_ = (c); emu::mfma_8k<ROWS, WIDEN>(__builtin_bit_cast(emu::vu32x4, a), __builtin_bit_cast(emu::vu32x4, b), acc_); return acc_; }())
+#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) EMU_MFMA(16, emu::kMfmaBf16, a, b, c)
+#define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) EMU_MFMA(16, emu::kMfmaF16, a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) EMU_MFMA(32, emu::kMfmaBf16, a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) EMU_MFMA(32, emu::kMfmaF16, a, b, c)
 #define __builtin_amdgcn_perm(s0, s1, sel) (emu::perm_b32(s0, s1, sel))
 #define __builtin_amdgcn_cvt_pk_f32_fp8(word, hi) (emu::cvt_pk_f32_fp8((unsigned)(word), hi))
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) (emu::mfma_f32<32>(a, b, c))
@@ -336,23 +311,26 @@ namespace mfma {
 typedef float f32x4_acc_t __attribute__((ext_vector_type(4)));
 typedef unsigned emu_u32x4 __attribute__((ext_vector_type(4)));
 
-inline void mfma16x16x32_bf16(const emu_u32x4 &a, const emu_u32x4 &b, f32x4_acc_t &c) { emu::mfma_8k<16>(a, b, c, emu::widen_bf16); }
-inline void mfma16x16x32_f16(const emu_u32x4 &a, const emu_u32x4 &b, f32x4_acc_t &c) { emu::mfma_8k<16>(a, b, c, emu::widen_f16); }
+inline void mfma16x16x32_bf16(const emu_u32x4 &a, const emu_u32x4 &b, f32x4_acc_t &c) { emu::mfma_8k<16, emu::kMfmaBf16>(a, b, c); }
+inline void mfma16x16x32_f16(const emu_u32x4 &a, const emu_u32x4 &b, f32x4_acc_t &c) { emu::mfma_8k<16, emu::kMfmaF16>(a, b, c); }
 typedef int emu_i32x8 __attribute__((ext_vector_type(8)));
 template <int FMT> inline void mfma16x16x128_f8(const emu_i32x8 &a, const emu_i32x8 &b, f32x4_acc_t &c) { emu::mfma_f8<16, FMT>(a, b, c); }
 inline void mfma_results_settle() {}
 
-inline void emu_set_m0(unsigned v) { emu::m0 = v; emu::m0_written = true; }
-inline void dma16_raw(const char *gptr, unsigned lds_addr) { emu_set_m0(lds_addr); emu::dma16(gptr, emu::m0); }
-inline void dma16_sbase(const char *sbase, unsigned voff, unsigned lds_addr) { emu_set_m0(lds_addr); emu::dma16(sbase + voff, emu::m0); }
+inline void emu_set_m0(unsigned v) { EMU_M0 = v; EMU_M0_WRITTEN = true; }
+inline void dma16_raw(const char *gptr, unsigned lds_addr) { emu_set_m0(lds_addr); emu::dma16(gptr, EMU_M0); }
+inline void dma16_sbase(const char *sbase, unsigned voff, unsigned lds_addr) { emu_set_m0(lds_addr); emu::dma16(sbase + voff, EMU_M0); }
 template <int IMM> inline void dma16_imm(const char *sbase, unsigned voff) {
     static_assert(IMM >= 0 && IMM < 4096, "the instruction's offset field as these kernels use it: 12 bits, not negative");
-    emu::dma16(sbase + voff + IMM, emu::m0 + (unsigned)IMM);
+    emu::dma16(sbase + voff + IMM, EMU_M0 + (unsigned)IMM);
 }
 template <int LIT> inline void m0_set(unsigned base) { emu_set_m0(base + (unsigned)LIT); }
 inline void m0_wait_state() {}
-// the lanes of a wavefront are separate threads here: where the kernels count on their executing together, they meet
-inline void wave_lds_fence() { emu::current()->wave[emu::flat_tid() / emu::kWave].wait(); }
+template <class V16> inline void scale16_in_place(V16 &v, float s) {
+    for (int e = 0; e < 16; e++) v[e] *= s;
+}
+// the lanes of a wavefront run one after the other here: where the kernels count on their executing together, they meet
+inline void wave_lds_fence() { emu::wave_meet(); }
 
 }  // namespace mfma
 }  // namespace hodu

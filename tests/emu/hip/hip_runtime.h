@@ -2,20 +2,27 @@
 // (no matrix-core, no LDS-DMA) kernels of hodu_amd/csrc use, so that a kernel's UNMODIFIED source can be compiled
 // for the host and run there -- a CPU build for checking indexing, masks and reductions without a GPU.
 //
-// Execution model: a launch runs its workgroups one after the other; the threads of a workgroup are real host
-// threads (so __shared__ can be a plain static), grouped into wavefronts of 64 whose cross-lane operations
-// (__shfl_xor) exchange through a per-wavefront buffer between two barriers.  Arithmetic is the host's: expf / exp
+// Execution model: a launch runs its workgroups one after the other (so __shared__ can be a plain static).  A
+// wavefront is a host thread; its 64 lanes are contexts of their own on that thread, each run until it reaches a point
+// where the wavefront has to meet (a cross-lane operation such as __shfl_xor, which exchanges through a per-wavefront
+// buffer) or the workgroup has to (__syncthreads), and resumed when the others have arrived.  Arithmetic is the host's: expf / exp
 // are libm's, bf16 / f16 conversions the host compiler's (round to nearest even), so results agree with the device
 // to rounding, not to the bit.  The 8-bit float conversions are written out below.  Nothing here knows about MFMA,
 // DPP, LDS-DMA or buffer instructions; stand-ins for
 // those the tile kernels use are in gfx950_insn_emu.hpp, for the translation units that want them.
 #pragma once
 
+#include <sys/mman.h>
+#include <ucontext.h>
+
 #include <cmath>
+#include <condition_variable>
 #include <cstdint>
 #include <cstdio>
-#include <condition_variable>
+#include <cstdlib>
 #include <cstring>
+#include <functional>
+#include <memory>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -54,7 +61,7 @@ inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { ret
 namespace emu {
 constexpr int kWave = 64, kMaxBlock = 1024;
 
-// a barrier whose parties may leave for good: a thread that returns from the kernel no longer counts, as on the GPU
+// a barrier whose parties may leave for good (here: the wavefronts' threads of one workgroup)
 class Barrier {
 public:
     void reset(unsigned parties) { parties_ = parties; waiting_ = 0; phase_ = 0; }
@@ -84,14 +91,102 @@ private:
     unsigned parties_ = 0, waiting_ = 0, phase_ = 0;
 };
 
+// A lane is a context of its own (stack, registers) that runs until it reaches a point where the wavefront or the
+// workgroup has to meet, and is resumed when everyone it waits for has arrived; a lane that has returned from the
+// kernel is waited for by nobody, as on the GPU.
+enum LaneState { kRunnable, kAtWaveMeet, kAtBlockBarrier, kDone };
+struct PendingDma { const char *src; unsigned lds_addr; };
+struct Lane {
+    ucontext_t uc;
+    LaneState state = kDone;
+    emu_uint3 tid;
+    unsigned flat = 0;
+    // per-wavefront registers and queues of the LDS-DMA model (gfx950_insn_emu.hpp), kept per lane
+    unsigned m0 = 0;
+    bool m0_written = false;
+    unsigned wide_phase = 0;
+    std::vector<PendingDma> dma_queue;
+};
 struct Block {
-    Barrier all;                       // __syncthreads
-    Barrier wave[kMaxBlock / kWave];   // cross-lane exchanges
+    Barrier all;  // __syncthreads, between the wavefronts' threads
     alignas(16) unsigned char xchg[kMaxBlock / kWave][kWave][16];
     alignas(16) unsigned char wide[2][kMaxBlock / kWave][kWave][64];  // operands of wavefront-wide instructions, two sets
 };
+struct WaveRun {
+    ucontext_t sched;
+    Lane lanes[kWave];
+    const std::function<void()> *kernel = nullptr;
+};
 inline Block *&current() { static Block *b = nullptr; return b; }
-inline thread_local emu_uint3 t_idx, b_idx, b_dim, g_dim;
+inline thread_local Lane *t_lane = nullptr;
+inline thread_local WaveRun *t_wave = nullptr;
+inline thread_local emu_uint3 b_idx, b_dim, g_dim;
+
+// stacks of all lanes of a workgroup, allocated once, an inaccessible page below each
+constexpr size_t kStackBytes = 1u << 20, kStackStride = kStackBytes + 4096;
+inline char *lane_stack(unsigned flat) {
+    static char *pool = [] {
+        void *p = mmap(nullptr, kStackStride * kMaxBlock, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+        if (p == MAP_FAILED) { perror("emu: lane stacks"); abort(); }
+        for (unsigned i = 0; i < (unsigned)kMaxBlock; i++) mprotect((char *)p + i * kStackStride, 4096, PROT_NONE);
+        return (char *)p;
+    }();
+    return pool + flat * kStackStride + 4096;
+}
+inline void lane_entry() {
+    (*t_wave->kernel)();
+    t_lane->state = kDone;  // returning resumes the scheduler (uc_link)
+}
+inline void lane_yield(LaneState why) {
+    t_lane->state = why;
+    swapcontext(&t_lane->uc, &t_wave->sched);
+}
+// every running lane of the wavefront arrives here before any goes on
+inline void wave_meet() { lane_yield(kAtWaveMeet); }
+
+inline void run_wave(Block &blk, const std::function<void()> &kernel, unsigned w, dim3 block) {
+    std::unique_ptr<WaveRun> owned(new WaveRun);
+    WaveRun &run = *owned;
+    run.kernel = &kernel;
+    t_wave = &run;
+    for (unsigned l = 0; l < (unsigned)kWave; l++) {
+        Lane &ln = run.lanes[l];
+        const unsigned t = w * kWave + l;
+        ln.flat = t;
+        ln.tid.x = t % block.x; ln.tid.y = (t / block.x) % block.y; ln.tid.z = t / (block.x * block.y);
+        ln.m0 = 0; ln.m0_written = false; ln.wide_phase = 0; ln.dma_queue.clear();
+        getcontext(&ln.uc);
+        ln.uc.uc_stack.ss_sp = lane_stack(t);
+        ln.uc.uc_stack.ss_size = kStackBytes;
+        ln.uc.uc_link = &run.sched;
+        makecontext(&ln.uc, lane_entry, 0);
+        ln.state = kRunnable;
+    }
+    for (;;) {
+        for (unsigned l = 0; l < (unsigned)kWave; l++)
+            if (run.lanes[l].state == kRunnable) {
+                t_lane = &run.lanes[l];
+                swapcontext(&run.sched, &run.lanes[l].uc);
+            }
+        unsigned meet = 0, barrier = 0, done = 0;
+        for (unsigned l = 0; l < (unsigned)kWave; l++) {
+            meet += run.lanes[l].state == kAtWaveMeet;
+            barrier += run.lanes[l].state == kAtBlockBarrier;
+            done += run.lanes[l].state == kDone;
+        }
+        if (done == (unsigned)kWave) break;
+        if (meet != 0 && barrier != 0) {
+            fprintf(stderr, "emu: wavefront %u diverged: %u lanes at a wavefront-wide instruction, %u at a workgroup barrier\n", w, meet, barrier);
+            abort();
+        }
+        if (barrier != 0) blk.all.wait();
+        for (unsigned l = 0; l < (unsigned)kWave; l++)
+            if (run.lanes[l].state != kDone) run.lanes[l].state = kRunnable;
+    }
+    t_lane = nullptr;
+    t_wave = nullptr;
+    blk.all.leave();
+}
 
 template <class K, class... Args> void launch(K kernel, dim3 grid, dim3 block, Args... args) {
     const unsigned nthreads = block.x * block.y * block.z;
@@ -99,40 +194,39 @@ template <class K, class... Args> void launch(K kernel, dim3 grid, dim3 block, A
         fprintf(stderr, "emu: a workgroup of %u threads is not whole wavefronts\n", nthreads);
         abort();
     }
-    Block blk;
+    static Block blk;  // (workgroups, and launches, run one at a time)
     current() = &blk;
+    const std::function<void()> call = [=] { kernel(args...); };
+    const unsigned waves = nthreads / kWave;
     for (unsigned bz = 0; bz < grid.z; bz++)
         for (unsigned by = 0; by < grid.y; by++)
             for (unsigned bx = 0; bx < grid.x; bx++) {
-                blk.all.reset(nthreads);
-                for (unsigned w = 0; w < nthreads / kWave; w++) blk.wave[w].reset(kWave);
+                blk.all.reset(waves);
+                auto body = [&, bx, by, bz](unsigned w) {
+                    b_idx.x = bx; b_idx.y = by; b_idx.z = bz;
+                    b_dim.x = block.x; b_dim.y = block.y; b_dim.z = block.z;
+                    g_dim.x = grid.x; g_dim.y = grid.y; g_dim.z = grid.z;
+                    run_wave(blk, call, w, block);
+                };
                 std::vector<std::thread> pool;
-                pool.reserve(nthreads);
-                for (unsigned t = 0; t < nthreads; t++)
-                    pool.emplace_back([=, &blk] {
-                        t_idx.x = t % block.x; t_idx.y = (t / block.x) % block.y; t_idx.z = t / (block.x * block.y);
-                        b_idx.x = bx; b_idx.y = by; b_idx.z = bz;
-                        b_dim.x = block.x; b_dim.y = block.y; b_dim.z = block.z;
-                        g_dim.x = grid.x; g_dim.y = grid.y; g_dim.z = grid.z;
-                        kernel(args...);
-                        blk.wave[t / kWave].leave();
-                        blk.all.leave();
-                    });
+                pool.reserve(waves - 1);
+                for (unsigned w = 1; w < waves; w++) pool.emplace_back(body, w);
+                body(0);
                 for (auto &th : pool) th.join();
             }
     current() = nullptr;
 }
-inline unsigned flat_tid() { return t_idx.x + b_dim.x * (t_idx.y + b_dim.y * t_idx.z); }
+inline unsigned flat_tid() { return t_lane->flat; }
 }  // namespace emu
 
-#define threadIdx (emu::t_idx)
+#define threadIdx (emu::t_lane->tid)
 #define blockIdx (emu::b_idx)
 #define blockDim (emu::b_dim)
 #define gridDim (emu::g_dim)
 // the parenthesised kernel name of a template instantiation arrives as one macro argument
 #define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) emu::launch(kernel, grid, block, __VA_ARGS__)
 
-inline void __syncthreads() { emu::current()->all.wait(); }
+inline void __syncthreads() { emu::lane_yield(emu::kAtBlockBarrier); }
 
 // every lane of the wavefront that is still running calls it; a lane that has returned from the kernel is not waited
 // for (its slot keeps what it wrote last)
@@ -142,10 +236,10 @@ template <class T> inline T __shfl_xor(T v, int lane_mask, int width = 64) {
     emu::Block *b = emu::current();
     const unsigned tid = emu::flat_tid(), w = tid / emu::kWave, lane = tid % emu::kWave;
     memcpy(b->xchg[w][lane], &v, sizeof(T));
-    b->wave[w].wait();
+    emu::wave_meet();
     T out;
     memcpy(&out, b->xchg[w][(lane ^ (unsigned)lane_mask) % emu::kWave], sizeof(T));
-    b->wave[w].wait();
+    emu::wave_meet();
     return out;
 }
 

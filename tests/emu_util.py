@@ -1,15 +1,16 @@
-"""Builds and loads the CPU build of the library's plain kernels (tests/emu): the unmodified sources of api.cpp,
-metadata.cpp, softmax.hip, cast.hip, reduce.hip, gemm_generic.hip and gemm_refsum.hip compiled for the host against a stand-in for
-<hip/hip_runtime.h> that runs a workgroup as host threads.  Test infrastructure: what it proves is indexing, masking,
-reduction structure and the entry points' argument handling -- arithmetic is the host's, so results are compared at the
-parity tolerances, bit for bit only where the kernel's arithmetic is integer or pure bit manipulation.  In that build
-the matrix-core launchers answer UNSUPPORTED, which routes every product to the generic kernel.
+"""Builds and loads the CPU build of the library's kernels (tests/emu): their unmodified sources compiled for the host
+against a stand-in for <hip/hip_runtime.h> that runs a wavefront as a host thread and its lanes as contexts on it, and
+against CPU models of the gfx950 instructions they use (tests/emu/gfx950_insn_emu.hpp).  Test infrastructure.
 
-A second library (build(mfma=True), Emu(mfma=True)) adds the matrix-core tile kernels of bf16, f16 and f8e4m3 weights --
-gemm_mfma.hip, gemm_mfma_{bf16,f16}.hip, gemm_mfma_mi16_{bf16,f16}.hip, gemm_mfma_w8a16.hip, unmodified -- against the instruction
-models of tests/emu/gfx950_insn_emu.hpp (MFMA lane layouts, LDS-DMA with M0 and the immediate offset, the LDS
-transpose reads, vmcnt).  Those kernels' sums are f32 sums of exact products, so on operands whose partial sums are
-exact the comparison with the oracle is bit for bit."""
+Two libraries.  build() / Emu: api.cpp, metadata.cpp, softmax.hip, cast.hip, reduce.hip, gemm_generic.hip and
+gemm_refsum.hip -- the kernels without matrix-core or LDS-DMA instructions; every other launcher answers UNSUPPORTED,
+which routes every product to the generic kernel.  Emu takes numpy arrays as operands.  build(mfma=True) / EmuContext:
+all kernel families, with the real variant selection; EmuContext is hodu_amd.ffi.Context over that library, so the
+GPU tests' helpers and test functions run against it unchanged.
+
+Arithmetic is the host's (libm's expf, one summation order inside an MFMA), so float results are compared at the
+parity tolerances and bit for bit only where the kernels' arithmetic is integer, pure bit manipulation, or exact by
+the choice of operands."""
 import ctypes
 import os
 import shutil
@@ -17,6 +18,8 @@ import subprocess
 from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
+
+from hodu_amd import ffi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EMU = os.path.join(ROOT, "tests", "emu")
@@ -28,7 +31,7 @@ LIB = os.path.join(OUT, "libhodu_emu.so")
 MFMA_SOURCES = [os.path.join(CSRC, f) for f in ("gemm_mfma.hip", "gemm_mfma_bf16.hip", "gemm_mfma_mi16_bf16.hip", "gemm_mfma_w8a16.hip",
                                                 "gemm_mfma_f16.hip", "gemm_mfma_mi16_f16.hip", "gemm_mfma_f32.hip", "gemm_mfma_i8.hip",
                                                 "gemm_mfma_i8_out.hip", "gemm_mfma_u8_out.hip", "gemm_mfma_f8.hip", "skinny.hip",
-                                                "gemv.hip", "gemv_rows.hip", "small_f32.hip", "gemm_f64.hip")]
+                                                "gemv.hip", "gemv_rows.hip", "small_f32.hip", "gemm_f64.hip", "attention.hip")]
 MFMA_LIB = os.path.join(OUT, "libhodu_emu_mfma.so")
 
 
@@ -40,7 +43,7 @@ def compiler():
 
 
 def _newest_input():
-    paths = list(SOURCES) + list(MFMA_SOURCES) + [os.path.join(EMU, "hip", "hip_runtime.h"), os.path.join(EMU, "gfx950_insn_emu.hpp"),
+    paths = list(SOURCES) + list(MFMA_SOURCES) + [os.path.join(EMU, "hip", "hip_runtime.h"), os.path.join(EMU, "gfx950_insn_emu.hpp"), os.path.join(EMU, "emu_models.cpp"),
                                                   os.path.join(ROOT, "include", "hodu_rocm_kernels.h"), os.path.abspath(__file__)]
     paths += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
     return max(os.path.getmtime(p) for p in paths)
@@ -64,7 +67,8 @@ def build(mfma=False):
     if mfma:
         # the plain kernels keep their static __shared__ arrays; only the runtime and the tile kernels see the models
         jobs = [(src, ".mfma" if src.endswith("emu_runtime.cpp") else "", ["-O0"] + (with_models if src.endswith("emu_runtime.cpp") else []))
-                for src in SOURCES] + [(src, ".mfma", ["-O0"] + with_models) for src in MFMA_SOURCES]
+                for src in SOURCES] + [(src, ".mfma", ["-O0"] + with_models) for src in MFMA_SOURCES] + \
+               [(os.path.join(EMU, "emu_models.cpp"), ".mfma", ["-O2", "-ffp-contract=off"])]
 
     def one(job):
         src, tag, extra = job
@@ -85,6 +89,29 @@ def build(mfma=False):
         raise RuntimeError(f"link of the CPU build failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, lib)
     return lib
+
+
+HOST_LIB = os.path.join(OUT, "libhodu_emu_host.so")
+
+
+def build_host():
+    """the host mirror's compiled library (hodu_amd/host/capi.cpp, unmodified) linked against the CPU build of all
+    kernels instead of the real kernel library; returns its path (None: no host clang)"""
+    kernels = build(mfma=True)
+    if kernels is None:
+        return None
+    host_dir = os.path.join(ROOT, "hodu_amd", "host")
+    inputs = [os.path.join(host_dir, f) for f in os.listdir(host_dir)] + [kernels]
+    if os.path.exists(HOST_LIB) and os.path.getmtime(HOST_LIB) > max(os.path.getmtime(p) for p in inputs):
+        return HOST_LIB
+    tmp = HOST_LIB + f".{os.getpid()}.tmp"
+    cmd = [compiler(), "-std=c++17", "-O1", "-fPIC", "-shared", f"-I{os.path.join(ROOT, 'include')}", f"-I{host_dir}",
+           os.path.join(host_dir, "capi.cpp"), "-o", tmp, f"-L{OUT}", "-lhodu_emu_mfma", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host mirror over the CPU build failed to build:\n{r.stderr[-4000:]}")
+    os.replace(tmp, HOST_LIB)
+    return HOST_LIB
 
 
 DTYPE_ID = {"bool": 0, "f8e4m3": 1, "f8e5m2": 2, "bf16": 3, "f16": 4, "f32": 5, "f64": 6, "u8": 7, "u16": 8, "u32": 9,
@@ -223,40 +250,91 @@ class GuardedBuffer:
             self.base = None
 
 
-class EmuContext(Emu):
-    """upload / alloc / fill / product / download / last_kernel / force_tile with hodu_amd.ffi.Context's signatures"""
+class EmuContext(ffi.Context):
+    """hodu_amd.ffi.Context over the CPU build: the same Python methods (product, product_ex, cast, sum, softmax, ..,
+    with their host-side extent checks) calling the same entry points of api.cpp, with "device" buffers that are host
+    memory between inaccessible pages.  The GPU tests' helpers and test functions run against it unchanged."""
 
-    def __init__(self, tight="end"):
-        super().__init__(mfma=True)
+    def __init__(self, tight="end", mfma=True):
+        path = build(mfma)
+        if path is None:
+            raise RuntimeError("no host clang++ to build tests/emu with")
+        self.lib = lib = ctypes.CDLL(path)
+        ffi.declare_compute(lib)
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        lib.emu_ctx_create.restype = vp
+        lib.emu_ctx_destroy.argtypes = [vp]
+        lib.emu_last_kernel.restype = ctypes.c_char_p
+        lib.emu_last_kernel.argtypes = [vp]
+        lib.emu_last_error.restype = ctypes.c_char_p
+        lib.emu_unsupported_first.restype = ctypes.c_char_p
+        lib.emu_force_tile.argtypes = [vp, ci]
+        lib.emu_force_splitk.argtypes = [vp, ci]
+        lib.emu_lds_fill.argtypes = [ci]
+        if mfma:
+            lib.emu_dma_lazy.argtypes = [ci]
+        self.handle = lib.emu_ctx_create()
+        self.device = 0
         self.tight = tight
 
-    def upload(self, arr):
-        arr = np.ascontiguousarray(arr)
-        buf = GuardedBuffer(arr.nbytes, self.tight)
-        buf.array(np.uint8)[:] = arr.view(np.uint8).ravel()
-        return buf
+    @property
+    def debug(self):
+        raise RuntimeError("the hooks library has no CPU build")
 
+    def close(self):
+        if self.handle is not None:
+            self.lib.emu_ctx_destroy(self.handle)
+            self.handle = None
+
+    def _check(self, rc):
+        if rc != 0:
+            raise ffi.HoduRocmError(rc, self.lib.emu_last_error().decode())
+        if self.lib.emu_unsupported_hits() != 0:
+            first = self.lib.emu_unsupported_first().decode()
+            self.lib.emu_unsupported_reset()
+            raise AssertionError(f"{self.last_kernel()} reached an instruction without a CPU stand-in: {first}")
+
+    # memory
     def alloc(self, nbytes):
         return GuardedBuffer(nbytes, self.tight)
+
+    def upload(self, host):
+        host = np.ascontiguousarray(host)
+        buf = GuardedBuffer(host.nbytes, self.tight)
+        buf.array(np.uint8)[:] = host.view(np.uint8).ravel()
+        return buf
+
+    def upload_into(self, buf, host, first_byte=0):
+        host = np.ascontiguousarray(host).view(np.uint8).ravel()
+        buf.array(np.uint8)[first_byte:first_byte + host.size] = host
+
+    def download(self, buf, dtype, count=None, first=0):
+        dtype = np.dtype(dtype)
+        n = buf.nbytes // dtype.itemsize - first if count is None else int(count)
+        if first < 0 or n < 0 or (first + n) * dtype.itemsize > buf.nbytes:
+            raise ffi.HoduRocmError(ffi.INVALID_ARG, "download: the range lies outside the buffer")
+        return buf.array(np.uint8)[first * dtype.itemsize:(first + n) * dtype.itemsize].view(dtype).copy()
 
     def fill(self, buf, byte):
         buf.array(np.uint8)[:] = byte
 
-    def download(self, buf, dtype, count=None):
-        return buf.array(dtype, count).copy()
+    def sync(self):
+        pass
 
-    def product(self, op, name, a, b, out, md):
-        fn = getattr(self.lib, f"hodu_rocm_{op}_{name}")
-        fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.POINTER(ctypes.c_size_t), ctypes.c_size_t]
-        arr, n = self._md(md)
-        self._check(fn(self.ctx, a.ptr, b.ptr, out.ptr, arr, n), f"{op}_{name}")
+    # hooks and diagnostics
+    def force_tile(self, tile):
+        self.lib.emu_force_tile(self.handle, int(tile))
 
-    def product_ex(self, op, name, a, b, out, md, steps):
-        """steps: hodu_amd.ffi.EpilogueStep values (ffi.add_row / mul_scalar / relu accept a GuardedBuffer)"""
-        steps = list(steps)
-        fn = getattr(self.lib, f"hodu_rocm_{op}_{name}_ex")
-        fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.POINTER(ctypes.c_size_t), ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t]
-        arr, n = self._md(md)
-        sarr = (type(steps[0]) * len(steps))(*steps) if steps else None
-        self._check(fn(self.ctx, a.ptr, b.ptr, out.ptr, arr, n, ctypes.cast(sarr, ctypes.c_void_p) if steps else None, len(steps)),
-                    f"{op}_{name}_ex")
+    def force_splitk(self, splits):
+        self.lib.emu_force_splitk(self.handle, int(splits))
+
+    def last_kernel(self):
+        return self.lib.emu_last_kernel(self.handle).decode()
+
+    def dma_lazy(self, model):
+        """LDS-DMA bytes arrive at issue (0), only when an s_waitcnt vmcnt retires them (1), or one load later than
+        that (2: a model under which a correct kernel must FAIL)"""
+        self.lib.emu_dma_lazy(int(model))
+
+    def lds_fill(self, byte):
+        self.lib.emu_lds_fill(int(byte))

@@ -1,0 +1,110 @@
+"""The GPU test files, run unmodified against the CPU build.
+
+tests/emu_util.EmuContext is hodu_amd.ffi.Context over the CPU build of the kernels (their unmodified source against
+CPU models of the gfx950 instructions, tests/emu/gfx950_insn_emu.hpp), so a GPU test function that takes the `ctx`
+fixture can be handed one: same inputs, same entry points, same variant selection, same comparison with the oracle,
+same expected kernel names.  This file collects those functions from the GPU test modules, expands their
+parametrisations, and runs each case as a test of its own.
+
+Two uses.  Every one of these cases passes on the hardware, so each is a check of the instruction models against a
+kernel the hardware has run (a model that disagrees with the hardware fails the kernel written for the hardware).  And
+with the models pinned that way, the same run is a regression test of the kernels' indexing, edge handling and
+selection logic where no GPU is at hand.
+
+By default the cases that take more than a few seconds each are skipped; HODU_EMU_ALL=1 runs them too (about a
+quarter of an hour on 8 cores).  Not run here at all: tests that time kernels or use the debug library, the host
+mirror's tests (tests/test_gpu_host_tensor.py: a compiled library of its own that links the real one), and the tests
+at BASELINE's full sizes (tests/test_gpu_configs.py, tests/test_gpu_large_extents.py)."""
+import importlib
+import inspect
+import itertools
+import os
+
+import pytest
+
+import emu_util
+
+pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host clang++ for the CPU build")
+
+SUITES = ["test_gpu_products", "test_gpu_mfma", "test_gpu_exact", "test_gpu_epilogue", "test_gpu_skinny", "test_gpu_small_f32",
+          "test_gpu_f64", "test_gpu_casts", "test_gpu_sum", "test_gpu_softmax", "test_gpu_attention",
+          # GPU tests of code that has not run on a GPU, kept under names pytest does not collect: they run here
+          "wip_pipe16r", "wip_softmax_masked", "wip_reference_sums"]
+# needs the debug library (timing, thousands of launches)
+EXCLUDED = {"test_gpu_skinny.test_split_k_arrival_protocol_over_thousands_of_launches",
+            "wip_softmax_masked.test_attention_with_a_padding_mask_against_float64"}  # (the host mirror)
+# more than a few seconds per case in the CPU build
+HEAVY = {
+    "test_gpu_mfma.test_every_variant_ragged", "test_gpu_mfma.test_native_f8_products",
+    "test_gpu_mfma.test_pipelined_f8_weight_16x16_instruction", "test_gpu_mfma.test_pipelined_kk_16x16_instruction",
+    "test_gpu_mfma.test_pipelined_kk_variants", "test_gpu_mfma.test_pipelined_row_dense_variants", "test_gpu_mfma.test_split_k",
+    "test_gpu_mfma.test_unaligned_operands",
+    "test_gpu_exact.test_16x16_instruction_tile_is_exact_and_equals_the_32x32_one",
+    "test_gpu_exact.test_16x16_instruction_tile_with_f8_weights_is_exact",
+    "test_gpu_exact.test_config3_m16_takes_the_split_k_kernel_exactly", "test_gpu_exact.test_f8_weight_pipelined_tiles",
+    "test_gpu_exact.test_native_f8_products_narrow_the_exact_sum_once", "test_gpu_exact.test_one_pass_and_split_k_skinny",
+    "test_gpu_exact.test_pipelined_split_k_through_the_workspace", "test_gpu_exact.test_row_streaming_gemv",
+    "test_gpu_epilogue.test_16x16_instruction_tiles", "test_gpu_epilogue.test_linear_layer_of_config3",
+    "test_gpu_epilogue.test_pipelined_kernels", "test_gpu_epilogue.test_small_m_kernels",
+    "test_gpu_skinny.test_gemv_rowstream", "test_gpu_skinny.test_row_dense_weight", "test_gpu_skinny.test_split_k_across_workgroups",
+    "test_gpu_small_f32.test_large_products_keep_the_tile_kernels",
+    "test_gpu_softmax.test_causal_mask", "test_gpu_softmax.test_long_and_strided_rows",
+    "wip_pipe16r.test_respaced_16x16_instruction_all_layouts", "wip_pipe16r.test_respaced_is_exact_on_exact_operands",
+    "wip_pipe16r.test_respaced_f8_weight_tile_is_exact",
+}
+RUN_ALL = os.environ.get("HODU_EMU_ALL", "") not in ("", "0")
+
+
+def _expansions(fn):
+    names, lists = [], []
+    for mark in getattr(fn, "pytestmark", []):
+        if mark.name != "parametrize":
+            continue
+        argnames = [a.strip() for a in mark.args[0].split(",")] if isinstance(mark.args[0], str) else list(mark.args[0])
+        names.append(argnames)
+        lists.append(list(mark.args[1]))
+    for combo in itertools.product(*lists):
+        kwargs = {}
+        for argnames, value in zip(names, combo):
+            if hasattr(value, "values") and hasattr(value, "marks"):  # pytest.param
+                values = value.values
+            else:
+                values = value if len(argnames) > 1 else (value,)
+            kwargs.update(zip(argnames, values))
+        yield kwargs
+
+
+def _cases():
+    for modname in SUITES:
+        mod = importlib.import_module(modname)
+        for name, fn in inspect.getmembers(mod, inspect.isfunction):
+            full = f"{modname}.{name}"
+            if not name.startswith("test_") or fn.__module__ != modname or full in EXCLUDED:
+                continue
+            params = list(inspect.signature(fn).parameters)
+            for kwargs in _expansions(fn):
+                if params[:1] != ["ctx"] or set(params[1:]) != set(kwargs):
+                    continue  # wants a fixture this file does not provide
+                ident = full.replace("test_gpu_", "", 1).replace("wip_", "unrun_on_gpu_", 1) + ("[" + "-".join(str(v) for v in kwargs.values()) + "]" if kwargs else "")
+                marks = [pytest.mark.skip(reason="slow in the CPU build: set HODU_EMU_ALL=1")] if full in HEAVY and not RUN_ALL else []
+                yield pytest.param(fn, kwargs, id=ident, marks=marks)
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = emu_util.EmuContext(tight="end")
+    c.dma_lazy(1)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("fn,kwargs", list(_cases()))
+def test_gpu_test_passes_in_the_cpu_build(ctx, fn, kwargs):
+    ctx.force_tile(-1)
+    ctx.force_splitk(-1)
+    try:
+        fn(ctx, **kwargs)
+    finally:
+        ctx.force_tile(-1)
+        ctx.force_splitk(-1)
+        ctx.set_reference_sums(False)

@@ -1,0 +1,49 @@
+"""The Tensor-level path in the CPU build: hodu_amd.tensor over the host mirror's compiled library
+(hodu_amd/host/capi.cpp, unmodified) linked against the CPU build of the kernels (tests/emu_util.py) instead of the
+real kernel library.  Every test function of tests/test_gpu_host_tensor.py -- Tensor::matmul's rank routing, broadcast
+batches, deferred casts, the copy / no-copy equivalence, Linear, the VJP products, sum_to_shape, attention, .hdt
+ingestion -- runs unchanged, plus scaled_dot_product_attention with an attn_mask (which has not run on a GPU)."""
+import inspect
+
+import pytest
+
+import emu_util
+from hodu_amd import tensor as T
+
+pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host clang++ for the CPU build")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def host_mirror_over_the_cpu_build():
+    saved_path, saved_lib = T.HOST_LIB_PATH, T._lib
+    T.HOST_LIB_PATH, T._lib = emu_util.build_host(), None
+    yield
+    T.HOST_LIB_PATH, T._lib = saved_path, saved_lib
+
+
+def _cases():
+    import test_gpu_host_tensor as suite
+    import wip_softmax_masked
+    for mod, names in ((suite, None), (wip_softmax_masked, {"test_attention_with_a_padding_mask_against_float64"})):
+        for name, fn in inspect.getmembers(mod, inspect.isfunction):
+            if not name.startswith("test_") or fn.__module__ != mod.__name__ or (names is not None and name not in names):
+                continue
+            marks = [m for m in getattr(fn, "pytestmark", []) if m.name == "parametrize"]
+            assert len(marks) <= 1
+            if not marks:
+                yield pytest.param(fn, {}, id=name)
+                continue
+            argnames = [a.strip() for a in marks[0].args[0].split(",")]
+            for value in marks[0].args[1]:
+                values = value if len(argnames) > 1 else (value,)
+                yield pytest.param(fn, dict(zip(argnames, values)), id=f"{name}[{'-'.join(str(v) for v in values)}]")
+
+
+@pytest.mark.parametrize("fn,kwargs", list(_cases()))
+def test_tensor_level_test_passes_in_the_cpu_build(fn, kwargs, tmp_path):
+    params = inspect.signature(fn).parameters
+    if "tmp_path" in params:
+        kwargs = dict(kwargs, tmp_path=tmp_path)
+    if "ctx" in params:
+        kwargs = dict(kwargs, ctx=None)  # (the masked-attention test takes the fixture and does not use it)
+    fn(**kwargs)

@@ -22,14 +22,20 @@ V = H.View
 @pytest.fixture(scope="module")
 def ctx():
     c = ffi.Context(0)
-    c.set_reference_sums(True)
     yield c
     c.set_reference_sums(False)
     c.close()
 
 
+@pytest.fixture(autouse=True)
+def _mode_off_afterwards(ctx):
+    yield
+    ctx.set_reference_sums(False)
+
+
 @pytest.mark.parametrize("dt", NARROW)
 def test_reference_bytes(ctx, dt):
+    ctx.set_reference_sums(True)
     cases = [("dot", V([37, 29]), V([29, 41]), True), ("dot", V([33, 64]), V([20, 64]).t(), False),
              ("dot", V([70, 50]).t(), V([70, 9], offset=5), False),
              ("matmul", V([3, 2, 9, 12]), V([12, 7]).broadcast_to([3, 2, 12, 7]), False),
@@ -46,6 +52,7 @@ def test_reference_bytes(ctx, dt):
 
 
 def test_switching_off_restores_the_f32_sums(ctx):
+    ctx.set_reference_sums(True)
     lv, rv = V([300, 512]), V([260, 512]).t()
     a, b = tame("bf16", lv.span(), 7), tame("bf16", rv.span(), 8)
     md = H.dot_md(lv, rv)

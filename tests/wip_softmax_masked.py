@@ -86,7 +86,7 @@ def test_bool_and_i8_masks(ctx):
 
 def test_attention_with_a_padding_mask_against_float64(ctx):
     """scaled_dot_product_attention(q, k, v, attn_mask) through the host mirror: a [B, 1, 1, Sk] padding mask; three
-    launches (the fused kernel has no mask operand); held to the float64 function at the products' 2e-2"""
+    launches (the fused kernel has no mask operand); held to the float64 function at the products' 2e-2 of the sum's size"""
     B, Hh, S, D = 2, 4, 96, 64
     g = np.random.default_rng(77)
     q, k, v = (g.standard_normal((B, Hh, S, D)).astype(np.float32) for _ in range(3))
@@ -106,5 +106,9 @@ def test_attention_with_a_padding_mask_against_float64(ctx):
     s = q64 @ k64.transpose(0, 1, 3, 2) * scale
     s = np.where(keep.astype(bool), s, -np.inf)
     p = np.exp(s - s.max(-1, keepdims=True))
-    want = (p / p.sum(-1, keepdims=True)) @ v64
-    assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), 0.25))
+    p = p / p.sum(-1, keepdims=True)
+    want = p @ v64
+    # the three-launch path rounds the scores to bf16 twice (product, scale) and the probabilities once: relative errors
+    # of every p_j of up to 2^-8 |s|, i.e. an error of the output that scales with sum_j p_j |v_j| -- the size of the sum,
+    # not of its (possibly cancelling) value; with as few as 33 unmasked keys that floor matters
+    assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), p @ np.abs(v64)))
