@@ -72,6 +72,31 @@ def _steps_array(steps):
     return (EpilogueStep * max(1, len(steps)))(*steps), len(steps)
 
 
+def declare_runtime(lib: ctypes.CDLL):
+    """argument types of the context, memory and timing entry points"""
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    lib.hodu_rocm_device_count.argtypes = [ctypes.POINTER(ci)]
+    lib.hodu_rocm_ctx_create.argtypes = [ci, ctypes.POINTER(vp)]
+    lib.hodu_rocm_ctx_destroy.argtypes = [vp]
+    lib.hodu_rocm_alloc.argtypes = [vp, sz, ctypes.POINTER(vp)]
+    lib.hodu_rocm_free.argtypes = [vp, vp]
+    lib.hodu_rocm_memcpy_h2d.argtypes = [vp, vp, vp, sz]
+    lib.hodu_rocm_memcpy_d2h.argtypes = [vp, vp, vp, sz]
+    lib.hodu_rocm_memcpy_d2d.argtypes = [vp, vp, vp, sz]
+    lib.hodu_rocm_memset.argtypes = [vp, vp, ci, sz]
+    lib.hodu_rocm_sync.argtypes = [vp]
+    lib.hodu_rocm_last_error.argtypes = [vp]
+    lib.hodu_rocm_last_error.restype = ctypes.c_char_p
+    lib.hodu_rocm_last_kernel.argtypes = [vp]
+    lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
+    lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
+                                          ctypes.POINTER(sz)]
+    lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
+    lib.hodu_rocm_timer_start.argtypes = [vp, vp]
+    lib.hodu_rocm_timer_stop.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
+    lib.hodu_rocm_timer_destroy.argtypes = [vp, vp]
+
+
 def declare_compute(lib: ctypes.CDLL):
     """argument types of the compute entry points (everything in include/hodu_rocm_kernels.h that launches kernels)"""
     vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
@@ -102,28 +127,7 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build the HIP extension first (python -m hodu_amd.build). "
             "hodu_amd has no CPU fallback.")
     lib = ctypes.CDLL(LIB_PATH)
-    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
-    szp = ctypes.POINTER(ctypes.c_size_t)
-    lib.hodu_rocm_device_count.argtypes = [ctypes.POINTER(ci)]
-    lib.hodu_rocm_ctx_create.argtypes = [ci, ctypes.POINTER(vp)]
-    lib.hodu_rocm_ctx_destroy.argtypes = [vp]
-    lib.hodu_rocm_alloc.argtypes = [vp, sz, ctypes.POINTER(vp)]
-    lib.hodu_rocm_free.argtypes = [vp, vp]
-    lib.hodu_rocm_memcpy_h2d.argtypes = [vp, vp, vp, sz]
-    lib.hodu_rocm_memcpy_d2h.argtypes = [vp, vp, vp, sz]
-    lib.hodu_rocm_memcpy_d2d.argtypes = [vp, vp, vp, sz]
-    lib.hodu_rocm_memset.argtypes = [vp, vp, ci, sz]
-    lib.hodu_rocm_sync.argtypes = [vp]
-    lib.hodu_rocm_last_error.argtypes = [vp]
-    lib.hodu_rocm_last_error.restype = ctypes.c_char_p
-    lib.hodu_rocm_last_kernel.argtypes = [vp]
-    lib.hodu_rocm_last_kernel.restype = ctypes.c_char_p
-    lib.hodu_rocm_device_info.argtypes = [vp, ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
-                                          ctypes.POINTER(sz)]
-    lib.hodu_rocm_timer_create.argtypes = [vp, ctypes.POINTER(vp)]
-    lib.hodu_rocm_timer_start.argtypes = [vp, vp]
-    lib.hodu_rocm_timer_stop.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
-    lib.hodu_rocm_timer_destroy.argtypes = [vp, vp]
+    declare_runtime(lib)
     declare_compute(lib)
     _lib = lib
     return lib

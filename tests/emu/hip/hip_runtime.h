@@ -48,15 +48,53 @@ struct dim3 {
 };
 struct emu_uint3 { unsigned x = 0, y = 0, z = 0; };
 
+// ---- the runtime API the library's host code calls: one device, one implicit stream, everything synchronous --------
 typedef void *hipStream_t;
 typedef int hipError_t;
-constexpr hipError_t hipSuccess = 0, hipErrorOutOfMemory = 2;
-struct hipDeviceProp_t { int multiProcessorCount = 256; };
+constexpr hipError_t hipSuccess = 0, hipErrorOutOfMemory = 2, hipErrorInvalidValue = 1;
+struct hipDeviceProp_t {
+    char name[64] = "CPU build of the kernels";
+    char gcnArchName[64] = "gfx950:emulated";
+    int multiProcessorCount = 256;
+    int clockRate = 2400000;
+    size_t totalGlobalMem = (size_t)288 << 30;
+};
+namespace emu {
+// "device" memory: host memory between two inaccessible pages, the allocation's last 16-byte unit ending where the
+// second one begins (emu_alloc_tight(0): its first byte following the first one instead)
+void *device_alloc(size_t bytes);
+bool device_free(void *p);
+}  // namespace emu
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipSetDevice(int) { return hipSuccess; }
-inline const char *hipGetErrorString(hipError_t) { return "emulated"; }
+inline const char *hipGetErrorString(hipError_t e) { return e == hipErrorOutOfMemory ? "out of memory" : "emulated runtime error"; }
 enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize = 8 };
 inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { return hipSuccess; }
+inline hipError_t hipGetDeviceCount(int *n) { *n = 1; return hipSuccess; }
+inline hipError_t hipGetDeviceProperties(hipDeviceProp_t *p, int) { *p = hipDeviceProp_t(); return hipSuccess; }
+constexpr unsigned hipStreamNonBlocking = 1;
+inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { *s = nullptr; return hipSuccess; }
+inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
+inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+enum hipStreamCaptureStatus { hipStreamCaptureStatusNone = 0, hipStreamCaptureStatusActive = 1 };
+inline hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus *st) { *st = hipStreamCaptureStatusNone; return hipSuccess; }
+template <class T> inline hipError_t hipMalloc(T **p, size_t bytes) {
+    *p = (T *)emu::device_alloc(bytes);
+    return *p ? hipSuccess : hipErrorOutOfMemory;
+}
+inline hipError_t hipFree(void *p) { return (!p || emu::device_free(p)) ? hipSuccess : hipErrorInvalidValue; }
+enum hipMemcpyKind { hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
+inline hipError_t hipMemcpyAsync(void *dst, const void *src, size_t bytes, hipMemcpyKind, hipStream_t) { memmove(dst, src, bytes); return hipSuccess; }
+inline hipError_t hipMemsetAsync(void *dst, int byte, size_t bytes, hipStream_t) { memset(dst, byte, bytes); return hipSuccess; }
+// a __device__ variable is an ordinary one here, and its "device address" its address
+#define HIP_SYMBOL(x) (x)
+template <class T> inline hipError_t hipGetSymbolAddress(void **p, T &symbol) { *p = (void *)&symbol; return hipSuccess; }
+typedef void *hipEvent_t;
+inline hipError_t hipEventCreate(hipEvent_t *e) { *e = nullptr; return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
+inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventElapsedTime(float *ms, hipEvent_t, hipEvent_t) { *ms = 0.f; return hipSuccess; }
+inline hipError_t hipEventDestroy(hipEvent_t) { return hipSuccess; }
 
 namespace emu {
 constexpr int kWave = 64, kMaxBlock = 1024;

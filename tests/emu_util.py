@@ -31,7 +31,7 @@ LIB = os.path.join(OUT, "libhodu_emu.so")
 MFMA_SOURCES = [os.path.join(CSRC, f) for f in ("gemm_mfma.hip", "gemm_mfma_bf16.hip", "gemm_mfma_mi16_bf16.hip", "gemm_mfma_w8a16.hip",
                                                 "gemm_mfma_f16.hip", "gemm_mfma_mi16_f16.hip", "gemm_mfma_f32.hip", "gemm_mfma_i8.hip",
                                                 "gemm_mfma_i8_out.hip", "gemm_mfma_u8_out.hip", "gemm_mfma_f8.hip", "skinny.hip",
-                                                "gemv.hip", "gemv_rows.hip", "small_f32.hip", "gemm_f64.hip", "attention.hip")]
+                                                "gemv.hip", "gemv_rows.hip", "small_f32.hip", "gemm_f64.hip", "attention.hip", "runtime.cpp")]
 MFMA_LIB = os.path.join(OUT, "libhodu_emu_mfma.so")
 
 
@@ -60,7 +60,7 @@ def build(mfma=False):
     os.makedirs(OUT, exist_ok=True)
     flags = ["-std=c++17", "-fPIC", "-x", "c++", f"-I{EMU}", f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
              "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-psabi"]
-    with_models = ["-DEMU_WITH_MFMA", "-include", os.path.join(EMU, "gfx950_insn_emu.hpp")]
+    with_models = ["-DEMU_WITH_RUNTIME", "-include", os.path.join(EMU, "gfx950_insn_emu.hpp")]
     # Without optimisation: a fifth of the compile time (cast.hip alone takes a minute at -O1), and a run spends its
     # time starting threads and in the lanes' barriers, not in the kernels' arithmetic.
     jobs = [(src, "", ["-O0"]) for src in SOURCES]
@@ -121,8 +121,8 @@ DTYPE_ID = {"bool": 0, "f8e4m3": 1, "f8e5m2": 2, "bf16": 3, "f16": 4, "f32": 5, 
 class Emu:
     """the entry points of api.cpp as compiled for the host; every pointer argument is a numpy array"""
 
-    def __init__(self, mfma=False):
-        path = build(mfma)
+    def __init__(self):
+        path = build()
         if path is None:
             raise RuntimeError("no host clang++ to build tests/emu with")
         self.lib = lib = ctypes.CDLL(path)
@@ -139,11 +139,6 @@ class Emu:
         lib.hodu_rocm_cast.argtypes = [vp, ci, ci, vp, vp, szp, sz]
         lib.hodu_rocm_contiguous.argtypes = [vp, ci, vp, vp, szp, sz]
         lib.hodu_rocm_sum.argtypes = [vp, ci, vp, vp, szp, sz]
-        if mfma:
-            lib.emu_dma_lazy.argtypes = [ci]
-            lib.emu_lds_fill.argtypes = [ci]
-            lib.emu_force_tile.argtypes = [vp, ci]
-            lib.emu_force_splitk.argtypes = [vp, ci]
         self.ctx = lib.emu_ctx_create()
 
     def close(self):
@@ -169,21 +164,6 @@ class Emu:
     def set_reference_sums(self, on):
         self.lib.hodu_rocm_ctx_set_reference_sums.argtypes = [ctypes.c_void_p, ctypes.c_int]
         assert self.lib.hodu_rocm_ctx_set_reference_sums(self.ctx, int(on)) == 0
-
-    # the library with the tile kernels only
-    def force_tile(self, v):
-        self.lib.emu_force_tile(self.ctx, v)
-
-    def force_splitk(self, v):
-        self.lib.emu_force_splitk(self.ctx, v)
-
-    def dma_lazy(self, model):
-        """LDS-DMA bytes arrive at issue (0), only when an s_waitcnt vmcnt retires them (1), or one load later than
-        that (2: a model under which a correct kernel must FAIL)"""
-        self.lib.emu_dma_lazy(int(model))
-
-    def lds_fill(self, byte):
-        self.lib.emu_lds_fill(byte)
 
     def softmax(self, dt, x, out, md, causal=False):
         a, n = self._md(md)
@@ -214,122 +194,78 @@ class Emu:
         self._check(fn(self.ctx, a.ctypes.data, b.ctypes.data, out.ctypes.data, arr, n), f"{op}_{name}")
 
 
-# ---- a stand-in for hodu_amd.ffi.Context over the CPU build, so that the GPU tests' helpers run against it unchanged ----
-_libc = ctypes.CDLL(None, use_errno=True)
-_libc.mmap.restype = ctypes.c_void_p
-_libc.mmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_long]
-_libc.munmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
-_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
-PAGE = 4096
-
-
-class GuardedBuffer:
-    """`nbytes` of "device" memory between two inaccessible pages: a kernel that reads or writes past either end of an
-    operand takes a segmentation fault here instead of a GPU memory fault there.  `tight` says which end touches its
-    guard page exactly ("end": the last 16-byte unit ends where the guard begins, the way a clamped row or a biased
-    pointer would overrun; "start": the first byte follows the front guard)."""
-
-    def __init__(self, nbytes, tight="end"):
-        body = max((nbytes + PAGE - 1) // PAGE, 1) * PAGE
-        self.total = body + 2 * PAGE
-        base = _libc.mmap(None, self.total, 3, 0x22, -1, 0)  # PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS
-        if base in (None, ctypes.c_void_p(-1).value):
-            raise MemoryError("mmap")
-        self.base = base
-        assert _libc.mprotect(base, PAGE, 0) == 0 and _libc.mprotect(base + PAGE + body, PAGE, 0) == 0
-        self.nbytes = nbytes
-        self.ptr = base + PAGE + (body - (nbytes + 15) // 16 * 16 if tight == "end" else 0)
-
-    def array(self, dtype, count=None):
-        count = self.nbytes // np.dtype(dtype).itemsize if count is None else count
-        return np.ctypeslib.as_array(ctypes.cast(self.ptr, ctypes.POINTER(ctypes.c_uint8)), (self.nbytes,)).view(dtype)[:count]
-
-    def free(self):
-        if self.base:
-            _libc.munmap(self.base, self.total)
-            self.base = None
-
-
+# ---- hodu_amd.ffi.Context over the CPU build, so that the GPU tests' helpers and test functions run against it unchanged ----
 class EmuContext(ffi.Context):
-    """hodu_amd.ffi.Context over the CPU build: the same Python methods (product, product_ex, cast, sum, softmax, ..,
-    with their host-side extent checks) calling the same entry points of api.cpp, with "device" buffers that are host
-    memory between inaccessible pages.  The GPU tests' helpers and test functions run against it unchanged."""
+    """hodu_amd.ffi.Context with the CPU build of the whole library (build(mfma=True): every kernel family, api.cpp,
+    runtime.cpp) in the place of the HIP library: the same Python methods with their host-side extent checks, the same
+    entry points, hodu_rocm_alloc handing out host memory between two inaccessible pages.  What it adds are the two
+    testing hooks and the scratch report (the debug library has no CPU build) and the switches of the instruction
+    models."""
 
-    def __init__(self, tight="end", mfma=True):
-        path = build(mfma)
-        if path is None:
-            raise RuntimeError("no host clang++ to build tests/emu with")
-        self.lib = lib = ctypes.CDLL(path)
-        ffi.declare_compute(lib)
-        vp, ci = ctypes.c_void_p, ctypes.c_int
-        lib.emu_ctx_create.restype = vp
-        lib.emu_ctx_destroy.argtypes = [vp]
-        lib.emu_last_kernel.restype = ctypes.c_char_p
-        lib.emu_last_kernel.argtypes = [vp]
-        lib.emu_last_error.restype = ctypes.c_char_p
-        lib.emu_unsupported_first.restype = ctypes.c_char_p
-        lib.emu_force_tile.argtypes = [vp, ci]
-        lib.emu_force_splitk.argtypes = [vp, ci]
-        lib.emu_lds_fill.argtypes = [ci]
-        if mfma:
+    _emu_lib = None
+
+    @classmethod
+    def library(cls):
+        if cls._emu_lib is None:
+            path = build(mfma=True)
+            if path is None:
+                raise RuntimeError("no host clang++ to build tests/emu with")
+            lib = ctypes.CDLL(path)
+            ffi.declare_runtime(lib)
+            ffi.declare_compute(lib)
+            vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+            lib.emu_unsupported_first.restype = ctypes.c_char_p
+            lib.emu_force_tile.argtypes = [vp, ci]
+            lib.emu_force_splitk.argtypes = [vp, ci]
+            lib.emu_scratch_state.argtypes = [vp, ctypes.POINTER(sz), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+            lib.emu_lds_fill.argtypes = [ci]
+            lib.emu_alloc_tight.argtypes = [ci]
             lib.emu_dma_lazy.argtypes = [ci]
-        self.handle = lib.emu_ctx_create()
-        self.device = 0
+            cls._emu_lib = lib
+        return cls._emu_lib
+
+    def __init__(self, device=0, tight="end"):
+        self.lib = self.library()
+        h = ctypes.c_void_p()
+        rc = self.lib.hodu_rocm_ctx_create(int(device), ctypes.byref(h))
+        self.handle = h.value if rc == 0 else None
+        if rc != 0:
+            raise ffi.HoduRocmError(rc, self.lib.hodu_rocm_last_error(None).decode())
+        self.device = device
         self.tight = tight
+
+    @property
+    def tight(self):
+        return self._tight
+
+    @tight.setter
+    def tight(self, where):
+        """which end of an allocation touches its guard page: "end" (a clamped row or a biased pointer would overrun
+        there) or "start"; applies to allocations made from now on, by any context"""
+        self._tight = where
+        self.lib.emu_alloc_tight(int(where == "end"))
 
     @property
     def debug(self):
         raise RuntimeError("the hooks library has no CPU build")
 
-    def close(self):
-        if self.handle is not None:
-            self.lib.emu_ctx_destroy(self.handle)
-            self.handle = None
-
     def _check(self, rc):
-        if rc != 0:
-            raise ffi.HoduRocmError(rc, self.lib.emu_last_error().decode())
+        super()._check(rc)
         if self.lib.emu_unsupported_hits() != 0:
             first = self.lib.emu_unsupported_first().decode()
             self.lib.emu_unsupported_reset()
             raise AssertionError(f"{self.last_kernel()} reached an instruction without a CPU stand-in: {first}")
 
-    # memory
-    def alloc(self, nbytes):
-        return GuardedBuffer(nbytes, self.tight)
-
-    def upload(self, host):
-        host = np.ascontiguousarray(host)
-        buf = GuardedBuffer(host.nbytes, self.tight)
-        buf.array(np.uint8)[:] = host.view(np.uint8).ravel()
-        return buf
-
-    def upload_into(self, buf, host, first_byte=0):
-        host = np.ascontiguousarray(host).view(np.uint8).ravel()
-        buf.array(np.uint8)[first_byte:first_byte + host.size] = host
-
-    def download(self, buf, dtype, count=None, first=0):
-        dtype = np.dtype(dtype)
-        n = buf.nbytes // dtype.itemsize - first if count is None else int(count)
-        if first < 0 or n < 0 or (first + n) * dtype.itemsize > buf.nbytes:
-            raise ffi.HoduRocmError(ffi.INVALID_ARG, "download: the range lies outside the buffer")
-        return buf.array(np.uint8)[first * dtype.itemsize:(first + n) * dtype.itemsize].view(dtype).copy()
-
-    def fill(self, buf, byte):
-        buf.array(np.uint8)[:] = byte
-
-    def sync(self):
-        pass
-
-    # hooks and diagnostics
     def force_tile(self, tile):
         self.lib.emu_force_tile(self.handle, int(tile))
 
     def force_splitk(self, splits):
         self.lib.emu_force_splitk(self.handle, int(splits))
 
-    def last_kernel(self):
-        return self.lib.emu_last_kernel(self.handle).decode()
+    def scratch_state(self):
+        ws, arr, fixed = ctypes.c_size_t(), ctypes.c_int(), ctypes.c_int()
+        self.lib.emu_scratch_state(self.handle, ctypes.byref(ws), ctypes.byref(arr), ctypes.byref(fixed))
+        return {"workspace_bytes": ws.value, "arrival_allocated": bool(arr.value), "fixed": bool(fixed.value)}
 
     def dma_lazy(self, model):
         """LDS-DMA bytes arrive at issue (0), only when an s_waitcnt vmcnt retires them (1), or one load later than

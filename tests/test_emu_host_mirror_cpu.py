@@ -39,7 +39,19 @@ def _cases():
                 yield pytest.param(fn, dict(zip(argnames, values)), id=f"{name}[{'-'.join(str(v) for v in values)}]")
 
 
-@pytest.mark.parametrize("fn,kwargs", list(_cases()))
+def _collected():
+    """(a failure to collect must not take the other test files' collection down with it: it becomes one failing case)"""
+    try:
+        return list(_cases())
+    except Exception as e:  # noqa: BLE001
+        message = f"{type(e).__name__}: {e}"
+
+        def collection_failed():
+            raise RuntimeError(f"collecting the Tensor-level test functions failed: {message}")
+        return [pytest.param(collection_failed, {}, id="collection")]
+
+
+@pytest.mark.parametrize("fn,kwargs", _collected())
 def test_tensor_level_test_passes_in_the_cpu_build(fn, kwargs, tmp_path):
     params = inspect.signature(fn).parameters
     if "tmp_path" in params:
