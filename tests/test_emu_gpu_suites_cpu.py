@@ -29,12 +29,13 @@ pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host cla
 
 SUITES = ["test_gpu_products", "test_gpu_mfma", "test_gpu_exact", "test_gpu_epilogue", "test_gpu_skinny", "test_gpu_small_f32",
           "test_gpu_f64", "test_gpu_casts", "test_gpu_sum", "test_gpu_softmax", "test_gpu_attention", "test_zz_no_alloc",
-          # GPU tests of code that has not run on a GPU, kept under names pytest does not collect: they run here
-          "wip_pipe16r", "wip_softmax_masked", "wip_reference_sums"]
+          "test_zx_softmax_masked", "test_zy_reference_sums",
+          # the GPU test of kernels that have not run on a GPU, kept under a name pytest does not collect: it runs here
+          "wip_pipe16r"]
 # needs the debug library (timing, thousands of launches)
 EXCLUDED = {"test_gpu_skinny.test_split_k_arrival_protocol_over_thousands_of_launches",
             "test_zz_no_alloc.test_captured_into_a_graph_and_replayed",  # (graph capture and timing: the debug library)
-            "wip_softmax_masked.test_attention_with_a_padding_mask_against_float64"}  # (the host mirror)
+            "test_zx_softmax_masked.test_attention_with_a_padding_mask_against_float64"}  # (the host mirror)
 # more than a few seconds per case in the CPU build
 HEAVY = {
     "test_gpu_mfma.test_every_variant_ragged", "test_gpu_mfma.test_native_f8_products",

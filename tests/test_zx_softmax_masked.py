@@ -1,7 +1,7 @@
-"""NOT collected (the file name keeps pytest off it): hodu_rocm_softmax_masked and the attn_mask path of
-scaled_dot_product_attention have been compiled but have never run on a GPU.  Run by naming the file:
-
-    python -u -m pytest tests/wip_softmax_masked.py -x -v --timeout 120 --timeout-method thread
+"""GPU parity of hodu_rocm_softmax_masked and of the attn_mask path of scaled_dot_product_attention
+(crates/hodu_nn/src/modules/attention.rs:40-56).  (The file name sorts it behind the tests of the kernels that have a
+longer history on the hardware; these cases also run against the CPU build of the same kernel source,
+tests/test_emu_gpu_suites_cpu.py and tests/test_emu_host_mirror_cpu.py.)
 
 The comparator is oracle.softmax_masked_spec, pinned on the CPU by tests/test_oracle_softmax_masked_cpu.py.
 Tolerances as in test_gpu_softmax.py: f32 1e-5, bf16 / f16 2e-2, f64 1e-12 relative; a masked entry of a row that

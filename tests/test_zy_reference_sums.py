@@ -1,8 +1,7 @@
-"""NOT collected (the file name keeps pytest off it): hodu_rocm_ctx_set_reference_sums on the GPU.  The kernel
-(hodu_amd/csrc/gemm_refsum.hip) is held bit for bit to the oracle's reference-faithful products and to the compiled
-reference in the CPU build (tests/test_emu_reference_sums_cpu.py) and has not run on a GPU.  Run it by naming the file:
-
-    python -u -m pytest tests/wip_reference_sums.py -x -v --timeout 120 --timeout-method thread
+"""GPU parity of hodu_rocm_ctx_set_reference_sums: narrow-float products in the reference's own arithmetic must store
+the reference's bytes.  The kernel (hodu_amd/csrc/gemm_refsum.hip) is held bit for bit to the oracle's
+reference-faithful products and to the compiled reference in the CPU build (tests/test_emu_reference_sums_cpu.py); the
+file name sorts this test behind those of the kernels with a longer history on the hardware.
 
 What the GPU run adds to the CPU one: that the device's frexpf / ldexpf / float-to-int conversions and its f32 multiply
 and add (denormals kept, no contraction into an FMA) give the reference's bytes."""
