@@ -172,6 +172,9 @@ int hodu_host_view(const hodu_host_tensor *a, const size_t *shape, const size_t 
 
 /* 0 = reproduce the reference's forced copies, 1 = strided views go to the kernel as they are */
 void hodu_host_set_matmul_mode(int mode) { matmul_mode() = mode == 0 ? MatmulMode::Reference : MatmulMode::NoCopy; }
+int hodu_host_set_reference_sums(int device, int on) {
+    return guarded([&] { RocmDevice::get(device)->set_reference_sums(on != 0); });
+}
 void hodu_host_stats(long *cast_kernels, long *contiguous_kernels, long *product_kernels, long *fused_products,
                      long long *bytes_copied) {
     Stats &s = stats();

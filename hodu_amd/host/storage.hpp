@@ -69,6 +69,10 @@ public:
         if (rc != HODU_ROCM_OK)
             throw Error(ErrorKind::RocmKernelError, std::string(what) + ": " + hodu_rocm_last_error(ctx_));
     }
+    // products of f8e4m3 / f8e5m2 / bf16 / f16 on this device in the CPU backend's arithmetic -- the running sum
+    // re-rounded to the dtype after every multiply and add (crates/hodu_cpu_kernels/kernels/ops_matrix.c:196-240,
+    // :351-354) -- for comparing devices byte for byte; off by default
+    void set_reference_sums(bool on) const { check(hodu_rocm_ctx_set_reference_sums(ctx_, on ? 1 : 0), "set_reference_sums"); }
 
 private:
     RocmDevice(int id, hodu_rocm_ctx *ctx) : id_(id), ctx_(ctx) {}

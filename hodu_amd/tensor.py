@@ -86,6 +86,7 @@ def load() -> ctypes.CDLL:
     lib.hodu_host_view.argtypes = [vp, szp, szp, sz, sz, vpp]
     lib.hodu_host_set_matmul_mode.argtypes = [ci]
     lib.hodu_host_set_matmul_mode.restype = None
+    lib.hodu_host_set_reference_sums.argtypes = [ci, ci]
     lib.hodu_host_stats.argtypes = [ctypes.POINTER(ctypes.c_long)] * 4 + [ctypes.POINTER(ctypes.c_longlong)]
     lib.hodu_host_stats.restype = None
     lib.hodu_host_stats_reset.restype = None
@@ -101,6 +102,15 @@ def set_matmul_mode(mode: str):
     """'reference': copy non-contiguous operands before broadcasting like hodu does today;
     'nocopy': hand strided / broadcast views to the kernel unchanged (the default)."""
     load().hodu_host_set_matmul_mode({"reference": 0, "nocopy": 1}[mode])
+
+
+def set_reference_sums(on: bool, device: int = 0):
+    """products of f8e4m3 / f8e5m2 / bf16 / f16 on the device in the CPU backend's arithmetic (the running sum re-rounded
+    to the dtype after every multiply and add): hodu's CPU bytes, at a scalar loop's speed; off by default"""
+    lib = load()
+    rc = lib.hodu_host_set_reference_sums(int(device), int(bool(on)))
+    if rc != 0:
+        raise HoduError(rc, lib.hodu_host_last_error().decode())
 
 
 def stats(reset: bool = False) -> dict:

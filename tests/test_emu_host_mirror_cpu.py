@@ -59,3 +59,24 @@ def test_tensor_level_test_passes_in_the_cpu_build(fn, kwargs, tmp_path):
     if "ctx" in params:
         kwargs = dict(kwargs, ctx=None)  # (the masked-attention test takes the fixture and does not use it)
     fn(**kwargs)
+
+
+def test_reference_sums_through_the_tensor_api():
+    """Tensor::matmul of bf16 tensors with the device switched to the reference's arithmetic stores the bytes of
+    hodu_cpu_matmul_bf16 (the oracle's reference-faithful product); switched back, the f32-accumulated ones"""
+    import numpy as np
+
+    import helpers as H
+    import oracle
+    a = H.random_storage("bf16", 3 * 20 * 48, 1)
+    b = H.random_storage("bf16", 48 * 24, 2)
+    ta, tb = T.Tensor.from_bits(a, "bf16", [3, 20, 48]), T.Tensor.from_bits(b, "bf16", [48, 24])
+    md = H.matmul_md(H.View([3, 20, 48]), H.View([48, 24]).broadcast_to([3, 48, 24]))
+    T.set_reference_sums(True)
+    try:
+        got = ta.matmul(tb).to_bits()
+    finally:
+        T.set_reference_sums(False)
+    assert np.array_equal(got, oracle.matmul_asis("bf16", a, b, md))
+    own = ta.matmul(tb).to_bits()
+    assert not np.array_equal(own, got)
