@@ -1,6 +1,5 @@
 // Test infrastructure: CPU stand-ins for the instruction wrappers of hodu_amd/csrc/gfx950_insn.hpp and for the gfx950
-// builtins the matrix-core kernel headers use, so that the tile kernels' unmodified source runs in the CPU build
-// (tests/emu/hip/hip_runtime.h).  A translation unit gets this file through -include, ahead of everything else.
+// builtins the kernels use, so that their unmodified source runs in the CPU build (tests/emu/hip/hip_runtime.h).  A translation unit gets this file through -include, ahead of everything else.
 //
 // What is modelled, as this repository understands the hardware (the kernels that have run on a GPU and pass their
 // tests there are the evidence for the model; a kernel that has not is checked against the model, not against the
@@ -9,13 +8,13 @@
 //     first operand and of column r of the second; it then holds D[4 g + e][r], e = 0..3, added to its accumulator;
 //   * v_mfma_f32_32x32x16_{bf16,f16}: lane (r = lane % 32, h = lane / 32) supplies k = 8 h .. 8 h + 7 of row / column r;
 //     it then holds D[8 (e / 4) + 4 h + e % 4][r], e = 0..15;
-//   * the other shapes alike, with the k a lane supplies: one (f32 32 x 32 x 2 and 16 x 16 x 4, f64 16 x 16 x 4), 16
-//     bytes (i8 32 x 32 x 32 and 16 x 16 x 64), 32 bytes (the 8-bit float forms 32 x 32 x 64 and 16 x 16 x 128 with
-//     unit scales);
+//   * the other shapes alike, with the k a lane supplies: one (f32 32 x 32 x 2 and 16 x 16 x 4; f64 16 x 16 x 4, which
+//     holds D[4 e + g][r] instead), 16 bytes (i8 32 x 32 x 32 and 16 x 16 x 64), 32 bytes (the 8-bit float forms
+//     32 x 32 x 64 and 16 x 16 x 128 with unit scales);
+//     all sum in the accumulator's type with k ascending (the hardware's order inside one instruction is not
+//     architected; the tests that compare bit for bit use operands whose products and partial sums are exact);
 //   * v_dot2_f32_bf16, v_readlane, v_mov with the DPP controls quad_perm / row_mirror / row_half_mirror, ballot,
 //     v_permlane32_swap;
-//     both sum in f32 with k ascending (the hardware's order inside one instruction is not architected; the tests that
-//     compare bit for bit use operands whose products and partial sums are exact);
 //   * global_load_lds_dwordx4: lane l copies 16 bytes from (base + lane offset + immediate) to LDS at M0 + immediate
 //     + 16 l: the immediate moves both addresses.  M0 is a per-wavefront register, kept per lane here (every lane
 //     writes the same value); a DMA before any M0 write aborts;
