@@ -44,6 +44,12 @@ template <int FMT> __device__ __forceinline__ void mfma16x16x128_f8(const i32x8_
 // inserts nothing between the last matrix instruction and the first read of an accumulator behind the loop.  The
 // hardware wants idle wait states there -- up to 18 when a 16-pass instruction's result is read by a vector
 // instruction, fewer for the 4- and 8-pass instructions used here -- and does not interlock: these are they.
+// The statement orders memory accesses, not registers: the compiler may, and in some kernels does, schedule reads of
+// accumulators in front of it -- of those the epilogue needs first, which the loop's last slice wrote some sixty
+// matrix instructions earlier.  (Naming the last-written accumulators as operands of the statement does not help:
+// the register allocator then copies them to other registers in front of it, which is the read to be avoided.)
+// tests/test_isa_hazards_cpu.py holds the generated code to the rule itself: no instruction names a register the
+// final two matrix instructions wrote until 18 wait states have passed.
 __device__ __forceinline__ void mfma_results_settle() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
 
 // LDS-DMA: 16 bytes per lane from global memory straight into LDS at M0 + lane * 16 (+ the immediate offset, which
