@@ -1,7 +1,8 @@
 """Rules the hardware does not enforce, checked on the generated code of the kernels that write instructions in
 assembly (hodu_amd/csrc/gfx950_insn.hpp).  The compiler's hazard recogniser inserts wait states for the instructions
 it emits itself; it does not see inside an asm statement, so for those the kernels place the wait states by hand --
-and this test reads the gfx950 assembly hipcc generates for them (cross-compiled here, no GPU) and holds it to the
+and this test reads the gfx950 assembly hipcc generates for them (cross-compiled here, no GPU; the f8e4m3-weight tile
+kernels through tests/isa/mi16_f8w_kernels.hip, which instantiates them alone) and holds it to the
 rules:
 
  * results of an MFMA are not interlocked: between a matrix instruction and an instruction that reads the accumulation
@@ -22,8 +23,11 @@ import os
 import re
 import shutil
 import subprocess
+from concurrent.futures import ThreadPoolExecutor
 
 import pytest
+
+from hodu_amd.build import FLAGS as BUILD_FLAGS
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "hodu_amd", "csrc")
@@ -32,13 +36,24 @@ pytestmark = pytest.mark.skipif(HIPCC is None, reason="no hipcc to generate the 
 MFMA_RESULT_WAIT_STATES = 18
 
 
-def assembly_of(source, tmp_path_factory):
-    out = tmp_path_factory.mktemp("isa") / (source + ".s")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "--cuda-device-only", "-S", f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}", os.path.join(CSRC, source), "-o", str(out)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr[-2000:]
-    return out.read_text().split("\n")
+SOURCES = {"tile16": os.path.join(CSRC, "gemm_mfma_mi16_bf16.hip"), "f8_tiles": os.path.join(CSRC, "gemm_mfma_f8.hip"),
+           "tile16_f8w": os.path.join(ROOT, "tests", "isa", "mi16_f8w_kernels.hip")}
+
+
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    """{name: lines of the gfx950 assembly of SOURCES[name]}, the three compiled side by side"""
+    out_dir = tmp_path_factory.mktemp("isa")
+
+    def one(item):
+        name, source = item
+        out = out_dir / (name + ".s")
+        cmd = [HIPCC, *BUILD_FLAGS, "--cuda-device-only", "-S", source, "-o", str(out)]  # the library's own flags
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        return name, out.read_text().split("\n")
+    with ThreadPoolExecutor(max_workers=3) as pool:
+        return dict(pool.map(one, SOURCES.items()))
 
 
 def kernels_in(lines, name_part):
@@ -103,28 +118,35 @@ def loads_too_close_to_an_m0_write(insns):
 
 
 @pytest.fixture(scope="module")
-def tile16(tmp_path_factory):
-    return assembly_of("gemm_mfma_mi16_bf16.hip", tmp_path_factory)
+def tile16(assembly):
+    return assembly["tile16"]
 
 
 @pytest.fixture(scope="module")
-def f8_tiles(tmp_path_factory):
-    return assembly_of("gemm_mfma_f8.hip", tmp_path_factory)
+def f8_tiles(assembly):
+    return assembly["f8_tiles"]
 
 
-def test_accumulators_are_read_only_after_the_wait_states(tile16, f8_tiles):
+@pytest.fixture(scope="module")
+def tile16_f8w(assembly):
+    return assembly["tile16_f8w"]
+
+
+def test_accumulators_are_read_only_after_the_wait_states(tile16, f8_tiles, tile16_f8w):
     checked = 0
-    for lines, part in ((tile16, "mfma_pipe16_kernel"), (tile16, "mfma_pipe16r_kernel"), (f8_tiles, "mfma_pipe_f8x16_kernel")):
+    for lines, part in ((tile16, "mfma_pipe16_kernel"), (tile16, "mfma_pipe16r_kernel"), (f8_tiles, "mfma_pipe_f8x16_kernel"),
+                        (tile16_f8w, "mfma_pipe16_f8w_kernel"), (tile16_f8w, "mfma_pipe16r_f8w_kernel")):
         kernels = kernels_in(lines, part)
         assert kernels, part
         for name, insns in kernels.items():
             assert wait_states_before_the_last_results_are_read(insns) >= MFMA_RESULT_WAIT_STATES, name
             checked += 1
-    assert checked == 4 + 8 + 2  # four layout pairs; the respaced form with and without fused steps; e4m3 and e5m2
+    assert checked == 4 + 8 + 2 + 2 + 2  # four layout pairs; the respaced form with and without fused steps; e4m3 and e5m2;
+    # f8e4m3 weights k-dense and row-dense, both forms
 
 
-def test_an_instruction_separates_every_m0_write_from_the_load_that_uses_it(tile16, f8_tiles):
-    for lines, part in ((tile16, "mfma_pipe16"), (f8_tiles, "mfma_pipe_f8")):
+def test_an_instruction_separates_every_m0_write_from_the_load_that_uses_it(tile16, f8_tiles, tile16_f8w):
+    for lines, part in ((tile16, "mfma_pipe16"), (f8_tiles, "mfma_pipe_f8"), (tile16_f8w, "mfma_pipe16")):
         for name, insns in kernels_in(lines, part).items():
             assert any(s.startswith("global_load_lds") for s in insns), name
             assert loads_too_close_to_an_m0_write(insns) == [], name
@@ -158,3 +180,15 @@ def test_respaced_kernels_m0_bookkeeping(tile16):
             half = len(pieces) // 2
             assert pieces[:half] == list(range(pieces[0], pieces[0] + half * 1024, 1024)), (name, base, pieces)
             assert pieces[half:] == list(range(pieces[half], pieces[half] + half * 1024, 1024)), (name, base, pieces)
+
+
+def test_tile_kernels_keep_their_accumulators_in_registers(assembly):
+    """no scratch memory in any of these kernels: a rolled loop over the accumulators, or a spill, would put them there
+    (the library is built with a raised unroll threshold for that reason; this test uses its flags)"""
+    seen = 0
+    for lines in assembly.values():
+        text = "\n".join(lines)
+        for name, size in re.findall(r"\.amdhsa_kernel (\S*mfma_pipe\S*)[\s\S]*?\.amdhsa_private_segment_fixed_size (\d+)", text):
+            assert int(size) == 0, (name, size)
+            seen += 1
+    assert seen >= 18
