@@ -133,15 +133,8 @@ def load() -> ctypes.CDLL:
     return lib
 
 
-def load_debug() -> ctypes.CDLL:
-    """Load the hooks library (include/hodu_rocm_debug.h); it links against the kernel library."""
-    global _debug_lib
-    if _debug_lib is not None:
-        return _debug_lib
-    load()
-    if not os.path.exists(DEBUG_LIB_PATH):
-        raise ImportError(f"{DEBUG_LIB_PATH} is missing: build it first (python -m hodu_amd.build)")
-    lib = ctypes.CDLL(DEBUG_LIB_PATH)
+def declare_debug(lib: ctypes.CDLL):
+    """argument types of the hooks library (include/hodu_rocm_debug.h)"""
     vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
     szp, fp = ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_float)
     vpp = ctypes.POINTER(vp)
@@ -158,6 +151,18 @@ def load_debug() -> ctypes.CDLL:
     lib.hodu_rocm_debug_mfma_clock.argtypes = [vp, ci, vp, ci, fp, ctypes.POINTER(ctypes.c_double),
                                                ctypes.POINTER(ctypes.c_double)]
     lib.hodu_rocm_debug_read_floor.argtypes = [vp, vpp, sz, sz, ci, fp, fp]
+
+
+def load_debug() -> ctypes.CDLL:
+    """Load the hooks library (include/hodu_rocm_debug.h); it links against the kernel library."""
+    global _debug_lib
+    if _debug_lib is not None:
+        return _debug_lib
+    load()
+    if not os.path.exists(DEBUG_LIB_PATH):
+        raise ImportError(f"{DEBUG_LIB_PATH} is missing: build it first (python -m hodu_amd.build)")
+    lib = ctypes.CDLL(DEBUG_LIB_PATH)
+    declare_debug(lib)
     _debug_lib = lib
     return lib
 

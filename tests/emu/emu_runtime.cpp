@@ -1,6 +1,5 @@
 // Test infrastructure: the CPU build's own part -- the workgroup's LDS, guarded "device" memory, the switches of the
-// instruction models, and exports the tests read the context through (the debug library has no CPU build).  Built
-// twice.  In the library of all kernels (EMU_WITH_RUNTIME) the library's real runtime.cpp is compiled beside it, against
+// instruction models.  Built twice.  In the library of all kernels (EMU_WITH_RUNTIME) the library's real runtime.cpp is compiled beside it, against
 // the runtime API of tests/emu/hip/hip_runtime.h.  In the small library of the plain kernels (softmax, casts, sums,
 // the generic and reference-sum products) this file also stands in for runtime.cpp -- error text, workspace, a bare
 // context -- and every other kernel family's launcher answers UNSUPPORTED, which routes every product to the generic
@@ -104,14 +103,6 @@ void emu_ctx_destroy(hodu_rocm_ctx *ctx) {
 extern "C" {
 const char *emu_last_kernel(hodu_rocm_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
 const char *emu_last_error(void) { return hodu::get_error(); }
-// the testing hooks and the scratch report of the debug library
-void emu_force_tile(hodu_rocm_ctx *ctx, int v) { ctx->force_tile = v; }
-void emu_force_splitk(hodu_rocm_ctx *ctx, int v) { ctx->force_splits = v; }
-void emu_scratch_state(hodu_rocm_ctx *ctx, size_t *workspace_bytes, int *arrival_allocated, int *in_fixed_mode) {
-    *workspace_bytes = ctx->workspace.bytes;
-    *arrival_allocated = ctx->arrival != nullptr;
-    *in_fixed_mode = ctx->fixed_scratch;
-}
 // fills LDS with a pattern, so that a kernel that reads what it has not written does not find the last launch's data
 void emu_lds_fill(int byte) { memset(emu::lds_base(), byte, emu::kLdsBytes); }
 // where an allocation touches its guard page: 1 its end (the default), 0 its start
@@ -122,5 +113,13 @@ const char *emu_unsupported_first(void) { return emu::no_such_instruction_first(
 void emu_unsupported_reset(void) { emu::no_such_instruction_hits() = 0; }
 #ifdef EMU_WITH_RUNTIME
 void emu_dma_lazy(int model) { emu::dma_lazy() = model; }
+// the two probes of the debug library that are kernels written around inline assembly (clock_probe.hip) have no CPU build;
+// the rest of it (csrc_debug/timing.cpp: hooks, scratch report, timing loops, graph replay) is compiled as it is
+int hodu_rocm_debug_mfma_clock(hodu_rocm_ctx *, int, const void *, int, float *, double *, double *) {
+    return hodu::fail(HODU_ROCM_UNSUPPORTED, "the matrix-core clock probe has no CPU build");
+}
+int hodu_rocm_debug_read_floor(hodu_rocm_ctx *, const void *const *, size_t, size_t, int, float *, float *) {
+    return hodu::fail(HODU_ROCM_UNSUPPORTED, "the streaming-read probe has no CPU build");
+}
 #endif
 }

@@ -15,6 +15,7 @@
 #include <sys/mman.h>
 #include <ucontext.h>
 
+#include <chrono>
 #include <cmath>
 #include <condition_variable>
 #include <cstdint>
@@ -76,8 +77,41 @@ constexpr unsigned hipStreamNonBlocking = 1;
 inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { *s = nullptr; return hipSuccess; }
 inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
 inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+// Graphs: while the (one) stream is being captured, a kernel launch or a memset is recorded instead of run; launching
+// the instantiated graph runs the recorded nodes in order.
+struct emu_graph { std::vector<std::function<void()>> nodes; };
+typedef emu_graph *hipGraph_t;
+typedef emu_graph *hipGraphExec_t;
+typedef void *hipGraphNode_t;
+namespace emu {
+inline emu_graph *&capturing() { static emu_graph *g = nullptr; return g; }
+}  // namespace emu
 enum hipStreamCaptureStatus { hipStreamCaptureStatusNone = 0, hipStreamCaptureStatusActive = 1 };
-inline hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus *st) { *st = hipStreamCaptureStatusNone; return hipSuccess; }
+enum hipStreamCaptureMode { hipStreamCaptureModeGlobal = 0, hipStreamCaptureModeThreadLocal = 1, hipStreamCaptureModeRelaxed = 2 };
+inline hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus *st) {
+    *st = emu::capturing() ? hipStreamCaptureStatusActive : hipStreamCaptureStatusNone;
+    return hipSuccess;
+}
+inline hipError_t hipStreamBeginCapture(hipStream_t, hipStreamCaptureMode) {
+    if (emu::capturing()) return hipErrorInvalidValue;
+    emu::capturing() = new emu_graph;
+    return hipSuccess;
+}
+inline hipError_t hipStreamEndCapture(hipStream_t, hipGraph_t *g) {
+    *g = emu::capturing();
+    emu::capturing() = nullptr;
+    return *g ? hipSuccess : hipErrorInvalidValue;
+}
+inline hipError_t hipGraphInstantiate(hipGraphExec_t *exec, hipGraph_t g, hipGraphNode_t *, char *, size_t) {
+    *exec = new emu_graph(*g);
+    return hipSuccess;
+}
+inline hipError_t hipGraphLaunch(hipGraphExec_t exec, hipStream_t) {
+    for (auto &node : exec->nodes) node();
+    return hipSuccess;
+}
+inline hipError_t hipGraphExecDestroy(hipGraphExec_t exec) { delete exec; return hipSuccess; }
+inline hipError_t hipGraphDestroy(hipGraph_t g) { delete g; return hipSuccess; }
 template <class T> inline hipError_t hipMalloc(T **p, size_t bytes) {
     *p = (T *)emu::device_alloc(bytes);
     return *p ? hipSuccess : hipErrorOutOfMemory;
@@ -85,16 +119,26 @@ template <class T> inline hipError_t hipMalloc(T **p, size_t bytes) {
 inline hipError_t hipFree(void *p) { return (!p || emu::device_free(p)) ? hipSuccess : hipErrorInvalidValue; }
 enum hipMemcpyKind { hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
 inline hipError_t hipMemcpyAsync(void *dst, const void *src, size_t bytes, hipMemcpyKind, hipStream_t) { memmove(dst, src, bytes); return hipSuccess; }
-inline hipError_t hipMemsetAsync(void *dst, int byte, size_t bytes, hipStream_t) { memset(dst, byte, bytes); return hipSuccess; }
+inline hipError_t hipMemcpy(void *dst, const void *src, size_t bytes, hipMemcpyKind) { memmove(dst, src, bytes); return hipSuccess; }
+inline hipError_t hipMemsetAsync(void *dst, int byte, size_t bytes, hipStream_t) {
+    if (emu::capturing()) emu::capturing()->nodes.push_back([=] { memset(dst, byte, bytes); });
+    else memset(dst, byte, bytes);
+    return hipSuccess;
+}
 // a __device__ variable is an ordinary one here, and its "device address" its address
 #define HIP_SYMBOL(x) (x)
 template <class T> inline hipError_t hipGetSymbolAddress(void **p, T &symbol) { *p = (void *)&symbol; return hipSuccess; }
-typedef void *hipEvent_t;
-inline hipError_t hipEventCreate(hipEvent_t *e) { *e = nullptr; return hipSuccess; }
-inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
+// events: the host's clock at the moment of recording (everything before it on the one stream has run by then)
+struct emu_event { std::chrono::steady_clock::time_point at; };
+typedef emu_event *hipEvent_t;
+inline hipError_t hipEventCreate(hipEvent_t *e) { *e = new emu_event{std::chrono::steady_clock::now()}; return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t e, hipStream_t) { e->at = std::chrono::steady_clock::now(); return hipSuccess; }
 inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
-inline hipError_t hipEventElapsedTime(float *ms, hipEvent_t, hipEvent_t) { *ms = 0.f; return hipSuccess; }
-inline hipError_t hipEventDestroy(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventElapsedTime(float *ms, hipEvent_t a, hipEvent_t b) {
+    *ms = std::chrono::duration<float, std::milli>(b->at - a->at).count();
+    return hipSuccess;
+}
+inline hipError_t hipEventDestroy(hipEvent_t e) { delete e; return hipSuccess; }
 
 namespace emu {
 constexpr int kWave = 64, kMaxBlock = 1024;
@@ -226,16 +270,10 @@ inline void run_wave(Block &blk, const std::function<void()> &kernel, unsigned w
     blk.all.leave();
 }
 
-template <class K, class... Args> void launch(K kernel, dim3 grid, dim3 block, Args... args) {
-    const unsigned nthreads = block.x * block.y * block.z;
-    if (nthreads == 0 || nthreads > (unsigned)kMaxBlock || nthreads % kWave != 0) {
-        fprintf(stderr, "emu: a workgroup of %u threads is not whole wavefronts\n", nthreads);
-        abort();
-    }
+inline void run_grid(const std::function<void()> &call, dim3 grid, dim3 block) {
     static Block blk;  // (workgroups, and launches, run one at a time)
     current() = &blk;
-    const std::function<void()> call = [=] { kernel(args...); };
-    const unsigned waves = nthreads / kWave;
+    const unsigned waves = block.x * block.y * block.z / kWave;
     for (unsigned bz = 0; bz < grid.z; bz++)
         for (unsigned by = 0; by < grid.y; by++)
             for (unsigned bx = 0; bx < grid.x; bx++) {
@@ -253,6 +291,17 @@ template <class K, class... Args> void launch(K kernel, dim3 grid, dim3 block, A
                 for (auto &th : pool) th.join();
             }
     current() = nullptr;
+}
+
+template <class K, class... Args> void launch(K kernel, dim3 grid, dim3 block, Args... args) {
+    const unsigned nthreads = block.x * block.y * block.z;
+    if (nthreads == 0 || nthreads > (unsigned)kMaxBlock || nthreads % kWave != 0) {
+        fprintf(stderr, "emu: a workgroup of %u threads is not whole wavefronts\n", nthreads);
+        abort();
+    }
+    const std::function<void()> call = [=] { kernel(args...); };
+    if (emu_graph *g = capturing()) g->nodes.push_back([=] { run_grid(call, grid, block); });  // recorded, run at graph launch
+    else run_grid(call, grid, block);
 }
 inline unsigned flat_tid() { return t_lane->flat; }
 }  // namespace emu

@@ -31,7 +31,8 @@ LIB = os.path.join(OUT, "libhodu_emu.so")
 MFMA_SOURCES = [os.path.join(CSRC, f) for f in ("gemm_mfma.hip", "gemm_mfma_bf16.hip", "gemm_mfma_mi16_bf16.hip", "gemm_mfma_w8a16.hip",
                                                 "gemm_mfma_f16.hip", "gemm_mfma_mi16_f16.hip", "gemm_mfma_f32.hip", "gemm_mfma_i8.hip",
                                                 "gemm_mfma_i8_out.hip", "gemm_mfma_u8_out.hip", "gemm_mfma_f8.hip", "skinny.hip",
-                                                "gemv.hip", "gemv_rows.hip", "small_f32.hip", "gemm_f64.hip", "attention.hip", "runtime.cpp")]
+                                                "gemv.hip", "gemv_rows.hip", "small_f32.hip", "gemm_f64.hip", "attention.hip", "runtime.cpp")] + \
+               [os.path.join(ROOT, "hodu_amd", "csrc_debug", "timing.cpp")]
 MFMA_LIB = os.path.join(OUT, "libhodu_emu_mfma.so")
 
 
@@ -197,10 +198,9 @@ class Emu:
 # ---- hodu_amd.ffi.Context over the CPU build, so that the GPU tests' helpers and test functions run against it unchanged ----
 class EmuContext(ffi.Context):
     """hodu_amd.ffi.Context with the CPU build of the whole library (build(mfma=True): every kernel family, api.cpp,
-    runtime.cpp) in the place of the HIP library: the same Python methods with their host-side extent checks, the same
-    entry points, hodu_rocm_alloc handing out host memory between two inaccessible pages.  What it adds are the two
-    testing hooks and the scratch report (the debug library has no CPU build) and the switches of the instruction
-    models."""
+    runtime.cpp, the debug library's timing.cpp) in the place of the HIP libraries: the same Python methods with their
+    host-side extent checks, the same entry points and hooks, hodu_rocm_alloc handing out host memory between two
+    inaccessible pages.  What it adds are the switches of the instruction models."""
 
     _emu_lib = None
 
@@ -213,14 +213,11 @@ class EmuContext(ffi.Context):
             lib = ctypes.CDLL(path)
             ffi.declare_runtime(lib)
             ffi.declare_compute(lib)
-            vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+            ffi.declare_debug(lib)
             lib.emu_unsupported_first.restype = ctypes.c_char_p
-            lib.emu_force_tile.argtypes = [vp, ci]
-            lib.emu_force_splitk.argtypes = [vp, ci]
-            lib.emu_scratch_state.argtypes = [vp, ctypes.POINTER(sz), ctypes.POINTER(ci), ctypes.POINTER(ci)]
-            lib.emu_lds_fill.argtypes = [ci]
-            lib.emu_alloc_tight.argtypes = [ci]
-            lib.emu_dma_lazy.argtypes = [ci]
+            lib.emu_lds_fill.argtypes = [ctypes.c_int]
+            lib.emu_alloc_tight.argtypes = [ctypes.c_int]
+            lib.emu_dma_lazy.argtypes = [ctypes.c_int]
             cls._emu_lib = lib
         return cls._emu_lib
 
@@ -247,7 +244,7 @@ class EmuContext(ffi.Context):
 
     @property
     def debug(self):
-        raise RuntimeError("the hooks library has no CPU build")
+        return self.lib  # the hooks are part of the same library here
 
     def _check(self, rc):
         super()._check(rc)
@@ -255,17 +252,6 @@ class EmuContext(ffi.Context):
             first = self.lib.emu_unsupported_first().decode()
             self.lib.emu_unsupported_reset()
             raise AssertionError(f"{self.last_kernel()} reached an instruction without a CPU stand-in: {first}")
-
-    def force_tile(self, tile):
-        self.lib.emu_force_tile(self.handle, int(tile))
-
-    def force_splitk(self, splits):
-        self.lib.emu_force_splitk(self.handle, int(splits))
-
-    def scratch_state(self):
-        ws, arr, fixed = ctypes.c_size_t(), ctypes.c_int(), ctypes.c_int()
-        self.lib.emu_scratch_state(self.handle, ctypes.byref(ws), ctypes.byref(arr), ctypes.byref(fixed))
-        return {"workspace_bytes": ws.value, "arrival_allocated": bool(arr.value), "fixed": bool(fixed.value)}
 
     def dma_lazy(self, model):
         """LDS-DMA bytes arrive at issue (0), only when an s_waitcnt vmcnt retires them (1), or one load later than

@@ -12,10 +12,12 @@ with the models pinned that way, the same run is a regression test of the kernel
 selection logic where no GPU is at hand.
 
 By default the cases that take more than a few seconds each are skipped; HODU_EMU_ALL=1 runs them too (about a
-quarter of an hour on 8 cores).  Not run here: tests that time kernels, capture graphs or otherwise need the debug
-library, the Tensor-level tests (tests/test_emu_host_mirror_cpu.py runs those), BASELINE's config 5 and config 3 at
-M = 4096 at their full sizes (hours here; configs 1 to 4 otherwise do run at full size) and
-tests/test_gpu_large_extents.py (operands of several GiB)."""
+third of an hour on 8 cores).  The debug library's hooks, timing loops and graph replay are part of the CPU build, so
+tests that use them run too (a graph is recorded and replayed by the stand-in runtime; times are the host's).  Not run here:
+one test of thousands of large launches, the Tensor-level tests (tests/test_emu_host_mirror_cpu.py runs those) and
+tests/test_gpu_large_extents.py (operands of several GiB).  BASELINE's five configurations run at their full sizes
+(tests/test_gpu_configs.py): 1, 2, 3 up to M = 256 and 4 with HODU_EMU_ALL=1, config 3 at M = 4096 and config 5 -- three
+minutes and a quarter of an hour per case -- with HODU_EMU_ALL=2."""
 import importlib
 import inspect
 import itertools
@@ -31,15 +33,10 @@ pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host cla
 SUITES = ["test_gpu_products", "test_gpu_mfma", "test_gpu_exact", "test_gpu_epilogue", "test_gpu_skinny", "test_gpu_small_f32",
           "test_gpu_f64", "test_gpu_casts", "test_gpu_sum", "test_gpu_softmax", "test_gpu_attention", "test_zz_no_alloc",
           "test_zx_softmax_masked", "test_zy_reference_sums",
-          "test_gpu_configs",  # BASELINE's configurations at their full sizes: 1 - 4 (3 up to M = 256)
+          "test_gpu_configs",  # BASELINE's five configurations at their full sizes
           # the GPU test of kernels that have not run on a GPU, kept under a name pytest does not collect: it runs here
           "wip_pipe16r"]
-# needs the debug library (timing, thousands of launches)
-EXCLUDED = {"test_gpu_skinny.test_split_k_arrival_protocol_over_thousands_of_launches",
-            "test_zz_no_alloc.test_captured_into_a_graph_and_replayed",  # (graph capture and timing: the debug library)
-            # hours in the CPU build: config 5 (2 x 4096 x 4096 x 14336 per weight kind) and config 3 at M = 4096
-            "test_gpu_configs.test_config5_mlp_broadcast", "test_gpu_configs.test_config3_fp8_weight_linear[4096-448.0]",
-            "test_gpu_configs.test_config3_fp8_weight_linear[4096-240.0]",
+EXCLUDED = {"test_gpu_skinny.test_split_k_arrival_protocol_over_thousands_of_launches",  # (thousands of large launches)
             "test_zx_softmax_masked.test_attention_with_a_padding_mask_against_float64"}  # (the host mirror)
 # more than a few seconds per case in the CPU build
 HEAVY = {
@@ -59,12 +56,18 @@ HEAVY = {
     "test_gpu_softmax.test_causal_mask", "test_gpu_softmax.test_long_and_strided_rows",
     "test_zz_no_alloc.test_two_calls_in_a_row_the_second_smaller", "test_zz_no_alloc.test_a_fresh_context_allocates_nothing_for_it",
     "test_zz_no_alloc.test_scratch_beyond_the_limit_is_refused", "test_zz_no_alloc.test_shapes_without_scratch",
+    "test_zz_no_alloc.test_captured_into_a_graph_and_replayed",
     "test_gpu_configs.test_config2_bf16_batched_transposed", "test_gpu_configs.test_config3_fp8_weight_linear",
     "test_gpu_configs.test_config4_int8_valued_i32",
     "wip_pipe16r.test_respaced_16x16_instruction_all_layouts", "wip_pipe16r.test_respaced_is_exact_on_exact_operands",
     "wip_pipe16r.test_respaced_f8_weight_tile_is_exact",
 }
-RUN_ALL = os.environ.get("HODU_EMU_ALL", "") not in ("", "0")
+# a quarter of an hour and more per case: config 5 (2 x 4096 x 4096 x 14336 per weight kind: 16 and 18 minutes on 8 cores)
+# and config 3 at M = 4096 (3 minutes per scale)
+VERY_HEAVY = {"test_gpu_configs.test_config5_mlp_broadcast", "test_gpu_configs.test_config3_fp8_weight_linear[4096-448.0]",
+              "test_gpu_configs.test_config3_fp8_weight_linear[4096-240.0]"}
+LEVEL = int(os.environ.get("HODU_EMU_ALL", "0") or 0)
+RUN_ALL = LEVEL >= 1
 
 
 def _expansions(fn):
@@ -97,10 +100,15 @@ def _cases():
             for kwargs in _expansions(fn):
                 if set(params) - {"ctx"} != set(kwargs):
                     continue  # wants a fixture this file does not provide
-                if full + "[" + "-".join(str(v) for v in kwargs.values()) + "]" in EXCLUDED:
+                case = full + "[" + "-".join(str(v) for v in kwargs.values()) + "]"
+                if case in EXCLUDED:
                     continue
                 ident = full.replace("test_gpu_", "", 1).replace("wip_", "unrun_on_gpu_", 1) + ("[" + "-".join(str(v) for v in kwargs.values()) + "]" if kwargs else "")
-                marks = [pytest.mark.skip(reason="slow in the CPU build: set HODU_EMU_ALL=1")] if full in HEAVY and not RUN_ALL else []
+                marks = []
+                if (full in VERY_HEAVY or case in VERY_HEAVY) and LEVEL < 2:
+                    marks = [pytest.mark.skip(reason="a quarter of an hour and more in the CPU build: set HODU_EMU_ALL=2")]
+                elif full in HEAVY and not RUN_ALL:
+                    marks = [pytest.mark.skip(reason="slow in the CPU build: set HODU_EMU_ALL=1")]
                 yield pytest.param(fn, kwargs, id=ident, marks=marks)
 
 
