@@ -4,6 +4,8 @@ import json
 import os
 import sys
 
+import pytest
+
 sys.path.insert(0, os.path.join(os.path.dirname(__file__), ".."))
 import bench  # noqa: E402
 
@@ -71,3 +73,26 @@ def test_line_without_cpu_leg():
     results, _ = _canned()
     line, _ = bench.assemble_line(5, 2, "c5_down_bf16", 4.81e11, 2.684e8, results, None, None)
     assert "cpu_baseline" not in line and line["steps"] == 5 and line["warmup"] == 2
+
+
+@pytest.mark.skipif(os.environ.get("HODU_EMU_ALL", "0") in ("", "0"), reason="slow in the CPU build: set HODU_EMU_ALL=1")
+def test_timed_cases_and_the_line_against_the_cpu_build():
+    """bench.py's own per-case routine -- buffers, the timing loop of the debug library, the in-run parity check of a
+    timed output buffer -- on config 1 and config 3 at M = 1 at their full sizes against the CPU build of the library
+    (tests/emu_util.py), and the JSON line assembled from those rows.  The times are the emulation's and mean nothing."""
+    import emu_util
+    if emu_util.compiler() is None:
+        pytest.skip("no host clang++ for the CPU build")
+    ctx = emu_util.EmuContext()
+    try:
+        cases = {c.key: c for c in bench.build_cases({"c1", "c3"})}
+        rows = [bench.time_case(ctx, cases["c1"], 2, 1, exact_steps=True), bench.time_case(ctx, cases["c3_m1"], 2, 1, headline=(2, 1))]
+    finally:
+        ctx.close()
+    assert [r["kernel"] for r in rows] == ["small_f32_KM", "gemv_bf16_f8w_walk"]
+    assert all(r["parity"] and r["parity"]["rows_checked"] >= 1 for r in rows)
+    line, _ = bench.assemble_line(2, 1, "c3_m1", cases["c3_m1"].flops, cases["c3_m1"].alg_bytes, rows, None, None)
+    text = json.dumps(line, separators=(",", ":"))
+    assert len(text) < bench.LINE_LIMIT
+    per_config = json.loads(text)["roofline"]["per_config"]
+    assert [(row[0], row[2], row[6]) for row in per_config] == [("c1", "mfma", "small_f32_KM"), ("c3_m1", "hbm", "gemv_bf16_f8w_walk")]
