@@ -13,6 +13,8 @@
 // fused step would have to pick one of the two.
 #pragma once
 
+#include <type_traits>
+
 #include "device_types.hpp"
 
 namespace hodu {
@@ -93,6 +95,14 @@ HODU_EPI_NONE(HODU_F8E4M3)
 HODU_EPI_NONE(HODU_F8E5M2)
 #undef HODU_EPI_NONE
 
+// a * b in the type the reference computes in.  Two 16-bit integers would be promoted to int, where 65535 * 65535
+// overflows -- undefined, although every compiler in sight produces the wrapped product the reference's
+// `uint16_t x = a * b` means; multiplied as unsigned the wrap is what the language says.
+template <class W> __device__ __forceinline__ W epi_mul(W a, W b) {
+    if constexpr (std::is_integral<W>::value && sizeof(W) == 2) return (W)((unsigned)a * (unsigned)b);
+    else return (W)(a * b);
+}
+
 // v: the element the product alone would store at column n of its row; returns what the fused launch stores.
 // e.n is the same for every lane, so a product without an epilogue pays one scalar compare per call.  The loop over
 // the steps stays rolled and every step narrows in one place: the routine is inlined at every store site of every
@@ -112,7 +122,7 @@ __device__ __forceinline__ typename EpiElem<DT>::T epilogue_apply(const DevEpilo
         if (s.op == EPI_ADD_ROW) {
             r = (W)(x + E::widen(static_cast<const T *>(s.vec)[n * s.stride]));
         } else if (s.op == EPI_MUL_SCALAR) {
-            r = (W)(x * E::widen(__builtin_bit_cast(T, (U)s.scalar)));
+            r = epi_mul<W>(x, E::widen(__builtin_bit_cast(T, (U)s.scalar)));
         } else if (E::floating) {  // EPI_RELU
             r = x > (W)0 ? x : (W)0;
         }
@@ -177,7 +187,7 @@ __device__ __forceinline__ void epilogue_apply_prepared(const EpiPrepared<DT, EP
             for (int k = 0; k < EPV; k++) r[k] = (W)(r[k] + p.k[i][k]);
         } else if (p.op[i] == EPI_MUL_SCALAR) {
 #pragma unroll
-            for (int k = 0; k < EPV; k++) r[k] = (W)(r[k] * p.k[i][0]);
+            for (int k = 0; k < EPV; k++) r[k] = epi_mul<W>(r[k], p.k[i][0]);
         } else if (E::floating) {  // EPI_RELU
 #pragma unroll
             for (int k = 0; k < EPV; k++) r[k] = r[k] > (W)0 ? r[k] : (W)0;
@@ -213,7 +223,7 @@ __device__ __forceinline__ void epilogue_apply_prepared_group(const EpiPrepared<
 #pragma unroll
             for (int q = 0; q < G; q++)
 #pragma unroll
-                for (int k = 0; k < EPV; k++) r[q][k] = E::widen(E::narrow((W)(r[q][k] * p.k[i][0])));
+                for (int k = 0; k < EPV; k++) r[q][k] = E::widen(E::narrow(epi_mul<W>(r[q][k], p.k[i][0])));
         } else if (E::floating) {  // EPI_RELU
 #pragma unroll
             for (int q = 0; q < G; q++)

@@ -23,7 +23,8 @@ from hodu_amd import ffi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EMU = os.path.join(ROOT, "tests", "emu")
-OUT = os.path.join(EMU, "_build")
+SANITIZE = os.environ.get("HODU_EMU_SANITIZE", "") not in ("", "0")  # an undefined-behaviour-checked build of its own
+OUT = os.path.join(EMU, "_build_ubsan" if SANITIZE else "_build")
 CSRC = os.path.join(ROOT, "hodu_amd", "csrc")
 SOURCES = [os.path.join(CSRC, f) for f in ("api.cpp", "metadata.cpp", "softmax.hip", "cast.hip", "reduce.hip", "gemm_generic.hip", "gemm_refsum.hip")] + \
           [os.path.join(EMU, "emu_runtime.cpp")]
@@ -59,8 +60,14 @@ def build(mfma=False):
     if os.path.exists(lib) and os.path.getmtime(lib) > _newest_input():
         return lib
     os.makedirs(OUT, exist_ok=True)
+    sanitize = SANITIZE
     flags = ["-std=c++17", "-fPIC", "-x", "c++", f"-I{EMU}", f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
              "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-psabi"]
+    if sanitize:
+        # undefined behaviour in the kernels' and the host code's own arithmetic (signed overflow in index arithmetic,
+        # shifts, out-of-range conversions, indexing past a fixed-size array) aborts with a report.  Not the alignment
+        # check: the kernels' 16-byte accesses at element alignment are what the hardware does.
+        flags += ["-fsanitize=undefined", "-fno-sanitize=alignment,vptr,function", "-fno-sanitize-recover=all", "-g1"]
     with_models = ["-DEMU_WITH_RUNTIME", "-include", os.path.join(EMU, "gfx950_insn_emu.hpp")]
     # Without optimisation: a fifth of the compile time (cast.hip alone takes a minute at -O1), and a run spends its
     # time starting threads and in the lanes' barriers, not in the kernels' arithmetic.
@@ -85,7 +92,8 @@ def build(mfma=False):
     with ThreadPoolExecutor(max_workers=7) as ex:
         objs = list(ex.map(one, jobs))
     tmp = lib + f".{os.getpid()}.tmp"
-    r = subprocess.run([cxx, "-shared", "-o", tmp, *objs, "-lpthread"], capture_output=True, text=True)
+    r = subprocess.run([cxx, "-shared", "-o", tmp, *objs, "-lpthread", *(["-fsanitize=undefined", "-shared-libsan"] if sanitize else [])],
+                       capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link of the CPU build failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, lib)
