@@ -23,8 +23,11 @@ from hodu_amd import ffi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EMU = os.path.join(ROOT, "tests", "emu")
-SANITIZE = os.environ.get("HODU_EMU_SANITIZE", "") not in ("", "0")  # an undefined-behaviour-checked build of its own
-OUT = os.path.join(EMU, "_build_ubsan" if SANITIZE else "_build")
+# HODU_EMU_SANITIZE=1: an undefined-behaviour-checked build of its own; =thread: a race-checked one, which only a
+# program that carries the ThreadSanitizer runtime can load (build_race_driver, build_race_checked_python)
+RACE_CHECKED = os.environ.get("HODU_EMU_SANITIZE", "") == "thread"
+SANITIZE = os.environ.get("HODU_EMU_SANITIZE", "") not in ("", "0") and not RACE_CHECKED
+OUT = os.path.join(EMU, "_build_tsan" if RACE_CHECKED else "_build_ubsan" if SANITIZE else "_build")
 CSRC = os.path.join(ROOT, "hodu_amd", "csrc")
 SOURCES = [os.path.join(CSRC, f) for f in ("api.cpp", "metadata.cpp", "softmax.hip", "cast.hip", "reduce.hip", "gemm_generic.hip", "gemm_refsum.hip")] + \
           [os.path.join(EMU, "emu_runtime.cpp")]
@@ -51,16 +54,18 @@ def _newest_input():
     return max(os.path.getmtime(p) for p in paths)
 
 
-def build(mfma=False):
-    """compiles the CPU build unless it is newer than every input; returns the library's path (None: no host clang)"""
+def build(mfma=False, race_checked=RACE_CHECKED):
+    """compiles the CPU build unless it is newer than every input; returns the library's path (None: no host clang).
+    race_checked: a build of its own under ThreadSanitizer, for a natively linked program (build_race_driver)"""
     cxx = compiler()
     if cxx is None:
         return None
-    lib = MFMA_LIB if mfma else LIB
+    OUT = os.path.join(EMU, "_build_tsan") if race_checked else globals()["OUT"]
+    lib = os.path.join(OUT, os.path.basename(MFMA_LIB if mfma else LIB))
     if os.path.exists(lib) and os.path.getmtime(lib) > _newest_input():
         return lib
     os.makedirs(OUT, exist_ok=True)
-    sanitize = SANITIZE
+    sanitize = SANITIZE and not race_checked
     flags = ["-std=c++17", "-fPIC", "-x", "c++", f"-I{EMU}", f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
              "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-psabi"]
     if sanitize:
@@ -68,6 +73,11 @@ def build(mfma=False):
         # shifts, out-of-range conversions, indexing past a fixed-size array) aborts with a report.  Not the alignment
         # check: the kernels' 16-byte accesses at element alignment are what the hardware does.
         flags += ["-fsanitize=undefined", "-fno-sanitize=alignment,vptr,function", "-fno-sanitize-recover=all", "-g1"]
+    if race_checked:
+        # every load and store of the kernels' source is recorded per host thread, i.e. per wavefront.  Not function
+        # entries and exits: the lanes of a wavefront are contexts that one thread switches between in the middle of
+        # functions, which the sanitizer's per-thread call stack cannot follow (reports name the accessing line only).
+        flags += ["-fsanitize=thread", "-mllvm", "-tsan-instrument-func-entry-exit=0", "-g1"]
     with_models = ["-DEMU_WITH_RUNTIME", "-include", os.path.join(EMU, "gfx950_insn_emu.hpp")]
     # Without optimisation: a fifth of the compile time (cast.hip alone takes a minute at -O1), and a run spends its
     # time starting threads and in the lanes' barriers, not in the kernels' arithmetic.
@@ -93,11 +103,54 @@ def build(mfma=False):
         objs = list(ex.map(one, jobs))
     tmp = lib + f".{os.getpid()}.tmp"
     r = subprocess.run([cxx, "-shared", "-o", tmp, *objs, "-lpthread", *(["-fsanitize=undefined", "-shared-libsan"] if sanitize else [])],
-                       capture_output=True, text=True)
+                       capture_output=True, text=True)  # (race_checked: the program that links it brings the runtime)
     if r.returncode != 0:
         raise RuntimeError(f"link of the CPU build failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, lib)
     return lib
+
+
+def build_race_driver():
+    """tests/emu/race_driver.cpp linked with the ThreadSanitizer build of all kernels; returns the program's path"""
+    kernels = build(mfma=True, race_checked=True)
+    if kernels is None:
+        return None
+    out_dir = os.path.dirname(kernels)
+    exe, src = os.path.join(out_dir, "race_driver"), os.path.join(EMU, "race_driver.cpp")
+    if os.path.exists(exe) and os.path.getmtime(exe) > max(os.path.getmtime(kernels), os.path.getmtime(src)):
+        return exe
+    tmp = exe + f".{os.getpid()}.tmp"
+    cmd = [compiler(), "-std=c++17", "-O0", "-g1", "-fsanitize=thread", "-mllvm", "-tsan-instrument-func-entry-exit=0", "-x", "c++",
+           f"-I{EMU}", f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}", f"-I{os.path.join(ROOT, 'hodu_amd', 'csrc_debug')}",
+           "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-psabi", "-DEMU_WITH_RUNTIME", "-include", os.path.join(EMU, "gfx950_insn_emu.hpp"),
+           src, "-o", tmp, f"-L{out_dir}", "-lhodu_emu_mfma", "-lpthread", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"race driver failed to build:\n{r.stderr[-4000:]}")
+    os.replace(tmp, exe)
+    return exe
+
+
+def build_race_checked_python():
+    """tests/emu/python_host.cpp: this Python with the ThreadSanitizer runtime linked in; returns the program's path
+    (None: no host clang, or no Python headers / library to link)"""
+    import sysconfig
+    cxx, inc, libdir = compiler(), sysconfig.get_paths()["include"], sysconfig.get_config_var("LIBDIR")
+    ver = sysconfig.get_config_var("LDVERSION")
+    if cxx is None or not os.path.exists(os.path.join(inc, "Python.h")) or not ver:
+        return None
+    out_dir = os.path.join(EMU, "_build_tsan")
+    os.makedirs(out_dir, exist_ok=True)
+    exe, src = os.path.join(out_dir, "python_tsan"), os.path.join(EMU, "python_host.cpp")
+    if os.path.exists(exe) and os.path.getmtime(exe) > os.path.getmtime(src):
+        return exe
+    tmp = exe + f".{os.getpid()}.tmp"
+    r = subprocess.run([cxx, "-O1", "-fsanitize=thread", f"-I{inc}", src, "-o", tmp, f"-L{libdir}", f"-lpython{ver}", "-ldl", "-lm"],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        return None
+    os.replace(tmp, exe)
+    return exe
 
 
 HOST_LIB = os.path.join(OUT, "libhodu_emu_host.so")
