@@ -381,8 +381,9 @@ int hodu_rocm_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void
                                  (long)mask_layout[1 + nd], causal ? 1 : 0);
 }
 
-int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
-                        const size_t *md, size_t len, const void *scale, int causal) {
+static int attention_entry(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                           const size_t *md, size_t len, const void *scale, int causal, const void *mask, int mask_dtype,
+                           const size_t *mask_layout, size_t mask_layout_len, bool masked) {
     clear_error();
     if (!ctx) return fail(HODU_ROCM_INVALID_ARG, "attention: context is null");
     if (!q || !k || !v || !out || !scale) return fail(HODU_ROCM_INVALID_ARG, "attention: null pointer");
@@ -390,6 +391,23 @@ int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void
     AttentionArgs a;
     int rc = parse_attention_metadata(md, len, &a);
     if (rc) return rc;
+    AttentionMask m;
+    if (masked) {
+        if (!mask) return fail(HODU_ROCM_INVALID_ARG, "attention: null mask pointer");
+        if (mask == out) return fail(HODU_ROCM_INVALID_ARG, "attention: out aliases the mask");
+        if (mask_dtype != HODU_BOOL && mask_dtype != HODU_U8 && mask_dtype != HODU_I8)
+            return fail(HODU_ROCM_UNSUPPORTED, "attention: the mask is one byte per element (bool, u8 or i8), got dtype id %d", mask_dtype);
+        const size_t nd = (size_t)a.nb + 2;
+        if (!mask_layout || mask_layout_len != nd + 2 || mask_layout[0] != nd)
+            return fail(HODU_ROCM_INVALID_ARG, "attention: the mask layout is [nd, strides (nd).., offset] over the %zu dims of the scores", nd);
+        for (size_t i = 1; i < nd + 2; i++)
+            if (mask_layout[i] > 0x7FFFFFFFFFFFL) return fail(HODU_ROCM_INVALID_ARG, "attention: mask layout[%zu] out of range", i);
+        m.ptr = mask;
+        for (int d = 0; d < a.nb; d++) m.bs[d] = (long)mask_layout[1 + d];
+        m.row = (long)mask_layout[1 + a.nb];
+        m.key = (long)mask_layout[2 + a.nb];
+        m.off = (long)mask_layout[1 + nd];
+    }
     if (dtype == HODU_BF16) {
         uint16_t h;
         memcpy(&h, scale, 2);
@@ -406,11 +424,22 @@ int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void
     if (a.batches == 0 || a.sq == 0) return HODU_ROCM_OK;
     std::lock_guard<std::recursive_mutex> hold(ctx->mu);
     HODU_HIP(hipSetDevice(ctx->device));
-    rc = launch_attention(ctx, dtype, q, k, v, out, a);
+    rc = launch_attention(ctx, dtype, q, k, v, out, a, masked ? &m : nullptr);
     if (rc == HODU_ROCM_UNSUPPORTED)
         return fail(HODU_ROCM_UNSUPPORTED, "attention: the fused kernel needs head dim 64 or 128, at most %d batch dims, 16-byte aligned rows and a positive finite scale",
                     kKernelBatchDims);
     return rc;
+}
+
+int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                        const size_t *md, size_t len, const void *scale, int causal) {
+    return attention_entry(ctx, dtype, q, k, v, out, md, len, scale, causal, nullptr, 0, nullptr, 0, false);
+}
+
+int hodu_rocm_attention_masked(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                               const size_t *md, size_t len, const void *scale, int causal, const void *mask, int mask_dtype,
+                               const size_t *mask_layout, size_t mask_layout_len) {
+    return attention_entry(ctx, dtype, q, k, v, out, md, len, scale, causal, mask, mask_dtype, mask_layout, mask_layout_len, true);
 }
 
 int hodu_rocm_contiguous(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *md, size_t len) {

@@ -34,6 +34,17 @@
 // three-launch path and the reference), exp(scale * (s - m)) as one fused multiply-add into a base-2 exponential, P
 // (at most 2^8) rounded to the storage type only as the second product's operand, O accumulated in f32 and rounded
 // once.  The scale is the scalar in the storage type, widened.
+//
+// With an attn_mask (attention.rs:50-56; the MASKED instantiations, a kernel of their own so that the plain one's code
+// does not change): a lane reads the mask bytes of its row's 16 keys of a block in place, through the mask's own
+// strides (0 where it is broadcast), and a masked score becomes fill / scale, fill being what the reference's
+// masked_fill writes over the SCALED scores in a 16-bit type (get_neg_inf, attention.rs:88-96, through full_like's
+// rounding: -65504 in f16, -65536 in bf16) -- a finite value, so a row masked entirely comes out as the reference's
+// uniform average of V over all keys, and any open key zeroes the masked ones (exp(fill - max) = 0 in f32).  The
+// causal mask is filled the same way there, so with a mask the kernel walks every key block: a row whose open causal
+// keys are all masked averages over the future keys too.  Keys past Sk stay at -inf: they do not exist.
+#include <type_traits>
+
 #include "common.hpp"
 #include "device_types.hpp"
 #include "gemm_mfma_pipe.hpp"
@@ -79,6 +90,14 @@ struct DevAttention {
     int q_blocks;
 };
 
+struct DevMask {
+    const uint8_t *ptr;
+    long bs[kKernelBatchDims];  // element (= byte) strides over the batch dims, 0 where the mask is broadcast
+    long row, key, off;         // strides along Sq and Sk, offset
+    float fill_raw;             // the reference's fill value divided by the scale
+};
+struct NoMask {};
+
 template <int CK> struct Narrow;
 template <> struct Narrow<mfma::CK_BF16> {
     static __device__ __forceinline__ uint32_t pack(float lo, float hi) {  // one v_cvt_pk_bf16_f32
@@ -103,10 +122,11 @@ __device__ __forceinline__ float partner(float v) {
     return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
 }
 
-template <int CK, int D>
+template <int CK, int D, class MK>
 __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K,
                                                                const uint16_t *__restrict__ V, uint16_t *__restrict__ O,
-                                                               DevAttention a) {
+                                                               DevAttention a, MK mk) {
+    constexpr bool MASKED = !std::is_same<MK, NoMask>::value;
     typedef Compute32<CK> Cmp;
     typedef typename Cmp::acc_t acc_t;
     typedef AtGeom<D> G;
@@ -121,6 +141,8 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     const long batch = blockIdx.x % a.batches;
     const int q0 = (a.q_blocks - 1 - (int)(blockIdx.x / a.batches)) * AT_BQ;
     long qo = a.q_off, ko = a.k_off, vo = a.v_off;
+    [[maybe_unused]] long mo = 0;
+    if constexpr (MASKED) mo = mk.off;
     {
         long b = batch;
 #pragma unroll
@@ -129,12 +151,13 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
                 const long i = b % a.bshape[d];
                 b /= a.bshape[d];
                 qo += i * a.q_bs[d]; ko += i * a.k_bs[d]; vo += i * a.v_bs[d];
+                if constexpr (MASKED) mo += i * mk.bs[d];
             }
     }
 
     // keys this workgroup needs: with the causal mask nothing beyond its last query row
     int k_end = a.sk;
-    if (a.causal) {
+    if (!MASKED && a.causal) {
         const int last = q0 + AT_BQ < a.sq ? q0 + AT_BQ : a.sq;
         k_end = last < a.sk ? last : a.sk;
     }
@@ -231,13 +254,14 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     const int wave_row0 = q0 + qg * 32;  // the wavefront's first query row
     // the wavefront has nothing to do in a block whose 32 keys of its half lie past the end, or past the mask of all
     // its 32 rows; the tile needs the per-element mask at the ragged end of the keys and where it meets the diagonal
+    // (with an attn_mask every block takes the per-element path and the causal mask skips nothing: see the top)
     auto idle_in = [&](int kb) {
         const int key0 = kb * AT_BK + kh * 32;
-        return kb >= n_blocks || key0 >= a.sk || (a.causal && key0 > wave_row0 + 31);
+        return kb >= n_blocks || key0 >= a.sk || (!MASKED && a.causal && key0 > wave_row0 + 31);
     };
     auto edge_in = [&](int kb) {
         const int key0 = kb * AT_BK + kh * 32;
-        return key0 + 32 > a.sk || (a.causal && key0 + 31 > wave_row0);
+        return MASKED || key0 + 32 > a.sk || (a.causal && key0 + 31 > wave_row0);
     };
 
     // ---- the phases ----
@@ -265,11 +289,32 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     };
     auto mask = [&](acc_t &sc, int kb) {
         const int key0 = kb * AT_BK + kh * 32;
-        const int limit = a.causal && my_row < a.sk - 1 ? my_row : a.sk - 1;  // last key the row attends
+        if constexpr (MASKED) {
+            // the row's mask bytes of the lane's 16 keys (a row past Sq reads the last row's, a key past Sk the last key's)
+            const uint8_t *mrow = mk.ptr + mo + (long)q_row * mk.row;
+            uint8_t open[16];
 #pragma unroll
-        for (int q = 0; q < 4; q++)
+            for (int q = 0; q < 4; q++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) sc[4 * q + e] = key0 + 8 * q + 4 * lh + e > limit ? -INFINITY : sc[4 * q + e];
+                for (int e = 0; e < 4; e++) {
+                    const int key = key0 + 8 * q + 4 * lh + e;
+                    open[4 * q + e] = mrow[(long)(key < a.sk ? key : a.sk - 1) * mk.key];
+                }
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int key = key0 + 8 * q + 4 * lh + e;
+                    const bool filled = open[4 * q + e] == 0 || (a.causal && key > my_row);
+                    sc[4 * q + e] = key >= a.sk ? -INFINITY : filled ? mk.fill_raw : sc[4 * q + e];
+                }
+        } else {
+            const int limit = a.causal && my_row < a.sk - 1 ? my_row : a.sk - 1;  // last key the row attends
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) sc[4 * q + e] = key0 + 8 * q + 4 * lh + e > limit ? -INFINITY : sc[4 * q + e];
+        }
     };
     // The reference value m_run of a row (exponents are taken relative to it) follows the running maximum lazily: it
     // moves only when a block's maximum exceeds it by more than 8 in the base-2 exponent, so P stays below 2^8 --
@@ -440,8 +485,8 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
     __syncthreads();
     if (kh == 1) return;
     {
-        // the first half has seen key 0, which no row masks: its reference is finite; the second half's may be -inf
-        // (w2 = 0).  Any common reference gives the same quotient.
+        // the first half has seen key 0, which no row masks (an attn_mask fills it with a finite value): its reference
+        // is finite; the second half's may be -inf (w2 = 0).  Any common reference gives the same quotient.
         const float m2 = mg[0], l2 = mg[64];
         const float m = __builtin_fmaxf(m2, m_run);
         const float w1 = __builtin_amdgcn_exp2f((m_run - m) * a.scale_log2e), w2 = __builtin_amdgcn_exp2f((m2 - m) * a.scale_log2e);
@@ -471,7 +516,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
 
 // returns HODU_ROCM_UNSUPPORTED (no error text) when the fused kernel does not take the call
 int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
-                     const AttentionArgs &g) {
+                     const AttentionArgs &g, const AttentionMask *mask) {
     if (dtype != HODU_BF16 && dtype != HODU_F16) return HODU_ROCM_UNSUPPORTED;
     if ((g.d != 64 && g.d != 128) || g.sq < 1 || g.sk < 1 || g.batches < 1) return HODU_ROCM_UNSUPPORTED;
     // the row maximum is taken before the scale is applied: the scale must be positive (and finite)
@@ -500,20 +545,45 @@ int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k
     a.q_blocks = (int)((g.sq + AT_BQ - 1) / AT_BQ);
     const long blocks = g.batches * a.q_blocks;
     if (blocks > 0x7FFFFFFFL) return HODU_ROCM_UNSUPPORTED;
+    if (mask) {
+        DevMask mk{};
+        mk.ptr = (const uint8_t *)mask->ptr;
+        for (int d = 0; d < kKernelBatchDims; d++) mk.bs[d] = d < g.nb ? mask->bs[d] : 0;
+        mk.row = mask->row; mk.key = mask->key; mk.off = mask->off;
+        // what masked_fill writes over the scaled scores (get_neg_inf through full_like's rounding), before the scale
+        mk.fill_raw = (dtype == HODU_BF16 ? -65536.f : -65504.f) / g.scale;
+        auto launch_masked = [&](auto kernel, int lds, const char *name) -> int {
+            if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), lds)) return rc;
+            ctx->last_kernel = name;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(AT_NT), lds, ctx->stream, (const uint16_t *)q, (const uint16_t *)k,
+                               (const uint16_t *)v, (uint16_t *)out, a, mk);
+            return HODU_ROCM_OK;
+        };
+        int rc;
+        if (g.d == 128)
+            rc = dtype == HODU_BF16 ? launch_masked(attention_fwd_kernel<mfma::CK_BF16, 128, DevMask>, AtGeom<128>::LDS, "attention_masked_fwd_bf16")
+                                    : launch_masked(attention_fwd_kernel<mfma::CK_F16, 128, DevMask>, AtGeom<128>::LDS, "attention_masked_fwd_f16");
+        else
+            rc = dtype == HODU_BF16 ? launch_masked(attention_fwd_kernel<mfma::CK_BF16, 64, DevMask>, AtGeom<64>::LDS, "attention_masked_fwd_bf16_d64")
+                                    : launch_masked(attention_fwd_kernel<mfma::CK_F16, 64, DevMask>, AtGeom<64>::LDS, "attention_masked_fwd_f16_d64");
+        if (rc != HODU_ROCM_OK) return rc;
+        HODU_HIP(hipGetLastError());
+        return HODU_ROCM_OK;
+    }
     auto launch = [&](auto kernel, int lds, const char *name) -> int {
         if (int rc = ensure_dynamic_lds(ctx, reinterpret_cast<const void *>(kernel), lds)) return rc;
         ctx->last_kernel = name;
         hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(AT_NT), lds, ctx->stream, (const uint16_t *)q, (const uint16_t *)k,
-                           (const uint16_t *)v, (uint16_t *)out, a);
+                           (const uint16_t *)v, (uint16_t *)out, a, NoMask{});
         return HODU_ROCM_OK;
     };
     int rc;
     if (g.d == 128)
-        rc = dtype == HODU_BF16 ? launch(attention_fwd_kernel<mfma::CK_BF16, 128>, AtGeom<128>::LDS, "attention_fwd_bf16")
-                                : launch(attention_fwd_kernel<mfma::CK_F16, 128>, AtGeom<128>::LDS, "attention_fwd_f16");
+        rc = dtype == HODU_BF16 ? launch(attention_fwd_kernel<mfma::CK_BF16, 128, NoMask>, AtGeom<128>::LDS, "attention_fwd_bf16")
+                                : launch(attention_fwd_kernel<mfma::CK_F16, 128, NoMask>, AtGeom<128>::LDS, "attention_fwd_f16");
     else
-        rc = dtype == HODU_BF16 ? launch(attention_fwd_kernel<mfma::CK_BF16, 64>, AtGeom<64>::LDS, "attention_fwd_bf16_d64")
-                                : launch(attention_fwd_kernel<mfma::CK_F16, 64>, AtGeom<64>::LDS, "attention_fwd_f16_d64");
+        rc = dtype == HODU_BF16 ? launch(attention_fwd_kernel<mfma::CK_BF16, 64, NoMask>, AtGeom<64>::LDS, "attention_fwd_bf16_d64")
+                                : launch(attention_fwd_kernel<mfma::CK_F16, 64, NoMask>, AtGeom<64>::LDS, "attention_fwd_f16_d64");
     if (rc != HODU_ROCM_OK) return rc;
     HODU_HIP(hipGetLastError());
     return HODU_ROCM_OK;

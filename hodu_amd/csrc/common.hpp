@@ -242,9 +242,15 @@ struct AttentionArgs {
     bool causal = false;
 };
 int parse_attention_metadata(const size_t *md, size_t len, AttentionArgs *a);
+// an attn_mask read in place: one byte per element, strides (0 where broadcast) over [batch.., Sq, Sk]
+struct AttentionMask {
+    const void *ptr = nullptr;
+    long bs[16];
+    long row = 0, key = 0, off = 0;
+};
 // HODU_ROCM_UNSUPPORTED without an error text when the fused kernel does not take the call
 int launch_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
-                     const AttentionArgs &a);
+                     const AttentionArgs &a, const AttentionMask *mask = nullptr);
 
 int launch_cast(hodu_rocm_ctx *ctx, int src, int dst, const void *in, void *out, const Strided &s);
 int launch_gather(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const Strided &s);

@@ -113,6 +113,7 @@ def declare_compute(lib: ctypes.CDLL):
     lib.hodu_rocm_softmax.argtypes = [vp, ci, vp, vp, szp, sz, ci]
     lib.hodu_rocm_softmax_masked.argtypes = [vp, ci, vp, vp, szp, sz, ci, vp, ci, szp, sz]
     lib.hodu_rocm_attention.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci]
+    lib.hodu_rocm_attention_masked.argtypes = [vp, ci, vp, vp, vp, vp, szp, sz, vp, ci, vp, ci, szp, sz]
     lib.hodu_rocm_dot_bf16_f8e4m3w_noalloc.argtypes = [vp, vp, vp, vp, szp, sz]
     lib.hodu_rocm_ctx_set_reference_sums.argtypes = [vp, ci]
 
@@ -411,9 +412,11 @@ class Context:
         self._check(self.lib.hodu_rocm_softmax_masked(self.handle, DTYPE_ID[dt], x.ptr, out.ptr, arr, n_md, int(bool(causal)),
                                                       mask.ptr, DTYPE_ID[mask_dt], larr, n_l))
 
-    def attention(self, dt: str, q: DeviceBuffer, k: DeviceBuffer, v: DeviceBuffer, out: DeviceBuffer, md, scale, causal=False):
+    def attention(self, dt: str, q: DeviceBuffer, k: DeviceBuffer, v: DeviceBuffer, out: DeviceBuffer, md, scale, causal=False,
+                  mask: DeviceBuffer = None, mask_strides=None, mask_offset: int = 0, mask_dt: str = "u8"):
         """hodu_rocm_attention; md = [nb, batch_shape.., Sq, Sk, D, q_strides.., k_strides.., v_strides.., q_off, k_off,
-        v_off]; scale: 1-element array in dt's storage"""
+        v_off]; scale: 1-element array in dt's storage.  With mask (one byte per element, 0 = masked; mask_strides in
+        elements over [batch_shape.., Sq, Sk], 0 where the mask is broadcast): hodu_rocm_attention_masked"""
         m = [int(x) for x in md]
         nb = m[0] if m else 0
         if len(m) == 1 + nb + 3 + 3 * (nb + 2) + 3:
@@ -429,6 +432,16 @@ class Context:
                 raise HoduRocmError(INVALID_ARG, "attention: the output buffer is too small")
         arr, n = _md_array(md)
         sc = np.ascontiguousarray(scale).reshape(1)
+        if mask is not None:
+            strides = [int(x) for x in mask_strides]
+            if len(m) != 1 + nb + 3 + 3 * (nb + 2) + 3 or len(strides) != nb + 2:
+                raise HoduRocmError(INVALID_ARG, "attention: the mask layout needs one stride per dim of the scores")
+            if _view_span(m[1:1 + nb] + [m[1 + nb], m[2 + nb]], strides, int(mask_offset)) > mask.nbytes:
+                raise HoduRocmError(INVALID_ARG, "attention: the mask layout reaches past the mask buffer")
+            larr, n_l = _md_array([nb + 2] + strides + [int(mask_offset)])
+            self._check(self.lib.hodu_rocm_attention_masked(self.handle, DTYPE_ID[dt], q.ptr, k.ptr, v.ptr, out.ptr, arr, n,
+                                                            sc.ctypes.data, int(bool(causal)), mask.ptr, DTYPE_ID[mask_dt], larr, n_l))
+            return
         self._check(self.lib.hodu_rocm_attention(self.handle, DTYPE_ID[dt], q.ptr, k.ptr, v.ptr, out.ptr, arr, n,
                                                  sc.ctypes.data, int(bool(causal))))
 

@@ -238,9 +238,11 @@ public:
 
     // the whole of scaled_dot_product_attention as one launch, where the fused kernel takes the call (bf16 / f16,
     // head dim 64 or 128, dense aligned rows): *taken says whether it did.  md: hodu_rocm_attention's metadata.
+    // mask, mask_layout: the attn_mask (attention.rs:50-56) read in place, its layout already broadcast to the scores'
+    // shape [batch.., Sq, Sk] (stride 0 where it repeats); one byte per element, 0 = masked out.
     RocmStorage call_ops_attention(const RocmStorage &k, const RocmStorage &v, const Layout &ql, const Layout &kl, const Layout &vl,
                                    const Metadata &md, size_t out_elems, const unsigned char scale[8], bool causal,
-                                   bool *taken) const {
+                                   bool *taken, const RocmStorage *mask = nullptr, const Layout *mask_layout = nullptr) const {
         check_span(ql, "attention q");
         k.check_span(kl, "attention k");
         v.check_span(vl, "attention v");
@@ -249,8 +251,18 @@ public:
         if (deferred() || k.deferred() || v.deferred() || k.dtype_ != dtype_ || v.dtype_ != dtype_ ||
             k.dev_->id() != dev_->id() || v.dev_->id() != dev_->id() || out_elems == 0)
             return out;
-        const int rc = hodu_rocm_attention(dev_->ctx(), (int)dtype_, ptr(), k.ptr(), v.ptr(), (void *)out.ptr(), md.data(),
-                                           md.size(), scale, causal ? 1 : 0);
+        int rc;
+        if (mask) {
+            mask->check_span(*mask_layout, "attention mask");
+            if (mask->deferred() || dtype_size(mask->dtype()) != 1 || mask->dev_->id() != dev_->id()) return out;
+            Metadata ml{mask_layout->ndim()};
+            ml.insert(ml.end(), mask_layout->strides().begin(), mask_layout->strides().end());
+            ml.push_back(mask_layout->offset());
+            rc = hodu_rocm_attention_masked(dev_->ctx(), (int)dtype_, ptr(), k.ptr(), v.ptr(), (void *)out.ptr(), md.data(), md.size(),
+                                            scale, causal ? 1 : 0, mask->ptr(), (int)mask->dtype(), ml.data(), ml.size());
+        } else
+            rc = hodu_rocm_attention(dev_->ctx(), (int)dtype_, ptr(), k.ptr(), v.ptr(), (void *)out.ptr(), md.data(),
+                                     md.size(), scale, causal ? 1 : 0);
         if (rc == HODU_ROCM_UNSUPPORTED) return out;
         dev_->check(rc, "attention");
         stats().attention_kernels++;

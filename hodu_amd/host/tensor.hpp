@@ -253,23 +253,18 @@ public:
     }
 
     // scaled_dot_product_attention (hodu_nn/src/modules/attention.rs:25-70) without dropout:
-    // softmax(Q K^T / sqrt(d_k) [+ causal mask]) V.  One launch where the fused kernel applies (bf16 / f16, head dim
-    // 64 or 128, dense aligned rows); otherwise three -- the scale rides in the first product's store, the mask and the
-    // five softmax kernels are one kernel, the second product is plain.
+    // softmax(Q K^T / sqrt(d_k) [+ causal mask] [+ attn_mask]) V.  One launch where the fused kernel applies (bf16 / f16,
+    // head dim 64 or 128, dense aligned rows); otherwise three -- the scale rides in the first product's store, the masks
+    // and the five softmax kernels are one kernel, the second product is plain.
     static Tensor scaled_dot_product_attention(const Tensor &q, const Tensor &k, const Tensor &v, bool is_causal,
                                                const Tensor *attn_mask = nullptr) {
         if (q.layout().ndim() < 2) throw Error(ErrorKind::InvalidArgument, "attention: query needs at least two dimensions");
         const double scale = 1.0 / std::sqrt((double)q.shape().back());
         unsigned char bits[8];
         const size_t n = scalar_bits(q.dtype(), scale, bits);
-        if (attn_mask) {
-            // with an attn_mask (1 = attend, 0 = mask out; attention.rs:50-56) the function is three launches: the one
-            // kernel has no mask operand.  The mask is read in place by the softmax, broadcast over batch and heads.
-            const Tensor scores = q.matmul_then(k.transpose(-2, -1), {Then::mul_scalar(bits, n)});
-            return scores.softmax_masked(*attn_mask, is_causal).matmul(v);
-        }
         // one kernel where it applies: q [.., Sq, D], k and v [.., Sk, D] with the batch dims broadcast the way the
-        // two matmuls would broadcast them
+        // two matmuls would broadcast them; an attn_mask (1 = attend, 0 = mask out; attention.rs:50-56) is read in
+        // place, broadcast against the scores the way masked_fill's where3 broadcasts it
         const size_t qn = q.layout().ndim(), kn = k.layout().ndim(), vn = v.layout().ndim();
         if (kn >= 2 && vn >= 2 && q.shape()[qn - 1] == k.shape()[kn - 1] && k.shape()[kn - 2] == v.shape()[vn - 2] &&
             v.shape()[vn - 1] == q.shape()[qn - 1]) {
@@ -305,13 +300,29 @@ public:
                 Dims out_shape = batch;
                 out_shape.push_back(q.shape()[qn - 2]);
                 out_shape.push_back(q.shape()[qn - 1]);
-                bool taken = false;
-                auto out = std::make_shared<RocmStorage>(q.storage_->call_ops_attention(*k.storage_, *v.storage_, ql, kl, vl, md,
-                                                                                        product(out_shape), bits, is_causal, &taken));
-                if (taken) return Tensor(out, Layout::from_shape(out_shape));
+                bool taken = false, mask_fits = true;
+                Layout ml;
+                if (attn_mask) {
+                    Dims scores_shape = batch;
+                    scores_shape.push_back(q.shape()[qn - 2]);
+                    scores_shape.push_back(k.shape()[kn - 2]);
+                    try {
+                        ml = attn_mask->layout().broadcast_to(scores_shape);
+                    } catch (const Error &) {
+                        mask_fits = false;  // the three launches below report it
+                    }
+                }
+                if (mask_fits) {
+                    auto out = std::make_shared<RocmStorage>(q.storage_->call_ops_attention(
+                        *k.storage_, *v.storage_, ql, kl, vl, md, product(out_shape), bits, is_causal, &taken,
+                        attn_mask ? attn_mask->storage_.get() : nullptr, attn_mask ? &ml : nullptr));
+                    if (taken) return Tensor(out, Layout::from_shape(out_shape));
+                }
             }
         }
+        // three launches: the scale rides in the first product's store, the masks and the softmax are one kernel
         const Tensor scores = q.matmul_then(k.transpose(-2, -1), {Then::mul_scalar(bits, n)});
+        if (attn_mask) return scores.softmax_masked(*attn_mask, is_causal).matmul(v);
         return scores.softmax(-1, is_causal).matmul(v);
     }
 

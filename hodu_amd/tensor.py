@@ -295,8 +295,9 @@ def scalar_bits(dtype: str, value: float) -> np.ndarray:
 def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False,
                                  attn_mask: Optional[Tensor] = None) -> Tensor:
     """hodu_nn's scaled_dot_product_attention (crates/hodu_nn/src/modules/attention.rs:25-70) without dropout: one launch
-    where the fused kernel applies (bf16 / f16, head dim 64 or 128, no attn_mask), otherwise three (product with the
-    scale in its store, masked softmax, product).  attn_mask: 1 = attend, 0 = mask out, broadcast against the scores."""
+    where the fused kernel applies (bf16 / f16, head dim 64 or 128, dense aligned rows; with or without attn_mask),
+    otherwise three (product with the scale in its store, masked softmax, product).  attn_mask: a bool / u8 / i8 tensor,
+    1 = attend, 0 = mask out, broadcast against the scores and read in place."""
     out = ctypes.c_void_p()
     if attn_mask is not None:
         rc = load().hodu_host_attention_masked(q._h, k._h, v._h, attn_mask._h, int(is_causal), ctypes.byref(out))

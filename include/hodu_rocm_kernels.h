@@ -266,6 +266,19 @@ int hodu_rocm_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void
 int hodu_rocm_attention(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
                         const size_t *metadata, size_t metadata_len, const void *scale, int causal);
 
+/* The same with scaled_dot_product_attention's attn_mask (crates/hodu_nn/src/modules/attention.rs:50-56:
+ * masked_fill(mask.eq_scalar(0), get_neg_inf(dtype)) over the scaled scores) as part of the one kernel.  mask, mask_dtype:
+ * as for hodu_rocm_softmax_masked; mask_layout (host): [nd, strides (nd).., offset] in elements over the SCORES' shape
+ * [batch.., Sq, Sk] (nd = nb + 2), stride 0 where the mask is broadcast -- read in place, never expanded.  A masked
+ * score counts as what the reference fills it with in a 16-bit type (:88-96: the dtype's rounding of -65504, a finite
+ * value), the causal mask likewise when both are given: a row with an open key gives its masked keys weight exp(fill -
+ * max) = 0, a row masked entirely is the uniform average over all Sk keys, as in the reference.  Same conditions and
+ * the same HODU_ROCM_UNSUPPORTED as hodu_rocm_attention; the caller's other path is hodu_rocm_matmul_<dt>_ex with
+ * MUL_SCALAR, hodu_rocm_softmax_masked, hodu_rocm_matmul_<dt>. */
+int hodu_rocm_attention_masked(hodu_rocm_ctx *ctx, int dtype, const void *q, const void *k, const void *v, void *out,
+                               const size_t *metadata, size_t metadata_len, const void *scale, int causal,
+                               const void *mask, int mask_dtype, const size_t *mask_layout, size_t mask_layout_len);
+
 #ifdef __cplusplus
 }
 #endif

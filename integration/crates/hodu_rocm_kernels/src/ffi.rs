@@ -58,9 +58,18 @@ extern "C" {
     pub fn hodu_rocm_softmax(ctx: *mut hodu_rocm_ctx, dtype: c_int, input: *const c_void, out: *mut c_void,
                              metadata: *const usize, metadata_len: usize, causal: c_int) -> c_int;
 
+    // attn_mask (attention.rs:50-56) folded in: one byte per element, 0 = masked out, read through its own strides
+    pub fn hodu_rocm_softmax_masked(ctx: *mut hodu_rocm_ctx, dtype: c_int, input: *const c_void, out: *mut c_void,
+                                    metadata: *const usize, metadata_len: usize, causal: c_int, mask: *const c_void,
+                                    mask_dtype: c_int, mask_layout: *const usize, mask_layout_len: usize) -> c_int;
+
     pub fn hodu_rocm_attention(ctx: *mut hodu_rocm_ctx, dtype: c_int, q: *const c_void, k: *const c_void, v: *const c_void,
                                out: *mut c_void, metadata: *const usize, metadata_len: usize, scale: *const c_void,
                                causal: c_int) -> c_int;
+    pub fn hodu_rocm_attention_masked(ctx: *mut hodu_rocm_ctx, dtype: c_int, q: *const c_void, k: *const c_void,
+                                      v: *const c_void, out: *mut c_void, metadata: *const usize, metadata_len: usize,
+                                      scale: *const c_void, causal: c_int, mask: *const c_void, mask_dtype: c_int,
+                                      mask_layout: *const usize, mask_layout_len: usize) -> c_int;
 
     // deferred casts fused into the product: bf16 x f8e4m3 bytes -> bf16, i8 x i8 -> i32
     pub fn hodu_rocm_matmul_bf16_f8e4m3w(ctx: *mut hodu_rocm_ctx, lhs: *const c_void, rhs: *const c_void, out: *mut c_void,

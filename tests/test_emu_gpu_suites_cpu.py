@@ -32,7 +32,7 @@ pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host cla
 
 SUITES = ["test_gpu_products", "test_gpu_mfma", "test_gpu_exact", "test_gpu_epilogue", "test_gpu_skinny", "test_gpu_small_f32",
           "test_gpu_f64", "test_gpu_casts", "test_gpu_sum", "test_gpu_softmax", "test_gpu_attention", "test_zz_no_alloc",
-          "test_zx_softmax_masked", "test_zy_reference_sums",
+          "test_zx_softmax_masked", "test_zx_attention_masked", "test_zy_reference_sums",
           "test_gpu_configs",  # BASELINE's five configurations at their full sizes
           # the GPU test of kernels that have not run on a GPU, kept under a name pytest does not collect: it runs here
           "wip_pipe16r"]
