@@ -37,12 +37,12 @@ MFMA_RESULT_WAIT_STATES = 18
 
 
 SOURCES = {"tile16": os.path.join(CSRC, "gemm_mfma_mi16_bf16.hip"), "f8_tiles": os.path.join(CSRC, "gemm_mfma_f8.hip"),
-           "tile16_f8w": os.path.join(ROOT, "tests", "isa", "mi16_f8w_kernels.hip")}
+           "tile16_f8w": os.path.join(ROOT, "tests", "isa", "mi16_f8w_kernels.hip"), "attention": os.path.join(CSRC, "attention.hip")}
 
 
 @pytest.fixture(scope="module")
 def assembly(tmp_path_factory):
-    """{name: lines of the gfx950 assembly of SOURCES[name]}, the three compiled side by side"""
+    """{name: lines of the gfx950 assembly of SOURCES[name]}, compiled side by side"""
     out_dir = tmp_path_factory.mktemp("isa")
 
     def one(item):
@@ -52,7 +52,7 @@ def assembly(tmp_path_factory):
         r = subprocess.run(cmd, capture_output=True, text=True)
         assert r.returncode == 0, r.stderr[-2000:]
         return name, out.read_text().split("\n")
-    with ThreadPoolExecutor(max_workers=3) as pool:
+    with ThreadPoolExecutor(max_workers=4) as pool:
         return dict(pool.map(one, SOURCES.items()))
 
 
@@ -145,11 +145,15 @@ def test_accumulators_are_read_only_after_the_wait_states(tile16, f8_tiles, tile
     # f8e4m3 weights k-dense and row-dense, both forms
 
 
-def test_an_instruction_separates_every_m0_write_from_the_load_that_uses_it(tile16, f8_tiles, tile16_f8w):
-    for lines, part in ((tile16, "mfma_pipe16"), (f8_tiles, "mfma_pipe_f8"), (tile16_f8w, "mfma_pipe16")):
+def test_an_instruction_separates_every_m0_write_from_the_load_that_uses_it(tile16, f8_tiles, tile16_f8w, assembly):
+    checked = 0
+    for lines, part in ((tile16, "mfma_pipe16"), (f8_tiles, "mfma_pipe_f8"), (tile16_f8w, "mfma_pipe16"),
+                        (assembly["attention"], "attention_fwd_kernel")):
         for name, insns in kernels_in(lines, part).items():
             assert any(s.startswith("global_load_lds") for s in insns), name
             assert loads_too_close_to_an_m0_write(insns) == [], name
+            checked += 1
+    assert checked >= 12 + 4 + 4 + 8  # .. and the attention kernel: two types x two head dims, with and without a mask
 
 
 def test_respaced_kernels_m0_bookkeeping(tile16):
