@@ -373,14 +373,15 @@ def compact_row(r):
     return row
 
 
-def attention_probe(ctx, steps, d=128):
+def attention_probe(ctx, steps, d=128, heads=32, s_len=2048):
     """not a BASELINE configuration: hodu_nn's scaled_dot_product_attention (causal, bf16, 32 heads x 2048 x d) as
     the one fused kernel, and as the three launches the host mirror falls back to -- Q K^T with the scale in its
-    store, masked softmax, P V -- each timed with HIP events around `steps` back-to-back launches"""
+    store, masked softmax, P V -- each timed with HIP events around `steps` back-to-back launches; and, beside them,
+    the same function with a [1, Sk] padding attn_mask (a quarter of the keys masked, no causal mask) as one kernel and
+    its middle launch of the three"""
     import helpers as H
     from hodu_amd import ffi
     V = H.View
-    heads, s_len = 32, 2048
     q, k, v = (ctx.upload(bf16(normal(950 + i, heads * s_len * d))) for i in range(3))
     scores, probs = ctx.alloc(heads * s_len * s_len * 2), ctx.alloc(heads * s_len * s_len * 2)
     out = ctx.alloc(heads * s_len * d * 2)
@@ -396,6 +397,12 @@ def attention_probe(ctx, steps, d=128):
     md_at = [1, heads, s_len, s_len, d] + [s_len * d, d, 1] * 3 + [0, 0, 0]
     scale_bits = bf16(np.array([1.0 / np.sqrt(d)], dtype=np.float32))
     legs["fused_one_kernel"] = lambda: ctx.attention("bf16", q, k, v, out, md_at, scale_bits, True)
+    keep = np.ones(s_len, np.uint8)
+    keep[s_len - s_len // 4:] = 0
+    mask = ctx.upload(keep)
+    legs["softmax_padding_mask"] = lambda: ctx.softmax_masked("bf16", scores, probs, md_sm, mask, [0, 0, 1])
+    legs["fused_padding_mask"] = lambda: ctx.attention("bf16", q, k, v, out, md_at, scale_bits, False, mask=mask, mask_strides=[0, 0, 1])
+    beside = ("fused_one_kernel", "softmax_padding_mask", "fused_padding_mask")  # not part of the three-launch total
     res, total = {}, 0.0
     for name, fn in legs.items():
         for _ in range(3):
@@ -407,17 +414,17 @@ def attention_probe(ctx, steps, d=128):
             fn()
         us = t.stop_ms() * 1e3 / steps
         res[name] = {"us": us, "kernel": ctx.last_kernel()}
-        total += us if name != "fused_one_kernel" else 0.0
+        total += us if name not in beside else 0.0
     flops = 2 * 2.0 * heads * s_len * s_len * d
     res["qk_scaled"]["tflops"] = flops / 2 / res["qk_scaled"]["us"] / 1e6
     res["pv"]["tflops"] = flops / 2 / res["pv"]["us"] / 1e6
     res["softmax_causal"]["gbs"] = 2.0 * heads * s_len * s_len * 2 / res["softmax_causal"]["us"] / 1e3
-    for b in (q, k, v, scores, probs, out):
+    for b in (q, k, v, scores, probs, out, mask):
         b.free()
     # the causal mask halves the useful work; rates count the unmasked half only for the fused kernel
     res["fused_one_kernel"]["tflops_useful"] = flops / 2 / res["fused_one_kernel"]["us"] / 1e6
     return {"config": "attention", "shape": f"bf16 q,k,v [{heads},{s_len},{d}], causal", "us_three_launches": total,
-            "us_fused": res["fused_one_kernel"]["us"], "legs": res}
+            "us_fused": res["fused_one_kernel"]["us"], "us_fused_padding_mask": res["fused_padding_mask"]["us"], "legs": res}
 
 
 def cast_cases():

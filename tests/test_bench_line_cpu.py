@@ -96,3 +96,20 @@ def test_timed_cases_and_the_line_against_the_cpu_build():
     assert len(text) < bench.LINE_LIMIT
     per_config = json.loads(text)["roofline"]["per_config"]
     assert [(row[0], row[2], row[6]) for row in per_config] == [("c1", "mfma", "small_f32_KM"), ("c3_m1", "hbm", "gemv_bf16_f8w_walk")]
+
+
+def test_attention_probe_against_the_cpu_build():
+    """`bench.py --only attention`'s routine at a reduced size against the CPU build: every leg launches the kernel it
+    names (the times are the emulation's and mean nothing)"""
+    import emu_util
+    if emu_util.compiler() is None:
+        pytest.skip("no host clang++ for the CPU build")
+    ctx = emu_util.EmuContext()
+    try:
+        res = bench.attention_probe(ctx, 1, 64, heads=2, s_len=128)
+    finally:
+        ctx.close()
+    kernels = {name: leg["kernel"] for name, leg in res["legs"].items()}
+    assert kernels["fused_one_kernel"] == "attention_fwd_bf16_d64" and kernels["fused_padding_mask"] == "attention_masked_fwd_bf16_d64"
+    assert kernels["softmax_causal"].startswith("softmax_") and kernels["softmax_padding_mask"] == "softmax_masked"
+    assert res["us_three_launches"] == pytest.approx(sum(res["legs"][n]["us"] for n in ("qk_scaled", "softmax_causal", "pv")))
