@@ -287,12 +287,14 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
 #pragma unroll
         for (int e = 0; e < 16; e++) sc[e] = 0.f;
     };
-    auto mask = [&](acc_t &sc, int kb) {
-        const int key0 = kb * AT_BK + kh * 32;
+    // the attn_mask bytes of the lane's 16 keys of block kb (a row past Sq reads the last row's, a key past Sk the last
+    // key's); fetched one block ahead, so that the loads are in flight during a whole iteration
+    struct NoBytes {};
+    typedef typename std::conditional<MASKED, uint8_t[16], NoBytes>::type mask_bytes_t;
+    auto load_mask = [&](int kb, mask_bytes_t &open) {
         if constexpr (MASKED) {
-            // the row's mask bytes of the lane's 16 keys (a row past Sq reads the last row's, a key past Sk the last key's)
+            const int key0 = kb * AT_BK + kh * 32;
             const uint8_t *mrow = mk.ptr + mo + (long)q_row * mk.row;
-            uint8_t open[16];
 #pragma unroll
             for (int q = 0; q < 4; q++)
 #pragma unroll
@@ -300,6 +302,11 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
                     const int key = key0 + 8 * q + 4 * lh + e;
                     open[4 * q + e] = mrow[(long)(key < a.sk ? key : a.sk - 1) * mk.key];
                 }
+        }
+    };
+    auto mask = [&](acc_t &sc, int kb, const mask_bytes_t &open) {
+        const int key0 = kb * AT_BK + kh * 32;
+        if constexpr (MASKED) {
 #pragma unroll
             for (int q = 0; q < 4; q++)
 #pragma unroll
@@ -443,8 +450,11 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
             fast_block(kb + 1, 1, s_odd, s_cur);
         }
     }
+    mask_bytes_t open_cur, open_next;
+    load_mask(kb, open_cur);  // (kb = 0 here with a mask: its blocks all take this loop; block 0 exists)
     for (; kb < n_blocks; kb++) {
         next_loads(kb);
+        if (kb + 1 < n_blocks) load_mask(kb + 1, open_next);
         acc_t s_next;
         zero(s_next);
         if (!idle_in(kb + 1)) {
@@ -456,7 +466,7 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
             u32x2_t vf0[AT_D / 32][2], vf1[AT_D / 32][2];
             read_v(vf0, kb & 1, 0);
             read_v(vf1, kb & 1, 1);
-            mask(s_cur, kb);
+            mask(s_cur, kb, open_cur);
             if (row_max(s_cur)) rescale_o();
             float l_blk = 0.f;
             const u32x4_t pf0 = probs(s_cur, 0, l_blk);
@@ -466,6 +476,10 @@ __global__ __launch_bounds__(AT_NT, 1) void attention_fwd_kernel(const uint16_t 
             finish_row_sum(l_blk);
         }
         s_cur = s_next;
+        if constexpr (MASKED) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) open_cur[i] = open_next[i];
+        }
         publish();
     }
 
