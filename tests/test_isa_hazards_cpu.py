@@ -37,7 +37,8 @@ MFMA_RESULT_WAIT_STATES = 18
 
 
 SOURCES = {"tile16": os.path.join(CSRC, "gemm_mfma_mi16_bf16.hip"), "f8_tiles": os.path.join(CSRC, "gemm_mfma_f8.hip"),
-           "tile16_f8w": os.path.join(ROOT, "tests", "isa", "mi16_f8w_kernels.hip"), "attention": os.path.join(CSRC, "attention.hip")}
+           "tile16_f8w": os.path.join(ROOT, "tests", "isa", "mi16_f8w_kernels.hip"), "attention": os.path.join(CSRC, "attention.hip"),
+           "builtin_offsets": os.path.join(ROOT, "tests", "isa", "lds_dma_builtin_offsets.hip")}
 
 
 @pytest.fixture(scope="module")
@@ -52,7 +53,7 @@ def assembly(tmp_path_factory):
         r = subprocess.run(cmd, capture_output=True, text=True)
         assert r.returncode == 0, r.stderr[-2000:]
         return name, out.read_text().split("\n")
-    with ThreadPoolExecutor(max_workers=4) as pool:
+    with ThreadPoolExecutor(max_workers=5) as pool:
         return dict(pool.map(one, SOURCES.items()))
 
 
@@ -196,3 +197,17 @@ def test_tile_kernels_keep_their_accumulators_in_registers(assembly):
             assert int(size) == 0, (name, size)
             seen += 1
     assert seen >= 18
+
+
+def test_the_compiler_reads_the_dma_immediate_as_the_respaced_kernels_do(assembly):
+    """The respaced kernels rest on one reading of the ISA document: the immediate offset of global_load_lds_dwordx4
+    moves the LDS address as well as the global one.  The compiler's builtin for the same instruction documents its
+    offset argument as applied to both addresses, and lowers two loads from one global base to one LDS base at offsets
+    of 1 and 2 KB to ONE M0 write and two instructions that differ in their immediate only -- the same reading (were
+    the LDS address M0's alone, both loads would land on the same 1 KB)."""
+    insns = [line.split(";")[0].strip() for line in assembly["builtin_offsets"]]
+    m0_writes = [s for s in insns if re.match(r"s_\w+ m0,", s)]
+    loads = [s for s in insns if s.startswith("global_load_lds_dwordx4")]
+    assert len(m0_writes) == 1 and len(loads) == 2, (m0_writes, loads)
+    operands = [re.match(r"global_load_lds_dwordx4 (\S+ \S+) offset:(\d+)$", s).groups() for s in loads]
+    assert operands[0][0] == operands[1][0] and [int(o[1]) for o in operands] == [1024, 2048], loads
