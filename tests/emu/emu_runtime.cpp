@@ -86,7 +86,7 @@ NOT_IN_THIS_LIBRARY(launch_small_f32)
 NOT_IN_THIS_LIBRARY(launch_gemm_f64)
 NOT_IN_THIS_LIBRARY(launch_skinny)
 NOT_IN_THIS_LIBRARY(launch_gemv_rows)
-int launch_attention(hodu_rocm_ctx *, int, const void *, const void *, const void *, void *, const AttentionArgs &) {
+int launch_attention(hodu_rocm_ctx *, int, const void *, const void *, const void *, void *, const AttentionArgs &, const AttentionMask *) {
     return HODU_ROCM_UNSUPPORTED;
 }
 }  // namespace hodu

@@ -13,7 +13,8 @@ what the result-comparing tests cannot do: they only see the interleavings the h
  * the same program's hand-offs with the barrier left out, or the wait placed behind the barrier, must be reported:
    the detector has teeth;
  * opt-in (HODU_EMU_ALL=1): every pytest file that drives the CPU build, run by a Python that carries the sanitizer
-   (tests/emu/python_host.cpp), i.e. every kernel family the GPU tests cover.
+   (tests/emu/python_host.cpp), i.e. every kernel family the GPU tests cover, at the case set those files run by
+   default (ten minutes); HODU_EMU_ALL=2: at their own HODU_EMU_ALL=1 set (more than an hour).
 """
 import glob
 import os
@@ -64,13 +65,14 @@ SUITES = ["test_emu_mfma_cpu.py", "test_emu_kernel_families_cpu.py", "test_emu_p
           "test_emu_reference_sums_cpu.py", "test_emu_gpu_suites_cpu.py", "test_emu_host_mirror_cpu.py"]
 
 
-@pytest.mark.skipif(os.environ.get("HODU_EMU_ALL", "") in ("", "0"), reason="about half an hour; set HODU_EMU_ALL=1")
+@pytest.mark.skipif(os.environ.get("HODU_EMU_ALL", "") in ("", "0"), reason="ten minutes; set HODU_EMU_ALL=1")
 def test_every_kernel_family_under_the_race_detector(tmp_path):
     python = emu_util.build_race_checked_python()
     if python is None:
         pytest.skip("no Python headers or library to link the sanitizer-carrying interpreter")
     log = str(tmp_path / "report")
-    env = dict(TSAN_OPTIONS=OPTIONS + f" exitcode=0 log_path={log}", HODU_EMU_SANITIZE="thread", PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    env = dict(TSAN_OPTIONS=OPTIONS + f" exitcode=0 log_path={log}", HODU_EMU_SANITIZE="thread", PYTHONPATH=os.pathsep.join(p for p in sys.path if p),
+               HODU_EMU_ALL="1" if os.environ.get("HODU_EMU_ALL") == "2" else "0")
     pytest_args = ["-q", "-x", "-p", "no:cacheprovider"]
     # the test that runs kernels under a deliberately wrong arrival model must be reported: the detector sees the kernels
     r = run([python, "-m", "pytest", os.path.join("tests", "test_emu_mfma_cpu.py"), *pytest_args, "-k", "one_load_too_late"], **env)
