@@ -1,0 +1,162 @@
+"""Randomly drawn layouts through the C ABI of the CPU build, against the oracle.
+
+The hand-picked layouts of the GPU test files name the cases somebody thought of.  Here shapes, storage orders,
+slices with steps, offsets, size-1 and stride-0 broadcasts are drawn at random (seeded: the same cases every run), so
+that the host's classification of an operand (dense along k, dense along rows, element-wise; aligned or not), the
+choice of kernel family, ragged edges and batch decomposition meet combinations nobody listed -- with every operand
+allocated tight against an inaccessible page at its end or, every other case, at its start, so a kernel variant that
+reads one element outside what its layout addresses faults instead of passing.  The comparison is the GPU tests' own
+(tests/gpu_util.py, test_gpu_sum.py, test_gpu_softmax.py, test_gpu_casts.py): bit for bit for integers and casts,
+the stated tolerances for floats."""
+import os
+
+import numpy as np
+import pytest
+
+import emu_util
+import helpers as H
+import oracle
+from gpu_util import FUSED, check_product
+from hodu_amd import ffi
+
+pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host clang++ for the CPU build")
+V = H.View
+MORE = int(os.environ.get("HODU_EMU_ALL", "0") or 0) > 0
+ROUNDS = 40 if MORE else 8  # multiplies the cases per dtype and family
+
+
+@pytest.fixture(scope="module")
+def contexts():
+    made = {"end": emu_util.EmuContext(tight="end"), "start": emu_util.EmuContext(tight="start")}
+    yield made
+    for c in made.values():
+        c.close()
+
+
+def random_view(g, shape, may_broadcast=(), tame=False):
+    """a view of logical `shape` over some storage: dims stored in a random order, each possibly a slice (with a step)
+    of a longer storage dim, a random offset; dims listed in may_broadcast may get stride 0.  tame: the innermost
+    stored dim is dense and every other stride and the offset are multiples of 16 elements, the layouts the
+    vector-loading kernels take"""
+    n = len(shape)
+    order = list(g.permutation(n))                      # storage order, outermost first
+    if tame and n >= 2 and order[-1] < n - 2:           # a matrix dim innermost, batch dims anywhere outside
+        i = order.index(n - 1 if g.random() < 0.5 else n - 2)
+        order[i], order[-1] = order[-1], order[i]
+    step = [int(g.choice([1, 1, 1, 2, 3])) for _ in range(n)]
+    extra = [int(g.choice([0, 0, 16, 32] if tame else [0, 0, 8, 3, 1])) for _ in range(n)]
+    if tame and n:
+        step[order[-1]] = 1
+    stored = [(shape[d] - 1) * step[d] + 1 + extra[d] if shape[d] > 0 else extra[d] + 1 for d in range(n)]
+    if tame and n:
+        stored[order[-1]] = -(-stored[order[-1]] // 16) * 16
+    strides, acc = [0] * n, 1
+    for d in reversed(order):
+        strides[d] = acc * step[d]
+        acc *= stored[d]
+    for d in may_broadcast:
+        if g.random() < 0.35:
+            strides[d] = 0
+    return V(list(shape), strides, int(g.choice([0, 0, 16, 48] if tame else [0, 0, 8, 16, 3, 5])))
+
+
+def dims(g, choices):
+    return int(g.choice(choices))
+
+
+M_CHOICES = [1, 2, 3, 4, 5, 16, 17, 31, 33, 64, 65, 100, 128, 130, 257, 300]
+K_CHOICES = [1, 7, 8, 16, 31, 64, 65, 128, 136, 192, 200, 256, 260, 512]
+
+
+def product_case(g):
+    m, n, k = dims(g, M_CHOICES), dims(g, M_CHOICES), dims(g, K_CHOICES)
+    while m * n * k > 6_000_000:
+        m = max(1, m // 2)
+    tame = g.random() < 0.65
+    if tame and g.random() < 0.75:  # .. and extents in whole vectors, as the vector-loading kernels need them
+        m, n, k = (v if v == 1 and g.random() < 0.5 else -(-v // 16) * 16 for v in (m, n, k))
+    if g.random() < 0.5:
+        return "dot", random_view(g, [m, k], tame=tame), random_view(g, [k, n], tame=tame)
+    nb = int(g.integers(0, 3))
+    batch = [int(g.integers(1, 4)) for _ in range(nb)]
+    while int(np.prod(batch + [m, n, k], dtype=np.int64)) > 6_000_000 and batch:
+        batch.pop()
+    # either side may lack leading batch dims or hold extent 1 where the other has more (broadcast by shape), or hold
+    # the full extent with stride 0 (broadcast by stride)
+    def side(rows, cols):
+        keep = int(g.integers(0, len(batch) + 1))
+        shape = [b if g.random() < 0.7 else 1 for b in batch[len(batch) - keep:]] + [rows, cols]
+        return random_view(g, shape, may_broadcast=range(len(shape) - 2), tame=tame)
+    return "matmul", side(m, k), side(k, n)
+
+
+@pytest.mark.parametrize("dt", ffi.PRODUCT_DTYPES + list(FUSED))
+def test_products_over_random_layouts(contexts, dt):
+    g = np.random.default_rng(1000 + sum(map(ord, dt)))
+    scale = 2.0 if dt.startswith("f8") else 1.0
+    for n in range(3 * ROUNDS):
+        op, lv, rv = product_case(g)
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        try:
+            check_product(ctx, op, dt, lv, rv, seed=n, scale=scale)
+        except AssertionError as e:
+            raise AssertionError(f"{op} {dt} case {n}: lhs {lv.shape} {lv.strides} +{lv.offset}, rhs {rv.shape} {rv.strides} +{rv.offset}, "
+                                 f"kernel {ctx.last_kernel()}: {e}") from None
+
+
+def test_casts_and_gathers_over_random_layouts(contexts):
+    from test_gpu_casts import gpu_cast, in_domain, same
+    g = np.random.default_rng(2024)
+    names = list(oracle.DTYPE_ID)
+    for n in range(20 * ROUNDS):
+        nd = int(g.integers(1, 5))
+        shape = [dims(g, [1, 2, 3, 5, 8, 17, 33, 64, 70]) for _ in range(nd)]
+        while int(np.prod(shape, dtype=np.int64)) > 200_000:
+            shape[int(np.argmax(shape))] //= 2
+        v = random_view(g, shape, may_broadcast=range(nd))
+        md = H.cast_md(v)
+        src, dst = names[int(g.integers(len(names)))], names[int(g.integers(len(names)))]
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        x = in_domain(src, dst, H.random_storage(src, max(v.span(), 1), 77 + n, 3.0))
+        want = oracle.cast(src, dst, x, md, decode=oracle.F8_OCP)
+        assert same(gpu_cast(ctx, src, dst, x, md), want, dst), (n, src, dst, v.shape, v.strides, v.offset, ctx.last_kernel())
+        want = oracle.contiguous(src, x, md)
+        assert same(gpu_cast(ctx, "contiguous", src, x, md), want, src), (n, src, v.shape, v.strides, v.offset, ctx.last_kernel())
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f32", "f64", "i32", "u8", "f8e4m3"])
+def test_sums_over_random_layouts(contexts, dt):
+    from test_gpu_sum import check_sum
+    g = np.random.default_rng(3000 + sum(map(ord, dt)))
+    for n in range(4 * ROUNDS):
+        nd = int(g.integers(1, 5))
+        shape = [dims(g, [1, 2, 3, 5, 8, 17, 33, 64, 130]) for _ in range(nd)]
+        while int(np.prod(shape, dtype=np.int64)) > 150_000:
+            shape[int(np.argmax(shape))] //= 2
+        v = random_view(g, shape, may_broadcast=range(nd))
+        reduced = sorted(int(d) for d in g.choice(nd, size=int(g.integers(1, nd + 1)), replace=False))
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        try:
+            check_sum(ctx, dt, v, reduced, bool(g.integers(2)), seed=n)
+        except AssertionError as e:
+            raise AssertionError(f"sum {dt} case {n}: {v.shape} {v.strides} +{v.offset} over {reduced}, kernel {ctx.last_kernel()}: {e}") from None
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64"])
+def test_softmax_over_random_layouts(contexts, dt):
+    from test_gpu_softmax import check_softmax
+    g = np.random.default_rng(4000 + sum(map(ord, dt)))
+    for n in range(4 * ROUNDS):
+        nd = int(g.integers(1, 5))
+        shape = [dims(g, [1, 2, 3, 5, 8, 17, 33, 64, 130, 700]) for _ in range(nd)]
+        while int(np.prod(shape, dtype=np.int64)) > 100_000:
+            shape[int(np.argmax(shape))] //= 2
+        v = random_view(g, shape)
+        dim = int(g.integers(nd))
+        causal = dim == nd - 1 and nd >= 2 and bool(g.integers(2))
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        try:
+            check_softmax(ctx, dt, v, dim, causal, seed=n)
+        except AssertionError as e:
+            raise AssertionError(f"softmax {dt} case {n}: {v.shape} {v.strides} +{v.offset} dim {dim} causal {causal}, "
+                                 f"kernel {ctx.last_kernel()}: {e}") from None
