@@ -14,7 +14,8 @@
 //     [features]): one thread per output vector would leave most of the chip idle, so the reduced index space is cut
 //     into chunks, one workgroup per (64 output vectors, chunk), its four wavefronts taking every fourth row; the
 //     chunks' partial sums (in the accumulate type) go through the context's workspace and a second kernel adds
-//     them in chunk order and rounds once;
+//     them in chunk order and rounds once.  Few outputs with a long reduction take this form whatever their layout (a
+//     strided tensor summed to a scalar): uncoalesced reads across a whole chip beat one lane walking the tensor alone;
 //   * the innermost reduced dim is dense (a row sum): a wavefront owns an output, its lanes stride over that dim
 //     (16 bytes per lane when alignment allows), and the lane sums meet in a butterfly; few long rows (sum_all of a
 //     large tensor is one) are cut into chunks across workgroups in the same two-kernel way.
@@ -364,7 +365,8 @@ template <class E> int run(hodu_rocm_ctx *ctx, const void *in, void *out, const 
     const long threads = vec ? r.n_out / V : r.n_out;
     // few outputs and a long reduction: cut the reduced index space into chunks (see the top of the file)
     const long cus = ctx->props.multiProcessorCount;
-    if (out_dense && threads < cus * 256 && r.reduce_size >= 64) {
+    // (whatever the outputs' layout: a lane per output walking a long reduction alone is the slowest choice there is)
+    if (threads < cus * 256 && r.reduce_size >= 64) {
         typedef typename E::acc A;
         const long xblocks = (threads + 63) / 64;
         long chunks = (4 * cus + xblocks - 1) / xblocks;           // about four workgroups per CU
