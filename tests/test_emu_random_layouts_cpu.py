@@ -33,14 +33,17 @@ def contexts():
         c.close()
 
 
-def random_view(g, shape, may_broadcast=(), tame=False):
+def random_view(g, shape, may_broadcast=(), tame=False, inner=None):
     """a view of logical `shape` over some storage: dims stored in a random order, each possibly a slice (with a step)
     of a longer storage dim, a random offset; dims listed in may_broadcast may get stride 0.  tame: the innermost
     stored dim is dense and every other stride and the offset are multiples of 16 elements, the layouts the
-    vector-loading kernels take"""
+    vector-loading kernels take; inner: the dim that is stored innermost"""
     n = len(shape)
     order = list(g.permutation(n))                      # storage order, outermost first
-    if tame and n >= 2 and order[-1] < n - 2:           # a matrix dim innermost, batch dims anywhere outside
+    if inner is not None:                               # this dim innermost
+        i = order.index(inner)
+        order[i], order[-1] = order[-1], order[i]
+    elif tame and n >= 2 and order[-1] < n - 2:         # a matrix dim innermost, batch dims anywhere outside
         i = order.index(n - 1 if g.random() < 0.5 else n - 2)
         order[i], order[-1] = order[-1], order[i]
     step = [int(g.choice([1, 1, 1, 2, 3])) for _ in range(n)]
@@ -160,3 +163,38 @@ def test_softmax_over_random_layouts(contexts, dt):
         except AssertionError as e:
             raise AssertionError(f"softmax {dt} case {n}: {v.shape} {v.strides} +{v.offset} dim {dim} causal {causal}, "
                                  f"kernel {ctx.last_kernel()}: {e}") from None
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_attention_over_random_layouts(contexts, dt):
+    """the one-kernel attention with and without an attn_mask: q, k, v as views with the head dim innermost and
+    everything else in any order (heads interleaved with positions, k and v shared across batch dims by stride 0), the
+    mask as any view that broadcasts against the scores"""
+    from test_gpu_attention import check_attention
+    from test_zx_attention_masked import check as check_masked
+    g = np.random.default_rng(5000 + sum(map(ord, dt)))
+    for n in range(3 * ROUNDS):
+        d = int(g.choice([64, 128]))
+        batch = [int(g.integers(1, 4)) for _ in range(int(g.integers(0, 3)))]
+        sq, sk = dims(g, [1, 2, 31, 33, 64, 100, 128, 130, 200]), dims(g, [1, 5, 32, 63, 64, 65, 127, 129, 200, 300])
+        while int(np.prod(batch, dtype=np.int64)) * sq * sk > 150_000 and batch:
+            batch.pop()
+        nb = len(batch)
+        qv = random_view(g, batch + [sq, d], tame=True, inner=nb + 1)
+        kv = random_view(g, batch + [sk, d], may_broadcast=range(nb), tame=True, inner=nb + 1)
+        vv = random_view(g, batch + [sk, d], may_broadcast=range(nb), tame=True, inner=nb + 1)
+        causal = bool(g.integers(2))
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        what = f"attention {dt} case {n}: batch {batch} {sq}x{sk} d {d} causal {causal}, q {qv.strides} +{qv.offset}, k {kv.strides} +{kv.offset}, v {vv.strides} +{vv.offset}"
+        try:
+            if n % 3 == 0:
+                check_attention(ctx, dt, batch, sq, sk, causal, seed=n, qv=qv, kv=kv, vv=vv, d=d)
+            else:
+                keep = int(g.integers(1, nb + 3))  # trailing dims of the scores the mask has
+                mshape = [e if g.random() < 0.6 else 1 for e in (batch + [sq, sk])[nb + 2 - keep:]]
+                mv = random_view(g, mshape, may_broadcast=range(len(mshape)))
+                what += f", mask {mv.shape} {mv.strides} +{mv.offset}"
+                check_masked(ctx, dt, batch, sq, sk, mv, causal, seed=n, d=d, density=float(g.choice([0.05, 0.5, 0.9])),
+                             close_key0=bool(g.integers(2)), qv=qv, kv=kv, vv=vv)
+        except AssertionError as e:
+            raise AssertionError(f"{what}: {e}") from None
