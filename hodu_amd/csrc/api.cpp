@@ -34,11 +34,15 @@ int dispatch_one(hodu_rocm_ctx *ctx, int kind, int dtype, const void *a, const v
     // A matrix times a vector, [M, K] x [K, 1] (what Tensor::matmul makes of a 2-D and a 1-D tensor,
     // crates/hodu_core/src/tensor/ops/matrix.rs:50-66), is the transposed problem of one row against the matrix as
     // the weight, [1, K] x [K, M], and the [M, 1] output is the same memory as [1, M]: the few-rows kernels take it.
-    if (g.N == 1 && g.M > 1 && g.batches == 1 && kind == PK_SAME && g.epi.n == 0 && ctx->force_tile < 0) {
+    // Fused steps go along: they are element-wise, and a vector added along an output row of one element is that one
+    // element for every output (stride 0 in the transposed problem).
+    if (g.N == 1 && g.M > 1 && g.batches == 1 && kind == PK_SAME && ctx->force_tile < 0) {
         DevProduct t = g;
         t.M = 1; t.N = g.M;
         t.a_m = g.b_n; t.a_k = g.b_k; t.a_off = g.b_off;
         t.b_k = g.a_k; t.b_n = g.a_m; t.b_off = g.a_off;
+        for (int i = 0; i < t.epi.n; i++)
+            if (t.epi.step[i].op == HODU_ROCM_EPI_ADD_ROW) t.epi.step[i].stride = 0;
         const int rc = dispatch_few_rows(ctx, kind, dtype, b, a, c, t);
         if (rc != HODU_ROCM_UNSUPPORTED) return rc;
     }

@@ -198,3 +198,24 @@ def test_attention_over_random_layouts(contexts, dt):
                              close_key0=bool(g.integers(2)), qv=qv, kv=kv, vv=vv)
         except AssertionError as e:
             raise AssertionError(f"{what}: {e}") from None
+
+
+@pytest.mark.parametrize("dt", ffi.EPILOGUE_DTYPES + ["bf16_f8e4m3w"])
+def test_fused_steps_over_random_layouts(contexts, dt):
+    """the product with add(bias) / mul_scalar / relu in its store equals the plain product followed by the reference's
+    own kernels, bit for bit, whatever kernel family the layout selects"""
+    from test_gpu_epilogue import FLOATS, SPECS, check_fused
+    g = np.random.default_rng(6000 + sum(map(ord, dt)))
+    for n in range(2 * ROUNDS):
+        op, lv, rv = product_case(g)
+        if 0 in lv.shape or 0 in rv.shape:
+            continue
+        spec = SPECS[int(g.integers(len(SPECS)))]
+        if dt not in FLOATS and dt != "bf16_f8e4m3w" and ("relu",) in spec:
+            spec = SPECS[0]
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        try:
+            check_fused(ctx, op, dt, lv, rv, spec, seed=n, must_change=False)
+        except AssertionError as e:
+            raise AssertionError(f"{op} {dt} + {spec} case {n}: lhs {lv.shape} {lv.strides} +{lv.offset}, rhs {rv.shape} {rv.strides} "
+                                 f"+{rv.offset}, kernel {ctx.last_kernel()}: {e}") from None
