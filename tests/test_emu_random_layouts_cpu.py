@@ -22,7 +22,7 @@ from hodu_amd import ffi
 pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host clang++ for the CPU build")
 V = H.View
 MORE = int(os.environ.get("HODU_EMU_ALL", "0") or 0) > 0
-ROUNDS = 40 if MORE else 8  # multiplies the cases per dtype and family
+ROUNDS = 40 if MORE else 6  # multiplies the cases per dtype and family
 
 
 @pytest.fixture(scope="module")
@@ -219,3 +219,87 @@ def test_fused_steps_over_random_layouts(contexts, dt):
         except AssertionError as e:
             raise AssertionError(f"{op} {dt} + {spec} case {n}: lhs {lv.shape} {lv.strides} +{lv.offset}, rhs {rv.shape} {rv.strides} "
                                  f"+{rv.offset}, kernel {ctx.last_kernel()}: {e}") from None
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "i8", "u8", "f8e4m3", "f8e5m2", "bf16_f8e4m3w", "i32_i8i8"])
+def test_pinned_tiles_and_k_cuts_over_random_layouts(contexts, dt):
+    """the same draw with the testing hooks pinning a tile of the matrix-core kernels (general and pipelined, 256 x 256
+    down to 64 x 64, the 16 x 16 x 32 tile and its respaced form) and a number of K ranges: the large tiles on small,
+    ragged, oddly laid out products, where the automatic choice never puts them.  A hook that does not apply to a
+    layout leaves the choice to the dispatcher; whatever runs must be right"""
+    g = np.random.default_rng(7000 + sum(map(ord, dt)))
+    for n in range(4 * ROUNDS):
+        op, lv, rv = product_case(g)
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        hook, cuts = int(g.choice([0, 1, 2, 3, 10, 11, 12, 13, 15, 16])), int(g.choice([-1, -1, 1, 2, 3]))
+        ctx.force_tile(hook)
+        ctx.force_splitk(cuts)
+        try:
+            check_product(ctx, op, dt, lv, rv, seed=n, scale=2.0 if dt.startswith("f8") else 1.0)
+        except AssertionError as e:
+            raise AssertionError(f"{op} {dt} case {n}, hook {hook}, {cuts} K ranges: lhs {lv.shape} {lv.strides} +{lv.offset}, rhs {rv.shape} "
+                                 f"{rv.strides} +{rv.offset}, kernel {ctx.last_kernel()}: {e}") from None
+        finally:
+            ctx.force_tile(-1)
+            ctx.force_splitk(-1)
+
+
+@pytest.mark.parametrize("dt", ["f8e4m3", "f8e5m2", "bf16", "f16"])
+def test_reference_sums_over_random_layouts(contexts, dt):
+    """with the context switched to the reference's arithmetic, narrow-float products store the reference's bytes
+    (the oracle's reference-faithful product) over any layout"""
+    from gpu_util import run_product
+    from test_emu_reference_sums_cpu import same_bytes
+    g = np.random.default_rng(8000 + sum(map(ord, dt)))
+    for n in range(2 * ROUNDS):
+        op, lv, rv = product_case(g)
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        a = H.random_storage(dt, max(lv.span(), 1), 100 + n, 0.5 if dt == "f8e4m3" else 1.0)
+        b = H.random_storage(dt, max(rv.span(), 1), 200 + n, 0.5 if dt == "f8e4m3" else 1.0)
+        md = H.dot_md(lv, rv) if op == "dot" else H.matmul_md(lv, rv)
+        ctx.set_reference_sums(True)
+        try:
+            got = run_product(ctx, op, dt, a, b, md)
+            kernel = ctx.last_kernel()
+        finally:
+            ctx.set_reference_sums(False)
+        want = (oracle.dot_asis if op == "dot" else oracle.matmul_asis)(dt, a, b, md)
+        bad = same_bytes(dt, got, want)
+        assert kernel == f"reference_sums_{dt}" or got.size == 0, kernel
+        assert bad.size == 0, (f"{op} {dt} case {n}: lhs {lv.shape} {lv.strides} +{lv.offset}, rhs {rv.shape} {rv.strides} +{rv.offset}: "
+                               f"{bad.size} of {got.size} outputs differ, first at {bad[:5]}")
+
+
+def test_the_entry_point_that_allocates_nothing_over_random_shapes(contexts):
+    """hodu_rocm_dot_bf16_f8e4m3w_noalloc against the allocating entry point: the same kernel and the same bytes, from
+    one row against a small weight to shapes that are cut along K through the static scratch"""
+    from test_zz_no_alloc import both
+    g = np.random.default_rng(9000)
+    for n in range(2 * ROUNDS):
+        m = dims(g, [1, 2, 4, 5, 12, 16, 17, 64, 128, 200])
+        k = dims(g, [64, 128, 192, 256, 512, 1024, 4096])
+        n_cols = dims(g, [16, 48, 128, 200, 256, 512, 1040])
+        while m * k * n_cols > 40_000_000:
+            n_cols = max(16, n_cols // 2)
+        both(contexts["end" if n % 2 == 0 else "start"], m, n_cols, k, 10 * n)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64"])
+def test_masked_softmax_over_random_layouts(contexts, dt):
+    from test_zx_softmax_masked import check as check_masked_softmax
+    g = np.random.default_rng(9500 + sum(map(ord, dt)))
+    for n in range(3 * ROUNDS):
+        nd = int(g.integers(1, 5))
+        shape = [dims(g, [1, 2, 3, 5, 8, 17, 33, 64, 130, 700]) for _ in range(nd)]
+        while int(np.prod(shape, dtype=np.int64)) > 60_000:
+            shape[int(np.argmax(shape))] //= 2
+        v = random_view(g, shape)
+        keep = int(g.integers(1, nd + 1))
+        mask_shape = [e if g.random() < 0.6 else 1 for e in shape[nd - keep:]]
+        mask_shape[-1] = shape[-1]  # (the helper opens entry 0 of every mask row)
+        causal = nd >= 2 and bool(g.integers(2))
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        try:
+            check_masked_softmax(ctx, dt, v, mask_shape, causal=causal, seed=n)
+        except AssertionError as e:
+            raise AssertionError(f"masked softmax {dt} case {n}: {v.shape} {v.strides} +{v.offset}, mask {mask_shape}, causal {causal}: {e}") from None
