@@ -1,0 +1,136 @@
+"""Randomly drawn Tensor-level programs through the host mirror (hodu_amd.tensor over hodu_amd/host/capi.cpp, linked
+against the CPU build of the kernels) against numpy.
+
+A program is a pair of tensors, each taken through a random chain of view operations (transpose, slice with a step,
+unsqueeze + broadcast, reshape of a contiguous tensor), then a matmul -- ranks 1 to 4 on either side, batch dims
+broadcast the way Tensor::matmul broadcasts them (crates/hodu_core/src/tensor/ops/matrix.rs:14-120) -- optionally
+followed by sum over random dims and the matmul's VJP (a vector against a batched matrix is refused, as it is there).  Values are small integers in i32 and f32, so every product,
+sum and gradient is exact and compared for equality; numpy applies the same view operations to its own arrays."""
+import numpy as np
+import pytest
+
+import emu_util
+from hodu_amd import tensor as T
+
+pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host clang++ for the CPU build")
+NP = {"i32": np.int32, "f32": np.float32, "i64": np.int64}
+BITS = {"i32": np.uint32, "f32": np.uint32, "i64": np.uint64}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def host_mirror_over_the_cpu_build():
+    saved_path, saved_lib = T.HOST_LIB_PATH, T._lib
+    T.HOST_LIB_PATH, T._lib = emu_util.build_host(), None
+    yield
+    T.HOST_LIB_PATH, T._lib = saved_path, saved_lib
+
+
+def make(g, dt, shape):
+    a = g.integers(-4, 5, size=shape).astype(NP[dt])
+    return T.Tensor.from_bits(a.reshape(-1).view(BITS[dt]), dt, list(shape)), a
+
+
+def values(t, dt):
+    return t.to_bits().view(NP[dt]).reshape(t.shape)
+
+
+def random_views(g, t, a, want_shape):
+    """takes (tensor, array) of any shape whose size is that of a padded want_shape to a view of want_shape"""
+    # start: storage holds want_shape with every dim padded and in a random order
+    n = len(want_shape)
+    for d in range(n):                                   # slice every dim back to its extent, some with a step
+        have = a.shape[d]
+        step = 2 if have >= 2 * want_shape[d] and want_shape[d] > 0 else 1
+        start = int(g.integers(0, have - (want_shape[d] - 1) * step)) if want_shape[d] > 0 else 0
+        end = start + (want_shape[d] - 1) * step + 1 if want_shape[d] > 0 else start
+        t, a = t.slice(d, start, end, step), a[(slice(None),) * d + (slice(start, end, step),)]
+    return t, a
+
+
+def operand(g, dt, shape):
+    """a tensor of logical `shape` reached through random views of a larger, permuted storage"""
+    n = len(shape)
+    perm = list(g.permutation(n))
+    padded = [s * int(g.choice([1, 1, 2])) + int(g.choice([0, 0, 1, 3])) for s in shape]
+    t, a = make(g, dt, [padded[p] for p in perm])        # stored in permuted order
+    inv = [perm.index(d) for d in range(n)]
+    # undo the permutation with transposes (a sequence of swaps)
+    order = list(perm)
+    for d in range(n):
+        j = order.index(d)
+        if j != d:
+            t, a = t.transpose(d, j), np.swapaxes(a, d, j)
+            order[d], order[j] = order[j], order[d]
+    t, a = random_views(g, t, a, shape)
+    assert list(a.shape) == list(shape) and inv is not None
+    return t, a
+
+
+def broadcastable_batches(g):
+    nb = int(g.integers(0, 3))
+    full = [int(g.integers(1, 4)) for _ in range(nb)]
+    def side():
+        keep = int(g.integers(0, nb + 1))
+        return [b if g.random() < 0.7 else 1 for b in full[nb - keep:]]
+    return side(), side()
+
+
+@pytest.fixture(params=["nocopy", "reference"])
+def mode(request):
+    """'reference' copies non-contiguous operands and materialises broadcast batches the way hodu does today, 'nocopy'
+    hands the views to the kernels: the same values either way"""
+    T.set_matmul_mode(request.param)
+    yield request.param
+    T.set_matmul_mode("nocopy")
+
+
+@pytest.mark.parametrize("dt", ["i32", "f32", "i64"])
+def test_matmul_programs(dt, mode):
+    g = np.random.default_rng(11000 + sum(map(ord, dt)))
+    for n in range(120):
+        m, k, cols = (int(g.choice([1, 2, 3, 8, 16, 17, 33, 64])) for _ in range(3))
+        lb, rb = broadcastable_batches(g)
+        kind = int(g.integers(0, 10))
+        if kind == 0:
+            ls, rs = [k], [k]                            # two vectors
+        elif kind == 1:
+            ls, rs = [k], [k, cols]                      # vector x matrix
+        elif kind == 2:
+            ls, rs = [m, k], [k]                         # matrix x vector
+        elif kind == 3:                                  # a vector against a batched matrix: the reference refuses
+            (ta, _), (tb, _) = operand(g, dt, [2, m, k]), operand(g, dt, [k])
+            with pytest.raises(T.HoduError, match="IncompatibleShapes"):
+                ta.matmul(tb)
+            with pytest.raises(T.HoduError, match="IncompatibleShapes"):
+                tb.matmul(operand(g, dt, [2, k, cols])[0])
+            continue
+        else:
+            ls, rs = lb + [m, k], rb + [k, cols]
+        (ta, a), (tb, b) = operand(g, dt, ls), operand(g, dt, rs)
+        what = f"{dt} case {n}: {ls} {ta.layout()} x {rs} {tb.layout()}"
+        out = ta.matmul(tb)
+        want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+        assert np.abs(want).max(initial=0) < 2 ** 24
+        assert list(out.shape) == list(want.shape), what
+        assert np.array_equal(values(out, dt).astype(np.float64), want), what
+        if want.ndim >= 1 and g.random() < 0.5:          # a sum over some dims of the product
+            dims = sorted(int(d) for d in g.choice(want.ndim, size=int(g.integers(1, want.ndim + 1)), replace=False))
+            keep = bool(g.integers(2))
+            got = out.sum(dims, keep)
+            assert np.array_equal(values(got, dt).astype(np.float64), want.sum(axis=tuple(dims), keepdims=keep)), what + f" sum {dims} {keep}"
+        if len(ls) >= 2 and len(rs) >= 2 and g.random() < 0.5:  # the gradient of sum(out * grad) w.r.t. both operands
+            tg, grad = make(g, dt, list(want.shape))
+            da, db = T.matmul_vjp(ta, tb, tg)
+            g64, a64, b64 = grad.astype(np.float64), a.astype(np.float64), b.astype(np.float64)
+            want_a = np.matmul(g64, np.swapaxes(b64, -1, -2))
+            want_b = np.matmul(np.swapaxes(a64, -1, -2), g64)
+            # summed back to the operand's shape where matmul had broadcast it
+            def to_shape(x, shape):
+                while x.ndim > len(shape):
+                    x = x.sum(axis=0)
+                for d, s in enumerate(shape):
+                    if s == 1 and x.shape[d] != 1:
+                        x = x.sum(axis=d, keepdims=True)
+                return x
+            assert np.array_equal(values(da, dt).astype(np.float64), to_shape(want_a, ls)), what + " dA"
+            assert np.array_equal(values(db, dt).astype(np.float64), to_shape(want_b, rs)), what + " dB"
