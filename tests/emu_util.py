@@ -26,8 +26,9 @@ EMU = os.path.join(ROOT, "tests", "emu")
 # HODU_EMU_SANITIZE=1: an undefined-behaviour-checked build of its own; =thread: a race-checked one, which only a
 # program that carries the ThreadSanitizer runtime can load (build_race_driver, build_race_checked_python)
 RACE_CHECKED = os.environ.get("HODU_EMU_SANITIZE", "") == "thread"
-SANITIZE = os.environ.get("HODU_EMU_SANITIZE", "") not in ("", "0") and not RACE_CHECKED
-OUT = os.path.join(EMU, "_build_tsan" if RACE_CHECKED else "_build_ubsan" if SANITIZE else "_build")
+ADDRESS_CHECKED = os.environ.get("HODU_EMU_SANITIZE", "") == "address"  # likewise, with AddressSanitizer
+SANITIZE = os.environ.get("HODU_EMU_SANITIZE", "") not in ("", "0") and not RACE_CHECKED and not ADDRESS_CHECKED
+OUT = os.path.join(EMU, "_build_tsan" if RACE_CHECKED else "_build_asan" if ADDRESS_CHECKED else "_build_ubsan" if SANITIZE else "_build")
 CSRC = os.path.join(ROOT, "hodu_amd", "csrc")
 SOURCES = [os.path.join(CSRC, f) for f in ("api.cpp", "metadata.cpp", "softmax.hip", "cast.hip", "reduce.hip", "gemm_generic.hip", "gemm_refsum.hip")] + \
           [os.path.join(EMU, "emu_runtime.cpp")]
@@ -73,6 +74,10 @@ def build(mfma=False, race_checked=RACE_CHECKED):
         # shifts, out-of-range conversions, indexing past a fixed-size array) aborts with a report.  Not the alignment
         # check: the kernels' 16-byte accesses at element alignment are what the hardware does.
         flags += ["-fsanitize=undefined", "-fno-sanitize=alignment,vptr,function", "-fno-sanitize-recover=all", "-g1"]
+    if ADDRESS_CHECKED and not race_checked:
+        # every access of host code and kernels against the red zones around heap blocks, globals (the LDS array, the
+        # static scratch) and stack frames (the kernels' fixed-size register arrays)
+        flags += ["-fsanitize=address", "-fno-omit-frame-pointer", "-g1"]
     if race_checked:
         # every load and store of the kernels' source is recorded per host thread, i.e. per wavefront.  Not function
         # entries and exits: the lanes of a wavefront are contexts that one thread switches between in the middle of
@@ -131,21 +136,21 @@ def build_race_driver():
     return exe
 
 
-def build_race_checked_python():
-    """tests/emu/python_host.cpp: this Python with the ThreadSanitizer runtime linked in; returns the program's path
-    (None: no host clang, or no Python headers / library to link)"""
+def build_race_checked_python(sanitizer="thread"):
+    """tests/emu/python_host.cpp: this Python with the ThreadSanitizer (or AddressSanitizer) runtime linked in; returns
+    the program's path (None: no host clang, or no Python headers / library to link)"""
     import sysconfig
     cxx, inc, libdir = compiler(), sysconfig.get_paths()["include"], sysconfig.get_config_var("LIBDIR")
     ver = sysconfig.get_config_var("LDVERSION")
     if cxx is None or not os.path.exists(os.path.join(inc, "Python.h")) or not ver:
         return None
-    out_dir = os.path.join(EMU, "_build_tsan")
+    out_dir = os.path.join(EMU, "_build_tsan" if sanitizer == "thread" else "_build_asan")
     os.makedirs(out_dir, exist_ok=True)
-    exe, src = os.path.join(out_dir, "python_tsan"), os.path.join(EMU, "python_host.cpp")
+    exe, src = os.path.join(out_dir, "python_tsan" if sanitizer == "thread" else "python_asan"), os.path.join(EMU, "python_host.cpp")
     if os.path.exists(exe) and os.path.getmtime(exe) > os.path.getmtime(src):
         return exe
     tmp = exe + f".{os.getpid()}.tmp"
-    r = subprocess.run([cxx, "-O1", "-fsanitize=thread", f"-I{inc}", src, "-o", tmp, f"-L{libdir}", f"-lpython{ver}", "-ldl", "-lm"],
+    r = subprocess.run([cxx, "-O1", f"-fsanitize={sanitizer}", f"-I{inc}", src, "-o", tmp, f"-L{libdir}", f"-lpython{ver}", "-ldl", "-lm"],
                        capture_output=True, text=True)
     if r.returncode != 0:
         return None
@@ -168,7 +173,8 @@ def build_host():
         return HOST_LIB
     tmp = HOST_LIB + f".{os.getpid()}.tmp"
     cmd = [compiler(), "-std=c++17", "-O1", "-fPIC", "-shared", f"-I{os.path.join(ROOT, 'include')}", f"-I{host_dir}",
-           os.path.join(host_dir, "capi.cpp"), "-o", tmp, f"-L{OUT}", "-lhodu_emu_mfma", "-Wl,-rpath,$ORIGIN"]
+           os.path.join(host_dir, "capi.cpp"), "-o", tmp, f"-L{OUT}", "-lhodu_emu_mfma", "-Wl,-rpath,$ORIGIN",
+           *(["-fsanitize=address", "-fno-omit-frame-pointer", "-g1"] if ADDRESS_CHECKED else [])]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"host mirror over the CPU build failed to build:\n{r.stderr[-4000:]}")
