@@ -35,8 +35,8 @@
 // (at most 2^8) rounded to the storage type only as the second product's operand, O accumulated in f32 and rounded
 // once.  The scale is the scalar in the storage type, widened.
 //
-// With an attn_mask (attention.rs:50-56; the MASKED instantiations, a kernel of their own so that the plain one's code
-// does not change): a lane reads the mask bytes of its row's 16 keys of a block in place, through the mask's own
+// With an attn_mask (attention.rs:50-56; the instantiations with a mask operand -- everything they add is behind
+// `if constexpr`, so the plain instantiations' code does not change): a lane reads the mask bytes of its row's 16 keys of a block in place, through the mask's own
 // strides (0 where it is broadcast), and a masked score becomes fill / scale, fill being what the reference's
 // masked_fill writes over the SCALED scores in a 16-bit type (get_neg_inf, attention.rs:88-96, through full_like's
 // rounding: -65504 in f16, -65536 in bf16) -- a finite value, so a row masked entirely comes out as the reference's

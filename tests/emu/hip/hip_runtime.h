@@ -274,22 +274,68 @@ inline void run_grid(const std::function<void()> &call, dim3 grid, dim3 block) {
     static Block blk;  // (workgroups, and launches, run one at a time)
     current() = &blk;
     const unsigned waves = block.x * block.y * block.z / kWave;
+    // The threads of wavefronts 1.. live for the whole launch and are handed one workgroup after the other (the
+    // calling thread is wavefront 0): `turn` counts the workgroups started, `finished` the wavefronts done with the
+    // current one.
+    struct Shift {
+        std::mutex mu;
+        std::condition_variable cv;
+        unsigned long turn = 0;
+        unsigned finished = 0;
+        bool over = false;
+        emu_uint3 idx;
+    } shift;
+    auto body = [&](unsigned w, emu_uint3 idx) {
+        b_idx = idx;
+        b_dim.x = block.x; b_dim.y = block.y; b_dim.z = block.z;
+        g_dim.x = grid.x; g_dim.y = grid.y; g_dim.z = grid.z;
+        run_wave(blk, call, w, block);
+    };
+    std::vector<std::thread> pool;
+    pool.reserve(waves - 1);
+    for (unsigned w = 1; w < waves; w++)
+        pool.emplace_back([&, w] {
+            unsigned long seen = 0;
+            for (;;) {
+                emu_uint3 idx;
+                {
+                    std::unique_lock<std::mutex> hold(shift.mu);
+                    shift.cv.wait(hold, [&] { return shift.over || shift.turn != seen; });
+                    if (shift.over) return;
+                    seen = shift.turn;
+                    idx = shift.idx;
+                }
+                body(w, idx);
+                {
+                    std::lock_guard<std::mutex> hold(shift.mu);
+                    shift.finished++;
+                }
+                shift.cv.notify_all();
+            }
+        });
     for (unsigned bz = 0; bz < grid.z; bz++)
         for (unsigned by = 0; by < grid.y; by++)
             for (unsigned bx = 0; bx < grid.x; bx++) {
                 blk.all.reset(waves);
-                auto body = [&, bx, by, bz](unsigned w) {
-                    b_idx.x = bx; b_idx.y = by; b_idx.z = bz;
-                    b_dim.x = block.x; b_dim.y = block.y; b_dim.z = block.z;
-                    g_dim.x = grid.x; g_dim.y = grid.y; g_dim.z = grid.z;
-                    run_wave(blk, call, w, block);
-                };
-                std::vector<std::thread> pool;
-                pool.reserve(waves - 1);
-                for (unsigned w = 1; w < waves; w++) pool.emplace_back(body, w);
-                body(0);
-                for (auto &th : pool) th.join();
+                emu_uint3 idx;
+                idx.x = bx; idx.y = by; idx.z = bz;
+                {
+                    std::lock_guard<std::mutex> hold(shift.mu);
+                    shift.idx = idx;
+                    shift.finished = 0;
+                    shift.turn++;
+                }
+                shift.cv.notify_all();
+                body(0, idx);
+                std::unique_lock<std::mutex> hold(shift.mu);
+                shift.cv.wait(hold, [&] { return shift.finished == waves - 1; });
             }
+    {
+        std::lock_guard<std::mutex> hold(shift.mu);
+        shift.over = true;
+    }
+    shift.cv.notify_all();
+    for (auto &th : pool) th.join();
     current() = nullptr;
 }
 
