@@ -115,3 +115,30 @@ def test_f32_against_the_reference_five_kernel_chain():
     chain = ref.softmax_chain_f32(filled.ravel(), full)
     o32, o64 = oracle.softmax_masked_spec("f32", x, H.reduce_md(V(full), [2], True), mask.ravel(), [33, 0, 1])
     assert np.allclose(chain, o64, rtol=3e-6, atol=1e-12) and np.allclose(chain, o32, rtol=3e-6, atol=1e-12)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_the_masked_attention_tests_float64_function_is_this_softmax_between_two_products(dt, causal):
+    """tests/test_zx_attention_masked.py compares the one-kernel attention with a float64 function of its own; that
+    function's probabilities are the oracle's masked softmax of the (unrounded) scaled scores -- fill value, causal mask
+    and rows masked entirely included"""
+    import test_zx_attention_masked as A
+    g = np.random.default_rng(5)
+    b, sq, sk, d = 2, 9, 13, 8
+    q, k, v = (g.standard_normal((b, n, d)) for n in (sq, sk, sk))
+    keep = (g.random((b, 1, sk)) < 0.6).astype(np.uint8)
+    keep[1, 0, :] = 0  # a batch whose every row is masked entirely
+    scale = 0.35
+    want, _, p, _ = A.reference(q, k, v, scale, causal, keep, A.FILL[dt])
+    # the oracle takes the scores in a storage type: f64 holds them exactly
+    scores = q @ np.swapaxes(k, -1, -2) * scale
+    md = H.reduce_md(H.View([b, sq, sk]), [2], True)
+    _, o64 = oracle.softmax_masked_spec("f64", scores.ravel(), md, keep.ravel(), [sk, 0, 1], 0, causal)
+    # f64's fill is -inf: identical wherever a row has an open key; rows masked entirely are uniform in the 16-bit types
+    o64 = o64.reshape(b, sq, sk)
+    open_rows = ~np.isnan(o64).any(-1)
+    assert open_rows[0].all() and not open_rows[1].any()
+    assert np.allclose(p[open_rows], o64[open_rows], rtol=1e-12, atol=1e-300)
+    assert np.allclose(p[~open_rows], 1.0 / sk)
+    assert np.allclose(want, p @ v)
