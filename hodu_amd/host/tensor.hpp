@@ -209,11 +209,20 @@ public:
 
     // softmax(-1) of masked_fill(mask.eq_scalar(0), get_neg_inf(dtype)) (attention.rs:50-56, :88-96) as one launch: the
     // mask broadcasts against the scores the way masked_fill's where3 broadcasts it (right-aligned, extent 1 repeats)
-    Tensor softmax_masked(const Tensor &mask, bool causal = false) const {
+    Tensor softmax_masked(const Tensor &mask_any, bool causal = false) const {
         if (layout_.ndim() == 0) throw Error(ErrorKind::InvalidArgument, "softmax: a scalar has no last dim");
+        const Tensor mask = mask_any.as_mask_bytes();
         const Layout ml = mask.layout().broadcast_to(shape());
         auto out = std::make_shared<RocmStorage>(storage_->call_ops_softmax_masked(layout_, causal, *mask.storage_, ml));
         return Tensor(out, Layout::from_shape(shape()));
+    }
+    // `mask.eq_scalar(0)` (attention.rs:52) takes a mask of any dtype; the kernels read one byte per element, 0 = masked
+    // out.  bool / u8 / i8 are that already; anything else goes through to_dtype(BOOL), whose x != 0 is the same predicate
+    // (-0.0 masks, a NaN attends).
+    Tensor as_mask_bytes() const {
+        const DType d = dtype();
+        const bool bytes = (d == DType::BOOL || d == DType::U8 || d == DType::I8) && !storage_->deferred();
+        return bytes ? *this : to_dtype(DType::BOOL);
     }
 
     // `value` as a scalar of dtype `dt`, round-to-nearest-even (what Scalar::to_dtype does through the `half` crate's
@@ -262,6 +271,7 @@ public:
         const double scale = 1.0 / std::sqrt((double)q.shape().back());
         unsigned char bits[8];
         const size_t n = scalar_bits(q.dtype(), scale, bits);
+        const Tensor mask_bytes = attn_mask ? attn_mask->as_mask_bytes() : q;  // (q: a placeholder nobody reads)
         // one kernel where it applies: q [.., Sq, D], k and v [.., Sk, D] with the batch dims broadcast the way the
         // two matmuls would broadcast them; an attn_mask (1 = attend, 0 = mask out; attention.rs:50-56) is read in
         // place, broadcast against the scores the way masked_fill's where3 broadcasts it
@@ -307,7 +317,7 @@ public:
                     scores_shape.push_back(q.shape()[qn - 2]);
                     scores_shape.push_back(k.shape()[kn - 2]);
                     try {
-                        ml = attn_mask->layout().broadcast_to(scores_shape);
+                        ml = mask_bytes.layout().broadcast_to(scores_shape);
                     } catch (const Error &) {
                         mask_fits = false;  // the three launches below report it
                     }
@@ -315,14 +325,14 @@ public:
                 if (mask_fits) {
                     auto out = std::make_shared<RocmStorage>(q.storage_->call_ops_attention(
                         *k.storage_, *v.storage_, ql, kl, vl, md, product(out_shape), bits, is_causal, &taken,
-                        attn_mask ? attn_mask->storage_.get() : nullptr, attn_mask ? &ml : nullptr));
+                        attn_mask ? mask_bytes.storage_.get() : nullptr, attn_mask ? &ml : nullptr));
                     if (taken) return Tensor(out, Layout::from_shape(out_shape));
                 }
             }
         }
         // three launches: the scale rides in the first product's store, the masks and the softmax are one kernel
         const Tensor scores = q.matmul_then(k.transpose(-2, -1), {Then::mul_scalar(bits, n)});
-        if (attn_mask) return scores.softmax_masked(*attn_mask, is_causal).matmul(v);
+        if (attn_mask) return scores.softmax_masked(mask_bytes, is_causal).matmul(v);
         return scores.softmax(-1, is_causal).matmul(v);
     }
 

@@ -245,7 +245,7 @@ int hodu_rocm_softmax(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, 
  * mask, a [Sq, Sk] mask shared by every head) -- the mask is read in place, never expanded.  Masked scores count as
  * what the reference fills them with: -inf in f32 / f64, the dtype's rounding of -65504 in f16 / bf16 (:88-96), so a
  * masked entry of a row that has an open one is an exact zero, a row masked entirely is uniform (16-bit types) or NaN
- * (f32 / f64).  A mask of another dtype is cast by the caller (hodu_rocm_cast to u8) or compared on its side. */
+ * (f32 / f64).  A mask of another dtype is cast by the caller with hodu_rocm_cast to bool (x != 0: -0.0 masks, a NaN attends, as eq_scalar(0) has it). */
 int hodu_rocm_softmax_masked(hodu_rocm_ctx *ctx, int dtype, const void *in, void *out, const size_t *metadata,
                              size_t metadata_len, int causal, const void *mask, int mask_dtype,
                              const size_t *mask_layout, size_t mask_layout_len);

@@ -37,7 +37,8 @@ SUITES = ["test_gpu_products", "test_gpu_mfma", "test_gpu_exact", "test_gpu_epil
           # the GPU test of kernels that have not run on a GPU, kept under a name pytest does not collect: it runs here
           "wip_pipe16r"]
 EXCLUDED = {"test_gpu_skinny.test_split_k_arrival_protocol_over_thousands_of_launches",  # (thousands of large launches)
-            "test_zx_softmax_masked.test_attention_with_a_padding_mask_against_float64"}  # (the host mirror)
+            "test_zx_softmax_masked.test_attention_with_a_padding_mask_against_float64",  # (the host mirror: these two
+            "test_zx_softmax_masked.test_a_mask_of_another_dtype_is_its_nonzero_pattern"}  #  run in test_emu_host_mirror_cpu.py)
 # more than a few seconds per case in the CPU build
 HEAVY = {
     "test_gpu_mfma.test_every_variant_ragged", "test_gpu_mfma.test_native_f8_products",

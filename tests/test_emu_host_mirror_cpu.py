@@ -24,7 +24,8 @@ def host_mirror_over_the_cpu_build():
 def _cases():
     import test_gpu_host_tensor as suite
     import test_zx_softmax_masked
-    for mod, names in ((suite, None), (test_zx_softmax_masked, {"test_attention_with_a_padding_mask_against_float64"})):
+    for mod, names in ((suite, None), (test_zx_softmax_masked, {"test_attention_with_a_padding_mask_against_float64",
+                                                                  "test_a_mask_of_another_dtype_is_its_nonzero_pattern"})):
         for name, fn in inspect.getmembers(mod, inspect.isfunction):
             if not name.startswith("test_") or fn.__module__ != mod.__name__ or (names is not None and name not in names):
                 continue

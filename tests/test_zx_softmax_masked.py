@@ -117,3 +117,28 @@ def test_attention_with_a_padding_mask_against_float64(ctx, D, launches):
     # of every p_j of up to 2^-8 |s|, i.e. an error of the output that scales with sum_j p_j |v_j| -- the size of the sum,
     # not of its (possibly cancelling) value; with as few as 33 unmasked keys that floor matters
     assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), p @ np.abs(v64)))
+
+
+@pytest.mark.parametrize("D", [64, 32])
+def test_a_mask_of_another_dtype_is_its_nonzero_pattern(ctx, D):
+    """`mask.eq_scalar(0)` (attention.rs:52) takes any dtype: an f32 mask holding -0.0 (masks), 0.5 and a NaN (attend)
+    gives the bytes of the u8 mask with the same nonzero pattern, through the one kernel (D = 64) and the three launches"""
+    B, Hh, S = 2, 2, 40
+    g = np.random.default_rng(1)
+    q, k, v = (H.f32_to_bf16_rne(g.standard_normal(B * Hh * S * D).astype(np.float32)) for _ in range(3))
+    tq, tk, tv = (T.Tensor.from_bits(b, "bf16", [B, Hh, S, D]) for b in (q, k, v))
+    keep = np.ones((B, 1, 1, S), np.float32)
+    keep[0, ..., 30:] = 0.0
+    keep[1, ..., 5:9] = -0.0
+    keep[1, ..., 20] = 0.5
+    keep[1, ..., 21] = np.nan
+    pattern = np.ones((B, 1, 1, S), np.uint8)
+    pattern[0, ..., 30:] = 0
+    pattern[1, ..., 5:9] = 0
+    as_f32 = T.Tensor.from_bits(keep.ravel().view(np.uint32), "f32", [B, 1, 1, S])
+    as_u8 = T.Tensor.from_bits(pattern.ravel(), "u8", [B, 1, 1, S])
+    for causal in (False, True):
+        T.stats(reset=True)
+        got = T.scaled_dot_product_attention(tq, tk, tv, causal, as_f32).to_bits()
+        assert T.stats()["cast_kernels"] == 1
+        assert np.array_equal(got, T.scaled_dot_product_attention(tq, tk, tv, causal, as_u8).to_bits())
