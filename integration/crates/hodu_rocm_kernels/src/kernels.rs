@@ -101,3 +101,57 @@ pub fn call_ops_contiguous(ctx: &Context, dtype: u8, input: &DeviceBuf, out: &De
 pub fn call_ops_sum(ctx: &Context, dtype: u8, input: &DeviceBuf, out: &DeviceBuf, metadata: &[usize]) -> Result<()> {
     ctx.check(unsafe { ffi::hodu_rocm_sum(ctx.raw(), dtype as c_int, input.as_ptr(), out.as_mut_ptr(), metadata.as_ptr(), metadata.len()) })
 }
+
+/// An `attn_mask` (crates/hodu_nn/src/modules/attention.rs:50-56) read in place: one byte per element (`dtype`: hodu's
+/// discriminant of BOOL, U8 or I8; anything else goes through `call_ops_cast` to BOOL first), 0 = masked out.
+/// `layout` = [nd, strides over the masked tensor's shape.., offset] in elements, stride 0 where the mask is broadcast
+/// (`Layout::broadcast_to(shape)` gives exactly these strides).
+pub struct MaskArg<'a> {
+    pub buf: &'a DeviceBuf,
+    pub dtype: u8,
+    pub layout: &'a [usize],
+}
+
+/// Tensor::softmax (tensor/ops/normalization.rs:4-21) as one kernel; metadata = reduce_metadata of the input layout with
+/// the softmax dim as the one reduced dim (keep_dim).  `causal` folds attention's is_causal mask in (last dim only);
+/// with `mask` the softmax runs along the last dim over masked_fill(mask.eq_scalar(0), get_neg_inf(dtype)).
+pub fn call_ops_softmax(ctx: &Context, dtype: u8, input: &DeviceBuf, out: &DeviceBuf, metadata: &[usize], causal: bool,
+                        mask: Option<MaskArg>) -> Result<()> {
+    let rc = match mask {
+        None => unsafe {
+            ffi::hodu_rocm_softmax(ctx.raw(), dtype as c_int, input.as_ptr(), out.as_mut_ptr(), metadata.as_ptr(), metadata.len(),
+                                   causal as c_int)
+        },
+        Some(m) => unsafe {
+            ffi::hodu_rocm_softmax_masked(ctx.raw(), dtype as c_int, input.as_ptr(), out.as_mut_ptr(), metadata.as_ptr(),
+                                          metadata.len(), causal as c_int, m.buf.as_ptr(), m.dtype as c_int, m.layout.as_ptr(),
+                                          m.layout.len())
+        },
+    };
+    ctx.check(rc)
+}
+
+/// scaled_dot_product_attention (attention.rs:25-70, without dropout) as one kernel.  metadata: [nb, batch_shape..,
+/// Sq, Sk, D, q_strides (nb + 2).., k_strides.., v_strides.., q_off, k_off, v_off]; `scale`: the scalar in `dtype`'s
+/// storage (what mul_scalar would receive); a mask's layout runs over [batch.., Sq, Sk].  Ok(false): the kernel does
+/// not take this call (dtype, head dim, alignment) and nothing was launched -- the caller runs the three launches
+/// (call_ops_matmul with a MUL_SCALAR step, call_ops_softmax, call_ops_matmul).
+pub fn call_ops_attention(ctx: &Context, dtype: u8, q: &DeviceBuf, k: &DeviceBuf, v: &DeviceBuf, out: &DeviceBuf,
+                          metadata: &[usize], scale: &[u8], causal: bool, mask: Option<MaskArg>) -> Result<bool> {
+    let rc = match mask {
+        None => unsafe {
+            ffi::hodu_rocm_attention(ctx.raw(), dtype as c_int, q.as_ptr(), k.as_ptr(), v.as_ptr(), out.as_mut_ptr(),
+                                     metadata.as_ptr(), metadata.len(), scale.as_ptr() as *const core::ffi::c_void, causal as c_int)
+        },
+        Some(m) => unsafe {
+            ffi::hodu_rocm_attention_masked(ctx.raw(), dtype as c_int, q.as_ptr(), k.as_ptr(), v.as_ptr(), out.as_mut_ptr(),
+                                            metadata.as_ptr(), metadata.len(), scale.as_ptr() as *const core::ffi::c_void,
+                                            causal as c_int, m.buf.as_ptr(), m.dtype as c_int, m.layout.as_ptr(), m.layout.len())
+        },
+    };
+    match ctx.check(rc) {
+        Ok(()) => Ok(true),
+        Err(e) if e.is_unsupported() => Ok(false),
+        Err(e) => Err(e),
+    }
+}
