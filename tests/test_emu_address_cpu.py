@@ -28,10 +28,10 @@ def test_tensor_level_and_random_layouts_under_the_address_sanitizer():
     # do not follow; leaks are the interpreter's own
     env = {**os.environ, "HODU_EMU_SANITIZE": "address", "HODU_EMU_ALL": "0", "PYTHONPATH": os.pathsep.join(p for p in sys.path if p),
            "ASAN_OPTIONS": "detect_stack_use_after_return=0:detect_leaks=0:verify_asan_link_order=0"}
-    # (the no-alloc entry point's shapes, thousands of workgroups each, take too long under this sanitizer: its static
-    # scratch is covered by tests/test_zz_no_alloc.py's cases in the plain and the race-checked CPU build)
+    # (the no-alloc entry point's shapes and the masked softmax's rows, thousands of workgroups each, take too long
+    # under this sanitizer; both run in the plain and the race-checked CPU build)
     r = subprocess.run([python, "-m", "pytest", *[os.path.join("tests", f) for f in FILES], "-q", "-x", "-p", "no:cacheprovider",
-                        "-k", "not allocates_nothing"],
+                        "-k", "not allocates_nothing and not masked_softmax"],
                        capture_output=True, text=True, cwd=ROOT, env=env)
     assert "AddressSanitizer" not in r.stderr and "AddressSanitizer" not in r.stdout, (r.stdout[-3000:] + r.stderr[-3000:])
     assert r.returncode == 0 and " passed" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
