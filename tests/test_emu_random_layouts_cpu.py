@@ -214,11 +214,19 @@ def test_fused_steps_over_random_layouts(contexts, dt):
         if dt not in FLOATS and dt != "bf16_f8e4m3w" and ("relu",) in spec:
             spec = SPECS[0]
         ctx = contexts["end" if n % 2 == 0 else "start"]
+        # every other case with a tile (and a number of K ranges) pinned, for the kinds that have matrix-core tiles
+        hook = int(g.choice([0, 1, 2, 3, 10, 11, 12, 13, 15, 16])) if n % 2 and dt in ("bf16", "f16", "f32", "i8", "u8", "bf16_f8e4m3w") else -1
+        cuts = int(g.choice([-1, 1, 2, 3])) if hook >= 0 else -1
+        ctx.force_tile(hook)
+        ctx.force_splitk(cuts)
         try:
             check_fused(ctx, op, dt, lv, rv, spec, seed=n, must_change=False)
         except AssertionError as e:
-            raise AssertionError(f"{op} {dt} + {spec} case {n}: lhs {lv.shape} {lv.strides} +{lv.offset}, rhs {rv.shape} {rv.strides} "
-                                 f"+{rv.offset}, kernel {ctx.last_kernel()}: {e}") from None
+            raise AssertionError(f"{op} {dt} + {spec} case {n}, hook {hook}, {cuts} K ranges: lhs {lv.shape} {lv.strides} +{lv.offset}, "
+                                 f"rhs {rv.shape} {rv.strides} +{rv.offset}, kernel {ctx.last_kernel()}: {e}") from None
+        finally:
+            ctx.force_tile(-1)
+            ctx.force_splitk(-1)
 
 
 @pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "i8", "u8", "f8e4m3", "f8e5m2", "bf16_f8e4m3w", "i32_i8i8"])
