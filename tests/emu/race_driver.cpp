@@ -4,7 +4,7 @@
 // access of the kernels' unmodified source and reports such a pair.  The lanes of one wavefront are contexts on one
 // thread and cannot race with each other.
 //
-// The driver runs products through the C ABI with the testing hook pinning one tile kernel after the other, under the
+// The driver runs products and the one-kernel attention through the C ABI with the testing hook pinning one tile kernel after the other, under the
 // earliest and the latest model of LDS-DMA arrival (a refill that comes too early for a slower reader shows under the
 // first, a wait that comes too late under the second), checks each result against the integer product (operands are
 // small integers: every partial sum is exact), and exits non-zero on a wrong result; ThreadSanitizer makes the exit
@@ -129,6 +129,73 @@ int run(hodu_rocm_ctx *ctx, const Case &c) {
     hodu_rocm_free(ctx, dc);
     return bad;
 }
+// the one-kernel attention (eight wavefronts share K / V blocks in LDS and meet in pairs at the end), with and without an
+// attn_mask, against a plain float loop
+int attention(hodu_rocm_ctx *ctx, int d, int sq, int sk, bool causal, bool masked) {
+    const int heads = 2;
+    std::vector<uint16_t> q((size_t)heads * sq * d), k((size_t)heads * sk * d), v((size_t)heads * sk * d);
+    std::vector<uint8_t> keep((size_t)sk);
+    uint32_t seed = 777u + (uint32_t)(d + sq + sk);
+    for (auto &x : q) x = bf16_of((int)(lcg(seed) >> 29) - 4);
+    for (auto &x : k) x = bf16_of((int)(lcg(seed) >> 30) - 2);
+    for (auto &x : v) x = bf16_of((int)(lcg(seed) >> 28) - 8);
+    for (int j = 0; j < sk; j++) keep[j] = j == 0 || (lcg(seed) >> 30) != 0;
+    void *dq, *dk, *dv, *dm, *dout;
+    if (hodu_rocm_alloc(ctx, 2 * q.size(), &dq) || hodu_rocm_alloc(ctx, 2 * k.size(), &dk) || hodu_rocm_alloc(ctx, 2 * v.size(), &dv) ||
+        hodu_rocm_alloc(ctx, keep.size(), &dm) || hodu_rocm_alloc(ctx, 2 * q.size(), &dout))
+        return 1;
+    hodu_rocm_memcpy_h2d(ctx, dq, q.data(), 2 * q.size());
+    hodu_rocm_memcpy_h2d(ctx, dk, k.data(), 2 * k.size());
+    hodu_rocm_memcpy_h2d(ctx, dv, v.data(), 2 * v.size());
+    hodu_rocm_memcpy_h2d(ctx, dm, keep.data(), keep.size());
+    const size_t md[] = {1, (size_t)heads, (size_t)sq, (size_t)sk, (size_t)d, (size_t)sq * d, (size_t)d, 1, (size_t)sk * d, (size_t)d, 1,
+                         (size_t)sk * d, (size_t)d, 1, 0, 0, 0};
+    const float scale = 0.125f;  // exact in bf16
+    const uint16_t scale_bits = 0x3E00;
+    const size_t mask_layout[] = {3, 0, 0, 1, 0};  // one [Sk] mask for every head and row
+    hodu_rocm_debug_force_tile(ctx, -1);
+    const int rc = masked ? hodu_rocm_attention_masked(ctx, HODU_BF16, dq, dk, dv, dout, md, 17, &scale_bits, causal, dm, HODU_U8, mask_layout, 5)
+                          : hodu_rocm_attention(ctx, HODU_BF16, dq, dk, dv, dout, md, 17, &scale_bits, causal);
+    int bad = 0;
+    if (rc != 0) {
+        fprintf(stderr, "attention: status %d: %s\n", rc, hodu_rocm_last_error(ctx));
+        bad = 1;
+    } else {
+        std::vector<uint16_t> out(q.size());
+        hodu_rocm_memcpy_d2h(ctx, out.data(), dout, 2 * out.size());
+        std::vector<double> p((size_t)sk);
+        for (int h = 0; h < heads && !bad; h++)
+            for (int i = 0; i < sq && !bad; i++) {
+                double top = -1e300, sum = 0;
+                for (int j = 0; j < sk; j++) {
+                    double s = 0;
+                    for (int c = 0; c < d; c++) s += (double)f32_of(q[((size_t)h * sq + i) * d + c]) * f32_of(k[((size_t)h * sk + j) * d + c]);
+                    s *= scale;
+                    const bool filled = (masked && !keep[j]) || (causal && j > i);
+                    p[j] = filled ? (masked ? -65536.0 : -1e300) : s;
+                    top = p[j] > top ? p[j] : top;
+                }
+                for (int j = 0; j < sk; j++) sum += (p[j] = std::exp(p[j] - top));
+                for (int c = 0; c < d; c++) {
+                    double want = 0, size = 0;
+                    for (int j = 0; j < sk; j++) {
+                        want += p[j] / sum * f32_of(v[((size_t)h * sk + j) * d + c]);
+                        size += p[j] / sum * std::fabs(f32_of(v[((size_t)h * sk + j) * d + c]));
+                    }
+                    const double got = f32_of(out[((size_t)h * sq + i) * d + c]);
+                    if (!(std::fabs(got - want) <= 2e-2 * size + 1e-3)) {
+                        fprintf(stderr, "attention head %d row %d column %d: %g, the function gives %g\n", h, i, c, got, want);
+                        bad = 1;
+                        break;
+                    }
+                }
+            }
+    }
+    printf("%-44s %-44s %s\n", masked ? "attention with a mask" : "attention", hodu_rocm_last_kernel(ctx), bad ? "WRONG" : "ok");
+    fflush(stdout);
+    for (void *b : {dq, dk, dv, dm, dout}) hodu_rocm_free(ctx, b);
+    return bad;
+}
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -167,6 +234,10 @@ int main(int argc, char **argv) {
         printf("LDS-DMA arrival model %d\n", model);
         for (const Case &c : cases) bad |= run(ctx, c);
         bad |= handoff(ctx, true, true);
+        bad |= attention(ctx, 128, 200, 300, true, false);
+        bad |= attention(ctx, 64, 130, 200, false, false);
+        bad |= attention(ctx, 128, 130, 200, true, true);
+        bad |= attention(ctx, 64, 200, 300, false, true);
     }
     hodu_rocm_ctx_destroy(ctx);
     return bad;

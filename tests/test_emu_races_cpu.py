@@ -9,7 +9,8 @@ what the result-comparing tests cannot do: they only see the interleavings the h
 
  * tests/emu/race_driver.cpp, a native program: products through the C ABI, the testing hook pinning each tile kernel
    (general, pipelined 32x32x16, 16x16x32 and its respaced form; bf16 and f8e4m3 weights; both right-operand layouts;
-   K cut across workgroups; the few-rows kernel), under the earliest and the latest model of LDS-DMA arrival;
+   K cut across workgroups; the few-rows kernel) and the one-kernel attention with and without a mask, under the
+   earliest and the latest model of LDS-DMA arrival;
  * the same program's hand-offs with the barrier left out, or the wait placed behind the barrier, must be reported:
    the detector has teeth;
  * opt-in (HODU_EMU_ALL=1): every pytest file that drives the CPU build, run by a Python that carries the sanitizer
@@ -48,9 +49,9 @@ def test_tile_kernels_have_no_race_between_wavefronts(driver):
     assert "ThreadSanitizer" not in r.stderr, r.stderr[:3000]
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     lines = [ln for ln in r.stdout.split("\n") if ln.endswith(" ok")]
-    assert len(lines) == 32 and not any("WRONG" in ln for ln in r.stdout.split("\n"))
+    assert len(lines) == 40 and not any("WRONG" in ln for ln in r.stdout.split("\n"))
     for kernel in ("mfma_bf16_256x256_KK", "mfma_bf16_pipe256x256_KK_splitk3", "mfma_bf16_pipe256x256mi16_KM", "mfma_bf16_pipe256x256mi16_KK_r",
-                   "mfma_bf16_f8w_pipe256x256mi16_KM_r", "skinny_bf16_f8w"):
+                   "mfma_bf16_f8w_pipe256x256mi16_KM_r", "skinny_bf16_f8w", "attention_fwd_bf16", "attention_masked_fwd_bf16_d64"):
         assert sum(kernel in ln.split() for ln in lines) == 2, kernel  # once per arrival model
 
 
