@@ -206,6 +206,15 @@ def test_small_m_kernels(ctx, name):
                             expect_kernel="gemv_")
 
 
+@pytest.mark.parametrize("name", ["bf16", "f16", "f32"])
+def test_matrix_times_vector_keeps_the_few_rows_route_with_steps(ctx, name):
+    """[M, K] x [K, 1] runs as the transposed one-row product; fused steps go along (a vector added along an output row
+    of one element is that element for every output)"""
+    for n, spec in enumerate(SPECS):
+        check_fused(ctx, "dot", name, V([300, 1040]), V([1040, 1]), spec, seed=n, expect_kernel=("gemv_", "skinny_"))
+    check_fused(ctx, "dot", name, V([64, 512], offset=8), V([512, 1], [3, 0]), SPECS[3], seed=9)  # a strided vector
+
+
 def test_linear_layer_of_config3(ctx):
     """x[16, 4096] (bf16) times the f8e4m3 weight [4096, 4096] passed transposed, plus a bf16 bias: the layer the
     fused entry point exists for, at its real size"""

@@ -115,6 +115,15 @@ def test_strided_inputs(ctx, dt):
     check_sum(ctx, dt, V([12, 64], offset=5), [0], False, 14, "sum_by_output")
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16", "i32"])
+def test_few_outputs_that_are_not_dense_take_the_chunked_kernels_too(ctx, dt):
+    """a strided tensor summed to a scalar, and a handful of stepped outputs with a long stepped reduction: cut into
+    chunks across workgroups like the dense case, not walked by one lane per output"""
+    check_sum(ctx, dt, V([500, 300]).t(), [0, 1], False, 1, "sum_chunks")
+    check_sum(ctx, dt, V([4, 3000], [2, 8]), [1], False, 2, "sum_chunks")
+    check_sum(ctx, dt, V([4, 3000], [2, 8], offset=3), [1], True, 3, "sum_chunks")
+
+
 def test_config5_weight_gradient_shape(ctx):
     """[8, 512, 1024] bf16 partial gradients summed over the batch: every input element read once"""
     check_sum(ctx, "bf16", V([8, 512, 1024]), [0], False, 15, "sum_by_output_vec")
