@@ -10,12 +10,18 @@ from hodu_amd import ffi, tensor
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def test_layout_algebra_and_metadata_encoders(tmp_path):
-    """The C++ checks hold the reference tests' metadata literals and brute-force view enumeration."""
+@pytest.mark.parametrize("sanitized", [False, True])
+def test_layout_algebra_and_metadata_encoders(tmp_path, sanitized):
+    """The C++ checks hold the reference tests' metadata literals and brute-force view enumeration; once more with the
+    address and undefined-behaviour sanitizers on the host code."""
     exe = tmp_path / "host_layout_tests"
-    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-O1", f"-I{ROOT}/hodu_amd/host",
-                           "-o", str(exe), f"{ROOT}/tests/host/host_layout_tests.cpp"])
-    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    extra = ["-fsanitize=address,undefined", "-fno-sanitize-recover=all"] if sanitized else []
+    built = subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-O1", *extra, f"-I{ROOT}/hodu_amd/host",
+                            "-o", str(exe), f"{ROOT}/tests/host/host_layout_tests.cpp"], capture_output=True, text=True)
+    if sanitized and built.returncode != 0 and ("sanitize" in built.stderr or "asan" in built.stderr):
+        pytest.skip("this g++ has no sanitizer runtimes")
+    assert built.returncode == 0, built.stderr[-3000:]
+    out = subprocess.run([str(exe)], capture_output=True, text=True, env={**os.environ, "ASAN_OPTIONS": "verify_asan_link_order=0"})
     assert out.returncode == 0, out.stdout + out.stderr
     assert "passed" in out.stdout
 
