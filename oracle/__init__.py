@@ -52,8 +52,12 @@ _lib = None
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        build()
-        _lib = ctypes.CDLL(os.path.join(_HERE, "liboracle.so"))
+        # HODU_ORACLE_LIB: another build of hodu_oracle.c to check the checker with (`make -C oracle ubsan` writes one
+        # compiled with the undefined-behaviour sanitizer)
+        other = os.environ.get("HODU_ORACLE_LIB")
+        if not other:
+            build()
+        _lib = ctypes.CDLL(os.path.abspath(other) if other else os.path.join(_HERE, "liboracle.so"))
         _lib.oracle_f8e4m3_to_f32.restype = ctypes.c_float
         _lib.oracle_f8e4m3_to_f32.argtypes = [ctypes.c_uint8, ctypes.c_int]
         _lib.oracle_f32_to_f8e4m3.restype = ctypes.c_uint8
