@@ -134,3 +134,31 @@ def test_matmul_programs(dt, mode):
                 return x
             assert np.array_equal(values(da, dt).astype(np.float64), to_shape(want_a, ls)), what + " dA"
             assert np.array_equal(values(db, dt).astype(np.float64), to_shape(want_b, rs)), what + " dB"
+
+
+def test_linear_layers_with_deferred_f8_weights():
+    """hodu_nn's Linear on random shapes -- input [batch.., rows, K] in bf16, weight [N, K] stored as f8e4m3 and cast with a
+    deferred to_dtype, an optional bias and ReLU in the product's store -- from one row (the GEMV kernels) over few rows
+    to tiles: integer values, so the product is exact and every step is the reference kernel's own arithmetic on it"""
+    import helpers as H
+    from test_gpu_host_tensor import _oracle_after
+    g = np.random.default_rng(12000)
+    for n in range(60):
+        lead = [int(g.integers(1, 4)) for _ in range(int(g.integers(0, 3)))]
+        rows, k, cols = int(g.choice([1, 2, 4, 5, 16, 33, 130])), int(g.choice([64, 128, 200, 512, 1024])), int(g.choice([16, 48, 100, 256, 520]))
+        x = H.f32_to_bf16_rne(g.integers(-4, 5, size=int(np.prod(lead + [rows, k]))).astype(np.float32))
+        w8 = H.f32_to_ocp_e4m3_rne(g.integers(-8, 9, size=cols * k).astype(np.float64))
+        b = H.f32_to_bf16_rne(g.integers(-100, 101, size=cols).astype(np.float32))
+        tx = T.Tensor.from_bits(x, "bf16", lead + [rows, k])
+        tw = T.Tensor.from_bits(w8, "f8e4m3", [cols, k]).to_dtype("bf16")
+        assert tw.physical_dtype == "f8e4m3"
+        with_bias, relu = bool(g.integers(2)), bool(g.integers(2))
+        exact = H.bf16_to_f32(x).astype(np.float64).reshape(-1, k) @ H.ocp_e4m3_decode(w8).astype(np.float64).reshape(cols, k).T
+        assert np.abs(exact).max() < 2 ** 24
+        plain = H.f32_to_bf16_rne(exact.astype(np.float32).ravel())
+        what = f"case {n}: {lead + [rows, k]} x [{cols}, {k}]^T bias {with_bias} relu {relu}"
+        assert np.array_equal(tx.matmul(tw.t()).to_bits(), plain), what
+        steps = ([("add", b, H.View([cols]))] if with_bias else []) + ([("relu",)] if relu else [])
+        got = T.Linear(tw, T.Tensor.from_bits(b, "bf16", [cols]) if with_bias else None).forward(tx, relu=relu)
+        assert list(got.shape) == lead + [rows, cols], what
+        assert np.array_equal(got.to_bits(), _oracle_after("bf16", plain, lead + [rows, cols], steps)), what
