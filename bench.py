@@ -865,7 +865,7 @@ def main():
     ap.add_argument("--configs", default="c1,c2,c3,c4,c5,f8,f64,fused,bwd,casts")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default="", help="time exactly one case key (e.g. c5_down_bf16) and print its result")
-    ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin the MFMA tile variant (0..3)")
+    ap.add_argument("--force-tile", type=int, default=-1, help="testing hook: pin a kernel variant (include/hodu_rocm_debug.h; 15 and 16: the 16 x 16 x 32 tile and its respaced form)")
     ap.add_argument("--graph", action="store_true", help="with --only: replay the K launches as one HIP graph")
     ap.add_argument("--force-splitk", type=int, default=-1, help="testing hook: pin the number of K ranges")
     args = ap.parse_args()
