@@ -232,7 +232,7 @@ def test_fused_steps_over_random_layouts(contexts, dt):
 @pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64", "i8", "u8", "f8e4m3", "f8e5m2", "bf16_f8e4m3w", "i32_i8i8"])
 def test_pinned_tiles_and_k_cuts_over_random_layouts(contexts, dt):
     """the same draw with the testing hooks pinning a tile of the matrix-core kernels (general and pipelined, 256 x 256
-    down to 64 x 64, the 16 x 16 x 32 tile and its respaced form, the few-rows kernel's shapes, the small-f32 kernel at any size,
+    down to 64 x 64, the 16 x 16 x 32 tile and its respaced form, the GEMV and few-rows kernels' shapes, the small-f32 kernel at any size,
     the f64 tiles) and a number of K ranges: the large tiles on small,
     ragged, oddly laid out products, where the automatic choice never puts them.  A hook that does not apply to a
     layout leaves the choice to the dispatcher; whatever runs must be right"""
@@ -240,7 +240,7 @@ def test_pinned_tiles_and_k_cuts_over_random_layouts(contexts, dt):
     for n in range(4 * ROUNDS):
         op, lv, rv = product_case(g)
         ctx = contexts["end" if n % 2 == 0 else "start"]
-        hooks = {"f64": [41, 42, 43], "f32": [0, 1, 2, 3, 10, 11, 12, 13, 40]}.get(dt, [0, 1, 2, 3, 10, 11, 12, 13, 14, 15, 16, 35, 36, 37, 38, 39])
+        hooks = {"f64": [41, 42, 43], "f32": [0, 1, 2, 3, 10, 11, 12, 13, 40]}.get(dt, [0, 1, 2, 3, 10, 11, 12, 13, 14, 15, 16, 30, 31, 32, 33, 34, 35, 36, 37, 38, 39])
         hook, cuts = int(g.choice(hooks)), int(g.choice([-1, -1, 1, 2, 3]))
         ctx.force_tile(hook)
         ctx.force_splitk(cuts)
