@@ -313,3 +313,29 @@ def test_masked_softmax_over_random_layouts(contexts, dt):
             check_masked_softmax(ctx, dt, v, mask_shape, causal=causal, seed=n)
         except AssertionError as e:
             raise AssertionError(f"masked softmax {dt} case {n}: {v.shape} {v.strides} +{v.offset}, mask {mask_shape}, causal {causal}: {e}") from None
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "bf16_f8e4m3w", "i32_i8i8"])
+def test_decode_shapes_over_random_sizes_and_pinned_variants(contexts, dt):
+    """one to sixteen rows against a weight stored [N, K] (a Linear layer at decode) or [K, N]: the GEMV, few-rows and
+    row-dense GEMV kernels at random sizes and offsets, automatic and with every shape of theirs pinned"""
+    g = np.random.default_rng(10000 + sum(map(ord, dt)))
+    for n in range(4 * ROUNDS):
+        m = int(g.integers(1, 17))
+        k = int(g.choice([64, 128, 200, 256, 520, 1024, 2048, 4096]))
+        cols = int(g.choice([1, 16, 33, 128, 200, 256, 1040]))
+        while m * k * cols > 8_000_000:
+            cols = max(1, cols // 2)
+        off = int(g.choice([0, 0, 16, 64, 3]))
+        lv = V([m, k], offset=int(g.choice([0, 16, 5])))
+        rv = V([cols, k], offset=off).t() if g.random() < 0.7 else V([k, cols], offset=off)
+        hook = int(g.choice([-1, -1, 30, 31, 32, 33, 34, 35, 36, 37, 38, 39]))
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        ctx.force_tile(hook)
+        try:
+            check_product(ctx, "dot", dt, lv, rv, seed=n)
+        except AssertionError as e:
+            raise AssertionError(f"dot {dt} case {n}, hook {hook}: [{m}, {k}] +{lv.offset} x {rv.shape} {rv.strides} +{rv.offset}, "
+                                 f"kernel {ctx.last_kernel()}: {e}") from None
+        finally:
+            ctx.force_tile(-1)
