@@ -339,3 +339,22 @@ def test_decode_shapes_over_random_sizes_and_pinned_variants(contexts, dt):
                                  f"kernel {ctx.last_kernel()}: {e}") from None
         finally:
             ctx.force_tile(-1)
+
+
+@pytest.mark.parametrize("dt", ffi.PRODUCT_DTYPES)
+def test_products_of_two_long_vectors_over_random_lengths_and_strides(contexts, dt):
+    """[1, K] x [K, 1] (Tensor::matmul of two 1-D tensors): K cut into chunks across workgroups, dense and strided
+    vectors, ragged last chunks, offsets"""
+    g = np.random.default_rng(13000 + sum(map(ord, dt)))
+    scale = 0.25 if dt in ("f8e4m3", "f8e5m2") else 1.0
+    for n in range(ROUNDS):
+        k = int(g.integers(5000, 150_000))
+        sa, sb = int(g.choice([1, 1, 2, 3])), int(g.choice([1, 1, 2, 5]))
+        lv = V([1, k], [0, sa], int(g.choice([0, 16, 3])))
+        rv = V([k, 1], [sb, 0], int(g.choice([0, 16, 7])))
+        ctx = contexts["end" if n % 2 == 0 else "start"]
+        try:
+            check_product(ctx, "dot", dt, lv, rv, seed=n, scale=scale)
+        except AssertionError as e:
+            raise AssertionError(f"dot {dt} case {n}: K {k}, strides {sa} / {sb}, offsets {lv.offset} / {rv.offset}, "
+                                 f"kernel {ctx.last_kernel()}: {e}") from None
