@@ -162,3 +162,24 @@ def test_linear_layers_with_deferred_f8_weights():
         got = T.Linear(tw, T.Tensor.from_bits(b, "bf16", [cols]) if with_bias else None).forward(tx, relu=relu)
         assert list(got.shape) == lead + [rows, cols], what
         assert np.array_equal(got.to_bits(), _oracle_after("bf16", plain, lead + [rows, cols], steps)), what
+
+
+@pytest.mark.parametrize("dt", ["i32", "f32"])
+def test_weight_gradients_with_the_batch_folded_into_the_contraction(dt, mode):
+    """matmul_vjp of a batched contiguous input against a 2-D weight (every Linear): the weight's gradient is ONE product
+    over batch x rows in 'nocopy' mode, the batched product followed by sums in 'reference' mode -- the same integers"""
+    g = np.random.default_rng(14000 + sum(map(ord, dt)))
+    for n in range(40):
+        lead = [int(g.integers(1, 5)) for _ in range(int(g.integers(1, 3)))]
+        m, k, cols = (int(g.choice([1, 3, 8, 16, 33, 64])) for _ in range(3))
+        (ta, a), (tb, b), (tg, grad) = make(g, dt, lead + [m, k]), make(g, dt, [k, cols]), make(g, dt, lead + [m, cols])
+        T.stats(reset=True)
+        da, db = T.matmul_vjp(ta, tb, tg)
+        st = T.stats()
+        a64, b64, g64 = (x.astype(np.float64) for x in (a, b, grad))
+        what = f"{dt} {mode} case {n}: {lead + [m, k]} x {[k, cols]}"
+        assert np.array_equal(values(da, dt).astype(np.float64), g64 @ b64.T), what
+        want_b = a64.reshape(-1, k).T @ g64.reshape(-1, cols)
+        assert list(db.shape) == [k, cols] and np.array_equal(values(db, dt).astype(np.float64), want_b), what
+        if mode == "nocopy":
+            assert st["sum_kernels"] == 0, (what, st)  # folded: no [B, K, N] intermediate to sum
