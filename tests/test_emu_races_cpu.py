@@ -63,7 +63,7 @@ def test_a_hand_off_without_its_barrier_or_wait_is_reported(driver, fault):
 
 
 SUITES = ["test_emu_mfma_cpu.py", "test_emu_kernel_families_cpu.py", "test_emu_plain_kernels_cpu.py", "test_emu_softmax_cpu.py",
-          "test_emu_reference_sums_cpu.py", "test_emu_gpu_suites_cpu.py", "test_emu_host_mirror_cpu.py", "test_emu_random_layouts_cpu.py"]
+          "test_emu_reference_sums_cpu.py", "test_emu_gpu_suites_cpu.py", "test_emu_host_mirror_cpu.py", "test_emu_random_layouts_cpu.py", "test_emu_random_tensors_cpu.py"]
 
 
 @pytest.mark.skipif(os.environ.get("HODU_EMU_ALL", "") in ("", "0"), reason="ten minutes; set HODU_EMU_ALL=1")
