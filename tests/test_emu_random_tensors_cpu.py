@@ -15,6 +15,7 @@ from hodu_amd import tensor as T
 pytestmark = pytest.mark.skipif(emu_util.compiler() is None, reason="no host clang++ for the CPU build")
 NP = {"i32": np.int32, "f32": np.float32, "i64": np.int64}
 BITS = {"i32": np.uint32, "f32": np.uint32, "i64": np.uint64}
+BITS_BY_SIZE = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -183,3 +184,31 @@ def test_weight_gradients_with_the_batch_folded_into_the_contraction(dt, mode):
         assert list(db.shape) == [k, cols] and np.array_equal(values(db, dt).astype(np.float64), want_b), what
         if mode == "nocopy":
             assert st["sum_kernels"] == 0, (what, st)  # folded: no [B, K, N] intermediate to sum
+
+
+def test_to_dtype_of_random_views_matches_the_cast_oracle():
+    """to_dtype of a transposed, stepped-slice view for random dtype pairs (the deferred pairs f8e4m3 -> bf16 and i8 -> i32
+    included: read back, they must be the cast's values), against the oracle's cast of the same logical elements"""
+    import helpers as H
+    import oracle
+    from test_gpu_casts import in_domain, same
+    g = np.random.default_rng(15000)
+    names = list(oracle.DTYPE_ID)
+    for n in range(150):
+        src, dst = names[int(g.integers(len(names)))], names[int(g.integers(len(names)))]
+        nd = int(g.integers(1, 4))
+        stored = [int(g.choice([1, 2, 5, 8, 17, 40])) for _ in range(nd)]
+        bits = in_domain(src, dst, H.random_storage(src, int(np.prod(stored)), 50 + n, 3.0))
+        t, a = T.Tensor.from_bits(bits.view(BITS_BY_SIZE[bits.dtype.itemsize]), src, stored), bits.reshape(stored)
+        if nd >= 2 and g.random() < 0.6:
+            d1, d2 = (int(x) for x in g.choice(nd, size=2, replace=False))
+            t, a = t.transpose(d1, d2), np.swapaxes(a, d1, d2)
+        for d in range(nd):
+            if a.shape[d] >= 4 and g.random() < 0.5:
+                start, step = int(g.integers(0, 2)), int(g.choice([1, 2]))
+                t, a = t.slice(d, start, a.shape[d], step), a[(slice(None),) * d + (slice(start, None, step),)]
+        logical = np.ascontiguousarray(a).reshape(-1)
+        want = oracle.cast(src, dst, logical, H.cast_md(H.View(list(a.shape))), decode=oracle.F8_OCP)
+        got = t.to_dtype(dst)
+        assert list(got.shape) == list(a.shape)
+        assert same(got.to_bits().view(oracle.STORAGE[dst]), want, dst), (n, src, dst, list(a.shape), t.layout())
