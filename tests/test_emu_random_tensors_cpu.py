@@ -212,3 +212,53 @@ def test_to_dtype_of_random_views_matches_the_cast_oracle():
         got = t.to_dtype(dst)
         assert list(got.shape) == list(a.shape)
         assert same(got.to_bits().view(oracle.STORAGE[dst]), want, dst), (n, src, dst, list(a.shape), t.layout())
+
+
+def test_attention_programs_with_random_masks():
+    """scaled_dot_product_attention through the Tensor API: q against k / v that lack or repeat batch dims, an optional
+    attn_mask of any broadcastable shape and of u8 / bool / f32 dtype, is_causal or not; bf16 at head dims 64 / 128 (the
+    one kernel) and 32 (three launches), f32 (three launches); against the float64 function, a masked score filled with
+    what the reference's masked_fill writes in the dtype"""
+    import helpers as H
+    g = np.random.default_rng(16000)
+    for n in range(40):
+        dt = "bf16" if g.random() < 0.75 else "f32"
+        d = int(g.choice([32, 64, 128])) if dt == "bf16" else int(g.choice([16, 64]))
+        batch = [int(g.integers(1, 4)) for _ in range(int(g.integers(0, 3)))]
+        sq, sk = int(g.choice([1, 7, 33, 64, 100])), int(g.choice([1, 9, 32, 65, 130]))
+        kv_batch = [b if g.random() < 0.6 else 1 for b in batch][int(g.integers(0, len(batch) + 1)):]
+        def bits(shape, seed):
+            x = np.random.default_rng(seed).standard_normal(shape).astype(np.float32)
+            if dt == "bf16":
+                b = H.f32_to_bf16_rne(x.ravel())
+                return T.Tensor.from_bits(b, "bf16", list(shape)), H.bf16_to_f32(b).astype(np.float64).reshape(shape)
+            return T.Tensor.from_bits(x.ravel().view(np.uint32), "f32", list(shape)), x.astype(np.float64)
+        (tq, q), (tk, k), (tv, v) = bits(batch + [sq, d], 3 * n), bits(kv_batch + [sk, d], 3 * n + 1), bits(kv_batch + [sk, d], 3 * n + 2)
+        causal, masked = bool(g.integers(2)), bool(g.integers(3))
+        keep, tm = None, None
+        if masked:
+            full = batch + [sq, sk]
+            mshape = [e if g.random() < 0.6 else 1 for e in full[int(g.integers(0, len(full))):]]
+            keep = (g.random(mshape) < 0.7).astype(np.uint8)
+            keep[..., 0] = 1
+            mdt = str(g.choice(["u8", "bool", "f32"]))
+            mbits = keep.astype(np.float32).ravel().view(np.uint32) if mdt == "f32" else keep.ravel()
+            tm = T.Tensor.from_bits(mbits, mdt, mshape)
+        got_t = T.scaled_dot_product_attention(tq, tk, tv, causal, tm)
+        scale = float(H.bf16_to_f32(T.scalar_bits("bf16", 1.0 / np.sqrt(float(d))))[0]) if dt == "bf16" else float(np.float32(1.0 / np.sqrt(float(d))))
+        s = q @ np.swapaxes(k, -1, -2) * scale
+        filled = np.zeros(s.shape, bool)
+        if masked:
+            filled |= np.broadcast_to(keep == 0, s.shape)
+        if causal:
+            filled |= np.arange(sk)[None, :] > np.arange(sq)[:, None]
+        s = np.where(filled, -65536.0 if dt == "bf16" else -np.inf, s)
+        p = np.exp(s - s.max(-1, keepdims=True))
+        p = p / p.sum(-1, keepdims=True)
+        want = p @ v
+        raw = got_t.to_bits()
+        got = (H.bf16_to_f32(raw) if dt == "bf16" else raw.view(np.float32)).astype(np.float64).reshape(want.shape)
+        tol = 2e-2 if dt == "bf16" else 1e-4
+        size = np.maximum(np.abs(want), p @ np.abs(np.broadcast_to(v, want.shape[:-2] + v.shape[-2:])))
+        assert list(got_t.shape) == list(want.shape)
+        assert np.all(np.abs(got - want) <= tol * size + 1e-30), (n, dt, d, batch, kv_batch, sq, sk, causal, masked, float(np.abs(got - want).max()))
